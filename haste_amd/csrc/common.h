@@ -1,0 +1,86 @@
+// Host-side plumbing shared by every translation unit of libhaste_hip.so:
+// error codes, argument checks, the per-stream device workspace and the
+// internal (non-exported) launch helpers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+
+#include "../../include/haste_hip.h"
+
+namespace haste_hip {
+
+// Records the text of a failed HIP call for haste_hip_last_runtime_error().
+void set_runtime_error(hipError_t err, const char* what);
+
+#define HASTE_HIP_TRY(expr)                                   \
+  do {                                                        \
+    hipError_t err__ = (expr);                                \
+    if (err__ != hipSuccess) {                                \
+      ::haste_hip::set_runtime_error(err__, #expr);           \
+      return HASTE_HIP_ERROR_RUNTIME;                         \
+    }                                                         \
+  } while (0)
+
+#define HASTE_HIP_REQUIRE(cond)                               \
+  do {                                                        \
+    if (!(cond)) return HASTE_HIP_ERROR_INVALID_ARGUMENT;     \
+  } while (0)
+
+#define HASTE_HIP_PROPAGATE(expr)                             \
+  do {                                                        \
+    int rc__ = (expr);                                        \
+    if (rc__ != HASTE_HIP_OK) return rc__;                    \
+  } while (0)
+
+// Layout of the control block at the start of a workspace (all zero between
+// kernels; every kernel that uses a field restores it to zero before it exits).
+constexpr int kMaxGroups = 64;        // batch tiles a persistent kernel may have
+constexpr int kCounterStride = 32;    // uint32 slots between counters (128 B apart)
+struct ControlBlock {
+  unsigned int step_counter[kMaxGroups * kCounterStride];  // per-group step barrier
+  unsigned int exit_counter[kMaxGroups * kCounterStride];  // per-group "left the loop" count
+  unsigned int grid_exit_counter[kCounterStride];          // all workgroups of a launch
+  unsigned int tile_counter[4096];                         // split-K arrivals per output tile
+  unsigned int abort_flag[kCounterStride];                 // set when a barrier wait gives up
+};
+
+// A block of device memory owned by the library and tied to one (device, stream):
+// the control block followed by a scratch area that grows on demand.  Work that
+// uses it is ordered by the stream, so one workspace per stream is race free.
+struct Workspace {
+  ControlBlock* control = nullptr;   // device
+  float* scratch = nullptr;          // device
+  size_t scratch_bytes = 0;
+  unsigned int* host_status = nullptr;      // pinned host word the kernels report aborts to
+  unsigned int* host_status_dev = nullptr;  // the same word as the device addresses it
+};
+
+// Returns the workspace of (current device, stream) with at least `scratch_bytes`
+// of scratch, creating or growing it if needed.
+int get_workspace(hipStream_t stream, size_t scratch_bytes, Workspace* out);
+
+// Checks (without synchronizing) whether a persistent kernel launched earlier on
+// this workspace reported a barrier time-out; if so re-zeroes the control block and
+// returns HASTE_HIP_ERROR_STEP_BARRIER once.
+int check_and_clear_abort(hipStream_t stream, Workspace* ws);
+
+int device_cu_count();
+
+// C[M,N] = op(A)*B (+C): fp32 MFMA GEMM on `stream`. `ws` supplies split-K scratch.
+int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
+             const float* A, int lda, const float* B, int ldb,
+             float* C, int ldc, bool accumulate);
+
+// Row-wise layer norm kernels (rows x dim), used stand-alone and by the LN cells.
+int layer_norm_forward(hipStream_t stream, int rows, int dim, const float* gamma,
+                       const float* beta, const float* x, float* y, float* cache);
+int layer_norm_backward(hipStream_t stream, int rows, int dim, const float* gamma,
+                        const float* x, const float* dy, float* dx, float* dgamma,
+                        float* dbeta);
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+}  // namespace haste_hip

@@ -1,0 +1,497 @@
+// LSTM forward and backward passes: one MFMA GEMM for the time-fused input
+// projection, one persistent kernel for the T-step recurrence (gate nonlinearities,
+// cell update, zoneout and optional DropConnect fused in), and for the backward pass
+// one persistent reverse-time kernel followed by the three batched GEMMs.
+//
+// Arithmetic follows reference lib/lstm_forward_gpu.cu.cc:55-86 and
+// lib/lstm_backward_gpu.cu.cc:47-95; orchestration replaces :313-366 and :319-405.
+#include "recurrent.h"
+
+namespace haste_hip {
+namespace {
+
+struct LstmFwdParams {
+  int training, T, N, H;
+  const float* R;       // [H,4H]
+  const float* b;       // [4H]
+  float* h;             // [T+1,N,H]
+  float* c;             // [T+1,N,H]
+  float* v;             // [T,N,4H] in: x*W, out (training): activations
+  float zoneout_prob;
+  const float* zoneout_mask;   // [T,N,H] or null
+  const float* dc_mask;        // DropConnect mask [H,4H] or null
+  float dc_scale;
+  ControlBlock* cb;
+  unsigned int* host_status;
+  unsigned int spin_limit;
+};
+
+// HS hidden units per workgroup = 4*CT (their 4 gate columns fill CT MFMA column tiles).
+template <int RT, int CT>
+__global__ __launch_bounds__(256, 1)
+void lstm_forward_kernel(LstmFwdParams p) {
+  constexpr int HS = 4 * CT;
+  constexpr int NB = 16 * RT;
+  constexpr int NCOLS = 16 * CT;
+  constexpr int PP = (NB * HS + 255) / 256;
+  constexpr int CHUNK = RT == 1 ? 8 : (RT == 2 ? 8 : 4);
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+
+  const int H = p.H, N = p.N, T = p.T;
+  const int Kpad = round_up(H, 64);
+  float* w_lds = lds;
+  float* red = lds + Kpad * NCOLS;
+
+  const int tid = threadIdx.x;
+  const int j0 = blockIdx.x * HS;
+  const int n0 = blockIdx.y * NB;
+  const size_t NH = (size_t)N * H;
+
+  GroupSync gs;
+  group_sync_init(gs, p.cb, blockIdx.y, gridDim.x, p.host_status, p.spin_limit);
+
+  // Resident slice: column c of the slice is gate c/HS, hidden unit j0 + c%HS.
+  for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
+    const int k = idx / NCOLS, cidx = idx % NCOLS;
+    const int gate = cidx / HS, j = j0 + cidx % HS;
+    float w = 0.f;
+    if (k < H && j < H) {
+      const size_t off = (size_t)k * 4 * H + gate * H + j;
+      w = p.R[off];
+      if (p.dc_mask != nullptr) w = w * p.dc_mask[off] * p.dc_scale;
+    }
+    w_lds[slice_index(k, cidx, NCOLS)] = w;
+  }
+
+  // Pointwise ownership: thread slot pp handles batch row n, hidden unit j.
+  int pn[PP], pj[PP], pl[PP], pc[PP];
+  bool act[PP];
+  float c_prev[PP], h_prev[PP], bias[PP][4];
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp) {
+    const int idx = tid + 256 * pp;
+    pl[pp] = idx / HS;           // local batch row
+    pc[pp] = idx % HS;           // local hidden unit
+    pn[pp] = n0 + pl[pp];
+    pj[pp] = j0 + pc[pp];
+    act[pp] = idx < NB * HS && pn[pp] < N && pj[pp] < H;
+    c_prev[pp] = 0.f;
+    h_prev[pp] = 0.f;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) bias[pp][g] = 0.f;
+    if (act[pp]) {
+      c_prev[pp] = p.c[(size_t)pn[pp] * H + pj[pp]];
+      h_prev[pp] = p.h[(size_t)pn[pp] * H + pj[pp]];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) bias[pp][g] = p.b[g * H + pj[pp]];
+    }
+  }
+  const bool zoneout = p.zoneout_prob != 0.f && p.zoneout_mask != nullptr;
+  const bool vec_ok = (H % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.h) & 15u) == 0);
+  __syncthreads();
+
+  for (int t = 0; t < T; ++t) {
+    // Inputs of this step that do not depend on the recurrence: issue before waiting.
+    float wx[PP][4], mk[PP];
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      mk[pp] = 1.f;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) wx[pp][g] = 0.f;
+      if (act[pp]) {
+        const float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) wx[pp][g] = vt[g * H];
+        if (zoneout && p.training) mk[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
+      }
+    }
+    if (t > 0) group_wait(gs);  // h[t] complete for this batch tile
+
+    float4_t acc[RT][CT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
+    slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, N - n0, H, Kpad, w_lds,
+                                vec_ok, acc);
+    store_partials<RT, CT>(red, acc);
+    __syncthreads();
+
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      if (act[pp]) {
+        float a[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          a[g] = wx[pp][g] + sum_partials<RT, CT>(red, pl[pp], g * HS + pc[pp]) + bias[pp][g];
+        const float gi = sigmoid_f(a[0]);
+        const float gg = tanhf(a[1]);
+        const float gf = sigmoid_f(a[2]);
+        const float go = sigmoid_f(a[3]);
+        if (p.training) {
+          float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+          vt[0] = gi;
+          vt[H] = gg;
+          vt[2 * H] = gf;
+          vt[3 * H] = go;
+        }
+        const float c_new = gf * c_prev[pp] + gi * gg;
+        float h_new = go * tanhf(c_new);
+        if (zoneout) {
+          if (p.training) h_new = (h_new - h_prev[pp]) * mk[pp] + h_prev[pp];
+          else h_new = p.zoneout_prob * h_prev[pp] + (1.0f - p.zoneout_prob) * h_new;
+        }
+        const size_t o = (size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp];
+        p.c[o] = c_new;
+        p.h[o] = h_new;
+        c_prev[pp] = c_new;
+        h_prev[pp] = h_new;
+      }
+    }
+    if (t + 1 < T) group_arrive(gs);  // publishes h[t+1]; also fences `red` reuse
+  }
+  group_leave(gs);
+}
+
+struct LstmBwdParams {
+  int T, N, H;
+  const float* R_t;     // [4H,H]
+  const float* c;       // [T+1,N,H]
+  const float* dh_new;  // [T+1,N,H]
+  const float* dc_new;  // [T+1,N,H]
+  float* db;            // [4H] accumulated
+  float* dh;            // [N,H] in/out
+  float* dc;            // [N,H] in/out
+  float* v;             // [T,N,4H] in: activations, out: gate gradients
+  const float* zoneout_mask;
+  float* db_partial;    // [batch tiles, 4H] scratch
+  ControlBlock* cb;
+  unsigned int* host_status;
+  unsigned int spin_limit;
+};
+
+// A workgroup owns 16 hidden units (HSB) for 16*RT batch rows; its slice of R_t is
+// [4H x 16]: dh[:, its units] = dv_t[:, all 4H] * R_t[:, its units].
+template <int RT>
+__global__ __launch_bounds__(256, 1)
+void lstm_backward_kernel(LstmBwdParams p) {
+  constexpr int HSB = 16;
+  constexpr int NB = 16 * RT;
+  constexpr int NCOLS = 16;
+  constexpr int PP = RT;  // NB*HSB/256
+  constexpr int CHUNK = RT == 1 ? 16 : (RT == 2 ? 8 : 4);
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  __shared__ unsigned int s_flag;
+
+  const int H = p.H, N = p.N, T = p.T;
+  const int K = 4 * H;
+  const int Kpad = round_up(K, 64);
+  float* w_lds = lds;
+  float* red = lds + Kpad * NCOLS;  // 4*NB*NCOLS floats, also reused for the db reduction
+
+  const int tid = threadIdx.x;
+  const int j0 = blockIdx.x * HSB;
+  const int n0 = blockIdx.y * NB;
+  const size_t NH = (size_t)N * H;
+
+  GroupSync gs;
+  group_sync_init(gs, p.cb, blockIdx.y, gridDim.x, p.host_status, p.spin_limit);
+
+  for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
+    const int k = idx / NCOLS, cidx = idx % NCOLS;
+    float w = 0.f;
+    if (k < K && j0 + cidx < H) w = p.R_t[(size_t)k * H + j0 + cidx];
+    w_lds[slice_index(k, cidx, NCOLS)] = w;
+  }
+
+  int pn[PP], pj[PP], pl[PP], pc[PP];
+  bool act[PP];
+  float dh[PP], dc[PP], dbacc[PP][4];
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp) {
+    const int idx = tid + 256 * pp;
+    pl[pp] = idx / HSB;
+    pc[pp] = idx % HSB;
+    pn[pp] = n0 + pl[pp];
+    pj[pp] = j0 + pc[pp];
+    act[pp] = pn[pp] < N && pj[pp] < H;
+    dh[pp] = act[pp] ? p.dh[(size_t)pn[pp] * H + pj[pp]] : 0.f;
+    dc[pp] = act[pp] ? p.dc[(size_t)pn[pp] * H + pj[pp]] : 0.f;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) dbacc[pp][g] = 0.f;
+  }
+  const bool zoneout = p.zoneout_mask != nullptr;
+  const bool vec_ok = (H % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.v) & 15u) == 0);
+  __syncthreads();
+
+  // Step inputs that do not depend on the recurrence, fetched one step ahead.
+  struct StepIn { float vt[4], c0, c1, dhn, dcn, m; };
+  StepIn nxt[PP];
+  auto fetch = [&](int t) {
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      StepIn s = {{0.f, 0.f, 0.f, 0.f}, 0.f, 0.f, 0.f, 0.f, 1.f};
+      if (act[pp] && t >= 0) {
+        const size_t e = (size_t)pn[pp] * H + pj[pp];
+        const float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) s.vt[g] = vt[g * H];
+        s.c0 = p.c[(size_t)t * NH + e];
+        s.c1 = p.c[(size_t)(t + 1) * NH + e];
+        s.dhn = p.dh_new[(size_t)(t + 1) * NH + e];
+        s.dcn = p.dc_new[(size_t)(t + 1) * NH + e];
+        if (zoneout) s.m = p.zoneout_mask[(size_t)t * NH + e];
+      }
+      nxt[pp] = s;
+    }
+  };
+  fetch(T - 1);
+
+  for (int t = T - 1; t >= 0; --t) {
+    float dh_keep[PP];
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      dh_keep[pp] = 0.f;
+      if (act[pp]) {
+        const StepIn s = nxt[pp];
+        const float gi = s.vt[0], gg = s.vt[1], gf = s.vt[2], go = s.vt[3];
+        float dc_total = s.dcn + dc[pp];
+        float dh_total = s.dhn + dh[pp];
+        const float c_tanh = tanhf(s.c1);
+        if (zoneout) {
+          dh_keep[pp] = (1.0f - s.m) * dh_total;
+          dh_total = s.m * dh_total;
+        }
+        const float do_ = c_tanh * dh_total;
+        const float dc_tanh = go * dh_total;
+        dc_total += d_tanh_f(c_tanh) * dc_tanh;
+        const float df = s.c0 * dc_total;
+        dc[pp] = gf * dc_total;
+        const float di = gg * dc_total;
+        const float dg = gi * dc_total;
+        const float dv_i = d_sigmoid_f(gi) * di;
+        const float dv_g = d_tanh_f(gg) * dg;
+        const float dv_f = d_sigmoid_f(gf) * df;
+        const float dv_o = d_sigmoid_f(go) * do_;
+        float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+        vt[0] = dv_i;
+        vt[H] = dv_g;
+        vt[2 * H] = dv_f;
+        vt[3 * H] = dv_o;
+        dbacc[pp][0] += dv_i;
+        dbacc[pp][1] += dv_g;
+        dbacc[pp][2] += dv_f;
+        dbacc[pp][3] += dv_o;
+      }
+    }
+    group_arrive(gs);   // dv_t of this workgroup's columns is published
+    fetch(t - 1);       // overlap next step's loads with the wait
+    group_wait(gs);     // all 4H columns of dv_t are complete for this batch tile
+
+    float4_t acc[RT][1];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) acc[rt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
+    slice_matmul<RT, 1, CHUNK>(p.v + ((size_t)t * N + n0) * 4 * H, 4 * H, N - n0, K, Kpad, w_lds,
+                               vec_ok, acc);
+    store_partials<RT, 1>(red, acc);
+    __syncthreads();
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp)
+      dh[pp] = dh_keep[pp] + sum_partials<RT, 1>(red, pl[pp], pc[pp]);
+    // `red` is next written after the __syncthreads inside the next group_arrive.
+  }
+
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp) {
+    if (act[pp]) {
+      p.dh[(size_t)pn[pp] * H + pj[pp]] = dh[pp];
+      p.dc[(size_t)pn[pp] * H + pj[pp]] = dc[pp];
+    }
+  }
+
+  // Bias gradient: sum over this tile's rows in LDS (fixed order), park per tile,
+  // and let the last workgroup of the launch add the tiles in order.
+  __syncthreads();
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) red[(pl[pp] * 4 + g) * HSB + pc[pp]] = act[pp] ? dbacc[pp][g] : 0.f;
+  __syncthreads();
+  if (tid < 4 * HSB) {
+    const int g = tid / HSB, jj = tid % HSB;
+    float s = 0.f;
+    for (int r = 0; r < NB; ++r) s += red[(r * 4 + g) * HSB + jj];
+    if (j0 + jj < H) p.db_partial[(size_t)blockIdx.y * 4 * H + g * H + j0 + jj] = s;
+  }
+  group_leave(gs);
+  if (grid_last_arrival(p.cb, gridDim.x * gridDim.y, &s_flag)) {
+    for (int col = tid; col < 4 * H; col += 256) {
+      float s = 0.f;
+      for (int bt = 0; bt < (int)gridDim.y; ++bt) s += p.db_partial[(size_t)bt * 4 * H + col];
+      p.db[col] += s;
+    }
+  }
+}
+
+size_t fwd_lds_bytes(int H, int RT, int CT) {
+  const int Kpad = (H + 63) / 64 * 64;
+  return ((size_t)Kpad * 16 * CT + 4 * 16 * RT * 16 * CT) * sizeof(float);
+}
+
+size_t bwd_lds_bytes(int K, int RT) {
+  const int Kpad = (K + 63) / 64 * 64;
+  const size_t red = (size_t)4 * 16 * RT * 16;
+  return ((size_t)Kpad * 16 + red) * sizeof(float);
+}
+
+template <typename KernelT, typename ParamsT>
+int launch_persistent(KernelT kernel, dim3 grid, size_t lds_bytes, ParamsT& params,
+                      hipStream_t stream) {
+  HASTE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+  int per_cu = 0;
+  HASTE_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, lds_bytes));
+  const long long capacity = (long long)per_cu * device_cu_count();
+  if ((long long)grid.x * grid.y > capacity) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  void* args[] = {&params};
+  HASTE_HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<const void*>(kernel), grid, dim3(256),
+                                           args, (unsigned int)lds_bytes, stream));
+  return HASTE_HIP_OK;
+}
+
+constexpr size_t kMaxLdsBytes = 160 * 1024;
+
+}  // namespace
+
+// Picks (RT, CT) for a forward recurrence with G gate blocks; shared with the GRU.
+// Preference: widest column tile that fits the LDS and the cooperative grid.
+int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int H,
+                      const float* W, const float* R, const float* b, const float* x,
+                      float* h, float* c, float* v, float zoneout_prob,
+                      const float* zoneout_mask, const float* dc_mask, float dc_scale) {
+  HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
+  HASTE_HIP_REQUIRE(W && R && b && x && h && c && v);
+  Workspace ws;
+  HASTE_HIP_PROPAGATE(get_workspace(stream, 0, &ws));
+  HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
+
+  // v = x * W for all steps at once.
+  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 4 * H, C, x, C, W, 4 * H, v, 4 * H, false));
+
+  LstmFwdParams p;
+  p.training = training; p.T = T; p.N = N; p.H = H;
+  p.R = R; p.b = b; p.h = h; p.c = c; p.v = v;
+  p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
+  p.dc_mask = dc_mask; p.dc_scale = dc_scale;
+  p.cb = ws.control; p.host_status = ws.host_status_dev; p.spin_limit = kSpinLimit;
+
+  const int cus = device_cu_count();
+  // Candidates in order of preference: fewer rows per workgroup first (more CUs busy).
+  struct Cand { int rt, ct; };
+  const Cand cands[] = {{1, 2}, {1, 4}, {1, 1}, {2, 2}, {2, 4}, {2, 1}, {4, 2}, {4, 4}, {4, 1}};
+  for (const Cand& cd : cands) {
+    const int HS = 4 * cd.ct, NB = 16 * cd.rt;
+    const int gx = (H + HS - 1) / HS, gy = (N + NB - 1) / NB;
+    if (gy > kMaxGroups || (long long)gx * gy > cus) continue;
+    const size_t lds = fwd_lds_bytes(H, cd.rt, cd.ct);
+    if (lds > kMaxLdsBytes) continue;
+    dim3 grid(gx, gy);
+#define HASTE_LAUNCH_FWD(RT_, CT_)                                                         \
+    if (cd.rt == RT_ && cd.ct == CT_)                                                      \
+      return launch_persistent(lstm_forward_kernel<RT_, CT_>, grid, lds, p, stream);
+    HASTE_LAUNCH_FWD(1, 1) HASTE_LAUNCH_FWD(1, 2) HASTE_LAUNCH_FWD(1, 4)
+    HASTE_LAUNCH_FWD(2, 1) HASTE_LAUNCH_FWD(2, 2) HASTE_LAUNCH_FWD(2, 4)
+    HASTE_LAUNCH_FWD(4, 1) HASTE_LAUNCH_FWD(4, 2) HASTE_LAUNCH_FWD(4, 4)
+#undef HASTE_LAUNCH_FWD
+  }
+  return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+}
+
+int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
+                       const float* W_t, const float* R_t, const float* x_t,
+                       const float* h, const float* c, const float* dh_new, const float* dc_new,
+                       float* dx, float* dW, float* dR, float* db, float* dh, float* dc, float* v,
+                       const float* zoneout_mask) {
+  HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
+  HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && c && dh_new && dc_new);
+  HASTE_HIP_REQUIRE(dx && dW && dR && db && dh && dc && v);
+  const int cus = device_cu_count();
+  const int gx = (H + 15) / 16;
+  int rt = 0;
+  for (int cand : {1, 2, 4}) {
+    const int gy = (N + 16 * cand - 1) / (16 * cand);
+    if (gy <= kMaxGroups && (long long)gx * gy <= cus && bwd_lds_bytes(4 * H, cand) <= kMaxLdsBytes) {
+      rt = cand;
+      break;
+    }
+  }
+  if (rt == 0) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  const int gy = (N + 16 * rt - 1) / (16 * rt);
+
+  Workspace ws;
+  HASTE_HIP_PROPAGATE(get_workspace(stream, (size_t)gy * 4 * H * sizeof(float), &ws));
+  HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
+
+  LstmBwdParams p;
+  p.T = T; p.N = N; p.H = H;
+  p.R_t = R_t; p.c = c; p.dh_new = dh_new; p.dc_new = dc_new;
+  p.db = db; p.dh = dh; p.dc = dc; p.v = v; p.zoneout_mask = zoneout_mask;
+  p.db_partial = ws.scratch;
+  p.cb = ws.control; p.host_status = ws.host_status_dev; p.spin_limit = kSpinLimit;
+  const size_t lds = bwd_lds_bytes(4 * H, rt);
+  dim3 grid(gx, gy);
+  int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  if (rt == 1) rc = launch_persistent(lstm_backward_kernel<1>, grid, lds, p, stream);
+  if (rt == 2) rc = launch_persistent(lstm_backward_kernel<2>, grid, lds, p, stream);
+  if (rt == 4) rc = launch_persistent(lstm_backward_kernel<4>, grid, lds, p, stream);
+  HASTE_HIP_PROPAGATE(rc);
+
+  // dW += x^T dv ; dR += h[0:T]^T dv ; dx = dv W^T  (dv now lives in v).
+  const int TN = T * N;
+  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, C, 4 * H, TN, x_t, TN, v, 4 * H, dW, 4 * H, true));
+  HASTE_HIP_PROPAGATE(gemm_f32(stream, true, H, 4 * H, TN, h, H, v, 4 * H, dR, 4 * H, true));
+  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, TN, C, 4 * H, v, 4 * H, W_t, C, dx, C, false));
+  return HASTE_HIP_OK;
+}
+
+}  // namespace haste_hip
+
+extern "C" {
+
+int haste_hip_lstm_forward_f32(int training, int steps, int batch_size, int input_size,
+                               int hidden_size,
+                               const float* W, const float* R, const float* b, const float* x,
+                               float* h, float* c, float* v, float* tmp_Rh,
+                               float zoneout_prob, const float* zoneout_mask, void* stream) {
+  (void)tmp_Rh;  // the recurrent product never leaves the chip
+  return haste_hip::lstm_forward_impl(haste_hip::as_stream(stream), training, steps, batch_size,
+                                      input_size, hidden_size, W, R, b, x, h, c, v, zoneout_prob,
+                                      zoneout_mask, nullptr, 1.0f);
+}
+
+int haste_hip_lstm_forward_dropconnect_f32(int training, int steps, int batch_size,
+                                           int input_size, int hidden_size,
+                                           const float* W, const float* R, const float* b,
+                                           const float* x, float* h, float* c, float* v,
+                                           float zoneout_prob, const float* zoneout_mask,
+                                           const float* dropconnect_mask, float dropconnect_scale,
+                                           void* stream) {
+  return haste_hip::lstm_forward_impl(haste_hip::as_stream(stream), training, steps, batch_size,
+                                      input_size, hidden_size, W, R, b, x, h, c, v, zoneout_prob,
+                                      zoneout_mask, dropconnect_mask, dropconnect_scale);
+}
+
+int haste_hip_lstm_backward_f32(int steps, int batch_size, int input_size, int hidden_size,
+                                const float* W_t, const float* R_t, const float* b,
+                                const float* x_t, const float* h, const float* c,
+                                const float* dh_new, const float* dc_new,
+                                float* dx, float* dW, float* dR, float* db,
+                                float* dh, float* dc, float* v,
+                                const float* zoneout_mask, void* stream) {
+  (void)b;  // unused by the reference as well (lib/lstm_backward_gpu.cu.cc:319-405)
+  return haste_hip::lstm_backward_impl(haste_hip::as_stream(stream), steps, batch_size, input_size,
+                                       hidden_size, W_t, R_t, x_t, h, c, dh_new, dc_new, dx, dW,
+                                       dR, db, dh, dc, v, zoneout_mask);
+}
+
+}  // extern "C"

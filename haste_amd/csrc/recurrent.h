@@ -1,0 +1,227 @@
+// Device-side building blocks of the persistent recurrence kernels.
+//
+// A recurrence kernel is one cooperative launch that runs all T steps.  The grid is
+// (column workgroups) x (batch tiles): a workgroup owns `HS` hidden units (all of
+// their gate columns) for the 16*RT batch rows of its tile, keeps its slice of the
+// recurrent weight matrix in LDS for the whole launch, and per step multiplies the
+// tile's rows of the exchanged activation (h_t forward, the gate gradients backward)
+// with that slice on the MFMA units.  Workgroups that share a batch tile form a
+// group and synchronise once per exchange through a counter in device memory;
+// different batch tiles never wait for each other.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+
+namespace haste_hip {
+
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+constexpr unsigned int kSpinLimit = 1u << 24;  // polls before a barrier wait gives up
+
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float d_sigmoid_f(float y) { return y * (1.0f - y); }
+__device__ __forceinline__ float d_tanh_f(float y) { return 1.0f - y * y; }
+
+// Per-workgroup view of its group's step barrier.
+struct GroupSync {
+  unsigned int* counter;       // arrivals so far (monotonic within a launch)
+  unsigned int* exit_counter;  // workgroups of the group that have left the time loop
+  unsigned int* abort_flag;    // device-wide: some wait gave up
+  unsigned int* host_status;   // pinned host word mirrored from abort_flag
+  unsigned int group_size;
+  unsigned int arrivals;       // barriers this workgroup has arrived at
+  unsigned int spin_limit;
+};
+
+__device__ __forceinline__ void group_sync_init(GroupSync& g, ControlBlock* cb, int group,
+                                                unsigned int group_size,
+                                                unsigned int* host_status,
+                                                unsigned int spin_limit) {
+  g.counter = &cb->step_counter[group * kCounterStride];
+  g.exit_counter = &cb->exit_counter[group * kCounterStride];
+  g.abort_flag = &cb->abort_flag[0];
+  g.host_status = host_status;
+  g.group_size = group_size;
+  g.arrivals = 0;
+  g.spin_limit = spin_limit;
+}
+
+// Publishes every global store this workgroup has made so far to the rest of the
+// group and counts the workgroup as arrived.  Called by all threads.
+__device__ __forceinline__ void group_arrive(GroupSync& g) {
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    __hip_atomic_fetch_add(g.counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  g.arrivals += 1;
+}
+
+// Blocks until every workgroup of the group has made as many arrivals as this one.
+// The wait is bounded: after spin_limit polls (or when another workgroup has given
+// up) it raises the abort flag and returns, so that every wavefront still reaches the
+// end of the kernel.  Called by all threads.
+__device__ __forceinline__ void group_wait(GroupSync& g) {
+  if (threadIdx.x == 0) {
+    const unsigned int target = g.arrivals * g.group_size;
+    unsigned int spins = 0;
+    while (__hip_atomic_load(g.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+      __builtin_amdgcn_s_sleep(1);
+      ++spins;
+      if ((spins & 255u) == 0u) {
+        if (__hip_atomic_load(g.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) break;
+        if (spins >= g.spin_limit) {
+          __hip_atomic_store(g.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(g.host_status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+          break;
+        }
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  }
+  __syncthreads();
+}
+
+// Leaves the group: the last workgroup out puts the group's counters back to zero so
+// that the next launch on this stream finds the control block clean.
+__device__ __forceinline__ void group_leave(GroupSync& g) {
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const unsigned int old =
+        __hip_atomic_fetch_add(g.exit_counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (old == g.group_size - 1) {
+      __hip_atomic_store(g.counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(g.exit_counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+// True in exactly one workgroup of the launch: the last to call it.  Stores made by
+// the other workgroups before their call are visible to that workgroup afterwards.
+// `flag` is a word of LDS.  Called by all threads.
+__device__ __forceinline__ bool grid_last_arrival(ControlBlock* cb, unsigned int total_workgroups,
+                                                  unsigned int* flag) {
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    const unsigned int old = __hip_atomic_fetch_add(&cb->grid_exit_counter[0], 1u, __ATOMIC_RELAXED,
+                                                    __HIP_MEMORY_SCOPE_AGENT);
+    const bool last = old == total_workgroups - 1;
+    if (last) {
+      __hip_atomic_store(&cb->grid_exit_counter[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    }
+    *flag = last ? 1u : 0u;
+  }
+  __syncthreads();
+  return *flag != 0u;
+}
+
+__device__ __forceinline__ int round_up(int x, int m) { return (x + m - 1) / m * m; }
+
+// LDS image of a weight slice: element (k, col) of a [Kpad x NCOLS] slice lives at
+// float index (((k/16)*4 + (k%16)/4) * NCOLS + col) * 4 + k%4, i.e. the 4 consecutive
+// k a lane feeds to 4 consecutive 16x16x4 MFMAs are one 16-byte LDS read, and the 16
+// lanes of a k-quarter read 16 consecutive such vectors (no bank conflicts).
+__device__ __forceinline__ int slice_index(int k, int col, int ncols) {
+  return ((((k >> 4) << 2) + ((k & 15) >> 2)) * ncols + col) * 4 + (k & 3);
+}
+
+__device__ __forceinline__ float4_t load_a4(const float* p, int valid, bool vec_ok) {
+  float4_t v = {0.f, 0.f, 0.f, 0.f};
+  if (valid >= 4 && vec_ok) {
+    v = *reinterpret_cast<const float4_t*>(p);
+  } else {
+    if (valid > 0) v.x = p[0];
+    if (valid > 1) v.y = p[1];
+    if (valid > 2) v.z = p[2];
+    if (valid > 3) v.w = p[3];
+  }
+  return v;
+}
+
+// acc[rt][ct] += A[16*RT rows, K] * slice[K, 16*CT] for this wavefront's quarter of K.
+// `a` points at row 0 of the batch tile (row stride a_ld floats, K contiguous);
+// rows >= rows_valid and k >= K read as zero.  The four wavefronts of the workgroup
+// each take Kpad/4 consecutive k; the caller adds their accumulators.
+// Accumulator element r of acc[rt][ct] in lane l is row 16*rt + 4*(l/16) + r,
+// column 16*ct + l%16.
+template <int RT, int CT, int CHUNK>
+__device__ __forceinline__ void slice_matmul(const float* __restrict__ a, int a_ld, int rows_valid,
+                                             int K, int Kpad, const float* w_lds, bool vec_ok,
+                                             float4_t (&acc)[RT][CT]) {
+  constexpr int NCOLS = 16 * CT;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int row = lane & 15;
+  const int kq = lane >> 4;
+  const int groups = Kpad >> 6;  // k-groups of 16 per wavefront
+  const int g_first = wave * groups;
+
+  for (int g0 = 0; g0 < groups; g0 += CHUNK) {
+    float4_t av[CHUNK][RT];
+#pragma unroll
+    for (int gi = 0; gi < CHUNK; ++gi) {
+      const int k = (g_first + g0 + gi) * 16 + kq * 4;
+      const bool live = g0 + gi < groups;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const int rr = rt * 16 + row;
+        const int valid = (live && rr < rows_valid) ? (K - k) : 0;
+        av[gi][rt] = load_a4(a + (size_t)rr * a_ld + k, valid, vec_ok);
+      }
+    }
+#pragma unroll
+    for (int gi = 0; gi < CHUNK; ++gi) {
+      if (g0 + gi < groups) {
+        const int kg = g_first + g0 + gi;
+        const float* wp = w_lds + ((kg * 4 + kq) * NCOLS + row) * 4;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+          const float4_t b = *reinterpret_cast<const float4_t*>(wp + ct * 64);
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) {
+            acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].x, b.x, acc[rt][ct], 0, 0, 0);
+            acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].y, b.y, acc[rt][ct], 0, 0, 0);
+            acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].z, b.z, acc[rt][ct], 0, 0, 0);
+            acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].w, b.w, acc[rt][ct], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+}
+
+// Writes this wavefront's accumulators to red[wave][16*RT][16*CT] in LDS.
+template <int RT, int CT>
+__device__ __forceinline__ void store_partials(float* red, const float4_t (&acc)[RT][CT]) {
+  constexpr int NCOLS = 16 * CT;
+  constexpr int NB = 16 * RT;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  float* base = red + wave * NB * NCOLS;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      const int col = ct * 16 + (lane & 15);
+      const int r0 = rt * 16 + (lane >> 4) * 4;
+      base[(r0 + 0) * NCOLS + col] = acc[rt][ct].x;
+      base[(r0 + 1) * NCOLS + col] = acc[rt][ct].y;
+      base[(r0 + 2) * NCOLS + col] = acc[rt][ct].z;
+      base[(r0 + 3) * NCOLS + col] = acc[rt][ct].w;
+    }
+}
+
+// Sum over the four wavefronts of element (row, col) written by store_partials.
+template <int RT, int CT>
+__device__ __forceinline__ float sum_partials(const float* red, int row, int col) {
+  constexpr int NCOLS = 16 * CT;
+  constexpr int NB = 16 * RT;
+  const float* p = red + row * NCOLS + col;
+  return (p[0] + p[NB * NCOLS]) + (p[2 * NB * NCOLS] + p[3 * NB * NCOLS]);
+}
+
+}  // namespace haste_hip

@@ -1,0 +1,139 @@
+// Library runtime: version, error text, and the per-(device, stream) workspace cache.
+#include "common.h"
+
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <utility>
+
+namespace haste_hip {
+
+namespace {
+
+thread_local std::string g_last_error;
+
+struct Key {
+  int device;
+  hipStream_t stream;
+  bool operator<(const Key& o) const {
+    return device != o.device ? device < o.device : stream < o.stream;
+  }
+};
+
+std::mutex g_mutex;
+std::map<Key, Workspace> g_workspaces;
+std::map<int, int> g_cu_count;
+
+// Clears a range of device words with a kernel rather than a memset node, so that
+// callers may record the library's work into a HIP graph.
+__global__ void fill_zero_kernel(unsigned int* p, size_t n) {
+  size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
+}  // namespace
+
+void set_runtime_error(hipError_t err, const char* what) {
+  char buf[512];
+  std::snprintf(buf, sizeof(buf), "%s: %s (%d)", what, hipGetErrorString(err), (int)err);
+  g_last_error = buf;
+  (void)hipGetLastError();  // do not leave the error for an unrelated later call
+}
+
+int device_cu_count() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  auto it = g_cu_count.find(dev);
+  if (it != g_cu_count.end()) return it->second;
+  int n = 0;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
+  g_cu_count[dev] = n;
+  return n;
+}
+
+int get_workspace(hipStream_t stream, size_t scratch_bytes, Workspace* out) {
+  int dev = 0;
+  HASTE_HIP_TRY(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_mutex);
+  Workspace& ws = g_workspaces[Key{dev, stream}];
+  if (ws.control == nullptr) {
+    HASTE_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&ws.control), sizeof(ControlBlock)));
+    const size_t words = sizeof(ControlBlock) / sizeof(unsigned int);
+    fill_zero_kernel<<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream>>>(
+        reinterpret_cast<unsigned int*>(ws.control), words);
+    HASTE_HIP_TRY(hipGetLastError());
+    HASTE_HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&ws.host_status), 64,
+                                hipHostMallocMapped));
+    std::memset(ws.host_status, 0, 64);
+    HASTE_HIP_TRY(hipHostGetDevicePointer(reinterpret_cast<void**>(&ws.host_status_dev),
+                                          ws.host_status, 0));
+  }
+  if (ws.scratch_bytes < scratch_bytes) {
+    // Growing replaces the buffer; work already enqueued on the stream may still be
+    // using the old one, so the stream is drained first (rare: sizes stabilise
+    // after the first call of each shape).
+    if (ws.scratch != nullptr) {
+      HASTE_HIP_TRY(hipStreamSynchronize(stream));
+      HASTE_HIP_TRY(hipFree(ws.scratch));
+      ws.scratch = nullptr;
+      ws.scratch_bytes = 0;
+    }
+    size_t bytes = (scratch_bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+    HASTE_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&ws.scratch), bytes));
+    ws.scratch_bytes = bytes;
+  }
+  *out = ws;
+  return HASTE_HIP_OK;
+}
+
+int check_and_clear_abort(hipStream_t stream, Workspace* ws) {
+  volatile unsigned int* status = ws->host_status;
+  if (status == nullptr || *status == 0u) return HASTE_HIP_OK;
+  *status = 0u;
+  const size_t words = sizeof(ControlBlock) / sizeof(unsigned int);
+  fill_zero_kernel<<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream>>>(
+      reinterpret_cast<unsigned int*>(ws->control), words);
+  HASTE_HIP_TRY(hipGetLastError());
+  return HASTE_HIP_ERROR_STEP_BARRIER;
+}
+
+}  // namespace haste_hip
+
+extern "C" {
+
+int haste_hip_version(void) { return 100; }  // 0.1.0
+
+const char* haste_hip_error_string(int code) {
+  switch (code) {
+    case HASTE_HIP_OK: return "ok";
+    case HASTE_HIP_ERROR_INVALID_ARGUMENT: return "invalid argument (null pointer or non-positive dimension)";
+    case HASTE_HIP_ERROR_UNSUPPORTED_SIZE: return "unsupported size (recurrent weight slice does not fit on chip or batch too large for one cooperative grid)";
+    case HASTE_HIP_ERROR_RUNTIME: return "HIP runtime error";
+    case HASTE_HIP_ERROR_STEP_BARRIER: return "a persistent kernel launched earlier timed out at its step barrier";
+    default: return "unknown error code";
+  }
+}
+
+const char* haste_hip_last_runtime_error(void) { return haste_hip::g_last_error.c_str(); }
+
+int haste_hip_release_workspaces(void) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return HASTE_HIP_ERROR_RUNTIME;
+  std::lock_guard<std::mutex> lock(haste_hip::g_mutex);
+  for (auto it = haste_hip::g_workspaces.begin(); it != haste_hip::g_workspaces.end();) {
+    if (it->first.device == dev) {
+      if (it->second.scratch) (void)hipFree(it->second.scratch);
+      if (it->second.control) (void)hipFree(it->second.control);
+      if (it->second.host_status) (void)hipHostFree(it->second.host_status);
+      it = haste_hip::g_workspaces.erase(it);
+    } else {
+      ++it;
+    }
+  }
+  return HASTE_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,83 @@
+"""Op-level interface: the functions the reference exposes from its PyTorch binding
+(`haste_pytorch_lib.<cell>_forward / <cell>_backward`, reference
+frameworks/pytorch/{lstm,gru,indrnn,layer_norm_lstm,layer_norm_gru,layer_norm_indrnn}.cc),
+with the same argument order, allocation protocol and return tuples, implemented by
+calls into libhaste_hip.so.  Tensors are float32, contiguous, on the GPU; torch is
+used only to allocate device memory and to name the current stream.
+"""
+import torch
+
+from . import lib
+
+
+def _check(*tensors):
+    # reference frameworks/pytorch/support.h:20-22 (CHECK_INPUT)
+    for t in tensors:
+        if not t.is_cuda:
+            raise ValueError("tensor must be a GPU tensor")
+        if not t.is_contiguous():
+            raise ValueError("tensor must be contiguous")
+        if t.dtype != torch.float32:
+            raise ValueError("only float32 is implemented")
+
+
+def _mask_or_none(has_zoneout, zoneout_mask):
+    return zoneout_mask if has_zoneout else None
+
+
+def gemm(a, b, out=None, trans_a=False, accumulate=False):
+    """out[M,N] = op(a) @ b (+ out). a is [M,K], or [K,M] when trans_a."""
+    _check(a, b)
+    K, M = (a.shape if trans_a else (a.shape[1], a.shape[0]))
+    N = b.shape[1]
+    assert b.shape[0] == K
+    if out is None:
+        assert not accumulate
+        out = torch.empty(M, N, device=a.device, dtype=a.dtype)
+    lib.call("haste_hip_gemm_f32", int(trans_a), M, N, K, a, a.stride(0), b, b.stride(0),
+             out, out.stride(0), int(accumulate))
+    return out
+
+
+# ---- LSTM (reference frameworks/pytorch/lstm.cc:31-157) ---------------------
+def lstm_forward(training, zoneout_prob, x, h0, c0, kernel, recurrent_kernel, bias, zoneout_mask,
+                 dropconnect_mask=None, dropconnect_scale=1.0):
+    T, N, C = x.shape
+    H = recurrent_kernel.shape[0]
+    has_zoneout = bool(zoneout_prob) and zoneout_mask.numel() > 0
+    _check(x, h0, c0, kernel, recurrent_kernel, bias, zoneout_mask)
+    opts = dict(device=x.device, dtype=x.dtype)
+    output = torch.empty(T + 1, N, H, **opts)
+    output_state = torch.empty(T + 1, N, H, **opts)
+    cache = torch.empty(T, N, 4 * H, **opts)
+    output[0] = h0
+    output_state[0] = c0
+    zp = float(zoneout_prob) if has_zoneout else 0.0
+    mask = _mask_or_none(has_zoneout, zoneout_mask)
+    if dropconnect_mask is None:
+        lib.call("haste_hip_lstm_forward_f32", bool(training), T, N, C, H, kernel, recurrent_kernel,
+                 bias, x, output, output_state, cache, None, zp, mask)
+    else:
+        _check(dropconnect_mask)
+        lib.call("haste_hip_lstm_forward_dropconnect_f32", bool(training), T, N, C, H, kernel,
+                 recurrent_kernel, bias, x, output, output_state, cache, zp, mask,
+                 dropconnect_mask, float(dropconnect_scale))
+    return output, output_state, cache
+
+
+def lstm_backward(x_t, kernel_t, recurrent_kernel_t, bias, zoneout_mask, h, c, cache, dh_new, dc_new):
+    C, T, N = x_t.shape
+    H = recurrent_kernel_t.shape[1]
+    has_zoneout = zoneout_mask.numel() > 0
+    _check(x_t, kernel_t, recurrent_kernel_t, bias, zoneout_mask, h, c, cache, dh_new, dc_new)
+    opts = dict(device=x_t.device, dtype=x_t.dtype)
+    dx = torch.empty(T, N, C, **opts)
+    dW = torch.zeros(C, 4 * H, **opts)
+    dR = torch.zeros(H, 4 * H, **opts)
+    db = torch.zeros(4 * H, **opts)
+    dh = torch.zeros(N, H, **opts)
+    dc = torch.zeros(N, H, **opts)
+    lib.call("haste_hip_lstm_backward_f32", T, N, C, H, kernel_t, recurrent_kernel_t, bias, x_t,
+             h, c, dh_new, dc_new, dx, dW, dR, db, dh, dc, cache,
+             _mask_or_none(has_zoneout, zoneout_mask))
+    return dx, dh, dc, dW, dR, db

@@ -1,0 +1,239 @@
+/* C ABI of libhaste_hip.so: the MI355X (gfx950) implementation of the fused-RNN
+ * hot path behind the libhaste C++ API.
+ *
+ * Every entry point takes plain ints, floats and device pointers; `stream` is a
+ * hipStream_t passed as void* (NULL = the null stream).  All work is enqueued on
+ * that stream and the call returns without waiting for it.  All tensors are
+ * caller-allocated device memory, row-major, rightmost index fastest
+ * (T steps, N batch, C input size, H hidden size), exactly as the reference
+ * documents them in lib/haste.h:18-26.  Return value: 0 on success, otherwise one
+ * of the HASTE_HIP_ERROR_* codes; nothing is launched when an argument check fails.
+ *
+ * Each *_forward / *_backward entry point is what the corresponding
+ * haste::v0::<cell>::ForwardPass<float>::Run / BackwardPass<float>::Run binds to
+ * (see include/haste/ *.h for the header-only C++ adapters).
+ */
+#ifndef HASTE_HIP_H_
+#define HASTE_HIP_H_
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HASTE_HIP_OK 0
+#define HASTE_HIP_ERROR_INVALID_ARGUMENT 1  /* null pointer, non-positive dimension */
+#define HASTE_HIP_ERROR_UNSUPPORTED_SIZE 2  /* recurrent slice does not fit on chip / in the grid */
+#define HASTE_HIP_ERROR_RUNTIME 3           /* a HIP runtime call failed */
+#define HASTE_HIP_ERROR_STEP_BARRIER 4      /* an earlier persistent kernel gave up waiting at its step barrier */
+
+/* Library version as major*10000 + minor*100 + patch. */
+int haste_hip_version(void);
+
+/* Human-readable text for a return code. */
+const char* haste_hip_error_string(int code);
+
+/* Text of the last HIP runtime error seen by the calling thread ("" if none). */
+const char* haste_hip_last_runtime_error(void);
+
+/* Largest hidden size whose recurrent weight slice the persistent kernels can keep
+ * on chip for `gates` gate blocks (4 LSTM, 3 GRU) and `batch_size` rows on the
+ * current device; 0 if none. */
+int haste_hip_max_hidden_size(int gates, int batch_size);
+
+/* Drops this thread's cached per-stream workspaces on the current device (frees
+ * device memory; the caller must have synchronized the streams that used them). */
+int haste_hip_release_workspaces(void);
+
+/* C[M,N] = op(A)[M,K] * B[K,N] (+ C if accumulate != 0); fp32 MFMA.
+ * trans_a == 0: A is [M,K] with leading dimension lda; trans_a != 0: A is stored
+ * as [K,M] with leading dimension lda.  Replaces the cuBLAS calls the reference
+ * makes through lib/blas.h:48-61. */
+int haste_hip_gemm_f32(int trans_a, int M, int N, int K,
+                       const float* A, int lda, const float* B, int ldb,
+                       float* C, int ldc, int accumulate, void* stream);
+
+/* ---- LSTM ----------------------------------------------------------------
+ * reference lib/haste/lstm.h:118-129 (ForwardPass::Run), lib/lstm_forward_gpu.cu.cc:313-366.
+ * W[C,4H] R[H,4H] b[4H] x[T,N,C] h,c[T+1,N,H] (slot 0 preset by the caller)
+ * v[T,N,4H] (training: activations i,g,f,o on return) tmp_Rh[N,4H] (unused scratch,
+ * may be NULL) zoneout_mask[T,N,H] or NULL. */
+int haste_hip_lstm_forward_f32(int training, int steps, int batch_size, int input_size,
+                               int hidden_size,
+                               const float* W, const float* R, const float* b, const float* x,
+                               float* h, float* c, float* v, float* tmp_Rh,
+                               float zoneout_prob, const float* zoneout_mask, void* stream);
+
+/* Same, with DropConnect fused into the load of R: the recurrence uses
+ * R[i] * dropconnect_mask[i] * dropconnect_scale.  The reference applies this in
+ * Python before calling the op (frameworks/pytorch/lstm.py:252); mask NULL = plain R. */
+int haste_hip_lstm_forward_dropconnect_f32(int training, int steps, int batch_size,
+                                           int input_size, int hidden_size,
+                                           const float* W, const float* R, const float* b,
+                                           const float* x, float* h, float* c, float* v,
+                                           float zoneout_prob, const float* zoneout_mask,
+                                           const float* dropconnect_mask, float dropconnect_scale,
+                                           void* stream);
+
+/* reference lib/haste/lstm.h:248-265 (BackwardPass::Run), lib/lstm_backward_gpu.cu.cc:319-405.
+ * W_t[4H,C] R_t[4H,H] b[4H] (unused) x_t[C,T,N] h,c[T+1,N,H] dh_new,dc_new[T+1,N,H]
+ * dx[T,N,C] (assigned) dW[C,4H] dR[H,4H] db[4H] (accumulated into) dh,dc[N,H] (in/out,
+ * zero on entry, d h0 / d c0 on return) v[T,N,4H] (in: activations, out: gate gradients)
+ * zoneout_mask[T,N,H] or NULL. */
+int haste_hip_lstm_backward_f32(int steps, int batch_size, int input_size, int hidden_size,
+                                const float* W_t, const float* R_t, const float* b,
+                                const float* x_t, const float* h, const float* c,
+                                const float* dh_new, const float* dc_new,
+                                float* dx, float* dW, float* dR, float* db,
+                                float* dh, float* dc, float* v,
+                                const float* zoneout_mask, void* stream);
+
+/* ---- GRU -------------------------------------------------------------------
+ * reference lib/haste/gru.h:86-98, lib/gru_forward_gpu.cu.cc:314-371.
+ * W[C,3H] R[H,3H] bx,br[3H] x[T,N,C] h[T+1,N,H] v[T,N,4H] = (z,r,g,Rh_g+br_g)
+ * (training only; may be NULL otherwise) tmp_Wx[T,N,3H] tmp_Rh[N,3H] (unused, may be NULL). */
+int haste_hip_gru_forward_f32(int training, int steps, int batch_size, int input_size,
+                              int hidden_size,
+                              const float* W, const float* R, const float* bx, const float* br,
+                              const float* x, float* h, float* v, float* tmp_Wx, float* tmp_Rh,
+                              float zoneout_prob, const float* zoneout_mask, void* stream);
+
+/* GRU forward with DropConnect fused into the load of R (frameworks/pytorch/gru.py:257). */
+int haste_hip_gru_forward_dropconnect_f32(int training, int steps, int batch_size,
+                                          int input_size, int hidden_size,
+                                          const float* W, const float* R, const float* bx,
+                                          const float* br, const float* x, float* h, float* v,
+                                          float* tmp_Wx, float zoneout_prob,
+                                          const float* zoneout_mask,
+                                          const float* dropconnect_mask, float dropconnect_scale,
+                                          void* stream);
+
+/* reference lib/haste/gru.h:191-209, lib/gru_backward_gpu.cu.cc:321-409.
+ * dp,dq[T,N,3H] are outputs/scratch; dbx,dbr,dW,dR accumulated; dx assigned; dh in/out. */
+int haste_hip_gru_backward_f32(int steps, int batch_size, int input_size, int hidden_size,
+                               const float* W_t, const float* R_t, const float* bx,
+                               const float* br, const float* x_t, const float* h, const float* v,
+                               const float* dh_new, float* dx, float* dW, float* dR,
+                               float* dbx, float* dbr, float* dh, float* dp, float* dq,
+                               const float* zoneout_mask, void* stream);
+
+/* ---- Layer norm --------------------------------------------------------------
+ * reference lib/haste/layer_norm.h:30-49, lib/layer_norm_forward_gpu.cu.cc:96-150.
+ * y = (x-mean)*invstd*gamma (+beta if non-NULL), eps 1e-5, biased variance;
+ * cache[rows,2] = (mean, invstd) (may be NULL). */
+int haste_hip_layer_norm_forward_f32(int rows, int dim, const float* gamma, const float* beta,
+                                     const float* x, float* y, float* cache, void* stream);
+
+/* reference lib/haste/layer_norm.h:63-79, lib/layer_norm_backward_gpu.cu.cc:101-165.
+ * dx may alias dy.  dgamma (and dbeta if non-NULL) are accumulated into.  Statistics
+ * are recomputed from x; `cache` is accepted for signature parity and not read. */
+int haste_hip_layer_norm_backward_f32(int rows, int dim, const float* gamma, const float* x,
+                                      const float* dy, float* dx, float* dgamma, float* dbeta,
+                                      const float* cache, void* stream);
+
+/* ---- LayerNorm LSTM ----------------------------------------------------------
+ * reference lib/haste/layer_norm_lstm.h:75-92, lib/layer_norm_lstm_forward_gpu.cu.cc:276-340.
+ * The three layer_norm::ForwardPass objects of the reference are passed flattened:
+ * ln1 (on xW, rows T*N, dim 4H): gamma1[4H], cache1[T*N,2];
+ * ln2 (on hR per step):          gamma2[4H], cache2[T*N,2];
+ * ln3 (on c per step, dim H):    gamma_h[H], beta_h[H], cache3[T*N,2]. */
+int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_size,
+                                          int input_size, int hidden_size,
+                                          const float* W, const float* R, const float* b,
+                                          const float* x, float* h, float* c,
+                                          float* act_Wx, float* tmp_Rh,
+                                          const float* gamma1, float* cache1,
+                                          float* act_Wx_norm, float* act_Rh,
+                                          const float* gamma2, float* cache2,
+                                          const float* gamma_h, const float* beta_h, float* cache3,
+                                          float* act_c_norm,
+                                          float zoneout_prob, const float* zoneout_mask,
+                                          void* stream);
+
+/* reference lib/haste/layer_norm_lstm.h:160-183, lib/layer_norm_lstm_backward_gpu.cu.cc:255-352.
+ * act_Wx, act_Wx_norm, act_Rh, act_c_norm are consumed (overwritten with gradients).
+ * dgamma1, dgamma2 [4H], dgamma_h, dbeta_h [H] are accumulated into. */
+int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_size,
+                                           int hidden_size,
+                                           const float* W_t, const float* R_t, const float* b,
+                                           const float* x_t, const float* h, const float* c,
+                                           const float* dh_new, const float* dc_new,
+                                           float* dx, float* dW, float* dR, float* db,
+                                           float* dh, float* dc,
+                                           float* act_Wx, const float* gamma1, float* dgamma1,
+                                           float* act_Wx_norm, float* act_Rh,
+                                           const float* gamma2, float* dgamma2,
+                                           const float* gamma_h, const float* beta_h,
+                                           float* dgamma_h, float* dbeta_h,
+                                           float* act_c_norm,
+                                           const float* zoneout_mask, void* stream);
+
+/* ---- LayerNorm GRU -----------------------------------------------------------
+ * reference lib/haste/layer_norm_gru.h:72-88, lib/layer_norm_gru_forward_gpu.cu.cc:242-305. */
+int haste_hip_layer_norm_gru_forward_f32(int training, int steps, int batch_size,
+                                         int input_size, int hidden_size,
+                                         const float* W, const float* R, const float* bx,
+                                         const float* br, const float* x, float* h, float* v,
+                                         float* act_Wx, const float* gamma1, float* cache1,
+                                         float* tmp_Wx_norm, float* act_Rh,
+                                         const float* gamma2, float* cache2, float* tmp_Rh_norm,
+                                         float zoneout_prob, const float* zoneout_mask,
+                                         void* stream);
+
+/* reference lib/haste/layer_norm_gru.h:164-184, lib/layer_norm_gru_backward_gpu.cu.cc:219-310.
+ * act_Wx / act_Rh are the pre-norm activations saved by the forward pass (the `x` of the
+ * reference's layer_norm1 / layer_norm2 BackwardPass objects). dp, dq are overwritten
+ * with the gradients w.r.t. the pre-norm activations, as in the reference. */
+int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_size,
+                                          int hidden_size,
+                                          const float* W_t, const float* R_t, const float* bx,
+                                          const float* br, const float* x_t, const float* h,
+                                          const float* v, const float* dh_new,
+                                          float* dx, float* dW, float* dR, float* dbx, float* dbr,
+                                          float* dh, float* dp, float* dq,
+                                          const float* act_Wx, const float* gamma1, float* dgamma1,
+                                          const float* act_Rh, const float* gamma2, float* dgamma2,
+                                          const float* zoneout_mask, void* stream);
+
+/* ---- IndRNN --------------------------------------------------------------------
+ * reference lib/haste/indrnn.h:37-47, lib/indrnn_forward_gpu.cu.cc:114-210.
+ * W[C,H] u[H] b[H] x[T,N,C] h[T+1,N,H] workspace[T,N,H]. */
+int haste_hip_indrnn_forward_f32(int training, int steps, int batch_size, int input_size,
+                                 int hidden_size,
+                                 const float* W, const float* u, const float* b, const float* x,
+                                 float* h, float* workspace,
+                                 float zoneout_prob, const float* zoneout_mask, void* stream);
+
+/* reference lib/haste/indrnn.h:66-80, lib/indrnn_backward_gpu.cu.cc:122-207.
+ * dW[C,H] and dx are assigned; du, db accumulated; dh in/out; workspace[T,N,H] out. */
+int haste_hip_indrnn_backward_f32(int steps, int batch_size, int input_size, int hidden_size,
+                                  const float* W_t, const float* u, const float* b,
+                                  const float* x_t, const float* h, const float* dh_new,
+                                  float* dx, float* dW, float* du, float* db, float* dh,
+                                  float* workspace, const float* zoneout_mask, void* stream);
+
+/* ---- LayerNorm IndRNN ----------------------------------------------------------
+ * reference lib/haste/layer_norm_indrnn.h:37-49, lib/layer_norm_indrnn_forward_gpu.cu.cc:114-213. */
+int haste_hip_layer_norm_indrnn_forward_f32(int training, int steps, int batch_size,
+                                            int input_size, int hidden_size,
+                                            const float* W, const float* u, const float* b,
+                                            const float* x, float* h, float* workspace,
+                                            float* act_Wx, const float* gamma1, float* cache1,
+                                            float zoneout_prob, const float* zoneout_mask,
+                                            void* stream);
+
+/* reference lib/haste/layer_norm_indrnn.h:68-83, lib/layer_norm_indrnn_backward_gpu.cu.cc:122-209. */
+int haste_hip_layer_norm_indrnn_backward_f32(int steps, int batch_size, int input_size,
+                                             int hidden_size,
+                                             const float* W_t, const float* u, const float* b,
+                                             const float* x_t, const float* h,
+                                             const float* dh_new,
+                                             float* dx, float* dW, float* du, float* db, float* dh,
+                                             float* workspace,
+                                             const float* act_Wx, const float* gamma1,
+                                             float* dgamma1,
+                                             const float* zoneout_mask, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif  /* HASTE_HIP_H_ */

@@ -1,0 +1,50 @@
+"""fp32 MFMA GEMM vs fp64 NumPy matmul, through the C-ABI (haste_hip_gemm_f32)."""
+import numpy as np
+import pytest
+
+from util import dev, host, relerr
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [
+    # (trans_a, M, N, K)
+    (False, 128, 128, 16), (False, 256, 384, 64), (False, 100, 200, 50), (False, 1, 1, 1),
+    (False, 37, 53, 29), (True, 128, 128, 32), (True, 70, 130, 45), (True, 5, 20, 33),
+    (False, 6400, 2048, 512),   # x*W of the metric config
+    (False, 512, 2048, 6400),   # dW: split along K
+    (True, 512, 2048, 6400),    # dR: split along K, A = h^T
+    (False, 6400, 512, 2048),   # dx
+    (False, 96, 96, 5000),      # split-K with ragged tiles
+]
+
+
+@pytest.mark.parametrize("trans_a,M,N,K", SHAPES)
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_gemm_matches_numpy(trans_a, M, N, K, accumulate):
+    from haste_amd import ops
+    import torch
+    r = np.random.default_rng(M * 7 + N * 3 + K)
+    a = r.standard_normal((K, M) if trans_a else (M, K)).astype(np.float32)
+    b = r.standard_normal((K, N)).astype(np.float32)
+    c0 = r.standard_normal((M, N)).astype(np.float32)
+    print("gemm", trans_a, M, N, K, accumulate, flush=True)
+    out = dev(c0)
+    ops.gemm(dev(a), dev(b), out=out, trans_a=trans_a, accumulate=accumulate)
+    torch.cuda.synchronize()
+    a64 = a.astype(np.float64)
+    ref = (a64.T if trans_a else a64) @ b.astype(np.float64)
+    if accumulate:
+        ref = ref + c0
+    assert relerr(host(out), ref) < 1e-5  # fp32 accumulation over K up to 6400
+
+
+def test_gemm_split_k_is_run_to_run_identical():
+    from haste_amd import ops
+    import torch
+    r = np.random.default_rng(5)
+    a = dev(r.standard_normal((512, 6400)))
+    b = dev(r.standard_normal((6400, 2048)))
+    o1 = ops.gemm(a, b)
+    o2 = ops.gemm(a, b)
+    torch.cuda.synchronize()
+    assert torch.equal(o1, o2)

@@ -1,0 +1,90 @@
+"""LSTM forward/backward on the GPU (through the C-ABI) vs the fp64 oracle."""
+import numpy as np
+import pytest
+
+from oracle import haste_oracle as O
+from util import TOL, dev, host, problem, relerr
+
+pytestmark = pytest.mark.gpu
+
+# (T, N, C, H): tiny, ragged (sizes that are not multiples of any tile), and config-like
+SHAPES = [(1, 1, 1, 1), (3, 2, 3, 4), (5, 3, 7, 5), (6, 17, 20, 36), (4, 16, 32, 64),
+          (10, 33, 48, 128), (8, 64, 64, 256), (12, 16, 128, 256), (6, 128, 96, 512)]
+
+
+def run_lstm(p, training, zoneout_prob, T, N, C, H):
+    from haste_amd import ops
+    import torch
+    mask = dev(p["mask"])
+    h, c, cache = ops.lstm_forward(training, zoneout_prob, dev(p["x"]), dev(p["h0"]), dev(p["c0"]),
+                                   dev(p["W"]), dev(p["R"]), dev(p["b"]), mask)
+    torch.cuda.synchronize()
+    return h, c, cache, mask
+
+
+@pytest.mark.parametrize("zoneout", [0.0, 0.3])
+@pytest.mark.parametrize("T,N,C,H", SHAPES)
+def test_lstm_training_forward_backward(T, N, C, H, zoneout):
+    from haste_amd import ops
+    import torch
+    print("lstm fwd+bwd", T, N, C, H, zoneout, flush=True)
+    p = problem(100 + T + N + C + H, T, N, C, H, 4, zoneout)
+    h, c, cache, mask = run_lstm(p, True, zoneout, T, N, C, H)
+    ho, co, vo = O.lstm_forward(p["W"], p["R"], p["b"], p["x"], p["h0"], p["c0"], True, zoneout, p["mask"])
+    assert relerr(host(h), ho) < TOL
+    assert relerr(host(c), co) < TOL
+    assert relerr(host(cache), vo) < TOL
+
+    x_t = dev(p["x"]).permute(2, 0, 1).contiguous()
+    W_t = dev(p["W"]).t().contiguous()
+    R_t = dev(p["R"]).t().contiguous()
+    dx, dh, dc, dW, dR, db = ops.lstm_backward(x_t, W_t, R_t, dev(p["b"]), mask, h, c, cache,
+                                               dev(p["dh_new"]), dev(p["dc_new"]))
+    torch.cuda.synchronize()
+    ref = O.lstm_backward(p["W"], p["R"], p["b"], p["x"], ho, co, vo, p["dh_new"], p["dc_new"], p["mask"])
+    for name, ours, theirs in zip(("dx", "dW", "dR", "db", "dh0", "dc0", "dv"),
+                                  (dx, dW, dR, db, dh, dc, cache), ref):
+        assert relerr(host(ours), theirs) < TOL, name
+
+
+@pytest.mark.parametrize("zoneout", [0.0, 0.25])
+def test_lstm_inference_forward(zoneout):
+    T, N, C, H = 20, 16, 128, 256
+    p = problem(7, T, N, C, H, 4, zoneout)
+    h, c, _, _ = run_lstm(p, False, zoneout, T, N, C, H)
+    ho, co, _ = O.lstm_forward(p["W"], p["R"], p["b"], p["x"], p["h0"], p["c0"], False, zoneout, p["mask"])
+    assert relerr(host(h), ho) < TOL
+    assert relerr(host(c), co) < TOL
+
+
+def test_lstm_dropconnect_fused_equals_premasked_weights():
+    from haste_amd import ops
+    import torch
+    T, N, C, H = 6, 8, 16, 64
+    p = problem(9, T, N, C, H, 4)
+    r = np.random.default_rng(3)
+    m = (r.uniform(size=p["R"].shape) >= 0.05).astype(np.float64)
+    scale = 1.0 / 0.95
+    args = (True, 0.0, dev(p["x"]), dev(p["h0"]), dev(p["c0"]), dev(p["W"]))
+    h1, c1, v1 = ops.lstm_forward(*args, dev(p["R"]), dev(p["b"]), dev(None),
+                                  dropconnect_mask=dev(m), dropconnect_scale=scale)
+    R_eff = (dev(p["R"]) * dev(m)) * np.float32(scale)
+    h2, c2, v2 = ops.lstm_forward(*args, R_eff.contiguous(), dev(p["b"]), dev(None))
+    torch.cuda.synchronize()
+    assert torch.equal(h1, h2) and torch.equal(c1, c2) and torch.equal(v1, v2)
+
+
+def test_lstm_accumulates_into_weight_gradients_and_is_deterministic():
+    from haste_amd import ops
+    import torch
+    T, N, C, H = 7, 32, 24, 64
+    p = problem(11, T, N, C, H, 4, 0.2)
+    outs = []
+    for _ in range(2):
+        h, c, cache, mask = run_lstm(p, True, 0.2, T, N, C, H)
+        x_t = dev(p["x"]).permute(2, 0, 1).contiguous()
+        outs.append(ops.lstm_backward(x_t, dev(p["W"]).t().contiguous(), dev(p["R"]).t().contiguous(),
+                                      dev(p["b"]), mask, h, c, cache, dev(p["dh_new"]), dev(p["dc_new"])))
+    torch.cuda.synchronize()
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
