@@ -1,0 +1,197 @@
+"""Benchmark of the hot path on one MI355X.
+
+Metric (BASELINE.json): LSTM forward + backward, ms per batch, at N=64, T=100,
+C=H=512, fp32; plus microseconds per timestep of streaming inference at N=1, T=2000.
+
+One step = ForwardPass::Run (training) + the caller-side transposes of x, W, R +
+BackwardPass::Run, as the reference's benchmark times it
+(benchmarks/benchmark_lstm.cc:399-465).  Inputs are synthetic, seeded, and resident in
+HBM before the timed region.  Prints one JSON line.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-budget", type=float, default=15.0)
+    return ap.parse_args()
+
+
+def make_inputs(T, N, C, H, seed=0, forget_bias=1.0):
+    r = np.random.default_rng(seed)
+    k = 1.0 / np.sqrt(H)
+    W = r.uniform(-k, k, (C, 4 * H)).astype(np.float32)
+    R = r.uniform(-k, k, (H, 4 * H)).astype(np.float32)
+    b = np.zeros(4 * H, np.float32)
+    b[2 * H:3 * H] = forget_bias
+    x = r.standard_normal((T, N, C)).astype(np.float32)
+    dy = r.standard_normal((T, N, H)).astype(np.float32)
+    dhT = r.standard_normal((N, H)).astype(np.float32)
+    dcT = r.standard_normal((N, H)).astype(np.float32)
+    return W, R, b, x, dy, dhT, dcT
+
+
+def profile_read(lib, name):
+    total = ctypes.c_double(0.0)
+    count = ctypes.c_int(0)
+    rc = lib.haste_hip_profile_read(name.encode(), ctypes.byref(total), ctypes.byref(count))
+    if rc != 0:
+        raise RuntimeError("haste_hip_profile_read failed: %d" % rc)
+    return total.value, count.value
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the path has no multi-GPU component "
+              "(got --gpus %d)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from haste_amd import lib as hlib, ops
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    lib = hlib.load()
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+
+    # ---- metric config: LSTM fwd+bwd N=64 T=100 C=H=512 -----------------------
+    T, N, C, H = 100, 64, 512, 512
+    W, R, b, x, dy, dhT, dcT = make_inputs(T, N, C, H)
+    Wd, Rd, bd, xd = (torch.from_numpy(a).to(dev) for a in (W, R, b, x))
+    h0 = torch.zeros(N, H, device=dev)
+    c0 = torch.zeros(N, H, device=dev)
+    dh_new = torch.zeros(T + 1, N, H, device=dev)
+    dh_new[1:] = torch.from_numpy(dy).to(dev)
+    dh_new[T] += torch.from_numpy(dhT).to(dev)
+    dc_new = torch.zeros(T + 1, N, H, device=dev)
+    dc_new[T] = torch.from_numpy(dcT).to(dev)
+    no_mask = torch.empty(0, 0, 0, device=dev)
+
+    def step():
+        h, c, cache = ops.lstm_forward(True, 0.0, xd, h0, c0, Wd, Rd, bd, no_mask)
+        x_t = xd.permute(2, 0, 1).contiguous()
+        W_t = Wd.t().contiguous()
+        R_t = Rd.t().contiguous()
+        return ops.lstm_backward(x_t, W_t, R_t, bd, no_mask, h, c, cache, dh_new, dc_new)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(args.steps):
+        step()
+    ev1.record()
+    torch.cuda.synchronize()
+    ms_per_step = ev0.elapsed_time(ev1) / args.steps
+
+    # Same K steps again with per-kernel event timing switched on in the library.
+    lib.haste_hip_profile_reset()
+    lib.haste_hip_profile_enable(1)
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    lib.haste_hip_profile_enable(0)
+    f_gemm = 2.0 * T * N * C * 4 * H  # each of the 4 GEMMs (C == H)
+    f_rec = 2.0 * T * N * H * 4 * H
+    kernels = {}
+    for name, flops in (("gemm_f32", f_gemm), ("lstm_forward_recurrence", f_rec),
+                        ("lstm_backward_recurrence", f_rec)):
+        total_ms, count = profile_read(lib, name)
+        avg_ms = total_ms / max(count, 1)
+        kernels[name] = {"launches_per_step": count / args.steps, "avg_ms": round(avg_ms, 5),
+                         "ms_per_step": round(total_ms / args.steps, 5),
+                         "tflops": round(flops / (avg_ms * 1e-3) / 1e12, 3) if avg_ms > 0 else None}
+    lib.haste_hip_profile_reset()
+    dominant = max(kernels, key=lambda k: kernels[k]["ms_per_step"])
+    dom = kernels[dominant]
+    roofline = {"kernel": dominant, "bound": "mfma", "achieved": dom["tflops"],
+                "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(dom["tflops"] / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None}
+    total_flops = 3.0 * (2.0 * T * N * C * 4 * H + f_rec)
+
+    # ---- streaming inference: N=1 T=2000 C=H=512, microseconds per timestep -----
+    T1, N1 = 2000, 1
+    W1, R1, b1, x1, *_ = make_inputs(T1, N1, C, H, seed=1, forget_bias=0.0)
+    W1d, R1d, b1d, x1d = (torch.from_numpy(a).to(dev) for a in (W1, R1, b1, x1))
+    h01 = torch.zeros(N1, H, device=dev)
+    c01 = torch.zeros(N1, H, device=dev)
+
+    def stream_step():
+        return ops.lstm_forward(False, 0.0, x1d, h01, c01, W1d, R1d, b1d, no_mask)
+
+    for _ in range(3):
+        stream_step()
+    torch.cuda.synchronize()
+    lib.haste_hip_profile_enable(1)
+    reps = 10
+    ev0.record()
+    for _ in range(reps):
+        stream_step()
+    ev1.record()
+    torch.cuda.synchronize()
+    lib.haste_hip_profile_enable(0)
+    us_per_step_total = ev0.elapsed_time(ev1) * 1e3 / reps / T1
+    rec_ms, rec_n = profile_read(lib, "lstm_forward_recurrence")
+    lib.haste_hip_profile_reset()
+    us_per_step_rec = rec_ms * 1e3 / max(rec_n, 1) / T1
+    b_step = 4.0 * (4 * H * H + 2 * 4 * H + 4 * H)  # R + Wx_t + b + h,c in + h,c out
+    stream_gbs = b_step / (us_per_step_rec * 1e-6) / 1e9
+    streaming = {"workload": "LSTM inference N=1 T=2000 C=H=512 fp32",
+                 "us_per_timestep": round(us_per_step_total, 4),
+                 "us_per_timestep_recurrence_kernel": round(us_per_step_rec, 4),
+                 "roofline": {"bound": "hbm", "achieved": round(stream_gbs, 1), "peak": PEAK_HBM_GBS,
+                              "unit": "GB/s", "frac": round(stream_gbs / PEAK_HBM_GBS, 4),
+                              "bytes_per_step_model": b_step,
+                              "note": "streamed-R byte model; R is kept on chip, so this is an "
+                                      "equivalent bandwidth, not HBM traffic"}}
+
+    # ---- CPU baseline: torch.nn.LSTM fwd+bwd on the host cores (bounded sample) ---
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import cpu_baseline
+        threads = torch.get_num_threads()
+        sec, iters = cpu_baseline.time_lstm_fwd_bwd(W, R, b, x, dy, budget_s=args.cpu_budget)
+        sec1, it1 = cpu_baseline.time_lstm_inference(W1, R1, b1, x1[:500], budget_s=5.0)
+        cpu = {"value": round(sec * 1e3, 3), "unit": "ms/batch", "cores": threads, "kind": "port",
+               "sample": "torch.nn.LSTM fwd+bwd fp32 on host CPU, same weights via the native "
+                         "weight map, N=64 T=100 C=H=512, median of %d iterations; "
+                         "os.cpu_count=%d" % (iters, os.cpu_count()),
+               "n1_us_per_timestep": round(sec1 * 1e6 / 500, 3),
+               "n1_sample": "torch.nn.LSTM inference N=1, first 500 of 2000 steps, median of %d" % it1}
+
+    out = {
+        "metric": "LSTM fwd+bwd ms/batch (N=64,T=100,H=512 fp32)",
+        "value": round(ms_per_step, 4), "unit": "ms/batch",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "LSTM training fwd+bwd N=64 T=100 C=H=512 fp32, forget bias 1, "
+                               "caller-side transposes inside the timed step"},
+        "achieved_tflops_whole_step": round(total_flops / (ms_per_step * 1e-3) / 1e12, 3),
+        "roofline": roofline,
+        "kernels": kernels,
+        "streaming_n1": streaming,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

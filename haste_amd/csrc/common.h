@@ -81,6 +81,18 @@ int layer_norm_backward(hipStream_t stream, int rows, int dim, const float* gamm
                         const float* x, const float* dy, float* dx, float* dgamma,
                         float* dbeta);
 
+// Brackets the launches made during its lifetime with a pair of events on `stream`
+// when profiling has been switched on (haste_hip_profile_enable); otherwise does
+// nothing.  `name` must be a string literal.
+class ScopedKernelTimer {
+ public:
+  ScopedKernelTimer(const char* name, hipStream_t stream);
+  ~ScopedKernelTimer();
+ private:
+  hipStream_t stream_;
+  int slot_;
+};
+
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
 }  // namespace haste_hip

@@ -190,8 +190,6 @@ void gemm_f32_kernel(int M, int N, int K,
 
   // Split-K: park the partial tile, then the last arrival folds all partials of the
   // tile into C in split order.
-  float* mine = partial + ((size_t)split * tiles_n * gridDim.y + 0);  // placeholder, set below
-  (void)mine;
   const size_t tile_elems = (size_t)BM * BN;
   float* part_tile = partial + ((size_t)tile * splits + split) * tile_elems;
 #pragma unroll
@@ -267,6 +265,7 @@ int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
   const int b_vec_ok = aligned16(B) && (ldb % 4 == 0);
   const int total = (int)(tiles * splits);
   dim3 grid((unsigned)total), block(256);
+  ScopedKernelTimer timer("gemm_f32", stream);
   if (trans_a) {
     gemm_f32_kernel<true><<<grid, block, 0, stream>>>(
         M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, tiles_n, total, splits,

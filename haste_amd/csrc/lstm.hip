@@ -333,34 +333,6 @@ void lstm_backward_kernel(LstmBwdParams p) {
   }
 }
 
-size_t fwd_lds_bytes(int H, int RT, int CT) {
-  const int Kpad = (H + 63) / 64 * 64;
-  return ((size_t)Kpad * 16 * CT + 4 * 16 * RT * 16 * CT) * sizeof(float);
-}
-
-size_t bwd_lds_bytes(int K, int RT) {
-  const int Kpad = (K + 63) / 64 * 64;
-  const size_t red = (size_t)4 * 16 * RT * 16;
-  return ((size_t)Kpad * 16 + red) * sizeof(float);
-}
-
-template <typename KernelT, typename ParamsT>
-int launch_persistent(KernelT kernel, dim3 grid, size_t lds_bytes, ParamsT& params,
-                      hipStream_t stream) {
-  HASTE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-  int per_cu = 0;
-  HASTE_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, lds_bytes));
-  const long long capacity = (long long)per_cu * device_cu_count();
-  if ((long long)grid.x * grid.y > capacity) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
-  void* args[] = {&params};
-  HASTE_HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<const void*>(kernel), grid, dim3(256),
-                                           args, (unsigned int)lds_bytes, stream));
-  return HASTE_HIP_OK;
-}
-
-constexpr size_t kMaxLdsBytes = 160 * 1024;
-
 }  // namespace
 
 // Picks (RT, CT) for a forward recurrence with G gate blocks; shared with the GRU.
@@ -398,7 +370,8 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
     dim3 grid(gx, gy);
 #define HASTE_LAUNCH_FWD(RT_, CT_)                                                         \
     if (cd.rt == RT_ && cd.ct == CT_)                                                      \
-      return launch_persistent(lstm_forward_kernel<RT_, CT_>, grid, lds, p, stream);
+      return launch_persistent("lstm_forward_recurrence", lstm_forward_kernel<RT_, CT_>, grid, lds, \
+                               p, stream);
     HASTE_LAUNCH_FWD(1, 1) HASTE_LAUNCH_FWD(1, 2) HASTE_LAUNCH_FWD(1, 4)
     HASTE_LAUNCH_FWD(2, 1) HASTE_LAUNCH_FWD(2, 2) HASTE_LAUNCH_FWD(2, 4)
     HASTE_LAUNCH_FWD(4, 1) HASTE_LAUNCH_FWD(4, 2) HASTE_LAUNCH_FWD(4, 4)
@@ -441,9 +414,9 @@ int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   const size_t lds = bwd_lds_bytes(4 * H, rt);
   dim3 grid(gx, gy);
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
-  if (rt == 1) rc = launch_persistent(lstm_backward_kernel<1>, grid, lds, p, stream);
-  if (rt == 2) rc = launch_persistent(lstm_backward_kernel<2>, grid, lds, p, stream);
-  if (rt == 4) rc = launch_persistent(lstm_backward_kernel<4>, grid, lds, p, stream);
+  if (rt == 1) rc = launch_persistent("lstm_backward_recurrence", lstm_backward_kernel<1>, grid, lds, p, stream);
+  if (rt == 2) rc = launch_persistent("lstm_backward_recurrence", lstm_backward_kernel<2>, grid, lds, p, stream);
+  if (rt == 4) rc = launch_persistent("lstm_backward_recurrence", lstm_backward_kernel<4>, grid, lds, p, stream);
   HASTE_HIP_PROPAGATE(rc);
 
   // dW += x^T dv ; dR += h[0:T]^T dv ; dx = dv W^T  (dv now lives in v).

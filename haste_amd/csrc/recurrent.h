@@ -224,4 +224,36 @@ __device__ __forceinline__ float sum_partials(const float* red, int row, int col
   return (p[0] + p[NB * NCOLS]) + (p[2 * NB * NCOLS] + p[3 * NB * NCOLS]);
 }
 
+// ---- host side ---------------------------------------------------------------------
+// LDS bytes of a forward kernel (slice [Kpad x 16*CT] + 4 wavefront partial tiles).
+inline size_t fwd_lds_bytes(int H, int RT, int CT) {
+  const int Kpad = (H + 63) / 64 * 64;
+  return ((size_t)Kpad * 16 * CT + 4 * 16 * RT * 16 * CT) * sizeof(float);
+}
+
+inline size_t bwd_lds_bytes(int K, int RT) {
+  const int Kpad = (K + 63) / 64 * 64;
+  const size_t red = (size_t)4 * 16 * RT * 16;
+  return ((size_t)Kpad * 16 + red) * sizeof(float);
+}
+
+template <typename KernelT, typename ParamsT>
+int launch_persistent(const char* name, KernelT kernel, dim3 grid, size_t lds_bytes, ParamsT& params,
+                      hipStream_t stream) {
+  HASTE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+  int per_cu = 0;
+  HASTE_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, lds_bytes));
+  const long long capacity = (long long)per_cu * device_cu_count();
+  if ((long long)grid.x * grid.y > capacity) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  void* args[] = {&params};
+  ScopedKernelTimer timer(name, stream);
+  HASTE_HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<const void*>(kernel), grid, dim3(256),
+                                           args, (unsigned int)lds_bytes, stream));
+  return HASTE_HIP_OK;
+}
+
+constexpr size_t kMaxLdsBytes = 160 * 1024;  // LDS per workgroup on gfx950
+
+
 }  // namespace haste_hip

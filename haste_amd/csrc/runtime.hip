@@ -7,6 +7,7 @@
 #include <mutex>
 #include <string>
 #include <utility>
+#include <vector>
 
 namespace haste_hip {
 
@@ -33,7 +34,33 @@ __global__ void fill_zero_kernel(unsigned int* p, size_t n) {
   if (i < n) p[i] = 0u;
 }
 
+struct TimedLaunch {
+  const char* name;
+  hipEvent_t start, stop;
+};
+bool g_profile_on = false;
+std::vector<TimedLaunch> g_timed;
+
 }  // namespace
+
+ScopedKernelTimer::ScopedKernelTimer(const char* name, hipStream_t stream)
+    : stream_(stream), slot_(-1) {
+  if (!g_profile_on) return;
+  TimedLaunch t;
+  t.name = name;
+  if (hipEventCreate(&t.start) != hipSuccess) return;
+  if (hipEventCreate(&t.stop) != hipSuccess) { (void)hipEventDestroy(t.start); return; }
+  (void)hipEventRecord(t.start, stream);
+  std::lock_guard<std::mutex> lock(g_mutex);
+  g_timed.push_back(t);
+  slot_ = (int)g_timed.size() - 1;
+}
+
+ScopedKernelTimer::~ScopedKernelTimer() {
+  if (slot_ < 0) return;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  if (slot_ < (int)g_timed.size()) (void)hipEventRecord(g_timed[slot_].stop, stream_);
+}
 
 void set_runtime_error(hipError_t err, const char* what) {
   char buf[512];
@@ -118,6 +145,42 @@ const char* haste_hip_error_string(int code) {
 }
 
 const char* haste_hip_last_runtime_error(void) { return haste_hip::g_last_error.c_str(); }
+
+int haste_hip_profile_enable(int on) {
+  std::lock_guard<std::mutex> lock(haste_hip::g_mutex);
+  haste_hip::g_profile_on = on != 0;
+  return HASTE_HIP_OK;
+}
+
+int haste_hip_profile_reset(void) {
+  std::lock_guard<std::mutex> lock(haste_hip::g_mutex);
+  for (auto& t : haste_hip::g_timed) {
+    (void)hipEventSynchronize(t.stop);
+    (void)hipEventDestroy(t.start);
+    (void)hipEventDestroy(t.stop);
+  }
+  haste_hip::g_timed.clear();
+  return HASTE_HIP_OK;
+}
+
+int haste_hip_profile_read(const char* name, double* total_ms, int* launches) {
+  if (name == nullptr || total_ms == nullptr || launches == nullptr)
+    return HASTE_HIP_ERROR_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> lock(haste_hip::g_mutex);
+  double total = 0.0;
+  int count = 0;
+  for (auto& t : haste_hip::g_timed) {
+    if (std::strcmp(t.name, name) != 0) continue;
+    if (hipEventSynchronize(t.stop) != hipSuccess) return HASTE_HIP_ERROR_RUNTIME;
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, t.start, t.stop) != hipSuccess) return HASTE_HIP_ERROR_RUNTIME;
+    total += ms;
+    ++count;
+  }
+  *total_ms = total;
+  *launches = count;
+  return HASTE_HIP_OK;
+}
 
 int haste_hip_release_workspaces(void) {
   int dev = 0;

@@ -44,6 +44,17 @@ int haste_hip_max_hidden_size(int gates, int batch_size);
  * device memory; the caller must have synchronized the streams that used them). */
 int haste_hip_release_workspaces(void);
 
+/* Per-kernel timing, off by default.  While enabled, every kernel the library
+ * launches is bracketed by a pair of HIP events recorded on the stream the kernel
+ * runs on.  haste_hip_profile_read waits for those events and returns, for the kernel
+ * called `name` ("gemm_f32", "lstm_forward_recurrence", "lstm_backward_recurrence", ...),
+ * the summed duration in milliseconds and the number of launches since the last reset.
+ * The reference has only cudaEvent timers in its benchmarks
+ * (benchmarks/benchmark_lstm.cc:49-63); this is their in-library counterpart. */
+int haste_hip_profile_enable(int on);
+int haste_hip_profile_reset(void);
+int haste_hip_profile_read(const char* name, double* total_ms, int* launches);
+
 /* C[M,N] = op(A)[M,K] * B[K,N] (+ C if accumulate != 0); fp32 MFMA.
  * trans_a == 0: A is [M,K] with leading dimension lda; trans_a != 0: A is stored
  * as [K,M] with leading dimension lda.  Replaces the cuBLAS calls the reference
