@@ -35,13 +35,14 @@ void set_runtime_error(hipError_t err, const char* what);
     if (rc__ != HASTE_HIP_OK) return rc__;                    \
   } while (0)
 
-// Layout of the control block at the start of a workspace (all zero between
-// kernels; every kernel that uses a field restores it to zero before it exits).
+// Layout of the control block of a workspace.  The counters are zero between kernels
+// (a kernel that uses one restores it before it exits); the step flags only ever
+// grow: each persistent launch is given a fresh range of values (an epoch).
 constexpr int kMaxGroups = 64;        // batch tiles a persistent kernel may have
+constexpr int kMaxWorkgroups = 2048;  // workgroups a persistent kernel may have
 constexpr int kCounterStride = 32;    // uint32 slots between counters (128 B apart)
 struct ControlBlock {
-  unsigned int step_counter[kMaxGroups * kCounterStride];  // per-group step barrier
-  unsigned int exit_counter[kMaxGroups * kCounterStride];  // per-group "left the loop" count
+  unsigned int step_flags[kMaxWorkgroups];                 // per-workgroup arrival counts
   unsigned int grid_exit_counter[kCounterStride];          // all workgroups of a launch
   unsigned int tile_counter[4096];                         // split-K arrivals per output tile
   unsigned int abort_flag[kCounterStride];                 // set when a barrier wait gives up
@@ -54,6 +55,7 @@ struct Workspace {
   ControlBlock* control = nullptr;   // device
   float* scratch = nullptr;          // device
   size_t scratch_bytes = 0;
+  unsigned int epoch = 0;            // step-flag values handed out so far
   unsigned int* host_status = nullptr;      // pinned host word the kernels report aborts to
   unsigned int* host_status_dev = nullptr;  // the same word as the device addresses it
 };
@@ -61,6 +63,10 @@ struct Workspace {
 // Returns the workspace of (current device, stream) with at least `scratch_bytes`
 // of scratch, creating or growing it if needed.
 int get_workspace(hipStream_t stream, size_t scratch_bytes, Workspace* out);
+
+// Reserves `count` consecutive step-flag values on the workspace of (current device,
+// stream) and returns the value before the first of them.
+int reserve_epochs(hipStream_t stream, unsigned int count, unsigned int* base);
 
 // Checks (without synchronizing) whether a persistent kernel launched earlier on
 // this workspace reported a barrier time-out; if so re-zeroes the control block and

@@ -1,0 +1,458 @@
+// GRU forward and backward passes (gate order z, r, g; "reset-after" variant):
+// one MFMA GEMM for x*W over all steps, one persistent kernel for the recurrence with
+// the gate math, zoneout and optional DropConnect fused in; backward is a persistent
+// reverse-time kernel followed by three batched GEMMs.
+//
+// Arithmetic follows reference lib/gru_forward_gpu.cu.cc:46-84 and
+// lib/gru_backward_gpu.cu.cc:45-95; orchestration replaces :314-371 and :321-409.
+#include "recurrent.h"
+
+namespace haste_hip {
+namespace {
+
+struct GruFwdParams {
+  int training, T, N, H;
+  const float* R;        // [H,3H]
+  const float* bx;       // [3H]
+  const float* br;       // [3H]
+  float* h;              // [T+1,N,H]
+  float* v;              // [T,N,4H] (training) or null
+  const float* Wx;       // [T,N,3H] = x*W
+  float zoneout_prob;
+  const float* zoneout_mask;
+  const float* dc_mask;  // DropConnect mask [H,3H] or null
+  float dc_scale;
+  ControlBlock* cb;
+  unsigned int* host_status;
+  unsigned int spin_limit;
+  unsigned int epoch;
+};
+
+// HS hidden units per workgroup; their 3 gate columns occupy 3*HS of the 16*CT slice
+// columns (the rest are zero padding).
+template <int RT, int CT, int HS>
+__global__ __launch_bounds__(256, 1)
+void gru_forward_kernel(GruFwdParams p) {
+  static_assert(3 * HS <= 16 * CT, "slice too narrow");
+  constexpr int NB = 16 * RT;
+  constexpr int NCOLS = 16 * CT;
+  constexpr int PP = (NB * HS + 255) / 256;
+  constexpr int CHUNK = RT == 4 ? 4 : 8;
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+
+  const int H = p.H, N = p.N, T = p.T;
+  const int Kpad = round_up(H, 64);
+  float* w_lds = lds;
+  float* red = lds + Kpad * NCOLS;
+
+  const int tid = threadIdx.x;
+  const int j0 = blockIdx.x * HS;
+  const int n0 = blockIdx.y * NB;
+  const size_t NH = (size_t)N * H;
+
+  GroupSync gs;
+  group_sync_init(gs, p.cb, blockIdx.y, gridDim.x, blockIdx.x, p.epoch, p.host_status, p.spin_limit);
+
+  for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
+    const int k = idx / NCOLS, cidx = idx % NCOLS;
+    const int gate = cidx / HS, j = j0 + cidx % HS;
+    float w = 0.f;
+    if (k < H && gate < 3 && j < H) {
+      const size_t off = (size_t)k * 3 * H + gate * H + j;
+      w = p.R[off];
+      if (p.dc_mask != nullptr) w = w * p.dc_mask[off] * p.dc_scale;
+    }
+    w_lds[slice_index(k, cidx, NCOLS)] = w;
+  }
+
+  int pn[PP], pj[PP], pl[PP], pc[PP];
+  bool act[PP];
+  float h_prev[PP], bxv[PP][3], brv[PP][3];
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp) {
+    const int idx = tid + 256 * pp;
+    pl[pp] = idx / HS;
+    pc[pp] = idx % HS;
+    pn[pp] = n0 + pl[pp];
+    pj[pp] = j0 + pc[pp];
+    act[pp] = idx < NB * HS && pn[pp] < N && pj[pp] < H;
+    h_prev[pp] = 0.f;
+#pragma unroll
+    for (int g = 0; g < 3; ++g) bxv[pp][g] = brv[pp][g] = 0.f;
+    if (act[pp]) {
+      h_prev[pp] = p.h[(size_t)pn[pp] * H + pj[pp]];
+#pragma unroll
+      for (int g = 0; g < 3; ++g) {
+        bxv[pp][g] = p.bx[g * H + pj[pp]];
+        brv[pp][g] = p.br[g * H + pj[pp]];
+      }
+    }
+  }
+  const bool zoneout = p.zoneout_prob != 0.f && p.zoneout_mask != nullptr;
+  const bool vec_ok = (H % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.h) & 15u) == 0);
+  __syncthreads();
+
+  for (int t = 0; t < T; ++t) {
+    float wx[PP][3], mk[PP];
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      mk[pp] = 1.f;
+#pragma unroll
+      for (int g = 0; g < 3; ++g) wx[pp][g] = 0.f;
+      if (act[pp]) {
+        const float* wt = p.Wx + ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 3; ++g) wx[pp][g] = wt[g * H];
+        if (zoneout && p.training) mk[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
+      }
+    }
+    if (t > 0) group_wait(gs);
+
+    float4_t acc[RT][CT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
+    slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, N - n0, H, Kpad, w_lds,
+                                vec_ok, acc);
+    store_partials<RT, CT>(red, acc);
+    __syncthreads();
+
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      if (act[pp]) {
+        float rh[3];
+#pragma unroll
+        for (int g = 0; g < 3; ++g) rh[g] = sum_partials<RT, CT>(red, pl[pp], g * HS + pc[pp]);
+        const float z = sigmoid_f(wx[pp][0] + rh[0] + bxv[pp][0] + brv[pp][0]);
+        const float r = sigmoid_f(wx[pp][1] + rh[1] + bxv[pp][1] + brv[pp][1]);
+        const float qg = rh[2] + brv[pp][2];
+        const float g = tanhf(wx[pp][2] + r * qg + bxv[pp][2]);
+        if (p.training) {
+          float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+          vt[0] = z;
+          vt[H] = r;
+          vt[2 * H] = g;
+          vt[3 * H] = qg;
+        }
+        float h_new = z * h_prev[pp] + (1.0f - z) * g;
+        if (zoneout) {
+          if (p.training) h_new = (h_new - h_prev[pp]) * mk[pp] + h_prev[pp];
+          else h_new = p.zoneout_prob * h_prev[pp] + (1.0f - p.zoneout_prob) * h_new;
+        }
+        store_exchanged(&p.h[(size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp]], h_new);
+        h_prev[pp] = h_new;
+      }
+    }
+    if (t + 1 < T) group_arrive(gs);
+  }
+}
+
+struct GruBwdParams {
+  int T, N, H;
+  const float* R_t;     // [3H,H]
+  const float* h;       // [T+1,N,H]
+  const float* v;       // [T,N,4H]
+  const float* dh_new;  // [T+1,N,H]
+  float* dbx;           // [3H] accumulated
+  float* dbr;           // [3H] accumulated
+  float* dh;            // [N,H] in/out
+  float* dp;            // [T,N,3H]
+  float* dq;            // [T,N,3H]
+  const float* zoneout_mask;
+  float* db_partial;    // [batch tiles, 6H] scratch
+  ControlBlock* cb;
+  unsigned int* host_status;
+  unsigned int spin_limit;
+  unsigned int epoch;
+};
+
+template <int RT>
+__global__ __launch_bounds__(256, 1)
+void gru_backward_kernel(GruBwdParams p) {
+  constexpr int HSB = 16;
+  constexpr int NB = 16 * RT;
+  constexpr int NCOLS = 16;
+  constexpr int PP = RT;
+  constexpr int CHUNK = RT == 1 ? 16 : (RT == 2 ? 8 : 4);
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  __shared__ unsigned int s_flag;
+
+  const int H = p.H, N = p.N, T = p.T;
+  const int K = 3 * H;
+  const int Kpad = round_up(K, 64);
+  float* w_lds = lds;
+  float* red = lds + Kpad * NCOLS;  // max(4*NB*16, NB*6*16) floats
+
+  const int tid = threadIdx.x;
+  const int j0 = blockIdx.x * HSB;
+  const int n0 = blockIdx.y * NB;
+  const size_t NH = (size_t)N * H;
+
+  GroupSync gs;
+  group_sync_init(gs, p.cb, blockIdx.y, gridDim.x, blockIdx.x, p.epoch, p.host_status, p.spin_limit);
+
+  for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
+    const int k = idx / NCOLS, cidx = idx % NCOLS;
+    float w = 0.f;
+    if (k < K && j0 + cidx < H) w = p.R_t[(size_t)k * H + j0 + cidx];
+    w_lds[slice_index(k, cidx, NCOLS)] = w;
+  }
+
+  int pn[PP], pj[PP], pl[PP], pc[PP];
+  bool act[PP];
+  float dh[PP], dbacc[PP][6];
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp) {
+    const int idx = tid + 256 * pp;
+    pl[pp] = idx / HSB;
+    pc[pp] = idx % HSB;
+    pn[pp] = n0 + pl[pp];
+    pj[pp] = j0 + pc[pp];
+    act[pp] = pn[pp] < N && pj[pp] < H;
+    dh[pp] = act[pp] ? p.dh[(size_t)pn[pp] * H + pj[pp]] : 0.f;
+#pragma unroll
+    for (int g = 0; g < 6; ++g) dbacc[pp][g] = 0.f;
+  }
+  const bool zoneout = p.zoneout_mask != nullptr;
+  const bool vec_ok = (reinterpret_cast<uintptr_t>(p.dq) & 15u) == 0 && (K % 4 == 0);
+  __syncthreads();
+
+  struct StepIn { float vt[4], h0, dhn, m; };
+  StepIn nxt[PP];
+  auto fetch = [&](int t) {
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      StepIn s = {{0.f, 0.f, 0.f, 0.f}, 0.f, 0.f, 1.f};
+      if (act[pp] && t >= 0) {
+        const size_t e = (size_t)pn[pp] * H + pj[pp];
+        const float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) s.vt[g] = vt[g * H];
+        s.h0 = p.h[(size_t)t * NH + e];
+        s.dhn = p.dh_new[(size_t)(t + 1) * NH + e];
+        if (zoneout) s.m = p.zoneout_mask[(size_t)t * NH + e];
+      }
+      nxt[pp] = s;
+    }
+  };
+  fetch(T - 1);
+
+  for (int t = T - 1; t >= 0; --t) {
+    float dh_keep[PP];
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      dh_keep[pp] = 0.f;
+      if (act[pp]) {
+        const StepIn s = nxt[pp];
+        const float z = s.vt[0], r = s.vt[1], g = s.vt[2], qg = s.vt[3];
+        float dh_total = s.dhn + dh[pp];
+        if (zoneout) {
+          dh_keep[pp] = (1.0f - s.m) * dh_total;
+          dh_total = s.m * dh_total;
+          dh_keep[pp] += z * dh_total;
+        } else {
+          dh_keep[pp] = z * dh_total;
+        }
+        const float dg = (1.0f - z) * dh_total;
+        const float dz = (s.h0 - g) * dh_total;
+        const float dp_g = d_tanh_f(g) * dg;
+        const float dq_g = dp_g * r;
+        const float dr = dp_g * qg;
+        const float dp_r = d_sigmoid_f(r) * dr;
+        const float dp_z = d_sigmoid_f(z) * dz;
+        const size_t o3 = ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
+        p.dp[o3] = dp_z;
+        p.dp[o3 + H] = dp_r;
+        p.dp[o3 + 2 * H] = dp_g;
+        store_exchanged(&p.dq[o3], dp_z);
+        store_exchanged(&p.dq[o3 + H], dp_r);
+        store_exchanged(&p.dq[o3 + 2 * H], dq_g);
+        dbacc[pp][0] += dp_z;
+        dbacc[pp][1] += dp_r;
+        dbacc[pp][2] += dp_g;
+        dbacc[pp][3] += dp_z;
+        dbacc[pp][4] += dp_r;
+        dbacc[pp][5] += dq_g;
+      }
+    }
+    group_arrive(gs);
+    fetch(t - 1);
+    group_wait(gs);
+
+    float4_t acc[RT][1];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) acc[rt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
+    slice_matmul<RT, 1, CHUNK>(p.dq + ((size_t)t * N + n0) * 3 * H, 3 * H, N - n0, K, Kpad, w_lds,
+                               vec_ok, acc);
+    store_partials<RT, 1>(red, acc);
+    __syncthreads();
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp)
+      dh[pp] = dh_keep[pp] + sum_partials<RT, 1>(red, pl[pp], pc[pp]);
+  }
+
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp)
+    if (act[pp]) p.dh[(size_t)pn[pp] * H + pj[pp]] = dh[pp];
+
+  __syncthreads();
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp)
+#pragma unroll
+    for (int g = 0; g < 6; ++g) red[(pl[pp] * 6 + g) * HSB + pc[pp]] = act[pp] ? dbacc[pp][g] : 0.f;
+  __syncthreads();
+  if (tid < 6 * HSB) {
+    const int g = tid / HSB, jj = tid % HSB;
+    float s = 0.f;
+    for (int r = 0; r < NB; ++r) s += red[(r * 6 + g) * HSB + jj];
+    if (j0 + jj < H) p.db_partial[(size_t)blockIdx.y * 6 * H + g * H + j0 + jj] = s;
+  }
+  if (grid_last_arrival(p.cb, gridDim.x * gridDim.y, &s_flag)) {
+    for (int col = tid; col < 6 * H; col += 256) {
+      float s = 0.f;
+      for (int bt = 0; bt < (int)gridDim.y; ++bt) s += p.db_partial[(size_t)bt * 6 * H + col];
+      if (col < 3 * H) p.dbx[col] += s;
+      else p.dbr[col - 3 * H] += s;
+    }
+  }
+}
+
+}  // namespace
+
+int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int H,
+                     const float* W, const float* R, const float* bx, const float* br,
+                     const float* x, float* h, float* v, float* tmp_Wx, float zoneout_prob,
+                     const float* zoneout_mask, const float* dc_mask, float dc_scale) {
+  HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
+  HASTE_HIP_REQUIRE(W && R && bx && br && x && h && tmp_Wx);
+  HASTE_HIP_REQUIRE(!training || v != nullptr);
+  Workspace ws;
+  HASTE_HIP_PROPAGATE(get_workspace(stream, 0, &ws));
+  HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
+  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 3 * H, C, x, C, W, 3 * H, tmp_Wx, 3 * H, false));
+
+  GruFwdParams p;
+  p.training = training; p.T = T; p.N = N; p.H = H;
+  p.R = R; p.bx = bx; p.br = br; p.h = h; p.v = v; p.Wx = tmp_Wx;
+  p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
+  p.dc_mask = dc_mask; p.dc_scale = dc_scale;
+  p.cb = ws.control; p.host_status = ws.host_status_dev; p.spin_limit = kSpinLimit;
+  HASTE_HIP_PROPAGATE(reserve_epochs(stream, (unsigned)T + 1, &p.epoch));
+
+  const int cus = device_cu_count();
+  struct Cand { int rt, ct, hs; };
+  const Cand cands[] = {{1, 2, 8}, {1, 3, 16}, {1, 1, 4}, {2, 2, 8}, {2, 3, 16}, {2, 1, 4},
+                        {4, 2, 8}, {4, 3, 16}, {4, 1, 4}};
+  for (const Cand& cd : cands) {
+    const int NB = 16 * cd.rt;
+    const int gx = (H + cd.hs - 1) / cd.hs, gy = (N + NB - 1) / NB;
+    if (gy > kMaxGroups || (long long)gx * gy > cus || gx * gy > kMaxWorkgroups) continue;
+    const size_t lds = fwd_lds_bytes(H, cd.rt, cd.ct);
+    if (lds > kMaxLdsBytes) continue;
+    dim3 grid(gx, gy);
+#define HASTE_LAUNCH_FWD(RT_, CT_, HS_)                                                       \
+    if (cd.rt == RT_ && cd.ct == CT_)                                                         \
+      return launch_persistent("gru_forward_recurrence", gru_forward_kernel<RT_, CT_, HS_>,   \
+                               grid, lds, p, stream);
+    HASTE_LAUNCH_FWD(1, 1, 4) HASTE_LAUNCH_FWD(1, 2, 8) HASTE_LAUNCH_FWD(1, 3, 16)
+    HASTE_LAUNCH_FWD(2, 1, 4) HASTE_LAUNCH_FWD(2, 2, 8) HASTE_LAUNCH_FWD(2, 3, 16)
+    HASTE_LAUNCH_FWD(4, 1, 4) HASTE_LAUNCH_FWD(4, 2, 8) HASTE_LAUNCH_FWD(4, 3, 16)
+#undef HASTE_LAUNCH_FWD
+  }
+  return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+}
+
+int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
+                      const float* W_t, const float* R_t, const float* x_t, const float* h,
+                      const float* v, const float* dh_new, float* dx, float* dW, float* dR,
+                      float* dbx, float* dbr, float* dh, float* dp, float* dq,
+                      const float* zoneout_mask) {
+  HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
+  HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && v && dh_new);
+  HASTE_HIP_REQUIRE(dx && dW && dR && dbx && dbr && dh && dp && dq);
+  const int cus = device_cu_count();
+  const int gx = (H + 15) / 16;
+  int rt = 0;
+  for (int cand : {1, 2, 4}) {
+    const int gy = (N + 16 * cand - 1) / (16 * cand);
+    const size_t lds = bwd_lds_bytes(3 * H, cand) + (size_t)2 * 16 * cand * 16 * sizeof(float);
+    if (gy <= kMaxGroups && (long long)gx * gy <= cus && gx * gy <= kMaxWorkgroups &&
+        lds <= kMaxLdsBytes) {
+      rt = cand;
+      break;
+    }
+  }
+  if (rt == 0) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  const int gy = (N + 16 * rt - 1) / (16 * rt);
+
+  Workspace ws;
+  HASTE_HIP_PROPAGATE(get_workspace(stream, (size_t)gy * 6 * H * sizeof(float), &ws));
+  HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
+
+  GruBwdParams p;
+  p.T = T; p.N = N; p.H = H;
+  p.R_t = R_t; p.h = h; p.v = v; p.dh_new = dh_new;
+  p.dbx = dbx; p.dbr = dbr; p.dh = dh; p.dp = dp; p.dq = dq; p.zoneout_mask = zoneout_mask;
+  p.db_partial = ws.scratch;
+  p.cb = ws.control; p.host_status = ws.host_status_dev; p.spin_limit = kSpinLimit;
+  HASTE_HIP_PROPAGATE(reserve_epochs(stream, (unsigned)T + 1, &p.epoch));
+  // the reduction of the bias gradients needs NB*6*16 floats, more than the 4 partial tiles
+  const size_t lds = bwd_lds_bytes(3 * H, rt) + (size_t)2 * 16 * rt * 16 * sizeof(float);
+  dim3 grid(gx, gy);
+  int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  if (rt == 1) rc = launch_persistent("gru_backward_recurrence", gru_backward_kernel<1>, grid, lds, p, stream);
+  if (rt == 2) rc = launch_persistent("gru_backward_recurrence", gru_backward_kernel<2>, grid, lds, p, stream);
+  if (rt == 4) rc = launch_persistent("gru_backward_recurrence", gru_backward_kernel<4>, grid, lds, p, stream);
+  HASTE_HIP_PROPAGATE(rc);
+
+  const int TN = T * N;
+  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, TN, C, 3 * H, dp, 3 * H, W_t, C, dx, C, false));
+  HASTE_HIP_PROPAGATE(gemm_f32(stream, true, H, 3 * H, TN, h, H, dq, 3 * H, dR, 3 * H, true));
+  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, C, 3 * H, TN, x_t, TN, dp, 3 * H, dW, 3 * H, true));
+  return HASTE_HIP_OK;
+}
+
+}  // namespace haste_hip
+
+extern "C" {
+
+int haste_hip_gru_forward_f32(int training, int steps, int batch_size, int input_size,
+                              int hidden_size,
+                              const float* W, const float* R, const float* bx, const float* br,
+                              const float* x, float* h, float* v, float* tmp_Wx, float* tmp_Rh,
+                              float zoneout_prob, const float* zoneout_mask, void* stream) {
+  (void)tmp_Rh;
+  return haste_hip::gru_forward_impl(haste_hip::as_stream(stream), training, steps, batch_size,
+                                     input_size, hidden_size, W, R, bx, br, x, h, v, tmp_Wx,
+                                     zoneout_prob, zoneout_mask, nullptr, 1.0f);
+}
+
+int haste_hip_gru_forward_dropconnect_f32(int training, int steps, int batch_size,
+                                          int input_size, int hidden_size,
+                                          const float* W, const float* R, const float* bx,
+                                          const float* br, const float* x, float* h, float* v,
+                                          float* tmp_Wx, float zoneout_prob,
+                                          const float* zoneout_mask,
+                                          const float* dropconnect_mask, float dropconnect_scale,
+                                          void* stream) {
+  return haste_hip::gru_forward_impl(haste_hip::as_stream(stream), training, steps, batch_size,
+                                     input_size, hidden_size, W, R, bx, br, x, h, v, tmp_Wx,
+                                     zoneout_prob, zoneout_mask, dropconnect_mask,
+                                     dropconnect_scale);
+}
+
+int haste_hip_gru_backward_f32(int steps, int batch_size, int input_size, int hidden_size,
+                               const float* W_t, const float* R_t, const float* bx,
+                               const float* br, const float* x_t, const float* h, const float* v,
+                               const float* dh_new, float* dx, float* dW, float* dR,
+                               float* dbx, float* dbr, float* dh, float* dp, float* dq,
+                               const float* zoneout_mask, void* stream) {
+  (void)bx;
+  (void)br;
+  return haste_hip::gru_backward_impl(haste_hip::as_stream(stream), steps, batch_size, input_size,
+                                      hidden_size, W_t, R_t, x_t, h, v, dh_new, dx, dW, dR, dbx,
+                                      dbr, dh, dp, dq, zoneout_mask);
+}
+
+}  // extern "C"

@@ -1,0 +1,258 @@
+// IndRNN and LayerNormIndRNN forward and backward passes.
+//
+// The recurrence h_{t+1} = tanh((xW)_t + u*h_t + b) is elementwise, so there is no
+// exchange between threads: one thread owns one (batch row, hidden unit) pair and
+// walks all T steps.  The only cost is the serial chain of HBM loads, so each thread
+// keeps a block of U future steps' operands in flight while it computes the current
+// block.  Consecutive lanes own consecutive hidden units (coalesced 256-byte rows).
+//
+// Arithmetic follows reference lib/indrnn_forward_gpu.cu.cc:44-62 and
+// lib/indrnn_backward_gpu.cu.cc:46-73; orchestration replaces :114-210 and :122-207
+// (and lib/layer_norm_indrnn_{forward,backward}_gpu.cu.cc:114-213 / 122-209).
+#include "recurrent.h"
+
+namespace haste_hip {
+namespace {
+
+constexpr int U = 8;  // steps of operands kept in flight per thread
+
+template <bool TRAINING, bool ZONEOUT>
+__global__ __launch_bounds__(256)
+void indrnn_forward_kernel(int T, int N, int H, const float* __restrict__ Wx,
+                           const float* __restrict__ u, const float* __restrict__ b,
+                           float* __restrict__ h, float zoneout_prob,
+                           const float* __restrict__ mask) {
+  const int j = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int n = blockIdx.y * 4 + (threadIdx.x >> 6);
+  if (j >= H || n >= N) return;
+  const size_t NH = (size_t)N * H;
+  const size_t idx = (size_t)n * H + j;
+  const float uj = u[j], bj = b[j];
+  float hv = h[idx];
+
+  float wx_cur[U], mk_cur[U], wx_nxt[U], mk_nxt[U];
+  auto fetch = [&](int t0, float (&wx)[U], float (&mk)[U]) {
+#pragma unroll
+    for (int i = 0; i < U; ++i) {
+      const int t = t0 + i;
+      wx[i] = t < T ? Wx[(size_t)t * NH + idx] : 0.f;
+      mk[i] = (ZONEOUT && TRAINING && t < T) ? mask[(size_t)t * NH + idx] : 1.f;
+    }
+  };
+  fetch(0, wx_cur, mk_cur);
+  for (int t0 = 0; t0 < T; t0 += U) {
+    fetch(t0 + U, wx_nxt, mk_nxt);
+#pragma unroll
+    for (int i = 0; i < U; ++i) {
+      const int t = t0 + i;
+      if (t < T) {
+        float hn = tanhf(wx_cur[i] + uj * hv + bj);
+        if (ZONEOUT) {
+          if (TRAINING) hn = (hn - hv) * mk_cur[i] + hv;
+          else hn = zoneout_prob * hv + (1.0f - zoneout_prob) * hn;
+        }
+        h[(size_t)(t + 1) * NH + idx] = hn;
+        hv = hn;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < U; ++i) { wx_cur[i] = wx_nxt[i]; mk_cur[i] = mk_nxt[i]; }
+  }
+}
+
+template <bool ZONEOUT>
+__global__ __launch_bounds__(256)
+void indrnn_backward_kernel(int T, int N, int H, const float* __restrict__ u,
+                            const float* __restrict__ h, const float* __restrict__ dh_new,
+                            float* __restrict__ du, float* __restrict__ db,
+                            float* __restrict__ dh, float* __restrict__ dk,
+                            const float* __restrict__ mask, float* __restrict__ partial,
+                            ControlBlock* cb) {
+  __shared__ float red[2][4][64];
+  __shared__ unsigned int s_flag;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int j = blockIdx.x * 64 + lane;
+  const int n = blockIdx.y * 4 + w;
+  const bool live = j < H && n < N;
+  const size_t NH = (size_t)N * H;
+  const size_t idx = live ? (size_t)n * H + j : 0;
+  const float uj = live ? u[j] : 0.f;
+  float dh_io = live ? dh[idx] : 0.f;
+  float du_sum = 0.f, db_sum = 0.f;
+
+  struct In { float hn, hp, d, m; };
+  In cur[U], nxt[U];
+  auto fetch = [&](int t_hi, In (&s)[U]) {
+#pragma unroll
+    for (int i = 0; i < U; ++i) {
+      const int t = t_hi - i;
+      In v = {0.f, 0.f, 0.f, 1.f};
+      if (live && t >= 0) {
+        v.hn = h[(size_t)(t + 1) * NH + idx];
+        v.hp = h[(size_t)t * NH + idx];
+        v.d = dh_new[(size_t)(t + 1) * NH + idx];
+        if (ZONEOUT) v.m = mask[(size_t)t * NH + idx];
+      }
+      s[i] = v;
+    }
+  };
+  fetch(T - 1, cur);
+  for (int t_hi = T - 1; t_hi >= 0; t_hi -= U) {
+    fetch(t_hi - U, nxt);
+#pragma unroll
+    for (int i = 0; i < U; ++i) {
+      const int t = t_hi - i;
+      if (live && t >= 0) {
+        float dh_total = cur[i].d + dh_io;
+        float keep = 0.f;
+        if (ZONEOUT) {
+          keep = (1.0f - cur[i].m) * dh_total;
+          dh_total = cur[i].m * dh_total;
+        }
+        const float k = d_tanh_f(cur[i].hn) * dh_total;
+        dk[(size_t)t * NH + idx] = k;
+        dh_io = keep + uj * k;
+        du_sum += cur[i].hp * k;
+        db_sum += k;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < U; ++i) cur[i] = nxt[i];
+  }
+  if (live) dh[idx] = dh_io;
+
+  // Column sums over the batch: 4 rows per workgroup in LDS, then workgroups in order.
+  red[0][w][lane] = du_sum;
+  red[1][w][lane] = db_sum;
+  __syncthreads();
+  if (threadIdx.x < 128) {
+    const int which = threadIdx.x >> 6;
+    const float s = (red[which][0][lane] + red[which][1][lane]) + (red[which][2][lane] + red[which][3][lane]);
+    if (j < H) partial[((size_t)blockIdx.y * 2 + which) * H + j] = s;
+  }
+  if (grid_last_arrival(cb, gridDim.x * gridDim.y, &s_flag)) {
+    for (int c = threadIdx.x; c < 2 * H; c += 256) {
+      const int which = c / H, col = c % H;
+      float s = 0.f;
+      for (int by = 0; by < (int)gridDim.y; ++by) s += partial[((size_t)by * 2 + which) * H + col];
+      if (which == 0) du[col] += s;
+      else db[col] += s;
+    }
+  }
+}
+
+int run_forward_recurrence(hipStream_t stream, int training, int T, int N, int H, const float* Wx,
+                           const float* u, const float* b, float* h, float zoneout_prob,
+                           const float* mask) {
+  const bool zoneout = zoneout_prob != 0.f && mask != nullptr;
+  dim3 grid((H + 63) / 64, (N + 3) / 4), block(256);
+  ScopedKernelTimer timer("indrnn_forward_recurrence", stream);
+  if (training && zoneout)
+    indrnn_forward_kernel<true, true><<<grid, block, 0, stream>>>(T, N, H, Wx, u, b, h, zoneout_prob, mask);
+  else if (training)
+    indrnn_forward_kernel<true, false><<<grid, block, 0, stream>>>(T, N, H, Wx, u, b, h, 0.f, nullptr);
+  else if (zoneout)
+    indrnn_forward_kernel<false, true><<<grid, block, 0, stream>>>(T, N, H, Wx, u, b, h, zoneout_prob, mask);
+  else
+    indrnn_forward_kernel<false, false><<<grid, block, 0, stream>>>(T, N, H, Wx, u, b, h, 0.f, nullptr);
+  HASTE_HIP_TRY(hipGetLastError());
+  return HASTE_HIP_OK;
+}
+
+int run_backward_recurrence(hipStream_t stream, int T, int N, int H, const float* u, const float* h,
+                            const float* dh_new, float* du, float* db, float* dh, float* dk,
+                            const float* mask) {
+  dim3 grid((H + 63) / 64, (N + 3) / 4), block(256);
+  Workspace ws;
+  HASTE_HIP_PROPAGATE(get_workspace(stream, (size_t)grid.y * 2 * H * sizeof(float), &ws));
+  ScopedKernelTimer timer("indrnn_backward_recurrence", stream);
+  if (mask != nullptr)
+    indrnn_backward_kernel<true><<<grid, block, 0, stream>>>(T, N, H, u, h, dh_new, du, db, dh, dk,
+                                                              mask, ws.scratch, ws.control);
+  else
+    indrnn_backward_kernel<false><<<grid, block, 0, stream>>>(T, N, H, u, h, dh_new, du, db, dh, dk,
+                                                               nullptr, ws.scratch, ws.control);
+  HASTE_HIP_TRY(hipGetLastError());
+  return HASTE_HIP_OK;
+}
+
+}  // namespace
+}  // namespace haste_hip
+
+extern "C" {
+
+using namespace haste_hip;
+
+int haste_hip_indrnn_forward_f32(int training, int steps, int batch_size, int input_size,
+                                 int hidden_size,
+                                 const float* W, const float* u, const float* b, const float* x,
+                                 float* h, float* workspace,
+                                 float zoneout_prob, const float* zoneout_mask, void* stream) {
+  const int T = steps, N = batch_size, C = input_size, H = hidden_size;
+  HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
+  HASTE_HIP_REQUIRE(W && u && b && x && h && workspace);
+  hipStream_t s = as_stream(stream);
+  HASTE_HIP_PROPAGATE(gemm_f32(s, false, T * N, H, C, x, C, W, H, workspace, H, false));
+  return run_forward_recurrence(s, training, T, N, H, workspace, u, b, h, zoneout_prob, zoneout_mask);
+}
+
+int haste_hip_indrnn_backward_f32(int steps, int batch_size, int input_size, int hidden_size,
+                                  const float* W_t, const float* u, const float* b,
+                                  const float* x_t, const float* h, const float* dh_new,
+                                  float* dx, float* dW, float* du, float* db, float* dh,
+                                  float* workspace, const float* zoneout_mask, void* stream) {
+  (void)b;
+  const int T = steps, N = batch_size, C = input_size, H = hidden_size;
+  HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
+  HASTE_HIP_REQUIRE(W_t && u && x_t && h && dh_new && dx && dW && du && db && dh && workspace);
+  hipStream_t s = as_stream(stream);
+  HASTE_HIP_PROPAGATE(run_backward_recurrence(s, T, N, H, u, h, dh_new, du, db, dh, workspace,
+                                              zoneout_mask));
+  // dW = x^T dk (assigned, as in the reference); dx = dk W^T.
+  HASTE_HIP_PROPAGATE(gemm_f32(s, false, C, H, T * N, x_t, T * N, workspace, H, dW, H, false));
+  HASTE_HIP_PROPAGATE(gemm_f32(s, false, T * N, C, H, workspace, H, W_t, C, dx, C, false));
+  return HASTE_HIP_OK;
+}
+
+int haste_hip_layer_norm_indrnn_forward_f32(int training, int steps, int batch_size,
+                                            int input_size, int hidden_size,
+                                            const float* W, const float* u, const float* b,
+                                            const float* x, float* h, float* workspace,
+                                            float* act_Wx, const float* gamma1, float* cache1,
+                                            float zoneout_prob, const float* zoneout_mask,
+                                            void* stream) {
+  const int T = steps, N = batch_size, C = input_size, H = hidden_size;
+  HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
+  HASTE_HIP_REQUIRE(W && u && b && x && h && workspace && act_Wx && gamma1);
+  hipStream_t s = as_stream(stream);
+  HASTE_HIP_PROPAGATE(gemm_f32(s, false, T * N, H, C, x, C, W, H, act_Wx, H, false));
+  HASTE_HIP_PROPAGATE(layer_norm_forward(s, T * N, H, gamma1, nullptr, act_Wx, workspace, cache1));
+  return run_forward_recurrence(s, training, T, N, H, workspace, u, b, h, zoneout_prob, zoneout_mask);
+}
+
+int haste_hip_layer_norm_indrnn_backward_f32(int steps, int batch_size, int input_size,
+                                             int hidden_size,
+                                             const float* W_t, const float* u, const float* b,
+                                             const float* x_t, const float* h,
+                                             const float* dh_new,
+                                             float* dx, float* dW, float* du, float* db, float* dh,
+                                             float* workspace,
+                                             const float* act_Wx, const float* gamma1,
+                                             float* dgamma1,
+                                             const float* zoneout_mask, void* stream) {
+  (void)b;
+  const int T = steps, N = batch_size, C = input_size, H = hidden_size;
+  HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
+  HASTE_HIP_REQUIRE(W_t && u && x_t && h && dh_new && dx && dW && du && db && dh && workspace);
+  HASTE_HIP_REQUIRE(act_Wx && gamma1 && dgamma1);
+  hipStream_t s = as_stream(stream);
+  HASTE_HIP_PROPAGATE(run_backward_recurrence(s, T, N, H, u, h, dh_new, du, db, dh, workspace,
+                                              zoneout_mask));
+  HASTE_HIP_PROPAGATE(layer_norm_backward(s, T * N, H, gamma1, act_Wx, workspace, workspace,
+                                          dgamma1, nullptr));
+  HASTE_HIP_PROPAGATE(gemm_f32(s, false, C, H, T * N, x_t, T * N, workspace, H, dW, H, false));
+  HASTE_HIP_PROPAGATE(gemm_f32(s, false, T * N, C, H, workspace, H, W_t, C, dx, C, false));
+  return HASTE_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,275 @@
+// Row-wise layer normalisation, forward and backward, one wavefront per row.
+//
+// A row lives in the registers of one 64-lane wavefront for the whole computation;
+// every reduction (mean, variance, the three sums of the backward pass) is a
+// cross-lane butterfly, so a row is read from memory once and nothing is staged in
+// LDS.  The backward pass recomputes mean and 1/std from x instead of reading them
+// back.  The per-column gradients of gamma and beta are accumulated in registers over
+// the rows a wavefront handles, combined per workgroup, parked, and added up in a fixed
+// order by the last workgroup to finish.
+//
+// Arithmetic follows reference lib/layer_norm_forward_gpu.cu.cc:45-87 and
+// lib/layer_norm_backward_gpu.cu.cc:46-92 (eps 1e-5, biased variance).
+#include "recurrent.h"
+
+namespace haste_hip {
+namespace {
+
+constexpr float kEps = 1e-5f;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+// Element e of a lane's register image of a row is column col_of(e); with VEC the
+// lane owns runs of 4 consecutive columns so that loads and stores are 16 bytes.
+template <bool VEC>
+__device__ __forceinline__ int col_of(int e, int lane) {
+  return VEC ? ((lane + 64 * (e >> 2)) * 4 + (e & 3)) : (lane + 64 * e);
+}
+
+template <int E, bool VEC>
+__device__ __forceinline__ void load_row(const float* __restrict__ p, int D, int lane, float (&r)[E]) {
+  if (VEC) {
+#pragma unroll
+    for (int i = 0; i < E / 4; ++i) {
+      const int c = (lane + 64 * i) * 4;
+      float4_t v = {0.f, 0.f, 0.f, 0.f};
+      if (c < D) v = *reinterpret_cast<const float4_t*>(p + c);
+      r[4 * i + 0] = v.x; r[4 * i + 1] = v.y; r[4 * i + 2] = v.z; r[4 * i + 3] = v.w;
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int c = lane + 64 * e;
+      r[e] = c < D ? p[c] : 0.f;
+    }
+  }
+}
+
+template <int E, bool VEC>
+__device__ __forceinline__ void store_row(float* __restrict__ p, int D, int lane, const float (&r)[E]) {
+  if (VEC) {
+#pragma unroll
+    for (int i = 0; i < E / 4; ++i) {
+      const int c = (lane + 64 * i) * 4;
+      if (c < D) {
+        float4_t v = {r[4 * i + 0], r[4 * i + 1], r[4 * i + 2], r[4 * i + 3]};
+        *reinterpret_cast<float4_t*>(p + c) = v;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int c = lane + 64 * e;
+      if (c < D) p[c] = r[e];
+    }
+  }
+}
+
+// mean and 1/sqrt(biased variance + eps) of the row held in r (two-pass, in registers).
+template <int E, bool VEC>
+__device__ __forceinline__ void row_stats(const float (&r)[E], int D, int lane, float& mean, float& invstd) {
+  float s = 0.f;
+#pragma unroll
+  for (int e = 0; e < E; ++e) s += r[e];  // padding elements are zero
+  mean = wave_sum(s) / (float)D;
+  float q = 0.f;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const float d = r[e] - mean;
+    q += (col_of<VEC>(e, lane) < D) ? d * d : 0.f;
+  }
+  invstd = 1.0f / sqrtf(wave_sum(q) / (float)D + kEps);
+}
+
+template <int E, bool VEC>
+__global__ __launch_bounds__(256)
+void layer_norm_forward_kernel(int rows, int D, const float* __restrict__ gamma,
+                               const float* __restrict__ beta, const float* x,
+                               float* y, float* __restrict__ cache) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  float g[E], b[E];
+  load_row<E, VEC>(gamma, D, lane, g);
+  if (beta != nullptr) load_row<E, VEC>(beta, D, lane, b);
+  for (int row = blockIdx.x * 4 + wave; row < rows; row += gridDim.x * 4) {
+    float r[E];
+    load_row<E, VEC>(x + (size_t)row * D, D, lane, r);
+    float mean, invstd;
+    row_stats<E, VEC>(r, D, lane, mean, invstd);
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      float v = (r[e] - mean) * invstd * g[e];
+      if (beta != nullptr) v += b[e];
+      r[e] = v;
+    }
+    store_row<E, VEC>(y + (size_t)row * D, D, lane, r);
+    if (cache != nullptr && lane == 0) {
+      cache[(size_t)row * 2 + 0] = mean;
+      cache[(size_t)row * 2 + 1] = invstd;
+    }
+  }
+}
+
+template <int E, bool VEC>
+__global__ __launch_bounds__(256)
+void layer_norm_backward_kernel(int rows, int D, const float* __restrict__ gamma,
+                                const float* x, const float* dy, float* dx,
+                                float* __restrict__ dgamma, float* __restrict__ dbeta,
+                                float* __restrict__ partial, ControlBlock* cb) {
+  __shared__ unsigned int s_flag;
+  extern __shared__ __attribute__((aligned(16))) float lds[];  // [4][2][E*64]
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  float g[E], dg_acc[E], db_acc[E];
+  load_row<E, VEC>(gamma, D, lane, g);
+#pragma unroll
+  for (int e = 0; e < E; ++e) dg_acc[e] = db_acc[e] = 0.f;
+
+  for (int row = blockIdx.x * 4 + wave; row < rows; row += gridDim.x * 4) {
+    float r[E], d[E];
+    load_row<E, VEC>(x + (size_t)row * D, D, lane, r);
+    load_row<E, VEC>(dy + (size_t)row * D, D, lane, d);
+    float mean, invstd;
+    row_stats<E, VEC>(r, D, lane, mean, invstd);
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const bool in = col_of<VEC>(e, lane) < D;
+      const float xc = in ? r[e] - mean : 0.f;
+      r[e] = xc;
+      const float gdy = g[e] * d[e];
+      dg_acc[e] += xc * invstd * d[e];
+      db_acc[e] += d[e];
+      s0 += xc * gdy;
+      s1 += xc;
+      s2 += gdy;
+    }
+    s0 = wave_sum(s0);
+    s1 = wave_sum(s1);
+    s2 = wave_sum(s2);
+    const float dsigma = -0.5f * s0 * invstd * invstd * invstd;
+    const float dmu = (-2.0f * s1 * dsigma / (float)D) - (s2 * invstd);
+#pragma unroll
+    for (int e = 0; e < E; ++e)
+      r[e] = (2.0f * r[e] * dsigma / (float)D) + (invstd * (g[e] * d[e])) + (dmu / (float)D);
+    store_row<E, VEC>(dx + (size_t)row * D, D, lane, r);
+  }
+
+  // Combine the four wavefronts (fixed order), park the workgroup's column sums.
+  float* mine = lds + wave * 2 * E * 64;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    mine[e * 64 + lane] = dg_acc[e];
+    mine[E * 64 + e * 64 + lane] = db_acc[e];
+  }
+  __syncthreads();
+  float* part = partial + (size_t)blockIdx.x * 2 * D;
+  for (int idx = threadIdx.x; idx < 2 * E * 64; idx += 256) {
+    const int which = idx / (E * 64), rem = idx % (E * 64);
+    const int e = rem / 64, l = rem % 64;
+    const int c = col_of<VEC>(e, l);
+    if (c < D) {
+      const float s = (lds[idx] + lds[2 * E * 64 + idx]) + (lds[4 * E * 64 + idx] + lds[6 * E * 64 + idx]);
+      part[which * D + c] = s;
+    }
+  }
+  if (grid_last_arrival(cb, gridDim.x, &s_flag)) {
+    for (int c = threadIdx.x; c < 2 * D; c += 256) {
+      float s = 0.f;
+      for (int b = 0; b < (int)gridDim.x; ++b) s += partial[(size_t)b * 2 * D + c];
+      if (c < D) dgamma[c] += s;
+      else if (dbeta != nullptr) dbeta[c - D] += s;
+    }
+  }
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Smallest supported register image (elements per lane) covering D columns; 0 if none.
+int elements_per_lane(int D, bool vec) {
+  const int per = vec ? 256 : 64;
+  const int units = (D + per - 1) / per;
+  for (int u : {1, 2, 4, 8, 16}) if (units <= u) return vec ? 4 * u : u;
+  return 0;
+}
+
+}  // namespace
+
+int layer_norm_forward(hipStream_t stream, int rows, int dim, const float* gamma,
+                       const float* beta, const float* x, float* y, float* cache) {
+  HASTE_HIP_REQUIRE(rows > 0 && dim > 0 && gamma && x && y);
+  const bool vec = dim % 4 == 0 && aligned16(gamma) && aligned16(x) && aligned16(y) &&
+                   (beta == nullptr || aligned16(beta));
+  const int E = elements_per_lane(dim, vec);
+  if (E == 0) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  const int cus = device_cu_count();
+  int grid = (rows + 3) / 4;
+  if (grid > 16 * cus) grid = 16 * cus;
+  ScopedKernelTimer timer("layer_norm_forward", stream);
+#define HASTE_LN_FWD(E_, VEC_)                                                            \
+  if (E == E_ && vec == VEC_)                                                             \
+    layer_norm_forward_kernel<E_, VEC_><<<dim3(grid), dim3(256), 0, stream>>>(            \
+        rows, dim, gamma, beta, x, y, cache);
+  HASTE_LN_FWD(4, true) HASTE_LN_FWD(8, true) HASTE_LN_FWD(16, true) HASTE_LN_FWD(32, true)
+  HASTE_LN_FWD(64, true)
+  HASTE_LN_FWD(1, false) HASTE_LN_FWD(2, false) HASTE_LN_FWD(4, false) HASTE_LN_FWD(8, false)
+  HASTE_LN_FWD(16, false)
+#undef HASTE_LN_FWD
+  HASTE_HIP_TRY(hipGetLastError());
+  return HASTE_HIP_OK;
+}
+
+int layer_norm_backward(hipStream_t stream, int rows, int dim, const float* gamma,
+                        const float* x, const float* dy, float* dx, float* dgamma,
+                        float* dbeta) {
+  HASTE_HIP_REQUIRE(rows > 0 && dim > 0 && gamma && x && dy && dx && dgamma);
+  const bool vec = dim % 4 == 0 && aligned16(gamma) && aligned16(x) && aligned16(dy) && aligned16(dx);
+  const int E = elements_per_lane(dim, vec);
+  if (E == 0) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  const int cus = device_cu_count();
+  int grid = (rows + 3) / 4;
+  if (grid > 2 * cus) grid = 2 * cus;
+  Workspace ws;
+  HASTE_HIP_PROPAGATE(get_workspace(stream, (size_t)grid * 2 * dim * sizeof(float), &ws));
+  const size_t lds = (size_t)4 * 2 * E * 64 * sizeof(float);
+  ScopedKernelTimer timer("layer_norm_backward", stream);
+#define HASTE_LN_BWD(E_, VEC_)                                                            \
+  if (E == E_ && vec == VEC_) {                                                           \
+    HASTE_HIP_TRY(hipFuncSetAttribute(                                                    \
+        reinterpret_cast<const void*>(layer_norm_backward_kernel<E_, VEC_>),              \
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                           \
+    layer_norm_backward_kernel<E_, VEC_><<<dim3(grid), dim3(256), lds, stream>>>(         \
+        rows, dim, gamma, x, dy, dx, dgamma, dbeta, ws.scratch, ws.control);              \
+  }
+  HASTE_LN_BWD(4, true) HASTE_LN_BWD(8, true) HASTE_LN_BWD(16, true) HASTE_LN_BWD(32, true)
+  HASTE_LN_BWD(64, true)
+  HASTE_LN_BWD(1, false) HASTE_LN_BWD(2, false) HASTE_LN_BWD(4, false) HASTE_LN_BWD(8, false)
+  HASTE_LN_BWD(16, false)
+#undef HASTE_LN_BWD
+  HASTE_HIP_TRY(hipGetLastError());
+  return HASTE_HIP_OK;
+}
+
+}  // namespace haste_hip
+
+extern "C" {
+
+int haste_hip_layer_norm_forward_f32(int rows, int dim, const float* gamma, const float* beta,
+                                     const float* x, float* y, float* cache, void* stream) {
+  return haste_hip::layer_norm_forward(haste_hip::as_stream(stream), rows, dim, gamma, beta, x, y,
+                                       cache);
+}
+
+int haste_hip_layer_norm_backward_f32(int rows, int dim, const float* gamma, const float* x,
+                                      const float* dy, float* dx, float* dgamma, float* dbeta,
+                                      const float* cache, void* stream) {
+  (void)cache;  // statistics are recomputed from x
+  return haste_hip::layer_norm_backward(haste_hip::as_stream(stream), rows, dim, gamma, x, dy, dx,
+                                        dgamma, dbeta);
+}
+
+}  // extern "C"

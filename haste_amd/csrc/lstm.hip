@@ -24,6 +24,7 @@ struct LstmFwdParams {
   ControlBlock* cb;
   unsigned int* host_status;
   unsigned int spin_limit;
+  unsigned int epoch;
 };
 
 // HS hidden units per workgroup = 4*CT (their 4 gate columns fill CT MFMA column tiles).
@@ -48,7 +49,7 @@ void lstm_forward_kernel(LstmFwdParams p) {
   const size_t NH = (size_t)N * H;
 
   GroupSync gs;
-  group_sync_init(gs, p.cb, blockIdx.y, gridDim.x, p.host_status, p.spin_limit);
+  group_sync_init(gs, p.cb, blockIdx.y, gridDim.x, blockIdx.x, p.epoch, p.host_status, p.spin_limit);
 
   // Resident slice: column c of the slice is gate c/HS, hidden unit j0 + c%HS.
   for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
@@ -143,14 +144,13 @@ void lstm_forward_kernel(LstmFwdParams p) {
         }
         const size_t o = (size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp];
         p.c[o] = c_new;
-        p.h[o] = h_new;
+        store_exchanged(&p.h[o], h_new);
         c_prev[pp] = c_new;
         h_prev[pp] = h_new;
       }
     }
     if (t + 1 < T) group_arrive(gs);  // publishes h[t+1]; also fences `red` reuse
   }
-  group_leave(gs);
 }
 
 struct LstmBwdParams {
@@ -168,6 +168,7 @@ struct LstmBwdParams {
   ControlBlock* cb;
   unsigned int* host_status;
   unsigned int spin_limit;
+  unsigned int epoch;
 };
 
 // A workgroup owns 16 hidden units (HSB) for 16*RT batch rows; its slice of R_t is
@@ -195,7 +196,7 @@ void lstm_backward_kernel(LstmBwdParams p) {
   const size_t NH = (size_t)N * H;
 
   GroupSync gs;
-  group_sync_init(gs, p.cb, blockIdx.y, gridDim.x, p.host_status, p.spin_limit);
+  group_sync_init(gs, p.cb, blockIdx.y, gridDim.x, blockIdx.x, p.epoch, p.host_status, p.spin_limit);
 
   for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
     const int k = idx / NCOLS, cidx = idx % NCOLS;
@@ -274,10 +275,10 @@ void lstm_backward_kernel(LstmBwdParams p) {
         const float dv_f = d_sigmoid_f(gf) * df;
         const float dv_o = d_sigmoid_f(go) * do_;
         float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
-        vt[0] = dv_i;
-        vt[H] = dv_g;
-        vt[2 * H] = dv_f;
-        vt[3 * H] = dv_o;
+        store_exchanged(vt, dv_i);
+        store_exchanged(vt + H, dv_g);
+        store_exchanged(vt + 2 * H, dv_f);
+        store_exchanged(vt + 3 * H, dv_o);
         dbacc[pp][0] += dv_i;
         dbacc[pp][1] += dv_g;
         dbacc[pp][2] += dv_f;
@@ -323,7 +324,6 @@ void lstm_backward_kernel(LstmBwdParams p) {
     for (int r = 0; r < NB; ++r) s += red[(r * 4 + g) * HSB + jj];
     if (j0 + jj < H) p.db_partial[(size_t)blockIdx.y * 4 * H + g * H + j0 + jj] = s;
   }
-  group_leave(gs);
   if (grid_last_arrival(p.cb, gridDim.x * gridDim.y, &s_flag)) {
     for (int col = tid; col < 4 * H; col += 256) {
       float s = 0.f;
@@ -356,6 +356,7 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
   p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
   p.dc_mask = dc_mask; p.dc_scale = dc_scale;
   p.cb = ws.control; p.host_status = ws.host_status_dev; p.spin_limit = kSpinLimit;
+  HASTE_HIP_PROPAGATE(reserve_epochs(stream, (unsigned)T + 1, &p.epoch));
 
   const int cus = device_cu_count();
   // Candidates in order of preference: fewer rows per workgroup first (more CUs busy).
@@ -364,7 +365,7 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
   for (const Cand& cd : cands) {
     const int HS = 4 * cd.ct, NB = 16 * cd.rt;
     const int gx = (H + HS - 1) / HS, gy = (N + NB - 1) / NB;
-    if (gy > kMaxGroups || (long long)gx * gy > cus) continue;
+    if (gy > kMaxGroups || (long long)gx * gy > cus || gx * gy > kMaxWorkgroups) continue;
     const size_t lds = fwd_lds_bytes(H, cd.rt, cd.ct);
     if (lds > kMaxLdsBytes) continue;
     dim3 grid(gx, gy);
@@ -411,6 +412,7 @@ int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   p.db = db; p.dh = dh; p.dc = dc; p.v = v; p.zoneout_mask = zoneout_mask;
   p.db_partial = ws.scratch;
   p.cb = ws.control; p.host_status = ws.host_status_dev; p.spin_limit = kSpinLimit;
+  HASTE_HIP_PROPAGATE(reserve_epochs(stream, (unsigned)T + 1, &p.epoch));
   const size_t lds = bwd_lds_bytes(4 * H, rt);
   dim3 grid(gx, gy);
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;

@@ -24,78 +24,100 @@ __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf
 __device__ __forceinline__ float d_sigmoid_f(float y) { return y * (1.0f - y); }
 __device__ __forceinline__ float d_tanh_f(float y) { return 1.0f - y * y; }
 
-// Per-workgroup view of its group's step barrier.
+// ---- Exchange between workgroups inside one launch --------------------------------
+// The 8 XCDs of the chip have separate L2 caches, so data one workgroup writes and
+// another reads in the same launch must not rest in an L2.  Such data is written and
+// read with agent-scope accesses (the sc1 forms of global_store / global_load, which
+// go to the memory side), and everything else uses ordinary cached accesses: no
+// cache-wide write-back or invalidate is needed at a step boundary.
+__device__ __forceinline__ void store_exchanged(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_exchanged(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// 16-byte aligned p.
+__device__ __forceinline__ float4_t load_exchanged4(const float* p) {
+  const unsigned long long* q = reinterpret_cast<const unsigned long long*>(p);
+  const unsigned long long lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const unsigned long long hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  float4_t v;
+  v.x = __uint_as_float((unsigned int)lo);
+  v.y = __uint_as_float((unsigned int)(lo >> 32));
+  v.z = __uint_as_float((unsigned int)hi);
+  v.w = __uint_as_float((unsigned int)(hi >> 32));
+  return v;
+}
+
+// Per-workgroup view of its group's step barrier: one flag word per workgroup holding
+// the number of arrivals it has made (offset by a per-launch epoch so that the words
+// never need clearing).  Arriving is one store; waiting is one wavefront reading the
+// group's flags side by side, so no read-modify-write traffic is serialised.
 struct GroupSync {
-  unsigned int* counter;       // arrivals so far (monotonic within a launch)
-  unsigned int* exit_counter;  // workgroups of the group that have left the time loop
+  unsigned int* flags;         // this group's flag words, one per workgroup
   unsigned int* abort_flag;    // device-wide: some wait gave up
   unsigned int* host_status;   // pinned host word mirrored from abort_flag
   unsigned int group_size;
-  unsigned int arrivals;       // barriers this workgroup has arrived at
+  unsigned int my_index;
+  unsigned int epoch;          // value of the flags after `arrivals` arrivals is epoch + arrivals
+  unsigned int arrivals;
   unsigned int spin_limit;
 };
 
-__device__ __forceinline__ void group_sync_init(GroupSync& g, ControlBlock* cb, int group,
-                                                unsigned int group_size,
-                                                unsigned int* host_status,
+__device__ __forceinline__ void group_sync_init(GroupSync& g, ControlBlock* cb, unsigned int group,
+                                                unsigned int group_size, unsigned int my_index,
+                                                unsigned int epoch, unsigned int* host_status,
                                                 unsigned int spin_limit) {
-  g.counter = &cb->step_counter[group * kCounterStride];
-  g.exit_counter = &cb->exit_counter[group * kCounterStride];
+  g.flags = &cb->step_flags[group * group_size];
   g.abort_flag = &cb->abort_flag[0];
   g.host_status = host_status;
   g.group_size = group_size;
+  g.my_index = my_index;
+  g.epoch = epoch;
   g.arrivals = 0;
   g.spin_limit = spin_limit;
 }
 
-// Publishes every global store this workgroup has made so far to the rest of the
-// group and counts the workgroup as arrived.  Called by all threads.
+// Counts the workgroup as arrived once every exchanged store its threads have issued
+// has completed.  Called by all threads.
 __device__ __forceinline__ void group_arrive(GroupSync& g) {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  if (threadIdx.x == 0) {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-    __hip_atomic_fetch_add(g.counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
   g.arrivals += 1;
+  if (threadIdx.x == 0)
+    __hip_atomic_store(&g.flags[g.my_index], g.epoch + g.arrivals, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Blocks until every workgroup of the group has made as many arrivals as this one.
 // The wait is bounded: after spin_limit polls (or when another workgroup has given
 // up) it raises the abort flag and returns, so that every wavefront still reaches the
-// end of the kernel.  Called by all threads.
+// end of the kernel.  Called by all threads; exchanged loads may follow directly.
 __device__ __forceinline__ void group_wait(GroupSync& g) {
-  if (threadIdx.x == 0) {
-    const unsigned int target = g.arrivals * g.group_size;
+  if (threadIdx.x < 64) {
+    const unsigned int target = g.epoch + g.arrivals;
     unsigned int spins = 0;
-    while (__hip_atomic_load(g.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+    for (;;) {
+      bool ok = true;
+      for (unsigned int i = threadIdx.x; i < g.group_size; i += 64) {
+        const unsigned int f =
+            __hip_atomic_load(&g.flags[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ok = ok && (int)(f - target) >= 0;
+      }
+      if (__all(ok)) break;
       __builtin_amdgcn_s_sleep(1);
       ++spins;
       if ((spins & 255u) == 0u) {
-        if (__hip_atomic_load(g.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) break;
-        if (spins >= g.spin_limit) {
+        unsigned int ab = __hip_atomic_load(g.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (spins >= g.spin_limit && threadIdx.x == 0) {
           __hip_atomic_store(g.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           __hip_atomic_store(g.host_status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-          break;
         }
+        if (ab != 0u || spins >= g.spin_limit) break;
       }
     }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   }
   __syncthreads();
-}
-
-// Leaves the group: the last workgroup out puts the group's counters back to zero so
-// that the next launch on this stream finds the control block clean.
-__device__ __forceinline__ void group_leave(GroupSync& g) {
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    const unsigned int old =
-        __hip_atomic_fetch_add(g.exit_counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (old == g.group_size - 1) {
-      __hip_atomic_store(g.counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(g.exit_counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-  }
 }
 
 // True in exactly one workgroup of the launch: the last to call it.  Stores made by
@@ -129,15 +151,16 @@ __device__ __forceinline__ int slice_index(int k, int col, int ncols) {
   return ((((k >> 4) << 2) + ((k & 15) >> 2)) * ncols + col) * 4 + (k & 3);
 }
 
+// Guarded 4-float read of exchanged data: elements beyond `valid` read as zero.
 __device__ __forceinline__ float4_t load_a4(const float* p, int valid, bool vec_ok) {
   float4_t v = {0.f, 0.f, 0.f, 0.f};
   if (valid >= 4 && vec_ok) {
-    v = *reinterpret_cast<const float4_t*>(p);
+    v = load_exchanged4(p);
   } else {
-    if (valid > 0) v.x = p[0];
-    if (valid > 1) v.y = p[1];
-    if (valid > 2) v.z = p[2];
-    if (valid > 3) v.w = p[3];
+    if (valid > 0) v.x = load_exchanged(p);
+    if (valid > 1) v.y = load_exchanged(p + 1);
+    if (valid > 2) v.z = load_exchanged(p + 2);
+    if (valid > 3) v.w = load_exchanged(p + 3);
   }
   return v;
 }

@@ -116,6 +116,17 @@ int get_workspace(hipStream_t stream, size_t scratch_bytes, Workspace* out) {
   return HASTE_HIP_OK;
 }
 
+int reserve_epochs(hipStream_t stream, unsigned int count, unsigned int* base) {
+  int dev = 0;
+  HASTE_HIP_TRY(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_mutex);
+  auto it = g_workspaces.find(Key{dev, stream});
+  if (it == g_workspaces.end()) return HASTE_HIP_ERROR_INVALID_ARGUMENT;
+  *base = it->second.epoch;
+  it->second.epoch += count;
+  return HASTE_HIP_OK;
+}
+
 int check_and_clear_abort(hipStream_t stream, Workspace* ws) {
   volatile unsigned int* status = ws->host_status;
   if (status == nullptr || *status == 0u) return HASTE_HIP_OK;

@@ -81,3 +81,141 @@ def lstm_backward(x_t, kernel_t, recurrent_kernel_t, bias, zoneout_mask, h, c, c
              h, c, dh_new, dc_new, dx, dW, dR, db, dh, dc, cache,
              _mask_or_none(has_zoneout, zoneout_mask))
     return dx, dh, dc, dW, dR, db
+
+
+# ---- GRU (reference frameworks/pytorch/gru.cc:30-163) -----------------------
+def gru_forward(training, zoneout_prob, x, h0, kernel, recurrent_kernel, bias, recurrent_bias,
+                zoneout_mask, dropconnect_mask=None, dropconnect_scale=1.0):
+    T, N, C = x.shape
+    H = recurrent_kernel.shape[0]
+    has_zoneout = bool(zoneout_prob) and zoneout_mask.numel() > 0
+    _check(x, h0, kernel, recurrent_kernel, bias, recurrent_bias, zoneout_mask)
+    opts = dict(device=x.device, dtype=x.dtype)
+    output = torch.empty(T + 1, N, H, **opts)
+    cache = torch.empty(T, N, 4 * H, **opts)
+    tmp_Wx = torch.empty(T, N, 3 * H, **opts)
+    output[0] = h0
+    zp = float(zoneout_prob) if has_zoneout else 0.0
+    mask = _mask_or_none(has_zoneout, zoneout_mask)
+    if dropconnect_mask is None:
+        lib.call("haste_hip_gru_forward_f32", bool(training), T, N, C, H, kernel, recurrent_kernel,
+                 bias, recurrent_bias, x, output, cache if training else None, tmp_Wx, None, zp, mask)
+    else:
+        _check(dropconnect_mask)
+        lib.call("haste_hip_gru_forward_dropconnect_f32", bool(training), T, N, C, H, kernel,
+                 recurrent_kernel, bias, recurrent_bias, x, output, cache if training else None,
+                 tmp_Wx, zp, mask, dropconnect_mask, float(dropconnect_scale))
+    return output, cache
+
+
+def gru_backward(x_t, kernel_t, recurrent_kernel_t, bias, recurrent_bias, zoneout_mask, h, cache,
+                 dh_new):
+    C, T, N = x_t.shape
+    H = recurrent_kernel_t.shape[1]
+    has_zoneout = zoneout_mask.numel() > 0
+    _check(x_t, kernel_t, recurrent_kernel_t, bias, recurrent_bias, zoneout_mask, h, cache, dh_new)
+    opts = dict(device=x_t.device, dtype=x_t.dtype)
+    dx = torch.empty(T, N, C, **opts)
+    dW = torch.zeros(C, 3 * H, **opts)
+    dR = torch.zeros(H, 3 * H, **opts)
+    dbx = torch.zeros(3 * H, **opts)
+    dbr = torch.zeros(3 * H, **opts)
+    dh = torch.zeros(N, H, **opts)
+    dp = torch.empty(T, N, 3 * H, **opts)
+    dq = torch.empty(T, N, 3 * H, **opts)
+    lib.call("haste_hip_gru_backward_f32", T, N, C, H, kernel_t, recurrent_kernel_t, bias,
+             recurrent_bias, x_t, h, cache, dh_new, dx, dW, dR, dbx, dbr, dh, dp, dq,
+             _mask_or_none(has_zoneout, zoneout_mask))
+    return dx, dh, dW, dR, dbx, dbr
+
+
+# ---- Layer norm (reference lib/haste/layer_norm.h) ---------------------------
+def layer_norm_forward(x, gamma, beta=None):
+    _check(x, gamma)
+    rows, dim = x.numel() // x.shape[-1], x.shape[-1]
+    y = torch.empty_like(x)
+    cache = torch.empty(rows, 2, device=x.device, dtype=x.dtype)
+    lib.call("haste_hip_layer_norm_forward_f32", rows, dim, gamma, beta, x, y, cache)
+    return y, cache
+
+
+def layer_norm_backward(x, gamma, dy, cache=None, with_beta=True, in_place=False):
+    _check(x, gamma, dy)
+    rows, dim = x.numel() // x.shape[-1], x.shape[-1]
+    dx = dy if in_place else torch.empty_like(x)
+    dgamma = torch.zeros_like(gamma)
+    dbeta = torch.zeros_like(gamma) if with_beta else None
+    lib.call("haste_hip_layer_norm_backward_f32", rows, dim, gamma, x, dy, dx, dgamma, dbeta, cache)
+    return dx, dgamma, dbeta
+
+
+# ---- IndRNN (reference frameworks/pytorch/indrnn.cc:30-140) -------------------
+def indrnn_forward(training, zoneout_prob, x, h0, kernel, recurrent_scale, bias, zoneout_mask):
+    T, N, C = x.shape
+    H = recurrent_scale.shape[0]
+    has_zoneout = bool(zoneout_prob) and zoneout_mask.numel() > 0
+    _check(x, h0, kernel, recurrent_scale, bias, zoneout_mask)
+    opts = dict(device=x.device, dtype=x.dtype)
+    output = torch.empty(T + 1, N, H, **opts)
+    workspace = torch.empty(T, N, H, **opts)
+    output[0] = h0
+    lib.call("haste_hip_indrnn_forward_f32", bool(training), T, N, C, H, kernel, recurrent_scale,
+             bias, x, output, workspace, float(zoneout_prob) if has_zoneout else 0.0,
+             _mask_or_none(has_zoneout, zoneout_mask))
+    return output
+
+
+def indrnn_backward(x_t, kernel_t, recurrent_scale, bias, zoneout_mask, h, dh_new):
+    C, T, N = x_t.shape
+    H = recurrent_scale.shape[0]
+    has_zoneout = zoneout_mask.numel() > 0
+    _check(x_t, kernel_t, recurrent_scale, bias, zoneout_mask, h, dh_new)
+    opts = dict(device=x_t.device, dtype=x_t.dtype)
+    dx = torch.empty(T, N, C, **opts)
+    dW = torch.zeros(C, H, **opts)
+    du = torch.zeros(H, **opts)
+    db = torch.zeros_like(bias)
+    dh = torch.zeros(N, H, **opts)
+    workspace = torch.empty(T, N, H, **opts)
+    lib.call("haste_hip_indrnn_backward_f32", T, N, C, H, kernel_t, recurrent_scale, bias, x_t, h,
+             dh_new, dx, dW, du, db, dh, workspace, _mask_or_none(has_zoneout, zoneout_mask))
+    return dx, dh, dW, du, db
+
+
+# ---- LayerNorm IndRNN (reference frameworks/pytorch/layer_norm_indrnn.cc:31-174) ----
+def layer_norm_indrnn_forward(training, zoneout_prob, x, h0, kernel, recurrent_scale, bias, gamma,
+                              zoneout_mask):
+    T, N, C = x.shape
+    H = recurrent_scale.shape[0]
+    has_zoneout = bool(zoneout_prob) and zoneout_mask.numel() > 0
+    _check(x, h0, kernel, recurrent_scale, bias, gamma, zoneout_mask)
+    opts = dict(device=x.device, dtype=x.dtype)
+    output = torch.empty(T + 1, N, H, **opts)
+    workspace = torch.empty(T, N, H, **opts)
+    act_Wx = torch.empty(T, N, H, **opts)
+    act_Wx_norm_cache = torch.empty(T, N, 2, **opts)
+    output[0] = h0
+    lib.call("haste_hip_layer_norm_indrnn_forward_f32", bool(training), T, N, C, H, kernel,
+             recurrent_scale, bias, x, output, workspace, act_Wx, gamma[0], act_Wx_norm_cache,
+             float(zoneout_prob) if has_zoneout else 0.0, _mask_or_none(has_zoneout, zoneout_mask))
+    return output, act_Wx, act_Wx_norm_cache
+
+
+def layer_norm_indrnn_backward(x_t, kernel_t, recurrent_scale, bias, gamma, zoneout_mask, h, act_Wx,
+                               act_Wx_norm_cache, dh_new):
+    C, T, N = x_t.shape
+    H = recurrent_scale.shape[0]
+    has_zoneout = zoneout_mask.numel() > 0
+    _check(x_t, kernel_t, recurrent_scale, bias, gamma, zoneout_mask, h, act_Wx, dh_new)
+    opts = dict(device=x_t.device, dtype=x_t.dtype)
+    dx = torch.empty(T, N, C, **opts)
+    dW = torch.zeros(C, H, **opts)
+    du = torch.zeros(H, **opts)
+    db = torch.zeros_like(bias)
+    dh = torch.zeros(N, H, **opts)
+    workspace = torch.empty(T, N, H, **opts)
+    dgamma = torch.zeros_like(gamma)
+    lib.call("haste_hip_layer_norm_indrnn_backward_f32", T, N, C, H, kernel_t, recurrent_scale, bias,
+             x_t, h, dh_new, dx, dW, du, db, dh, workspace, act_Wx, gamma[0], dgamma[0],
+             _mask_or_none(has_zoneout, zoneout_mask))
+    return dx, dh, dW, du, db, dgamma

@@ -1,0 +1,65 @@
+"""GRU forward/backward on the GPU (through the C-ABI) vs the fp64 oracle."""
+import numpy as np
+import pytest
+
+from oracle import haste_oracle as O
+from util import TOL, dev, host, problem, relerr
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(1, 1, 1, 1), (3, 2, 3, 4), (5, 3, 7, 5), (6, 17, 20, 36), (4, 16, 32, 64),
+          (10, 33, 48, 128), (8, 64, 64, 256), (6, 128, 96, 512)]
+
+
+@pytest.mark.parametrize("zoneout", [0.0, 0.3])
+@pytest.mark.parametrize("T,N,C,H", SHAPES)
+def test_gru_training_forward_backward(T, N, C, H, zoneout):
+    from haste_amd import ops
+    import torch
+    print("gru fwd+bwd", T, N, C, H, zoneout, flush=True)
+    p = problem(200 + T + N + C + H, T, N, C, H, 3, zoneout)
+    mask = dev(p["mask"])
+    h, cache = ops.gru_forward(True, zoneout, dev(p["x"]), dev(p["h0"]), dev(p["W"]), dev(p["R"]),
+                               dev(p["b"]), dev(p["b2"]), mask)
+    torch.cuda.synchronize()
+    ho, vo = O.gru_forward(p["W"], p["R"], p["b"], p["b2"], p["x"], p["h0"], True, zoneout, p["mask"])
+    assert relerr(host(h), ho) < TOL
+    assert relerr(host(cache), vo) < TOL
+    x_t = dev(p["x"]).permute(2, 0, 1).contiguous()
+    outs = ops.gru_backward(x_t, dev(p["W"]).t().contiguous(), dev(p["R"]).t().contiguous(),
+                            dev(p["b"]), dev(p["b2"]), mask, h, cache, dev(p["dh_new"]))
+    torch.cuda.synchronize()
+    dx, dW, dR, dbx, dbr, dh0, _, _ = O.gru_backward(p["W"], p["R"], p["b"], p["b2"], p["x"], ho, vo,
+                                                     p["dh_new"], p["mask"])
+    for name, ours, theirs in zip(("dx", "dh0", "dW", "dR", "dbx", "dbr"), outs,
+                                  (dx, dh0, dW, dR, dbx, dbr)):
+        assert relerr(host(ours), theirs) < TOL, name
+
+
+@pytest.mark.parametrize("zoneout", [0.0, 0.25])
+def test_gru_inference_forward(zoneout):
+    from haste_amd import ops
+    import torch
+    T, N, C, H = 20, 16, 128, 256
+    p = problem(8, T, N, C, H, 3, zoneout)
+    h, _ = ops.gru_forward(False, zoneout, dev(p["x"]), dev(p["h0"]), dev(p["W"]), dev(p["R"]),
+                           dev(p["b"]), dev(p["b2"]), dev(p["mask"]))
+    torch.cuda.synchronize()
+    ho, _ = O.gru_forward(p["W"], p["R"], p["b"], p["b2"], p["x"], p["h0"], False, zoneout, p["mask"])
+    assert relerr(host(h), ho) < TOL
+
+
+def test_gru_dropconnect_fused_equals_premasked_weights():
+    from haste_amd import ops
+    import torch
+    T, N, C, H = 6, 8, 16, 64
+    p = problem(9, T, N, C, H, 3)
+    m = (np.random.default_rng(3).uniform(size=p["R"].shape) >= 0.05).astype(np.float64)
+    scale = 1.0 / 0.95
+    args = (True, 0.0, dev(p["x"]), dev(p["h0"]), dev(p["W"]))
+    h1, v1 = ops.gru_forward(*args, dev(p["R"]), dev(p["b"]), dev(p["b2"]), dev(None),
+                             dropconnect_mask=dev(m), dropconnect_scale=scale)
+    R_eff = ((dev(p["R"]) * dev(m)) * np.float32(scale)).contiguous()
+    h2, v2 = ops.gru_forward(*args, R_eff, dev(p["b"]), dev(p["b2"]), dev(None))
+    torch.cuda.synchronize()
+    assert torch.equal(h1, h2) and torch.equal(v1, v2)
