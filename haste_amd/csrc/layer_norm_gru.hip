@@ -1,0 +1,548 @@
+// LayerNormGRU forward and backward passes.
+//
+// Forward: GEMM x*W, stand-alone layer norm over all T*N rows, then one persistent
+// kernel in which the per-step layer norm of h*R (3H columns) is computed inside the
+// step through a per-row moment exchange (two group barriers per step).  Backward
+// mirrors it in reverse time, then a stand-alone layer-norm backward and three GEMMs.
+//
+// Arithmetic follows reference lib/layer_norm_gru_forward_gpu.cu.cc:25-83 and
+// lib/layer_norm_gru_backward_gpu.cu.cc:25-95; orchestration replaces :242-305 and :219-310.
+#include "ln_exchange.h"
+
+namespace haste_hip {
+namespace {
+
+struct LnGruFwdParams {
+  int training, T, N, H;
+  const float* R;        // [H,3H]
+  const float* bx;       // [3H]
+  const float* br;       // [3H]
+  float* h;              // [T+1,N,H]
+  float* v;              // [T,N,4H] or null
+  const float* Wxn;      // [T,N,3H] LN1(x*W)
+  float* act_Rh;         // [T,N,3H] out
+  const float* gamma2;   // [3H]
+  float* cache2;         // [T*N,2] or null
+  float zoneout_prob;
+  const float* zoneout_mask;
+  float* part2;          // exchange [groups][gx][NB][2]
+  ControlBlock* cb;
+  unsigned int* host_status;
+  unsigned int spin_limit;
+  unsigned int epoch;
+};
+
+template <int RT, int CT, int HS>
+__global__ __launch_bounds__(256, 1)
+void ln_gru_forward_kernel(LnGruFwdParams p) {
+  static_assert(3 * HS <= 16 * CT, "slice too narrow");
+  constexpr int NB = 16 * RT;
+  constexpr int NCOLS = 16 * CT;
+  constexpr int PP = (NB * HS + 255) / 256;
+  constexpr int CHUNK = RT == 4 ? 4 : 8;
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+
+  const int H = p.H, N = p.N, T = p.T;
+  const int Kpad = round_up(H, 64);
+  float* w_lds = lds;
+  float* red = lds + Kpad * NCOLS;
+  float* stat = red + 4 * NB * NCOLS;
+
+  const int tid = threadIdx.x;
+  const int gx = gridDim.x;
+  const int j0 = blockIdx.x * HS;
+  const int n0 = blockIdx.y * NB;
+  const size_t NH = (size_t)N * H;
+  const int own_units = (H - j0) < HS ? (H - j0) : HS;
+  const int last_units = H - (gx - 1) * HS;
+  float* part2 = p.part2 + (size_t)blockIdx.y * gx * NB * 2;
+
+  GroupSync gs;
+  group_sync_init(gs, p.cb, blockIdx.y, gx, blockIdx.x, p.epoch, p.host_status, p.spin_limit);
+
+  for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
+    const int k = idx / NCOLS, cidx = idx % NCOLS;
+    const int gate = cidx / HS, j = j0 + cidx % HS;
+    float w = 0.f;
+    if (k < H && gate < 3 && j < H) w = p.R[(size_t)k * 3 * H + gate * H + j];
+    w_lds[slice_index(k, cidx, NCOLS)] = w;
+  }
+
+  int pn[PP], pj[PP], pl[PP], pc[PP];
+  bool act[PP], colok[PP];
+  float h_prev[PP], bxv[PP][3], brv[PP][3], g2[PP][3];
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp) {
+    const int idx = tid + 256 * pp;
+    pl[pp] = idx / HS;
+    pc[pp] = idx % HS;
+    pn[pp] = n0 + pl[pp];
+    pj[pp] = j0 + pc[pp];
+    colok[pp] = idx < NB * HS && pj[pp] < H;
+    act[pp] = colok[pp] && pn[pp] < N;
+    h_prev[pp] = act[pp] ? p.h[(size_t)pn[pp] * H + pj[pp]] : 0.f;
+#pragma unroll
+    for (int g = 0; g < 3; ++g) {
+      bxv[pp][g] = colok[pp] ? p.bx[g * H + pj[pp]] : 0.f;
+      brv[pp][g] = colok[pp] ? p.br[g * H + pj[pp]] : 0.f;
+      g2[pp][g] = colok[pp] ? p.gamma2[g * H + pj[pp]] : 0.f;
+    }
+  }
+  const bool zoneout = p.zoneout_prob != 0.f && p.zoneout_mask != nullptr;
+  const bool vec_ok = (H % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.h) & 15u) == 0);
+  __syncthreads();
+
+  for (int t = 0; t < T; ++t) {
+    float wx[PP][3], mk[PP];
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      mk[pp] = 1.f;
+#pragma unroll
+      for (int g = 0; g < 3; ++g) wx[pp][g] = 0.f;
+      if (act[pp]) {
+        const float* wt = p.Wxn + ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 3; ++g) wx[pp][g] = wt[g * H];
+        if (zoneout && p.training) mk[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
+      }
+    }
+    if (t > 0) group_wait(gs);
+
+    float4_t acc[RT][CT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
+    slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, N - n0, H, Kpad, w_lds,
+                                vec_ok, acc);
+    store_partials<RT, CT>(red, acc);
+    __syncthreads();
+
+    float rh[PP][3];
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      float s = 0.f;
+#pragma unroll
+      for (int g = 0; g < 3; ++g) {
+        rh[pp][g] = colok[pp] ? sum_partials<RT, CT>(red, pl[pp], g * HS + pc[pp]) : 0.f;
+        s += rh[pp][g];
+      }
+      if (act[pp]) {
+        float* ar = p.act_Rh + ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 3; ++g) ar[g * H] = rh[pp][g];
+      }
+      const float mean = segment_sum<HS>(s) / (3.0f * (float)own_units);
+      float q = 0.f;
+#pragma unroll
+      for (int g = 0; g < 3; ++g) {
+        const float d = rh[pp][g] - mean;
+        q += colok[pp] ? d * d : 0.f;
+      }
+      q = segment_sum<HS>(q);
+      if (pc[pp] == 0 && tid + 256 * pp < NB * HS)
+        store_exchanged2(part2 + ((size_t)blockIdx.x * NB + pl[pp]) * 2, mean, q);
+    }
+    group_arrive(gs);
+    group_wait(gs);
+    merge_row_moments<NB>(part2, gx, 3.0f * HS, 3.0f * last_units, 3.0f * H, stat);
+    __syncthreads();
+
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      if (act[pp]) {
+        const float mu = stat[pl[pp] * 2], is = stat[pl[pp] * 2 + 1];
+        float rn[3];
+#pragma unroll
+        for (int g = 0; g < 3; ++g) rn[g] = (rh[pp][g] - mu) * is * g2[pp][g];
+        const float z = sigmoid_f(wx[pp][0] + rn[0] + bxv[pp][0] + brv[pp][0]);
+        const float r = sigmoid_f(wx[pp][1] + rn[1] + bxv[pp][1] + brv[pp][1]);
+        const float qg = rn[2] + brv[pp][2];
+        const float g = tanhf(wx[pp][2] + r * qg + bxv[pp][2]);
+        if (p.training) {
+          float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+          vt[0] = z;
+          vt[H] = r;
+          vt[2 * H] = g;
+          vt[3 * H] = qg;
+        }
+        float h_new = z * h_prev[pp] + (1.0f - z) * g;
+        if (zoneout) {
+          if (p.training) h_new = (h_new - h_prev[pp]) * mk[pp] + h_prev[pp];
+          else h_new = p.zoneout_prob * h_prev[pp] + (1.0f - p.zoneout_prob) * h_new;
+        }
+        store_exchanged(&p.h[(size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp]], h_new);
+        h_prev[pp] = h_new;
+        if (blockIdx.x == 0 && pc[pp] == 0 && p.cache2 != nullptr) {
+          p.cache2[((size_t)t * N + pn[pp]) * 2 + 0] = mu;
+          p.cache2[((size_t)t * N + pn[pp]) * 2 + 1] = is;
+        }
+      }
+    }
+    if (t + 1 < T) group_arrive(gs);
+    else __syncthreads();
+  }
+}
+
+struct LnGruBwdParams {
+  int T, N, H;
+  const float* R_t;      // [3H,H]
+  const float* h;        // [T+1,N,H]
+  const float* v;        // [T,N,4H]
+  const float* dh_new;   // [T+1,N,H]
+  float* dbx;            // [3H]
+  float* dbr;            // [3H]
+  float* dh;             // [N,H]
+  float* dp;             // [T,N,3H]
+  float* dq;             // [T,N,3H] out: gradient w.r.t. h*R before its norm
+  const float* act_Rh;   // [T,N,3H]
+  const float* gamma2;   // [3H]
+  float* dgamma2;        // [3H]
+  const float* cache2;   // [T*N,2]
+  const float* zoneout_mask;
+  float* part;           // exchange [groups][gx][NB][4]
+  float* col_partial;    // [batch tiles][9][H]
+  ControlBlock* cb;
+  unsigned int* host_status;
+  unsigned int spin_limit;
+  unsigned int epoch;
+};
+
+template <int RT>
+__global__ __launch_bounds__(256, 1)
+void ln_gru_backward_kernel(LnGruBwdParams p) {
+  constexpr int HSB = 16;
+  constexpr int NB = 16 * RT;
+  constexpr int NCOLS = 16;
+  constexpr int PP = RT;
+  constexpr int CHUNK = RT == 1 ? 16 : (RT == 2 ? 8 : 4);
+  constexpr int NACC = 9;  // dbx x3, dbr x3, dgamma2 x3
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  __shared__ unsigned int s_flag;
+
+  const int H = p.H, N = p.N, T = p.T;
+  const int K = 3 * H;
+  const int Kpad = round_up(K, 64);
+  float* w_lds = lds;
+  float* red = lds + Kpad * NCOLS;
+  float* sums = red + NB * NACC * HSB;
+
+  const int tid = threadIdx.x;
+  const int gx = gridDim.x;
+  const int j0 = blockIdx.x * HSB;
+  const int n0 = blockIdx.y * NB;
+  const size_t NH = (size_t)N * H;
+  float* part = p.part + (size_t)blockIdx.y * gx * NB * 4;
+
+  GroupSync gs;
+  group_sync_init(gs, p.cb, blockIdx.y, gx, blockIdx.x, p.epoch, p.host_status, p.spin_limit);
+
+  for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
+    const int k = idx / NCOLS, cidx = idx % NCOLS;
+    float w = 0.f;
+    if (k < K && j0 + cidx < H) w = p.R_t[(size_t)k * H + j0 + cidx];
+    w_lds[slice_index(k, cidx, NCOLS)] = w;
+  }
+
+  int pn[PP], pj[PP], pl[PP], pc[PP];
+  bool act[PP];
+  float dh[PP], accs[PP][NACC], g2[PP][3];
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp) {
+    const int idx = tid + 256 * pp;
+    pl[pp] = idx / HSB;
+    pc[pp] = idx % HSB;
+    pn[pp] = n0 + pl[pp];
+    pj[pp] = j0 + pc[pp];
+    act[pp] = pn[pp] < N && pj[pp] < H;
+    dh[pp] = act[pp] ? p.dh[(size_t)pn[pp] * H + pj[pp]] : 0.f;
+#pragma unroll
+    for (int g = 0; g < 3; ++g) g2[pp][g] = pj[pp] < H ? p.gamma2[g * H + pj[pp]] : 0.f;
+#pragma unroll
+    for (int a = 0; a < NACC; ++a) accs[pp][a] = 0.f;
+  }
+  const bool zoneout = p.zoneout_mask != nullptr;
+  const bool vec_ok = (reinterpret_cast<uintptr_t>(p.dq) & 15u) == 0 && (K % 4 == 0);
+  __syncthreads();
+
+  struct StepIn { float vt[4], rh[3], h0, dhn, m, mu2, is2; };
+  StepIn nxt[PP];
+  auto fetch = [&](int t) {
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      StepIn s = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f}, 0.f, 0.f, 1.f, 0.f, 0.f};
+      if (act[pp] && t >= 0) {
+        const size_t e = (size_t)pn[pp] * H + pj[pp];
+        const float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+        const float* ar = p.act_Rh + ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) s.vt[g] = vt[(size_t)g * H];
+#pragma unroll
+        for (int g = 0; g < 3; ++g) s.rh[g] = ar[(size_t)g * H];
+        s.h0 = p.h[(size_t)t * NH + e];
+        s.dhn = p.dh_new[(size_t)(t + 1) * NH + e];
+        if (zoneout) s.m = p.zoneout_mask[(size_t)t * NH + e];
+        s.mu2 = p.cache2[((size_t)t * N + pn[pp]) * 2];
+        s.is2 = p.cache2[((size_t)t * N + pn[pp]) * 2 + 1];
+      }
+      nxt[pp] = s;
+    }
+  };
+  fetch(T - 1);
+
+  const float inv3H = 1.0f / (float)(3 * H);
+  for (int t = T - 1; t >= 0; --t) {
+    StepIn s[PP];
+    float dh_keep[PP], xc[PP][3], gd[PP][3];
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      s[pp] = nxt[pp];
+      dh_keep[pp] = 0.f;
+      float t0 = 0.f, t1 = 0.f, t2 = 0.f;
+#pragma unroll
+      for (int g = 0; g < 3; ++g) xc[pp][g] = gd[pp][g] = 0.f;
+      if (act[pp]) {
+        const float z = s[pp].vt[0], r = s[pp].vt[1], g = s[pp].vt[2], qg = s[pp].vt[3];
+        float dh_total = s[pp].dhn + dh[pp];
+        if (zoneout) {
+          dh_keep[pp] = (1.0f - s[pp].m) * dh_total;
+          dh_total = s[pp].m * dh_total;
+          dh_keep[pp] += z * dh_total;
+        } else {
+          dh_keep[pp] = z * dh_total;
+        }
+        const float dg = (1.0f - z) * dh_total;
+        const float dz = (s[pp].h0 - g) * dh_total;
+        const float dp_g = d_tanh_f(g) * dg;
+        const float dq_g = dp_g * r;
+        const float dr = dp_g * qg;
+        const float dp_r = d_sigmoid_f(r) * dr;
+        const float dp_z = d_sigmoid_f(z) * dz;
+        const size_t o3 = ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
+        p.dp[o3] = dp_z;
+        p.dp[o3 + H] = dp_r;
+        p.dp[o3 + 2 * H] = dp_g;
+        const float dqv[3] = {dp_z, dp_r, dq_g};
+        accs[pp][0] += dp_z;
+        accs[pp][1] += dp_r;
+        accs[pp][2] += dp_g;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+          accs[pp][3 + k] += dqv[k];
+          xc[pp][k] = s[pp].rh[k] - s[pp].mu2;
+          gd[pp][k] = g2[pp][k] * dqv[k];
+          accs[pp][6 + k] += xc[pp][k] * s[pp].is2 * dqv[k];
+          t0 += xc[pp][k] * gd[pp][k];
+          t1 += xc[pp][k];
+          t2 += gd[pp][k];
+        }
+      }
+      t0 = segment_sum<HSB>(t0);
+      t1 = segment_sum<HSB>(t1);
+      t2 = segment_sum<HSB>(t2);
+      if (pc[pp] == 0)
+        store_exchanged4(part + ((size_t)blockIdx.x * NB + pl[pp]) * 4, t0, t1, t2, 0.f);
+    }
+    group_arrive(gs);
+    group_wait(gs);
+    sum_row_partials<NB>(part, gx, sums);
+    __syncthreads();
+
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      if (act[pp]) {
+        const float is2 = s[pp].is2;
+        const float dsigma = -0.5f * sums[pl[pp] * 4 + 0] * is2 * is2 * is2;
+        const float dmu = (-2.0f * sums[pl[pp] * 4 + 1] * dsigma * inv3H) - (sums[pl[pp] * 4 + 2] * is2);
+        float* dqt = p.dq + ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+          store_exchanged(dqt + (size_t)k * H,
+                          (2.0f * xc[pp][k] * dsigma * inv3H) + (is2 * gd[pp][k]) + (dmu * inv3H));
+      }
+    }
+    group_arrive(gs);
+    fetch(t - 1);
+    group_wait(gs);
+
+    float4_t acc[RT][1];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) acc[rt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
+    slice_matmul<RT, 1, CHUNK>(p.dq + ((size_t)t * N + n0) * 3 * H, 3 * H, N - n0, K, Kpad, w_lds,
+                               vec_ok, acc);
+    store_partials<RT, 1>(red, acc);
+    __syncthreads();
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp)
+      dh[pp] = dh_keep[pp] + sum_partials<RT, 1>(red, pl[pp], pc[pp]);
+  }
+
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp)
+    if (act[pp]) p.dh[(size_t)pn[pp] * H + pj[pp]] = dh[pp];
+
+  __syncthreads();
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp)
+#pragma unroll
+    for (int a = 0; a < NACC; ++a)
+      red[(pl[pp] * NACC + a) * HSB + pc[pp]] = act[pp] ? accs[pp][a] : 0.f;
+  __syncthreads();
+  if (tid < NACC * HSB) {
+    const int a = tid / HSB, jj = tid % HSB;
+    float sum = 0.f;
+    for (int r = 0; r < NB; ++r) sum += red[(r * NACC + a) * HSB + jj];
+    if (j0 + jj < H) p.col_partial[((size_t)blockIdx.y * NACC + a) * H + j0 + jj] = sum;
+  }
+  if (grid_last_arrival(p.cb, gridDim.x * gridDim.y, &s_flag)) {
+    for (int idx = tid; idx < NACC * H; idx += 256) {
+      const int a = idx / H, col = idx % H;
+      float sum = 0.f;
+      for (int bt = 0; bt < (int)gridDim.y; ++bt) sum += p.col_partial[((size_t)bt * NACC + a) * H + col];
+      if (a < 3) p.dbx[a * H + col] += sum;
+      else if (a < 6) p.dbr[(a - 3) * H + col] += sum;
+      else p.dgamma2[(a - 6) * H + col] += sum;
+    }
+  }
+}
+
+}  // namespace
+}  // namespace haste_hip
+
+extern "C" {
+
+using namespace haste_hip;
+
+int haste_hip_layer_norm_gru_forward_f32(int training, int steps, int batch_size,
+                                         int input_size, int hidden_size,
+                                         const float* W, const float* R, const float* bx,
+                                         const float* br, const float* x, float* h, float* v,
+                                         float* act_Wx, const float* gamma1, float* cache1,
+                                         float* tmp_Wx_norm, float* act_Rh,
+                                         const float* gamma2, float* cache2, float* tmp_Rh_norm,
+                                         float zoneout_prob, const float* zoneout_mask,
+                                         void* stream_) {
+  (void)tmp_Rh_norm;
+  const int T = steps, N = batch_size, C = input_size, H = hidden_size;
+  HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
+  HASTE_HIP_REQUIRE(W && R && bx && br && x && h && act_Wx && gamma1 && tmp_Wx_norm && act_Rh && gamma2);
+  HASTE_HIP_REQUIRE(!training || v != nullptr);
+  hipStream_t stream = as_stream(stream_);
+  const int cus = device_cu_count();
+
+  struct Cand { int rt, ct, hs; };
+  const Cand cands[] = {{1, 2, 8}, {1, 3, 16}, {1, 1, 4}, {2, 2, 8}, {2, 3, 16}, {2, 1, 4},
+                        {4, 2, 8}, {4, 3, 16}, {4, 1, 4}};
+  const Cand* pick = nullptr;
+  int gx = 0, gy = 0;
+  size_t lds = 0;
+  for (const Cand& cd : cands) {
+    const int NB = 16 * cd.rt;
+    gx = (H + cd.hs - 1) / cd.hs;
+    gy = (N + NB - 1) / NB;
+    lds = fwd_lds_bytes(H, cd.rt, cd.ct) + (size_t)NB * 2 * sizeof(float);
+    if (gy > kMaxGroups || (long long)gx * gy > cus || gx * gy > kMaxWorkgroups) continue;
+    if (lds > kMaxLdsBytes) continue;
+    pick = &cd;
+    break;
+  }
+  if (pick == nullptr) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  const int NB = 16 * pick->rt;
+  const size_t part_floats = (size_t)gy * gx * NB * 2;
+
+  Workspace ws;
+  HASTE_HIP_PROPAGATE(get_workspace(stream, part_floats * sizeof(float), &ws));
+  HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
+
+  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 3 * H, C, x, C, W, 3 * H, act_Wx, 3 * H, false));
+  HASTE_HIP_PROPAGATE(layer_norm_forward(stream, T * N, 3 * H, gamma1, nullptr, act_Wx, tmp_Wx_norm, cache1));
+
+  LnGruFwdParams p;
+  p.training = training; p.T = T; p.N = N; p.H = H;
+  p.R = R; p.bx = bx; p.br = br; p.h = h; p.v = v; p.Wxn = tmp_Wx_norm; p.act_Rh = act_Rh;
+  p.gamma2 = gamma2; p.cache2 = cache2;
+  p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
+  p.part2 = ws.scratch;
+  p.cb = ws.control; p.host_status = ws.host_status_dev; p.spin_limit = kSpinLimit;
+  HASTE_HIP_PROPAGATE(reserve_epochs(stream, 2u * (unsigned)T + 1, &p.epoch));
+  dim3 grid(gx, gy);
+#define HASTE_LAUNCH(RT_, CT_, HS_)                                                          \
+  if (pick->rt == RT_ && pick->ct == CT_)                                                    \
+    return launch_persistent("layer_norm_gru_forward_recurrence",                            \
+                             ln_gru_forward_kernel<RT_, CT_, HS_>, grid, lds, p, stream);
+  HASTE_LAUNCH(1, 1, 4) HASTE_LAUNCH(1, 2, 8) HASTE_LAUNCH(1, 3, 16)
+  HASTE_LAUNCH(2, 1, 4) HASTE_LAUNCH(2, 2, 8) HASTE_LAUNCH(2, 3, 16)
+  HASTE_LAUNCH(4, 1, 4) HASTE_LAUNCH(4, 2, 8) HASTE_LAUNCH(4, 3, 16)
+#undef HASTE_LAUNCH
+  return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+}
+
+int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_size,
+                                          int hidden_size,
+                                          const float* W_t, const float* R_t, const float* bx,
+                                          const float* br, const float* x_t, const float* h,
+                                          const float* v, const float* dh_new,
+                                          float* dx, float* dW, float* dR, float* dbx, float* dbr,
+                                          float* dh, float* dp, float* dq,
+                                          const float* act_Wx, const float* gamma1, float* dgamma1,
+                                          const float* act_Rh, const float* gamma2, float* dgamma2,
+                                          const float* cache2,
+                                          const float* zoneout_mask, void* stream_) {
+  (void)bx;
+  (void)br;
+  const int T = steps, N = batch_size, C = input_size, H = hidden_size;
+  HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
+  HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && v && dh_new && dx && dW && dR && dbx && dbr && dh);
+  HASTE_HIP_REQUIRE(dp && dq && act_Wx && gamma1 && dgamma1 && act_Rh && gamma2 && dgamma2 && cache2);
+  hipStream_t stream = as_stream(stream_);
+  const int cus = device_cu_count();
+  const int gx = (H + 15) / 16;
+  int rt = 0;
+  size_t lds = 0;
+  for (int cand : {1, 2, 4}) {
+    const int gy = (N + 16 * cand - 1) / (16 * cand);
+    const int NB = 16 * cand;
+    const int Kpad = (3 * H + 63) / 64 * 64;
+    lds = ((size_t)Kpad * 16 + (size_t)NB * 9 * 16 + (size_t)NB * 4) * sizeof(float);
+    if (gy <= kMaxGroups && (long long)gx * gy <= cus && gx * gy <= kMaxWorkgroups &&
+        lds <= kMaxLdsBytes) {
+      rt = cand;
+      break;
+    }
+  }
+  if (rt == 0) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  const int NB = 16 * rt;
+  const int gy = (N + NB - 1) / NB;
+  const size_t part_floats = (size_t)gy * gx * NB * 4;
+  const size_t col_floats = (size_t)gy * 9 * H;
+
+  Workspace ws;
+  HASTE_HIP_PROPAGATE(get_workspace(stream, (part_floats + col_floats) * sizeof(float), &ws));
+  HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
+
+  LnGruBwdParams p;
+  p.T = T; p.N = N; p.H = H;
+  p.R_t = R_t; p.h = h; p.v = v; p.dh_new = dh_new;
+  p.dbx = dbx; p.dbr = dbr; p.dh = dh; p.dp = dp; p.dq = dq;
+  p.act_Rh = act_Rh; p.gamma2 = gamma2; p.dgamma2 = dgamma2; p.cache2 = cache2;
+  p.zoneout_mask = zoneout_mask;
+  p.part = ws.scratch; p.col_partial = ws.scratch + part_floats;
+  p.cb = ws.control; p.host_status = ws.host_status_dev; p.spin_limit = kSpinLimit;
+  HASTE_HIP_PROPAGATE(reserve_epochs(stream, 2u * (unsigned)T + 1, &p.epoch));
+  dim3 grid(gx, gy);
+  int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  const char* name = "layer_norm_gru_backward_recurrence";
+  if (rt == 1) rc = launch_persistent(name, ln_gru_backward_kernel<1>, grid, lds, p, stream);
+  if (rt == 2) rc = launch_persistent(name, ln_gru_backward_kernel<2>, grid, lds, p, stream);
+  if (rt == 4) rc = launch_persistent(name, ln_gru_backward_kernel<4>, grid, lds, p, stream);
+  HASTE_HIP_PROPAGATE(rc);
+
+  const int TN = T * N;
+  HASTE_HIP_PROPAGATE(layer_norm_backward(stream, TN, 3 * H, gamma1, act_Wx, dp, dp, dgamma1, nullptr));
+  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, TN, C, 3 * H, dp, 3 * H, W_t, C, dx, C, false));
+  HASTE_HIP_PROPAGATE(gemm_f32(stream, true, H, 3 * H, TN, h, H, dq, 3 * H, dR, 3 * H, true));
+  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, C, 3 * H, TN, x_t, TN, dp, 3 * H, dW, 3 * H, true));
+  return HASTE_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,658 @@
+// LayerNormLSTM forward and backward passes.
+//
+// Forward: GEMM x*W, one stand-alone layer norm over all T*N rows, then one persistent
+// kernel for the recurrence in which the two per-step layer norms (on h*R over 4H
+// columns and on the new cell state over H columns) are computed inside the step:
+// each workgroup reduces its own columns, the group exchanges per-row moments, and a
+// step therefore has three group barriers (h_t ready, norm of h*R, norm of c).
+// Backward mirrors it in reverse time (three barriers per step as well), then one
+// stand-alone layer-norm backward over all rows and the three batched GEMMs.
+//
+// Arithmetic follows reference lib/layer_norm_lstm_forward_gpu.cu.cc:50-71,95-108 and
+// lib/layer_norm_lstm_backward_gpu.cu.cc:44-64,84-117; orchestration replaces
+// :276-340 and :255-352.
+#include "ln_exchange.h"
+
+namespace haste_hip {
+namespace {
+
+struct LnLstmFwdParams {
+  int training, T, N, H;
+  const float* R;         // [H,4H]
+  const float* b;         // [4H]
+  float* h;               // [T+1,N,H]
+  float* c;               // [T+1,N,H]
+  float* v;               // act_Wx_norm [T,N,4H]: in LN1(x*W), out (training) gate activations
+  float* act_Rh;          // [T,N,4H] out: h*R before its norm
+  const float* gamma2;    // [4H]
+  float* cache2;          // [T*N,2] or null
+  const float* gamma_h;   // [H]
+  const float* beta_h;    // [H]
+  float* cache3;          // [T*N,2] or null
+  float* act_c_norm;      // [T,N,H] out
+  float zoneout_prob;
+  const float* zoneout_mask;
+  float* part2;           // exchange [groups][gx][NB][2]
+  float* part3;           // exchange [groups][gx][NB][2]
+  ControlBlock* cb;
+  unsigned int* host_status;
+  unsigned int spin_limit;
+  unsigned int epoch;
+};
+
+template <int RT, int CT>
+__global__ __launch_bounds__(256, 1)
+void ln_lstm_forward_kernel(LnLstmFwdParams p) {
+  constexpr int HS = 4 * CT;
+  constexpr int NB = 16 * RT;
+  constexpr int NCOLS = 16 * CT;
+  constexpr int PP = (NB * HS + 255) / 256;
+  constexpr int CHUNK = RT == 4 ? 4 : 8;
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+
+  const int H = p.H, N = p.N, T = p.T;
+  const int Kpad = round_up(H, 64);
+  float* w_lds = lds;
+  float* red = lds + Kpad * NCOLS;
+  float* stat = red + 4 * NB * NCOLS;  // [NB][2]
+
+  const int tid = threadIdx.x;
+  const int gx = gridDim.x;
+  const int j0 = blockIdx.x * HS;
+  const int n0 = blockIdx.y * NB;
+  const size_t NH = (size_t)N * H;
+  const int own_units = (H - j0) < HS ? (H - j0) : HS;     // valid hidden units here
+  const int last_units = H - (gx - 1) * HS;                 // ... in the last workgroup
+  float* part2 = p.part2 + (size_t)blockIdx.y * gx * NB * 2;
+  float* part3 = p.part3 + (size_t)blockIdx.y * gx * NB * 2;
+
+  GroupSync gs;
+  group_sync_init(gs, p.cb, blockIdx.y, gx, blockIdx.x, p.epoch, p.host_status, p.spin_limit);
+
+  for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
+    const int k = idx / NCOLS, cidx = idx % NCOLS;
+    const int gate = cidx / HS, j = j0 + cidx % HS;
+    float w = 0.f;
+    if (k < H && j < H) w = p.R[(size_t)k * 4 * H + gate * H + j];
+    w_lds[slice_index(k, cidx, NCOLS)] = w;
+  }
+
+  int pn[PP], pj[PP], pl[PP], pc[PP];
+  bool act[PP], colok[PP];
+  float c_prev[PP], h_prev[PP], bias[PP][4], g2[PP][4], gh[PP], bh[PP];
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp) {
+    const int idx = tid + 256 * pp;
+    pl[pp] = idx / HS;
+    pc[pp] = idx % HS;
+    pn[pp] = n0 + pl[pp];
+    pj[pp] = j0 + pc[pp];
+    colok[pp] = idx < NB * HS && pj[pp] < H;
+    act[pp] = colok[pp] && pn[pp] < N;
+    c_prev[pp] = h_prev[pp] = gh[pp] = bh[pp] = 0.f;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) bias[pp][g] = g2[pp][g] = 0.f;
+    if (colok[pp]) {
+      gh[pp] = p.gamma_h[pj[pp]];
+      bh[pp] = p.beta_h[pj[pp]];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        bias[pp][g] = p.b[g * H + pj[pp]];
+        g2[pp][g] = p.gamma2[g * H + pj[pp]];
+      }
+    }
+    if (act[pp]) {
+      c_prev[pp] = p.c[(size_t)pn[pp] * H + pj[pp]];
+      h_prev[pp] = p.h[(size_t)pn[pp] * H + pj[pp]];
+    }
+  }
+  const bool zoneout = p.zoneout_prob != 0.f && p.zoneout_mask != nullptr;
+  const bool vec_ok = (H % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.h) & 15u) == 0);
+  __syncthreads();
+
+  for (int t = 0; t < T; ++t) {
+    float wx[PP][4], mk[PP];
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      mk[pp] = 1.f;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) wx[pp][g] = 0.f;
+      if (act[pp]) {
+        const float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) wx[pp][g] = vt[g * H];
+        if (zoneout && p.training) mk[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
+      }
+    }
+    if (t > 0) group_wait(gs);  // h[t]
+
+    float4_t acc[RT][CT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
+    slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, N - n0, H, Kpad, w_lds,
+                                vec_ok, acc);
+    store_partials<RT, CT>(red, acc);
+    __syncthreads();
+
+    // h*R of the owned columns; moments of those columns per row, published.
+    float rh[PP][4];
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      float s = 0.f;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        rh[pp][g] = colok[pp] ? sum_partials<RT, CT>(red, pl[pp], g * HS + pc[pp]) : 0.f;
+        s += rh[pp][g];
+      }
+      if (act[pp]) {
+        float* ar = p.act_Rh + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) ar[g * H] = rh[pp][g];
+      }
+      const float cnt = 4.0f * (float)own_units;
+      const float mean = segment_sum<HS>(s) / cnt;
+      float q = 0.f;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const float d = rh[pp][g] - mean;
+        q += colok[pp] ? d * d : 0.f;
+      }
+      q = segment_sum<HS>(q);
+      if (pc[pp] == 0 && tid + 256 * pp < NB * HS)
+        store_exchanged2(part2 + ((size_t)blockIdx.x * NB + pl[pp]) * 2, mean, q);
+    }
+    group_arrive(gs);
+    group_wait(gs);  // every workgroup's moments of h*R
+    merge_row_moments<NB>(part2, gx, 4.0f * HS, 4.0f * last_units, 4.0f * H, stat);
+    __syncthreads();
+
+    float go[PP], c_new[PP];
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      const float mu = stat[pl[pp] * 2], is = stat[pl[pp] * 2 + 1];
+      go[pp] = 0.f;
+      c_new[pp] = 0.f;
+      if (act[pp]) {
+        float a[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          a[g] = wx[pp][g] + (rh[pp][g] - mu) * is * g2[pp][g] + bias[pp][g];
+        const float gi = sigmoid_f(a[0]);
+        const float gg = tanhf(a[1]);
+        const float gf = sigmoid_f(a[2]);
+        go[pp] = sigmoid_f(a[3]);
+        if (p.training) {
+          float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+          vt[0] = gi;
+          vt[H] = gg;
+          vt[2 * H] = gf;
+          vt[3 * H] = go[pp];
+        }
+        c_new[pp] = gf * c_prev[pp] + gi * gg;
+        p.c[(size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp]] = c_new[pp];
+        c_prev[pp] = c_new[pp];
+        if (blockIdx.x == 0 && pc[pp] == 0 && p.cache2 != nullptr) {
+          p.cache2[((size_t)t * N + pn[pp]) * 2 + 0] = mu;
+          p.cache2[((size_t)t * N + pn[pp]) * 2 + 1] = is;
+        }
+      }
+      // moments of the new cell state over the owned hidden units
+      const float cv = colok[pp] ? c_new[pp] : 0.f;
+      const float mean = segment_sum<HS>(cv) / (float)own_units;
+      const float d = cv - mean;
+      const float q = segment_sum<HS>(colok[pp] ? d * d : 0.f);
+      if (pc[pp] == 0 && tid + 256 * pp < NB * HS)
+        store_exchanged2(part3 + ((size_t)blockIdx.x * NB + pl[pp]) * 2, mean, q);
+    }
+    group_arrive(gs);
+    group_wait(gs);  // every workgroup's moments of c
+    merge_row_moments<NB>(part3, gx, (float)HS, (float)last_units, (float)H, stat);
+    __syncthreads();
+
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      if (act[pp]) {
+        const float mu = stat[pl[pp] * 2], is = stat[pl[pp] * 2 + 1];
+        const float cn = (c_new[pp] - mu) * is * gh[pp] + bh[pp];
+        const size_t e = (size_t)pn[pp] * H + pj[pp];
+        p.act_c_norm[(size_t)t * NH + e] = cn;
+        float h_new = go[pp] * tanhf(cn);
+        if (zoneout) {
+          if (p.training) h_new = (h_new - h_prev[pp]) * mk[pp] + h_prev[pp];
+          else h_new = p.zoneout_prob * h_prev[pp] + (1.0f - p.zoneout_prob) * h_new;
+        }
+        store_exchanged(&p.h[(size_t)(t + 1) * NH + e], h_new);
+        h_prev[pp] = h_new;
+        if (blockIdx.x == 0 && pc[pp] == 0 && p.cache3 != nullptr) {
+          p.cache3[((size_t)t * N + pn[pp]) * 2 + 0] = mu;
+          p.cache3[((size_t)t * N + pn[pp]) * 2 + 1] = is;
+        }
+      }
+    }
+    if (t + 1 < T) group_arrive(gs);  // publishes h[t+1]; also orders reuse of red/stat
+    else __syncthreads();
+  }
+}
+
+struct LnLstmBwdParams {
+  int T, N, H;
+  const float* R_t;        // [4H,H]
+  const float* c;          // [T+1,N,H]
+  const float* dh_new;     // [T+1,N,H]
+  const float* dc_new;     // [T+1,N,H]
+  float* db;               // [4H]
+  float* dh;               // [N,H]
+  float* dc;               // [N,H]
+  float* v;                // act_Wx_norm: in gate activations, out gate gradients
+  float* act_Rh;           // in h*R before its norm, out gradient w.r.t. it
+  const float* gamma2;     // [4H]
+  float* dgamma2;          // [4H]
+  const float* cache2;     // [T*N,2]
+  const float* gamma_h;    // [H]
+  float* dgamma_h;         // [H]
+  float* dbeta_h;          // [H]
+  const float* cache3;     // [T*N,2]
+  const float* act_c_norm; // [T,N,H]
+  const float* zoneout_mask;
+  float* part_a;           // exchange [groups][gx][NB][4]
+  float* part_b;           // exchange [groups][gx][NB][4]
+  float* col_partial;      // [batch tiles][10][H]
+  ControlBlock* cb;
+  unsigned int* host_status;
+  unsigned int spin_limit;
+  unsigned int epoch;
+};
+
+template <int RT>
+__global__ __launch_bounds__(256, 1)
+void ln_lstm_backward_kernel(LnLstmBwdParams p) {
+  constexpr int HSB = 16;
+  constexpr int NB = 16 * RT;
+  constexpr int NCOLS = 16;
+  constexpr int PP = RT;
+  constexpr int CHUNK = RT == 1 ? 16 : (RT == 2 ? 8 : 4);
+  constexpr int NACC = 10;  // db x4, dgamma2 x4, dgamma_h, dbeta_h
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  __shared__ unsigned int s_flag;
+
+  const int H = p.H, N = p.N, T = p.T;
+  const int K = 4 * H;
+  const int Kpad = round_up(K, 64);
+  float* w_lds = lds;
+  float* red = lds + Kpad * NCOLS;       // NB*NACC*16 floats (>= 4*NB*16)
+  float* sums = red + NB * NACC * HSB;   // [NB][4]
+
+  const int tid = threadIdx.x;
+  const int gx = gridDim.x;
+  const int j0 = blockIdx.x * HSB;
+  const int n0 = blockIdx.y * NB;
+  const size_t NH = (size_t)N * H;
+  float* part_a = p.part_a + (size_t)blockIdx.y * gx * NB * 4;
+  float* part_b = p.part_b + (size_t)blockIdx.y * gx * NB * 4;
+
+  GroupSync gs;
+  group_sync_init(gs, p.cb, blockIdx.y, gx, blockIdx.x, p.epoch, p.host_status, p.spin_limit);
+
+  for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
+    const int k = idx / NCOLS, cidx = idx % NCOLS;
+    float w = 0.f;
+    if (k < K && j0 + cidx < H) w = p.R_t[(size_t)k * H + j0 + cidx];
+    w_lds[slice_index(k, cidx, NCOLS)] = w;
+  }
+
+  int pn[PP], pj[PP], pl[PP], pc[PP];
+  bool act[PP];
+  float dh[PP], dc[PP], accs[PP][NACC], g2[PP][4], gh[PP];
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp) {
+    const int idx = tid + 256 * pp;
+    pl[pp] = idx / HSB;
+    pc[pp] = idx % HSB;
+    pn[pp] = n0 + pl[pp];
+    pj[pp] = j0 + pc[pp];
+    act[pp] = pn[pp] < N && pj[pp] < H;
+    dh[pp] = act[pp] ? p.dh[(size_t)pn[pp] * H + pj[pp]] : 0.f;
+    dc[pp] = act[pp] ? p.dc[(size_t)pn[pp] * H + pj[pp]] : 0.f;
+    gh[pp] = pj[pp] < H ? p.gamma_h[pj[pp]] : 0.f;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) g2[pp][g] = pj[pp] < H ? p.gamma2[g * H + pj[pp]] : 0.f;
+#pragma unroll
+    for (int a = 0; a < NACC; ++a) accs[pp][a] = 0.f;
+  }
+  const bool zoneout = p.zoneout_mask != nullptr;
+  const bool vec_ok = (reinterpret_cast<uintptr_t>(p.act_Rh) & 15u) == 0;
+  __syncthreads();
+
+  struct StepIn { float vt[4], rh[4], c0, c1, dhn, dcn, m, cn, mu2, is2, mu3, is3; };
+  StepIn nxt[PP];
+  auto fetch = [&](int t) {
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      StepIn s = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, 0.f, 0.f, 0.f, 0.f, 1.f, 0.f,
+                  0.f, 0.f, 0.f, 0.f};
+      if (act[pp] && t >= 0) {
+        const size_t e = (size_t)pn[pp] * H + pj[pp];
+        const size_t e4 = ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          s.vt[g] = p.v[e4 + (size_t)g * H];
+          s.rh[g] = p.act_Rh[e4 + (size_t)g * H];
+        }
+        s.c0 = p.c[(size_t)t * NH + e];
+        s.c1 = p.c[(size_t)(t + 1) * NH + e];
+        s.dhn = p.dh_new[(size_t)(t + 1) * NH + e];
+        s.dcn = p.dc_new[(size_t)(t + 1) * NH + e];
+        s.cn = p.act_c_norm[(size_t)t * NH + e];
+        if (zoneout) s.m = p.zoneout_mask[(size_t)t * NH + e];
+        const size_t r = ((size_t)t * N + pn[pp]) * 2;
+        s.mu2 = p.cache2[r];
+        s.is2 = p.cache2[r + 1];
+        s.mu3 = p.cache3[r];
+        s.is3 = p.cache3[r + 1];
+      }
+      nxt[pp] = s;
+    }
+  };
+  fetch(T - 1);
+
+  const float invH = 1.0f / (float)H;
+  const float inv4H = 1.0f / (float)(4 * H);
+  for (int t = T - 1; t >= 0; --t) {
+    StepIn s[PP];
+    float dh_keep[PP], dv_o[PP], xc3[PP], gd3[PP];
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      s[pp] = nxt[pp];
+      dh_keep[pp] = dv_o[pp] = xc3[pp] = gd3[pp] = 0.f;
+      if (act[pp]) {
+        float dh_total = s[pp].dhn + dh[pp];
+        if (zoneout) {
+          dh_keep[pp] = (1.0f - s[pp].m) * dh_total;
+          dh_total = s[pp].m * dh_total;
+        }
+        const float go = s[pp].vt[3];
+        const float c_tanh = tanhf(s[pp].cn);
+        const float do_ = c_tanh * dh_total;
+        const float dln3 = d_tanh_f(c_tanh) * (go * dh_total);
+        dv_o[pp] = d_sigmoid_f(go) * do_;
+        xc3[pp] = s[pp].c1 - s[pp].mu3;
+        gd3[pp] = gh[pp] * dln3;
+        accs[pp][8] += xc3[pp] * s[pp].is3 * dln3;
+        accs[pp][9] += dln3;
+      }
+      const float s0 = segment_sum<HSB>(xc3[pp] * gd3[pp]);
+      const float s1 = segment_sum<HSB>(xc3[pp]);
+      const float s2 = segment_sum<HSB>(gd3[pp]);
+      if (pc[pp] == 0)
+        store_exchanged4(part_a + ((size_t)blockIdx.x * NB + pl[pp]) * 4, s0, s1, s2, 0.f);
+    }
+    group_arrive(gs);
+    group_wait(gs);  // row sums of the cell-state norm
+    sum_row_partials<NB>(part_a, gx, sums);
+    __syncthreads();
+
+    float xc2[PP][4], gd2[PP][4];
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      float t0 = 0.f, t1 = 0.f, t2 = 0.f;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) xc2[pp][g] = gd2[pp][g] = 0.f;
+      if (act[pp]) {
+        const float is3 = s[pp].is3;
+        const float dsigma = -0.5f * sums[pl[pp] * 4 + 0] * is3 * is3 * is3;
+        const float dmu = (-2.0f * sums[pl[pp] * 4 + 1] * dsigma * invH) - (sums[pl[pp] * 4 + 2] * is3);
+        const float dc_ln = (2.0f * xc3[pp] * dsigma * invH) + (is3 * gd3[pp]) + (dmu * invH);
+        const float gi = s[pp].vt[0], gg = s[pp].vt[1], gf = s[pp].vt[2];
+        const float dc_total = s[pp].dcn + dc[pp] + dc_ln;
+        const float df = s[pp].c0 * dc_total;
+        dc[pp] = gf * dc_total;
+        const float di = gg * dc_total;
+        const float dg = gi * dc_total;
+        float dv[4];
+        dv[0] = d_sigmoid_f(gi) * di;
+        dv[1] = d_tanh_f(gg) * dg;
+        dv[2] = d_sigmoid_f(gf) * df;
+        dv[3] = dv_o[pp];
+        float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          vt[(size_t)g * H] = dv[g];
+          accs[pp][g] += dv[g];
+          xc2[pp][g] = s[pp].rh[g] - s[pp].mu2;
+          gd2[pp][g] = g2[pp][g] * dv[g];
+          accs[pp][4 + g] += xc2[pp][g] * s[pp].is2 * dv[g];
+          t0 += xc2[pp][g] * gd2[pp][g];
+          t1 += xc2[pp][g];
+          t2 += gd2[pp][g];
+        }
+      }
+      t0 = segment_sum<HSB>(t0);
+      t1 = segment_sum<HSB>(t1);
+      t2 = segment_sum<HSB>(t2);
+      if (pc[pp] == 0)
+        store_exchanged4(part_b + ((size_t)blockIdx.x * NB + pl[pp]) * 4, t0, t1, t2, 0.f);
+    }
+    group_arrive(gs);
+    group_wait(gs);  // row sums of the h*R norm
+    sum_row_partials<NB>(part_b, gx, sums);
+    __syncthreads();
+
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      if (act[pp]) {
+        const float is2 = s[pp].is2;
+        const float dsigma = -0.5f * sums[pl[pp] * 4 + 0] * is2 * is2 * is2;
+        const float dmu = (-2.0f * sums[pl[pp] * 4 + 1] * dsigma * inv4H) - (sums[pl[pp] * 4 + 2] * is2);
+        float* ar = p.act_Rh + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          store_exchanged(ar + (size_t)g * H,
+                          (2.0f * xc2[pp][g] * dsigma * inv4H) + (is2 * gd2[pp][g]) + (dmu * inv4H));
+      }
+    }
+    group_arrive(gs);
+    fetch(t - 1);
+    group_wait(gs);  // gradient w.r.t. h*R complete for this batch tile
+
+    float4_t acc[RT][1];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) acc[rt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
+    slice_matmul<RT, 1, CHUNK>(p.act_Rh + ((size_t)t * N + n0) * 4 * H, 4 * H, N - n0, K, Kpad,
+                               w_lds, vec_ok, acc);
+    store_partials<RT, 1>(red, acc);
+    __syncthreads();
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp)
+      dh[pp] = dh_keep[pp] + sum_partials<RT, 1>(red, pl[pp], pc[pp]);
+  }
+
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp) {
+    if (act[pp]) {
+      p.dh[(size_t)pn[pp] * H + pj[pp]] = dh[pp];
+      p.dc[(size_t)pn[pp] * H + pj[pp]] = dc[pp];
+    }
+  }
+
+  // Column sums (bias and norm-scale gradients): rows of this tile in LDS, then tiles in order.
+  __syncthreads();
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp)
+#pragma unroll
+    for (int a = 0; a < NACC; ++a)
+      red[(pl[pp] * NACC + a) * HSB + pc[pp]] = act[pp] ? accs[pp][a] : 0.f;
+  __syncthreads();
+  if (tid < NACC * HSB) {
+    const int a = tid / HSB, jj = tid % HSB;
+    float sum = 0.f;
+    for (int r = 0; r < NB; ++r) sum += red[(r * NACC + a) * HSB + jj];
+    if (j0 + jj < H) p.col_partial[((size_t)blockIdx.y * NACC + a) * H + j0 + jj] = sum;
+  }
+  if (grid_last_arrival(p.cb, gridDim.x * gridDim.y, &s_flag)) {
+    for (int idx = tid; idx < NACC * H; idx += 256) {
+      const int a = idx / H, col = idx % H;
+      float sum = 0.f;
+      for (int bt = 0; bt < (int)gridDim.y; ++bt) sum += p.col_partial[((size_t)bt * NACC + a) * H + col];
+      if (a < 4) p.db[a * H + col] += sum;
+      else if (a < 8) p.dgamma2[(a - 4) * H + col] += sum;
+      else if (a == 8) p.dgamma_h[col] += sum;
+      else p.dbeta_h[col] += sum;
+    }
+  }
+}
+
+}  // namespace
+}  // namespace haste_hip
+
+extern "C" {
+
+using namespace haste_hip;
+
+int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_size,
+                                          int input_size, int hidden_size,
+                                          const float* W, const float* R, const float* b,
+                                          const float* x, float* h, float* c,
+                                          float* act_Wx, float* tmp_Rh,
+                                          const float* gamma1, float* cache1,
+                                          float* act_Wx_norm, float* act_Rh,
+                                          const float* gamma2, float* cache2,
+                                          const float* gamma_h, const float* beta_h, float* cache3,
+                                          float* act_c_norm,
+                                          float zoneout_prob, const float* zoneout_mask,
+                                          void* stream_) {
+  (void)tmp_Rh;
+  const int T = steps, N = batch_size, C = input_size, H = hidden_size;
+  HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
+  HASTE_HIP_REQUIRE(W && R && b && x && h && c && act_Wx && gamma1 && act_Wx_norm && act_Rh);
+  HASTE_HIP_REQUIRE(gamma2 && gamma_h && beta_h && act_c_norm);
+  hipStream_t stream = as_stream(stream_);
+  const int cus = device_cu_count();
+
+  struct Cand { int rt, ct; };
+  const Cand cands[] = {{1, 2}, {1, 4}, {1, 1}, {2, 2}, {2, 4}, {2, 1}, {4, 2}, {4, 4}, {4, 1}};
+  const Cand* pick = nullptr;
+  int gx = 0, gy = 0;
+  size_t lds = 0;
+  for (const Cand& cd : cands) {
+    const int HS = 4 * cd.ct, NB = 16 * cd.rt;
+    gx = (H + HS - 1) / HS;
+    gy = (N + NB - 1) / NB;
+    lds = fwd_lds_bytes(H, cd.rt, cd.ct) + (size_t)NB * 2 * sizeof(float);
+    if (gy > kMaxGroups || (long long)gx * gy > cus || gx * gy > kMaxWorkgroups) continue;
+    if (lds > kMaxLdsBytes) continue;
+    pick = &cd;
+    break;
+  }
+  if (pick == nullptr) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  const int NB = 16 * pick->rt;
+  const size_t part_floats = (size_t)gy * gx * NB * 2;
+
+  Workspace ws;
+  HASTE_HIP_PROPAGATE(get_workspace(stream, 2 * part_floats * sizeof(float), &ws));
+  HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
+
+  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 4 * H, C, x, C, W, 4 * H, act_Wx, 4 * H, false));
+  HASTE_HIP_PROPAGATE(layer_norm_forward(stream, T * N, 4 * H, gamma1, nullptr, act_Wx, act_Wx_norm, cache1));
+
+  LnLstmFwdParams p;
+  p.training = training; p.T = T; p.N = N; p.H = H;
+  p.R = R; p.b = b; p.h = h; p.c = c; p.v = act_Wx_norm; p.act_Rh = act_Rh;
+  p.gamma2 = gamma2; p.cache2 = cache2; p.gamma_h = gamma_h; p.beta_h = beta_h; p.cache3 = cache3;
+  p.act_c_norm = act_c_norm; p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
+  p.part2 = ws.scratch; p.part3 = ws.scratch + part_floats;
+  p.cb = ws.control; p.host_status = ws.host_status_dev; p.spin_limit = kSpinLimit;
+  HASTE_HIP_PROPAGATE(reserve_epochs(stream, 3u * (unsigned)T + 1, &p.epoch));
+  dim3 grid(gx, gy);
+#define HASTE_LAUNCH(RT_, CT_)                                                               \
+  if (pick->rt == RT_ && pick->ct == CT_)                                                    \
+    return launch_persistent("layer_norm_lstm_forward_recurrence",                           \
+                             ln_lstm_forward_kernel<RT_, CT_>, grid, lds, p, stream);
+  HASTE_LAUNCH(1, 1) HASTE_LAUNCH(1, 2) HASTE_LAUNCH(1, 4)
+  HASTE_LAUNCH(2, 1) HASTE_LAUNCH(2, 2) HASTE_LAUNCH(2, 4)
+  HASTE_LAUNCH(4, 1) HASTE_LAUNCH(4, 2) HASTE_LAUNCH(4, 4)
+#undef HASTE_LAUNCH
+  return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+}
+
+int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_size,
+                                           int hidden_size,
+                                           const float* W_t, const float* R_t, const float* b,
+                                           const float* x_t, const float* h, const float* c,
+                                           const float* dh_new, const float* dc_new,
+                                           float* dx, float* dW, float* dR, float* db,
+                                           float* dh, float* dc,
+                                           float* act_Wx, const float* gamma1, float* dgamma1,
+                                           float* act_Wx_norm, float* act_Rh,
+                                           const float* gamma2, float* dgamma2,
+                                           const float* cache2,
+                                           const float* gamma_h, const float* beta_h,
+                                           float* dgamma_h, float* dbeta_h,
+                                           const float* cache3,
+                                           float* act_c_norm,
+                                           const float* zoneout_mask, void* stream_) {
+  (void)b;
+  (void)beta_h;
+  const int T = steps, N = batch_size, C = input_size, H = hidden_size;
+  HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
+  HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && c && dh_new && dc_new);
+  HASTE_HIP_REQUIRE(dx && dW && dR && db && dh && dc && act_Wx && gamma1 && dgamma1);
+  HASTE_HIP_REQUIRE(act_Wx_norm && act_Rh && gamma2 && dgamma2 && cache2 && gamma_h);
+  HASTE_HIP_REQUIRE(dgamma_h && dbeta_h && cache3 && act_c_norm);
+  hipStream_t stream = as_stream(stream_);
+  const int cus = device_cu_count();
+  const int gx = (H + 15) / 16;
+  int rt = 0;
+  size_t lds = 0;
+  for (int cand : {1, 2, 4}) {
+    const int gy = (N + 16 * cand - 1) / (16 * cand);
+    const int NB = 16 * cand;
+    const int Kpad = (4 * H + 63) / 64 * 64;
+    lds = ((size_t)Kpad * 16 + (size_t)NB * 10 * 16 + (size_t)NB * 4) * sizeof(float);
+    if (gy <= kMaxGroups && (long long)gx * gy <= cus && gx * gy <= kMaxWorkgroups &&
+        lds <= kMaxLdsBytes) {
+      rt = cand;
+      break;
+    }
+  }
+  if (rt == 0) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  const int NB = 16 * rt;
+  const int gy = (N + NB - 1) / NB;
+  const size_t part_floats = (size_t)gy * gx * NB * 4;
+  const size_t col_floats = (size_t)gy * 10 * H;
+
+  Workspace ws;
+  HASTE_HIP_PROPAGATE(get_workspace(stream, (2 * part_floats + col_floats) * sizeof(float), &ws));
+  HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
+
+  LnLstmBwdParams p;
+  p.T = T; p.N = N; p.H = H;
+  p.R_t = R_t; p.c = c; p.dh_new = dh_new; p.dc_new = dc_new;
+  p.db = db; p.dh = dh; p.dc = dc; p.v = act_Wx_norm; p.act_Rh = act_Rh;
+  p.gamma2 = gamma2; p.dgamma2 = dgamma2; p.cache2 = cache2;
+  p.gamma_h = gamma_h; p.dgamma_h = dgamma_h; p.dbeta_h = dbeta_h; p.cache3 = cache3;
+  p.act_c_norm = act_c_norm; p.zoneout_mask = zoneout_mask;
+  p.part_a = ws.scratch; p.part_b = ws.scratch + part_floats;
+  p.col_partial = ws.scratch + 2 * part_floats;
+  p.cb = ws.control; p.host_status = ws.host_status_dev; p.spin_limit = kSpinLimit;
+  HASTE_HIP_PROPAGATE(reserve_epochs(stream, 3u * (unsigned)T + 1, &p.epoch));
+  dim3 grid(gx, gy);
+  int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  const char* name = "layer_norm_lstm_backward_recurrence";
+  if (rt == 1) rc = launch_persistent(name, ln_lstm_backward_kernel<1>, grid, lds, p, stream);
+  if (rt == 2) rc = launch_persistent(name, ln_lstm_backward_kernel<2>, grid, lds, p, stream);
+  if (rt == 4) rc = launch_persistent(name, ln_lstm_backward_kernel<4>, grid, lds, p, stream);
+  HASTE_HIP_PROPAGATE(rc);
+
+  // Gradient through the norm of x*W (in place over act_Wx), then the batched products.
+  const int TN = T * N;
+  HASTE_HIP_PROPAGATE(layer_norm_backward(stream, TN, 4 * H, gamma1, act_Wx, act_Wx_norm, act_Wx,
+                                          dgamma1, nullptr));
+  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, C, 4 * H, TN, x_t, TN, act_Wx, 4 * H, dW, 4 * H, true));
+  HASTE_HIP_PROPAGATE(gemm_f32(stream, true, H, 4 * H, TN, h, H, act_Rh, 4 * H, dR, 4 * H, true));
+  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, TN, C, 4 * H, act_Wx, 4 * H, W_t, C, dx, C, false));
+  return HASTE_HIP_OK;
+}
+
+}  // extern "C"

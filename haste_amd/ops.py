@@ -219,3 +219,107 @@ def layer_norm_indrnn_backward(x_t, kernel_t, recurrent_scale, bias, gamma, zone
              x_t, h, dh_new, dx, dW, du, db, dh, workspace, act_Wx, gamma[0], dgamma[0],
              _mask_or_none(has_zoneout, zoneout_mask))
     return dx, dh, dW, du, db, dgamma
+
+
+# ---- LayerNorm LSTM (reference frameworks/pytorch/layer_norm_lstm.cc:31-297) ---------
+def layer_norm_lstm_forward(training, zoneout_prob, x, h0, c0, kernel, recurrent_kernel, bias,
+                            gamma, gamma_h, beta_h, zoneout_mask):
+    T, N, C = x.shape
+    H = recurrent_kernel.shape[0]
+    has_zoneout = bool(zoneout_prob) and zoneout_mask.numel() > 0
+    _check(x, h0, c0, kernel, recurrent_kernel, bias, gamma, gamma_h, beta_h, zoneout_mask)
+    opts = dict(device=x.device, dtype=x.dtype)
+    output = torch.zeros(T + 1, N, H, **opts)
+    output_state = torch.zeros(T + 1, N, H, **opts)
+    act_Wx = torch.empty(T, N, 4 * H, **opts)
+    act_Wx_norm = torch.empty(T, N, 4 * H, **opts)
+    act_Wx_norm_cache = torch.empty(T, N, 2, **opts)
+    act_Rh = torch.empty(T, N, 4 * H, **opts)
+    act_Rh_norm_cache = torch.empty(T, N, 2, **opts)
+    act_c_norm = torch.empty(T, N, H, **opts)
+    act_c_norm_cache = torch.empty(T, N, 2, **opts)
+    output[0] = h0
+    output_state[0] = c0
+    lib.call("haste_hip_layer_norm_lstm_forward_f32", bool(training), T, N, C, H, kernel,
+             recurrent_kernel, bias, x, output, output_state, act_Wx, None,
+             gamma[0], act_Wx_norm_cache, act_Wx_norm, act_Rh, gamma[1], act_Rh_norm_cache,
+             gamma_h, beta_h, act_c_norm_cache, act_c_norm,
+             float(zoneout_prob) if has_zoneout else 0.0, _mask_or_none(has_zoneout, zoneout_mask))
+    return (output, output_state, act_Wx, act_Wx_norm, act_Wx_norm_cache, act_Rh, act_Rh_norm_cache,
+            act_c_norm, act_c_norm_cache)
+
+
+def layer_norm_lstm_backward(x_t, kernel_t, recurrent_kernel_t, bias, gamma, gamma_h, beta_h,
+                             zoneout_mask, h, c, act_Wx, act_Wx_norm, act_Wx_norm_cache, act_Rh,
+                             act_Rh_norm_cache, act_c_norm, act_c_norm_cache, dh_new, dc_new):
+    C, T, N = x_t.shape
+    H = recurrent_kernel_t.shape[1]
+    has_zoneout = zoneout_mask.numel() > 0
+    _check(x_t, kernel_t, recurrent_kernel_t, bias, gamma, gamma_h, beta_h, zoneout_mask, h, c,
+           act_Wx, act_Wx_norm, act_Wx_norm_cache, act_Rh, act_Rh_norm_cache, act_c_norm,
+           act_c_norm_cache, dh_new, dc_new)
+    opts = dict(device=x_t.device, dtype=x_t.dtype)
+    dx = torch.empty(T, N, C, **opts)
+    dW = torch.zeros(C, 4 * H, **opts)
+    dR = torch.zeros(H, 4 * H, **opts)
+    db = torch.zeros(4 * H, **opts)
+    dgamma = torch.zeros_like(gamma)
+    dgamma_h = torch.zeros_like(gamma_h)
+    dbeta_h = torch.zeros_like(beta_h)
+    dh = torch.zeros(N, H, **opts)
+    dc = torch.zeros(N, H, **opts)
+    lib.call("haste_hip_layer_norm_lstm_backward_f32", T, N, C, H, kernel_t, recurrent_kernel_t,
+             bias, x_t, h, c, dh_new, dc_new, dx, dW, dR, db, dh, dc,
+             act_Wx, gamma[0], dgamma[0], act_Wx_norm, act_Rh, gamma[1], dgamma[1],
+             act_Rh_norm_cache, gamma_h, beta_h, dgamma_h, dbeta_h, act_c_norm_cache, act_c_norm,
+             _mask_or_none(has_zoneout, zoneout_mask))
+    return dx, dh, dc, dW, dR, db, dgamma, dgamma_h, dbeta_h
+
+
+# ---- LayerNorm GRU (reference frameworks/pytorch/layer_norm_gru.cc:30-230) -----------
+def layer_norm_gru_forward(training, zoneout_prob, x, h0, kernel, recurrent_kernel, bias,
+                           recurrent_bias, gamma, zoneout_mask):
+    T, N, C = x.shape
+    H = recurrent_kernel.shape[0]
+    has_zoneout = bool(zoneout_prob) and zoneout_mask.numel() > 0
+    _check(x, h0, kernel, recurrent_kernel, bias, recurrent_bias, gamma, zoneout_mask)
+    opts = dict(device=x.device, dtype=x.dtype)
+    output = torch.empty(T + 1, N, H, **opts)
+    cache = torch.empty(T, N, 4 * H, **opts)
+    act_Wx = torch.empty(T, N, 3 * H, **opts)
+    tmp_Wx_norm = torch.empty(T, N, 3 * H, **opts)
+    act_Wx_norm_cache = torch.empty(T, N, 2, **opts)
+    act_Rh = torch.empty(T, N, 3 * H, **opts)
+    act_Rh_norm_cache = torch.empty(T, N, 2, **opts)
+    output[0] = h0
+    lib.call("haste_hip_layer_norm_gru_forward_f32", bool(training), T, N, C, H, kernel,
+             recurrent_kernel, bias, recurrent_bias, x, output, cache if training else None,
+             act_Wx, gamma[0], act_Wx_norm_cache, tmp_Wx_norm, act_Rh, gamma[1], act_Rh_norm_cache,
+             None, float(zoneout_prob) if has_zoneout else 0.0,
+             _mask_or_none(has_zoneout, zoneout_mask))
+    return output, cache, act_Wx, act_Wx_norm_cache, act_Rh, act_Rh_norm_cache
+
+
+def layer_norm_gru_backward(x_t, kernel_t, recurrent_kernel_t, bias, recurrent_bias, gamma,
+                            zoneout_mask, h, cache, act_Wx, act_Wx_norm_cache, act_Rh,
+                            act_Rh_norm_cache, dh_new):
+    C, T, N = x_t.shape
+    H = recurrent_kernel_t.shape[1]
+    has_zoneout = zoneout_mask.numel() > 0
+    _check(x_t, kernel_t, recurrent_kernel_t, bias, recurrent_bias, gamma, zoneout_mask, h, cache,
+           act_Wx, act_Wx_norm_cache, act_Rh, act_Rh_norm_cache, dh_new)
+    opts = dict(device=x_t.device, dtype=x_t.dtype)
+    dx = torch.empty(T, N, C, **opts)
+    dW = torch.zeros(C, 3 * H, **opts)
+    dR = torch.zeros(H, 3 * H, **opts)
+    dbx = torch.zeros(3 * H, **opts)
+    dbr = torch.zeros(3 * H, **opts)
+    dh = torch.zeros(N, H, **opts)
+    dp = torch.empty(T, N, 3 * H, **opts)
+    dq = torch.empty(T, N, 3 * H, **opts)
+    dgamma = torch.zeros_like(gamma)
+    lib.call("haste_hip_layer_norm_gru_backward_f32", T, N, C, H, kernel_t, recurrent_kernel_t, bias,
+             recurrent_bias, x_t, h, cache, dh_new, dx, dW, dR, dbx, dbr, dh, dp, dq,
+             act_Wx, gamma[0], dgamma[0], act_Rh, gamma[1], dgamma[1], act_Rh_norm_cache,
+             _mask_or_none(has_zoneout, zoneout_mask))
+    return dx, dh, dW, dR, dbx, dbr, dgamma

@@ -161,8 +161,10 @@ int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_siz
                                           void* stream);
 
 /* reference lib/haste/layer_norm_lstm.h:160-183, lib/layer_norm_lstm_backward_gpu.cu.cc:255-352.
- * act_Wx, act_Wx_norm, act_Rh, act_c_norm are consumed (overwritten with gradients).
- * dgamma1, dgamma2 [4H], dgamma_h, dbeta_h [H] are accumulated into. */
+ * act_Wx, act_Wx_norm, act_Rh are consumed (overwritten with gradients); act_c_norm is
+ * read.  dgamma1, dgamma2 [4H], dgamma_h, dbeta_h [H] are accumulated into.
+ * cache2, cache3 [T*N,2] are the (mean, 1/std) caches the forward pass wrote for the
+ * per-step norms (the reference's layer_norm2 / layer_norm3 objects hold them). */
 int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_size,
                                            int hidden_size,
                                            const float* W_t, const float* R_t, const float* b,
@@ -173,8 +175,10 @@ int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_
                                            float* act_Wx, const float* gamma1, float* dgamma1,
                                            float* act_Wx_norm, float* act_Rh,
                                            const float* gamma2, float* dgamma2,
+                                           const float* cache2,
                                            const float* gamma_h, const float* beta_h,
                                            float* dgamma_h, float* dbeta_h,
+                                           const float* cache3,
                                            float* act_c_norm,
                                            const float* zoneout_mask, void* stream);
 
@@ -193,7 +197,8 @@ int haste_hip_layer_norm_gru_forward_f32(int training, int steps, int batch_size
 /* reference lib/haste/layer_norm_gru.h:164-184, lib/layer_norm_gru_backward_gpu.cu.cc:219-310.
  * act_Wx / act_Rh are the pre-norm activations saved by the forward pass (the `x` of the
  * reference's layer_norm1 / layer_norm2 BackwardPass objects). dp, dq are overwritten
- * with the gradients w.r.t. the pre-norm activations, as in the reference. */
+ * with the gradients w.r.t. the pre-norm activations, as in the reference.
+ * cache2 [T*N,2] is the (mean, 1/std) cache the forward pass wrote for the per-step norm. */
 int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_size,
                                           int hidden_size,
                                           const float* W_t, const float* R_t, const float* bx,
@@ -203,6 +208,7 @@ int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_s
                                           float* dh, float* dp, float* dq,
                                           const float* act_Wx, const float* gamma1, float* dgamma1,
                                           const float* act_Rh, const float* gamma2, float* dgamma2,
+                                          const float* cache2,
                                           const float* zoneout_mask, void* stream);
 
 /* ---- IndRNN --------------------------------------------------------------------

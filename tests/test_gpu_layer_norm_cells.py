@@ -1,0 +1,93 @@
+"""LayerNormLSTM and LayerNormGRU on the GPU (through the C-ABI) vs the fp64 oracle."""
+import numpy as np
+import pytest
+
+from oracle import haste_oracle as O
+from util import TOL, dev, host, problem, relerr
+
+pytestmark = pytest.mark.gpu
+
+# The smallest case keeps H >= 4 and C >= 2: a layer norm over one or two elements has a
+# constant output, and with C == 1 the norm of x*W does not depend on the scale of x, so
+# those input gradients are pure rounding noise to which no relative tolerance applies.
+SHAPES = [(1, 1, 3, 4), (3, 2, 3, 4), (5, 3, 7, 5), (6, 17, 20, 36), (4, 16, 32, 64),
+          (10, 33, 48, 128), (8, 32, 64, 256), (6, 64, 96, 512)]
+
+
+@pytest.mark.parametrize("zoneout", [0.0, 0.3])
+@pytest.mark.parametrize("T,N,C,H", SHAPES)
+def test_layer_norm_lstm_training_forward_backward(T, N, C, H, zoneout):
+    from haste_amd import ops
+    import torch
+    print("ln_lstm", T, N, C, H, zoneout, flush=True)
+    p = problem(400 + T + N + C + H, T, N, C, H, 4, zoneout)
+    mask = dev(p["mask"])
+    gam, gh, bh = dev(p["gamma"]), dev(p["gamma_h"]), dev(p["beta_h"])
+    outs = ops.layer_norm_lstm_forward(True, zoneout, dev(p["x"]), dev(p["h0"]), dev(p["c0"]),
+                                       dev(p["W"]), dev(p["R"]), dev(p["b"]), gam, gh, bh, mask)
+    torch.cuda.synchronize()
+    h, c, act_Wx, act_Wx_norm, cache1, act_Rh, cache2, act_c_norm, cache3 = outs
+    fwd = O.layer_norm_lstm_forward(p["W"], p["R"], p["b"], p["gamma"], p["gamma_h"], p["beta_h"],
+                                    p["x"], p["h0"], p["c0"], True, zoneout, p["mask"])
+    assert relerr(host(h), fwd["h"]) < TOL
+    assert relerr(host(c), fwd["c"]) < TOL
+    assert relerr(host(act_Wx_norm), fwd["v"]) < TOL
+    assert relerr(host(act_Rh), fwd["act_Rh"]) < TOL
+    assert relerr(host(act_c_norm), fwd["act_c_norm"]) < TOL
+    assert relerr(host(cache2), fwd["cache2"]) < TOL
+    assert relerr(host(cache3), fwd["cache3"]) < TOL
+    x_t = dev(p["x"]).permute(2, 0, 1).contiguous()
+    grads = ops.layer_norm_lstm_backward(
+        x_t, dev(p["W"]).t().contiguous(), dev(p["R"]).t().contiguous(), dev(p["b"]), gam, gh, bh,
+        mask, h, c, act_Wx, act_Wx_norm, cache1, act_Rh, cache2, act_c_norm, cache3,
+        dev(p["dh_new"]), dev(p["dc_new"]))
+    torch.cuda.synchronize()
+    g = O.layer_norm_lstm_backward(p["W"], p["R"], p["b"], p["gamma"], p["gamma_h"], p["beta_h"],
+                                   p["x"], fwd, p["dh_new"], p["dc_new"], p["mask"])
+    names = ("dx", "dh0", "dc0", "dW", "dR", "db", "dgamma", "dgamma_h", "dbeta_h")
+    for name, ours in zip(names, grads):
+        assert relerr(host(ours), g[name]) < TOL, name
+
+
+@pytest.mark.parametrize("zoneout", [0.0, 0.3])
+@pytest.mark.parametrize("T,N,C,H", SHAPES)
+def test_layer_norm_gru_training_forward_backward(T, N, C, H, zoneout):
+    from haste_amd import ops
+    import torch
+    print("ln_gru", T, N, C, H, zoneout, flush=True)
+    p = problem(500 + T + N + C + H, T, N, C, H, 3, zoneout)
+    mask = dev(p["mask"])
+    gam = dev(p["gamma"])
+    h, cache, act_Wx, cache1, act_Rh, cache2 = ops.layer_norm_gru_forward(
+        True, zoneout, dev(p["x"]), dev(p["h0"]), dev(p["W"]), dev(p["R"]), dev(p["b"]),
+        dev(p["b2"]), gam, mask)
+    torch.cuda.synchronize()
+    fwd = O.layer_norm_gru_forward(p["W"], p["R"], p["b"], p["b2"], p["gamma"], p["x"], p["h0"],
+                                   True, zoneout, p["mask"])
+    assert relerr(host(h), fwd["h"]) < TOL
+    assert relerr(host(cache), fwd["v"]) < TOL
+    assert relerr(host(act_Rh), fwd["act_Rh"]) < TOL
+    x_t = dev(p["x"]).permute(2, 0, 1).contiguous()
+    grads = ops.layer_norm_gru_backward(
+        x_t, dev(p["W"]).t().contiguous(), dev(p["R"]).t().contiguous(), dev(p["b"]), dev(p["b2"]),
+        gam, mask, h, cache, act_Wx, cache1, act_Rh, cache2, dev(p["dh_new"]))
+    torch.cuda.synchronize()
+    g = O.layer_norm_gru_backward(p["W"], p["R"], p["b"], p["b2"], p["gamma"], p["x"], fwd,
+                                  p["dh_new"], p["mask"])
+    for name, ours in zip(("dx", "dh0", "dW", "dR", "dbx", "dbr", "dgamma"), grads):
+        assert relerr(host(ours), g[name]) < TOL, name
+
+
+def test_layer_norm_lstm_inference_forward():
+    from haste_amd import ops
+    import torch
+    T, N, C, H = 15, 8, 32, 128
+    p = problem(6, T, N, C, H, 4, 0.2)
+    outs = ops.layer_norm_lstm_forward(False, 0.2, dev(p["x"]), dev(p["h0"]), dev(p["c0"]),
+                                       dev(p["W"]), dev(p["R"]), dev(p["b"]), dev(p["gamma"]),
+                                       dev(p["gamma_h"]), dev(p["beta_h"]), dev(p["mask"]))
+    torch.cuda.synchronize()
+    fwd = O.layer_norm_lstm_forward(p["W"], p["R"], p["b"], p["gamma"], p["gamma_h"], p["beta_h"],
+                                    p["x"], p["h0"], p["c0"], False, 0.2, p["mask"])
+    assert relerr(host(outs[0]), fwd["h"]) < TOL
+    assert relerr(host(outs[1]), fwd["c"]) < TOL
