@@ -51,5 +51,21 @@ def build(force=True, verbose=False):
     return LIB_PATH
 
 
+def build_cpp_api_check(verbose=False):
+    """Compiles tests/cpp/api_check.cpp, a C++ caller of include/haste.h, against the library."""
+    root = os.path.dirname(HERE)
+    src = os.path.join(root, "tests", "cpp", "api_check.cpp")
+    out = os.path.join(root, "tests", "cpp", "api_check")
+    cmd = [HIPCC, "-O2", "-std=c++17", "-I" + os.path.join(root, "include"), src, "-o", out,
+           "-L" + HERE, "-lhaste_hip", "-Wl,-rpath,$ORIGIN/../../haste_amd"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("api_check build failed:\n%s\n%s" % (res.stdout, res.stderr))
+    if verbose:
+        print("built", out)
+    return out
+
+
 if __name__ == "__main__":
-    build(force="--force" in sys.argv or True, verbose=True)
+    build(force=True, verbose=True)
+    build_cpp_api_check(verbose=True)

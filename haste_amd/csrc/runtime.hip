@@ -157,6 +157,36 @@ const char* haste_hip_error_string(int code) {
 
 const char* haste_hip_last_runtime_error(void) { return haste_hip::g_last_error.c_str(); }
 
+int haste_hip_max_hidden_size(int gates, int batch_size) {
+  if (gates < 1 || gates > 4 || batch_size < 1) return 0;
+  const int cus = haste_hip::device_cu_count();
+  if (cus <= 0) return 0;
+  const long long lds_limit = 160 * 1024;
+  auto fits = [&](int H) {
+    bool fwd = false, bwd = false;
+    for (int rt : {1, 2, 4}) {
+      const int gy = (batch_size + 16 * rt - 1) / (16 * rt);
+      if (gy > haste_hip::kMaxGroups) continue;
+      for (int hs : {4, 8, 16}) {
+        const int ct = (gates * hs + 15) / 16;
+        const long long kpad = (H + 63) / 64 * 64;
+        const long long lds = (kpad * 16 * ct + 4LL * 16 * rt * 16 * ct + 32LL * rt) * 4;
+        const long long gx = (H + hs - 1) / hs;
+        if (lds <= lds_limit && gx * gy <= cus) fwd = true;
+      }
+      const long long kpad = ((long long)gates * H + 63) / 64 * 64;
+      const long long lds = (kpad * 16 + 16LL * rt * 10 * 16 + 64LL * rt) * 4;
+      const long long gx = (H + 15) / 16;
+      if (lds <= lds_limit && gx * gy <= cus) bwd = true;
+    }
+    return fwd && bwd;
+  };
+  int best = 0;
+  for (int H = 16; H <= 8192; H += 16)
+    if (fits(H)) best = H;
+  return best;
+}
+
 int haste_hip_profile_enable(int on) {
   std::lock_guard<std::mutex> lock(haste_hip::g_mutex);
   haste_hip::g_profile_on = on != 0;

@@ -1,0 +1,293 @@
+// Exercises the libhaste-compatible C++ classes (include/haste.h) the way a C++ caller
+// of the reference would (cf. reference examples/lstm.cc:72-200): device buffers,
+// ForwardPass::Run, host-side transposes, BackwardPass::Run.  Reads one problem from a
+// raw float32 file, writes every output to another; tests/test_gpu_cpp_api.py feeds it
+// seeded inputs and checks the outputs against the oracle.
+//
+// usage: api_check <cell> <T> <N> <C> <H> <zoneout_prob> <in.bin> <out.bin>
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "haste.h"
+
+using namespace haste::v0;
+
+#define CHECK_HIP(e)                                                                   \
+  do {                                                                                 \
+    hipError_t err_ = (e);                                                             \
+    if (err_ != hipSuccess) {                                                          \
+      std::fprintf(stderr, "%s failed: %s\n", #e, hipGetErrorString(err_));            \
+      std::exit(3);                                                                    \
+    }                                                                                  \
+  } while (0)
+
+struct DeviceBuf {
+  float* p = nullptr;
+  size_t n = 0;
+  explicit DeviceBuf(size_t count) : n(count) {
+    CHECK_HIP(hipMalloc(reinterpret_cast<void**>(&p), (count ? count : 1) * sizeof(float)));
+    CHECK_HIP(hipMemset(p, 0, (count ? count : 1) * sizeof(float)));
+  }
+  DeviceBuf(const std::vector<float>& h) : DeviceBuf(h.size()) {
+    if (n) CHECK_HIP(hipMemcpy(p, h.data(), n * sizeof(float), hipMemcpyHostToDevice));
+  }
+  ~DeviceBuf() { (void)hipFree(p); }
+  std::vector<float> host() const {
+    std::vector<float> h(n);
+    if (n) CHECK_HIP(hipMemcpy(h.data(), p, n * sizeof(float), hipMemcpyDeviceToHost));
+    return h;
+  }
+  DeviceBuf(const DeviceBuf&) = delete;
+  DeviceBuf& operator=(const DeviceBuf&) = delete;
+};
+
+static FILE* g_in = nullptr;
+static FILE* g_out = nullptr;
+
+static std::vector<float> read_tensor(size_t count) {
+  std::vector<float> v(count);
+  if (count && std::fread(v.data(), sizeof(float), count, g_in) != count) {
+    std::fprintf(stderr, "input file too short\n");
+    std::exit(4);
+  }
+  return v;
+}
+
+static void write_tensor(const DeviceBuf& b) {
+  const std::vector<float> h = b.host();
+  std::fwrite(h.data(), sizeof(float), h.size(), g_out);
+}
+
+// [rows, cols] -> [cols, rows]
+static std::vector<float> transpose(const std::vector<float>& a, size_t rows, size_t cols) {
+  std::vector<float> t(a.size());
+  for (size_t r = 0; r < rows; ++r)
+    for (size_t c = 0; c < cols; ++c) t[c * rows + r] = a[r * cols + c];
+  return t;
+}
+
+static void require_ok(int status, const char* what) {
+  if (status != HASTE_HIP_OK) {
+    std::fprintf(stderr, "%s: %s [%s]\n", what, haste_hip_error_string(status),
+                 haste_hip_last_runtime_error());
+    std::exit(5);
+  }
+}
+
+int main(int argc, char** argv) {
+  if (argc != 9) {
+    std::fprintf(stderr, "usage: api_check <cell> T N C H zoneout in.bin out.bin\n");
+    return 2;
+  }
+  const std::string cell = argv[1];
+  const int T = std::atoi(argv[2]), N = std::atoi(argv[3]), C = std::atoi(argv[4]), H = std::atoi(argv[5]);
+  const float zoneout = (float)std::atof(argv[6]);
+  g_in = std::fopen(argv[7], "rb");
+  g_out = std::fopen(argv[8], "wb");
+  if (!g_in || !g_out) { std::fprintf(stderr, "cannot open files\n"); return 2; }
+
+  hipStream_t stream;
+  CHECK_HIP(hipStreamCreate(&stream));
+  hipblasHandle_t blas = nullptr;  // accepted and ignored by the library
+  const size_t TN = (size_t)T * N, NH = (size_t)N * H;
+  const bool has_mask = zoneout > 0.f;
+
+  if (cell == "lstm" || cell == "layer_norm_lstm") {
+    const bool ln = cell == "layer_norm_lstm";
+    const int G = 4;
+    std::vector<float> W = read_tensor((size_t)C * G * H), R = read_tensor((size_t)H * G * H),
+                       b = read_tensor((size_t)G * H), x = read_tensor(TN * C), h0 = read_tensor(NH),
+                       c0 = read_tensor(NH), dh_new = read_tensor((T + 1) * NH),
+                       dc_new = read_tensor((T + 1) * NH);
+    std::vector<float> gamma, gamma_h, beta_h;
+    if (ln) { gamma = read_tensor((size_t)2 * G * H); gamma_h = read_tensor(H); beta_h = read_tensor(H); }
+    std::vector<float> mask = read_tensor(has_mask ? TN * H : 0);
+
+    DeviceBuf dW_(W), dR_(R), db_(b), dx_(x), dmask(mask);
+    std::vector<float> hinit((T + 1) * NH, 0.f), cinit((T + 1) * NH, 0.f);
+    std::memcpy(hinit.data(), h0.data(), NH * sizeof(float));
+    std::memcpy(cinit.data(), c0.data(), NH * sizeof(float));
+    DeviceBuf h(hinit), c(cinit), v(TN * G * H), tmp_Rh((size_t)N * G * H);
+    DeviceBuf act_Wx(ln ? TN * G * H : 0), act_Rh(ln ? TN * G * H : 0), act_c_norm(ln ? TN * H : 0);
+    DeviceBuf cache1(ln ? TN * 2 : 0), cache2(ln ? TN * 2 : 0), cache3(ln ? TN * 2 : 0);
+    DeviceBuf dgamma(gamma), dgamma_h(gamma_h), dbeta_h(beta_h);
+    const float* maskp = has_mask ? dmask.p : nullptr;
+
+    if (!ln) {
+      lstm::ForwardPass<float> fwd(true, N, C, H, blas, stream);
+      fwd.Run(T, dW_.p, dR_.p, db_.p, dx_.p, h.p, c.p, v.p, tmp_Rh.p, zoneout, maskp);
+      require_ok(fwd.last_status(), "lstm forward");
+    } else {
+      layer_norm::ForwardPass<float> ln1(T * N, G * H, dgamma.p, nullptr, cache1.p);
+      layer_norm::ForwardPass<float> ln2(T * N, G * H, dgamma.p + G * H, nullptr, cache2.p);
+      layer_norm::ForwardPass<float> ln3(T * N, H, dgamma_h.p, dbeta_h.p, cache3.p);
+      layer_norm_lstm::ForwardPass<float> fwd(true, N, C, H, blas, stream);
+      fwd.Run(T, dW_.p, dR_.p, db_.p, dx_.p, h.p, c.p, act_Wx.p, tmp_Rh.p, ln1, v.p, act_Rh.p, ln2,
+              ln3, act_c_norm.p, zoneout, maskp);
+      require_ok(fwd.last_status(), "layer_norm_lstm forward");
+    }
+    CHECK_HIP(hipStreamSynchronize(stream));
+    write_tensor(h);
+    write_tensor(c);
+
+    DeviceBuf x_t(transpose(x, TN, C)), W_t(transpose(W, C, (size_t)G * H)),
+        R_t(transpose(R, H, (size_t)G * H)), ddh_new(dh_new), ddc_new(dc_new);
+    DeviceBuf gdx(TN * C), gdW((size_t)C * G * H), gdR((size_t)H * G * H), gdb((size_t)G * H), gdh(NH),
+        gdc(NH), gdgamma(ln ? (size_t)2 * G * H : 0), gdgamma_h(ln ? H : 0), gdbeta_h(ln ? H : 0);
+    if (!ln) {
+      lstm::BackwardPass<float> bwd(N, C, H, blas, stream);
+      bwd.Run(T, W_t.p, R_t.p, db_.p, x_t.p, h.p, c.p, ddh_new.p, ddc_new.p, gdx.p, gdW.p, gdR.p,
+              gdb.p, gdh.p, gdc.p, v.p, maskp);
+      require_ok(bwd.last_status(), "lstm backward");
+    } else {
+      layer_norm::BackwardPass<float> ln1(T * N, G * H, dgamma.p, nullptr, act_Wx.p, gdgamma.p, nullptr, cache1.p);
+      layer_norm::BackwardPass<float> ln2(T * N, G * H, dgamma.p + G * H, nullptr, act_Rh.p,
+                                          gdgamma.p + G * H, nullptr, cache2.p);
+      layer_norm::BackwardPass<float> ln3(T * N, H, dgamma_h.p, dbeta_h.p, c.p + NH, gdgamma_h.p,
+                                          gdbeta_h.p, cache3.p);
+      layer_norm_lstm::BackwardPass<float> bwd(N, C, H, blas, stream);
+      bwd.Run(T, W_t.p, R_t.p, db_.p, x_t.p, h.p, c.p, ddh_new.p, ddc_new.p, gdx.p, gdW.p, gdR.p,
+              gdb.p, gdh.p, gdc.p, act_Wx.p, ln1, v.p, act_Rh.p, ln2, ln3, act_c_norm.p, maskp);
+      require_ok(bwd.last_status(), "layer_norm_lstm backward");
+    }
+    CHECK_HIP(hipStreamSynchronize(stream));
+    write_tensor(gdx); write_tensor(gdW); write_tensor(gdR); write_tensor(gdb);
+    write_tensor(gdh); write_tensor(gdc);
+    if (ln) { write_tensor(gdgamma); write_tensor(gdgamma_h); write_tensor(gdbeta_h); }
+  } else if (cell == "gru" || cell == "layer_norm_gru") {
+    const bool ln = cell == "layer_norm_gru";
+    const int G = 3;
+    std::vector<float> W = read_tensor((size_t)C * G * H), R = read_tensor((size_t)H * G * H),
+                       bx = read_tensor((size_t)G * H), br = read_tensor((size_t)G * H),
+                       x = read_tensor(TN * C), h0 = read_tensor(NH), dh_new = read_tensor((T + 1) * NH);
+    std::vector<float> gamma;
+    if (ln) gamma = read_tensor((size_t)2 * G * H);
+    std::vector<float> mask = read_tensor(has_mask ? TN * H : 0);
+
+    DeviceBuf dW_(W), dR_(R), dbx_(bx), dbr_(br), dx_(x), dmask(mask), dgamma(gamma);
+    std::vector<float> hinit((T + 1) * NH, 0.f);
+    std::memcpy(hinit.data(), h0.data(), NH * sizeof(float));
+    DeviceBuf h(hinit), v(TN * 4 * H), tmp_Wx(TN * G * H), tmp_Rh((size_t)N * G * H);
+    DeviceBuf act_Wx(ln ? TN * G * H : 0), act_Rh(ln ? TN * G * H : 0), cache1(ln ? TN * 2 : 0),
+        cache2(ln ? TN * 2 : 0);
+    const float* maskp = has_mask ? dmask.p : nullptr;
+    if (!ln) {
+      gru::ForwardPass<float> fwd(true, N, C, H, blas, stream);
+      fwd.Run(T, dW_.p, dR_.p, dbx_.p, dbr_.p, dx_.p, h.p, v.p, tmp_Wx.p, tmp_Rh.p, zoneout, maskp);
+      require_ok(fwd.last_status(), "gru forward");
+    } else {
+      layer_norm::ForwardPass<float> ln1(T * N, G * H, dgamma.p, nullptr, cache1.p);
+      layer_norm::ForwardPass<float> ln2(T * N, G * H, dgamma.p + G * H, nullptr, cache2.p);
+      layer_norm_gru::ForwardPass<float> fwd(true, N, C, H, blas, stream);
+      fwd.Run(T, dW_.p, dR_.p, dbx_.p, dbr_.p, dx_.p, h.p, v.p, act_Wx.p, ln1, tmp_Wx.p, act_Rh.p,
+              ln2, tmp_Rh.p, zoneout, maskp);
+      require_ok(fwd.last_status(), "layer_norm_gru forward");
+    }
+    CHECK_HIP(hipStreamSynchronize(stream));
+    write_tensor(h);
+
+    DeviceBuf x_t(transpose(x, TN, C)), W_t(transpose(W, C, (size_t)G * H)),
+        R_t(transpose(R, H, (size_t)G * H)), ddh_new(dh_new);
+    DeviceBuf gdx(TN * C), gdW((size_t)C * G * H), gdR((size_t)H * G * H), gdbx((size_t)G * H),
+        gdbr((size_t)G * H), gdh(NH), dp(TN * G * H), dq(TN * G * H), gdgamma(ln ? (size_t)2 * G * H : 0);
+    if (!ln) {
+      gru::BackwardPass<float> bwd(N, C, H, blas, stream);
+      bwd.Run(T, W_t.p, R_t.p, dbx_.p, dbr_.p, x_t.p, h.p, v.p, ddh_new.p, gdx.p, gdW.p, gdR.p,
+              gdbx.p, gdbr.p, gdh.p, dp.p, dq.p, maskp);
+      require_ok(bwd.last_status(), "gru backward");
+    } else {
+      layer_norm::BackwardPass<float> ln1(T * N, G * H, dgamma.p, nullptr, act_Wx.p, gdgamma.p, nullptr, cache1.p);
+      layer_norm::BackwardPass<float> ln2(T * N, G * H, dgamma.p + G * H, nullptr, act_Rh.p,
+                                          gdgamma.p + G * H, nullptr, cache2.p);
+      layer_norm_gru::BackwardPass<float> bwd(N, C, H, blas, stream);
+      bwd.Run(T, W_t.p, R_t.p, dbx_.p, dbr_.p, x_t.p, h.p, v.p, ddh_new.p, gdx.p, gdW.p, gdR.p,
+              gdbx.p, gdbr.p, gdh.p, dp.p, dq.p, ln1, ln2, maskp);
+      require_ok(bwd.last_status(), "layer_norm_gru backward");
+    }
+    CHECK_HIP(hipStreamSynchronize(stream));
+    write_tensor(gdx); write_tensor(gdW); write_tensor(gdR); write_tensor(gdbx); write_tensor(gdbr);
+    write_tensor(gdh);
+    if (ln) write_tensor(gdgamma);
+  } else if (cell == "indrnn" || cell == "layer_norm_indrnn") {
+    const bool ln = cell == "layer_norm_indrnn";
+    std::vector<float> W = read_tensor((size_t)C * H), u = read_tensor(H), b = read_tensor(H),
+                       x = read_tensor(TN * C), h0 = read_tensor(NH), dh_new = read_tensor((T + 1) * NH);
+    std::vector<float> gamma;
+    if (ln) gamma = read_tensor((size_t)2 * H);
+    std::vector<float> mask = read_tensor(has_mask ? TN * H : 0);
+    DeviceBuf dW_(W), du_(u), db_(b), dx_(x), dmask(mask), dgamma(gamma);
+    std::vector<float> hinit((T + 1) * NH, 0.f);
+    std::memcpy(hinit.data(), h0.data(), NH * sizeof(float));
+    DeviceBuf h(hinit), workspace(TN * H), act_Wx(ln ? TN * H : 0), cache1(ln ? TN * 2 : 0);
+    const float* maskp = has_mask ? dmask.p : nullptr;
+    if (!ln) {
+      indrnn::ForwardPass<float> fwd(true, N, C, H, blas, stream);
+      fwd.Run(T, dW_.p, du_.p, db_.p, dx_.p, h.p, workspace.p, zoneout, maskp);
+      require_ok(fwd.last_status(), "indrnn forward");
+    } else {
+      layer_norm::ForwardPass<float> ln1(T * N, H, dgamma.p, nullptr, cache1.p);
+      layer_norm_indrnn::ForwardPass<float> fwd(true, N, C, H, blas, stream);
+      fwd.Run(T, dW_.p, du_.p, db_.p, dx_.p, h.p, workspace.p, act_Wx.p, ln1, zoneout, maskp);
+      require_ok(fwd.last_status(), "layer_norm_indrnn forward");
+    }
+    CHECK_HIP(hipStreamSynchronize(stream));
+    write_tensor(h);
+    DeviceBuf x_t(transpose(x, TN, C)), W_t(transpose(W, C, H)), ddh_new(dh_new);
+    DeviceBuf gdx(TN * C), gdW((size_t)C * H), gdu(H), gdb(H), gdh(NH), ws2(TN * H),
+        gdgamma(ln ? (size_t)2 * H : 0);
+    if (!ln) {
+      indrnn::BackwardPass<float> bwd(N, C, H, blas, stream);
+      bwd.Run(T, W_t.p, du_.p, db_.p, x_t.p, h.p, ddh_new.p, gdx.p, gdW.p, gdu.p, gdb.p, gdh.p,
+              ws2.p, maskp);
+      require_ok(bwd.last_status(), "indrnn backward");
+    } else {
+      layer_norm::BackwardPass<float> ln1(T * N, H, dgamma.p, nullptr, act_Wx.p, gdgamma.p, nullptr, cache1.p);
+      layer_norm_indrnn::BackwardPass<float> bwd(N, C, H, blas, stream);
+      bwd.Run(T, W_t.p, du_.p, db_.p, x_t.p, h.p, ddh_new.p, gdx.p, gdW.p, gdu.p, gdb.p, gdh.p,
+              ws2.p, ln1, maskp);
+      require_ok(bwd.last_status(), "layer_norm_indrnn backward");
+    }
+    CHECK_HIP(hipStreamSynchronize(stream));
+    write_tensor(gdx); write_tensor(gdW); write_tensor(gdu); write_tensor(gdb); write_tensor(gdh);
+    if (ln) write_tensor(gdgamma);
+  } else if (cell == "layer_norm") {
+    // rows = T*N, dim = H; forward in two partial calls, backward in two partial calls.
+    const int rows = T * N;
+    std::vector<float> x = read_tensor((size_t)rows * H), gamma = read_tensor(H), beta = read_tensor(H),
+                       dy = read_tensor((size_t)rows * H);
+    DeviceBuf dx_(x), dgamma(gamma), dbeta(beta), ddy(dy), y((size_t)rows * H), cache((size_t)rows * 2),
+        gdx((size_t)rows * H), gdgamma(H), gdbeta(H);
+    layer_norm::ForwardPass<float> fwd(rows, H, dgamma.p, dbeta.p, cache.p);
+    const int first = rows / 2;
+    fwd.RunPartial(stream, first, dx_.p, y.p);
+    require_ok(fwd.last_status(), "layer_norm forward");
+    if (rows - first > 0) {
+      fwd.RunPartial(stream, rows - first, dx_.p + (size_t)first * H, y.p + (size_t)first * H);
+      require_ok(fwd.last_status(), "layer_norm forward");
+    }
+    layer_norm::BackwardPass<float> bwd(rows, H, dgamma.p, dbeta.p, dx_.p, gdgamma.p, gdbeta.p, cache.p);
+    if (rows - first > 0) {
+      bwd.RunPartial(stream, rows - first, ddy.p + (size_t)first * H, gdx.p + (size_t)first * H);
+      require_ok(bwd.last_status(), "layer_norm backward");
+    }
+    if (first > 0) {
+      bwd.RunPartial(stream, first, ddy.p, gdx.p);
+      require_ok(bwd.last_status(), "layer_norm backward");
+    }
+    CHECK_HIP(hipStreamSynchronize(stream));
+    write_tensor(y); write_tensor(cache); write_tensor(gdx); write_tensor(gdgamma); write_tensor(gdbeta);
+  } else {
+    std::fprintf(stderr, "unknown cell %s\n", cell.c_str());
+    return 2;
+  }
+  std::fclose(g_in);
+  std::fclose(g_out);
+  CHECK_HIP(hipStreamDestroy(stream));
+  std::printf("ok\n");
+  return 0;
+}
