@@ -13,7 +13,6 @@ import ctypes
 import json
 import os
 import sys
-import time
 
 import numpy as np
 
@@ -28,6 +27,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget", type=float, default=15.0)
+    ap.add_argument("--workload", choices=["all", "metric", "streaming"], default="all",
+                    help="restrict the run to one workload (for profiling); the JSON line is "
+                         "only complete with 'all'")
     return ap.parse_args()
 
 
@@ -54,22 +56,8 @@ def profile_read(lib, name):
     return total.value, count.value
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: the path has no multi-GPU component "
-              "(got --gpus %d)" % args.gpus, file=sys.stderr)
-        sys.exit(2)
-    import torch
-    from haste_amd import lib as hlib, ops
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU", file=sys.stderr)
-        sys.exit(2)
-    lib = hlib.load()
-    torch.cuda.set_device(0)
-    dev = torch.device("cuda:0")
-
-    # ---- metric config: LSTM fwd+bwd N=64 T=100 C=H=512 -----------------------
+def run_metric(args, torch, lib, ops, dev):
+    """LSTM fwd+bwd N=64 T=100 C=H=512: ms per batch and the per-kernel breakdown."""
     T, N, C, H = 100, 64, 512, 512
     W, R, b, x, dy, dhT, dcT = make_inputs(T, N, C, H)
     Wd, Rd, bd, xd = (torch.from_numpy(a).to(dev) for a in (W, R, b, x))
@@ -101,7 +89,8 @@ def main():
     torch.cuda.synchronize()
     ms_per_step = ev0.elapsed_time(ev1) / args.steps
 
-    # Same K steps again with per-kernel event timing switched on in the library.
+    # The same K steps again with per-kernel event timing switched on in the library
+    # (events on the stream the kernels run on).
     lib.haste_hip_profile_reset()
     lib.haste_hip_profile_enable(1)
     for _ in range(args.steps):
@@ -115,23 +104,31 @@ def main():
                         ("lstm_backward_recurrence", f_rec)):
         total_ms, count = profile_read(lib, name)
         avg_ms = total_ms / max(count, 1)
+        tf = flops / (avg_ms * 1e-3) / 1e12 if avg_ms > 0 else 0.0
         kernels[name] = {"launches_per_step": count / args.steps, "avg_ms": round(avg_ms, 5),
                          "ms_per_step": round(total_ms / args.steps, 5),
-                         "tflops": round(flops / (avg_ms * 1e-3) / 1e12, 3) if avg_ms > 0 else None}
+                         "flops_per_launch": flops, "tflops": round(tf, 3),
+                         "frac_of_fp32_mfma_peak": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)}
     lib.haste_hip_profile_reset()
     dominant = max(kernels, key=lambda k: kernels[k]["ms_per_step"])
     dom = kernels[dominant]
     roofline = {"kernel": dominant, "bound": "mfma", "achieved": dom["tflops"],
                 "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(dom["tflops"] / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None}
-    total_flops = 3.0 * (2.0 * T * N * C * 4 * H + f_rec)
+    total_flops = 3.0 * (f_gemm + f_rec)
+    return dict(ms_per_step=ms_per_step, kernels=kernels, roofline=roofline,
+                tflops_whole_step=total_flops / (ms_per_step * 1e-3) / 1e12,
+                host=(W, R, b, x, dy))
 
-    # ---- streaming inference: N=1 T=2000 C=H=512, microseconds per timestep -----
-    T1, N1 = 2000, 1
+
+def run_streaming(args, torch, lib, ops, dev):
+    """LSTM inference N=1 T=2000 C=H=512: microseconds per timestep."""
+    T1, N1, C, H = 2000, 1, 512, 512
     W1, R1, b1, x1, *_ = make_inputs(T1, N1, C, H, seed=1, forget_bias=0.0)
     W1d, R1d, b1d, x1d = (torch.from_numpy(a).to(dev) for a in (W1, R1, b1, x1))
     h01 = torch.zeros(N1, H, device=dev)
     c01 = torch.zeros(N1, H, device=dev)
+    no_mask = torch.empty(0, 0, 0, device=dev)
 
     def stream_step():
         return ops.lstm_forward(False, 0.0, x1d, h01, c01, W1d, R1d, b1d, no_mask)
@@ -139,6 +136,9 @@ def main():
     for _ in range(3):
         stream_step()
     torch.cuda.synchronize()
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    lib.haste_hip_profile_reset()
     lib.haste_hip_profile_enable(1)
     reps = 10
     ev0.record()
@@ -147,25 +147,57 @@ def main():
     ev1.record()
     torch.cuda.synchronize()
     lib.haste_hip_profile_enable(0)
-    us_per_step_total = ev0.elapsed_time(ev1) * 1e3 / reps / T1
+    us_total = ev0.elapsed_time(ev1) * 1e3 / reps / T1
     rec_ms, rec_n = profile_read(lib, "lstm_forward_recurrence")
     lib.haste_hip_profile_reset()
-    us_per_step_rec = rec_ms * 1e3 / max(rec_n, 1) / T1
+    us_rec = rec_ms * 1e3 / max(rec_n, 1) / T1
     b_step = 4.0 * (4 * H * H + 2 * 4 * H + 4 * H)  # R + Wx_t + b + h,c in + h,c out
-    stream_gbs = b_step / (us_per_step_rec * 1e-6) / 1e9
-    streaming = {"workload": "LSTM inference N=1 T=2000 C=H=512 fp32",
-                 "us_per_timestep": round(us_per_step_total, 4),
-                 "us_per_timestep_recurrence_kernel": round(us_per_step_rec, 4),
-                 "roofline": {"bound": "hbm", "achieved": round(stream_gbs, 1), "peak": PEAK_HBM_GBS,
-                              "unit": "GB/s", "frac": round(stream_gbs / PEAK_HBM_GBS, 4),
-                              "bytes_per_step_model": b_step,
-                              "note": "streamed-R byte model; R is kept on chip, so this is an "
-                                      "equivalent bandwidth, not HBM traffic"}}
+    gbs = b_step / (us_rec * 1e-6) / 1e9
+    out = {"workload": "LSTM inference N=1 T=2000 C=H=512 fp32",
+           "us_per_timestep": round(us_total, 4),
+           "us_per_timestep_recurrence_kernel": round(us_rec, 4),
+           "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
+                        "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4),
+                        "bytes_per_step_model": b_step,
+                        "note": "streamed-R byte model; R is kept on chip, so this is an "
+                                "equivalent bandwidth, not HBM traffic"}}
+    return out, (W1, R1, b1, x1)
 
-    # ---- CPU baseline: torch.nn.LSTM fwd+bwd on the host cores (bounded sample) ---
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the path has no multi-GPU component "
+              "(got --gpus %d)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from haste_amd import lib as hlib, ops
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    lib = hlib.load()
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+
+    if args.workload == "metric":
+        m = run_metric(args, torch, lib, ops, dev)
+        print(json.dumps({"workload": "metric", "ms_per_step": round(m["ms_per_step"], 4),
+                          "kernels": m["kernels"]}))
+        return
+    if args.workload == "streaming":
+        s, _ = run_streaming(args, torch, lib, ops, dev)
+        print(json.dumps(s))
+        return
+
+    m = run_metric(args, torch, lib, ops, dev)
+    streaming, host1 = run_streaming(args, torch, lib, ops, dev)
+
+    # CPU baseline: torch.nn.LSTM fwd+bwd on the host cores (bounded sample).
     cpu = None
     if not args.no_cpu_baseline:
         from oracle import cpu_baseline
+        W, R, b, x, dy = m["host"]
+        W1, R1, b1, x1 = host1
         threads = torch.get_num_threads()
         sec, iters = cpu_baseline.time_lstm_fwd_bwd(W, R, b, x, dy, budget_s=args.cpu_budget)
         sec1, it1 = cpu_baseline.time_lstm_inference(W1, R1, b1, x1[:500], budget_s=5.0)
@@ -178,15 +210,15 @@ def main():
 
     out = {
         "metric": "LSTM fwd+bwd ms/batch (N=64,T=100,H=512 fp32)",
-        "value": round(ms_per_step, 4), "unit": "ms/batch",
+        "value": round(m["ms_per_step"], 4), "unit": "ms/batch",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak",
+        "ms_per_step": round(m["ms_per_step"], 4), "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "LSTM training fwd+bwd N=64 T=100 C=H=512 fp32, forget bias 1, "
                                "caller-side transposes inside the timed step"},
-        "achieved_tflops_whole_step": round(total_flops / (ms_per_step * 1e-3) / 1e12, 3),
-        "roofline": roofline,
-        "kernels": kernels,
+        "achieved_tflops_whole_step": round(m["tflops_whole_step"], 3),
+        "roofline": m["roofline"],
+        "kernels": m["kernels"],
         "streaming_n1": streaming,
         "cpu_baseline": cpu,
     }

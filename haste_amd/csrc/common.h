@@ -45,6 +45,7 @@ struct ControlBlock {
   unsigned int step_flags[kMaxWorkgroups];                 // per-workgroup arrival counts
   unsigned int grid_exit_counter[kCounterStride];          // all workgroups of a launch
   unsigned int tile_counter[4096];                         // split-K arrivals per output tile
+  unsigned int xcd_ticket[16 * kCounterStride];            // per-XCD role tickets (only ever grow)
   unsigned int abort_flag[kCounterStride];                 // set when a barrier wait gives up
 };
 
@@ -56,6 +57,7 @@ struct Workspace {
   float* scratch = nullptr;          // device
   size_t scratch_bytes = 0;
   unsigned int epoch = 0;            // step-flag values handed out so far
+  unsigned int ticket_base = 0;      // per-XCD tickets handed out so far
   unsigned int* host_status = nullptr;      // pinned host word the kernels report aborts to
   unsigned int* host_status_dev = nullptr;  // the same word as the device addresses it
 };
@@ -68,12 +70,19 @@ int get_workspace(hipStream_t stream, size_t scratch_bytes, Workspace* out);
 // stream) and returns the value before the first of them.
 int reserve_epochs(hipStream_t stream, unsigned int count, unsigned int* base);
 
+// Same for the per-XCD role tickets of a launch that places groups on XCDs.
+int reserve_tickets(hipStream_t stream, unsigned int count, unsigned int* base);
+
 // Checks (without synchronizing) whether a persistent kernel launched earlier on
 // this workspace reported a barrier time-out; if so re-zeroes the control block and
 // returns HASTE_HIP_ERROR_STEP_BARRIER once.
 int check_and_clear_abort(hipStream_t stream, Workspace* ws);
 
 int device_cu_count();
+
+// False when the environment variable HASTE_HIP_XCD_LOCAL is set to 0 (forces the
+// cross-XCD exchange path; for experiments).
+bool xcd_local_enabled();
 
 // C[M,N] = op(A)*B (+C): fp32 MFMA GEMM on `stream`. `ws` supplies split-K scratch.
 int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,

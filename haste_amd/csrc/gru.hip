@@ -22,10 +22,7 @@ struct GruFwdParams {
   const float* zoneout_mask;
   const float* dc_mask;  // DropConnect mask [H,3H] or null
   float dc_scale;
-  ControlBlock* cb;
-  unsigned int* host_status;
-  unsigned int spin_limit;
-  unsigned int epoch;
+  LaunchShape ls;
 };
 
 // HS hidden units per workgroup; their 3 gate columns occupy 3*HS of the 16*CT slice
@@ -37,8 +34,11 @@ void gru_forward_kernel(GruFwdParams p) {
   constexpr int NB = 16 * RT;
   constexpr int NCOLS = 16 * CT;
   constexpr int PP = (NB * HS + 255) / 256;
-  constexpr int CHUNK = RT == 4 ? 4 : 8;
+  constexpr int CHUNK = RT == 4 ? 2 : 4;
   extern __shared__ __attribute__((aligned(16))) float lds[];
+  __shared__ unsigned int s_role;
+  const Role role = take_role(p.ls, &s_role);
+  if (!role.active) return;
 
   const int H = p.H, N = p.N, T = p.T;
   const int Kpad = round_up(H, 64);
@@ -46,12 +46,12 @@ void gru_forward_kernel(GruFwdParams p) {
   float* red = lds + Kpad * NCOLS;
 
   const int tid = threadIdx.x;
-  const int j0 = blockIdx.x * HS;
-  const int n0 = blockIdx.y * NB;
+  const int j0 = role.cw * HS;
+  const int n0 = role.bt * NB;
   const size_t NH = (size_t)N * H;
 
   GroupSync gs;
-  group_sync_init(gs, p.cb, blockIdx.y, gridDim.x, blockIdx.x, p.epoch, p.host_status, p.spin_limit);
+  group_sync_init(gs, p.ls, role);
 
   for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
     const int k = idx / NCOLS, cidx = idx % NCOLS;
@@ -114,7 +114,7 @@ void gru_forward_kernel(GruFwdParams p) {
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
     slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, N - n0, H, Kpad, w_lds,
-                                vec_ok, acc);
+                                vec_ok, gs.same_xcd, acc);
     store_partials<RT, CT>(red, acc);
     __syncthreads();
 
@@ -140,7 +140,7 @@ void gru_forward_kernel(GruFwdParams p) {
           if (p.training) h_new = (h_new - h_prev[pp]) * mk[pp] + h_prev[pp];
           else h_new = p.zoneout_prob * h_prev[pp] + (1.0f - p.zoneout_prob) * h_new;
         }
-        store_exchanged(&p.h[(size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp]], h_new);
+        store_exchanged(gs, &p.h[(size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp]], h_new);
         h_prev[pp] = h_new;
       }
     }
@@ -161,10 +161,7 @@ struct GruBwdParams {
   float* dq;            // [T,N,3H]
   const float* zoneout_mask;
   float* db_partial;    // [batch tiles, 6H] scratch
-  ControlBlock* cb;
-  unsigned int* host_status;
-  unsigned int spin_limit;
-  unsigned int epoch;
+  LaunchShape ls;
 };
 
 template <int RT>
@@ -174,8 +171,11 @@ void gru_backward_kernel(GruBwdParams p) {
   constexpr int NB = 16 * RT;
   constexpr int NCOLS = 16;
   constexpr int PP = RT;
-  constexpr int CHUNK = RT == 1 ? 16 : (RT == 2 ? 8 : 4);
+  constexpr int CHUNK = RT == 1 ? 8 : (RT == 2 ? 4 : 2);
   extern __shared__ __attribute__((aligned(16))) float lds[];
+  __shared__ unsigned int s_role;
+  const Role role = take_role(p.ls, &s_role);
+  if (!role.active) return;
   __shared__ unsigned int s_flag;
 
   const int H = p.H, N = p.N, T = p.T;
@@ -185,12 +185,12 @@ void gru_backward_kernel(GruBwdParams p) {
   float* red = lds + Kpad * NCOLS;  // max(4*NB*16, NB*6*16) floats
 
   const int tid = threadIdx.x;
-  const int j0 = blockIdx.x * HSB;
-  const int n0 = blockIdx.y * NB;
+  const int j0 = role.cw * HSB;
+  const int n0 = role.bt * NB;
   const size_t NH = (size_t)N * H;
 
   GroupSync gs;
-  group_sync_init(gs, p.cb, blockIdx.y, gridDim.x, blockIdx.x, p.epoch, p.host_status, p.spin_limit);
+  group_sync_init(gs, p.ls, role);
 
   for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
     const int k = idx / NCOLS, cidx = idx % NCOLS;
@@ -265,9 +265,9 @@ void gru_backward_kernel(GruBwdParams p) {
         p.dp[o3] = dp_z;
         p.dp[o3 + H] = dp_r;
         p.dp[o3 + 2 * H] = dp_g;
-        store_exchanged(&p.dq[o3], dp_z);
-        store_exchanged(&p.dq[o3 + H], dp_r);
-        store_exchanged(&p.dq[o3 + 2 * H], dq_g);
+        store_exchanged(gs, &p.dq[o3], dp_z);
+        store_exchanged(gs, &p.dq[o3 + H], dp_r);
+        store_exchanged(gs, &p.dq[o3 + 2 * H], dq_g);
         dbacc[pp][0] += dp_z;
         dbacc[pp][1] += dp_r;
         dbacc[pp][2] += dp_g;
@@ -284,7 +284,7 @@ void gru_backward_kernel(GruBwdParams p) {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc[rt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
     slice_matmul<RT, 1, CHUNK>(p.dq + ((size_t)t * N + n0) * 3 * H, 3 * H, N - n0, K, Kpad, w_lds,
-                               vec_ok, acc);
+                               vec_ok, gs.same_xcd, acc);
     store_partials<RT, 1>(red, acc);
     __syncthreads();
 #pragma unroll
@@ -306,12 +306,12 @@ void gru_backward_kernel(GruBwdParams p) {
     const int g = tid / HSB, jj = tid % HSB;
     float s = 0.f;
     for (int r = 0; r < NB; ++r) s += red[(r * 6 + g) * HSB + jj];
-    if (j0 + jj < H) p.db_partial[(size_t)blockIdx.y * 6 * H + g * H + j0 + jj] = s;
+    if (j0 + jj < H) p.db_partial[(size_t)role.bt * 6 * H + g * H + j0 + jj] = s;
   }
-  if (grid_last_arrival(p.cb, gridDim.x * gridDim.y, &s_flag)) {
+  if (grid_last_arrival(p.ls.cb, (unsigned)(p.ls.gx * p.ls.gy), &s_flag)) {
     for (int col = tid; col < 6 * H; col += 256) {
       float s = 0.f;
-      for (int bt = 0; bt < (int)gridDim.y; ++bt) s += p.db_partial[(size_t)bt * 6 * H + col];
+      for (int bt = 0; bt < p.ls.gy; ++bt) s += p.db_partial[(size_t)bt * 6 * H + col];
       if (col < 3 * H) p.dbx[col] += s;
       else p.dbr[col - 3 * H] += s;
     }
@@ -337,29 +337,19 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
   p.R = R; p.bx = bx; p.br = br; p.h = h; p.v = v; p.Wx = tmp_Wx;
   p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
   p.dc_mask = dc_mask; p.dc_scale = dc_scale;
-  p.cb = ws.control; p.host_status = ws.host_status_dev; p.spin_limit = kSpinLimit;
-  HASTE_HIP_PROPAGATE(reserve_epochs(stream, (unsigned)T + 1, &p.epoch));
-
-  const int cus = device_cu_count();
-  struct Cand { int rt, ct, hs; };
-  const Cand cands[] = {{1, 2, 8}, {1, 3, 16}, {1, 1, 4}, {2, 2, 8}, {2, 3, 16}, {2, 1, 4},
-                        {4, 2, 8}, {4, 3, 16}, {4, 1, 4}};
-  for (const Cand& cd : cands) {
-    const int NB = 16 * cd.rt;
-    const int gx = (H + cd.hs - 1) / cd.hs, gy = (N + NB - 1) / NB;
-    if (gy > kMaxGroups || (long long)gx * gy > cus || gx * gy > kMaxWorkgroups) continue;
-    const size_t lds = fwd_lds_bytes(H, cd.rt, cd.ct);
-    if (lds > kMaxLdsBytes) continue;
-    dim3 grid(gx, gy);
+  const ForwardTile tile = pick_forward_tile(3, N, H, 0);
+  if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  LaunchPlan plan;
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.lds_bytes, (unsigned)T + 1, &plan));
+  p.ls = plan.shape;
 #define HASTE_LAUNCH_FWD(RT_, CT_, HS_)                                                       \
-    if (cd.rt == RT_ && cd.ct == CT_)                                                         \
-      return launch_persistent("gru_forward_recurrence", gru_forward_kernel<RT_, CT_, HS_>,   \
-                               grid, lds, p, stream);
-    HASTE_LAUNCH_FWD(1, 1, 4) HASTE_LAUNCH_FWD(1, 2, 8) HASTE_LAUNCH_FWD(1, 3, 16)
-    HASTE_LAUNCH_FWD(2, 1, 4) HASTE_LAUNCH_FWD(2, 2, 8) HASTE_LAUNCH_FWD(2, 3, 16)
-    HASTE_LAUNCH_FWD(4, 1, 4) HASTE_LAUNCH_FWD(4, 2, 8) HASTE_LAUNCH_FWD(4, 3, 16)
+  if (tile.rt == RT_ && tile.hs == HS_)                                                       \
+    return launch_persistent("gru_forward_recurrence", gru_forward_kernel<RT_, CT_, HS_>,     \
+                             plan, p, stream);
+  HASTE_LAUNCH_FWD(1, 1, 4) HASTE_LAUNCH_FWD(1, 2, 8) HASTE_LAUNCH_FWD(1, 3, 16)
+  HASTE_LAUNCH_FWD(2, 1, 4) HASTE_LAUNCH_FWD(2, 2, 8) HASTE_LAUNCH_FWD(2, 3, 16)
+  HASTE_LAUNCH_FWD(4, 1, 4) HASTE_LAUNCH_FWD(4, 2, 8) HASTE_LAUNCH_FWD(4, 3, 16)
 #undef HASTE_LAUNCH_FWD
-  }
   return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 }
 
@@ -371,23 +361,12 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
   HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && v && dh_new);
   HASTE_HIP_REQUIRE(dx && dW && dR && dbx && dbr && dh && dp && dq);
-  const int cus = device_cu_count();
-  const int gx = (H + 15) / 16;
-  int rt = 0;
-  for (int cand : {1, 2, 4}) {
-    const int gy = (N + 16 * cand - 1) / (16 * cand);
-    const size_t lds = bwd_lds_bytes(3 * H, cand) + (size_t)2 * 16 * cand * 16 * sizeof(float);
-    if (gy <= kMaxGroups && (long long)gx * gy <= cus && gx * gy <= kMaxWorkgroups &&
-        lds <= kMaxLdsBytes) {
-      rt = cand;
-      break;
-    }
-  }
-  if (rt == 0) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
-  const int gy = (N + 16 * rt - 1) / (16 * rt);
+  // per row: max(4 partial tiles, the 6 bias-gradient columns) of 16 floats
+  const BackwardTile tile = pick_backward_tile(3 * H, N, H, 96);
+  if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 
   Workspace ws;
-  HASTE_HIP_PROPAGATE(get_workspace(stream, (size_t)gy * 6 * H * sizeof(float), &ws));
+  HASTE_HIP_PROPAGATE(get_workspace(stream, (size_t)tile.gy * 6 * H * sizeof(float), &ws));
   HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 
   GruBwdParams p;
@@ -395,15 +374,14 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   p.R_t = R_t; p.h = h; p.v = v; p.dh_new = dh_new;
   p.dbx = dbx; p.dbr = dbr; p.dh = dh; p.dp = dp; p.dq = dq; p.zoneout_mask = zoneout_mask;
   p.db_partial = ws.scratch;
-  p.cb = ws.control; p.host_status = ws.host_status_dev; p.spin_limit = kSpinLimit;
-  HASTE_HIP_PROPAGATE(reserve_epochs(stream, (unsigned)T + 1, &p.epoch));
-  // the reduction of the bias gradients needs NB*6*16 floats, more than the 4 partial tiles
-  const size_t lds = bwd_lds_bytes(3 * H, rt) + (size_t)2 * 16 * rt * 16 * sizeof(float);
-  dim3 grid(gx, gy);
+  LaunchPlan plan;
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.lds_bytes, (unsigned)T + 1, &plan));
+  p.ls = plan.shape;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
-  if (rt == 1) rc = launch_persistent("gru_backward_recurrence", gru_backward_kernel<1>, grid, lds, p, stream);
-  if (rt == 2) rc = launch_persistent("gru_backward_recurrence", gru_backward_kernel<2>, grid, lds, p, stream);
-  if (rt == 4) rc = launch_persistent("gru_backward_recurrence", gru_backward_kernel<4>, grid, lds, p, stream);
+  const char* name = "gru_backward_recurrence";
+  if (tile.rt == 1) rc = launch_persistent(name, gru_backward_kernel<1>, plan, p, stream);
+  if (tile.rt == 2) rc = launch_persistent(name, gru_backward_kernel<2>, plan, p, stream);
+  if (tile.rt == 4) rc = launch_persistent(name, gru_backward_kernel<4>, plan, p, stream);
   HASTE_HIP_PROPAGATE(rc);
 
   const int TN = T * N;

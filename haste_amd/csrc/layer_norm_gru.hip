@@ -26,10 +26,7 @@ struct LnGruFwdParams {
   float zoneout_prob;
   const float* zoneout_mask;
   float* part2;          // exchange [groups][gx][NB][2]
-  ControlBlock* cb;
-  unsigned int* host_status;
-  unsigned int spin_limit;
-  unsigned int epoch;
+  LaunchShape ls;
 };
 
 template <int RT, int CT, int HS>
@@ -39,8 +36,11 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
   constexpr int NB = 16 * RT;
   constexpr int NCOLS = 16 * CT;
   constexpr int PP = (NB * HS + 255) / 256;
-  constexpr int CHUNK = RT == 4 ? 4 : 8;
+  constexpr int CHUNK = RT == 4 ? 2 : 4;
   extern __shared__ __attribute__((aligned(16))) float lds[];
+  __shared__ unsigned int s_role;
+  const Role role = take_role(p.ls, &s_role);
+  if (!role.active) return;
 
   const int H = p.H, N = p.N, T = p.T;
   const int Kpad = round_up(H, 64);
@@ -49,16 +49,16 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
   float* stat = red + 4 * NB * NCOLS;
 
   const int tid = threadIdx.x;
-  const int gx = gridDim.x;
-  const int j0 = blockIdx.x * HS;
-  const int n0 = blockIdx.y * NB;
+  const int gx = p.ls.gx;
+  const int j0 = role.cw * HS;
+  const int n0 = role.bt * NB;
   const size_t NH = (size_t)N * H;
   const int own_units = (H - j0) < HS ? (H - j0) : HS;
   const int last_units = H - (gx - 1) * HS;
-  float* part2 = p.part2 + (size_t)blockIdx.y * gx * NB * 2;
+  float* part2 = p.part2 + (size_t)role.bt * gx * NB * 2;
 
   GroupSync gs;
-  group_sync_init(gs, p.cb, blockIdx.y, gx, blockIdx.x, p.epoch, p.host_status, p.spin_limit);
+  group_sync_init(gs, p.ls, role);
 
   for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
     const int k = idx / NCOLS, cidx = idx % NCOLS;
@@ -114,7 +114,7 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
     slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, N - n0, H, Kpad, w_lds,
-                                vec_ok, acc);
+                                vec_ok, gs.same_xcd, acc);
     store_partials<RT, CT>(red, acc);
     __syncthreads();
 
@@ -141,7 +141,7 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
       }
       q = segment_sum<HS>(q);
       if (pc[pp] == 0 && tid + 256 * pp < NB * HS)
-        store_exchanged2(part2 + ((size_t)blockIdx.x * NB + pl[pp]) * 2, mean, q);
+        store_exchanged2(gs, part2 + ((size_t)role.cw * NB + pl[pp]) * 2, mean, q);
     }
     group_arrive(gs);
     group_wait(gs);
@@ -171,9 +171,9 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
           if (p.training) h_new = (h_new - h_prev[pp]) * mk[pp] + h_prev[pp];
           else h_new = p.zoneout_prob * h_prev[pp] + (1.0f - p.zoneout_prob) * h_new;
         }
-        store_exchanged(&p.h[(size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp]], h_new);
+        store_exchanged(gs, &p.h[(size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp]], h_new);
         h_prev[pp] = h_new;
-        if (blockIdx.x == 0 && pc[pp] == 0 && p.cache2 != nullptr) {
+        if (role.cw == 0 && pc[pp] == 0 && p.cache2 != nullptr) {
           p.cache2[((size_t)t * N + pn[pp]) * 2 + 0] = mu;
           p.cache2[((size_t)t * N + pn[pp]) * 2 + 1] = is;
         }
@@ -202,10 +202,7 @@ struct LnGruBwdParams {
   const float* zoneout_mask;
   float* part;           // exchange [groups][gx][NB][4]
   float* col_partial;    // [batch tiles][9][H]
-  ControlBlock* cb;
-  unsigned int* host_status;
-  unsigned int spin_limit;
-  unsigned int epoch;
+  LaunchShape ls;
 };
 
 template <int RT>
@@ -215,9 +212,12 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
   constexpr int NB = 16 * RT;
   constexpr int NCOLS = 16;
   constexpr int PP = RT;
-  constexpr int CHUNK = RT == 1 ? 16 : (RT == 2 ? 8 : 4);
+  constexpr int CHUNK = RT == 1 ? 8 : (RT == 2 ? 4 : 2);
   constexpr int NACC = 9;  // dbx x3, dbr x3, dgamma2 x3
   extern __shared__ __attribute__((aligned(16))) float lds[];
+  __shared__ unsigned int s_role;
+  const Role role = take_role(p.ls, &s_role);
+  if (!role.active) return;
   __shared__ unsigned int s_flag;
 
   const int H = p.H, N = p.N, T = p.T;
@@ -228,14 +228,14 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
   float* sums = red + NB * NACC * HSB;
 
   const int tid = threadIdx.x;
-  const int gx = gridDim.x;
-  const int j0 = blockIdx.x * HSB;
-  const int n0 = blockIdx.y * NB;
+  const int gx = p.ls.gx;
+  const int j0 = role.cw * HSB;
+  const int n0 = role.bt * NB;
   const size_t NH = (size_t)N * H;
-  float* part = p.part + (size_t)blockIdx.y * gx * NB * 4;
+  float* part = p.part + (size_t)role.bt * gx * NB * 4;
 
   GroupSync gs;
-  group_sync_init(gs, p.cb, blockIdx.y, gx, blockIdx.x, p.epoch, p.host_status, p.spin_limit);
+  group_sync_init(gs, p.ls, role);
 
   for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
     const int k = idx / NCOLS, cidx = idx % NCOLS;
@@ -341,7 +341,7 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
       t1 = segment_sum<HSB>(t1);
       t2 = segment_sum<HSB>(t2);
       if (pc[pp] == 0)
-        store_exchanged4(part + ((size_t)blockIdx.x * NB + pl[pp]) * 4, t0, t1, t2, 0.f);
+        store_exchanged4(gs, part + ((size_t)role.cw * NB + pl[pp]) * 4, t0, t1, t2, 0.f);
     }
     group_arrive(gs);
     group_wait(gs);
@@ -357,7 +357,7 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
         float* dqt = p.dq + ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
 #pragma unroll
         for (int k = 0; k < 3; ++k)
-          store_exchanged(dqt + (size_t)k * H,
+          store_exchanged(gs, dqt + (size_t)k * H,
                           (2.0f * xc[pp][k] * dsigma * inv3H) + (is2 * gd[pp][k]) + (dmu * inv3H));
       }
     }
@@ -369,7 +369,7 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc[rt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
     slice_matmul<RT, 1, CHUNK>(p.dq + ((size_t)t * N + n0) * 3 * H, 3 * H, N - n0, K, Kpad, w_lds,
-                               vec_ok, acc);
+                               vec_ok, gs.same_xcd, acc);
     store_partials<RT, 1>(red, acc);
     __syncthreads();
 #pragma unroll
@@ -392,13 +392,13 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
     const int a = tid / HSB, jj = tid % HSB;
     float sum = 0.f;
     for (int r = 0; r < NB; ++r) sum += red[(r * NACC + a) * HSB + jj];
-    if (j0 + jj < H) p.col_partial[((size_t)blockIdx.y * NACC + a) * H + j0 + jj] = sum;
+    if (j0 + jj < H) p.col_partial[((size_t)role.bt * NACC + a) * H + j0 + jj] = sum;
   }
-  if (grid_last_arrival(p.cb, gridDim.x * gridDim.y, &s_flag)) {
+  if (grid_last_arrival(p.ls.cb, (unsigned)(p.ls.gx * p.ls.gy), &s_flag)) {
     for (int idx = tid; idx < NACC * H; idx += 256) {
       const int a = idx / H, col = idx % H;
       float sum = 0.f;
-      for (int bt = 0; bt < (int)gridDim.y; ++bt) sum += p.col_partial[((size_t)bt * NACC + a) * H + col];
+      for (int bt = 0; bt < p.ls.gy; ++bt) sum += p.col_partial[((size_t)bt * NACC + a) * H + col];
       if (a < 3) p.dbx[a * H + col] += sum;
       else if (a < 6) p.dbr[(a - 3) * H + col] += sum;
       else p.dgamma2[(a - 6) * H + col] += sum;
@@ -428,26 +428,10 @@ int haste_hip_layer_norm_gru_forward_f32(int training, int steps, int batch_size
   HASTE_HIP_REQUIRE(W && R && bx && br && x && h && act_Wx && gamma1 && tmp_Wx_norm && act_Rh && gamma2);
   HASTE_HIP_REQUIRE(!training || v != nullptr);
   hipStream_t stream = as_stream(stream_);
-  const int cus = device_cu_count();
-
-  struct Cand { int rt, ct, hs; };
-  const Cand cands[] = {{1, 2, 8}, {1, 3, 16}, {1, 1, 4}, {2, 2, 8}, {2, 3, 16}, {2, 1, 4},
-                        {4, 2, 8}, {4, 3, 16}, {4, 1, 4}};
-  const Cand* pick = nullptr;
-  int gx = 0, gy = 0;
-  size_t lds = 0;
-  for (const Cand& cd : cands) {
-    const int NB = 16 * cd.rt;
-    gx = (H + cd.hs - 1) / cd.hs;
-    gy = (N + NB - 1) / NB;
-    lds = fwd_lds_bytes(H, cd.rt, cd.ct) + (size_t)NB * 2 * sizeof(float);
-    if (gy > kMaxGroups || (long long)gx * gy > cus || gx * gy > kMaxWorkgroups) continue;
-    if (lds > kMaxLdsBytes) continue;
-    pick = &cd;
-    break;
-  }
-  if (pick == nullptr) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
-  const int NB = 16 * pick->rt;
+  const ForwardTile tile = pick_forward_tile(3, N, H, 2 * sizeof(float));
+  if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  const int gx = tile.gx, gy = tile.gy;
+  const int NB = 16 * tile.rt;
   const size_t part_floats = (size_t)gy * gx * NB * 2;
 
   Workspace ws;
@@ -463,13 +447,13 @@ int haste_hip_layer_norm_gru_forward_f32(int training, int steps, int batch_size
   p.gamma2 = gamma2; p.cache2 = cache2;
   p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
   p.part2 = ws.scratch;
-  p.cb = ws.control; p.host_status = ws.host_status_dev; p.spin_limit = kSpinLimit;
-  HASTE_HIP_PROPAGATE(reserve_epochs(stream, 2u * (unsigned)T + 1, &p.epoch));
-  dim3 grid(gx, gy);
+  LaunchPlan plan;
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.lds_bytes, 2u * (unsigned)T + 1, &plan));
+  p.ls = plan.shape;
 #define HASTE_LAUNCH(RT_, CT_, HS_)                                                          \
-  if (pick->rt == RT_ && pick->ct == CT_)                                                    \
+  if (tile.rt == RT_ && tile.hs == HS_)                                                      \
     return launch_persistent("layer_norm_gru_forward_recurrence",                            \
-                             ln_gru_forward_kernel<RT_, CT_, HS_>, grid, lds, p, stream);
+                             ln_gru_forward_kernel<RT_, CT_, HS_>, plan, p, stream);
   HASTE_LAUNCH(1, 1, 4) HASTE_LAUNCH(1, 2, 8) HASTE_LAUNCH(1, 3, 16)
   HASTE_LAUNCH(2, 1, 4) HASTE_LAUNCH(2, 2, 8) HASTE_LAUNCH(2, 3, 16)
   HASTE_LAUNCH(4, 1, 4) HASTE_LAUNCH(4, 2, 8) HASTE_LAUNCH(4, 3, 16)
@@ -495,24 +479,11 @@ int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_s
   HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && v && dh_new && dx && dW && dR && dbx && dbr && dh);
   HASTE_HIP_REQUIRE(dp && dq && act_Wx && gamma1 && dgamma1 && act_Rh && gamma2 && dgamma2 && cache2);
   hipStream_t stream = as_stream(stream_);
-  const int cus = device_cu_count();
-  const int gx = (H + 15) / 16;
-  int rt = 0;
-  size_t lds = 0;
-  for (int cand : {1, 2, 4}) {
-    const int gy = (N + 16 * cand - 1) / (16 * cand);
-    const int NB = 16 * cand;
-    const int Kpad = (3 * H + 63) / 64 * 64;
-    lds = ((size_t)Kpad * 16 + (size_t)NB * 9 * 16 + (size_t)NB * 4) * sizeof(float);
-    if (gy <= kMaxGroups && (long long)gx * gy <= cus && gx * gy <= kMaxWorkgroups &&
-        lds <= kMaxLdsBytes) {
-      rt = cand;
-      break;
-    }
-  }
-  if (rt == 0) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  // per row: 9 column-sum accumulators of 16 floats (covers the 4 partial tiles) + 4 sums
+  const BackwardTile tile = pick_backward_tile(3 * H, N, H, 9 * 16 + 4);
+  if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  const int gx = tile.gx, gy = tile.gy, rt = tile.rt;
   const int NB = 16 * rt;
-  const int gy = (N + NB - 1) / NB;
   const size_t part_floats = (size_t)gy * gx * NB * 4;
   const size_t col_floats = (size_t)gy * 9 * H;
 
@@ -527,14 +498,14 @@ int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_s
   p.act_Rh = act_Rh; p.gamma2 = gamma2; p.dgamma2 = dgamma2; p.cache2 = cache2;
   p.zoneout_mask = zoneout_mask;
   p.part = ws.scratch; p.col_partial = ws.scratch + part_floats;
-  p.cb = ws.control; p.host_status = ws.host_status_dev; p.spin_limit = kSpinLimit;
-  HASTE_HIP_PROPAGATE(reserve_epochs(stream, 2u * (unsigned)T + 1, &p.epoch));
-  dim3 grid(gx, gy);
+  LaunchPlan plan;
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.lds_bytes, 2u * (unsigned)T + 1, &plan));
+  p.ls = plan.shape;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const char* name = "layer_norm_gru_backward_recurrence";
-  if (rt == 1) rc = launch_persistent(name, ln_gru_backward_kernel<1>, grid, lds, p, stream);
-  if (rt == 2) rc = launch_persistent(name, ln_gru_backward_kernel<2>, grid, lds, p, stream);
-  if (rt == 4) rc = launch_persistent(name, ln_gru_backward_kernel<4>, grid, lds, p, stream);
+  if (rt == 1) rc = launch_persistent(name, ln_gru_backward_kernel<1>, plan, p, stream);
+  if (rt == 2) rc = launch_persistent(name, ln_gru_backward_kernel<2>, plan, p, stream);
+  if (rt == 4) rc = launch_persistent(name, ln_gru_backward_kernel<4>, plan, p, stream);
   HASTE_HIP_PROPAGATE(rc);
 
   const int TN = T * N;

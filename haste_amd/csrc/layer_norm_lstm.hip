@@ -34,10 +34,7 @@ struct LnLstmFwdParams {
   const float* zoneout_mask;
   float* part2;           // exchange [groups][gx][NB][2]
   float* part3;           // exchange [groups][gx][NB][2]
-  ControlBlock* cb;
-  unsigned int* host_status;
-  unsigned int spin_limit;
-  unsigned int epoch;
+  LaunchShape ls;
 };
 
 template <int RT, int CT>
@@ -47,8 +44,11 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
   constexpr int NB = 16 * RT;
   constexpr int NCOLS = 16 * CT;
   constexpr int PP = (NB * HS + 255) / 256;
-  constexpr int CHUNK = RT == 4 ? 4 : 8;
+  constexpr int CHUNK = RT == 4 ? 2 : 4;
   extern __shared__ __attribute__((aligned(16))) float lds[];
+  __shared__ unsigned int s_role;
+  const Role role = take_role(p.ls, &s_role);
+  if (!role.active) return;
 
   const int H = p.H, N = p.N, T = p.T;
   const int Kpad = round_up(H, 64);
@@ -57,17 +57,17 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
   float* stat = red + 4 * NB * NCOLS;  // [NB][2]
 
   const int tid = threadIdx.x;
-  const int gx = gridDim.x;
-  const int j0 = blockIdx.x * HS;
-  const int n0 = blockIdx.y * NB;
+  const int gx = p.ls.gx;
+  const int j0 = role.cw * HS;
+  const int n0 = role.bt * NB;
   const size_t NH = (size_t)N * H;
   const int own_units = (H - j0) < HS ? (H - j0) : HS;     // valid hidden units here
   const int last_units = H - (gx - 1) * HS;                 // ... in the last workgroup
-  float* part2 = p.part2 + (size_t)blockIdx.y * gx * NB * 2;
-  float* part3 = p.part3 + (size_t)blockIdx.y * gx * NB * 2;
+  float* part2 = p.part2 + (size_t)role.bt * gx * NB * 2;
+  float* part3 = p.part3 + (size_t)role.bt * gx * NB * 2;
 
   GroupSync gs;
-  group_sync_init(gs, p.cb, blockIdx.y, gx, blockIdx.x, p.epoch, p.host_status, p.spin_limit);
+  group_sync_init(gs, p.ls, role);
 
   for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
     const int k = idx / NCOLS, cidx = idx % NCOLS;
@@ -132,7 +132,7 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
     slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, N - n0, H, Kpad, w_lds,
-                                vec_ok, acc);
+                                vec_ok, gs.same_xcd, acc);
     store_partials<RT, CT>(red, acc);
     __syncthreads();
 
@@ -161,7 +161,7 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
       }
       q = segment_sum<HS>(q);
       if (pc[pp] == 0 && tid + 256 * pp < NB * HS)
-        store_exchanged2(part2 + ((size_t)blockIdx.x * NB + pl[pp]) * 2, mean, q);
+        store_exchanged2(gs, part2 + ((size_t)role.cw * NB + pl[pp]) * 2, mean, q);
     }
     group_arrive(gs);
     group_wait(gs);  // every workgroup's moments of h*R
@@ -193,7 +193,7 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
         c_new[pp] = gf * c_prev[pp] + gi * gg;
         p.c[(size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp]] = c_new[pp];
         c_prev[pp] = c_new[pp];
-        if (blockIdx.x == 0 && pc[pp] == 0 && p.cache2 != nullptr) {
+        if (role.cw == 0 && pc[pp] == 0 && p.cache2 != nullptr) {
           p.cache2[((size_t)t * N + pn[pp]) * 2 + 0] = mu;
           p.cache2[((size_t)t * N + pn[pp]) * 2 + 1] = is;
         }
@@ -204,7 +204,7 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
       const float d = cv - mean;
       const float q = segment_sum<HS>(colok[pp] ? d * d : 0.f);
       if (pc[pp] == 0 && tid + 256 * pp < NB * HS)
-        store_exchanged2(part3 + ((size_t)blockIdx.x * NB + pl[pp]) * 2, mean, q);
+        store_exchanged2(gs, part3 + ((size_t)role.cw * NB + pl[pp]) * 2, mean, q);
     }
     group_arrive(gs);
     group_wait(gs);  // every workgroup's moments of c
@@ -223,9 +223,9 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
           if (p.training) h_new = (h_new - h_prev[pp]) * mk[pp] + h_prev[pp];
           else h_new = p.zoneout_prob * h_prev[pp] + (1.0f - p.zoneout_prob) * h_new;
         }
-        store_exchanged(&p.h[(size_t)(t + 1) * NH + e], h_new);
+        store_exchanged(gs, &p.h[(size_t)(t + 1) * NH + e], h_new);
         h_prev[pp] = h_new;
-        if (blockIdx.x == 0 && pc[pp] == 0 && p.cache3 != nullptr) {
+        if (role.cw == 0 && pc[pp] == 0 && p.cache3 != nullptr) {
           p.cache3[((size_t)t * N + pn[pp]) * 2 + 0] = mu;
           p.cache3[((size_t)t * N + pn[pp]) * 2 + 1] = is;
         }
@@ -259,10 +259,7 @@ struct LnLstmBwdParams {
   float* part_a;           // exchange [groups][gx][NB][4]
   float* part_b;           // exchange [groups][gx][NB][4]
   float* col_partial;      // [batch tiles][10][H]
-  ControlBlock* cb;
-  unsigned int* host_status;
-  unsigned int spin_limit;
-  unsigned int epoch;
+  LaunchShape ls;
 };
 
 template <int RT>
@@ -272,9 +269,12 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   constexpr int NB = 16 * RT;
   constexpr int NCOLS = 16;
   constexpr int PP = RT;
-  constexpr int CHUNK = RT == 1 ? 16 : (RT == 2 ? 8 : 4);
+  constexpr int CHUNK = RT == 1 ? 8 : (RT == 2 ? 4 : 2);
   constexpr int NACC = 10;  // db x4, dgamma2 x4, dgamma_h, dbeta_h
   extern __shared__ __attribute__((aligned(16))) float lds[];
+  __shared__ unsigned int s_role;
+  const Role role = take_role(p.ls, &s_role);
+  if (!role.active) return;
   __shared__ unsigned int s_flag;
 
   const int H = p.H, N = p.N, T = p.T;
@@ -285,15 +285,15 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   float* sums = red + NB * NACC * HSB;   // [NB][4]
 
   const int tid = threadIdx.x;
-  const int gx = gridDim.x;
-  const int j0 = blockIdx.x * HSB;
-  const int n0 = blockIdx.y * NB;
+  const int gx = p.ls.gx;
+  const int j0 = role.cw * HSB;
+  const int n0 = role.bt * NB;
   const size_t NH = (size_t)N * H;
-  float* part_a = p.part_a + (size_t)blockIdx.y * gx * NB * 4;
-  float* part_b = p.part_b + (size_t)blockIdx.y * gx * NB * 4;
+  float* part_a = p.part_a + (size_t)role.bt * gx * NB * 4;
+  float* part_b = p.part_b + (size_t)role.bt * gx * NB * 4;
 
   GroupSync gs;
-  group_sync_init(gs, p.cb, blockIdx.y, gx, blockIdx.x, p.epoch, p.host_status, p.spin_limit);
+  group_sync_init(gs, p.ls, role);
 
   for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
     const int k = idx / NCOLS, cidx = idx % NCOLS;
@@ -386,7 +386,7 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
       const float s1 = segment_sum<HSB>(xc3[pp]);
       const float s2 = segment_sum<HSB>(gd3[pp]);
       if (pc[pp] == 0)
-        store_exchanged4(part_a + ((size_t)blockIdx.x * NB + pl[pp]) * 4, s0, s1, s2, 0.f);
+        store_exchanged4(gs, part_a + ((size_t)role.cw * NB + pl[pp]) * 4, s0, s1, s2, 0.f);
     }
     group_arrive(gs);
     group_wait(gs);  // row sums of the cell-state norm
@@ -432,7 +432,7 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
       t1 = segment_sum<HSB>(t1);
       t2 = segment_sum<HSB>(t2);
       if (pc[pp] == 0)
-        store_exchanged4(part_b + ((size_t)blockIdx.x * NB + pl[pp]) * 4, t0, t1, t2, 0.f);
+        store_exchanged4(gs, part_b + ((size_t)role.cw * NB + pl[pp]) * 4, t0, t1, t2, 0.f);
     }
     group_arrive(gs);
     group_wait(gs);  // row sums of the h*R norm
@@ -448,7 +448,7 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
         float* ar = p.act_Rh + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
 #pragma unroll
         for (int g = 0; g < 4; ++g)
-          store_exchanged(ar + (size_t)g * H,
+          store_exchanged(gs, ar + (size_t)g * H,
                           (2.0f * xc2[pp][g] * dsigma * inv4H) + (is2 * gd2[pp][g]) + (dmu * inv4H));
       }
     }
@@ -460,7 +460,7 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc[rt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
     slice_matmul<RT, 1, CHUNK>(p.act_Rh + ((size_t)t * N + n0) * 4 * H, 4 * H, N - n0, K, Kpad,
-                               w_lds, vec_ok, acc);
+                               w_lds, vec_ok, gs.same_xcd, acc);
     store_partials<RT, 1>(red, acc);
     __syncthreads();
 #pragma unroll
@@ -488,13 +488,13 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
     const int a = tid / HSB, jj = tid % HSB;
     float sum = 0.f;
     for (int r = 0; r < NB; ++r) sum += red[(r * NACC + a) * HSB + jj];
-    if (j0 + jj < H) p.col_partial[((size_t)blockIdx.y * NACC + a) * H + j0 + jj] = sum;
+    if (j0 + jj < H) p.col_partial[((size_t)role.bt * NACC + a) * H + j0 + jj] = sum;
   }
-  if (grid_last_arrival(p.cb, gridDim.x * gridDim.y, &s_flag)) {
+  if (grid_last_arrival(p.ls.cb, (unsigned)(p.ls.gx * p.ls.gy), &s_flag)) {
     for (int idx = tid; idx < NACC * H; idx += 256) {
       const int a = idx / H, col = idx % H;
       float sum = 0.f;
-      for (int bt = 0; bt < (int)gridDim.y; ++bt) sum += p.col_partial[((size_t)bt * NACC + a) * H + col];
+      for (int bt = 0; bt < p.ls.gy; ++bt) sum += p.col_partial[((size_t)bt * NACC + a) * H + col];
       if (a < 4) p.db[a * H + col] += sum;
       else if (a < 8) p.dgamma2[(a - 4) * H + col] += sum;
       else if (a == 8) p.dgamma_h[col] += sum;
@@ -528,25 +528,10 @@ int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_siz
   HASTE_HIP_REQUIRE(W && R && b && x && h && c && act_Wx && gamma1 && act_Wx_norm && act_Rh);
   HASTE_HIP_REQUIRE(gamma2 && gamma_h && beta_h && act_c_norm);
   hipStream_t stream = as_stream(stream_);
-  const int cus = device_cu_count();
-
-  struct Cand { int rt, ct; };
-  const Cand cands[] = {{1, 2}, {1, 4}, {1, 1}, {2, 2}, {2, 4}, {2, 1}, {4, 2}, {4, 4}, {4, 1}};
-  const Cand* pick = nullptr;
-  int gx = 0, gy = 0;
-  size_t lds = 0;
-  for (const Cand& cd : cands) {
-    const int HS = 4 * cd.ct, NB = 16 * cd.rt;
-    gx = (H + HS - 1) / HS;
-    gy = (N + NB - 1) / NB;
-    lds = fwd_lds_bytes(H, cd.rt, cd.ct) + (size_t)NB * 2 * sizeof(float);
-    if (gy > kMaxGroups || (long long)gx * gy > cus || gx * gy > kMaxWorkgroups) continue;
-    if (lds > kMaxLdsBytes) continue;
-    pick = &cd;
-    break;
-  }
-  if (pick == nullptr) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
-  const int NB = 16 * pick->rt;
+  const ForwardTile tile = pick_forward_tile(4, N, H, 2 * sizeof(float));
+  if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  const int gx = tile.gx, gy = tile.gy;
+  const int NB = 16 * tile.rt;
   const size_t part_floats = (size_t)gy * gx * NB * 2;
 
   Workspace ws;
@@ -562,13 +547,13 @@ int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_siz
   p.gamma2 = gamma2; p.cache2 = cache2; p.gamma_h = gamma_h; p.beta_h = beta_h; p.cache3 = cache3;
   p.act_c_norm = act_c_norm; p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
   p.part2 = ws.scratch; p.part3 = ws.scratch + part_floats;
-  p.cb = ws.control; p.host_status = ws.host_status_dev; p.spin_limit = kSpinLimit;
-  HASTE_HIP_PROPAGATE(reserve_epochs(stream, 3u * (unsigned)T + 1, &p.epoch));
-  dim3 grid(gx, gy);
+  LaunchPlan plan;
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.lds_bytes, 3u * (unsigned)T + 1, &plan));
+  p.ls = plan.shape;
 #define HASTE_LAUNCH(RT_, CT_)                                                               \
-  if (pick->rt == RT_ && pick->ct == CT_)                                                    \
+  if (tile.rt == RT_ && tile.ct == CT_)                                                      \
     return launch_persistent("layer_norm_lstm_forward_recurrence",                           \
-                             ln_lstm_forward_kernel<RT_, CT_>, grid, lds, p, stream);
+                             ln_lstm_forward_kernel<RT_, CT_>, plan, p, stream);
   HASTE_LAUNCH(1, 1) HASTE_LAUNCH(1, 2) HASTE_LAUNCH(1, 4)
   HASTE_LAUNCH(2, 1) HASTE_LAUNCH(2, 2) HASTE_LAUNCH(2, 4)
   HASTE_LAUNCH(4, 1) HASTE_LAUNCH(4, 2) HASTE_LAUNCH(4, 4)
@@ -601,24 +586,11 @@ int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_
   HASTE_HIP_REQUIRE(act_Wx_norm && act_Rh && gamma2 && dgamma2 && cache2 && gamma_h);
   HASTE_HIP_REQUIRE(dgamma_h && dbeta_h && cache3 && act_c_norm);
   hipStream_t stream = as_stream(stream_);
-  const int cus = device_cu_count();
-  const int gx = (H + 15) / 16;
-  int rt = 0;
-  size_t lds = 0;
-  for (int cand : {1, 2, 4}) {
-    const int gy = (N + 16 * cand - 1) / (16 * cand);
-    const int NB = 16 * cand;
-    const int Kpad = (4 * H + 63) / 64 * 64;
-    lds = ((size_t)Kpad * 16 + (size_t)NB * 10 * 16 + (size_t)NB * 4) * sizeof(float);
-    if (gy <= kMaxGroups && (long long)gx * gy <= cus && gx * gy <= kMaxWorkgroups &&
-        lds <= kMaxLdsBytes) {
-      rt = cand;
-      break;
-    }
-  }
-  if (rt == 0) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  // per row: 10 column-sum accumulators of 16 floats (covers the 4 partial tiles) + 4 sums
+  const BackwardTile tile = pick_backward_tile(4 * H, N, H, 10 * 16 + 4);
+  if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  const int gx = tile.gx, gy = tile.gy, rt = tile.rt;
   const int NB = 16 * rt;
-  const int gy = (N + NB - 1) / NB;
   const size_t part_floats = (size_t)gy * gx * NB * 4;
   const size_t col_floats = (size_t)gy * 10 * H;
 
@@ -635,14 +607,14 @@ int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_
   p.act_c_norm = act_c_norm; p.zoneout_mask = zoneout_mask;
   p.part_a = ws.scratch; p.part_b = ws.scratch + part_floats;
   p.col_partial = ws.scratch + 2 * part_floats;
-  p.cb = ws.control; p.host_status = ws.host_status_dev; p.spin_limit = kSpinLimit;
-  HASTE_HIP_PROPAGATE(reserve_epochs(stream, 3u * (unsigned)T + 1, &p.epoch));
-  dim3 grid(gx, gy);
+  LaunchPlan plan;
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.lds_bytes, 3u * (unsigned)T + 1, &plan));
+  p.ls = plan.shape;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const char* name = "layer_norm_lstm_backward_recurrence";
-  if (rt == 1) rc = launch_persistent(name, ln_lstm_backward_kernel<1>, grid, lds, p, stream);
-  if (rt == 2) rc = launch_persistent(name, ln_lstm_backward_kernel<2>, grid, lds, p, stream);
-  if (rt == 4) rc = launch_persistent(name, ln_lstm_backward_kernel<4>, grid, lds, p, stream);
+  if (rt == 1) rc = launch_persistent(name, ln_lstm_backward_kernel<1>, plan, p, stream);
+  if (rt == 2) rc = launch_persistent(name, ln_lstm_backward_kernel<2>, plan, p, stream);
+  if (rt == 4) rc = launch_persistent(name, ln_lstm_backward_kernel<4>, plan, p, stream);
   HASTE_HIP_PROPAGATE(rc);
 
   // Gradient through the norm of x*W (in place over act_Wx), then the batched products.

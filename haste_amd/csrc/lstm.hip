@@ -21,10 +21,7 @@ struct LstmFwdParams {
   const float* zoneout_mask;   // [T,N,H] or null
   const float* dc_mask;        // DropConnect mask [H,4H] or null
   float dc_scale;
-  ControlBlock* cb;
-  unsigned int* host_status;
-  unsigned int spin_limit;
-  unsigned int epoch;
+  LaunchShape ls;
 };
 
 // HS hidden units per workgroup = 4*CT (their 4 gate columns fill CT MFMA column tiles).
@@ -35,8 +32,11 @@ void lstm_forward_kernel(LstmFwdParams p) {
   constexpr int NB = 16 * RT;
   constexpr int NCOLS = 16 * CT;
   constexpr int PP = (NB * HS + 255) / 256;
-  constexpr int CHUNK = RT == 1 ? 8 : (RT == 2 ? 8 : 4);
+  constexpr int CHUNK = RT == 4 ? 2 : 4;
   extern __shared__ __attribute__((aligned(16))) float lds[];
+  __shared__ unsigned int s_role;
+  const Role role = take_role(p.ls, &s_role);
+  if (!role.active) return;
 
   const int H = p.H, N = p.N, T = p.T;
   const int Kpad = round_up(H, 64);
@@ -44,12 +44,12 @@ void lstm_forward_kernel(LstmFwdParams p) {
   float* red = lds + Kpad * NCOLS;
 
   const int tid = threadIdx.x;
-  const int j0 = blockIdx.x * HS;
-  const int n0 = blockIdx.y * NB;
+  const int j0 = role.cw * HS;
+  const int n0 = role.bt * NB;
   const size_t NH = (size_t)N * H;
 
   GroupSync gs;
-  group_sync_init(gs, p.cb, blockIdx.y, gridDim.x, blockIdx.x, p.epoch, p.host_status, p.spin_limit);
+  group_sync_init(gs, p.ls, role);
 
   // Resident slice: column c of the slice is gate c/HS, hidden unit j0 + c%HS.
   for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
@@ -114,7 +114,7 @@ void lstm_forward_kernel(LstmFwdParams p) {
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
     slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, N - n0, H, Kpad, w_lds,
-                                vec_ok, acc);
+                                vec_ok, gs.same_xcd, acc);
     store_partials<RT, CT>(red, acc);
     __syncthreads();
 
@@ -144,7 +144,7 @@ void lstm_forward_kernel(LstmFwdParams p) {
         }
         const size_t o = (size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp];
         p.c[o] = c_new;
-        store_exchanged(&p.h[o], h_new);
+        store_exchanged(gs, &p.h[o], h_new);
         c_prev[pp] = c_new;
         h_prev[pp] = h_new;
       }
@@ -165,10 +165,7 @@ struct LstmBwdParams {
   float* v;             // [T,N,4H] in: activations, out: gate gradients
   const float* zoneout_mask;
   float* db_partial;    // [batch tiles, 4H] scratch
-  ControlBlock* cb;
-  unsigned int* host_status;
-  unsigned int spin_limit;
-  unsigned int epoch;
+  LaunchShape ls;
 };
 
 // A workgroup owns 16 hidden units (HSB) for 16*RT batch rows; its slice of R_t is
@@ -180,8 +177,11 @@ void lstm_backward_kernel(LstmBwdParams p) {
   constexpr int NB = 16 * RT;
   constexpr int NCOLS = 16;
   constexpr int PP = RT;  // NB*HSB/256
-  constexpr int CHUNK = RT == 1 ? 16 : (RT == 2 ? 8 : 4);
+  constexpr int CHUNK = RT == 1 ? 8 : (RT == 2 ? 4 : 2);
   extern __shared__ __attribute__((aligned(16))) float lds[];
+  __shared__ unsigned int s_role;
+  const Role role = take_role(p.ls, &s_role);
+  if (!role.active) return;
   __shared__ unsigned int s_flag;
 
   const int H = p.H, N = p.N, T = p.T;
@@ -191,12 +191,12 @@ void lstm_backward_kernel(LstmBwdParams p) {
   float* red = lds + Kpad * NCOLS;  // 4*NB*NCOLS floats, also reused for the db reduction
 
   const int tid = threadIdx.x;
-  const int j0 = blockIdx.x * HSB;
-  const int n0 = blockIdx.y * NB;
+  const int j0 = role.cw * HSB;
+  const int n0 = role.bt * NB;
   const size_t NH = (size_t)N * H;
 
   GroupSync gs;
-  group_sync_init(gs, p.cb, blockIdx.y, gridDim.x, blockIdx.x, p.epoch, p.host_status, p.spin_limit);
+  group_sync_init(gs, p.ls, role);
 
   for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
     const int k = idx / NCOLS, cidx = idx % NCOLS;
@@ -275,10 +275,10 @@ void lstm_backward_kernel(LstmBwdParams p) {
         const float dv_f = d_sigmoid_f(gf) * df;
         const float dv_o = d_sigmoid_f(go) * do_;
         float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
-        store_exchanged(vt, dv_i);
-        store_exchanged(vt + H, dv_g);
-        store_exchanged(vt + 2 * H, dv_f);
-        store_exchanged(vt + 3 * H, dv_o);
+        store_exchanged(gs, vt, dv_i);
+        store_exchanged(gs, vt + H, dv_g);
+        store_exchanged(gs, vt + 2 * H, dv_f);
+        store_exchanged(gs, vt + 3 * H, dv_o);
         dbacc[pp][0] += dv_i;
         dbacc[pp][1] += dv_g;
         dbacc[pp][2] += dv_f;
@@ -293,7 +293,7 @@ void lstm_backward_kernel(LstmBwdParams p) {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc[rt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
     slice_matmul<RT, 1, CHUNK>(p.v + ((size_t)t * N + n0) * 4 * H, 4 * H, N - n0, K, Kpad, w_lds,
-                               vec_ok, acc);
+                               vec_ok, gs.same_xcd, acc);
     store_partials<RT, 1>(red, acc);
     __syncthreads();
 #pragma unroll
@@ -322,12 +322,12 @@ void lstm_backward_kernel(LstmBwdParams p) {
     const int g = tid / HSB, jj = tid % HSB;
     float s = 0.f;
     for (int r = 0; r < NB; ++r) s += red[(r * 4 + g) * HSB + jj];
-    if (j0 + jj < H) p.db_partial[(size_t)blockIdx.y * 4 * H + g * H + j0 + jj] = s;
+    if (j0 + jj < H) p.db_partial[(size_t)role.bt * 4 * H + g * H + j0 + jj] = s;
   }
-  if (grid_last_arrival(p.cb, gridDim.x * gridDim.y, &s_flag)) {
+  if (grid_last_arrival(p.ls.cb, (unsigned)(p.ls.gx * p.ls.gy), &s_flag)) {
     for (int col = tid; col < 4 * H; col += 256) {
       float s = 0.f;
-      for (int bt = 0; bt < (int)gridDim.y; ++bt) s += p.db_partial[(size_t)bt * 4 * H + col];
+      for (int bt = 0; bt < p.ls.gy; ++bt) s += p.db_partial[(size_t)bt * 4 * H + col];
       p.db[col] += s;
     }
   }
@@ -355,29 +355,19 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
   p.R = R; p.b = b; p.h = h; p.c = c; p.v = v;
   p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
   p.dc_mask = dc_mask; p.dc_scale = dc_scale;
-  p.cb = ws.control; p.host_status = ws.host_status_dev; p.spin_limit = kSpinLimit;
-  HASTE_HIP_PROPAGATE(reserve_epochs(stream, (unsigned)T + 1, &p.epoch));
-
-  const int cus = device_cu_count();
-  // Candidates in order of preference: fewer rows per workgroup first (more CUs busy).
-  struct Cand { int rt, ct; };
-  const Cand cands[] = {{1, 2}, {1, 4}, {1, 1}, {2, 2}, {2, 4}, {2, 1}, {4, 2}, {4, 4}, {4, 1}};
-  for (const Cand& cd : cands) {
-    const int HS = 4 * cd.ct, NB = 16 * cd.rt;
-    const int gx = (H + HS - 1) / HS, gy = (N + NB - 1) / NB;
-    if (gy > kMaxGroups || (long long)gx * gy > cus || gx * gy > kMaxWorkgroups) continue;
-    const size_t lds = fwd_lds_bytes(H, cd.rt, cd.ct);
-    if (lds > kMaxLdsBytes) continue;
-    dim3 grid(gx, gy);
+  const ForwardTile tile = pick_forward_tile(4, N, H, 0);
+  if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  LaunchPlan plan;
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.lds_bytes, (unsigned)T + 1, &plan));
+  p.ls = plan.shape;
 #define HASTE_LAUNCH_FWD(RT_, CT_)                                                         \
-    if (cd.rt == RT_ && cd.ct == CT_)                                                      \
-      return launch_persistent("lstm_forward_recurrence", lstm_forward_kernel<RT_, CT_>, grid, lds, \
-                               p, stream);
-    HASTE_LAUNCH_FWD(1, 1) HASTE_LAUNCH_FWD(1, 2) HASTE_LAUNCH_FWD(1, 4)
-    HASTE_LAUNCH_FWD(2, 1) HASTE_LAUNCH_FWD(2, 2) HASTE_LAUNCH_FWD(2, 4)
-    HASTE_LAUNCH_FWD(4, 1) HASTE_LAUNCH_FWD(4, 2) HASTE_LAUNCH_FWD(4, 4)
+  if (tile.rt == RT_ && tile.ct == CT_)                                                    \
+    return launch_persistent("lstm_forward_recurrence", lstm_forward_kernel<RT_, CT_>, plan, p, \
+                             stream);
+  HASTE_LAUNCH_FWD(1, 1) HASTE_LAUNCH_FWD(1, 2) HASTE_LAUNCH_FWD(1, 4)
+  HASTE_LAUNCH_FWD(2, 1) HASTE_LAUNCH_FWD(2, 2) HASTE_LAUNCH_FWD(2, 4)
+  HASTE_LAUNCH_FWD(4, 1) HASTE_LAUNCH_FWD(4, 2) HASTE_LAUNCH_FWD(4, 4)
 #undef HASTE_LAUNCH_FWD
-  }
   return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 }
 
@@ -389,21 +379,11 @@ int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
   HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && c && dh_new && dc_new);
   HASTE_HIP_REQUIRE(dx && dW && dR && db && dh && dc && v);
-  const int cus = device_cu_count();
-  const int gx = (H + 15) / 16;
-  int rt = 0;
-  for (int cand : {1, 2, 4}) {
-    const int gy = (N + 16 * cand - 1) / (16 * cand);
-    if (gy <= kMaxGroups && (long long)gx * gy <= cus && bwd_lds_bytes(4 * H, cand) <= kMaxLdsBytes) {
-      rt = cand;
-      break;
-    }
-  }
-  if (rt == 0) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
-  const int gy = (N + 16 * rt - 1) / (16 * rt);
+  const BackwardTile tile = pick_backward_tile(4 * H, N, H, 64);
+  if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 
   Workspace ws;
-  HASTE_HIP_PROPAGATE(get_workspace(stream, (size_t)gy * 4 * H * sizeof(float), &ws));
+  HASTE_HIP_PROPAGATE(get_workspace(stream, (size_t)tile.gy * 4 * H * sizeof(float), &ws));
   HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 
   LstmBwdParams p;
@@ -411,14 +391,14 @@ int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   p.R_t = R_t; p.c = c; p.dh_new = dh_new; p.dc_new = dc_new;
   p.db = db; p.dh = dh; p.dc = dc; p.v = v; p.zoneout_mask = zoneout_mask;
   p.db_partial = ws.scratch;
-  p.cb = ws.control; p.host_status = ws.host_status_dev; p.spin_limit = kSpinLimit;
-  HASTE_HIP_PROPAGATE(reserve_epochs(stream, (unsigned)T + 1, &p.epoch));
-  const size_t lds = bwd_lds_bytes(4 * H, rt);
-  dim3 grid(gx, gy);
+  LaunchPlan plan;
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.lds_bytes, (unsigned)T + 1, &plan));
+  p.ls = plan.shape;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
-  if (rt == 1) rc = launch_persistent("lstm_backward_recurrence", lstm_backward_kernel<1>, grid, lds, p, stream);
-  if (rt == 2) rc = launch_persistent("lstm_backward_recurrence", lstm_backward_kernel<2>, grid, lds, p, stream);
-  if (rt == 4) rc = launch_persistent("lstm_backward_recurrence", lstm_backward_kernel<4>, grid, lds, p, stream);
+  const char* name = "lstm_backward_recurrence";
+  if (tile.rt == 1) rc = launch_persistent(name, lstm_backward_kernel<1>, plan, p, stream);
+  if (tile.rt == 2) rc = launch_persistent(name, lstm_backward_kernel<2>, plan, p, stream);
+  if (tile.rt == 4) rc = launch_persistent(name, lstm_backward_kernel<4>, plan, p, stream);
   HASTE_HIP_PROPAGATE(rc);
 
   // dW += x^T dv ; dR += h[0:T]^T dv ; dx = dv W^T  (dv now lives in v).

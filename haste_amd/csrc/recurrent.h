@@ -25,14 +25,15 @@ __device__ __forceinline__ float d_sigmoid_f(float y) { return y * (1.0f - y); }
 __device__ __forceinline__ float d_tanh_f(float y) { return 1.0f - y * y; }
 
 // ---- Exchange between workgroups inside one launch --------------------------------
-// The 8 XCDs of the chip have separate L2 caches, so data one workgroup writes and
-// another reads in the same launch must not rest in an L2.  Such data is written and
-// read with agent-scope accesses (the sc1 forms of global_store / global_load, which
-// go to the memory side), and everything else uses ordinary cached accesses: no
-// cache-wide write-back or invalidate is needed at a step boundary.
-__device__ __forceinline__ void store_exchanged(float* p, float v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
+// The 8 XCDs of the chip have separate L2 caches.  Data one workgroup writes and
+// another reads in the same launch is always READ with agent-scope loads (the sc1 form
+// of global_load: it never trusts the reader's L1, is served by the L2 when the line
+// was written through that L2, and otherwise comes from the memory side).  How it is
+// WRITTEN depends on where the readers are: when a whole group sits on one XCD an
+// ordinary store is enough (the shared L2 is the meeting point, ~0.25 us one way);
+// when the group spans XCDs the store is agent scope too (written through to the memory
+// side, ~0.4 us one way).  Everything else uses ordinary cached accesses: no cache-wide
+// write-back or invalidate is needed at a step boundary.
 __device__ __forceinline__ float load_exchanged(const float* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -49,6 +50,65 @@ __device__ __forceinline__ float4_t load_exchanged4(const float* p) {
   return v;
 }
 
+// What the host tells a persistent kernel about its launch.
+struct LaunchShape {
+  ControlBlock* cb;
+  unsigned int* host_status;   // pinned host word the kernel reports an abort to
+  unsigned int spin_limit;     // polls before a barrier wait gives up
+  unsigned int epoch;          // step flags of this launch count up from here
+  unsigned int ticket_base;    // per-XCD tickets of this launch count up from here
+  int gx, gy;                  // column workgroups per group, number of groups (batch tiles)
+  int xcd_local;               // 1: group g is the set of workgroups running on XCD g
+  int per_xcd;                 // workgroups this launch places on every XCD (xcd_local)
+};
+
+// The part of the problem a workgroup works on.
+struct Role {
+  int cw;       // column workgroup index inside the group
+  int bt;       // group = batch tile
+  bool active;  // false: nothing to do (surplus workgroup of an XCD-local launch)
+};
+
+__device__ __forceinline__ unsigned int xcc_id() {
+  unsigned int v;
+  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(v));
+  return v & 0xfu;
+}
+
+// Cross-XCD launches use the grid coordinates.  XCD-local launches fill every CU with one
+// workgroup; a workgroup reads which XCD it runs on and draws a ticket there: XCD x hosts
+// batch tile x and the ticket is the column index.  If an XCD turns out to host more
+// workgroups than the launch assumed, the launch is aborted (bounded waits, error status).
+// `word` is a word of LDS.  Called by all threads.
+__device__ __forceinline__ Role take_role(const LaunchShape& ls, unsigned int* word) {
+  Role r;
+  if (!ls.xcd_local) {
+    r.cw = blockIdx.x;
+    r.bt = blockIdx.y;
+    r.active = true;
+    return r;
+  }
+  if (threadIdx.x == 0) {
+    const unsigned int xcc = xcc_id();
+    const unsigned int ticket =
+        __hip_atomic_fetch_add(&ls.cb->xcd_ticket[xcc * kCounterStride], 1u, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT) - ls.ticket_base;
+    if (ticket >= (unsigned int)ls.per_xcd) {
+      __hip_atomic_store(&ls.cb->abort_flag[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(ls.host_status, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      *word = 0xffffffffu;
+    } else {
+      *word = (xcc << 16) | ticket;
+    }
+  }
+  __syncthreads();
+  const unsigned int w = *word;
+  r.bt = (int)(w >> 16);
+  r.cw = (int)(w & 0xffffu);
+  r.active = w != 0xffffffffu && r.bt < ls.gy && r.cw < ls.gx;
+  return r;
+}
+
 // Per-workgroup view of its group's step barrier: one flag word per workgroup holding
 // the number of arrivals it has made (offset by a per-launch epoch so that the words
 // never need clearing).  Arriving is one store; waiting is one wavefront reading the
@@ -62,20 +122,24 @@ struct GroupSync {
   unsigned int epoch;          // value of the flags after `arrivals` arrivals is epoch + arrivals
   unsigned int arrivals;
   unsigned int spin_limit;
+  bool same_xcd;               // every workgroup of the group shares one L2
 };
 
-__device__ __forceinline__ void group_sync_init(GroupSync& g, ControlBlock* cb, unsigned int group,
-                                                unsigned int group_size, unsigned int my_index,
-                                                unsigned int epoch, unsigned int* host_status,
-                                                unsigned int spin_limit) {
-  g.flags = &cb->step_flags[group * group_size];
-  g.abort_flag = &cb->abort_flag[0];
-  g.host_status = host_status;
-  g.group_size = group_size;
-  g.my_index = my_index;
-  g.epoch = epoch;
+__device__ __forceinline__ void group_sync_init(GroupSync& g, const LaunchShape& ls, const Role& r) {
+  g.flags = &ls.cb->step_flags[r.bt * ls.gx];
+  g.abort_flag = &ls.cb->abort_flag[0];
+  g.host_status = ls.host_status;
+  g.group_size = (unsigned int)ls.gx;
+  g.my_index = (unsigned int)r.cw;
+  g.epoch = ls.epoch;
   g.arrivals = 0;
-  g.spin_limit = spin_limit;
+  g.spin_limit = ls.spin_limit;
+  g.same_xcd = ls.xcd_local != 0;
+}
+
+__device__ __forceinline__ void store_exchanged(const GroupSync& g, float* p, float v) {
+  if (g.same_xcd) *p = v;
+  else __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Counts the workgroup as arrived once every exchanged store its threads have issued
@@ -84,9 +148,13 @@ __device__ __forceinline__ void group_arrive(GroupSync& g) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   g.arrivals += 1;
-  if (threadIdx.x == 0)
-    __hip_atomic_store(&g.flags[g.my_index], g.epoch + g.arrivals, __ATOMIC_RELAXED,
-                       __HIP_MEMORY_SCOPE_AGENT);
+  if (threadIdx.x == 0) {
+    if (g.same_xcd)
+      *reinterpret_cast<volatile unsigned int*>(&g.flags[g.my_index]) = g.epoch + g.arrivals;
+    else
+      __hip_atomic_store(&g.flags[g.my_index], g.epoch + g.arrivals, __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+  }
 }
 
 // Blocks until every workgroup of the group has made as many arrivals as this one.
@@ -118,6 +186,9 @@ __device__ __forceinline__ void group_wait(GroupSync& g) {
     }
   }
   __syncthreads();
+  // Same-XCD groups read the exchanged data with ordinary loads: drop what this CU's L1
+  // may still hold of those lines (the shared L2 has the new values).
+  if (g.same_xcd) asm volatile("buffer_inv sc0" ::: "memory");
 }
 
 // True in exactly one workgroup of the launch: the last to call it.  Stores made by
@@ -165,56 +236,152 @@ __device__ __forceinline__ float4_t load_a4(const float* p, int valid, bool vec_
   return v;
 }
 
+// Loads the A operands of k-groups [g, g+CHUNK) of this wavefront's quarter (see
+// slice_matmul).  Branch-free on the vector paths: out-of-range elements read element 0
+// of the tile and are zeroed afterwards.
+template <int RT, int CHUNK>
+__device__ __forceinline__ void load_a_chunk(const float* __restrict__ a, int a_ld, int rows_valid,
+                                             int K, int g_abs, int g_end, bool vec_ok, bool cached,
+                                             float4_t (&av)[CHUNK][RT]) {
+  const int lane = threadIdx.x & 63;
+  const int row = lane & 15;
+  const int kq = lane >> 4;
+  const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+  if (vec_ok && cached) {
+#pragma unroll
+    for (int gi = 0; gi < CHUNK; ++gi) {
+      const int k = (g_abs + gi) * 16 + kq * 4;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const int rr = rt * 16 + row;
+        const bool ok = g_abs + gi < g_end && rr < rows_valid && k < K;
+        const float* src = a + (ok ? (size_t)rr * a_ld + k : (size_t)0);
+        const float4_t v = *reinterpret_cast<const float4_t*>(src);
+        av[gi][rt] = ok ? v : zero4;
+      }
+    }
+  } else if (vec_ok) {
+#pragma unroll
+    for (int gi = 0; gi < CHUNK; ++gi) {
+      const int k = (g_abs + gi) * 16 + kq * 4;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const int rr = rt * 16 + row;
+        const bool ok = g_abs + gi < g_end && rr < rows_valid && k < K;
+        const float* src = a + (ok ? (size_t)rr * a_ld + k : (size_t)0);
+        const float4_t v = load_exchanged4(src);
+        av[gi][rt] = ok ? v : zero4;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int gi = 0; gi < CHUNK; ++gi) {
+      const int k = (g_abs + gi) * 16 + kq * 4;
+      const bool live = g_abs + gi < g_end;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const int rr = rt * 16 + row;
+        const int valid = (live && rr < rows_valid) ? (K - k) : 0;
+        av[gi][rt] = load_a4(a + (size_t)rr * a_ld + k, valid, false);
+      }
+    }
+  }
+}
+
+// MFMAs of k-groups [g_abs, g_abs+CHUNK): one straight-line block (no branches, so the
+// accumulators stay in the matrix unit's registers and the scheduler can hoist the LDS
+// reads of the slice columns ahead of the MFMAs that use them).  Consecutive MFMAs go to
+// different accumulators (two per output tile, alternating by k-group) so that none
+// waits for the result of the one before it.
+template <int RT, int CT, int CHUNK>
+__device__ __forceinline__ void mfma_chunk(const float* w_lds, int g_abs,
+                                           const float4_t (&av)[CHUNK][RT],
+                                           float4_t (&acc0)[RT][CT], float4_t (&acc1)[RT][CT]) {
+  constexpr int NCOLS = 16 * CT;
+  const int lane = threadIdx.x & 63;
+  const int row = lane & 15;
+  const int kq = lane >> 4;
+  const float* wp0 = w_lds + ((g_abs * 4 + kq) * NCOLS + row) * 4;
+#pragma unroll
+  for (int gi = 0; gi < CHUNK; ++gi) {
+    float4_t b[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+      b[ct] = *reinterpret_cast<const float4_t*>(wp0 + gi * 4 * NCOLS * 4 + ct * 64);
+    float4_t (&acc)[RT][CT] = (gi & 1) ? acc1 : acc0;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+        acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].x, b[ct].x, acc[rt][ct], 0, 0, 0);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+        acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].y, b[ct].y, acc[rt][ct], 0, 0, 0);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+        acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].z, b[ct].z, acc[rt][ct], 0, 0, 0);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+        acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].w, b[ct].w, acc[rt][ct], 0, 0, 0);
+  }
+}
+
 // acc[rt][ct] += A[16*RT rows, K] * slice[K, 16*CT] for this wavefront's quarter of K.
 // `a` points at row 0 of the batch tile (row stride a_ld floats, K contiguous);
 // rows >= rows_valid and k >= K read as zero.  The four wavefronts of the workgroup
 // each take Kpad/4 consecutive k; the caller adds their accumulators.
 // Accumulator element r of acc[rt][ct] in lane l is row 16*rt + 4*(l/16) + r,
 // column 16*ct + l%16.
+// `cached`: the tile may be read with ordinary loads (same-XCD group, L1 invalidated
+// after the barrier); otherwise agent-scope loads are used.  `vec_ok`: rows are 16-byte
+// aligned and K is a multiple of 4.
+// K is walked in chunks of CHUNK k-groups; the loads of the next chunk are issued before
+// the MFMAs of the current one, so they are in flight while the matrix unit works.  The
+// k-groups left over when the count is not a multiple of CHUNK are done one at a time.
 template <int RT, int CT, int CHUNK>
 __device__ __forceinline__ void slice_matmul(const float* __restrict__ a, int a_ld, int rows_valid,
                                              int K, int Kpad, const float* w_lds, bool vec_ok,
-                                             float4_t (&acc)[RT][CT]) {
-  constexpr int NCOLS = 16 * CT;
-  const int lane = threadIdx.x & 63;
+                                             bool cached, float4_t (&acc)[RT][CT]) {
   const int wave = threadIdx.x >> 6;
-  const int row = lane & 15;
-  const int kq = lane >> 4;
   const int groups = Kpad >> 6;  // k-groups of 16 per wavefront
-  const int g_first = wave * groups;
+  const int full = groups / CHUNK;
+  int g = wave * groups;
+  const int g_end = g + groups;
+  float4_t acc1[RT][CT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) acc1[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-  for (int g0 = 0; g0 < groups; g0 += CHUNK) {
-    float4_t av[CHUNK][RT];
+  if (full > 0) {
+    float4_t cur[CHUNK][RT], nxt[CHUNK][RT];
+    load_a_chunk<RT, CHUNK>(a, a_ld, rows_valid, K, g, g_end, vec_ok, cached, cur);
+    for (int c = 0; c < full; ++c) {
+      if (c + 1 < full)
+        load_a_chunk<RT, CHUNK>(a, a_ld, rows_valid, K, g + CHUNK, g_end, vec_ok, cached, nxt);
+      mfma_chunk<RT, CT, CHUNK>(w_lds, g, cur, acc, acc1);
 #pragma unroll
-    for (int gi = 0; gi < CHUNK; ++gi) {
-      const int k = (g_first + g0 + gi) * 16 + kq * 4;
-      const bool live = g0 + gi < groups;
+      for (int gi = 0; gi < CHUNK; ++gi)
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        const int rr = rt * 16 + row;
-        const int valid = (live && rr < rows_valid) ? (K - k) : 0;
-        av[gi][rt] = load_a4(a + (size_t)rr * a_ld + k, valid, vec_ok);
-      }
-    }
-#pragma unroll
-    for (int gi = 0; gi < CHUNK; ++gi) {
-      if (g0 + gi < groups) {
-        const int kg = g_first + g0 + gi;
-        const float* wp = w_lds + ((kg * 4 + kq) * NCOLS + row) * 4;
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-          const float4_t b = *reinterpret_cast<const float4_t*>(wp + ct * 64);
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt) {
-            acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].x, b.x, acc[rt][ct], 0, 0, 0);
-            acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].y, b.y, acc[rt][ct], 0, 0, 0);
-            acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].z, b.z, acc[rt][ct], 0, 0, 0);
-            acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].w, b.w, acc[rt][ct], 0, 0, 0);
-          }
-        }
-      }
+        for (int rt = 0; rt < RT; ++rt) cur[gi][rt] = nxt[gi][rt];
+      g += CHUNK;
     }
   }
+  for (; g < g_end; ++g) {
+    float4_t one[1][RT];
+    load_a_chunk<RT, 1>(a, a_ld, rows_valid, K, g, g_end, vec_ok, cached, one);
+    mfma_chunk<RT, CT, 1>(w_lds, g, one, acc, acc1);
+  }
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) acc[rt][ct] += acc1[rt][ct];
 }
 
 // Writes this wavefront's accumulators to red[wave][16*RT][16*CT] in LDS.
@@ -260,23 +427,131 @@ inline size_t bwd_lds_bytes(int K, int RT) {
   return ((size_t)Kpad * 16 + red) * sizeof(float);
 }
 
+// Host-side plan of a persistent launch: fills `shape` and the grid for (gx, gy).
+// An XCD-local launch is used when every group fits on one XCD (gx <= CUs per XCD,
+// gy <= XCDs); it fills the chip with one workgroup per CU (the LDS request is raised so
+// that two cannot share a CU) and lets the kernel sort the workgroups by XCD.
+struct LaunchPlan {
+  dim3 grid;
+  size_t lds_bytes;
+  LaunchShape shape;
+};
+
+constexpr int kXcdCount = 8;
+
+inline bool xcd_local_fits(int gx, int gy) {
+  const int cus = device_cu_count();
+  return xcd_local_enabled() && cus % kXcdCount == 0 && gy <= kXcdCount && gx <= cus / kXcdCount;
+}
+
+inline int plan_launch(hipStream_t stream, const Workspace& ws, int gx, int gy, size_t lds_bytes,
+                       unsigned int epochs, LaunchPlan* plan) {
+  plan->shape.cb = ws.control;
+  plan->shape.host_status = ws.host_status_dev;
+  plan->shape.spin_limit = kSpinLimit;
+  plan->shape.gx = gx;
+  plan->shape.gy = gy;
+  plan->shape.ticket_base = 0;
+  plan->shape.per_xcd = 0;
+  HASTE_HIP_PROPAGATE(reserve_epochs(stream, epochs, &plan->shape.epoch));
+  if (xcd_local_fits(gx, gy)) {
+    const int cus = device_cu_count();
+    plan->shape.xcd_local = 1;
+    plan->shape.per_xcd = cus / kXcdCount;
+    HASTE_HIP_PROPAGATE(reserve_tickets(stream, (unsigned)plan->shape.per_xcd, &plan->shape.ticket_base));
+    plan->grid = dim3((unsigned)cus);
+    const size_t one_per_cu = 84 * 1024;  // more than half of a CU's LDS
+    plan->lds_bytes = lds_bytes > one_per_cu ? lds_bytes : one_per_cu;
+  } else {
+    plan->shape.xcd_local = 0;
+    plan->grid = dim3((unsigned)gx, (unsigned)gy);
+    plan->lds_bytes = lds_bytes;
+  }
+  return HASTE_HIP_OK;
+}
+
 template <typename KernelT, typename ParamsT>
-int launch_persistent(const char* name, KernelT kernel, dim3 grid, size_t lds_bytes, ParamsT& params,
+int launch_persistent(const char* name, KernelT kernel, const LaunchPlan& plan, ParamsT& params,
                       hipStream_t stream) {
   HASTE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)plan.lds_bytes));
   int per_cu = 0;
-  HASTE_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, lds_bytes));
+  HASTE_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, plan.lds_bytes));
   const long long capacity = (long long)per_cu * device_cu_count();
-  if ((long long)grid.x * grid.y > capacity) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  if ((long long)plan.grid.x * plan.grid.y > capacity) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   void* args[] = {&params};
   ScopedKernelTimer timer(name, stream);
-  HASTE_HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<const void*>(kernel), grid, dim3(256),
-                                           args, (unsigned int)lds_bytes, stream));
+  HASTE_HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<const void*>(kernel), plan.grid,
+                                           dim3(256), args, (unsigned int)plan.lds_bytes, stream));
   return HASTE_HIP_OK;
 }
 
 constexpr size_t kMaxLdsBytes = 160 * 1024;  // LDS per workgroup on gfx950
+
+// Geometry of a forward recurrence: 16*rt batch rows and hs hidden units per workgroup
+// (their gate columns fill ct MFMA column tiles), gx column workgroups, gy batch tiles.
+struct ForwardTile {
+  int rt, ct, hs, gx, gy;
+  size_t lds_bytes;
+  bool ok;
+};
+
+// Prefers a geometry whose groups each fit on one XCD (most workgroups first), else the
+// cross-XCD geometry with the most parallelism that fits the chip.  `extra_lds_per_row` is
+// what the cell needs in LDS per batch row beyond the slice and the partial tiles.
+inline ForwardTile pick_forward_tile(int gates, int N, int H, size_t extra_lds_per_row) {
+  const int cus = device_cu_count();
+  ForwardTile best;
+  best.ok = false;
+  for (int pass = 0; pass < 2 && !best.ok; ++pass) {
+    const int hs_order_local[] = {4, 8, 16};
+    const int hs_order_cross[] = {8, 16, 4};
+    for (int rt : {1, 2, 4}) {
+      for (int i = 0; i < 3 && !best.ok; ++i) {
+        const int hs = pass == 0 ? hs_order_local[i] : hs_order_cross[i];
+        const int ct = (gates * hs + 15) / 16;
+        const int NB = 16 * rt;
+        const int gx = (H + hs - 1) / hs, gy = (N + NB - 1) / NB;
+        const size_t lds = fwd_lds_bytes(H, rt, ct) + extra_lds_per_row * NB;
+        if (lds > kMaxLdsBytes || gy > kMaxGroups || gx * gy > kMaxWorkgroups) continue;
+        if (pass == 0 ? !xcd_local_fits(gx, gy) : (long long)gx * gy > cus) continue;
+        best = ForwardTile{rt, ct, hs, gx, gy, lds, true};
+      }
+      if (best.ok) break;
+    }
+  }
+  return best;
+}
+
+// Geometry of a backward recurrence: 16 hidden units and 16*rt batch rows per workgroup.
+struct BackwardTile {
+  int rt, gx, gy;
+  size_t lds_bytes;
+  bool ok;
+};
+
+// K = gates*H is the contraction length; `extra_floats_per_row` is the LDS the cell needs
+// per batch row beyond the slice (at least the 4 partial tiles = 64 floats).
+inline BackwardTile pick_backward_tile(int K, int N, int H, size_t extra_floats_per_row) {
+  const int cus = device_cu_count();
+  const int gx = (H + 15) / 16;
+  const int Kpad = (K + 63) / 64 * 64;
+  BackwardTile best;
+  best.ok = false;
+  for (int pass = 0; pass < 2 && !best.ok; ++pass) {
+    for (int rt : {1, 2, 4}) {
+      const int NB = 16 * rt;
+      const int gy = (N + NB - 1) / NB;
+      const size_t lds = ((size_t)Kpad * 16 + extra_floats_per_row * NB) * sizeof(float);
+      if (lds > kMaxLdsBytes || gy > kMaxGroups || gx * gy > kMaxWorkgroups) continue;
+      if (pass == 0 ? !xcd_local_fits(gx, gy) : (long long)gx * gy > cus) continue;
+      best = BackwardTile{rt, gx, gy, lds, true};
+      break;
+    }
+  }
+  return best;
+}
 
 
 }  // namespace haste_hip

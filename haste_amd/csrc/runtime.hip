@@ -2,6 +2,7 @@
 #include "common.h"
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -69,6 +70,14 @@ void set_runtime_error(hipError_t err, const char* what) {
   (void)hipGetLastError();  // do not leave the error for an unrelated later call
 }
 
+bool xcd_local_enabled() {
+  static const bool enabled = [] {
+    const char* v = std::getenv("HASTE_HIP_XCD_LOCAL");
+    return v == nullptr || v[0] != '0';
+  }();
+  return enabled;
+}
+
 int device_cu_count() {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
@@ -127,10 +136,32 @@ int reserve_epochs(hipStream_t stream, unsigned int count, unsigned int* base) {
   return HASTE_HIP_OK;
 }
 
+int reserve_tickets(hipStream_t stream, unsigned int count, unsigned int* base) {
+  int dev = 0;
+  HASTE_HIP_TRY(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_mutex);
+  auto it = g_workspaces.find(Key{dev, stream});
+  if (it == g_workspaces.end()) return HASTE_HIP_ERROR_INVALID_ARGUMENT;
+  *base = it->second.ticket_base;
+  it->second.ticket_base += count;
+  return HASTE_HIP_OK;
+}
+
 int check_and_clear_abort(hipStream_t stream, Workspace* ws) {
   volatile unsigned int* status = ws->host_status;
   if (status == nullptr || *status == 0u) return HASTE_HIP_OK;
   *status = 0u;
+  {
+    // the control block is wiped below, so flag and ticket numbering restart from zero
+    int dev = 0;
+    HASTE_HIP_TRY(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(g_mutex);
+    auto it = g_workspaces.find(Key{dev, stream});
+    if (it != g_workspaces.end()) {
+      it->second.epoch = 0;
+      it->second.ticket_base = 0;
+    }
+  }
   const size_t words = sizeof(ControlBlock) / sizeof(unsigned int);
   fill_zero_kernel<<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream>>>(
       reinterpret_cast<unsigned int*>(ws->control), words);
