@@ -9,10 +9,10 @@
 // double-buffered LDS stage.  Both operand tiles sit in LDS k-major, so a wavefront
 // reads the 32 consecutive floats of one k for each half of its lanes, which is the
 // operand layout of the 32x32x2 instruction and is bank-conflict free.  Small
-// outputs with a long K (dW, dR: K = T*N) are split along K over several workgroups;
-// the last workgroup to arrive at a tile adds the partial sums in a fixed order, so
-// results do not depend on arrival order.  Workgroup ids are remapped so that each
-// XCD (one L2) works on a contiguous run of tiles.
+// outputs with a long K (dW, dR: K = T*N) are split along K over several workgroups
+// that park partial tiles; a second, bandwidth-bound kernel adds the splits in index
+// order, so results do not depend on scheduling.  Workgroup ids are remapped so that
+// each XCD (one L2) works on a contiguous run of tiles.
 #include "common.h"
 
 namespace haste_hip {
@@ -21,13 +21,9 @@ namespace {
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 128;
 constexpr int BN = 128;
 constexpr int BK = 16;
-constexpr int LDA_ROWMAJOR = BM + 2;  // A tile written with transposing scalar stores
-constexpr int LDA_KMAJOR = BM + 4;    // A tile written with 16-byte stores
 constexpr int LDB = BN + 4;
-constexpr int A_STAGE = BK * (BM + 4);
 constexpr int B_STAGE = BK * LDB;
 constexpr int kXcds = 8;
 
@@ -44,7 +40,9 @@ __device__ __forceinline__ float4_t load4_guarded(const float* p, int valid, boo
   return v;
 }
 
-template <bool TRANS_A>
+// BM x 128 output tile; BM = 128 (each wavefront a 64x64 quadrant) or 64 (each a 32x64
+// quadrant) for outputs too small to fill the chip with 128-row tiles.
+template <bool TRANS_A, int BM>
 __global__ __launch_bounds__(256, 2)
 void gemm_f32_kernel(int M, int N, int K,
                      const float* __restrict__ A, int lda,
@@ -52,12 +50,16 @@ void gemm_f32_kernel(int M, int N, int K,
                      float* __restrict__ C, int ldc, int accumulate,
                      int tiles_n, int total_blocks, int splits, int k_per_split,
                      int a_vec_ok, int b_vec_ok,
-                     float* __restrict__ partial, unsigned int* tile_counter) {
+                     float* __restrict__ partial) {
+  // A tile k-major in LDS: leading dimension BM+2 when it is written with transposing
+  // scalar stores (bank-conflict free), BM+4 when written with 16-byte stores.
+  constexpr int LDA = TRANS_A ? BM + 4 : BM + 2;
+  constexpr int A_STAGE = BK * (BM + 4);
+  constexpr int MI = BM / 64;       // 32x32 MFMA tiles per wavefront along M
+  constexpr int A_PASSES = BM / 64; // passes of 256 threads to load the A tile
   __shared__ __attribute__((aligned(16))) float smem[2 * A_STAGE + 2 * B_STAGE];
-  __shared__ unsigned int s_arrival;
   float* As = smem;
   float* Bs = smem + 2 * A_STAGE;
-  constexpr int LDA = TRANS_A ? LDA_KMAJOR : LDA_ROWMAJOR;
 
   // Workgroup ids are handed to the XCDs round-robin; give XCD x the x-th contiguous
   // chunk of the tile list so that neighbours in the list share an L2.
@@ -75,25 +77,28 @@ void gemm_f32_kernel(int M, int N, int K,
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm = (wave >> 1) * 64;
+  const int wm = (wave >> 1) * (32 * MI);
   const int wn = (wave & 1) * 64;
 
-  float16_t acc[2][2];
+  float16_t acc[MI][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  float4_t a_reg[2], b_reg[2];
+  float4_t a_reg[A_PASSES], b_reg[2];
+  // A tile stored [K][M] in memory: one pass covers (256*4/BM) k-rows of BM columns.
+  constexpr int TA_ROWS = 1024 / BM;
+  constexpr int TA_COLS = BM / 4;
 
   auto load_global = [&](int kk) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < A_PASSES; ++i) {
       if (TRANS_A) {
-        const int ak = (tid >> 5) + 8 * i;
-        const int am = (tid & 31) * 4;
+        const int ak = (tid / TA_COLS) + TA_ROWS * i;
+        const int am = (tid % TA_COLS) * 4;
         const int k = kk + ak, m = m0 + am;
         const int valid = (k < k_end) ? (M - m) : 0;
         a_reg[i] = load4_guarded(A + (size_t)k * lda + m, valid, a_vec_ok);
@@ -104,6 +109,9 @@ void gemm_f32_kernel(int M, int N, int K,
         const int valid = (m < M) ? (k_end - k) : 0;
         a_reg[i] = load4_guarded(A + (size_t)m * lda + k, valid, a_vec_ok);
       }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
       const int bk = (tid >> 5) + 8 * i;
       const int bn = (tid & 31) * 4;
       const int k = kk + bk, n = n0 + bn;
@@ -116,10 +124,10 @@ void gemm_f32_kernel(int M, int N, int K,
     float* as = As + buf * A_STAGE;
     float* bs = Bs + buf * B_STAGE;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < A_PASSES; ++i) {
       if (TRANS_A) {
-        const int ak = (tid >> 5) + 8 * i;
-        const int am = (tid & 31) * 4;
+        const int ak = (tid / TA_COLS) + TA_ROWS * i;
+        const int am = (tid % TA_COLS) * 4;
         *reinterpret_cast<float4_t*>(as + ak * LDA + am) = a_reg[i];
       } else {
         const int arow = (tid >> 2) + 64 * i;
@@ -129,6 +137,9 @@ void gemm_f32_kernel(int M, int N, int K,
         as[(ak + 2) * LDA + arow] = a_reg[i].z;
         as[(ak + 3) * LDA + arow] = a_reg[i].w;
       }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
       const int bk = (tid >> 5) + 8 * i;
       const int bn = (tid & 31) * 4;
       *reinterpret_cast<float4_t*>(bs + bk * LDB + bn) = b_reg[i];
@@ -140,14 +151,14 @@ void gemm_f32_kernel(int M, int N, int K,
     const float* bs = Bs + buf * B_STAGE + (lane >> 5) * LDB + wn + (lane & 31);
 #pragma unroll
     for (int k2 = 0; k2 < BK; k2 += 2) {
-      const float a0 = as[k2 * LDA];
-      const float a1 = as[k2 * LDA + 32];
       const float b0 = bs[k2 * LDB];
       const float b1 = bs[k2 * LDB + 32];
-      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < MI; ++i) {
+        const float av = as[k2 * LDA + 32 * i];
+        acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b0, acc[i][0], 0, 0, 0);
+        acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b1, acc[i][1], 0, 0, 0);
+      }
     }
   };
 
@@ -172,7 +183,7 @@ void gemm_f32_kernel(int M, int N, int K,
   const int row_in = (lane >> 5) * 4;
   if (splits == 1) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int col = n0 + wn + 32 * j + col_in;
@@ -188,39 +199,46 @@ void gemm_f32_kernel(int M, int N, int K,
     return;
   }
 
-  // Split-K: park the partial tile, then the last arrival folds all partials of the
-  // tile into C in split order.
-  const size_t tile_elems = (size_t)BM * BN;
-  float* part_tile = partial + ((size_t)tile * splits + split) * tile_elems;
+  // Split-K: park the partial tile in [split][M][N] layout; a second, bandwidth-bound
+  // kernel adds the splits in order (the kernel boundary makes the partials visible, so
+  // no cache-wide fence is needed here).
+  float* part = partial + (size_t)split * M * N;
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int c = wn + 32 * j + col_in;
+      const int col = n0 + wn + 32 * j + col_in;
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const int rr = wm + 32 * i + 8 * (e >> 2) + row_in + (e & 3);
-        part_tile[rr * BN + c] = acc[i][j][e];
+        const int row = m0 + wm + 32 * i + 8 * (e >> 2) + row_in + (e & 3);
+        if (row < M && col < N) part[(size_t)row * N + col] = acc[i][j][e];
       }
     }
-  __threadfence();
-  __syncthreads();
-  if (tid == 0) s_arrival = atomicAdd(&tile_counter[tile], 1u);
-  __syncthreads();
-  if (s_arrival != (unsigned)(splits - 1)) return;
-  __threadfence();
-  const float* base = partial + (size_t)tile * splits * tile_elems;
-  for (int idx = tid; idx < BM * BN; idx += 256) {
-    const int rr = idx / BN, c = idx % BN;
-    const int row = m0 + rr, col = n0 + c;
-    if (row < M && col < N) {
-      float s = 0.f;
-      for (int sp = 0; sp < splits; ++sp) s += base[(size_t)sp * tile_elems + idx];
-      float* p = C + (size_t)row * ldc + col;
+}
+
+// C (+)= sum over splits of partial[split][M][N], splits added in index order.
+__global__ __launch_bounds__(256)
+void splitk_reduce_kernel(int M, int N, int splits, const float* __restrict__ partial,
+                          float* __restrict__ C, int ldc, int accumulate, int vec_ok) {
+  const size_t MN = (size_t)M * N;
+  const size_t stride = (size_t)gridDim.x * 256;
+  if (vec_ok) {
+    for (size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4; i < MN; i += stride * 4) {
+      float4_t s = *reinterpret_cast<const float4_t*>(partial + i);
+      for (int sp = 1; sp < splits; ++sp) s += *reinterpret_cast<const float4_t*>(partial + sp * MN + i);
+      const size_t row = i / N, col = i % N;
+      float4_t* p = reinterpret_cast<float4_t*>(C + row * ldc + col);
+      *p = accumulate ? (*p + s) : s;
+    }
+  } else {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < MN; i += stride) {
+      float s = partial[i];
+      for (int sp = 1; sp < splits; ++sp) s += partial[sp * MN + i];
+      const size_t row = i / N, col = i % N;
+      float* p = C + row * ldc + col;
       *p = accumulate ? (*p + s) : s;
     }
   }
-  if (tid == 0) tile_counter[tile] = 0u;
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -233,47 +251,56 @@ int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
   HASTE_HIP_REQUIRE(M > 0 && N > 0 && K > 0);
   HASTE_HIP_REQUIRE(A != nullptr && B != nullptr && C != nullptr);
   HASTE_HIP_REQUIRE(lda >= (trans_a ? M : K) && ldb >= N && ldc >= N);
-  const int tiles_m = (M + BM - 1) / BM;
   const int tiles_n = (N + BN - 1) / BN;
-  const long long tiles = (long long)tiles_m * tiles_n;
-  HASTE_HIP_REQUIRE(tiles < (1ll << 30));
-  const int cus = device_cu_count();
+  const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
 
-  // Split K when the output alone cannot occupy the chip and K is long.
+  // Tile height: 64 rows only when the output has no more than that.  K splits: when the
+  // output tiles alone leave CUs without two workgroups each, K is cut into the smallest
+  // power-of-two number of pieces that does, as long as a piece keeps at least 256 of K
+  // (measured on the backward shapes: dW/dR 51 -> 91-99 TFLOP/s, dx 73 -> 82 TFLOP/s).
+  // The choice depends on the shape only, so results are reproducible.
+  const int bm = M <= 64 ? 64 : 128;
   int splits = 1;
-  if (cus > 0 && tiles * 2 <= cus && K >= 1024 && tiles <= 4096) {
-    splits = (int)((cus + tiles - 1) / tiles);
-    const int max_by_k = K / 256;
-    if (splits > max_by_k) splits = max_by_k;
-    if (splits > 32) splits = 32;
-    if (splits < 1) splits = 1;
+  {
+    const long long t = (long long)((M + bm - 1) / bm) * tiles_n;
+    while (t * splits < 2LL * cus && K / (splits * 2) >= 256 && splits < 32) splits *= 2;
   }
+  const int tiles_m = (M + bm - 1) / bm;
+  const long long tiles = (long long)tiles_m * tiles_n;
+  HASTE_HIP_REQUIRE(tiles < (1ll << 28));
   int k_per_split = (K + splits - 1) / splits;
   k_per_split = (k_per_split + BK - 1) / BK * BK;
   splits = (K + k_per_split - 1) / k_per_split;
 
   Workspace ws;
   float* partial = nullptr;
-  unsigned int* tile_counter = nullptr;
   if (splits > 1) {
-    const size_t bytes = (size_t)tiles * splits * BM * BN * sizeof(float);
+    const size_t bytes = (size_t)splits * M * N * sizeof(float);
     HASTE_HIP_PROPAGATE(get_workspace(stream, bytes, &ws));
     partial = ws.scratch;
-    tile_counter = ws.control->tile_counter;
   }
   const int a_vec_ok = aligned16(A) && (lda % 4 == 0) && (k_per_split % 4 == 0);
   const int b_vec_ok = aligned16(B) && (ldb % 4 == 0);
   const int total = (int)(tiles * splits);
   dim3 grid((unsigned)total), block(256);
   ScopedKernelTimer timer("gemm_f32", stream);
-  if (trans_a) {
-    gemm_f32_kernel<true><<<grid, block, 0, stream>>>(
-        M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, tiles_n, total, splits,
-        k_per_split, a_vec_ok, b_vec_ok, partial, tile_counter);
-  } else {
-    gemm_f32_kernel<false><<<grid, block, 0, stream>>>(
-        M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, tiles_n, total, splits,
-        k_per_split, a_vec_ok, b_vec_ok, partial, tile_counter);
+#define HASTE_GEMM_LAUNCH(TA_, BM_)                                                          \
+  if (trans_a == TA_ && bm == BM_)                                                           \
+    gemm_f32_kernel<TA_, BM_><<<grid, block, 0, stream>>>(                                   \
+        M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, tiles_n, total, splits,         \
+        k_per_split, a_vec_ok, b_vec_ok, partial);
+  HASTE_GEMM_LAUNCH(false, 128) HASTE_GEMM_LAUNCH(false, 64)
+  HASTE_GEMM_LAUNCH(true, 128) HASTE_GEMM_LAUNCH(true, 64)
+#undef HASTE_GEMM_LAUNCH
+  HASTE_HIP_TRY(hipGetLastError());
+  if (splits > 1) {
+    const size_t MN = (size_t)M * N;
+    const int vec = (N % 4 == 0) && (ldc % 4 == 0) && aligned16(C) && aligned16(partial);
+    size_t blocks = (MN / (vec ? 4 : 1) + 255) / 256;
+    if (blocks > (size_t)cus * 8) blocks = (size_t)cus * 8;
+    if (blocks < 1) blocks = 1;
+    splitk_reduce_kernel<<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
+        M, N, splits, partial, C, ldc, accumulate ? 1 : 0, vec);
   }
   HASTE_HIP_TRY(hipGetLastError());
   return HASTE_HIP_OK;
