@@ -80,6 +80,12 @@ int check_and_clear_abort(hipStream_t stream, Workspace* ws);
 
 int device_cu_count();
 
+// Keeps the persistent kernels of this process on one device in a single order even when
+// they are launched on different streams.  before == true: makes `stream` wait for the
+// previous persistent kernel (if it ran on another stream); before == false: records the
+// kernel just enqueued on `stream` as the one to wait for.
+int order_persistent_launches(hipStream_t stream, bool before);
+
 // False when the environment variable HASTE_HIP_XCD_LOCAL is set to 0 (forces the
 // cross-XCD exchange path; for experiments).
 bool xcd_local_enabled();

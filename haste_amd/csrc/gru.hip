@@ -47,7 +47,8 @@ void gru_forward_kernel(GruFwdParams p) {
 
   const int tid = threadIdx.x;
   const int j0 = role.cw * HS;
-  const int n0 = role.bt * NB;
+  const int n0 = role.bt * p.ls.tile_rows;
+  const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
 
   GroupSync gs;
@@ -75,7 +76,7 @@ void gru_forward_kernel(GruFwdParams p) {
     pc[pp] = idx % HS;
     pn[pp] = n0 + pl[pp];
     pj[pp] = j0 + pc[pp];
-    act[pp] = idx < NB * HS && pn[pp] < N && pj[pp] < H;
+    act[pp] = idx < NB * HS && pl[pp] < rows_here && pj[pp] < H;
     h_prev[pp] = 0.f;
 #pragma unroll
     for (int g = 0; g < 3; ++g) bxv[pp][g] = brv[pp][g] = 0.f;
@@ -113,7 +114,7 @@ void gru_forward_kernel(GruFwdParams p) {
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
-    slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, N - n0, H, Kpad, w_lds,
+    slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, rows_here, H, Kpad, w_lds,
                                 vec_ok, gs.same_xcd, acc);
     store_partials<RT, CT>(red, acc);
     __syncthreads();
@@ -186,7 +187,8 @@ void gru_backward_kernel(GruBwdParams p) {
 
   const int tid = threadIdx.x;
   const int j0 = role.cw * HSB;
-  const int n0 = role.bt * NB;
+  const int n0 = role.bt * p.ls.tile_rows;
+  const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
 
   GroupSync gs;
@@ -209,7 +211,7 @@ void gru_backward_kernel(GruBwdParams p) {
     pc[pp] = idx % HSB;
     pn[pp] = n0 + pl[pp];
     pj[pp] = j0 + pc[pp];
-    act[pp] = pn[pp] < N && pj[pp] < H;
+    act[pp] = pl[pp] < rows_here && pj[pp] < H;
     dh[pp] = act[pp] ? p.dh[(size_t)pn[pp] * H + pj[pp]] : 0.f;
 #pragma unroll
     for (int g = 0; g < 6; ++g) dbacc[pp][g] = 0.f;
@@ -283,7 +285,7 @@ void gru_backward_kernel(GruBwdParams p) {
     float4_t acc[RT][1];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc[rt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
-    slice_matmul<RT, 1, CHUNK>(p.dq + ((size_t)t * N + n0) * 3 * H, 3 * H, N - n0, K, Kpad, w_lds,
+    slice_matmul<RT, 1, CHUNK>(p.dq + ((size_t)t * N + n0) * 3 * H, 3 * H, rows_here, K, Kpad, w_lds,
                                vec_ok, gs.same_xcd, acc);
     store_partials<RT, 1>(red, acc);
     __syncthreads();
@@ -340,7 +342,7 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
   const ForwardTile tile = pick_forward_tile(3, N, H, 0);
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.lds_bytes, (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.tile_rows, tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;
 #define HASTE_LAUNCH_FWD(RT_, CT_, HS_)                                                       \
   if (tile.rt == RT_ && tile.hs == HS_)                                                       \
@@ -375,7 +377,7 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   p.dbx = dbx; p.dbr = dbr; p.dh = dh; p.dp = dp; p.dq = dq; p.zoneout_mask = zoneout_mask;
   p.db_partial = ws.scratch;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.lds_bytes, (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.tile_rows, tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const char* name = "gru_backward_recurrence";

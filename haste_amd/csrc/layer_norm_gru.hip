@@ -51,7 +51,8 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
   const int tid = threadIdx.x;
   const int gx = p.ls.gx;
   const int j0 = role.cw * HS;
-  const int n0 = role.bt * NB;
+  const int n0 = role.bt * p.ls.tile_rows;
+  const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
   const int own_units = (H - j0) < HS ? (H - j0) : HS;
   const int last_units = H - (gx - 1) * HS;
@@ -79,7 +80,7 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
     pn[pp] = n0 + pl[pp];
     pj[pp] = j0 + pc[pp];
     colok[pp] = idx < NB * HS && pj[pp] < H;
-    act[pp] = colok[pp] && pn[pp] < N;
+    act[pp] = colok[pp] && pl[pp] < rows_here;
     h_prev[pp] = act[pp] ? p.h[(size_t)pn[pp] * H + pj[pp]] : 0.f;
 #pragma unroll
     for (int g = 0; g < 3; ++g) {
@@ -113,7 +114,7 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
-    slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, N - n0, H, Kpad, w_lds,
+    slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, rows_here, H, Kpad, w_lds,
                                 vec_ok, gs.same_xcd, acc);
     store_partials<RT, CT>(red, acc);
     __syncthreads();
@@ -230,7 +231,8 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
   const int tid = threadIdx.x;
   const int gx = p.ls.gx;
   const int j0 = role.cw * HSB;
-  const int n0 = role.bt * NB;
+  const int n0 = role.bt * p.ls.tile_rows;
+  const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
   float* part = p.part + (size_t)role.bt * gx * NB * 4;
 
@@ -254,7 +256,7 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
     pc[pp] = idx % HSB;
     pn[pp] = n0 + pl[pp];
     pj[pp] = j0 + pc[pp];
-    act[pp] = pn[pp] < N && pj[pp] < H;
+    act[pp] = pl[pp] < rows_here && pj[pp] < H;
     dh[pp] = act[pp] ? p.dh[(size_t)pn[pp] * H + pj[pp]] : 0.f;
 #pragma unroll
     for (int g = 0; g < 3; ++g) g2[pp][g] = pj[pp] < H ? p.gamma2[g * H + pj[pp]] : 0.f;
@@ -368,7 +370,7 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
     float4_t acc[RT][1];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc[rt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
-    slice_matmul<RT, 1, CHUNK>(p.dq + ((size_t)t * N + n0) * 3 * H, 3 * H, N - n0, K, Kpad, w_lds,
+    slice_matmul<RT, 1, CHUNK>(p.dq + ((size_t)t * N + n0) * 3 * H, 3 * H, rows_here, K, Kpad, w_lds,
                                vec_ok, gs.same_xcd, acc);
     store_partials<RT, 1>(red, acc);
     __syncthreads();
@@ -448,7 +450,7 @@ int haste_hip_layer_norm_gru_forward_f32(int training, int steps, int batch_size
   p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
   p.part2 = ws.scratch;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.lds_bytes, 2u * (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.tile_rows, tile.lds_bytes, 2u * (unsigned)T + 1, &plan));
   p.ls = plan.shape;
 #define HASTE_LAUNCH(RT_, CT_, HS_)                                                          \
   if (tile.rt == RT_ && tile.hs == HS_)                                                      \
@@ -499,7 +501,7 @@ int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_s
   p.zoneout_mask = zoneout_mask;
   p.part = ws.scratch; p.col_partial = ws.scratch + part_floats;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.lds_bytes, 2u * (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.tile_rows, tile.lds_bytes, 2u * (unsigned)T + 1, &plan));
   p.ls = plan.shape;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const char* name = "layer_norm_gru_backward_recurrence";

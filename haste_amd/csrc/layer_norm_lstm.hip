@@ -59,7 +59,8 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
   const int tid = threadIdx.x;
   const int gx = p.ls.gx;
   const int j0 = role.cw * HS;
-  const int n0 = role.bt * NB;
+  const int n0 = role.bt * p.ls.tile_rows;
+  const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
   const int own_units = (H - j0) < HS ? (H - j0) : HS;     // valid hidden units here
   const int last_units = H - (gx - 1) * HS;                 // ... in the last workgroup
@@ -88,7 +89,7 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
     pn[pp] = n0 + pl[pp];
     pj[pp] = j0 + pc[pp];
     colok[pp] = idx < NB * HS && pj[pp] < H;
-    act[pp] = colok[pp] && pn[pp] < N;
+    act[pp] = colok[pp] && pl[pp] < rows_here;
     c_prev[pp] = h_prev[pp] = gh[pp] = bh[pp] = 0.f;
 #pragma unroll
     for (int g = 0; g < 4; ++g) bias[pp][g] = g2[pp][g] = 0.f;
@@ -131,7 +132,7 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
-    slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, N - n0, H, Kpad, w_lds,
+    slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, rows_here, H, Kpad, w_lds,
                                 vec_ok, gs.same_xcd, acc);
     store_partials<RT, CT>(red, acc);
     __syncthreads();
@@ -287,7 +288,8 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   const int tid = threadIdx.x;
   const int gx = p.ls.gx;
   const int j0 = role.cw * HSB;
-  const int n0 = role.bt * NB;
+  const int n0 = role.bt * p.ls.tile_rows;
+  const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
   float* part_a = p.part_a + (size_t)role.bt * gx * NB * 4;
   float* part_b = p.part_b + (size_t)role.bt * gx * NB * 4;
@@ -312,7 +314,7 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
     pc[pp] = idx % HSB;
     pn[pp] = n0 + pl[pp];
     pj[pp] = j0 + pc[pp];
-    act[pp] = pn[pp] < N && pj[pp] < H;
+    act[pp] = pl[pp] < rows_here && pj[pp] < H;
     dh[pp] = act[pp] ? p.dh[(size_t)pn[pp] * H + pj[pp]] : 0.f;
     dc[pp] = act[pp] ? p.dc[(size_t)pn[pp] * H + pj[pp]] : 0.f;
     gh[pp] = pj[pp] < H ? p.gamma_h[pj[pp]] : 0.f;
@@ -459,7 +461,7 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
     float4_t acc[RT][1];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc[rt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
-    slice_matmul<RT, 1, CHUNK>(p.act_Rh + ((size_t)t * N + n0) * 4 * H, 4 * H, N - n0, K, Kpad,
+    slice_matmul<RT, 1, CHUNK>(p.act_Rh + ((size_t)t * N + n0) * 4 * H, 4 * H, rows_here, K, Kpad,
                                w_lds, vec_ok, gs.same_xcd, acc);
     store_partials<RT, 1>(red, acc);
     __syncthreads();
@@ -548,7 +550,7 @@ int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_siz
   p.act_c_norm = act_c_norm; p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
   p.part2 = ws.scratch; p.part3 = ws.scratch + part_floats;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.lds_bytes, 3u * (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.tile_rows, tile.lds_bytes, 3u * (unsigned)T + 1, &plan));
   p.ls = plan.shape;
 #define HASTE_LAUNCH(RT_, CT_)                                                               \
   if (tile.rt == RT_ && tile.ct == CT_)                                                      \
@@ -608,7 +610,7 @@ int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_
   p.part_a = ws.scratch; p.part_b = ws.scratch + part_floats;
   p.col_partial = ws.scratch + 2 * part_floats;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.lds_bytes, 3u * (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.tile_rows, tile.lds_bytes, 3u * (unsigned)T + 1, &plan));
   p.ls = plan.shape;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const char* name = "layer_norm_lstm_backward_recurrence";

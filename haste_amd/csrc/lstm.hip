@@ -45,7 +45,8 @@ void lstm_forward_kernel(LstmFwdParams p) {
 
   const int tid = threadIdx.x;
   const int j0 = role.cw * HS;
-  const int n0 = role.bt * NB;
+  const int n0 = role.bt * p.ls.tile_rows;
+  const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
 
   GroupSync gs;
@@ -75,7 +76,7 @@ void lstm_forward_kernel(LstmFwdParams p) {
     pc[pp] = idx % HS;           // local hidden unit
     pn[pp] = n0 + pl[pp];
     pj[pp] = j0 + pc[pp];
-    act[pp] = idx < NB * HS && pn[pp] < N && pj[pp] < H;
+    act[pp] = idx < NB * HS && pl[pp] < rows_here && pj[pp] < H;
     c_prev[pp] = 0.f;
     h_prev[pp] = 0.f;
 #pragma unroll
@@ -113,7 +114,7 @@ void lstm_forward_kernel(LstmFwdParams p) {
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
-    slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, N - n0, H, Kpad, w_lds,
+    slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, rows_here, H, Kpad, w_lds,
                                 vec_ok, gs.same_xcd, acc);
     store_partials<RT, CT>(red, acc);
     __syncthreads();
@@ -192,7 +193,8 @@ void lstm_backward_kernel(LstmBwdParams p) {
 
   const int tid = threadIdx.x;
   const int j0 = role.cw * HSB;
-  const int n0 = role.bt * NB;
+  const int n0 = role.bt * p.ls.tile_rows;
+  const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
 
   GroupSync gs;
@@ -215,7 +217,7 @@ void lstm_backward_kernel(LstmBwdParams p) {
     pc[pp] = idx % HSB;
     pn[pp] = n0 + pl[pp];
     pj[pp] = j0 + pc[pp];
-    act[pp] = pn[pp] < N && pj[pp] < H;
+    act[pp] = pl[pp] < rows_here && pj[pp] < H;
     dh[pp] = act[pp] ? p.dh[(size_t)pn[pp] * H + pj[pp]] : 0.f;
     dc[pp] = act[pp] ? p.dc[(size_t)pn[pp] * H + pj[pp]] : 0.f;
 #pragma unroll
@@ -292,7 +294,7 @@ void lstm_backward_kernel(LstmBwdParams p) {
     float4_t acc[RT][1];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc[rt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
-    slice_matmul<RT, 1, CHUNK>(p.v + ((size_t)t * N + n0) * 4 * H, 4 * H, N - n0, K, Kpad, w_lds,
+    slice_matmul<RT, 1, CHUNK>(p.v + ((size_t)t * N + n0) * 4 * H, 4 * H, rows_here, K, Kpad, w_lds,
                                vec_ok, gs.same_xcd, acc);
     store_partials<RT, 1>(red, acc);
     __syncthreads();
@@ -358,7 +360,7 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
   const ForwardTile tile = pick_forward_tile(4, N, H, 0);
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.lds_bytes, (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.tile_rows, tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;
 #define HASTE_LAUNCH_FWD(RT_, CT_)                                                         \
   if (tile.rt == RT_ && tile.ct == CT_)                                                    \
@@ -392,7 +394,7 @@ int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   p.db = db; p.dh = dh; p.dc = dc; p.v = v; p.zoneout_mask = zoneout_mask;
   p.db_partial = ws.scratch;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.lds_bytes, (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.tile_rows, tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const char* name = "lstm_backward_recurrence";

@@ -58,6 +58,7 @@ struct LaunchShape {
   unsigned int epoch;          // step flags of this launch count up from here
   unsigned int ticket_base;    // per-XCD tickets of this launch count up from here
   int gx, gy;                  // column workgroups per group, number of groups (batch tiles)
+  int tile_rows;               // batch rows per group (<= 16*RT; 8 spreads small batches over more XCDs)
   int xcd_local;               // 1: group g is the set of workgroups running on XCD g
   int per_xcd;                 // workgroups this launch places on every XCD (xcd_local)
 };
@@ -444,13 +445,14 @@ inline bool xcd_local_fits(int gx, int gy) {
   return xcd_local_enabled() && cus % kXcdCount == 0 && gy <= kXcdCount && gx <= cus / kXcdCount;
 }
 
-inline int plan_launch(hipStream_t stream, const Workspace& ws, int gx, int gy, size_t lds_bytes,
-                       unsigned int epochs, LaunchPlan* plan) {
+inline int plan_launch(hipStream_t stream, const Workspace& ws, int gx, int gy, int tile_rows,
+                       size_t lds_bytes, unsigned int epochs, LaunchPlan* plan) {
   plan->shape.cb = ws.control;
   plan->shape.host_status = ws.host_status_dev;
   plan->shape.spin_limit = kSpinLimit;
   plan->shape.gx = gx;
   plan->shape.gy = gy;
+  plan->shape.tile_rows = tile_rows;
   plan->shape.ticket_base = 0;
   plan->shape.per_xcd = 0;
   HASTE_HIP_PROPAGATE(reserve_epochs(stream, epochs, &plan->shape.epoch));
@@ -470,6 +472,14 @@ inline int plan_launch(hipStream_t stream, const Workspace& ws, int gx, int gy, 
   return HASTE_HIP_OK;
 }
 
+// Launches a persistent kernel whose workgroups wait for each other, so all of them must
+// be resident at once: the grid is checked against what the chip can hold.  It is an
+// ordinary launch, not hipLaunchCooperativeKernel: the cooperative queue can be held by only
+// one process per device at a time (a second process gets hipErrorIllegalState), which
+// would make the library unusable from several workers sharing a GPU.  Two persistent kernels
+// of this process on different streams are ordered one after the other (see
+// order_persistent_launches) because two half-resident grids could starve each other; the
+// bounded step-barrier waits cover everything else (another process's long kernel).
 template <typename KernelT, typename ParamsT>
 int launch_persistent(const char* name, KernelT kernel, const LaunchPlan& plan, ParamsT& params,
                       hipStream_t stream) {
@@ -480,10 +490,13 @@ int launch_persistent(const char* name, KernelT kernel, const LaunchPlan& plan, 
   HASTE_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, plan.lds_bytes));
   const long long capacity = (long long)per_cu * device_cu_count();
   if ((long long)plan.grid.x * plan.grid.y > capacity) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
-  void* args[] = {&params};
-  ScopedKernelTimer timer(name, stream);
-  HASTE_HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<const void*>(kernel), plan.grid,
-                                           dim3(256), args, (unsigned int)plan.lds_bytes, stream));
+  HASTE_HIP_PROPAGATE(order_persistent_launches(stream, true));
+  {
+    ScopedKernelTimer timer(name, stream);
+    kernel<<<plan.grid, dim3(256), plan.lds_bytes, stream>>>(params);
+    HASTE_HIP_TRY(hipGetLastError());
+  }
+  HASTE_HIP_PROPAGATE(order_persistent_launches(stream, false));
   return HASTE_HIP_OK;
 }
 
@@ -492,7 +505,7 @@ constexpr size_t kMaxLdsBytes = 160 * 1024;  // LDS per workgroup on gfx950
 // Geometry of a forward recurrence: 16*rt batch rows and hs hidden units per workgroup
 // (their gate columns fill ct MFMA column tiles), gx column workgroups, gy batch tiles.
 struct ForwardTile {
-  int rt, ct, hs, gx, gy;
+  int rt, ct, hs, gx, gy, tile_rows;
   size_t lds_bytes;
   bool ok;
 };
@@ -516,7 +529,13 @@ inline ForwardTile pick_forward_tile(int gates, int N, int H, size_t extra_lds_p
         const size_t lds = fwd_lds_bytes(H, rt, ct) + extra_lds_per_row * NB;
         if (lds > kMaxLdsBytes || gy > kMaxGroups || gx * gy > kMaxWorkgroups) continue;
         if (pass == 0 ? !xcd_local_fits(gx, gy) : (long long)gx * gy > cus) continue;
-        best = ForwardTile{rt, ct, hs, gx, gy, lds, true};
+        best = ForwardTile{rt, ct, hs, gx, gy, NB, lds, true};
+        // Half-height tiles put a small batch on twice as many XCDs: the MFMA count per
+        // workgroup is unchanged, the exchanged rows each one reads are halved.
+        if (pass == 0 && rt == 1 && xcd_local_fits(gx, (N + 7) / 8)) {
+          best.tile_rows = 8;
+          best.gy = (N + 7) / 8;
+        }
       }
       if (best.ok) break;
     }
@@ -526,7 +545,7 @@ inline ForwardTile pick_forward_tile(int gates, int N, int H, size_t extra_lds_p
 
 // Geometry of a backward recurrence: 16 hidden units and 16*rt batch rows per workgroup.
 struct BackwardTile {
-  int rt, gx, gy;
+  int rt, gx, gy, tile_rows;
   size_t lds_bytes;
   bool ok;
 };
@@ -546,7 +565,11 @@ inline BackwardTile pick_backward_tile(int K, int N, int H, size_t extra_floats_
       const size_t lds = ((size_t)Kpad * 16 + extra_floats_per_row * NB) * sizeof(float);
       if (lds > kMaxLdsBytes || gy > kMaxGroups || gx * gy > kMaxWorkgroups) continue;
       if (pass == 0 ? !xcd_local_fits(gx, gy) : (long long)gx * gy > cus) continue;
-      best = BackwardTile{rt, gx, gy, lds, true};
+      best = BackwardTile{rt, gx, gy, NB, lds, true};
+      if (pass == 0 && rt == 1 && xcd_local_fits(gx, (N + 7) / 8)) {
+        best.tile_rows = 8;
+        best.gy = (N + 7) / 8;
+      }
       break;
     }
   }

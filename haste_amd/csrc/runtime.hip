@@ -70,6 +70,31 @@ void set_runtime_error(hipError_t err, const char* what) {
   (void)hipGetLastError();  // do not leave the error for an unrelated later call
 }
 
+namespace {
+struct LastPersistent {
+  hipEvent_t event = nullptr;
+  hipStream_t stream = nullptr;
+  bool valid = false;
+};
+std::map<int, LastPersistent> g_last_persistent;
+}  // namespace
+
+int order_persistent_launches(hipStream_t stream, bool before) {
+  int dev = 0;
+  HASTE_HIP_TRY(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_mutex);
+  LastPersistent& lp = g_last_persistent[dev];
+  if (before) {
+    if (lp.valid && lp.stream != stream) HASTE_HIP_TRY(hipStreamWaitEvent(stream, lp.event, 0));
+    return HASTE_HIP_OK;
+  }
+  if (lp.event == nullptr) HASTE_HIP_TRY(hipEventCreateWithFlags(&lp.event, hipEventDisableTiming));
+  HASTE_HIP_TRY(hipEventRecord(lp.event, stream));
+  lp.stream = stream;
+  lp.valid = true;
+  return HASTE_HIP_OK;
+}
+
 bool xcd_local_enabled() {
   static const bool enabled = [] {
     const char* v = std::getenv("HASTE_HIP_XCD_LOCAL");
