@@ -27,14 +27,13 @@ struct GruFwdParams {
 
 // HS hidden units per workgroup; their 3 gate columns occupy 3*HS of the 16*CT slice
 // columns (the rest are zero padding).
-template <int RT, int CT, int HS>
+// NB batch rows per workgroup.
+template <int NB, int CT, int HS>
 __global__ __launch_bounds__(256, 1)
 void gru_forward_kernel(GruFwdParams p) {
   static_assert(3 * HS <= 16 * CT, "slice too narrow");
-  constexpr int NB = 16 * RT;
   constexpr int NCOLS = 16 * CT;
   constexpr int PP = (NB * HS + 255) / 256;
-  constexpr int CHUNK = RT == 4 ? 2 : 4;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   __shared__ unsigned int s_role;
   const Role role = take_role(p.ls, &s_role);
@@ -109,14 +108,8 @@ void gru_forward_kernel(GruFwdParams p) {
     }
     if (t > 0) group_wait(gs);
 
-    float4_t acc[RT][CT];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
-    slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, rows_here, H, Kpad, w_lds,
-                                vec_ok, gs.same_xcd, acc);
-    store_partials<RT, CT>(red, acc);
+    slice_product<NB, CT, false>(p.h + (size_t)t * NH + (size_t)n0 * H, H, rows_here, H, Kpad, w_lds,
+                                 vec_ok, gs.same_xcd, red);
     __syncthreads();
 
 #pragma unroll
@@ -124,7 +117,7 @@ void gru_forward_kernel(GruFwdParams p) {
       if (act[pp]) {
         float rh[3];
 #pragma unroll
-        for (int g = 0; g < 3; ++g) rh[g] = sum_partials<RT, CT>(red, pl[pp], g * HS + pc[pp]);
+        for (int g = 0; g < 3; ++g) rh[g] = sum_product<NB, CT>(red, pl[pp], g * HS + pc[pp]);
         const float z = sigmoid_f(wx[pp][0] + rh[0] + bxv[pp][0] + brv[pp][0]);
         const float r = sigmoid_f(wx[pp][1] + rh[1] + bxv[pp][1] + brv[pp][1]);
         const float qg = rh[2] + brv[pp][2];
@@ -165,14 +158,12 @@ struct GruBwdParams {
   LaunchShape ls;
 };
 
-template <int RT>
+template <int NB>
 __global__ __launch_bounds__(256, 1)
 void gru_backward_kernel(GruBwdParams p) {
   constexpr int HSB = 16;
-  constexpr int NB = 16 * RT;
   constexpr int NCOLS = 16;
-  constexpr int PP = RT;
-  constexpr int CHUNK = RT == 1 ? 8 : (RT == 2 ? 4 : 2);
+  constexpr int PP = (NB * HSB + 255) / 256;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   __shared__ unsigned int s_role;
   const Role role = take_role(p.ls, &s_role);
@@ -183,7 +174,7 @@ void gru_backward_kernel(GruBwdParams p) {
   const int K = 3 * H;
   const int Kpad = round_up(K, 64);
   float* w_lds = lds;
-  float* red = lds + Kpad * NCOLS;  // max(4*NB*16, NB*6*16) floats
+  float* red = lds + Kpad * NCOLS;  // the partial tiles or NB*6*16 floats, whichever is more
 
   const int tid = threadIdx.x;
   const int j0 = role.cw * HSB;
@@ -211,7 +202,7 @@ void gru_backward_kernel(GruBwdParams p) {
     pc[pp] = idx % HSB;
     pn[pp] = n0 + pl[pp];
     pj[pp] = j0 + pc[pp];
-    act[pp] = pl[pp] < rows_here && pj[pp] < H;
+    act[pp] = idx < NB * HSB && pl[pp] < rows_here && pj[pp] < H;
     dh[pp] = act[pp] ? p.dh[(size_t)pn[pp] * H + pj[pp]] : 0.f;
 #pragma unroll
     for (int g = 0; g < 6; ++g) dbacc[pp][g] = 0.f;
@@ -282,16 +273,12 @@ void gru_backward_kernel(GruBwdParams p) {
     fetch(t - 1);
     group_wait(gs);
 
-    float4_t acc[RT][1];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) acc[rt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
-    slice_matmul<RT, 1, CHUNK>(p.dq + ((size_t)t * N + n0) * 3 * H, 3 * H, rows_here, K, Kpad, w_lds,
-                               vec_ok, gs.same_xcd, acc);
-    store_partials<RT, 1>(red, acc);
+    slice_product<NB, 1, true>(p.dq + ((size_t)t * N + n0) * 3 * H, 3 * H, rows_here, K, Kpad, w_lds,
+                               vec_ok, gs.same_xcd, red);
     __syncthreads();
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp)
-      dh[pp] = dh_keep[pp] + sum_partials<RT, 1>(red, pl[pp], pc[pp]);
+      if (tid + 256 * pp < NB * HSB) dh[pp] = dh_keep[pp] + sum_product<NB, 1>(red, pl[pp], pc[pp]);
   }
 
 #pragma unroll
@@ -301,8 +288,10 @@ void gru_backward_kernel(GruBwdParams p) {
   __syncthreads();
 #pragma unroll
   for (int pp = 0; pp < PP; ++pp)
+    if (tid + 256 * pp < NB * HSB) {
 #pragma unroll
-    for (int g = 0; g < 6; ++g) red[(pl[pp] * 6 + g) * HSB + pc[pp]] = act[pp] ? dbacc[pp][g] : 0.f;
+      for (int g = 0; g < 6; ++g) red[(pl[pp] * 6 + g) * HSB + pc[pp]] = act[pp] ? dbacc[pp][g] : 0.f;
+    }
   __syncthreads();
   if (tid < 6 * HSB) {
     const int g = tid / HSB, jj = tid % HSB;
@@ -342,15 +331,17 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
   const ForwardTile tile = pick_forward_tile(3, N, H, 0);
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.tile_rows, tile.lds_bytes, (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.nb, tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;
-#define HASTE_LAUNCH_FWD(RT_, CT_, HS_)                                                       \
-  if (tile.rt == RT_ && tile.hs == HS_)                                                       \
-    return launch_persistent("gru_forward_recurrence", gru_forward_kernel<RT_, CT_, HS_>,     \
+#define HASTE_LAUNCH_FWD(NB_, CT_, HS_)                                                       \
+  if (tile.nb == NB_ && tile.hs == HS_)                                                       \
+    return launch_persistent("gru_forward_recurrence", gru_forward_kernel<NB_, CT_, HS_>,     \
                              plan, p, stream);
-  HASTE_LAUNCH_FWD(1, 1, 4) HASTE_LAUNCH_FWD(1, 2, 8) HASTE_LAUNCH_FWD(1, 3, 16)
-  HASTE_LAUNCH_FWD(2, 1, 4) HASTE_LAUNCH_FWD(2, 2, 8) HASTE_LAUNCH_FWD(2, 3, 16)
   HASTE_LAUNCH_FWD(4, 1, 4) HASTE_LAUNCH_FWD(4, 2, 8) HASTE_LAUNCH_FWD(4, 3, 16)
+  HASTE_LAUNCH_FWD(8, 1, 4) HASTE_LAUNCH_FWD(8, 2, 8) HASTE_LAUNCH_FWD(8, 3, 16)
+  HASTE_LAUNCH_FWD(16, 1, 4) HASTE_LAUNCH_FWD(16, 2, 8) HASTE_LAUNCH_FWD(16, 3, 16)
+  HASTE_LAUNCH_FWD(32, 1, 4) HASTE_LAUNCH_FWD(32, 2, 8) HASTE_LAUNCH_FWD(32, 3, 16)
+  HASTE_LAUNCH_FWD(64, 1, 4) HASTE_LAUNCH_FWD(64, 2, 8) HASTE_LAUNCH_FWD(64, 3, 16)
 #undef HASTE_LAUNCH_FWD
   return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 }
@@ -363,8 +354,8 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
   HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && v && dh_new);
   HASTE_HIP_REQUIRE(dx && dW && dR && dbx && dbr && dh && dp && dq);
-  // per row: max(4 partial tiles, the 6 bias-gradient columns) of 16 floats
-  const BackwardTile tile = pick_backward_tile(3 * H, N, H, 96);
+  // per row: the partial tiles or the 6 bias-gradient columns of 16 floats
+  const BackwardTile tile = pick_backward_tile(3 * H, N, H, 6 * 16, 0);
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 
   Workspace ws;
@@ -377,13 +368,15 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   p.dbx = dbx; p.dbr = dbr; p.dh = dh; p.dp = dp; p.dq = dq; p.zoneout_mask = zoneout_mask;
   p.db_partial = ws.scratch;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.tile_rows, tile.lds_bytes, (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.nb, tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const char* name = "gru_backward_recurrence";
-  if (tile.rt == 1) rc = launch_persistent(name, gru_backward_kernel<1>, plan, p, stream);
-  if (tile.rt == 2) rc = launch_persistent(name, gru_backward_kernel<2>, plan, p, stream);
-  if (tile.rt == 4) rc = launch_persistent(name, gru_backward_kernel<4>, plan, p, stream);
+  if (tile.nb == 4) rc = launch_persistent(name, gru_backward_kernel<4>, plan, p, stream);
+  if (tile.nb == 8) rc = launch_persistent(name, gru_backward_kernel<8>, plan, p, stream);
+  if (tile.nb == 16) rc = launch_persistent(name, gru_backward_kernel<16>, plan, p, stream);
+  if (tile.nb == 32) rc = launch_persistent(name, gru_backward_kernel<32>, plan, p, stream);
+  if (tile.nb == 64) rc = launch_persistent(name, gru_backward_kernel<64>, plan, p, stream);
   HASTE_HIP_PROPAGATE(rc);
 
   const int TN = T * N;

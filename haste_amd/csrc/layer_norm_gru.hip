@@ -29,14 +29,13 @@ struct LnGruFwdParams {
   LaunchShape ls;
 };
 
-template <int RT, int CT, int HS>
+// NB batch rows per workgroup.
+template <int NB, int CT, int HS>
 __global__ __launch_bounds__(256, 1)
 void ln_gru_forward_kernel(LnGruFwdParams p) {
   static_assert(3 * HS <= 16 * CT, "slice too narrow");
-  constexpr int NB = 16 * RT;
   constexpr int NCOLS = 16 * CT;
   constexpr int PP = (NB * HS + 255) / 256;
-  constexpr int CHUNK = RT == 4 ? 2 : 4;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   __shared__ unsigned int s_role;
   const Role role = take_role(p.ls, &s_role);
@@ -46,7 +45,7 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
   const int Kpad = round_up(H, 64);
   float* w_lds = lds;
   float* red = lds + Kpad * NCOLS;
-  float* stat = red + 4 * NB * NCOLS;
+  float* stat = red + ProductTile<NB, CT>::kRedFloats;
 
   const int tid = threadIdx.x;
   const int gx = p.ls.gx;
@@ -75,7 +74,7 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
 #pragma unroll
   for (int pp = 0; pp < PP; ++pp) {
     const int idx = tid + 256 * pp;
-    pl[pp] = idx / HS;
+    pl[pp] = idx < NB * HS ? idx / HS : 0;  // surplus threads shadow row 0, never store
     pc[pp] = idx % HS;
     pn[pp] = n0 + pl[pp];
     pj[pp] = j0 + pc[pp];
@@ -109,14 +108,8 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
     }
     if (t > 0) group_wait(gs);
 
-    float4_t acc[RT][CT];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
-    slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, rows_here, H, Kpad, w_lds,
-                                vec_ok, gs.same_xcd, acc);
-    store_partials<RT, CT>(red, acc);
+    slice_product<NB, CT, false>(p.h + (size_t)t * NH + (size_t)n0 * H, H, rows_here, H, Kpad, w_lds,
+                                 vec_ok, gs.same_xcd, red);
     __syncthreads();
 
     float rh[PP][3];
@@ -125,7 +118,7 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
       float s = 0.f;
 #pragma unroll
       for (int g = 0; g < 3; ++g) {
-        rh[pp][g] = colok[pp] ? sum_partials<RT, CT>(red, pl[pp], g * HS + pc[pp]) : 0.f;
+        rh[pp][g] = colok[pp] ? sum_product<NB, CT>(red, pl[pp], g * HS + pc[pp]) : 0.f;
         s += rh[pp][g];
       }
       if (act[pp]) {
@@ -206,15 +199,15 @@ struct LnGruBwdParams {
   LaunchShape ls;
 };
 
-template <int RT>
+template <int NB>
 __global__ __launch_bounds__(256, 1)
 void ln_gru_backward_kernel(LnGruBwdParams p) {
   constexpr int HSB = 16;
-  constexpr int NB = 16 * RT;
   constexpr int NCOLS = 16;
-  constexpr int PP = RT;
-  constexpr int CHUNK = RT == 1 ? 8 : (RT == 2 ? 4 : 2);
+  constexpr int PP = (NB * HSB + 255) / 256;
   constexpr int NACC = 9;  // dbx x3, dbr x3, dgamma2 x3
+  constexpr int RED = NB * NACC * HSB > ProductTile<NB, 1>::kRedFloats
+                          ? NB * NACC * HSB : ProductTile<NB, 1>::kRedFloats;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   __shared__ unsigned int s_role;
   const Role role = take_role(p.ls, &s_role);
@@ -225,8 +218,8 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
   const int K = 3 * H;
   const int Kpad = round_up(K, 64);
   float* w_lds = lds;
-  float* red = lds + Kpad * NCOLS;
-  float* sums = red + NB * NACC * HSB;
+  float* red = lds + Kpad * NCOLS;  // the partial tiles, reused for the column sums
+  float* sums = red + RED;           // [NB][4]
 
   const int tid = threadIdx.x;
   const int gx = p.ls.gx;
@@ -247,16 +240,17 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
   }
 
   int pn[PP], pj[PP], pl[PP], pc[PP];
-  bool act[PP];
+  bool act[PP], own[PP];
   float dh[PP], accs[PP][NACC], g2[PP][3];
 #pragma unroll
   for (int pp = 0; pp < PP; ++pp) {
     const int idx = tid + 256 * pp;
-    pl[pp] = idx / HSB;
+    own[pp] = idx < NB * HSB;  // surplus threads of a short tile shadow row 0, never store
+    pl[pp] = own[pp] ? idx / HSB : 0;
     pc[pp] = idx % HSB;
     pn[pp] = n0 + pl[pp];
     pj[pp] = j0 + pc[pp];
-    act[pp] = pl[pp] < rows_here && pj[pp] < H;
+    act[pp] = own[pp] && pl[pp] < rows_here && pj[pp] < H;
     dh[pp] = act[pp] ? p.dh[(size_t)pn[pp] * H + pj[pp]] : 0.f;
 #pragma unroll
     for (int g = 0; g < 3; ++g) g2[pp][g] = pj[pp] < H ? p.gamma2[g * H + pj[pp]] : 0.f;
@@ -342,7 +336,7 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
       t0 = segment_sum<HSB>(t0);
       t1 = segment_sum<HSB>(t1);
       t2 = segment_sum<HSB>(t2);
-      if (pc[pp] == 0)
+      if (pc[pp] == 0 && own[pp])
         store_exchanged4(gs, part + ((size_t)role.cw * NB + pl[pp]) * 4, t0, t1, t2, 0.f);
     }
     group_arrive(gs);
@@ -367,16 +361,12 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
     fetch(t - 1);
     group_wait(gs);
 
-    float4_t acc[RT][1];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) acc[rt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
-    slice_matmul<RT, 1, CHUNK>(p.dq + ((size_t)t * N + n0) * 3 * H, 3 * H, rows_here, K, Kpad, w_lds,
-                               vec_ok, gs.same_xcd, acc);
-    store_partials<RT, 1>(red, acc);
+    slice_product<NB, 1, true>(p.dq + ((size_t)t * N + n0) * 3 * H, 3 * H, rows_here, K, Kpad, w_lds,
+                               vec_ok, gs.same_xcd, red);
     __syncthreads();
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp)
-      dh[pp] = dh_keep[pp] + sum_partials<RT, 1>(red, pl[pp], pc[pp]);
+      dh[pp] = dh_keep[pp] + sum_product<NB, 1>(red, pl[pp], pc[pp]);
   }
 
 #pragma unroll
@@ -388,7 +378,7 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
   for (int pp = 0; pp < PP; ++pp)
 #pragma unroll
     for (int a = 0; a < NACC; ++a)
-      red[(pl[pp] * NACC + a) * HSB + pc[pp]] = act[pp] ? accs[pp][a] : 0.f;
+      if (own[pp]) red[(pl[pp] * NACC + a) * HSB + pc[pp]] = act[pp] ? accs[pp][a] : 0.f;
   __syncthreads();
   if (tid < NACC * HSB) {
     const int a = tid / HSB, jj = tid % HSB;
@@ -433,7 +423,7 @@ int haste_hip_layer_norm_gru_forward_f32(int training, int steps, int batch_size
   const ForwardTile tile = pick_forward_tile(3, N, H, 2 * sizeof(float));
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const int gx = tile.gx, gy = tile.gy;
-  const int NB = 16 * tile.rt;
+  const int NB = tile.nb;
   const size_t part_floats = (size_t)gy * gx * NB * 2;
 
   Workspace ws;
@@ -450,15 +440,17 @@ int haste_hip_layer_norm_gru_forward_f32(int training, int steps, int batch_size
   p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
   p.part2 = ws.scratch;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.tile_rows, tile.lds_bytes, 2u * (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes, 2u * (unsigned)T + 1, &plan));
   p.ls = plan.shape;
-#define HASTE_LAUNCH(RT_, CT_, HS_)                                                          \
-  if (tile.rt == RT_ && tile.hs == HS_)                                                      \
+#define HASTE_LAUNCH(NB_, CT_, HS_)                                                          \
+  if (tile.nb == NB_ && tile.hs == HS_)                                                      \
     return launch_persistent("layer_norm_gru_forward_recurrence",                            \
-                             ln_gru_forward_kernel<RT_, CT_, HS_>, plan, p, stream);
-  HASTE_LAUNCH(1, 1, 4) HASTE_LAUNCH(1, 2, 8) HASTE_LAUNCH(1, 3, 16)
-  HASTE_LAUNCH(2, 1, 4) HASTE_LAUNCH(2, 2, 8) HASTE_LAUNCH(2, 3, 16)
+                             ln_gru_forward_kernel<NB_, CT_, HS_>, plan, p, stream);
   HASTE_LAUNCH(4, 1, 4) HASTE_LAUNCH(4, 2, 8) HASTE_LAUNCH(4, 3, 16)
+  HASTE_LAUNCH(8, 1, 4) HASTE_LAUNCH(8, 2, 8) HASTE_LAUNCH(8, 3, 16)
+  HASTE_LAUNCH(16, 1, 4) HASTE_LAUNCH(16, 2, 8) HASTE_LAUNCH(16, 3, 16)
+  HASTE_LAUNCH(32, 1, 4) HASTE_LAUNCH(32, 2, 8) HASTE_LAUNCH(32, 3, 16)
+  HASTE_LAUNCH(64, 1, 4) HASTE_LAUNCH(64, 2, 8) HASTE_LAUNCH(64, 3, 16)
 #undef HASTE_LAUNCH
   return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 }
@@ -481,11 +473,11 @@ int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_s
   HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && v && dh_new && dx && dW && dR && dbx && dbr && dh);
   HASTE_HIP_REQUIRE(dp && dq && act_Wx && gamma1 && dgamma1 && act_Rh && gamma2 && dgamma2 && cache2);
   hipStream_t stream = as_stream(stream_);
-  // per row: 9 column-sum accumulators of 16 floats (covers the 4 partial tiles) + 4 sums
-  const BackwardTile tile = pick_backward_tile(3 * H, N, H, 9 * 16 + 4);
+  // per row: 9 column-sum accumulators of 16 floats (or the partial tiles, whichever is more) + 4 sums
+  const BackwardTile tile = pick_backward_tile(3 * H, N, H, 9 * 16, 4);
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
-  const int gx = tile.gx, gy = tile.gy, rt = tile.rt;
-  const int NB = 16 * rt;
+  const int gx = tile.gx, gy = tile.gy;
+  const int NB = tile.nb;
   const size_t part_floats = (size_t)gy * gx * NB * 4;
   const size_t col_floats = (size_t)gy * 9 * H;
 
@@ -501,13 +493,15 @@ int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_s
   p.zoneout_mask = zoneout_mask;
   p.part = ws.scratch; p.col_partial = ws.scratch + part_floats;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.tile_rows, tile.lds_bytes, 2u * (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes, 2u * (unsigned)T + 1, &plan));
   p.ls = plan.shape;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const char* name = "layer_norm_gru_backward_recurrence";
-  if (rt == 1) rc = launch_persistent(name, ln_gru_backward_kernel<1>, plan, p, stream);
-  if (rt == 2) rc = launch_persistent(name, ln_gru_backward_kernel<2>, plan, p, stream);
-  if (rt == 4) rc = launch_persistent(name, ln_gru_backward_kernel<4>, plan, p, stream);
+  if (NB == 4) rc = launch_persistent(name, ln_gru_backward_kernel<4>, plan, p, stream);
+  if (NB == 8) rc = launch_persistent(name, ln_gru_backward_kernel<8>, plan, p, stream);
+  if (NB == 16) rc = launch_persistent(name, ln_gru_backward_kernel<16>, plan, p, stream);
+  if (NB == 32) rc = launch_persistent(name, ln_gru_backward_kernel<32>, plan, p, stream);
+  if (NB == 64) rc = launch_persistent(name, ln_gru_backward_kernel<64>, plan, p, stream);
   HASTE_HIP_PROPAGATE(rc);
 
   const int TN = T * N;

@@ -37,14 +37,13 @@ struct LnLstmFwdParams {
   LaunchShape ls;
 };
 
-template <int RT, int CT>
+// NB batch rows per workgroup.
+template <int NB, int CT>
 __global__ __launch_bounds__(256, 1)
 void ln_lstm_forward_kernel(LnLstmFwdParams p) {
   constexpr int HS = 4 * CT;
-  constexpr int NB = 16 * RT;
   constexpr int NCOLS = 16 * CT;
   constexpr int PP = (NB * HS + 255) / 256;
-  constexpr int CHUNK = RT == 4 ? 2 : 4;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   __shared__ unsigned int s_role;
   const Role role = take_role(p.ls, &s_role);
@@ -54,7 +53,7 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
   const int Kpad = round_up(H, 64);
   float* w_lds = lds;
   float* red = lds + Kpad * NCOLS;
-  float* stat = red + 4 * NB * NCOLS;  // [NB][2]
+  float* stat = red + ProductTile<NB, CT>::kRedFloats;  // [NB][2]
 
   const int tid = threadIdx.x;
   const int gx = p.ls.gx;
@@ -84,7 +83,7 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
 #pragma unroll
   for (int pp = 0; pp < PP; ++pp) {
     const int idx = tid + 256 * pp;
-    pl[pp] = idx / HS;
+    pl[pp] = idx < NB * HS ? idx / HS : 0;  // surplus threads shadow row 0, never store
     pc[pp] = idx % HS;
     pn[pp] = n0 + pl[pp];
     pj[pp] = j0 + pc[pp];
@@ -127,14 +126,8 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
     }
     if (t > 0) group_wait(gs);  // h[t]
 
-    float4_t acc[RT][CT];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
-    slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, rows_here, H, Kpad, w_lds,
-                                vec_ok, gs.same_xcd, acc);
-    store_partials<RT, CT>(red, acc);
+    slice_product<NB, CT, false>(p.h + (size_t)t * NH + (size_t)n0 * H, H, rows_here, H, Kpad, w_lds,
+                                 vec_ok, gs.same_xcd, red);
     __syncthreads();
 
     // h*R of the owned columns; moments of those columns per row, published.
@@ -144,7 +137,7 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
       float s = 0.f;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        rh[pp][g] = colok[pp] ? sum_partials<RT, CT>(red, pl[pp], g * HS + pc[pp]) : 0.f;
+        rh[pp][g] = colok[pp] ? sum_product<NB, CT>(red, pl[pp], g * HS + pc[pp]) : 0.f;
         s += rh[pp][g];
       }
       if (act[pp]) {
@@ -263,15 +256,15 @@ struct LnLstmBwdParams {
   LaunchShape ls;
 };
 
-template <int RT>
+template <int NB>
 __global__ __launch_bounds__(256, 1)
 void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   constexpr int HSB = 16;
-  constexpr int NB = 16 * RT;
   constexpr int NCOLS = 16;
-  constexpr int PP = RT;
-  constexpr int CHUNK = RT == 1 ? 8 : (RT == 2 ? 4 : 2);
+  constexpr int PP = (NB * HSB + 255) / 256;
   constexpr int NACC = 10;  // db x4, dgamma2 x4, dgamma_h, dbeta_h
+  constexpr int RED = NB * NACC * HSB > ProductTile<NB, 1>::kRedFloats
+                          ? NB * NACC * HSB : ProductTile<NB, 1>::kRedFloats;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   __shared__ unsigned int s_role;
   const Role role = take_role(p.ls, &s_role);
@@ -282,8 +275,8 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   const int K = 4 * H;
   const int Kpad = round_up(K, 64);
   float* w_lds = lds;
-  float* red = lds + Kpad * NCOLS;       // NB*NACC*16 floats (>= 4*NB*16)
-  float* sums = red + NB * NACC * HSB;   // [NB][4]
+  float* red = lds + Kpad * NCOLS;  // the partial tiles, reused for the column sums
+  float* sums = red + RED;           // [NB][4]
 
   const int tid = threadIdx.x;
   const int gx = p.ls.gx;
@@ -305,16 +298,17 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   }
 
   int pn[PP], pj[PP], pl[PP], pc[PP];
-  bool act[PP];
+  bool act[PP], own[PP];
   float dh[PP], dc[PP], accs[PP][NACC], g2[PP][4], gh[PP];
 #pragma unroll
   for (int pp = 0; pp < PP; ++pp) {
     const int idx = tid + 256 * pp;
-    pl[pp] = idx / HSB;
+    own[pp] = idx < NB * HSB;  // surplus threads of a short tile shadow row 0, never store
+    pl[pp] = own[pp] ? idx / HSB : 0;
     pc[pp] = idx % HSB;
     pn[pp] = n0 + pl[pp];
     pj[pp] = j0 + pc[pp];
-    act[pp] = pl[pp] < rows_here && pj[pp] < H;
+    act[pp] = own[pp] && pl[pp] < rows_here && pj[pp] < H;
     dh[pp] = act[pp] ? p.dh[(size_t)pn[pp] * H + pj[pp]] : 0.f;
     dc[pp] = act[pp] ? p.dc[(size_t)pn[pp] * H + pj[pp]] : 0.f;
     gh[pp] = pj[pp] < H ? p.gamma_h[pj[pp]] : 0.f;
@@ -387,7 +381,7 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
       const float s0 = segment_sum<HSB>(xc3[pp] * gd3[pp]);
       const float s1 = segment_sum<HSB>(xc3[pp]);
       const float s2 = segment_sum<HSB>(gd3[pp]);
-      if (pc[pp] == 0)
+      if (pc[pp] == 0 && own[pp])
         store_exchanged4(gs, part_a + ((size_t)role.cw * NB + pl[pp]) * 4, s0, s1, s2, 0.f);
     }
     group_arrive(gs);
@@ -433,7 +427,7 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
       t0 = segment_sum<HSB>(t0);
       t1 = segment_sum<HSB>(t1);
       t2 = segment_sum<HSB>(t2);
-      if (pc[pp] == 0)
+      if (pc[pp] == 0 && own[pp])
         store_exchanged4(gs, part_b + ((size_t)role.cw * NB + pl[pp]) * 4, t0, t1, t2, 0.f);
     }
     group_arrive(gs);
@@ -458,16 +452,12 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
     fetch(t - 1);
     group_wait(gs);  // gradient w.r.t. h*R complete for this batch tile
 
-    float4_t acc[RT][1];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) acc[rt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
-    slice_matmul<RT, 1, CHUNK>(p.act_Rh + ((size_t)t * N + n0) * 4 * H, 4 * H, rows_here, K, Kpad,
-                               w_lds, vec_ok, gs.same_xcd, acc);
-    store_partials<RT, 1>(red, acc);
+    slice_product<NB, 1, true>(p.act_Rh + ((size_t)t * N + n0) * 4 * H, 4 * H, rows_here, K, Kpad,
+                               w_lds, vec_ok, gs.same_xcd, red);
     __syncthreads();
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp)
-      dh[pp] = dh_keep[pp] + sum_partials<RT, 1>(red, pl[pp], pc[pp]);
+      dh[pp] = dh_keep[pp] + sum_product<NB, 1>(red, pl[pp], pc[pp]);
   }
 
 #pragma unroll
@@ -484,7 +474,7 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   for (int pp = 0; pp < PP; ++pp)
 #pragma unroll
     for (int a = 0; a < NACC; ++a)
-      red[(pl[pp] * NACC + a) * HSB + pc[pp]] = act[pp] ? accs[pp][a] : 0.f;
+      if (own[pp]) red[(pl[pp] * NACC + a) * HSB + pc[pp]] = act[pp] ? accs[pp][a] : 0.f;
   __syncthreads();
   if (tid < NACC * HSB) {
     const int a = tid / HSB, jj = tid % HSB;
@@ -533,7 +523,7 @@ int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_siz
   const ForwardTile tile = pick_forward_tile(4, N, H, 2 * sizeof(float));
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const int gx = tile.gx, gy = tile.gy;
-  const int NB = 16 * tile.rt;
+  const int NB = tile.nb;
   const size_t part_floats = (size_t)gy * gx * NB * 2;
 
   Workspace ws;
@@ -550,15 +540,17 @@ int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_siz
   p.act_c_norm = act_c_norm; p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
   p.part2 = ws.scratch; p.part3 = ws.scratch + part_floats;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.tile_rows, tile.lds_bytes, 3u * (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes, 3u * (unsigned)T + 1, &plan));
   p.ls = plan.shape;
-#define HASTE_LAUNCH(RT_, CT_)                                                               \
-  if (tile.rt == RT_ && tile.ct == CT_)                                                      \
+#define HASTE_LAUNCH(NB_, CT_)                                                               \
+  if (tile.nb == NB_ && tile.ct == CT_)                                                      \
     return launch_persistent("layer_norm_lstm_forward_recurrence",                           \
-                             ln_lstm_forward_kernel<RT_, CT_>, plan, p, stream);
-  HASTE_LAUNCH(1, 1) HASTE_LAUNCH(1, 2) HASTE_LAUNCH(1, 4)
-  HASTE_LAUNCH(2, 1) HASTE_LAUNCH(2, 2) HASTE_LAUNCH(2, 4)
+                             ln_lstm_forward_kernel<NB_, CT_>, plan, p, stream);
   HASTE_LAUNCH(4, 1) HASTE_LAUNCH(4, 2) HASTE_LAUNCH(4, 4)
+  HASTE_LAUNCH(8, 1) HASTE_LAUNCH(8, 2) HASTE_LAUNCH(8, 4)
+  HASTE_LAUNCH(16, 1) HASTE_LAUNCH(16, 2) HASTE_LAUNCH(16, 4)
+  HASTE_LAUNCH(32, 1) HASTE_LAUNCH(32, 2) HASTE_LAUNCH(32, 4)
+  HASTE_LAUNCH(64, 1) HASTE_LAUNCH(64, 2) HASTE_LAUNCH(64, 4)
 #undef HASTE_LAUNCH
   return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 }
@@ -588,11 +580,11 @@ int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_
   HASTE_HIP_REQUIRE(act_Wx_norm && act_Rh && gamma2 && dgamma2 && cache2 && gamma_h);
   HASTE_HIP_REQUIRE(dgamma_h && dbeta_h && cache3 && act_c_norm);
   hipStream_t stream = as_stream(stream_);
-  // per row: 10 column-sum accumulators of 16 floats (covers the 4 partial tiles) + 4 sums
-  const BackwardTile tile = pick_backward_tile(4 * H, N, H, 10 * 16 + 4);
+  // per row: 10 column-sum accumulators of 16 floats (or the partial tiles, whichever is more) + 4 sums
+  const BackwardTile tile = pick_backward_tile(4 * H, N, H, 10 * 16, 4);
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
-  const int gx = tile.gx, gy = tile.gy, rt = tile.rt;
-  const int NB = 16 * rt;
+  const int gx = tile.gx, gy = tile.gy;
+  const int NB = tile.nb;
   const size_t part_floats = (size_t)gy * gx * NB * 4;
   const size_t col_floats = (size_t)gy * 10 * H;
 
@@ -610,13 +602,15 @@ int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_
   p.part_a = ws.scratch; p.part_b = ws.scratch + part_floats;
   p.col_partial = ws.scratch + 2 * part_floats;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.tile_rows, tile.lds_bytes, 3u * (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes, 3u * (unsigned)T + 1, &plan));
   p.ls = plan.shape;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const char* name = "layer_norm_lstm_backward_recurrence";
-  if (rt == 1) rc = launch_persistent(name, ln_lstm_backward_kernel<1>, plan, p, stream);
-  if (rt == 2) rc = launch_persistent(name, ln_lstm_backward_kernel<2>, plan, p, stream);
-  if (rt == 4) rc = launch_persistent(name, ln_lstm_backward_kernel<4>, plan, p, stream);
+  if (NB == 4) rc = launch_persistent(name, ln_lstm_backward_kernel<4>, plan, p, stream);
+  if (NB == 8) rc = launch_persistent(name, ln_lstm_backward_kernel<8>, plan, p, stream);
+  if (NB == 16) rc = launch_persistent(name, ln_lstm_backward_kernel<16>, plan, p, stream);
+  if (NB == 32) rc = launch_persistent(name, ln_lstm_backward_kernel<32>, plan, p, stream);
+  if (NB == 64) rc = launch_persistent(name, ln_lstm_backward_kernel<64>, plan, p, stream);
   HASTE_HIP_PROPAGATE(rc);
 
   // Gradient through the norm of x*W (in place over act_Wx), then the batched products.

@@ -25,14 +25,13 @@ struct LstmFwdParams {
 };
 
 // HS hidden units per workgroup = 4*CT (their 4 gate columns fill CT MFMA column tiles).
-template <int RT, int CT>
+// NB batch rows per workgroup.
+template <int NB, int CT>
 __global__ __launch_bounds__(256, 1)
 void lstm_forward_kernel(LstmFwdParams p) {
   constexpr int HS = 4 * CT;
-  constexpr int NB = 16 * RT;
   constexpr int NCOLS = 16 * CT;
   constexpr int PP = (NB * HS + 255) / 256;
-  constexpr int CHUNK = RT == 4 ? 2 : 4;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   __shared__ unsigned int s_role;
   const Role role = take_role(p.ls, &s_role);
@@ -109,14 +108,8 @@ void lstm_forward_kernel(LstmFwdParams p) {
     }
     if (t > 0) group_wait(gs);  // h[t] complete for this batch tile
 
-    float4_t acc[RT][CT];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
-    slice_matmul<RT, CT, CHUNK>(p.h + (size_t)t * NH + (size_t)n0 * H, H, rows_here, H, Kpad, w_lds,
-                                vec_ok, gs.same_xcd, acc);
-    store_partials<RT, CT>(red, acc);
+    slice_product<NB, CT, false>(p.h + (size_t)t * NH + (size_t)n0 * H, H, rows_here, H, Kpad, w_lds,
+                                 vec_ok, gs.same_xcd, red);
     __syncthreads();
 
 #pragma unroll
@@ -125,7 +118,7 @@ void lstm_forward_kernel(LstmFwdParams p) {
         float a[4];
 #pragma unroll
         for (int g = 0; g < 4; ++g)
-          a[g] = wx[pp][g] + sum_partials<RT, CT>(red, pl[pp], g * HS + pc[pp]) + bias[pp][g];
+          a[g] = wx[pp][g] + sum_product<NB, CT>(red, pl[pp], g * HS + pc[pp]) + bias[pp][g];
         const float gi = sigmoid_f(a[0]);
         const float gg = tanhf(a[1]);
         const float gf = sigmoid_f(a[2]);
@@ -169,16 +162,14 @@ struct LstmBwdParams {
   LaunchShape ls;
 };
 
-// A workgroup owns 16 hidden units (HSB) for 16*RT batch rows; its slice of R_t is
+// A workgroup owns 16 hidden units (HSB) for NB batch rows; its slice of R_t is
 // [4H x 16]: dh[:, its units] = dv_t[:, all 4H] * R_t[:, its units].
-template <int RT>
+template <int NB>
 __global__ __launch_bounds__(256, 1)
 void lstm_backward_kernel(LstmBwdParams p) {
   constexpr int HSB = 16;
-  constexpr int NB = 16 * RT;
   constexpr int NCOLS = 16;
-  constexpr int PP = RT;  // NB*HSB/256
-  constexpr int CHUNK = RT == 1 ? 8 : (RT == 2 ? 4 : 2);
+  constexpr int PP = (NB * HSB + 255) / 256;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   __shared__ unsigned int s_role;
   const Role role = take_role(p.ls, &s_role);
@@ -189,7 +180,7 @@ void lstm_backward_kernel(LstmBwdParams p) {
   const int K = 4 * H;
   const int Kpad = round_up(K, 64);
   float* w_lds = lds;
-  float* red = lds + Kpad * NCOLS;  // 4*NB*NCOLS floats, also reused for the db reduction
+  float* red = lds + Kpad * NCOLS;  // the partial tiles, reused for the db reduction
 
   const int tid = threadIdx.x;
   const int j0 = role.cw * HSB;
@@ -217,7 +208,7 @@ void lstm_backward_kernel(LstmBwdParams p) {
     pc[pp] = idx % HSB;
     pn[pp] = n0 + pl[pp];
     pj[pp] = j0 + pc[pp];
-    act[pp] = pl[pp] < rows_here && pj[pp] < H;
+    act[pp] = idx < NB * HSB && pl[pp] < rows_here && pj[pp] < H;
     dh[pp] = act[pp] ? p.dh[(size_t)pn[pp] * H + pj[pp]] : 0.f;
     dc[pp] = act[pp] ? p.dc[(size_t)pn[pp] * H + pj[pp]] : 0.f;
 #pragma unroll
@@ -291,16 +282,12 @@ void lstm_backward_kernel(LstmBwdParams p) {
     fetch(t - 1);       // overlap next step's loads with the wait
     group_wait(gs);     // all 4H columns of dv_t are complete for this batch tile
 
-    float4_t acc[RT][1];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) acc[rt][0] = float4_t{0.f, 0.f, 0.f, 0.f};
-    slice_matmul<RT, 1, CHUNK>(p.v + ((size_t)t * N + n0) * 4 * H, 4 * H, rows_here, K, Kpad, w_lds,
-                               vec_ok, gs.same_xcd, acc);
-    store_partials<RT, 1>(red, acc);
+    slice_product<NB, 1, true>(p.v + ((size_t)t * N + n0) * 4 * H, 4 * H, rows_here, K, Kpad, w_lds,
+                               vec_ok, gs.same_xcd, red);
     __syncthreads();
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp)
-      dh[pp] = dh_keep[pp] + sum_partials<RT, 1>(red, pl[pp], pc[pp]);
+      if (tid + 256 * pp < NB * HSB) dh[pp] = dh_keep[pp] + sum_product<NB, 1>(red, pl[pp], pc[pp]);
     // `red` is next written after the __syncthreads inside the next group_arrive.
   }
 
@@ -317,8 +304,10 @@ void lstm_backward_kernel(LstmBwdParams p) {
   __syncthreads();
 #pragma unroll
   for (int pp = 0; pp < PP; ++pp)
+    if (tid + 256 * pp < NB * HSB) {
 #pragma unroll
-    for (int g = 0; g < 4; ++g) red[(pl[pp] * 4 + g) * HSB + pc[pp]] = act[pp] ? dbacc[pp][g] : 0.f;
+      for (int g = 0; g < 4; ++g) red[(pl[pp] * 4 + g) * HSB + pc[pp]] = act[pp] ? dbacc[pp][g] : 0.f;
+    }
   __syncthreads();
   if (tid < 4 * HSB) {
     const int g = tid / HSB, jj = tid % HSB;
@@ -337,8 +326,6 @@ void lstm_backward_kernel(LstmBwdParams p) {
 
 }  // namespace
 
-// Picks (RT, CT) for a forward recurrence with G gate blocks; shared with the GRU.
-// Preference: widest column tile that fits the LDS and the cooperative grid.
 int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int H,
                       const float* W, const float* R, const float* b, const float* x,
                       float* h, float* c, float* v, float zoneout_prob,
@@ -360,15 +347,17 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
   const ForwardTile tile = pick_forward_tile(4, N, H, 0);
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.tile_rows, tile.lds_bytes, (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.nb, tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;
-#define HASTE_LAUNCH_FWD(RT_, CT_)                                                         \
-  if (tile.rt == RT_ && tile.ct == CT_)                                                    \
-    return launch_persistent("lstm_forward_recurrence", lstm_forward_kernel<RT_, CT_>, plan, p, \
+#define HASTE_LAUNCH_FWD(NB_, CT_)                                                         \
+  if (tile.nb == NB_ && tile.ct == CT_)                                                    \
+    return launch_persistent("lstm_forward_recurrence", lstm_forward_kernel<NB_, CT_>, plan, p, \
                              stream);
-  HASTE_LAUNCH_FWD(1, 1) HASTE_LAUNCH_FWD(1, 2) HASTE_LAUNCH_FWD(1, 4)
-  HASTE_LAUNCH_FWD(2, 1) HASTE_LAUNCH_FWD(2, 2) HASTE_LAUNCH_FWD(2, 4)
   HASTE_LAUNCH_FWD(4, 1) HASTE_LAUNCH_FWD(4, 2) HASTE_LAUNCH_FWD(4, 4)
+  HASTE_LAUNCH_FWD(8, 1) HASTE_LAUNCH_FWD(8, 2) HASTE_LAUNCH_FWD(8, 4)
+  HASTE_LAUNCH_FWD(16, 1) HASTE_LAUNCH_FWD(16, 2) HASTE_LAUNCH_FWD(16, 4)
+  HASTE_LAUNCH_FWD(32, 1) HASTE_LAUNCH_FWD(32, 2) HASTE_LAUNCH_FWD(32, 4)
+  HASTE_LAUNCH_FWD(64, 1) HASTE_LAUNCH_FWD(64, 2) HASTE_LAUNCH_FWD(64, 4)
 #undef HASTE_LAUNCH_FWD
   return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 }
@@ -381,7 +370,7 @@ int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
   HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && c && dh_new && dc_new);
   HASTE_HIP_REQUIRE(dx && dW && dR && db && dh && dc && v);
-  const BackwardTile tile = pick_backward_tile(4 * H, N, H, 64);
+  const BackwardTile tile = pick_backward_tile(4 * H, N, H, 4 * 16, 0);
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 
   Workspace ws;
@@ -394,13 +383,15 @@ int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   p.db = db; p.dh = dh; p.dc = dc; p.v = v; p.zoneout_mask = zoneout_mask;
   p.db_partial = ws.scratch;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.tile_rows, tile.lds_bytes, (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.nb, tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const char* name = "lstm_backward_recurrence";
-  if (tile.rt == 1) rc = launch_persistent(name, lstm_backward_kernel<1>, plan, p, stream);
-  if (tile.rt == 2) rc = launch_persistent(name, lstm_backward_kernel<2>, plan, p, stream);
-  if (tile.rt == 4) rc = launch_persistent(name, lstm_backward_kernel<4>, plan, p, stream);
+  if (tile.nb == 4) rc = launch_persistent(name, lstm_backward_kernel<4>, plan, p, stream);
+  if (tile.nb == 8) rc = launch_persistent(name, lstm_backward_kernel<8>, plan, p, stream);
+  if (tile.nb == 16) rc = launch_persistent(name, lstm_backward_kernel<16>, plan, p, stream);
+  if (tile.nb == 32) rc = launch_persistent(name, lstm_backward_kernel<32>, plan, p, stream);
+  if (tile.nb == 64) rc = launch_persistent(name, lstm_backward_kernel<64>, plan, p, stream);
   HASTE_HIP_PROPAGATE(rc);
 
   // dW += x^T dv ; dR += h[0:T]^T dv ; dx = dv W^T  (dv now lives in v).

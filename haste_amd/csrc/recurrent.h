@@ -12,6 +12,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <utility>
+
 #include "common.h"
 
 namespace haste_hip {
@@ -290,8 +292,8 @@ __device__ __forceinline__ void load_a_chunk(const float* __restrict__ a, int a_
 }
 
 // MFMAs of k-groups [g_abs, g_abs+CHUNK): one straight-line block (no branches, so the
-// accumulators stay in the matrix unit's registers and the scheduler can hoist the LDS
-// reads of the slice columns ahead of the MFMAs that use them).  Consecutive MFMAs go to
+// accumulators stay in the matrix unit's registers); the LDS reads of the slice columns of
+// a k-group are issued before the MFMAs of the k-group ahead of it.  Consecutive MFMAs go to
 // different accumulators (two per output tile, alternating by k-group) so that none
 // waits for the result of the one before it.
 template <int RT, int CT, int CHUNK>
@@ -303,12 +305,19 @@ __device__ __forceinline__ void mfma_chunk(const float* w_lds, int g_abs,
   const int row = lane & 15;
   const int kq = lane >> 4;
   const float* wp0 = w_lds + ((g_abs * 4 + kq) * NCOLS + row) * 4;
+  float4_t bnext[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) bnext[ct] = *reinterpret_cast<const float4_t*>(wp0 + ct * 64);
 #pragma unroll
   for (int gi = 0; gi < CHUNK; ++gi) {
     float4_t b[CT];
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct)
-      b[ct] = *reinterpret_cast<const float4_t*>(wp0 + gi * 4 * NCOLS * 4 + ct * 64);
+    for (int ct = 0; ct < CT; ++ct) b[ct] = bnext[ct];
+    if (gi + 1 < CHUNK) {
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+        bnext[ct] = *reinterpret_cast<const float4_t*>(wp0 + (gi + 1) * 4 * NCOLS * 4 + ct * 64);
+    }
     float4_t (&acc)[RT][CT] = (gi & 1) ? acc1 : acc0;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
@@ -406,26 +415,261 @@ __device__ __forceinline__ void store_partials(float* red, const float4_t (&acc)
     }
 }
 
-// Sum over the four wavefronts of element (row, col) written by store_partials.
-template <int RT, int CT>
-__device__ __forceinline__ float sum_partials(const float* red, int row, int col) {
-  constexpr int NCOLS = 16 * CT;
-  constexpr int NB = 16 * RT;
-  const float* p = red + row * NCOLS + col;
-  return (p[0] + p[NB * NCOLS]) + (p[2 * NB * NCOLS] + p[3 * NB * NCOLS]);
+// ---- batch tiles of 4 or 8 rows ----------------------------------------------------
+// A 16x16x4 MFMA spends its full time on 16 rows however few are real.  Short tiles use
+// the 16-block 4x4x1 MFMA instead, with the A operand of one block broadcast to a group
+// of blocks (CBSZ/ABID): one instruction multiplies 4 batch rows by MC = 16, 32 or 64
+// slice columns for KS = 4, 2 or 1 values of k (lane group l/MC takes the k-th value),
+// so the matrix unit's time scales with the rows in steps of 4.
+
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+// f(std::integral_constant<int, i>) for i = 0 .. N-1, unrolled at compile time (MFMA
+// broadcast selectors must be immediates).
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+template <int CT>
+struct ShortTileShape {
+  static constexpr int NCOLS = 16 * CT;
+  static constexpr int CBSZ = NCOLS % 64 == 0 ? 4 : (NCOLS % 32 == 0 ? 3 : 2);
+  static constexpr int NBC = 1 << CBSZ;   // 4-column blocks sharing one A block
+  static constexpr int MC = 4 * NBC;      // slice columns per MFMA
+  static constexpr int KS = 16 / NBC;     // k values per MFMA = partial sums per wavefront
+  static constexpr int CTN = NCOLS / MC;  // MFMAs side by side to cover the slice columns
+};
+
+// A operands of CH "super-groups" of 64 consecutive k (super-group s covers k in
+// [64 s, 64 s + 64)); the wavefront takes super-groups s0, s0 + 4, ...  Lane l holds row
+// 4*rb + l%4 and k = 64 s + 4*(l/4) .. +3, so MFMA (j, abid) of lane group g multiplies
+// k = 64 s + 4*(g*NBC + abid) + j.
+template <int RB, int CH>
+__device__ __forceinline__ void load_a_rows4(const float* __restrict__ a, int a_ld, int rows_valid,
+                                             int K, int s0, int s_end, bool vec_ok, bool cached,
+                                             float4_t (&av)[CH][RB]) {
+  const int lane = threadIdx.x & 63;
+  const int r = lane & 3;
+  const int kb = (lane >> 2) * 4;
+  const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+  if (vec_ok && cached) {
+#pragma unroll
+    for (int ci = 0; ci < CH; ++ci) {
+      const int s = s0 + 4 * ci;
+      const int k = 64 * s + kb;
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const int rr = 4 * rb + r;
+        const bool ok = s < s_end && rr < rows_valid && k < K;
+        const float* src = a + (ok ? (size_t)rr * a_ld + k : (size_t)0);
+        const float4_t v = *reinterpret_cast<const float4_t*>(src);
+        av[ci][rb] = ok ? v : zero4;
+      }
+    }
+  } else if (vec_ok) {
+#pragma unroll
+    for (int ci = 0; ci < CH; ++ci) {
+      const int s = s0 + 4 * ci;
+      const int k = 64 * s + kb;
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const int rr = 4 * rb + r;
+        const bool ok = s < s_end && rr < rows_valid && k < K;
+        const float* src = a + (ok ? (size_t)rr * a_ld + k : (size_t)0);
+        const float4_t v = load_exchanged4(src);
+        av[ci][rb] = ok ? v : zero4;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int ci = 0; ci < CH; ++ci) {
+      const int s = s0 + 4 * ci;
+      const int k = 64 * s + kb;
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const int rr = 4 * rb + r;
+        const int valid = (s < s_end && rr < rows_valid) ? (K - k) : 0;
+        av[ci][rb] = load_a4(a + (size_t)rr * a_ld + k, valid, false);
+      }
+    }
+  }
+}
+
+// MFMAs of super-group s.  One 16-byte LDS read per (abid, column tile) feeds 4*RB MFMAs;
+// the read for abid+1 is issued before the MFMAs of abid.  Consecutive MFMAs on one
+// output tile alternate between two accumulators.
+template <int RB, int CT>
+__device__ __forceinline__ void mfma_rows4(const float* w_lds, int s, const float4_t (&av)[RB],
+                                           float4_t (&acc0)[RB][ShortTileShape<CT>::CTN],
+                                           float4_t (&acc1)[RB][ShortTileShape<CT>::CTN]) {
+  using S = ShortTileShape<CT>;
+  const int lane = threadIdx.x & 63;
+  const float* wp =
+      w_lds + ((16 * s + (lane / S::MC) * S::NBC) * S::NCOLS + lane % S::MC) * 4;
+  float4_t bnext[S::CTN];
+#pragma unroll
+  for (int ct = 0; ct < S::CTN; ++ct)
+    bnext[ct] = *reinterpret_cast<const float4_t*>(wp + ct * S::MC * 4);
+  static_for<S::NBC>([&](auto ac) {
+    constexpr int A = decltype(ac)::value;
+    float4_t b[S::CTN];
+#pragma unroll
+    for (int ct = 0; ct < S::CTN; ++ct) b[ct] = bnext[ct];
+    if constexpr (A + 1 < S::NBC) {
+#pragma unroll
+      for (int ct = 0; ct < S::CTN; ++ct)
+        bnext[ct] = *reinterpret_cast<const float4_t*>(wp + ((A + 1) * S::NCOLS + ct * S::MC) * 4);
+    }
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int ct = 0; ct < S::CTN; ++ct)
+        acc0[rb][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(av[rb].x, b[ct].x, acc0[rb][ct], S::CBSZ, A, 0);
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int ct = 0; ct < S::CTN; ++ct)
+        acc1[rb][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(av[rb].y, b[ct].y, acc1[rb][ct], S::CBSZ, A, 0);
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int ct = 0; ct < S::CTN; ++ct)
+        acc0[rb][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(av[rb].z, b[ct].z, acc0[rb][ct], S::CBSZ, A, 0);
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int ct = 0; ct < S::CTN; ++ct)
+        acc1[rb][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(av[rb].w, b[ct].w, acc1[rb][ct], S::CBSZ, A, 0);
+  });
+}
+
+// Product of a short tile: red[wave*KS + g][4*RB][16*CT] <- this wavefront's partial
+// tile of lane group g.  Accumulator element r of acc[rb][ct] in lane l is row 4*rb + r,
+// column ct*MC + l%MC, partial g = l/MC.
+template <int RB, int CT, int CH>
+__device__ __forceinline__ void short_tile_product(const float* __restrict__ a, int a_ld,
+                                                   int rows_valid, int K, int Kpad,
+                                                   const float* w_lds, bool vec_ok, bool cached,
+                                                   float* red) {
+  using S = ShortTileShape<CT>;
+  constexpr int NB = 4 * RB;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int s_end = Kpad >> 6;
+  const int mine = (s_end - wave + 3) >> 2;  // super-groups wave, wave+4, ...
+  const int full = mine / CH;
+  float4_t acc0[RB][S::CTN], acc1[RB][S::CTN];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int ct = 0; ct < S::CTN; ++ct) acc0[rb][ct] = acc1[rb][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  int s = wave;
+  if (full > 0) {
+    float4_t cur[CH][RB], nxt[CH][RB];
+    load_a_rows4<RB, CH>(a, a_ld, rows_valid, K, s, s_end, vec_ok, cached, cur);
+    for (int c = 0; c < full; ++c) {
+      if (c + 1 < full)
+        load_a_rows4<RB, CH>(a, a_ld, rows_valid, K, s + 4 * CH, s_end, vec_ok, cached, nxt);
+#pragma unroll
+      for (int ci = 0; ci < CH; ++ci) mfma_rows4<RB, CT>(w_lds, s + 4 * ci, cur[ci], acc0, acc1);
+#pragma unroll
+      for (int ci = 0; ci < CH; ++ci)
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) cur[ci][rb] = nxt[ci][rb];
+      s += 4 * CH;
+    }
+  }
+  for (; s < s_end; s += 4) {
+    float4_t one[1][RB];
+    load_a_rows4<RB, 1>(a, a_ld, rows_valid, K, s, s_end, vec_ok, cached, one);
+    mfma_rows4<RB, CT>(w_lds, s, one[0], acc0, acc1);
+  }
+
+  float* base = red + ((wave * S::KS + lane / S::MC) * NB) * S::NCOLS + lane % S::MC;
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int ct = 0; ct < S::CTN; ++ct) {
+      const float4_t v = acc0[rb][ct] + acc1[rb][ct];
+      float* q = base + (4 * rb) * S::NCOLS + ct * S::MC;
+      q[0] = v.x;
+      q[S::NCOLS] = v.y;
+      q[2 * S::NCOLS] = v.z;
+      q[3 * S::NCOLS] = v.w;
+    }
+}
+
+// ---- the product of one step, for any tile height ------------------------------------
+// NB batch rows (4, 8, or a multiple of 16) by 16*CT slice columns.  kPartials partial
+// tiles of [NB][16*CT] floats are left in `red`; sum_product adds them in a fixed order.
+template <int NB, int CT>
+struct ProductTile {
+  static_assert(NB == 4 || NB == 8 || NB % 16 == 0, "unsupported tile height");
+  static constexpr bool kShort = NB < 16;
+  static constexpr int NCOLS = 16 * CT;
+  static constexpr int kPartials = kShort ? 4 * ShortTileShape<CT>::KS : 4;
+  static constexpr int kRedFloats = kPartials * NB * NCOLS;
+};
+
+// red <- partial tiles of A[NB rows, K] * slice[K, 16*CT].  `a` points at row 0 of the
+// batch tile (row stride a_ld floats, K contiguous); rows >= rows_valid and k >= K read
+// as zero.  `cached`: the tile may be read with ordinary loads (same-XCD group, L1
+// invalidated after the barrier); otherwise agent-scope loads are used.  `vec_ok`: rows
+// are 16-byte aligned and K is a multiple of 4.  LONG_K selects deeper prefetch for
+// contractions much longer than the hidden size (the backward passes).
+template <int NB, int CT, bool LONG_K>
+__device__ __forceinline__ void slice_product(const float* __restrict__ a, int a_ld, int rows_valid,
+                                              int K, int Kpad, const float* w_lds, bool vec_ok,
+                                              bool cached, float* red) {
+  if constexpr (ProductTile<NB, CT>::kShort) {
+    short_tile_product<NB / 4, CT, LONG_K ? 8 : 2>(a, a_ld, rows_valid, K, Kpad, w_lds, vec_ok,
+                                                   cached, red);
+  } else {
+    constexpr int RT = NB / 16;
+    constexpr int CHUNK = LONG_K ? (RT == 1 ? 8 : (RT == 2 ? 4 : 2)) : (RT >= 4 ? 2 : 4);
+    float4_t acc[RT][CT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
+    slice_matmul<RT, CT, CHUNK>(a, a_ld, rows_valid, K, Kpad, w_lds, vec_ok, cached, acc);
+    store_partials<RT, CT>(red, acc);
+  }
+}
+
+// Element (row, col) of the product: the partial tiles written by slice_product, added
+// pairwise in a fixed order.
+template <int NB, int CT>
+__device__ __forceinline__ float sum_product(const float* red, int row, int col) {
+  using P = ProductTile<NB, CT>;
+  constexpr int STRIDE = NB * P::NCOLS;
+  const float* p = red + row * P::NCOLS + col;
+  float v[P::kPartials];
+#pragma unroll
+  for (int i = 0; i < P::kPartials; ++i) v[i] = p[i * STRIDE];
+#pragma unroll
+  for (int w = P::kPartials / 2; w > 0; w >>= 1)
+#pragma unroll
+    for (int i = 0; i < w; ++i) v[i] = v[2 * i] + v[2 * i + 1];
+  return v[0];
 }
 
 // ---- host side ---------------------------------------------------------------------
-// LDS bytes of a forward kernel (slice [Kpad x 16*CT] + 4 wavefront partial tiles).
-inline size_t fwd_lds_bytes(int H, int RT, int CT) {
-  const int Kpad = (H + 63) / 64 * 64;
-  return ((size_t)Kpad * 16 * CT + 4 * 16 * RT * 16 * CT) * sizeof(float);
+// Partial tiles slice_product leaves in LDS (ProductTile<nb, ct>::kPartials).
+inline int product_partials(int nb, int ct) {
+  if (nb >= 16) return 4;
+  const int ncols = 16 * ct;
+  return ncols % 64 == 0 ? 4 : (ncols % 32 == 0 ? 8 : 16);
 }
 
-inline size_t bwd_lds_bytes(int K, int RT) {
-  const int Kpad = (K + 63) / 64 * 64;
-  const size_t red = (size_t)4 * 16 * RT * 16;
-  return ((size_t)Kpad * 16 + red) * sizeof(float);
+// LDS bytes of a forward kernel (slice [Kpad x 16*ct] + the partial tiles of nb rows).
+inline size_t fwd_lds_bytes(int H, int nb, int ct) {
+  const int Kpad = (H + 63) / 64 * 64;
+  return ((size_t)Kpad * 16 * ct + (size_t)product_partials(nb, ct) * nb * 16 * ct) * sizeof(float);
 }
 
 // Host-side plan of a persistent launch: fills `shape` and the grid for (gx, gy).
@@ -502,15 +746,18 @@ int launch_persistent(const char* name, KernelT kernel, const LaunchPlan& plan, 
 
 constexpr size_t kMaxLdsBytes = 160 * 1024;  // LDS per workgroup on gfx950
 
-// Geometry of a forward recurrence: 16*rt batch rows and hs hidden units per workgroup
-// (their gate columns fill ct MFMA column tiles), gx column workgroups, gy batch tiles.
+// Geometry of a forward recurrence: nb batch rows and hs hidden units per workgroup
+// (their gate columns fill ct 16-column tiles), gx column workgroups, gy batch tiles.
 struct ForwardTile {
-  int rt, ct, hs, gx, gy, tile_rows;
+  int nb, ct, hs, gx, gy;
   size_t lds_bytes;
   bool ok;
 };
 
-// Prefers a geometry whose groups each fit on one XCD (most workgroups first), else the
+constexpr int kTileHeights[] = {4, 8, 16, 32, 64};
+
+// Prefers a geometry whose groups each fit on one XCD (shortest tiles first, which
+// spreads a small batch over the most XCDs; then the most column workgroups), else the
 // cross-XCD geometry with the most parallelism that fits the chip.  `extra_lds_per_row` is
 // what the cell needs in LDS per batch row beyond the slice and the partial tiles.
 inline ForwardTile pick_forward_tile(int gates, int N, int H, size_t extra_lds_per_row) {
@@ -520,22 +767,15 @@ inline ForwardTile pick_forward_tile(int gates, int N, int H, size_t extra_lds_p
   for (int pass = 0; pass < 2 && !best.ok; ++pass) {
     const int hs_order_local[] = {4, 8, 16};
     const int hs_order_cross[] = {8, 16, 4};
-    for (int rt : {1, 2, 4}) {
+    for (int nb : kTileHeights) {
       for (int i = 0; i < 3 && !best.ok; ++i) {
         const int hs = pass == 0 ? hs_order_local[i] : hs_order_cross[i];
         const int ct = (gates * hs + 15) / 16;
-        const int NB = 16 * rt;
-        const int gx = (H + hs - 1) / hs, gy = (N + NB - 1) / NB;
-        const size_t lds = fwd_lds_bytes(H, rt, ct) + extra_lds_per_row * NB;
+        const int gx = (H + hs - 1) / hs, gy = (N + nb - 1) / nb;
+        const size_t lds = fwd_lds_bytes(H, nb, ct) + extra_lds_per_row * nb;
         if (lds > kMaxLdsBytes || gy > kMaxGroups || gx * gy > kMaxWorkgroups) continue;
         if (pass == 0 ? !xcd_local_fits(gx, gy) : (long long)gx * gy > cus) continue;
-        best = ForwardTile{rt, ct, hs, gx, gy, NB, lds, true};
-        // Half-height tiles put a small batch on twice as many XCDs: the MFMA count per
-        // workgroup is unchanged, the exchanged rows each one reads are halved.
-        if (pass == 0 && rt == 1 && xcd_local_fits(gx, (N + 7) / 8)) {
-          best.tile_rows = 8;
-          best.gy = (N + 7) / 8;
-        }
+        best = ForwardTile{nb, ct, hs, gx, gy, lds, true};
       }
       if (best.ok) break;
     }
@@ -543,38 +783,36 @@ inline ForwardTile pick_forward_tile(int gates, int N, int H, size_t extra_lds_p
   return best;
 }
 
-// Geometry of a backward recurrence: 16 hidden units and 16*rt batch rows per workgroup.
+// Geometry of a backward recurrence: 16 hidden units and nb batch rows per workgroup.
 struct BackwardTile {
-  int rt, gx, gy, tile_rows;
+  int nb, gx, gy;
   size_t lds_bytes;
   bool ok;
 };
 
-// K = gates*H is the contraction length; `extra_floats_per_row` is the LDS the cell needs
-// per batch row beyond the slice (at least the 4 partial tiles = 64 floats).
-inline BackwardTile pick_backward_tile(int K, int N, int H, size_t extra_floats_per_row) {
+// K = gates*H is the contraction length.  Per batch row the kernel needs, beyond the
+// slice, max(`reduce_floats_per_row`, the partial tiles) + `extra_floats_per_row` floats.
+inline BackwardTile pick_backward_tile(int K, int N, int H, size_t reduce_floats_per_row,
+                                       size_t extra_floats_per_row) {
   const int cus = device_cu_count();
   const int gx = (H + 15) / 16;
   const int Kpad = (K + 63) / 64 * 64;
   BackwardTile best;
   best.ok = false;
   for (int pass = 0; pass < 2 && !best.ok; ++pass) {
-    for (int rt : {1, 2, 4}) {
-      const int NB = 16 * rt;
-      const int gy = (N + NB - 1) / NB;
-      const size_t lds = ((size_t)Kpad * 16 + extra_floats_per_row * NB) * sizeof(float);
+    for (int nb : kTileHeights) {
+      const int gy = (N + nb - 1) / nb;
+      size_t per_row = (size_t)product_partials(nb, 1) * 16;
+      if (per_row < reduce_floats_per_row) per_row = reduce_floats_per_row;
+      per_row += extra_floats_per_row;
+      const size_t lds = ((size_t)Kpad * 16 + per_row * nb) * sizeof(float);
       if (lds > kMaxLdsBytes || gy > kMaxGroups || gx * gy > kMaxWorkgroups) continue;
       if (pass == 0 ? !xcd_local_fits(gx, gy) : (long long)gx * gy > cus) continue;
-      best = BackwardTile{rt, gx, gy, NB, lds, true};
-      if (pass == 0 && rt == 1 && xcd_local_fits(gx, (N + 7) / 8)) {
-        best.tile_rows = 8;
-        best.gy = (N + 7) / 8;
-      }
+      best = BackwardTile{nb, gx, gy, lds, true};
       break;
     }
   }
   return best;
 }
-
 
 }  // namespace haste_hip
