@@ -22,6 +22,7 @@ struct GruFwdParams {
   const float* zoneout_mask;
   const float* dc_mask;  // DropConnect mask [H,3H] or null
   float dc_scale;
+  float* xh;             // exchange tiles of h: [batch tiles][2][Kpad/4][NB][4]
   LaunchShape ls;
 };
 
@@ -50,8 +51,16 @@ void gru_forward_kernel(GruFwdParams p) {
   const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
 
+  const int tile_floats = Kpad * NB;
+  float* xh = p.xh + (size_t)role.bt * 2 * tile_floats;
+  const TileBuffer xhb = make_tile_buffer(xh, 2 * tile_floats);
+
   GroupSync gs;
   group_sync_init(gs, p.ls, role);
+
+  // Own k range of the exchange tiles (the last workgroup also owns the padding).
+  zero_tile_share(gs, xh, tile_floats, NB, j0 / 4,
+                  (role.cw == p.ls.gx - 1 ? Kpad - j0 : HS) / 4);
 
   for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
     const int k = idx / NCOLS, cidx = idx % NCOLS;
@@ -89,8 +98,10 @@ void gru_forward_kernel(GruFwdParams p) {
     }
   }
   const bool zoneout = p.zoneout_prob != 0.f && p.zoneout_mask != nullptr;
-  const bool vec_ok = (H % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.h) & 15u) == 0);
-  __syncthreads();
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp)
+    if (act[pp]) store_exchanged(gs, &xh[xchg_index(pj[pp], pl[pp], NB)], h_prev[pp]);
+  group_arrive(gs);  // h[0] is published; the slice is complete in LDS
 
   for (int t = 0; t < T; ++t) {
     float wx[PP][3], mk[PP];
@@ -106,12 +117,13 @@ void gru_forward_kernel(GruFwdParams p) {
         if (zoneout && p.training) mk[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
       }
     }
-    if (t > 0) group_wait(gs);
+    group_wait(gs);  // h[t] complete for this batch tile
 
-    slice_product<NB, CT, false>(p.h + (size_t)t * NH + (size_t)n0 * H, H, rows_here, H, Kpad, w_lds,
-                                 vec_ok, gs.same_xcd, red);
+    tile_product<NB, CT, false>(xhb, (t & 1) * tile_floats, Kpad, w_lds, red);
     __syncthreads();
 
+    float saved[PP][4];  // z, r, g, q of the step for the caller's cache
+    float* xh_next = xh + ((t + 1) & 1) * tile_floats;
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
       if (act[pp]) {
@@ -122,23 +134,32 @@ void gru_forward_kernel(GruFwdParams p) {
         const float r = sigmoid_f(wx[pp][1] + rh[1] + bxv[pp][1] + brv[pp][1]);
         const float qg = rh[2] + brv[pp][2];
         const float g = tanhf(wx[pp][2] + r * qg + bxv[pp][2]);
-        if (p.training) {
-          float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
-          vt[0] = z;
-          vt[H] = r;
-          vt[2 * H] = g;
-          vt[3 * H] = qg;
-        }
+        saved[pp][0] = z;
+        saved[pp][1] = r;
+        saved[pp][2] = g;
+        saved[pp][3] = qg;
         float h_new = z * h_prev[pp] + (1.0f - z) * g;
         if (zoneout) {
           if (p.training) h_new = (h_new - h_prev[pp]) * mk[pp] + h_prev[pp];
           else h_new = p.zoneout_prob * h_prev[pp] + (1.0f - p.zoneout_prob) * h_new;
         }
-        store_exchanged(gs, &p.h[(size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp]], h_new);
+        if (t + 1 < T) store_exchanged(gs, &xh_next[xchg_index(pj[pp], pl[pp], NB)], h_new);
         h_prev[pp] = h_new;
       }
     }
-    if (t + 1 < T) group_arrive(gs);
+    if (t + 1 < T) group_arrive(gs);  // publishes h[t+1]; also fences `red` reuse
+    // The caller's copies are written behind the barrier: nobody in the launch waits for them.
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      if (act[pp]) {
+        if (p.training) {
+          float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+#pragma unroll
+          for (int g = 0; g < 4; ++g) vt[g * H] = saved[pp][g];
+        }
+        p.h[(size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp]] = h_prev[pp];
+      }
+    }
   }
 }
 
@@ -155,9 +176,18 @@ struct GruBwdParams {
   float* dq;            // [T,N,3H]
   const float* zoneout_mask;
   float* db_partial;    // [batch tiles, 6H] scratch
+  float* xdq;           // exchange tiles of dq: [batch tiles][2][Kpad/4][NB][4]
   LaunchShape ls;
 };
 
+// Contraction length of the backward recurrence inside the launch: k = 3*unit + gate over
+// the 16 units of every column workgroup, padded to the MFMA granularity.
+inline int gru_backward_k(int H) { return 48 * ((H + 15) / 16); }
+
+
+// A workgroup owns 16 hidden units for NB batch rows; its slice of R_t is [3H x 16].
+// Inside the launch the contraction index runs unit-major (k = 3*unit + gate), so every
+// workgroup publishes one contiguous k range of the exchange tile.
 template <int NB>
 __global__ __launch_bounds__(256, 1)
 void gru_backward_kernel(GruBwdParams p) {
@@ -171,8 +201,7 @@ void gru_backward_kernel(GruBwdParams p) {
   __shared__ unsigned int s_flag;
 
   const int H = p.H, N = p.N, T = p.T;
-  const int K = 3 * H;
-  const int Kpad = round_up(K, 64);
+  const int Kpad = round_up(48 * p.ls.gx, 64);
   float* w_lds = lds;
   float* red = lds + Kpad * NCOLS;  // the partial tiles or NB*6*16 floats, whichever is more
 
@@ -182,13 +211,23 @@ void gru_backward_kernel(GruBwdParams p) {
   const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
 
+  const int tile_floats = Kpad * NB;
+  float* xdq = p.xdq + (size_t)role.bt * 2 * tile_floats;
+  const TileBuffer xdqb = make_tile_buffer(xdq, 2 * tile_floats);
+
   GroupSync gs;
   group_sync_init(gs, p.ls, role);
 
+  // Own k range of the exchange tiles (the last workgroup also owns the padding); only
+  // rows and units of the problem are written afterwards.
+  zero_tile_share(gs, xdq, tile_floats, NB, 12 * role.cw,
+                  (role.cw == p.ls.gx - 1 ? Kpad - 48 * role.cw : 48) / 4);
+
   for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
     const int k = idx / NCOLS, cidx = idx % NCOLS;
+    const int unit = k / 3, gate = k % 3;
     float w = 0.f;
-    if (k < K && j0 + cidx < H) w = p.R_t[(size_t)k * H + j0 + cidx];
+    if (unit < H && j0 + cidx < H) w = p.R_t[((size_t)gate * H + unit) * H + j0 + cidx];
     w_lds[slice_index(k, cidx, NCOLS)] = w;
   }
 
@@ -208,7 +247,6 @@ void gru_backward_kernel(GruBwdParams p) {
     for (int g = 0; g < 6; ++g) dbacc[pp][g] = 0.f;
   }
   const bool zoneout = p.zoneout_mask != nullptr;
-  const bool vec_ok = (reinterpret_cast<uintptr_t>(p.dq) & 15u) == 0 && (K % 4 == 0);
   __syncthreads();
 
   struct StepIn { float vt[4], h0, dhn, m; };
@@ -232,7 +270,8 @@ void gru_backward_kernel(GruBwdParams p) {
   fetch(T - 1);
 
   for (int t = T - 1; t >= 0; --t) {
-    float dh_keep[PP];
+    float dh_keep[PP], dpv[PP][3], dqv[PP];
+    float* xdq_t = xdq + (t & 1) * tile_floats;
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
       dh_keep[pp] = 0.f;
@@ -254,13 +293,14 @@ void gru_backward_kernel(GruBwdParams p) {
         const float dr = dp_g * qg;
         const float dp_r = d_sigmoid_f(r) * dr;
         const float dp_z = d_sigmoid_f(z) * dz;
-        const size_t o3 = ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
-        p.dp[o3] = dp_z;
-        p.dp[o3 + H] = dp_r;
-        p.dp[o3 + 2 * H] = dp_g;
-        store_exchanged(gs, &p.dq[o3], dp_z);
-        store_exchanged(gs, &p.dq[o3 + H], dp_r);
-        store_exchanged(gs, &p.dq[o3 + 2 * H], dq_g);
+        float* xq = xdq_t + xchg_index(3 * pj[pp], pl[pp], NB);
+        store_exchanged(gs, xq, dp_z);
+        store_exchanged(gs, xdq_t + xchg_index(3 * pj[pp] + 1, pl[pp], NB), dp_r);
+        store_exchanged(gs, xdq_t + xchg_index(3 * pj[pp] + 2, pl[pp], NB), dq_g);
+        dpv[pp][0] = dp_z;
+        dpv[pp][1] = dp_r;
+        dpv[pp][2] = dp_g;
+        dqv[pp] = dq_g;
         dbacc[pp][0] += dp_z;
         dbacc[pp][1] += dp_r;
         dbacc[pp][2] += dp_g;
@@ -269,12 +309,24 @@ void gru_backward_kernel(GruBwdParams p) {
         dbacc[pp][5] += dq_g;
       }
     }
-    group_arrive(gs);
+    group_arrive(gs);  // dq_t of this workgroup's units is published
+    // The caller's copies are written behind the barrier: nobody in the launch waits for them.
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      if (act[pp]) {
+        const size_t o3 = ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
+        p.dp[o3] = dpv[pp][0];
+        p.dp[o3 + H] = dpv[pp][1];
+        p.dp[o3 + 2 * H] = dpv[pp][2];
+        p.dq[o3] = dpv[pp][0];
+        p.dq[o3 + H] = dpv[pp][1];
+        p.dq[o3 + 2 * H] = dqv[pp];
+      }
+    }
     fetch(t - 1);
-    group_wait(gs);
+    group_wait(gs);    // dq_t of every unit is complete for this batch tile
 
-    slice_product<NB, 1, true>(p.dq + ((size_t)t * N + n0) * 3 * H, 3 * H, rows_here, K, Kpad, w_lds,
-                               vec_ok, gs.same_xcd, red);
+    tile_product<NB, 1, true>(xdqb, (t & 1) * tile_floats, Kpad, w_lds, red);
     __syncthreads();
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp)
@@ -318,18 +370,21 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
   HASTE_HIP_REQUIRE(W && R && bx && br && x && h && tmp_Wx);
   HASTE_HIP_REQUIRE(!training || v != nullptr);
-  Workspace ws;
-  HASTE_HIP_PROPAGATE(get_workspace(stream, 0, &ws));
-  HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
+  const ForwardTile tile = pick_forward_tile(3, N, H, 0);
+  if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 3 * H, C, x, C, W, 3 * H, tmp_Wx, 3 * H, false));
+
+  // Taken after the GEMM, which may replace the stream's scratch buffer with a larger one.
+  Workspace ws;
+  HASTE_HIP_PROPAGATE(get_workspace(stream, exchange_floats(H, tile.nb, tile.gy) * sizeof(float), &ws));
+  HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 
   GruFwdParams p;
   p.training = training; p.T = T; p.N = N; p.H = H;
   p.R = R; p.bx = bx; p.br = br; p.h = h; p.v = v; p.Wx = tmp_Wx;
   p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
   p.dc_mask = dc_mask; p.dc_scale = dc_scale;
-  const ForwardTile tile = pick_forward_tile(3, N, H, 0);
-  if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  p.xh = ws.scratch;
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.nb, tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;
@@ -355,11 +410,13 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && v && dh_new);
   HASTE_HIP_REQUIRE(dx && dW && dR && dbx && dbr && dh && dp && dq);
   // per row: the partial tiles or the 6 bias-gradient columns of 16 floats
-  const BackwardTile tile = pick_backward_tile(3 * H, N, H, 6 * 16, 0);
+  const BackwardTile tile = pick_backward_tile(gru_backward_k(H), N, H, 6 * 16, 0);
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 
   Workspace ws;
-  HASTE_HIP_PROPAGATE(get_workspace(stream, (size_t)tile.gy * 6 * H * sizeof(float), &ws));
+  const size_t db_floats = ((size_t)tile.gy * 6 * H + 3) / 4 * 4;
+  const size_t xdq_floats = exchange_floats(gru_backward_k(H), tile.nb, tile.gy);
+  HASTE_HIP_PROPAGATE(get_workspace(stream, (db_floats + xdq_floats) * sizeof(float), &ws));
   HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 
   GruBwdParams p;
@@ -367,6 +424,7 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   p.R_t = R_t; p.h = h; p.v = v; p.dh_new = dh_new;
   p.dbx = dbx; p.dbr = dbr; p.dh = dh; p.dp = dp; p.dq = dq; p.zoneout_mask = zoneout_mask;
   p.db_partial = ws.scratch;
+  p.xdq = ws.scratch + db_floats;
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.nb, tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;

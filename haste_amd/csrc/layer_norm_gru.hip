@@ -26,6 +26,7 @@ struct LnGruFwdParams {
   float zoneout_prob;
   const float* zoneout_mask;
   float* part2;          // exchange [groups][gx][NB][2]
+  float* xh;             // exchange tiles of h: [batch tiles][2][Kpad/4][NB][4]
   LaunchShape ls;
 };
 
@@ -57,8 +58,15 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
   const int last_units = H - (gx - 1) * HS;
   float* part2 = p.part2 + (size_t)role.bt * gx * NB * 2;
 
+  const int tile_floats = Kpad * NB;
+  float* xh = p.xh + (size_t)role.bt * 2 * tile_floats;
+  const TileBuffer xhb = make_tile_buffer(xh, 2 * tile_floats);
+
   GroupSync gs;
   group_sync_init(gs, p.ls, role);
+
+  // Own k range of the exchange tiles (the last workgroup also owns the padding).
+  zero_tile_share(gs, xh, tile_floats, NB, j0 / 4, (role.cw == gx - 1 ? Kpad - j0 : HS) / 4);
 
   for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
     const int k = idx / NCOLS, cidx = idx % NCOLS;
@@ -89,8 +97,10 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
     }
   }
   const bool zoneout = p.zoneout_prob != 0.f && p.zoneout_mask != nullptr;
-  const bool vec_ok = (H % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.h) & 15u) == 0);
-  __syncthreads();
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp)
+    if (act[pp]) store_exchanged(gs, &xh[xchg_index(pj[pp], pl[pp], NB)], h_prev[pp]);
+  group_arrive(gs);  // h[0] is published; the slice is complete in LDS
 
   for (int t = 0; t < T; ++t) {
     float wx[PP][3], mk[PP];
@@ -106,10 +116,9 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
         if (zoneout && p.training) mk[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
       }
     }
-    if (t > 0) group_wait(gs);
+    group_wait(gs);  // h[t]
 
-    slice_product<NB, CT, false>(p.h + (size_t)t * NH + (size_t)n0 * H, H, rows_here, H, Kpad, w_lds,
-                                 vec_ok, gs.same_xcd, red);
+    tile_product<NB, CT, false>(xhb, (t & 1) * tile_floats, Kpad, w_lds, red);
     __syncthreads();
 
     float rh[PP][3];
@@ -165,7 +174,9 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
           if (p.training) h_new = (h_new - h_prev[pp]) * mk[pp] + h_prev[pp];
           else h_new = p.zoneout_prob * h_prev[pp] + (1.0f - p.zoneout_prob) * h_new;
         }
-        store_exchanged(gs, &p.h[(size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp]], h_new);
+        p.h[(size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp]] = h_new;
+        if (t + 1 < T)
+          store_exchanged(gs, &xh[((t + 1) & 1) * tile_floats + xchg_index(pj[pp], pl[pp], NB)], h_new);
         h_prev[pp] = h_new;
         if (role.cw == 0 && pc[pp] == 0 && p.cache2 != nullptr) {
           p.cache2[((size_t)t * N + pn[pp]) * 2 + 0] = mu;
@@ -196,8 +207,14 @@ struct LnGruBwdParams {
   const float* zoneout_mask;
   float* part;           // exchange [groups][gx][NB][4]
   float* col_partial;    // [batch tiles][9][H]
+  float* xdq;            // exchange tiles of dq: [batch tiles][2][Kpad/4][NB][4]
   LaunchShape ls;
 };
+
+// Contraction length of the backward recurrence inside the launch: k = 3*unit + gate over
+// the 16 units of every column workgroup.
+inline int ln_gru_backward_k(int H) { return 48 * ((H + 15) / 16); }
+
 
 template <int NB>
 __global__ __launch_bounds__(256, 1)
@@ -215,8 +232,7 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
   __shared__ unsigned int s_flag;
 
   const int H = p.H, N = p.N, T = p.T;
-  const int K = 3 * H;
-  const int Kpad = round_up(K, 64);
+  const int Kpad = round_up(48 * p.ls.gx, 64);
   float* w_lds = lds;
   float* red = lds + Kpad * NCOLS;  // the partial tiles, reused for the column sums
   float* sums = red + RED;           // [NB][4]
@@ -229,13 +245,23 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
   const size_t NH = (size_t)N * H;
   float* part = p.part + (size_t)role.bt * gx * NB * 4;
 
+  const int tile_floats = Kpad * NB;
+  float* xdq = p.xdq + (size_t)role.bt * 2 * tile_floats;
+  const TileBuffer xdqb = make_tile_buffer(xdq, 2 * tile_floats);
+
   GroupSync gs;
   group_sync_init(gs, p.ls, role);
 
+  // Own k range of the exchange tiles (the last workgroup also owns the padding); only
+  // rows and units of the problem are written afterwards.
+  zero_tile_share(gs, xdq, tile_floats, NB, 12 * role.cw,
+                  (role.cw == gx - 1 ? Kpad - 48 * role.cw : 48) / 4);
+
   for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
     const int k = idx / NCOLS, cidx = idx % NCOLS;
+    const int unit = k / 3, gate = k % 3;
     float w = 0.f;
-    if (k < K && j0 + cidx < H) w = p.R_t[(size_t)k * H + j0 + cidx];
+    if (unit < H && j0 + cidx < H) w = p.R_t[((size_t)gate * H + unit) * H + j0 + cidx];
     w_lds[slice_index(k, cidx, NCOLS)] = w;
   }
 
@@ -258,7 +284,6 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
     for (int a = 0; a < NACC; ++a) accs[pp][a] = 0.f;
   }
   const bool zoneout = p.zoneout_mask != nullptr;
-  const bool vec_ok = (reinterpret_cast<uintptr_t>(p.dq) & 15u) == 0 && (K % 4 == 0);
   __syncthreads();
 
   struct StepIn { float vt[4], rh[3], h0, dhn, m, mu2, is2; };
@@ -352,17 +377,18 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
         const float dmu = (-2.0f * sums[pl[pp] * 4 + 1] * dsigma * inv3H) - (sums[pl[pp] * 4 + 2] * is2);
         float* dqt = p.dq + ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
 #pragma unroll
-        for (int k = 0; k < 3; ++k)
-          store_exchanged(gs, dqt + (size_t)k * H,
-                          (2.0f * xc[pp][k] * dsigma * inv3H) + (is2 * gd[pp][k]) + (dmu * inv3H));
+        for (int k = 0; k < 3; ++k) {
+          const float d = (2.0f * xc[pp][k] * dsigma * inv3H) + (is2 * gd[pp][k]) + (dmu * inv3H);
+          store_exchanged(gs, xdq + (t & 1) * tile_floats + xchg_index(3 * pj[pp] + k, pl[pp], NB), d);
+          dqt[(size_t)k * H] = d;
+        }
       }
     }
     group_arrive(gs);
     fetch(t - 1);
-    group_wait(gs);
+    group_wait(gs);  // dq_t of every unit is complete for this batch tile
 
-    slice_product<NB, 1, true>(p.dq + ((size_t)t * N + n0) * 3 * H, 3 * H, rows_here, K, Kpad, w_lds,
-                               vec_ok, gs.same_xcd, red);
+    tile_product<NB, 1, true>(xdqb, (t & 1) * tile_floats, Kpad, w_lds, red);
     __syncthreads();
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp)
@@ -426,12 +452,14 @@ int haste_hip_layer_norm_gru_forward_f32(int training, int steps, int batch_size
   const int NB = tile.nb;
   const size_t part_floats = (size_t)gy * gx * NB * 2;
 
-  Workspace ws;
-  HASTE_HIP_PROPAGATE(get_workspace(stream, part_floats * sizeof(float), &ws));
-  HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
-
   HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 3 * H, C, x, C, W, 3 * H, act_Wx, 3 * H, false));
   HASTE_HIP_PROPAGATE(layer_norm_forward(stream, T * N, 3 * H, gamma1, nullptr, act_Wx, tmp_Wx_norm, cache1));
+
+  // Taken after the GEMM, which may replace the stream's scratch buffer with a larger one.
+  Workspace ws;
+  const size_t xh_floats = exchange_floats(H, NB, gy);
+  HASTE_HIP_PROPAGATE(get_workspace(stream, (part_floats + xh_floats) * sizeof(float), &ws));
+  HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 
   LnGruFwdParams p;
   p.training = training; p.T = T; p.N = N; p.H = H;
@@ -439,6 +467,7 @@ int haste_hip_layer_norm_gru_forward_f32(int training, int steps, int batch_size
   p.gamma2 = gamma2; p.cache2 = cache2;
   p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
   p.part2 = ws.scratch;
+  p.xh = ws.scratch + part_floats;
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes, 2u * (unsigned)T + 1, &plan));
   p.ls = plan.shape;
@@ -474,15 +503,16 @@ int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_s
   HASTE_HIP_REQUIRE(dp && dq && act_Wx && gamma1 && dgamma1 && act_Rh && gamma2 && dgamma2 && cache2);
   hipStream_t stream = as_stream(stream_);
   // per row: 9 column-sum accumulators of 16 floats (or the partial tiles, whichever is more) + 4 sums
-  const BackwardTile tile = pick_backward_tile(3 * H, N, H, 9 * 16, 4);
+  const BackwardTile tile = pick_backward_tile(ln_gru_backward_k(H), N, H, 9 * 16, 4);
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const int gx = tile.gx, gy = tile.gy;
   const int NB = tile.nb;
   const size_t part_floats = (size_t)gy * gx * NB * 4;
-  const size_t col_floats = (size_t)gy * 9 * H;
+  const size_t col_floats = ((size_t)gy * 9 * H + 3) / 4 * 4;
+  const size_t xdq_floats = exchange_floats(ln_gru_backward_k(H), NB, gy);
 
   Workspace ws;
-  HASTE_HIP_PROPAGATE(get_workspace(stream, (part_floats + col_floats) * sizeof(float), &ws));
+  HASTE_HIP_PROPAGATE(get_workspace(stream, (part_floats + col_floats + xdq_floats) * sizeof(float), &ws));
   HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 
   LnGruBwdParams p;
@@ -492,6 +522,7 @@ int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_s
   p.act_Rh = act_Rh; p.gamma2 = gamma2; p.dgamma2 = dgamma2; p.cache2 = cache2;
   p.zoneout_mask = zoneout_mask;
   p.part = ws.scratch; p.col_partial = ws.scratch + part_floats;
+  p.xdq = ws.scratch + part_floats + col_floats;
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes, 2u * (unsigned)T + 1, &plan));
   p.ls = plan.shape;

@@ -34,6 +34,7 @@ struct LnLstmFwdParams {
   const float* zoneout_mask;
   float* part2;           // exchange [groups][gx][NB][2]
   float* part3;           // exchange [groups][gx][NB][2]
+  float* xh;              // exchange tiles of h: [batch tiles][2][Kpad/4][NB][4]
   LaunchShape ls;
 };
 
@@ -66,8 +67,15 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
   float* part2 = p.part2 + (size_t)role.bt * gx * NB * 2;
   float* part3 = p.part3 + (size_t)role.bt * gx * NB * 2;
 
+  const int tile_floats = Kpad * NB;
+  float* xh = p.xh + (size_t)role.bt * 2 * tile_floats;
+  const TileBuffer xhb = make_tile_buffer(xh, 2 * tile_floats);
+
   GroupSync gs;
   group_sync_init(gs, p.ls, role);
+
+  // Own k range of the exchange tiles (the last workgroup also owns the padding).
+  zero_tile_share(gs, xh, tile_floats, NB, j0 / 4, (role.cw == gx - 1 ? Kpad - j0 : HS) / 4);
 
   for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
     const int k = idx / NCOLS, cidx = idx % NCOLS;
@@ -107,8 +115,10 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
     }
   }
   const bool zoneout = p.zoneout_prob != 0.f && p.zoneout_mask != nullptr;
-  const bool vec_ok = (H % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.h) & 15u) == 0);
-  __syncthreads();
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp)
+    if (act[pp]) store_exchanged(gs, &xh[xchg_index(pj[pp], pl[pp], NB)], h_prev[pp]);
+  group_arrive(gs);  // h[0] is published; the slice is complete in LDS
 
   for (int t = 0; t < T; ++t) {
     float wx[PP][4], mk[PP];
@@ -124,10 +134,9 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
         if (zoneout && p.training) mk[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
       }
     }
-    if (t > 0) group_wait(gs);  // h[t]
+    group_wait(gs);  // h[t]
 
-    slice_product<NB, CT, false>(p.h + (size_t)t * NH + (size_t)n0 * H, H, rows_here, H, Kpad, w_lds,
-                                 vec_ok, gs.same_xcd, red);
+    tile_product<NB, CT, false>(xhb, (t & 1) * tile_floats, Kpad, w_lds, red);
     __syncthreads();
 
     // h*R of the owned columns; moments of those columns per row, published.
@@ -217,7 +226,9 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
           if (p.training) h_new = (h_new - h_prev[pp]) * mk[pp] + h_prev[pp];
           else h_new = p.zoneout_prob * h_prev[pp] + (1.0f - p.zoneout_prob) * h_new;
         }
-        store_exchanged(gs, &p.h[(size_t)(t + 1) * NH + e], h_new);
+        p.h[(size_t)(t + 1) * NH + e] = h_new;
+        if (t + 1 < T)
+          store_exchanged(gs, &xh[((t + 1) & 1) * tile_floats + xchg_index(pj[pp], pl[pp], NB)], h_new);
         h_prev[pp] = h_new;
         if (role.cw == 0 && pc[pp] == 0 && p.cache3 != nullptr) {
           p.cache3[((size_t)t * N + pn[pp]) * 2 + 0] = mu;
@@ -253,6 +264,7 @@ struct LnLstmBwdParams {
   float* part_a;           // exchange [groups][gx][NB][4]
   float* part_b;           // exchange [groups][gx][NB][4]
   float* col_partial;      // [batch tiles][10][H]
+  float* xd;               // exchange tiles of the gradient w.r.t. h*R: [batch tiles][2][Kpad/4][NB][4]
   LaunchShape ls;
 };
 
@@ -272,8 +284,7 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   __shared__ unsigned int s_flag;
 
   const int H = p.H, N = p.N, T = p.T;
-  const int K = 4 * H;
-  const int Kpad = round_up(K, 64);
+  const int Kpad = 64 * p.ls.gx;  // k = 4*unit + gate over the 16 units of every workgroup
   float* w_lds = lds;
   float* red = lds + Kpad * NCOLS;  // the partial tiles, reused for the column sums
   float* sums = red + RED;           // [NB][4]
@@ -287,13 +298,18 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   float* part_a = p.part_a + (size_t)role.bt * gx * NB * 4;
   float* part_b = p.part_b + (size_t)role.bt * gx * NB * 4;
 
+  const int tile_floats = Kpad * NB;
+  float* xd = p.xd + (size_t)role.bt * 2 * tile_floats;
+  const TileBuffer xdb = make_tile_buffer(xd, 2 * tile_floats);
+
   GroupSync gs;
   group_sync_init(gs, p.ls, role);
 
   for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
     const int k = idx / NCOLS, cidx = idx % NCOLS;
+    const int unit = k >> 2, gate = k & 3;
     float w = 0.f;
-    if (k < K && j0 + cidx < H) w = p.R_t[(size_t)k * H + j0 + cidx];
+    if (unit < H && j0 + cidx < H) w = p.R_t[((size_t)gate * H + unit) * H + j0 + cidx];
     w_lds[slice_index(k, cidx, NCOLS)] = w;
   }
 
@@ -318,7 +334,6 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
     for (int a = 0; a < NACC; ++a) accs[pp][a] = 0.f;
   }
   const bool zoneout = p.zoneout_mask != nullptr;
-  const bool vec_ok = (reinterpret_cast<uintptr_t>(p.act_Rh) & 15u) == 0;
   __syncthreads();
 
   struct StepIn { float vt[4], rh[4], c0, c1, dhn, dcn, m, cn, mu2, is2, mu3, is3; };
@@ -435,25 +450,38 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
     sum_row_partials<NB>(part_b, gx, sums);
     __syncthreads();
 
+    float dr[PP][4];
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) dr[pp][g] = 0.f;
       if (act[pp]) {
         const float is2 = s[pp].is2;
         const float dsigma = -0.5f * sums[pl[pp] * 4 + 0] * is2 * is2 * is2;
         const float dmu = (-2.0f * sums[pl[pp] * 4 + 1] * dsigma * inv4H) - (sums[pl[pp] * 4 + 2] * is2);
-        float* ar = p.act_Rh + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
 #pragma unroll
         for (int g = 0; g < 4; ++g)
-          store_exchanged(gs, ar + (size_t)g * H,
-                          (2.0f * xc2[pp][g] * dsigma * inv4H) + (is2 * gd2[pp][g]) + (dmu * inv4H));
+          dr[pp][g] = (2.0f * xc2[pp][g] * dsigma * inv4H) + (is2 * gd2[pp][g]) + (dmu * inv4H);
       }
+      // rows and units beyond the problem are published as zeros
+      if (own[pp])
+        store_exchanged4(gs, xd + (t & 1) * tile_floats + ((size_t)pj[pp] * NB + pl[pp]) * 4,
+                         dr[pp][0], dr[pp][1], dr[pp][2], dr[pp][3]);
     }
     group_arrive(gs);
+    // The caller's copy is written behind the barrier: nobody in the launch waits for it.
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      if (act[pp]) {
+        float* ar = p.act_Rh + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) ar[(size_t)g * H] = dr[pp][g];
+      }
+    }
     fetch(t - 1);
     group_wait(gs);  // gradient w.r.t. h*R complete for this batch tile
 
-    slice_product<NB, 1, true>(p.act_Rh + ((size_t)t * N + n0) * 4 * H, 4 * H, rows_here, K, Kpad,
-                               w_lds, vec_ok, gs.same_xcd, red);
+    tile_product<NB, 1, true>(xdb, (t & 1) * tile_floats, Kpad, w_lds, red);
     __syncthreads();
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp)
@@ -526,12 +554,14 @@ int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_siz
   const int NB = tile.nb;
   const size_t part_floats = (size_t)gy * gx * NB * 2;
 
-  Workspace ws;
-  HASTE_HIP_PROPAGATE(get_workspace(stream, 2 * part_floats * sizeof(float), &ws));
-  HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
-
   HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 4 * H, C, x, C, W, 4 * H, act_Wx, 4 * H, false));
   HASTE_HIP_PROPAGATE(layer_norm_forward(stream, T * N, 4 * H, gamma1, nullptr, act_Wx, act_Wx_norm, cache1));
+
+  // Taken after the GEMM, which may replace the stream's scratch buffer with a larger one.
+  Workspace ws;
+  const size_t xh_floats = exchange_floats(H, NB, gy);
+  HASTE_HIP_PROPAGATE(get_workspace(stream, (2 * part_floats + xh_floats) * sizeof(float), &ws));
+  HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 
   LnLstmFwdParams p;
   p.training = training; p.T = T; p.N = N; p.H = H;
@@ -539,6 +569,7 @@ int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_siz
   p.gamma2 = gamma2; p.cache2 = cache2; p.gamma_h = gamma_h; p.beta_h = beta_h; p.cache3 = cache3;
   p.act_c_norm = act_c_norm; p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
   p.part2 = ws.scratch; p.part3 = ws.scratch + part_floats;
+  p.xh = ws.scratch + 2 * part_floats;
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes, 3u * (unsigned)T + 1, &plan));
   p.ls = plan.shape;
@@ -587,9 +618,11 @@ int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_
   const int NB = tile.nb;
   const size_t part_floats = (size_t)gy * gx * NB * 4;
   const size_t col_floats = (size_t)gy * 10 * H;
+  const size_t col_floats4 = (col_floats + 3) / 4 * 4;
 
   Workspace ws;
-  HASTE_HIP_PROPAGATE(get_workspace(stream, (2 * part_floats + col_floats) * sizeof(float), &ws));
+  const size_t xd_floats = exchange_floats(64 * gx, NB, gy);
+  HASTE_HIP_PROPAGATE(get_workspace(stream, (2 * part_floats + col_floats4 + xd_floats) * sizeof(float), &ws));
   HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 
   LnLstmBwdParams p;
@@ -601,6 +634,7 @@ int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_
   p.act_c_norm = act_c_norm; p.zoneout_mask = zoneout_mask;
   p.part_a = ws.scratch; p.part_b = ws.scratch + part_floats;
   p.col_partial = ws.scratch + 2 * part_floats;
+  p.xd = ws.scratch + 2 * part_floats + col_floats4;
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes, 3u * (unsigned)T + 1, &plan));
   p.ls = plan.shape;

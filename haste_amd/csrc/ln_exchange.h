@@ -26,18 +26,6 @@ __device__ __forceinline__ float segment_sum(float v) {
   return v;
 }
 
-__device__ __forceinline__ void store_exchanged2(const GroupSync& g, float* p, float a, float b) {
-  if (g.same_xcd) {
-    p[0] = a;
-    p[1] = b;
-    return;
-  }
-  const unsigned long long bits =
-      (unsigned long long)__float_as_uint(a) | ((unsigned long long)__float_as_uint(b) << 32);
-  __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), bits, __ATOMIC_RELAXED,
-                     __HIP_MEMORY_SCOPE_AGENT);
-}
-
 __device__ __forceinline__ void load_exchanged2(const float* p, float& a, float& b) {
   const unsigned long long bits = __hip_atomic_load(
       reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -118,12 +106,6 @@ __device__ __forceinline__ void sum_row_partials(const float* part, int gx, floa
       out[row * 4 + 2] = s2;
     }
   }
-}
-
-__device__ __forceinline__ void store_exchanged4(const GroupSync& g, float* p, float a, float b,
-                                                 float c, float d) {
-  store_exchanged2(g, p, a, b);
-  store_exchanged2(g, p + 2, c, d);
 }
 
 }  // namespace haste_hip

@@ -21,6 +21,7 @@ struct LstmFwdParams {
   const float* zoneout_mask;   // [T,N,H] or null
   const float* dc_mask;        // DropConnect mask [H,4H] or null
   float dc_scale;
+  float* xh;                   // exchange tiles of h: [batch tiles][2][Kpad/4][NB][4]
   LaunchShape ls;
 };
 
@@ -48,8 +49,17 @@ void lstm_forward_kernel(LstmFwdParams p) {
   const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
 
+  const int tile_floats = Kpad * NB;
+  float* xh = p.xh + (size_t)role.bt * 2 * tile_floats;
+
+  const TileBuffer xhb = make_tile_buffer(xh, 2 * tile_floats);
+
   GroupSync gs;
   group_sync_init(gs, p.ls, role);
+
+  // Own k range of the exchange tiles (the last workgroup also owns the padding).
+  zero_tile_share(gs, xh, tile_floats, NB, j0 / 4,
+                  (role.cw == p.ls.gx - 1 ? Kpad - j0 : HS) / 4);
 
   // Resident slice: column c of the slice is gate c/HS, hidden unit j0 + c%HS.
   for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
@@ -88,8 +98,10 @@ void lstm_forward_kernel(LstmFwdParams p) {
     }
   }
   const bool zoneout = p.zoneout_prob != 0.f && p.zoneout_mask != nullptr;
-  const bool vec_ok = (H % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.h) & 15u) == 0);
-  __syncthreads();
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp)
+    if (act[pp]) store_exchanged(gs, &xh[xchg_index(pj[pp], pl[pp], NB)], h_prev[pp]);
+  group_arrive(gs);  // h[0] is published; the slice is complete in LDS
 
   for (int t = 0; t < T; ++t) {
     // Inputs of this step that do not depend on the recurrence: issue before waiting.
@@ -106,12 +118,13 @@ void lstm_forward_kernel(LstmFwdParams p) {
         if (zoneout && p.training) mk[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
       }
     }
-    if (t > 0) group_wait(gs);  // h[t] complete for this batch tile
+    group_wait(gs);  // h[t] complete for this batch tile
 
-    slice_product<NB, CT, false>(p.h + (size_t)t * NH + (size_t)n0 * H, H, rows_here, H, Kpad, w_lds,
-                                 vec_ok, gs.same_xcd, red);
+    tile_product<NB, CT, false>(xhb, (t & 1) * tile_floats, Kpad, w_lds, red);
     __syncthreads();
 
+    float gate[PP][4];
+    float* xh_next = xh + ((t + 1) & 1) * tile_floats;
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
       if (act[pp]) {
@@ -119,31 +132,36 @@ void lstm_forward_kernel(LstmFwdParams p) {
 #pragma unroll
         for (int g = 0; g < 4; ++g)
           a[g] = wx[pp][g] + sum_product<NB, CT>(red, pl[pp], g * HS + pc[pp]) + bias[pp][g];
-        const float gi = sigmoid_f(a[0]);
-        const float gg = tanhf(a[1]);
-        const float gf = sigmoid_f(a[2]);
-        const float go = sigmoid_f(a[3]);
-        if (p.training) {
-          float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
-          vt[0] = gi;
-          vt[H] = gg;
-          vt[2 * H] = gf;
-          vt[3 * H] = go;
-        }
-        const float c_new = gf * c_prev[pp] + gi * gg;
-        float h_new = go * tanhf(c_new);
+        gate[pp][0] = sigmoid_f(a[0]);
+        gate[pp][1] = tanhf(a[1]);
+        gate[pp][2] = sigmoid_f(a[2]);
+        gate[pp][3] = sigmoid_f(a[3]);
+        const float c_new = gate[pp][2] * c_prev[pp] + gate[pp][0] * gate[pp][1];
+        float h_new = gate[pp][3] * tanhf(c_new);
         if (zoneout) {
           if (p.training) h_new = (h_new - h_prev[pp]) * mk[pp] + h_prev[pp];
           else h_new = p.zoneout_prob * h_prev[pp] + (1.0f - p.zoneout_prob) * h_new;
         }
-        const size_t o = (size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp];
-        p.c[o] = c_new;
-        store_exchanged(gs, &p.h[o], h_new);
+        if (t + 1 < T) store_exchanged(gs, &xh_next[xchg_index(pj[pp], pl[pp], NB)], h_new);
         c_prev[pp] = c_new;
         h_prev[pp] = h_new;
       }
     }
     if (t + 1 < T) group_arrive(gs);  // publishes h[t+1]; also fences `red` reuse
+    // The caller's copies are written behind the barrier: nobody in the launch waits for them.
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      if (act[pp]) {
+        if (p.training) {
+          float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+#pragma unroll
+          for (int g = 0; g < 4; ++g) vt[g * H] = gate[pp][g];
+        }
+        const size_t o = (size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp];
+        p.c[o] = c_prev[pp];
+        p.h[o] = h_prev[pp];
+      }
+    }
   }
 }
 
@@ -159,11 +177,14 @@ struct LstmBwdParams {
   float* v;             // [T,N,4H] in: activations, out: gate gradients
   const float* zoneout_mask;
   float* db_partial;    // [batch tiles, 4H] scratch
+  float* xdv;           // exchange tiles of the gate gradients: [batch tiles][2][Kpad/4][NB][4]
   LaunchShape ls;
 };
 
 // A workgroup owns 16 hidden units (HSB) for NB batch rows; its slice of R_t is
-// [4H x 16]: dh[:, its units] = dv_t[:, all 4H] * R_t[:, its units].
+// [4H x 16]: dh[:, its units] = dv_t[:, all 4H] * R_t[:, its units].  Inside the launch
+// the contraction index runs unit-major (k = 4*unit + gate), so a thread publishes the
+// four gate gradients of its (row, unit) with one 16-byte store.
 template <int NB>
 __global__ __launch_bounds__(256, 1)
 void lstm_backward_kernel(LstmBwdParams p) {
@@ -177,8 +198,7 @@ void lstm_backward_kernel(LstmBwdParams p) {
   __shared__ unsigned int s_flag;
 
   const int H = p.H, N = p.N, T = p.T;
-  const int K = 4 * H;
-  const int Kpad = round_up(K, 64);
+  const int Kpad = 64 * p.ls.gx;  // 4 gates of the 16 units of every workgroup
   float* w_lds = lds;
   float* red = lds + Kpad * NCOLS;  // the partial tiles, reused for the db reduction
 
@@ -191,10 +211,15 @@ void lstm_backward_kernel(LstmBwdParams p) {
   GroupSync gs;
   group_sync_init(gs, p.ls, role);
 
+  const int tile_floats = Kpad * NB;
+  float* xdv = p.xdv + (size_t)role.bt * 2 * tile_floats;
+  const TileBuffer xdvb = make_tile_buffer(xdv, 2 * tile_floats);
+
   for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
     const int k = idx / NCOLS, cidx = idx % NCOLS;
+    const int unit = k >> 2, gate = k & 3;
     float w = 0.f;
-    if (k < K && j0 + cidx < H) w = p.R_t[(size_t)k * H + j0 + cidx];
+    if (unit < H && j0 + cidx < H) w = p.R_t[((size_t)gate * H + unit) * H + j0 + cidx];
     w_lds[slice_index(k, cidx, NCOLS)] = w;
   }
 
@@ -215,7 +240,6 @@ void lstm_backward_kernel(LstmBwdParams p) {
     for (int g = 0; g < 4; ++g) dbacc[pp][g] = 0.f;
   }
   const bool zoneout = p.zoneout_mask != nullptr;
-  const bool vec_ok = (H % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.v) & 15u) == 0);
   __syncthreads();
 
   // Step inputs that do not depend on the recurrence, fetched one step ahead.
@@ -242,10 +266,13 @@ void lstm_backward_kernel(LstmBwdParams p) {
   fetch(T - 1);
 
   for (int t = T - 1; t >= 0; --t) {
-    float dh_keep[PP];
+    float dh_keep[PP], dv[PP][4];
+    float* xdv_t = xdv + (t & 1) * tile_floats;
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
       dh_keep[pp] = 0.f;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) dv[pp][g] = 0.f;
       if (act[pp]) {
         const StepIn s = nxt[pp];
         const float gi = s.vt[0], gg = s.vt[1], gf = s.vt[2], go = s.vt[3];
@@ -267,23 +294,32 @@ void lstm_backward_kernel(LstmBwdParams p) {
         const float dv_g = d_tanh_f(gg) * dg;
         const float dv_f = d_sigmoid_f(gf) * df;
         const float dv_o = d_sigmoid_f(go) * do_;
+        dv[pp][0] = dv_i;
+        dv[pp][1] = dv_g;
+        dv[pp][2] = dv_f;
+        dv[pp][3] = dv_o;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) dbacc[pp][g] += dv[pp][g];
+      }
+      // rows and units beyond the problem are published as zeros
+      if (tid + 256 * pp < NB * HSB)
+        store_exchanged4(gs, xdv_t + ((size_t)pj[pp] * NB + pl[pp]) * 4, dv[pp][0], dv[pp][1],
+                         dv[pp][2], dv[pp][3]);
+    }
+    group_arrive(gs);   // dv_t of this workgroup's units is published
+    // The caller's copy is written behind the barrier: nobody in the launch waits for it.
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      if (act[pp]) {
         float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
-        store_exchanged(gs, vt, dv_i);
-        store_exchanged(gs, vt + H, dv_g);
-        store_exchanged(gs, vt + 2 * H, dv_f);
-        store_exchanged(gs, vt + 3 * H, dv_o);
-        dbacc[pp][0] += dv_i;
-        dbacc[pp][1] += dv_g;
-        dbacc[pp][2] += dv_f;
-        dbacc[pp][3] += dv_o;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) vt[g * H] = dv[pp][g];
       }
     }
-    group_arrive(gs);   // dv_t of this workgroup's columns is published
     fetch(t - 1);       // overlap next step's loads with the wait
-    group_wait(gs);     // all 4H columns of dv_t are complete for this batch tile
+    group_wait(gs);     // dv_t of every unit is complete for this batch tile
 
-    slice_product<NB, 1, true>(p.v + ((size_t)t * N + n0) * 4 * H, 4 * H, rows_here, K, Kpad, w_lds,
-                               vec_ok, gs.same_xcd, red);
+    tile_product<NB, 1, true>(xdvb, (t & 1) * tile_floats, Kpad, w_lds, red);
     __syncthreads();
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp)
@@ -332,20 +368,22 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
                       const float* zoneout_mask, const float* dc_mask, float dc_scale) {
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
   HASTE_HIP_REQUIRE(W && R && b && x && h && c && v);
-  Workspace ws;
-  HASTE_HIP_PROPAGATE(get_workspace(stream, 0, &ws));
-  HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
-
+  const ForwardTile tile = pick_forward_tile(4, N, H, 0);
+  if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   // v = x * W for all steps at once.
   HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 4 * H, C, x, C, W, 4 * H, v, 4 * H, false));
+
+  // Taken after the GEMM, which may replace the stream's scratch buffer with a larger one.
+  Workspace ws;
+  HASTE_HIP_PROPAGATE(get_workspace(stream, exchange_floats(H, tile.nb, tile.gy) * sizeof(float), &ws));
+  HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 
   LstmFwdParams p;
   p.training = training; p.T = T; p.N = N; p.H = H;
   p.R = R; p.b = b; p.h = h; p.c = c; p.v = v;
   p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
   p.dc_mask = dc_mask; p.dc_scale = dc_scale;
-  const ForwardTile tile = pick_forward_tile(4, N, H, 0);
-  if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  p.xh = ws.scratch;
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.nb, tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;
@@ -374,7 +412,9 @@ int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 
   Workspace ws;
-  HASTE_HIP_PROPAGATE(get_workspace(stream, (size_t)tile.gy * 4 * H * sizeof(float), &ws));
+  const size_t db_floats = (size_t)tile.gy * 4 * H;
+  const size_t xdv_floats = exchange_floats(64 * tile.gx, tile.nb, tile.gy);
+  HASTE_HIP_PROPAGATE(get_workspace(stream, ((db_floats + 3) / 4 * 4 + xdv_floats) * sizeof(float), &ws));
   HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 
   LstmBwdParams p;
@@ -382,6 +422,7 @@ int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   p.R_t = R_t; p.c = c; p.dh_new = dh_new; p.dc_new = dc_new;
   p.db = db; p.dh = dh; p.dc = dc; p.v = v; p.zoneout_mask = zoneout_mask;
   p.db_partial = ws.scratch;
+  p.xdv = ws.scratch + (db_floats + 3) / 4 * 4;
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.nb, tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;

@@ -27,15 +27,17 @@ __device__ __forceinline__ float d_sigmoid_f(float y) { return y * (1.0f - y); }
 __device__ __forceinline__ float d_tanh_f(float y) { return 1.0f - y * y; }
 
 // ---- Exchange between workgroups inside one launch --------------------------------
-// The 8 XCDs of the chip have separate L2 caches.  Data one workgroup writes and
-// another reads in the same launch is always READ with agent-scope loads (the sc1 form
-// of global_load: it never trusts the reader's L1, is served by the L2 when the line
-// was written through that L2, and otherwise comes from the memory side).  How it is
-// WRITTEN depends on where the readers are: when a whole group sits on one XCD an
-// ordinary store is enough (the shared L2 is the meeting point, ~0.25 us one way);
-// when the group spans XCDs the store is agent scope too (written through to the memory
-// side, ~0.4 us one way).  Everything else uses ordinary cached accesses: no cache-wide
-// write-back or invalidate is needed at a step boundary.
+// The 8 XCDs of the chip have separate L2 caches, every CU has its own L1.  Data one
+// workgroup writes and another reads in the same launch is always READ with agent-scope
+// loads (the sc1 form of the load instructions): they never trust the reader's L1, which
+// nothing invalidates between the steps of a launch and which may still hold what the
+// address contained two steps ago; they are served by the L2 when the line was written
+// through that L2, and otherwise come from the memory side.  How the data is WRITTEN
+// depends on where the readers are: when a whole group sits on one XCD an ordinary store
+// is enough (the shared L2 is the meeting point, ~0.25 us one way); when the group spans
+// XCDs the store is agent scope too (written through to the memory side, ~0.4 us one
+// way).  Everything else uses ordinary cached accesses: no cache-wide write-back or
+// invalidate is needed at a step boundary.
 __device__ __forceinline__ float load_exchanged(const float* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -60,7 +62,7 @@ struct LaunchShape {
   unsigned int epoch;          // step flags of this launch count up from here
   unsigned int ticket_base;    // per-XCD tickets of this launch count up from here
   int gx, gy;                  // column workgroups per group, number of groups (batch tiles)
-  int tile_rows;               // batch rows per group (<= 16*RT; 8 spreads small batches over more XCDs)
+  int tile_rows;               // batch rows per group (the kernel's NB)
   int xcd_local;               // 1: group g is the set of workgroups running on XCD g
   int per_xcd;                 // workgroups this launch places on every XCD (xcd_local)
 };
@@ -145,6 +147,29 @@ __device__ __forceinline__ void store_exchanged(const GroupSync& g, float* p, fl
   else __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// 8-byte aligned p.
+__device__ __forceinline__ void store_exchanged2(const GroupSync& g, float* p, float a, float b) {
+  if (g.same_xcd) {
+    *reinterpret_cast<float2*>(p) = make_float2(a, b);
+    return;
+  }
+  const unsigned long long bits =
+      (unsigned long long)__float_as_uint(a) | ((unsigned long long)__float_as_uint(b) << 32);
+  __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), bits, __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// 16-byte aligned p.
+__device__ __forceinline__ void store_exchanged4(const GroupSync& g, float* p, float a, float b,
+                                                 float c, float d) {
+  if (g.same_xcd) {
+    *reinterpret_cast<float4_t*>(p) = float4_t{a, b, c, d};
+    return;
+  }
+  store_exchanged2(g, p, a, b);
+  store_exchanged2(g, p + 2, c, d);
+}
+
 // Counts the workgroup as arrived once every exchanged store its threads have issued
 // has completed.  Called by all threads.
 __device__ __forceinline__ void group_arrive(GroupSync& g) {
@@ -189,9 +214,6 @@ __device__ __forceinline__ void group_wait(GroupSync& g) {
     }
   }
   __syncthreads();
-  // Same-XCD groups read the exchanged data with ordinary loads: drop what this CU's L1
-  // may still hold of those lines (the shared L2 has the new values).
-  if (g.same_xcd) asm volatile("buffer_inv sc0" ::: "memory");
 }
 
 // True in exactly one workgroup of the launch: the last to call it.  Stores made by
@@ -223,72 +245,6 @@ __device__ __forceinline__ int round_up(int x, int m) { return (x + m - 1) / m *
 // lanes of a k-quarter read 16 consecutive such vectors (no bank conflicts).
 __device__ __forceinline__ int slice_index(int k, int col, int ncols) {
   return ((((k >> 4) << 2) + ((k & 15) >> 2)) * ncols + col) * 4 + (k & 3);
-}
-
-// Guarded 4-float read of exchanged data: elements beyond `valid` read as zero.
-__device__ __forceinline__ float4_t load_a4(const float* p, int valid, bool vec_ok) {
-  float4_t v = {0.f, 0.f, 0.f, 0.f};
-  if (valid >= 4 && vec_ok) {
-    v = load_exchanged4(p);
-  } else {
-    if (valid > 0) v.x = load_exchanged(p);
-    if (valid > 1) v.y = load_exchanged(p + 1);
-    if (valid > 2) v.z = load_exchanged(p + 2);
-    if (valid > 3) v.w = load_exchanged(p + 3);
-  }
-  return v;
-}
-
-// Loads the A operands of k-groups [g, g+CHUNK) of this wavefront's quarter (see
-// slice_matmul).  Branch-free on the vector paths: out-of-range elements read element 0
-// of the tile and are zeroed afterwards.
-template <int RT, int CHUNK>
-__device__ __forceinline__ void load_a_chunk(const float* __restrict__ a, int a_ld, int rows_valid,
-                                             int K, int g_abs, int g_end, bool vec_ok, bool cached,
-                                             float4_t (&av)[CHUNK][RT]) {
-  const int lane = threadIdx.x & 63;
-  const int row = lane & 15;
-  const int kq = lane >> 4;
-  const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
-  if (vec_ok && cached) {
-#pragma unroll
-    for (int gi = 0; gi < CHUNK; ++gi) {
-      const int k = (g_abs + gi) * 16 + kq * 4;
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        const int rr = rt * 16 + row;
-        const bool ok = g_abs + gi < g_end && rr < rows_valid && k < K;
-        const float* src = a + (ok ? (size_t)rr * a_ld + k : (size_t)0);
-        const float4_t v = *reinterpret_cast<const float4_t*>(src);
-        av[gi][rt] = ok ? v : zero4;
-      }
-    }
-  } else if (vec_ok) {
-#pragma unroll
-    for (int gi = 0; gi < CHUNK; ++gi) {
-      const int k = (g_abs + gi) * 16 + kq * 4;
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        const int rr = rt * 16 + row;
-        const bool ok = g_abs + gi < g_end && rr < rows_valid && k < K;
-        const float* src = a + (ok ? (size_t)rr * a_ld + k : (size_t)0);
-        const float4_t v = load_exchanged4(src);
-        av[gi][rt] = ok ? v : zero4;
-      }
-    }
-  } else {
-#pragma unroll
-    for (int gi = 0; gi < CHUNK; ++gi) {
-      const int k = (g_abs + gi) * 16 + kq * 4;
-      const bool live = g_abs + gi < g_end;
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        const int rr = rt * 16 + row;
-        const int valid = (live && rr < rows_valid) ? (K - k) : 0;
-        av[gi][rt] = load_a4(a + (size_t)rr * a_ld + k, valid, false);
-      }
-    }
-  }
 }
 
 // MFMAs of k-groups [g_abs, g_abs+CHUNK): one straight-line block (no branches, so the
@@ -342,58 +298,6 @@ __device__ __forceinline__ void mfma_chunk(const float* w_lds, int g_abs,
   }
 }
 
-// acc[rt][ct] += A[16*RT rows, K] * slice[K, 16*CT] for this wavefront's quarter of K.
-// `a` points at row 0 of the batch tile (row stride a_ld floats, K contiguous);
-// rows >= rows_valid and k >= K read as zero.  The four wavefronts of the workgroup
-// each take Kpad/4 consecutive k; the caller adds their accumulators.
-// Accumulator element r of acc[rt][ct] in lane l is row 16*rt + 4*(l/16) + r,
-// column 16*ct + l%16.
-// `cached`: the tile may be read with ordinary loads (same-XCD group, L1 invalidated
-// after the barrier); otherwise agent-scope loads are used.  `vec_ok`: rows are 16-byte
-// aligned and K is a multiple of 4.
-// K is walked in chunks of CHUNK k-groups; the loads of the next chunk are issued before
-// the MFMAs of the current one, so they are in flight while the matrix unit works.  The
-// k-groups left over when the count is not a multiple of CHUNK are done one at a time.
-template <int RT, int CT, int CHUNK>
-__device__ __forceinline__ void slice_matmul(const float* __restrict__ a, int a_ld, int rows_valid,
-                                             int K, int Kpad, const float* w_lds, bool vec_ok,
-                                             bool cached, float4_t (&acc)[RT][CT]) {
-  const int wave = threadIdx.x >> 6;
-  const int groups = Kpad >> 6;  // k-groups of 16 per wavefront
-  const int full = groups / CHUNK;
-  int g = wave * groups;
-  const int g_end = g + groups;
-  float4_t acc1[RT][CT];
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) acc1[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
-
-  if (full > 0) {
-    float4_t cur[CHUNK][RT], nxt[CHUNK][RT];
-    load_a_chunk<RT, CHUNK>(a, a_ld, rows_valid, K, g, g_end, vec_ok, cached, cur);
-    for (int c = 0; c < full; ++c) {
-      if (c + 1 < full)
-        load_a_chunk<RT, CHUNK>(a, a_ld, rows_valid, K, g + CHUNK, g_end, vec_ok, cached, nxt);
-      mfma_chunk<RT, CT, CHUNK>(w_lds, g, cur, acc, acc1);
-#pragma unroll
-      for (int gi = 0; gi < CHUNK; ++gi)
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) cur[gi][rt] = nxt[gi][rt];
-      g += CHUNK;
-    }
-  }
-  for (; g < g_end; ++g) {
-    float4_t one[1][RT];
-    load_a_chunk<RT, 1>(a, a_ld, rows_valid, K, g, g_end, vec_ok, cached, one);
-    mfma_chunk<RT, CT, 1>(w_lds, g, one, acc, acc1);
-  }
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) acc[rt][ct] += acc1[rt][ct];
-}
-
 // Writes this wavefront's accumulators to red[wave][16*RT][16*CT] in LDS.
 template <int RT, int CT>
 __device__ __forceinline__ void store_partials(float* red, const float4_t (&acc)[RT][CT]) {
@@ -443,72 +347,141 @@ struct ShortTileShape {
   static constexpr int CTN = NCOLS / MC;  // MFMAs side by side to cover the slice columns
 };
 
-// A operands of CH "super-groups" of 64 consecutive k (super-group s covers k in
-// [64 s, 64 s + 64)); the wavefront takes super-groups s0, s0 + 4, ...  Lane l holds row
-// 4*rb + l%4 and k = 64 s + 4*(l/4) .. +3, so MFMA (j, abid) of lane group g multiplies
-// k = 64 s + 4*(g*NBC + abid) + j.
-template <int RB, int CH>
-__device__ __forceinline__ void load_a_rows4(const float* __restrict__ a, int a_ld, int rows_valid,
-                                             int K, int s0, int s_end, bool vec_ok, bool cached,
-                                             float4_t (&av)[CH][RB]) {
+// ---- the product of one step, for any tile height ------------------------------------
+// NB batch rows (4, 8, or a multiple of 16) by 16*CT slice columns.  kPartials partial
+// tiles of [NB][16*CT] floats are left in `red` by tile_product; sum_product adds them in a
+// fixed order.
+template <int NB, int CT>
+struct ProductTile {
+  static_assert(NB == 4 || NB == 8 || NB % 16 == 0, "unsupported tile height");
+  static constexpr bool kShort = NB < 16;
+  static constexpr int NCOLS = 16 * CT;
+  static constexpr int kPartials = kShort ? 4 * ShortTileShape<CT>::KS : 4;
+  static constexpr int kRedFloats = kPartials * NB * NCOLS;
+};
+
+// ---- exchange tiles ------------------------------------------------------------------
+// What a step's product reads from the other workgroups (h[t], or the gate gradients of
+// step t) is kept by its producers in a copy laid out for the consumers: per batch tile
+// [Kpad/4][NB rows][4 consecutive k].  A wavefront's operand load is then one contiguous
+// kilobyte (rows of the public [N, K] layout would make each 4-lane group touch 4 lines),
+// needs no bounds checks (rows and k beyond the problem are kept at zero by whoever owns
+// them) and producers write 16 bytes at a time.  Two tiles alternate by step parity: a
+// workgroup may publish step t+1 while a slower one still reads step t.
+__device__ __forceinline__ int xchg_index(int k, int row, int nb) {
+  return ((k >> 2) * nb + row) * 4 + (k & 3);
+}
+
+// The two tiles of a group as a buffer resource: 16-byte loads that are served by the L2
+// (agent scope, the reader's L1 is never consulted: it may hold the tile's previous
+// contents) and return zero beyond the end.
+typedef unsigned int uint4_t __attribute__((ext_vector_type(4)));
+struct TileBuffer {
+  __amdgpu_buffer_rsrc_t rsrc;
+};
+
+__device__ __forceinline__ TileBuffer make_tile_buffer(float* tiles, int floats) {
+  TileBuffer b;
+  b.rsrc = __builtin_amdgcn_make_buffer_rsrc(tiles, 0, floats * 4, 0x00020000);
+  return b;
+}
+
+// float_index: multiple of 4.
+__device__ __forceinline__ float4_t load_tile4(const TileBuffer& b, int float_index) {
+  constexpr int kAgentScope = 16;  // the sc1 bit of the cache policy
+  const uint4_t v = __builtin_amdgcn_raw_buffer_load_b128(b.rsrc, float_index * 4, 0, kAgentScope);
+  return float4_t{__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z),
+                  __uint_as_float(v.w)};
+}
+
+// 16x16x4 path: A operands of k-groups [g_abs, g_abs+CHUNK) from an exchange tile of
+// 16*RT rows.  Lane l holds row l%16 (of each 16-row block) and k = 16 g + 4 (l/16) .. +3.
+template <int RT, int CHUNK>
+__device__ __forceinline__ void load_tile_chunk(const TileBuffer& xb, int tile_off, int g_abs,
+                                                int g_end, float4_t (&av)[CHUNK][RT]) {
+  constexpr int NB = 16 * RT;
   const int lane = threadIdx.x & 63;
-  const int r = lane & 3;
-  const int kb = (lane >> 2) * 4;
   const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
-  if (vec_ok && cached) {
+  const int base = tile_off + ((lane >> 4) * NB + (lane & 15)) * 4;
 #pragma unroll
-    for (int ci = 0; ci < CH; ++ci) {
-      const int s = s0 + 4 * ci;
-      const int k = 64 * s + kb;
+  for (int gi = 0; gi < CHUNK; ++gi) {
+    const bool ok = g_abs + gi < g_end;
+    const int g = ok ? g_abs + gi : g_abs;
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        const int rr = 4 * rb + r;
-        const bool ok = s < s_end && rr < rows_valid && k < K;
-        const float* src = a + (ok ? (size_t)rr * a_ld + k : (size_t)0);
-        const float4_t v = *reinterpret_cast<const float4_t*>(src);
-        av[ci][rb] = ok ? v : zero4;
-      }
-    }
-  } else if (vec_ok) {
-#pragma unroll
-    for (int ci = 0; ci < CH; ++ci) {
-      const int s = s0 + 4 * ci;
-      const int k = 64 * s + kb;
-#pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        const int rr = 4 * rb + r;
-        const bool ok = s < s_end && rr < rows_valid && k < K;
-        const float* src = a + (ok ? (size_t)rr * a_ld + k : (size_t)0);
-        const float4_t v = load_exchanged4(src);
-        av[ci][rb] = ok ? v : zero4;
-      }
-    }
-  } else {
-#pragma unroll
-    for (int ci = 0; ci < CH; ++ci) {
-      const int s = s0 + 4 * ci;
-      const int k = 64 * s + kb;
-#pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        const int rr = 4 * rb + r;
-        const int valid = (s < s_end && rr < rows_valid) ? (K - k) : 0;
-        av[ci][rb] = load_a4(a + (size_t)rr * a_ld + k, valid, false);
-      }
+    for (int rt = 0; rt < RT; ++rt) {
+      const float4_t v = load_tile4(xb, base + (g * 4 * NB + rt * 16) * 4);
+      av[gi][rt] = ok ? v : zero4;
     }
   }
 }
 
-// MFMAs of super-group s.  One 16-byte LDS read per (abid, column tile) feeds 4*RB MFMAs;
-// the read for abid+1 is issued before the MFMAs of abid.  Consecutive MFMAs on one
-// output tile alternate between two accumulators.
+template <int RT, int CT, int CHUNK>
+__device__ __forceinline__ void tall_tile_product(const TileBuffer& xb, int tile_off, int Kpad,
+                                                  const float* w_lds, float* red) {
+  const int wave = threadIdx.x >> 6;
+  const int groups = Kpad >> 6;  // k-groups of 16 per wavefront
+  const int full = groups / CHUNK;
+  int g = wave * groups;
+  const int g_end = g + groups;
+  float4_t acc[RT][CT], acc1[RT][CT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = acc1[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  if (full > 0) {
+    float4_t cur[CHUNK][RT], nxt[CHUNK][RT];
+    load_tile_chunk<RT, CHUNK>(xb, tile_off, g, g_end, cur);
+    for (int c = 0; c < full; ++c) {
+      if (c + 1 < full) load_tile_chunk<RT, CHUNK>(xb, tile_off, g + CHUNK, g_end, nxt);
+      mfma_chunk<RT, CT, CHUNK>(w_lds, g, cur, acc, acc1);
+#pragma unroll
+      for (int gi = 0; gi < CHUNK; ++gi)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) cur[gi][rt] = nxt[gi][rt];
+      g += CHUNK;
+    }
+  }
+  for (; g < g_end; ++g) {
+    float4_t one[1][RT];
+    load_tile_chunk<RT, 1>(xb, tile_off, g, g_end, one);
+    mfma_chunk<RT, CT, 1>(w_lds, g, one, acc, acc1);
+  }
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) acc[rt][ct] += acc1[rt][ct];
+  store_partials<RT, CT>(red, acc);
+}
+
+// 4x4x1 path: A operands of CH super-groups s0, s0+4, ... (64 k each) from an exchange
+// tile of 4*RB rows.  Lane l = 4*block + r holds row 4*rb + r; block g*NBC + a holds the
+// four k of float4 index 16 s + a*KS + g, which makes the KS lane groups of one MFMA read
+// adjacent float4 rows of the slice in LDS.
+template <int RB, int CT, int CH>
+__device__ __forceinline__ void load_tile_rows4(const TileBuffer& xb, int tile_off, int s0,
+                                                float4_t (&av)[CH][RB]) {
+  using S = ShortTileShape<CT>;
+  constexpr int NB = 4 * RB;
+  const int lane = threadIdx.x & 63;
+  const int block = lane >> 2;
+  const int k4 = (block % S::NBC) * S::KS + block / S::NBC;
+  const int base = tile_off + (k4 * NB + (lane & 3)) * 4;
+#pragma unroll
+  for (int ci = 0; ci < CH; ++ci)
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+      av[ci][rb] = load_tile4(xb, base + ((s0 + 4 * ci) * 16 * NB + 4 * rb) * 4);
+}
+
+// MFMAs of super-group s for the operand layout of load_tile_rows4.
 template <int RB, int CT>
-__device__ __forceinline__ void mfma_rows4(const float* w_lds, int s, const float4_t (&av)[RB],
-                                           float4_t (&acc0)[RB][ShortTileShape<CT>::CTN],
-                                           float4_t (&acc1)[RB][ShortTileShape<CT>::CTN]) {
+__device__ __forceinline__ void mfma_tile_rows4(const float* w_lds, int s, const float4_t (&av)[RB],
+                                                float4_t (&acc0)[RB][ShortTileShape<CT>::CTN],
+                                                float4_t (&acc1)[RB][ShortTileShape<CT>::CTN]) {
   using S = ShortTileShape<CT>;
   const int lane = threadIdx.x & 63;
-  const float* wp =
-      w_lds + ((16 * s + (lane / S::MC) * S::NBC) * S::NCOLS + lane % S::MC) * 4;
+  const float* wp = w_lds + ((16 * s + lane / S::MC) * S::NCOLS + lane % S::MC) * 4;
   float4_t bnext[S::CTN];
 #pragma unroll
   for (int ct = 0; ct < S::CTN; ++ct)
@@ -521,7 +494,8 @@ __device__ __forceinline__ void mfma_rows4(const float* w_lds, int s, const floa
     if constexpr (A + 1 < S::NBC) {
 #pragma unroll
       for (int ct = 0; ct < S::CTN; ++ct)
-        bnext[ct] = *reinterpret_cast<const float4_t*>(wp + ((A + 1) * S::NCOLS + ct * S::MC) * 4);
+        bnext[ct] = *reinterpret_cast<const float4_t*>(
+            wp + ((A + 1) * S::KS * S::NCOLS + ct * S::MC) * 4);
     }
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
@@ -546,21 +520,21 @@ __device__ __forceinline__ void mfma_rows4(const float* w_lds, int s, const floa
   });
 }
 
-// Product of a short tile: red[wave*KS + g][4*RB][16*CT] <- this wavefront's partial
-// tile of lane group g.  Accumulator element r of acc[rb][ct] in lane l is row 4*rb + r,
-// column ct*MC + l%MC, partial g = l/MC.
+// Product of a short exchange tile: red[wave*KS + g][4*RB][16*CT] <- this wavefront's
+// partial tile of lane group g (accumulator element r of acc[rb][ct] in lane l is row
+// 4*rb + r, column ct*MC + l%MC, partial g = l/MC).  The operand
+// loads of chunk c+1 (CH super-groups) are issued before the MFMAs of chunk c; the two
+// register buffers alternate so that nothing is copied.
 template <int RB, int CT, int CH>
-__device__ __forceinline__ void short_tile_product(const float* __restrict__ a, int a_ld,
-                                                   int rows_valid, int K, int Kpad,
-                                                   const float* w_lds, bool vec_ok, bool cached,
-                                                   float* red) {
+__device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int tile_off, int Kpad,
+                                                       const float* w_lds, float* red) {
   using S = ShortTileShape<CT>;
   constexpr int NB = 4 * RB;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int s_end = Kpad >> 6;
   const int mine = (s_end - wave + 3) >> 2;  // super-groups wave, wave+4, ...
-  const int full = mine / CH;
+  const int chunks = mine / CH;
   float4_t acc0[RB][S::CTN], acc1[RB][S::CTN];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb)
@@ -568,25 +542,27 @@ __device__ __forceinline__ void short_tile_product(const float* __restrict__ a, 
     for (int ct = 0; ct < S::CTN; ++ct) acc0[rb][ct] = acc1[rb][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
 
   int s = wave;
-  if (full > 0) {
-    float4_t cur[CH][RB], nxt[CH][RB];
-    load_a_rows4<RB, CH>(a, a_ld, rows_valid, K, s, s_end, vec_ok, cached, cur);
-    for (int c = 0; c < full; ++c) {
-      if (c + 1 < full)
-        load_a_rows4<RB, CH>(a, a_ld, rows_valid, K, s + 4 * CH, s_end, vec_ok, cached, nxt);
+  if (chunks > 0) {
+    float4_t buf0[CH][RB], buf1[CH][RB];
+    load_tile_rows4<RB, CT, CH>(xb, tile_off, s, buf0);
+    int c = 0;
+    for (;;) {
+      if (c + 1 < chunks) load_tile_rows4<RB, CT, CH>(xb, tile_off, s + 4 * CH, buf1);
 #pragma unroll
-      for (int ci = 0; ci < CH; ++ci) mfma_rows4<RB, CT>(w_lds, s + 4 * ci, cur[ci], acc0, acc1);
-#pragma unroll
-      for (int ci = 0; ci < CH; ++ci)
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) cur[ci][rb] = nxt[ci][rb];
+      for (int ci = 0; ci < CH; ++ci) mfma_tile_rows4<RB, CT>(w_lds, s + 4 * ci, buf0[ci], acc0, acc1);
       s += 4 * CH;
+      if (++c == chunks) break;
+      if (c + 1 < chunks) load_tile_rows4<RB, CT, CH>(xb, tile_off, s + 4 * CH, buf0);
+#pragma unroll
+      for (int ci = 0; ci < CH; ++ci) mfma_tile_rows4<RB, CT>(w_lds, s + 4 * ci, buf1[ci], acc0, acc1);
+      s += 4 * CH;
+      if (++c == chunks) break;
     }
   }
   for (; s < s_end; s += 4) {
     float4_t one[1][RB];
-    load_a_rows4<RB, 1>(a, a_ld, rows_valid, K, s, s_end, vec_ok, cached, one);
-    mfma_rows4<RB, CT>(w_lds, s, one[0], acc0, acc1);
+    load_tile_rows4<RB, CT, 1>(xb, tile_off, s, one);
+    mfma_tile_rows4<RB, CT>(w_lds, s, one[0], acc0, acc1);
   }
 
   float* base = red + ((wave * S::KS + lane / S::MC) * NB) * S::NCOLS + lane % S::MC;
@@ -603,45 +579,36 @@ __device__ __forceinline__ void short_tile_product(const float* __restrict__ a, 
     }
 }
 
-// ---- the product of one step, for any tile height ------------------------------------
-// NB batch rows (4, 8, or a multiple of 16) by 16*CT slice columns.  kPartials partial
-// tiles of [NB][16*CT] floats are left in `red`; sum_product adds them in a fixed order.
-template <int NB, int CT>
-struct ProductTile {
-  static_assert(NB == 4 || NB == 8 || NB % 16 == 0, "unsupported tile height");
-  static constexpr bool kShort = NB < 16;
-  static constexpr int NCOLS = 16 * CT;
-  static constexpr int kPartials = kShort ? 4 * ShortTileShape<CT>::KS : 4;
-  static constexpr int kRedFloats = kPartials * NB * NCOLS;
-};
-
-// red <- partial tiles of A[NB rows, K] * slice[K, 16*CT].  `a` points at row 0 of the
-// batch tile (row stride a_ld floats, K contiguous); rows >= rows_valid and k >= K read
-// as zero.  `cached`: the tile may be read with ordinary loads (same-XCD group, L1
-// invalidated after the barrier); otherwise agent-scope loads are used.  `vec_ok`: rows
-// are 16-byte aligned and K is a multiple of 4.  LONG_K selects deeper prefetch for
-// contractions much longer than the hidden size (the backward passes).
+// red <- partial tiles of tile[NB rows, Kpad] * slice[Kpad, 16*CT]; the exchange tile
+// starts at float `tile_off` of `xb`.  LONG_K selects deeper prefetch for contractions much
+// longer than the hidden size (the backward passes).
 template <int NB, int CT, bool LONG_K>
-__device__ __forceinline__ void slice_product(const float* __restrict__ a, int a_ld, int rows_valid,
-                                              int K, int Kpad, const float* w_lds, bool vec_ok,
-                                              bool cached, float* red) {
+__device__ __forceinline__ void tile_product(const TileBuffer& xb, int tile_off, int Kpad,
+                                             const float* w_lds, float* red) {
   if constexpr (ProductTile<NB, CT>::kShort) {
-    short_tile_product<NB / 4, CT, LONG_K ? 8 : 2>(a, a_ld, rows_valid, K, Kpad, w_lds, vec_ok,
-                                                   cached, red);
+    short_exchange_product<NB / 4, CT, LONG_K ? 4 : 2>(xb, tile_off, Kpad, w_lds, red);
   } else {
     constexpr int RT = NB / 16;
     constexpr int CHUNK = LONG_K ? (RT == 1 ? 8 : (RT == 2 ? 4 : 2)) : (RT >= 4 ? 2 : 4);
-    float4_t acc[RT][CT];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
-    slice_matmul<RT, CT, CHUNK>(a, a_ld, rows_valid, K, Kpad, w_lds, vec_ok, cached, acc);
-    store_partials<RT, CT>(red, acc);
+    tall_tile_product<RT, CT, CHUNK>(xb, tile_off, Kpad, w_lds, red);
   }
 }
 
-// Element (row, col) of the product: the partial tiles written by slice_product, added
+// Zeroes this workgroup's share of its group's two exchange tiles: float4 rows
+// [first4, first4 + count4) of [Kpad/4][NB][4], both parities.  The stores have completed
+// when it returns.  Called by all threads.
+__device__ __forceinline__ void zero_tile_share(const GroupSync& g, float* tiles, int tile_floats,
+                                                int nb, int first4, int count4) {
+  for (int i = threadIdx.x; i < count4 * nb; i += 256) {
+    float* q = tiles + ((size_t)first4 * nb + i) * 4;
+    store_exchanged4(g, q, 0.f, 0.f, 0.f, 0.f);
+    store_exchanged4(g, q + tile_floats, 0.f, 0.f, 0.f, 0.f);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+}
+
+// Element (row, col) of the product: the partial tiles written by tile_product, added
 // pairwise in a fixed order.
 template <int NB, int CT>
 __device__ __forceinline__ float sum_product(const float* red, int row, int col) {
@@ -745,6 +712,12 @@ int launch_persistent(const char* name, KernelT kernel, const LaunchPlan& plan, 
 }
 
 constexpr size_t kMaxLdsBytes = 160 * 1024;  // LDS per workgroup on gfx950
+
+// Floats of the two exchange tiles of every group (batch tile) for contraction length K.
+inline size_t exchange_floats(int K, int nb, int gy) {
+  const size_t Kpad = (size_t)(K + 63) / 64 * 64;
+  return 2 * Kpad * nb * gy;
+}
 
 // Geometry of a forward recurrence: nb batch rows and hs hidden units per workgroup
 // (their gate columns fill ct 16-column tiles), gx column workgroups, gy batch tiles.

@@ -8,7 +8,8 @@ from util import TOL, dev, host, problem, relerr
 pytestmark = pytest.mark.gpu
 
 SHAPES = [(1, 1, 1, 1), (3, 2, 3, 4), (5, 3, 7, 5), (6, 17, 20, 36), (4, 16, 32, 64),
-          (10, 33, 48, 128), (8, 64, 64, 256), (6, 128, 96, 512)]
+          (10, 33, 48, 128), (8, 64, 64, 256), (6, 128, 96, 512),
+          (3, 200, 16, 64), (2, 300, 8, 48), (2, 520, 8, 32)]
 
 
 @pytest.mark.parametrize("zoneout", [0.0, 0.3])

@@ -11,7 +11,8 @@ pytestmark = pytest.mark.gpu
 # constant output, and with C == 1 the norm of x*W does not depend on the scale of x, so
 # those input gradients are pure rounding noise to which no relative tolerance applies.
 SHAPES = [(1, 1, 3, 4), (3, 2, 3, 4), (5, 3, 7, 5), (6, 17, 20, 36), (4, 16, 32, 64),
-          (10, 33, 48, 128), (8, 32, 64, 256), (6, 64, 96, 512)]
+          (10, 33, 48, 128), (8, 32, 64, 256), (6, 64, 96, 512),
+          (3, 200, 16, 64), (2, 300, 8, 48), (2, 520, 8, 32)]
 
 
 @pytest.mark.parametrize("zoneout", [0.0, 0.3])
