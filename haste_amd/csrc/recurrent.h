@@ -474,49 +474,64 @@ __device__ __forceinline__ void load_tile_rows4(const TileBuffer& xb, int tile_o
       av[ci][rb] = load_tile4(xb, base + ((s0 + 4 * ci) * 16 * NB + 4 * rb) * 4);
 }
 
-// MFMAs of super-group s for the operand layout of load_tile_rows4.
-template <int RB, int CT>
-__device__ __forceinline__ void mfma_tile_rows4(const float* w_lds, int s, const float4_t (&av)[RB],
+// MFMAs of the CH super-groups s, s+4, ... for the operand layout of load_tile_rows4.
+// One 16-byte LDS read per (super-group, abid, column tile) feeds 4*RB MFMAs; the reads
+// run kLdsAhead steps ahead of the MFMAs that use them, across super-group boundaries.
+// Consecutive MFMAs on one output tile alternate between two accumulators.
+constexpr int kLdsAhead = 3;
+
+template <int RB, int CT, int CH>
+__device__ __forceinline__ void mfma_tile_rows4(const float* w_lds, int s,
+                                                const float4_t (&av)[CH][RB],
                                                 float4_t (&acc0)[RB][ShortTileShape<CT>::CTN],
                                                 float4_t (&acc1)[RB][ShortTileShape<CT>::CTN]) {
   using S = ShortTileShape<CT>;
+  constexpr int STEPS = CH * S::NBC;
   const int lane = threadIdx.x & 63;
   const float* wp = w_lds + ((16 * s + lane / S::MC) * S::NCOLS + lane % S::MC) * 4;
-  float4_t bnext[S::CTN];
+  // step i = (super-group i / NBC, abid i % NBC): float offset of its slice rows from wp
+  auto step_offset = [](int i) {
+    return ((i / S::NBC) * 64 + (i % S::NBC) * S::KS) * S::NCOLS * 4;
+  };
+  float4_t b[STEPS][S::CTN];
+  static_for<(kLdsAhead < STEPS ? kLdsAhead : STEPS)>([&](auto ic) {
+    constexpr int I = decltype(ic)::value;
 #pragma unroll
-  for (int ct = 0; ct < S::CTN; ++ct)
-    bnext[ct] = *reinterpret_cast<const float4_t*>(wp + ct * S::MC * 4);
-  static_for<S::NBC>([&](auto ac) {
-    constexpr int A = decltype(ac)::value;
-    float4_t b[S::CTN];
-#pragma unroll
-    for (int ct = 0; ct < S::CTN; ++ct) b[ct] = bnext[ct];
-    if constexpr (A + 1 < S::NBC) {
+    for (int ct = 0; ct < S::CTN; ++ct)
+      b[I][ct] = *reinterpret_cast<const float4_t*>(wp + step_offset(I) + ct * S::MC * 4);
+  });
+  static_for<STEPS>([&](auto ic) {
+    constexpr int I = decltype(ic)::value;
+    constexpr int A = I % S::NBC;
+    constexpr int CI = I / S::NBC;
+    if constexpr (I + kLdsAhead < STEPS) {
 #pragma unroll
       for (int ct = 0; ct < S::CTN; ++ct)
-        bnext[ct] = *reinterpret_cast<const float4_t*>(
-            wp + ((A + 1) * S::KS * S::NCOLS + ct * S::MC) * 4);
+        b[I + kLdsAhead][ct] = *reinterpret_cast<const float4_t*>(
+            wp + step_offset(I + kLdsAhead) + ct * S::MC * 4);
+      // keep the read here: the scheduler would otherwise sink it to just before its use
+      __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
       for (int ct = 0; ct < S::CTN; ++ct)
-        acc0[rb][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(av[rb].x, b[ct].x, acc0[rb][ct], S::CBSZ, A, 0);
+        acc0[rb][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(av[CI][rb].x, b[I][ct].x, acc0[rb][ct], S::CBSZ, A, 0);
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
       for (int ct = 0; ct < S::CTN; ++ct)
-        acc1[rb][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(av[rb].y, b[ct].y, acc1[rb][ct], S::CBSZ, A, 0);
+        acc1[rb][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(av[CI][rb].y, b[I][ct].y, acc1[rb][ct], S::CBSZ, A, 0);
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
       for (int ct = 0; ct < S::CTN; ++ct)
-        acc0[rb][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(av[rb].z, b[ct].z, acc0[rb][ct], S::CBSZ, A, 0);
+        acc0[rb][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(av[CI][rb].z, b[I][ct].z, acc0[rb][ct], S::CBSZ, A, 0);
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
       for (int ct = 0; ct < S::CTN; ++ct)
-        acc1[rb][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(av[rb].w, b[ct].w, acc1[rb][ct], S::CBSZ, A, 0);
+        acc1[rb][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(av[CI][rb].w, b[I][ct].w, acc1[rb][ct], S::CBSZ, A, 0);
   });
 }
 
@@ -548,13 +563,11 @@ __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int
     int c = 0;
     for (;;) {
       if (c + 1 < chunks) load_tile_rows4<RB, CT, CH>(xb, tile_off, s + 4 * CH, buf1);
-#pragma unroll
-      for (int ci = 0; ci < CH; ++ci) mfma_tile_rows4<RB, CT>(w_lds, s + 4 * ci, buf0[ci], acc0, acc1);
+      mfma_tile_rows4<RB, CT, CH>(w_lds, s, buf0, acc0, acc1);
       s += 4 * CH;
       if (++c == chunks) break;
       if (c + 1 < chunks) load_tile_rows4<RB, CT, CH>(xb, tile_off, s + 4 * CH, buf0);
-#pragma unroll
-      for (int ci = 0; ci < CH; ++ci) mfma_tile_rows4<RB, CT>(w_lds, s + 4 * ci, buf1[ci], acc0, acc1);
+      mfma_tile_rows4<RB, CT, CH>(w_lds, s, buf1, acc0, acc1);
       s += 4 * CH;
       if (++c == chunks) break;
     }
@@ -562,7 +575,7 @@ __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int
   for (; s < s_end; s += 4) {
     float4_t one[1][RB];
     load_tile_rows4<RB, CT, 1>(xb, tile_off, s, one);
-    mfma_tile_rows4<RB, CT>(w_lds, s, one[0], acc0, acc1);
+    mfma_tile_rows4<RB, CT, 1>(w_lds, s, one, acc0, acc1);
   }
 
   float* base = red + ((wave * S::KS + lane / S::MC) * NB) * S::NCOLS + lane % S::MC;
