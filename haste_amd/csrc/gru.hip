@@ -133,7 +133,7 @@ void gru_forward_kernel(GruFwdParams p) {
         const float z = sigmoid_f(wx[pp][0] + rh[0] + bxv[pp][0] + brv[pp][0]);
         const float r = sigmoid_f(wx[pp][1] + rh[1] + bxv[pp][1] + brv[pp][1]);
         const float qg = rh[2] + brv[pp][2];
-        const float g = tanhf(wx[pp][2] + r * qg + bxv[pp][2]);
+        const float g = tanh_f(wx[pp][2] + r * qg + bxv[pp][2]);
         saved[pp][0] = z;
         saved[pp][1] = r;
         saved[pp][2] = g;

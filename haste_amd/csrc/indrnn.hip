@@ -46,7 +46,7 @@ void indrnn_forward_kernel(int T, int N, int H, const float* __restrict__ Wx,
     for (int i = 0; i < U; ++i) {
       const int t = t0 + i;
       if (t < T) {
-        float hn = tanhf(wx_cur[i] + uj * hv + bj);
+        float hn = tanh_f(wx_cur[i] + uj * hv + bj);
         if (ZONEOUT) {
           if (TRAINING) hn = (hn - hv) * mk_cur[i] + hv;
           else hn = zoneout_prob * hv + (1.0f - zoneout_prob) * hn;

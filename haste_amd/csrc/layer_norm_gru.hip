@@ -161,7 +161,7 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
         const float z = sigmoid_f(wx[pp][0] + rn[0] + bxv[pp][0] + brv[pp][0]);
         const float r = sigmoid_f(wx[pp][1] + rn[1] + bxv[pp][1] + brv[pp][1]);
         const float qg = rn[2] + brv[pp][2];
-        const float g = tanhf(wx[pp][2] + r * qg + bxv[pp][2]);
+        const float g = tanh_f(wx[pp][2] + r * qg + bxv[pp][2]);
         if (p.training) {
           float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
           vt[0] = z;

@@ -183,7 +183,7 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
         for (int g = 0; g < 4; ++g)
           a[g] = wx[pp][g] + (rh[pp][g] - mu) * is * g2[pp][g] + bias[pp][g];
         const float gi = sigmoid_f(a[0]);
-        const float gg = tanhf(a[1]);
+        const float gg = tanh_f(a[1]);
         const float gf = sigmoid_f(a[2]);
         go[pp] = sigmoid_f(a[3]);
         if (p.training) {
@@ -221,7 +221,7 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
         const float cn = (c_new[pp] - mu) * is * gh[pp] + bh[pp];
         const size_t e = (size_t)pn[pp] * H + pj[pp];
         p.act_c_norm[(size_t)t * NH + e] = cn;
-        float h_new = go[pp] * tanhf(cn);
+        float h_new = go[pp] * tanh_f(cn);
         if (zoneout) {
           if (p.training) h_new = (h_new - h_prev[pp]) * mk[pp] + h_prev[pp];
           else h_new = p.zoneout_prob * h_prev[pp] + (1.0f - p.zoneout_prob) * h_new;
@@ -384,7 +384,7 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
           dh_total = s[pp].m * dh_total;
         }
         const float go = s[pp].vt[3];
-        const float c_tanh = tanhf(s[pp].cn);
+        const float c_tanh = tanh_f(s[pp].cn);
         const float do_ = c_tanh * dh_total;
         const float dln3 = d_tanh_f(c_tanh) * (go * dh_total);
         dv_o[pp] = d_sigmoid_f(go) * do_;

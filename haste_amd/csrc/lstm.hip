@@ -133,11 +133,11 @@ void lstm_forward_kernel(LstmFwdParams p) {
         for (int g = 0; g < 4; ++g)
           a[g] = wx[pp][g] + sum_product<NB, CT>(red, pl[pp], g * HS + pc[pp]) + bias[pp][g];
         gate[pp][0] = sigmoid_f(a[0]);
-        gate[pp][1] = tanhf(a[1]);
+        gate[pp][1] = tanh_f(a[1]);
         gate[pp][2] = sigmoid_f(a[2]);
         gate[pp][3] = sigmoid_f(a[3]);
         const float c_new = gate[pp][2] * c_prev[pp] + gate[pp][0] * gate[pp][1];
-        float h_new = gate[pp][3] * tanhf(c_new);
+        float h_new = gate[pp][3] * tanh_f(c_new);
         if (zoneout) {
           if (p.training) h_new = (h_new - h_prev[pp]) * mk[pp] + h_prev[pp];
           else h_new = p.zoneout_prob * h_prev[pp] + (1.0f - p.zoneout_prob) * h_new;
@@ -278,7 +278,7 @@ void lstm_backward_kernel(LstmBwdParams p) {
         const float gi = s.vt[0], gg = s.vt[1], gf = s.vt[2], go = s.vt[3];
         float dc_total = s.dcn + dc[pp];
         float dh_total = s.dhn + dh[pp];
-        const float c_tanh = tanhf(s.c1);
+        const float c_tanh = tanh_f(s.c1);
         if (zoneout) {
           dh_keep[pp] = (1.0f - s.m) * dh_total;
           dh_total = s.m * dh_total;
