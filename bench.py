@@ -27,9 +27,10 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget", type=float, default=15.0)
-    ap.add_argument("--workload", choices=["all", "metric", "streaming"], default="all",
+    ap.add_argument("--workload", choices=["all", "metric", "streaming", "copy"], default="all",
                     help="restrict the run to one workload (for profiling); the JSON line is "
-                         "only complete with 'all'")
+                         "only complete with 'all'.  'copy' runs a plain device copy of known "
+                         "size, the yardstick for the FETCH_SIZE / WRITE_SIZE counters")
     return ap.parse_args()
 
 
@@ -179,6 +180,16 @@ def main():
     torch.cuda.set_device(0)
     dev = torch.device("cuda:0")
 
+    if args.workload == "copy":
+        n = 256 * 1024 * 1024  # floats: 1 GiB read + 1 GiB written per copy
+        src = torch.ones(n, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"workload": "copy", "bytes_read_per_copy": 4 * n,
+                          "bytes_written_per_copy": 4 * n, "copies": args.steps}))
+        return
     if args.workload == "metric":
         m = run_metric(args, torch, lib, ops, dev)
         print(json.dumps({"workload": "metric", "ms_per_step": round(m["ms_per_step"], 4),
