@@ -19,6 +19,13 @@ import numpy as np
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 
+# HBM bytes per launch at the metric workload, from two rocprofv3 --pmc runs (FETCH_SIZE, then
+# WRITE_SIZE) scaled by what the same counters read for a 1 GiB device copy (--workload copy):
+# one FETCH_SIZE unit = 2.000 KiB, one WRITE_SIZE unit = 1.000 KiB.  A GEMM "launch" is the mean
+# of the step's four products, each with its share of the split-K reduce.
+MEASURED_TRAFFIC_BYTES = {"gemm_f32": 250.0e6, "lstm_forward_recurrence": 167.0e6,
+                          "lstm_backward_recurrence": 181.9e6}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -115,7 +122,8 @@ def run_metric(args, torch, lib, ops, dev):
     dom = kernels[dominant]
     roofline = {"kernel": dominant, "bound": "mfma", "achieved": dom["tflops"],
                 "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(dom["tflops"] / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None}
+                "frac": round(dom["tflops"] / PEAK_FP32_MFMA_TFLOPS, 4),
+                "traffic": MEASURED_TRAFFIC_BYTES.get(dominant)}
     total_flops = 3.0 * (f_gemm + f_rec)
     return dict(ms_per_step=ms_per_step, kernels=kernels, roofline=roofline,
                 tflops_whole_step=total_flops / (ms_per_step * 1e-3) / 1e12,
