@@ -44,7 +44,7 @@ constexpr int kCounterStride = 32;    // uint32 slots between counters (128 B ap
 struct ControlBlock {
   unsigned int step_flags[kMaxWorkgroups];                 // per-workgroup arrival counts
   unsigned int grid_exit_counter[kCounterStride];          // all workgroups of a launch
-  unsigned int tile_counter[4096];                         // split-K arrivals per output tile
+  unsigned int tile_counter[4096];                         // arrivals per column block at the end of a launch
   unsigned int xcd_ticket[16 * kCounterStride];            // per-XCD role tickets (only ever grow)
   unsigned int abort_flag[kCounterStride];                 // set when a barrier wait gives up
 };

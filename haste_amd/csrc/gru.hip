@@ -62,16 +62,13 @@ void gru_forward_kernel(GruFwdParams p) {
   zero_tile_share(gs, xh, tile_floats, NB, j0 / 4,
                   (role.cw == p.ls.gx - 1 ? Kpad - j0 : HS) / 4);
 
-  for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
-    const int k = idx / NCOLS, cidx = idx % NCOLS;
-    const int gate = cidx / HS, j = j0 + cidx % HS;
-    float w = 0.f;
-    if (k < H && gate < 3 && j < H) {
-      const size_t off = (size_t)k * 3 * H + gate * H + j;
-      w = p.R[off];
-      if (p.dc_mask != nullptr) w = w * p.dc_mask[off] * p.dc_scale;
-    }
-    w_lds[slice_index(k, cidx, NCOLS)] = w;
+  {
+    const bool fast = H % 4 == 0 && ((reinterpret_cast<uintptr_t>(p.R) |
+                                      reinterpret_cast<uintptr_t>(p.dc_mask)) & 15u) == 0;
+    fill_slice<NCOLS>(w_lds, Kpad, p.R, p.dc_mask, p.dc_scale, fast, [=](int k, int col) {
+      const int gate = col / HS, j = j0 + col % HS;
+      return (k < H && gate < 3 && j < H) ? (long long)k * 3 * H + gate * H + j : -1ll;
+    });
   }
 
   int pn[PP], pj[PP], pl[PP], pc[PP];
@@ -223,12 +220,12 @@ void gru_backward_kernel(GruBwdParams p) {
   zero_tile_share(gs, xdq, tile_floats, NB, 12 * role.cw,
                   (role.cw == p.ls.gx - 1 ? Kpad - 48 * role.cw : 48) / 4);
 
-  for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
-    const int k = idx / NCOLS, cidx = idx % NCOLS;
-    const int unit = k / 3, gate = k % 3;
-    float w = 0.f;
-    if (unit < H && j0 + cidx < H) w = p.R_t[((size_t)gate * H + unit) * H + j0 + cidx];
-    w_lds[slice_index(k, cidx, NCOLS)] = w;
+  {
+    const bool fast = H % 4 == 0 && (reinterpret_cast<uintptr_t>(p.R_t) & 15u) == 0;
+    fill_slice<NCOLS>(w_lds, Kpad, p.R_t, nullptr, 1.0f, fast, [=](int k, int col) {
+      const int unit = k / 3, gate = k % 3;
+      return (unit < H && j0 + col < H) ? ((long long)gate * H + unit) * H + j0 + col : -1ll;
+    });
   }
 
   int pn[PP], pj[PP], pl[PP], pc[PP];
@@ -349,12 +346,12 @@ void gru_backward_kernel(GruBwdParams p) {
     const int g = tid / HSB, jj = tid % HSB;
     float s = 0.f;
     for (int r = 0; r < NB; ++r) s += red[(r * 6 + g) * HSB + jj];
-    if (j0 + jj < H) p.db_partial[(size_t)role.bt * 6 * H + g * H + j0 + jj] = s;
+    if (j0 + jj < H) store_agent(&p.db_partial[(size_t)role.bt * 6 * H + g * H + j0 + jj], s);
   }
-  if (grid_last_arrival(p.ls.cb, (unsigned)(p.ls.gx * p.ls.gy), &s_flag)) {
-    for (int col = tid; col < 6 * H; col += 256) {
-      float s = 0.f;
-      for (int bt = 0; bt < p.ls.gy; ++bt) s += p.db_partial[(size_t)bt * 6 * H + col];
+  if (column_last_arrival(p.ls.cb, role.cw, (unsigned)p.ls.gy, &s_flag)) {
+    if (tid < 6 * HSB && j0 + tid % HSB < H) {
+      const int col = (tid / HSB) * H + j0 + tid % HSB;
+      const float s = sum_over_tiles(p.db_partial + col, (size_t)6 * H, p.ls.gy);
       if (col < 3 * H) p.dbx[col] += s;
       else p.dbr[col - 3 * H] += s;
     }

@@ -68,12 +68,12 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
   // Own k range of the exchange tiles (the last workgroup also owns the padding).
   zero_tile_share(gs, xh, tile_floats, NB, j0 / 4, (role.cw == gx - 1 ? Kpad - j0 : HS) / 4);
 
-  for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
-    const int k = idx / NCOLS, cidx = idx % NCOLS;
-    const int gate = cidx / HS, j = j0 + cidx % HS;
-    float w = 0.f;
-    if (k < H && gate < 3 && j < H) w = p.R[(size_t)k * 3 * H + gate * H + j];
-    w_lds[slice_index(k, cidx, NCOLS)] = w;
+  {
+    const bool fast = H % 4 == 0 && (reinterpret_cast<uintptr_t>(p.R) & 15u) == 0;
+    fill_slice<NCOLS>(w_lds, Kpad, p.R, nullptr, 1.0f, fast, [=](int k, int col) {
+      const int gate = col / HS, j = j0 + col % HS;
+      return (k < H && gate < 3 && j < H) ? (long long)k * 3 * H + gate * H + j : -1ll;
+    });
   }
 
   int pn[PP], pj[PP], pl[PP], pc[PP];
@@ -257,12 +257,12 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
   zero_tile_share(gs, xdq, tile_floats, NB, 12 * role.cw,
                   (role.cw == gx - 1 ? Kpad - 48 * role.cw : 48) / 4);
 
-  for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
-    const int k = idx / NCOLS, cidx = idx % NCOLS;
-    const int unit = k / 3, gate = k % 3;
-    float w = 0.f;
-    if (unit < H && j0 + cidx < H) w = p.R_t[((size_t)gate * H + unit) * H + j0 + cidx];
-    w_lds[slice_index(k, cidx, NCOLS)] = w;
+  {
+    const bool fast = H % 4 == 0 && (reinterpret_cast<uintptr_t>(p.R_t) & 15u) == 0;
+    fill_slice<NCOLS>(w_lds, Kpad, p.R_t, nullptr, 1.0f, fast, [=](int k, int col) {
+      const int unit = k / 3, gate = k % 3;
+      return (unit < H && j0 + col < H) ? ((long long)gate * H + unit) * H + j0 + col : -1ll;
+    });
   }
 
   int pn[PP], pj[PP], pl[PP], pc[PP];
@@ -410,13 +410,12 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
     const int a = tid / HSB, jj = tid % HSB;
     float sum = 0.f;
     for (int r = 0; r < NB; ++r) sum += red[(r * NACC + a) * HSB + jj];
-    if (j0 + jj < H) p.col_partial[((size_t)role.bt * NACC + a) * H + j0 + jj] = sum;
+    if (j0 + jj < H) store_agent(&p.col_partial[((size_t)role.bt * NACC + a) * H + j0 + jj], sum);
   }
-  if (grid_last_arrival(p.ls.cb, (unsigned)(p.ls.gx * p.ls.gy), &s_flag)) {
-    for (int idx = tid; idx < NACC * H; idx += 256) {
-      const int a = idx / H, col = idx % H;
-      float sum = 0.f;
-      for (int bt = 0; bt < p.ls.gy; ++bt) sum += p.col_partial[((size_t)bt * NACC + a) * H + col];
+  if (column_last_arrival(p.ls.cb, role.cw, (unsigned)p.ls.gy, &s_flag)) {
+    if (tid < NACC * HSB && j0 + tid % HSB < H) {
+      const int a = tid / HSB, col = j0 + tid % HSB;
+      const float sum = sum_over_tiles(p.col_partial + (size_t)a * H + col, (size_t)NACC * H, p.ls.gy);
       if (a < 3) p.dbx[a * H + col] += sum;
       else if (a < 6) p.dbr[(a - 3) * H + col] += sum;
       else p.dgamma2[(a - 6) * H + col] += sum;

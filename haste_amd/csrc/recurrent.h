@@ -253,6 +253,47 @@ __device__ __forceinline__ bool grid_last_arrival(ControlBlock* cb, unsigned int
   return *flag != 0u;
 }
 
+// Publishing without cache-wide fences: agent-scope stores (store_agent) before an arrival,
+// agent-scope loads (load_exchanged) after it.  The release/acquire fences of
+// grid_last_arrival write back and invalidate whole caches instead.
+__device__ __forceinline__ void store_agent(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// True in the last of the `gy` workgroups with column index `cw` (one per batch tile) to
+// call it; data is published with store_agent before and read with load_exchanged after
+// the call.  Lets every column block
+// finish its own column sums instead of one workgroup finishing all of them.
+__device__ __forceinline__ bool column_last_arrival(ControlBlock* cb, int cw, unsigned int gy,
+                                                    unsigned int* flag) {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const unsigned int old = __hip_atomic_fetch_add(&cb->tile_counter[cw], 1u, __ATOMIC_RELAXED,
+                                                    __HIP_MEMORY_SCOPE_AGENT);
+    const bool last = old == gy - 1;
+    if (last)
+      __hip_atomic_store(&cb->tile_counter[cw], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *flag = last ? 1u : 0u;
+  }
+  __syncthreads();
+  return *flag != 0u;
+}
+
+// base[0] + base[stride] + ... (gy terms, in that order), read with agent-scope loads that
+// are issued eight at a time.
+__device__ __forceinline__ float sum_over_tiles(const float* base, size_t stride, int gy) {
+  float s = 0.f;
+  for (int b0 = 0; b0 < gy; b0 += 8) {
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = b0 + i < gy ? load_exchanged(base + (size_t)(b0 + i) * stride) : 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s += v[i];
+  }
+  return s;
+}
+
 __device__ __forceinline__ int round_up(int x, int m) { return (x + m - 1) / m * m; }
 
 // LDS image of a weight slice: element (k, col) of a [Kpad x NCOLS] slice lives at
@@ -261,6 +302,69 @@ __device__ __forceinline__ int round_up(int x, int m) { return (x + m - 1) / m *
 // lanes of a k-quarter read 16 consecutive such vectors (no bank conflicts).
 __device__ __forceinline__ int slice_index(int k, int col, int ncols) {
   return ((((k >> 4) << 2) + ((k & 15) >> 2)) * ncols + col) * 4 + (k & 3);
+}
+
+// Fills the resident slice.  `offset(k, col)` is the element's index in `src` (and in
+// `mask`, when DropConnect is fused) or -1 for padding; the four columns of an aligned
+// column quad must be adjacent in memory whenever the quad's first and last are valid
+// (true for the gate-block layouts of R and R_t).  A thread takes 4 consecutive k of one
+// column quad: four 16-byte loads, all issued before the first use (several items per
+// thread are in flight at once), a 4x4 transpose in registers, four 16-byte LDS stores.
+// `fast`: src (and mask) are 16-byte aligned, every valid quad starts at a multiple of 4
+// elements and no quad is partly valid (row lengths and column origins are multiples of
+// 4); otherwise the slice is filled element by element.
+template <int NCOLS, class OffsetFn>
+__device__ __forceinline__ void fill_slice(float* w_lds, int Kpad, const float* __restrict__ src,
+                                           const float* __restrict__ mask, float scale, bool fast,
+                                           OffsetFn offset) {
+  const int tid = threadIdx.x;
+  if (!fast) {
+    for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
+      const int k = idx / NCOLS, col = idx % NCOLS;
+      const long long off = offset(k, col);
+      float w = 0.f;
+      if (off >= 0) {
+        w = src[off];
+        if (mask != nullptr) w = w * mask[off] * scale;
+      }
+      w_lds[slice_index(k, col, NCOLS)] = w;
+    }
+    return;
+  }
+  constexpr int QUADS = NCOLS / 4;
+  constexpr int UNROLL = 4;
+  const int items = (Kpad / 4) * QUADS;
+  const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+  for (int base = tid; base < items; base += 256 * UNROLL) {
+    float4_t v[UNROLL][4];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int item = base + 256 * u;
+      const int k4 = item / QUADS, col = (item % QUADS) * 4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const long long o0 = item < items ? offset(4 * k4 + i, col) : -1;
+        const long long o3 = item < items ? offset(4 * k4 + i, col + 3) : -1;
+        const bool whole = o0 >= 0 && o3 >= 0;
+        float4_t w = *reinterpret_cast<const float4_t*>(src + (whole ? o0 : 0));
+        if (mask != nullptr)
+          w = w * *reinterpret_cast<const float4_t*>(mask + (whole ? o0 : 0)) * scale;
+        v[u][i] = whole ? w : zero4;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int item = base + 256 * u;
+      if (item < items) {
+        const int k4 = item / QUADS, col = (item % QUADS) * 4;
+        float* dst = w_lds + ((size_t)k4 * NCOLS + col) * 4;
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          *reinterpret_cast<float4_t*>(dst + 4 * c) =
+              float4_t{v[u][0][c], v[u][1][c], v[u][2][c], v[u][3][c]};
+      }
+    }
+  }
 }
 
 // MFMAs of k-groups [g_abs, g_abs+CHUNK): one straight-line block (no branches, so the
