@@ -15,7 +15,8 @@ struct GruFwdParams {
   const float* R;        // [H,3H]
   const float* bx;       // [3H]
   const float* br;       // [3H]
-  float* h;              // [T+1,N,H]
+  const float* h;        // [N,H] state before the first step
+  float* h_out;          // [T,N,H] states after each step (may start at h + N*H)
   float* v;              // [T,N,4H] (training) or null
   const float* Wx;       // [T,N,3H] = x*W
   float zoneout_prob;
@@ -154,7 +155,7 @@ void gru_forward_kernel(GruFwdParams p) {
 #pragma unroll
           for (int g = 0; g < 4; ++g) vt[g * H] = saved[pp][g];
         }
-        p.h[(size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp]] = h_prev[pp];
+        p.h_out[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]] = h_prev[pp];
       }
     }
   }
@@ -163,9 +164,9 @@ void gru_forward_kernel(GruFwdParams p) {
 struct GruBwdParams {
   int T, N, H;
   const float* R_t;     // [3H,H]
-  const float* h;       // [T+1,N,H]
+  const float* h;       // [T,N,H] states before each step
   const float* v;       // [T,N,4H]
-  const float* dh_new;  // [T+1,N,H]
+  const float* dh_next; // [T,N,H] upstream gradient of the h each step produced
   float* dbx;           // [3H] accumulated
   float* dbr;           // [3H] accumulated
   float* dh;            // [N,H] in/out
@@ -258,7 +259,7 @@ void gru_backward_kernel(GruBwdParams p) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) s.vt[g] = vt[g * H];
         s.h0 = p.h[(size_t)t * NH + e];
-        s.dhn = p.dh_new[(size_t)(t + 1) * NH + e];
+        s.dhn = p.dh_next[(size_t)t * NH + e];
         if (zoneout) s.m = p.zoneout_mask[(size_t)t * NH + e];
       }
       nxt[pp] = s;
@@ -360,12 +361,14 @@ void gru_backward_kernel(GruBwdParams p) {
 
 }  // namespace
 
+// h: [N,H] state before the first step; h_out: [T,N,H] states after each step.
 int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int H,
                      const float* W, const float* R, const float* bx, const float* br,
-                     const float* x, float* h, float* v, float* tmp_Wx, float zoneout_prob,
-                     const float* zoneout_mask, const float* dc_mask, float dc_scale) {
+                     const float* x, const float* h, float* h_out, float* v, float* tmp_Wx,
+                     float zoneout_prob, const float* zoneout_mask, const float* dc_mask,
+                     float dc_scale) {
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
-  HASTE_HIP_REQUIRE(W && R && bx && br && x && h && tmp_Wx);
+  HASTE_HIP_REQUIRE(W && R && bx && br && x && h && h_out && tmp_Wx);
   HASTE_HIP_REQUIRE(!training || v != nullptr);
   const ForwardTile tile = pick_forward_tile(3, N, H, 0);
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
@@ -378,7 +381,7 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
 
   GruFwdParams p;
   p.training = training; p.T = T; p.N = N; p.H = H;
-  p.R = R; p.bx = bx; p.br = br; p.h = h; p.v = v; p.Wx = tmp_Wx;
+  p.R = R; p.bx = bx; p.br = br; p.h = h; p.h_out = h_out; p.v = v; p.Wx = tmp_Wx;
   p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
   p.dc_mask = dc_mask; p.dc_scale = dc_scale;
   p.xh = ws.scratch;
@@ -400,11 +403,11 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
 
 int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
                       const float* W_t, const float* R_t, const float* x_t, const float* h,
-                      const float* v, const float* dh_new, float* dx, float* dW, float* dR,
+                      const float* v, const float* dh_next, float* dx, float* dW, float* dR,
                       float* dbx, float* dbr, float* dh, float* dp, float* dq,
                       const float* zoneout_mask) {
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
-  HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && v && dh_new);
+  HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && v && dh_next);
   HASTE_HIP_REQUIRE(dx && dW && dR && dbx && dbr && dh && dp && dq);
   // per row: the partial tiles or the 6 bias-gradient columns of 16 floats
   const BackwardTile tile = pick_backward_tile(gru_backward_k(H), N, H, 6 * 16, 0);
@@ -418,7 +421,7 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
 
   GruBwdParams p;
   p.T = T; p.N = N; p.H = H;
-  p.R_t = R_t; p.h = h; p.v = v; p.dh_new = dh_new;
+  p.R_t = R_t; p.h = h; p.v = v; p.dh_next = dh_next;
   p.dbx = dbx; p.dbr = dbr; p.dh = dh; p.dp = dp; p.dq = dq; p.zoneout_mask = zoneout_mask;
   p.db_partial = ws.scratch;
   p.xdq = ws.scratch + db_floats;
@@ -451,8 +454,10 @@ int haste_hip_gru_forward_f32(int training, int steps, int batch_size, int input
                               const float* x, float* h, float* v, float* tmp_Wx, float* tmp_Rh,
                               float zoneout_prob, const float* zoneout_mask, void* stream) {
   (void)tmp_Rh;
+  HASTE_HIP_REQUIRE(h && batch_size > 0 && hidden_size > 0);
   return haste_hip::gru_forward_impl(haste_hip::as_stream(stream), training, steps, batch_size,
-                                     input_size, hidden_size, W, R, bx, br, x, h, v, tmp_Wx,
+                                     input_size, hidden_size, W, R, bx, br, x, h,
+                                     h + (size_t)batch_size * hidden_size, v, tmp_Wx,
                                      zoneout_prob, zoneout_mask, nullptr, 1.0f);
 }
 
@@ -464,8 +469,10 @@ int haste_hip_gru_forward_dropconnect_f32(int training, int steps, int batch_siz
                                           const float* zoneout_mask,
                                           const float* dropconnect_mask, float dropconnect_scale,
                                           void* stream) {
+  HASTE_HIP_REQUIRE(h && batch_size > 0 && hidden_size > 0);
   return haste_hip::gru_forward_impl(haste_hip::as_stream(stream), training, steps, batch_size,
-                                     input_size, hidden_size, W, R, bx, br, x, h, v, tmp_Wx,
+                                     input_size, hidden_size, W, R, bx, br, x, h,
+                                     h + (size_t)batch_size * hidden_size, v, tmp_Wx,
                                      zoneout_prob, zoneout_mask, dropconnect_mask,
                                      dropconnect_scale);
 }
@@ -478,7 +485,35 @@ int haste_hip_gru_backward_f32(int steps, int batch_size, int input_size, int hi
                                const float* zoneout_mask, void* stream) {
   (void)bx;
   (void)br;
+  HASTE_HIP_REQUIRE(dh_new && batch_size > 0 && hidden_size > 0);
   return haste_hip::gru_backward_impl(haste_hip::as_stream(stream), steps, batch_size, input_size,
+                                      hidden_size, W_t, R_t, x_t, h, v,
+                                      dh_new + (size_t)batch_size * hidden_size, dx, dW, dR, dbx,
+                                      dbr, dh, dp, dq, zoneout_mask);
+}
+
+int haste_hip_gru_forward_iterate_f32(int training, int batch_size, int input_size,
+                                      int hidden_size,
+                                      const float* W, const float* R, const float* bx,
+                                      const float* br, const float* x, const float* h,
+                                      float* h_out, float* v, float* tmp_Wx, float* tmp_Rh,
+                                      float zoneout_prob, const float* zoneout_mask,
+                                      void* stream) {
+  (void)tmp_Rh;
+  return haste_hip::gru_forward_impl(haste_hip::as_stream(stream), training, 1, batch_size,
+                                     input_size, hidden_size, W, R, bx, br, x, h, h_out, v, tmp_Wx,
+                                     zoneout_prob, zoneout_mask, nullptr, 1.0f);
+}
+
+int haste_hip_gru_backward_iterate_f32(int batch_size, int input_size, int hidden_size,
+                                       const float* W_t, const float* R_t, const float* bx,
+                                       const float* br, const float* x_t, const float* h,
+                                       const float* v, const float* dh_new, float* dx, float* dW,
+                                       float* dR, float* dbx, float* dbr, float* dh, float* dp,
+                                       float* dq, const float* zoneout_mask, void* stream) {
+  (void)bx;
+  (void)br;
+  return haste_hip::gru_backward_impl(haste_hip::as_stream(stream), 1, batch_size, input_size,
                                       hidden_size, W_t, R_t, x_t, h, v, dh_new, dx, dW, dR, dbx,
                                       dbr, dh, dp, dq, zoneout_mask);
 }

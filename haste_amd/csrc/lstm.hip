@@ -14,8 +14,10 @@ struct LstmFwdParams {
   int training, T, N, H;
   const float* R;       // [H,4H]
   const float* b;       // [4H]
-  float* h;             // [T+1,N,H]
-  float* c;             // [T+1,N,H]
+  const float* h;       // [N,H] state before the first step
+  const float* c;       // [N,H]
+  float* h_out;         // [T,N,H] states after each step (may start at h + N*H)
+  float* c_out;         // [T,N,H]
   float* v;             // [T,N,4H] in: x*W, out (training): activations
   float zoneout_prob;
   const float* zoneout_mask;   // [T,N,H] or null
@@ -154,9 +156,9 @@ void lstm_forward_kernel(LstmFwdParams p) {
 #pragma unroll
           for (int g = 0; g < 4; ++g) vt[g * H] = gate[pp][g];
         }
-        const size_t o = (size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp];
-        p.c[o] = c_prev[pp];
-        p.h[o] = h_prev[pp];
+        const size_t o = (size_t)t * NH + (size_t)pn[pp] * H + pj[pp];
+        p.c_out[o] = c_prev[pp];
+        p.h_out[o] = h_prev[pp];
       }
     }
   }
@@ -165,9 +167,10 @@ void lstm_forward_kernel(LstmFwdParams p) {
 struct LstmBwdParams {
   int T, N, H;
   const float* R_t;     // [4H,H]
-  const float* c;       // [T+1,N,H]
-  const float* dh_new;  // [T+1,N,H]
-  const float* dc_new;  // [T+1,N,H]
+  const float* c;       // [T,N,H] cell state before each step
+  const float* c_next;  // [T,N,H] cell state after each step (may be c + N*H)
+  const float* dh_next; // [T,N,H] upstream gradient of the h each step produced
+  const float* dc_next; // [T,N,H] same for c
   float* db;            // [4H] accumulated
   float* dh;            // [N,H] in/out
   float* dc;            // [N,H] in/out
@@ -252,9 +255,9 @@ void lstm_backward_kernel(LstmBwdParams p) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) s.vt[g] = vt[g * H];
         s.c0 = p.c[(size_t)t * NH + e];
-        s.c1 = p.c[(size_t)(t + 1) * NH + e];
-        s.dhn = p.dh_new[(size_t)(t + 1) * NH + e];
-        s.dcn = p.dc_new[(size_t)(t + 1) * NH + e];
+        s.c1 = p.c_next[(size_t)t * NH + e];
+        s.dhn = p.dh_next[(size_t)t * NH + e];
+        s.dcn = p.dc_next[(size_t)t * NH + e];
         if (zoneout) s.m = p.zoneout_mask[(size_t)t * NH + e];
       }
       nxt[pp] = s;
@@ -358,12 +361,14 @@ void lstm_backward_kernel(LstmBwdParams p) {
 
 }  // namespace
 
+// h, c: [N,H] state before the first step; h_out, c_out: [T,N,H] states after each step.
 int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int H,
                       const float* W, const float* R, const float* b, const float* x,
-                      float* h, float* c, float* v, float zoneout_prob,
-                      const float* zoneout_mask, const float* dc_mask, float dc_scale) {
+                      const float* h, const float* c, float* h_out, float* c_out, float* v,
+                      float zoneout_prob, const float* zoneout_mask, const float* dc_mask,
+                      float dc_scale) {
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
-  HASTE_HIP_REQUIRE(W && R && b && x && h && c && v);
+  HASTE_HIP_REQUIRE(W && R && b && x && h && c && h_out && c_out && v);
   const ForwardTile tile = pick_forward_tile(4, N, H, 0);
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   // v = x * W for all steps at once.
@@ -376,7 +381,7 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
 
   LstmFwdParams p;
   p.training = training; p.T = T; p.N = N; p.H = H;
-  p.R = R; p.b = b; p.h = h; p.c = c; p.v = v;
+  p.R = R; p.b = b; p.h = h; p.c = c; p.h_out = h_out; p.c_out = c_out; p.v = v;
   p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
   p.dc_mask = dc_mask; p.dc_scale = dc_scale;
   p.xh = ws.scratch;
@@ -396,13 +401,16 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
   return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 }
 
+// h, c: [T,N,H] states before each step; c_next: [T,N,H] cell states after each step;
+// dh_next, dc_next: [T,N,H] upstream gradients of the states each step produced.
 int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
                        const float* W_t, const float* R_t, const float* x_t,
-                       const float* h, const float* c, const float* dh_new, const float* dc_new,
+                       const float* h, const float* c, const float* c_next,
+                       const float* dh_next, const float* dc_next,
                        float* dx, float* dW, float* dR, float* db, float* dh, float* dc, float* v,
                        const float* zoneout_mask) {
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
-  HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && c && dh_new && dc_new);
+  HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && c && c_next && dh_next && dc_next);
   HASTE_HIP_REQUIRE(dx && dW && dR && db && dh && dc && v);
   const BackwardTile tile = pick_backward_tile(4 * H, N, H, 4 * 16, 0);
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
@@ -415,7 +423,7 @@ int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
 
   LstmBwdParams p;
   p.T = T; p.N = N; p.H = H;
-  p.R_t = R_t; p.c = c; p.dh_new = dh_new; p.dc_new = dc_new;
+  p.R_t = R_t; p.c = c; p.c_next = c_next; p.dh_next = dh_next; p.dc_next = dc_next;
   p.db = db; p.dh = dh; p.dc = dc; p.v = v; p.zoneout_mask = zoneout_mask;
   p.db_partial = ws.scratch;
   p.xdv = ws.scratch + (db_floats + 3) / 4 * 4;
@@ -449,9 +457,11 @@ int haste_hip_lstm_forward_f32(int training, int steps, int batch_size, int inpu
                                float* h, float* c, float* v, float* tmp_Rh,
                                float zoneout_prob, const float* zoneout_mask, void* stream) {
   (void)tmp_Rh;  // the recurrent product never leaves the chip
+  HASTE_HIP_REQUIRE(h && c && batch_size > 0 && hidden_size > 0);
+  const size_t NH = (size_t)batch_size * hidden_size;
   return haste_hip::lstm_forward_impl(haste_hip::as_stream(stream), training, steps, batch_size,
-                                      input_size, hidden_size, W, R, b, x, h, c, v, zoneout_prob,
-                                      zoneout_mask, nullptr, 1.0f);
+                                      input_size, hidden_size, W, R, b, x, h, c, h + NH, c + NH, v,
+                                      zoneout_prob, zoneout_mask, nullptr, 1.0f);
 }
 
 int haste_hip_lstm_forward_dropconnect_f32(int training, int steps, int batch_size,
@@ -461,9 +471,12 @@ int haste_hip_lstm_forward_dropconnect_f32(int training, int steps, int batch_si
                                            float zoneout_prob, const float* zoneout_mask,
                                            const float* dropconnect_mask, float dropconnect_scale,
                                            void* stream) {
+  HASTE_HIP_REQUIRE(h && c && batch_size > 0 && hidden_size > 0);
+  const size_t NH = (size_t)batch_size * hidden_size;
   return haste_hip::lstm_forward_impl(haste_hip::as_stream(stream), training, steps, batch_size,
-                                      input_size, hidden_size, W, R, b, x, h, c, v, zoneout_prob,
-                                      zoneout_mask, dropconnect_mask, dropconnect_scale);
+                                      input_size, hidden_size, W, R, b, x, h, c, h + NH, c + NH, v,
+                                      zoneout_prob, zoneout_mask, dropconnect_mask,
+                                      dropconnect_scale);
 }
 
 int haste_hip_lstm_backward_f32(int steps, int batch_size, int input_size, int hidden_size,
@@ -474,9 +487,37 @@ int haste_hip_lstm_backward_f32(int steps, int batch_size, int input_size, int h
                                 float* dh, float* dc, float* v,
                                 const float* zoneout_mask, void* stream) {
   (void)b;  // unused by the reference as well (lib/lstm_backward_gpu.cu.cc:319-405)
+  HASTE_HIP_REQUIRE(c && dh_new && dc_new && batch_size > 0 && hidden_size > 0);
+  const size_t NH = (size_t)batch_size * hidden_size;
   return haste_hip::lstm_backward_impl(haste_hip::as_stream(stream), steps, batch_size, input_size,
-                                       hidden_size, W_t, R_t, x_t, h, c, dh_new, dc_new, dx, dW,
-                                       dR, db, dh, dc, v, zoneout_mask);
+                                       hidden_size, W_t, R_t, x_t, h, c, c + NH, dh_new + NH,
+                                       dc_new + NH, dx, dW, dR, db, dh, dc, v, zoneout_mask);
+}
+
+int haste_hip_lstm_forward_iterate_f32(int training, int batch_size, int input_size,
+                                       int hidden_size,
+                                       const float* W, const float* R, const float* b,
+                                       const float* x, const float* h, const float* c,
+                                       float* h_out, float* c_out, float* v, float* tmp_Rh,
+                                       float zoneout_prob, const float* zoneout_mask,
+                                       void* stream) {
+  (void)tmp_Rh;
+  return haste_hip::lstm_forward_impl(haste_hip::as_stream(stream), training, 1, batch_size,
+                                      input_size, hidden_size, W, R, b, x, h, c, h_out, c_out, v,
+                                      zoneout_prob, zoneout_mask, nullptr, 1.0f);
+}
+
+int haste_hip_lstm_backward_iterate_f32(int batch_size, int input_size, int hidden_size,
+                                        const float* W_t, const float* R_t, const float* b,
+                                        const float* x_t, const float* h, const float* c,
+                                        const float* c_new, const float* dh_new,
+                                        const float* dc_new, float* dx, float* dW, float* dR,
+                                        float* db, float* dh, float* dc, float* v,
+                                        const float* zoneout_mask, void* stream) {
+  (void)b;
+  return haste_hip::lstm_backward_impl(haste_hip::as_stream(stream), 1, batch_size, input_size,
+                                       hidden_size, W_t, R_t, x_t, h, c, c_new, dh_new, dc_new, dx,
+                                       dW, dR, db, dh, dc, v, zoneout_mask);
 }
 
 }  // extern "C"

@@ -213,6 +213,19 @@ const char* haste_hip_error_string(int code) {
 
 const char* haste_hip_last_runtime_error(void) { return haste_hip::g_last_error.c_str(); }
 
+int haste_hip_stream_order(void* first, void* then) {
+  if (first == then) return HASTE_HIP_OK;
+  hipEvent_t ev;
+  HASTE_HIP_TRY(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+  hipError_t err = hipEventRecord(ev, haste_hip::as_stream(first));
+  if (err == hipSuccess) err = hipStreamWaitEvent(haste_hip::as_stream(then), ev, 0);
+  // Destroying a recorded event is legal: its resources are released once it has completed.
+  const hipError_t err2 = hipEventDestroy(ev);
+  HASTE_HIP_TRY(err);
+  HASTE_HIP_TRY(err2);
+  return HASTE_HIP_OK;
+}
+
 int haste_hip_max_hidden_size(int gates, int batch_size) {
   if (gates < 1 || gates > 4 || batch_size < 1) return 0;
   const int cus = haste_hip::device_cu_count();

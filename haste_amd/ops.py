@@ -83,6 +83,71 @@ def lstm_backward(x_t, kernel_t, recurrent_kernel_t, bias, zoneout_mask, h, c, c
     return dx, dh, dc, dW, dR, db
 
 
+# ---- single LSTM steps (reference lib/haste/lstm.h:73-86,201-219; no binding of the
+# reference exposes them, examples/lstm.cc:252,309 calls them from C++) ------------------
+def lstm_forward_iterate(training, zoneout_prob, x, h, c, kernel, recurrent_kernel, bias,
+                         zoneout_mask=None, h_out=None, c_out=None):
+    """One step: x[N,C], h,c[N,H] -> h_out,c_out[N,H], v[N,4H] (activations when training)."""
+    N, C = x.shape
+    H = recurrent_kernel.shape[0]
+    _check(x, h, c, kernel, recurrent_kernel, bias)
+    h_out = torch.empty_like(h) if h_out is None else h_out
+    c_out = torch.empty_like(c) if c_out is None else c_out
+    v = torch.empty(N, 4 * H, device=x.device, dtype=x.dtype)
+    has_zoneout = bool(zoneout_prob) and zoneout_mask is not None and zoneout_mask.numel() > 0
+    lib.call("haste_hip_lstm_forward_iterate_f32", bool(training), N, C, H, kernel, recurrent_kernel,
+             bias, x, h, c, h_out, c_out, v, None, float(zoneout_prob) if has_zoneout else 0.0,
+             zoneout_mask if has_zoneout else None)
+    return h_out, c_out, v
+
+
+def lstm_backward_iterate(x_t, kernel_t, recurrent_kernel_t, bias, h, c, c_new, dh_new, dc_new, v,
+                          dW, dR, db, dh, dc, zoneout_mask=None):
+    """One reverse step: x_t[C,N]; h,c = states before the step, c_new = cell state after it;
+    dW, dR, db are accumulated into, dh, dc updated in place, v consumed.  Returns dx[N,C]."""
+    C, N = x_t.shape
+    H = recurrent_kernel_t.shape[1]
+    _check(x_t, kernel_t, recurrent_kernel_t, bias, h, c, c_new, dh_new, dc_new, v, dW, dR, db, dh, dc)
+    dx = torch.empty(N, C, device=x_t.device, dtype=x_t.dtype)
+    has_zoneout = zoneout_mask is not None and zoneout_mask.numel() > 0
+    lib.call("haste_hip_lstm_backward_iterate_f32", N, C, H, kernel_t, recurrent_kernel_t, bias, x_t,
+             h, c, c_new, dh_new, dc_new, dx, dW, dR, db, dh, dc, v,
+             zoneout_mask if has_zoneout else None)
+    return dx
+
+
+# ---- single GRU steps (reference lib/haste/gru.h:72-84,172-189) -------------------------
+def gru_forward_iterate(training, zoneout_prob, x, h, kernel, recurrent_kernel, bias,
+                        recurrent_bias, zoneout_mask=None, h_out=None):
+    N, C = x.shape
+    H = recurrent_kernel.shape[0]
+    _check(x, h, kernel, recurrent_kernel, bias, recurrent_bias)
+    h_out = torch.empty_like(h) if h_out is None else h_out
+    v = torch.empty(N, 4 * H, device=x.device, dtype=x.dtype)
+    tmp_Wx = torch.empty(N, 3 * H, device=x.device, dtype=x.dtype)
+    has_zoneout = bool(zoneout_prob) and zoneout_mask is not None and zoneout_mask.numel() > 0
+    lib.call("haste_hip_gru_forward_iterate_f32", bool(training), N, C, H, kernel, recurrent_kernel,
+             bias, recurrent_bias, x, h, h_out, v, tmp_Wx, None,
+             float(zoneout_prob) if has_zoneout else 0.0, zoneout_mask if has_zoneout else None)
+    return h_out, v
+
+
+def gru_backward_iterate(x_t, kernel_t, recurrent_kernel_t, bias, recurrent_bias, h, v, dh_new,
+                         dW, dR, dbx, dbr, dh, zoneout_mask=None):
+    C, N = x_t.shape
+    H = recurrent_kernel_t.shape[1]
+    _check(x_t, kernel_t, recurrent_kernel_t, bias, recurrent_bias, h, v, dh_new, dW, dR, dbx, dbr, dh)
+    opts = dict(device=x_t.device, dtype=x_t.dtype)
+    dx = torch.empty(N, C, **opts)
+    dp = torch.empty(N, 3 * H, **opts)
+    dq = torch.empty(N, 3 * H, **opts)
+    has_zoneout = zoneout_mask is not None and zoneout_mask.numel() > 0
+    lib.call("haste_hip_gru_backward_iterate_f32", N, C, H, kernel_t, recurrent_kernel_t, bias,
+             recurrent_bias, x_t, h, v, dh_new, dx, dW, dR, dbx, dbr, dh, dp, dq,
+             zoneout_mask if has_zoneout else None)
+    return dx
+
+
 # ---- GRU (reference frameworks/pytorch/gru.cc:30-163) -----------------------
 def gru_forward(training, zoneout_prob, x, h0, kernel, recurrent_kernel, bias, recurrent_bias,
                 zoneout_mask, dropconnect_mask=None, dropconnect_scale=1.0):

@@ -37,7 +37,12 @@ class ForwardPass {
         T* tmp_Wx,
         T* tmp_Rh,
         const float zoneout_prob,
-        const T* zoneout_mask);
+        const T* zoneout_mask) {
+      data_.status = haste_hip_gru_forward_iterate_f32(
+          data_.training, data_.batch_size, data_.input_size, data_.hidden_size,
+          W, R, bx, br, x, h, h_out, v, tmp_Wx, tmp_Rh, zoneout_prob, zoneout_mask,
+          detail::stream_arg(data_.stream));
+    }
 
     // W[C,3H] R[H,3H] bx,br[3H] x[T,N,C]; h[T+1,N,H] with slot 0 preset; v[T,N,4H]
     // (z, r, g, Rh_g+br_g; may be null when not training); tmp_Wx[T,N,3H] receives x*W;
@@ -99,7 +104,12 @@ class BackwardPass {
         T* dh,
         T* dp,
         T* dq,
-        const T* zoneout_mask);
+        const T* zoneout_mask) {
+      data_.status = haste_hip_gru_backward_iterate_f32(
+          data_.batch_size, data_.input_size, data_.hidden_size,
+          W_t, R_t, bx, br, x_t, h, v, dh_new, dx, dW, dR, dbx, dbr, dh, dp, dq, zoneout_mask,
+          detail::stream_arg(data_.stream));
+    }
 
     // W_t[3H,C] R_t[3H,H] x_t[C,T,N] h[T+1,N,H] v[T,N,4H] dh_new[T+1,N,H];
     // dx[T,N,C] assigned; dW,dR,dbx,dbr accumulated into; dh[N,H] in/out;

@@ -27,7 +27,7 @@ class ForwardPass {
     ~ForwardPass() {}
 
     // One step.  W[C,4H] R[H,4H] b[4H] x[N,C] h,c[N,H] -> h_out,c_out[N,H]; v[N,4H];
-    // tmp_Rh is unused.  h_out/c_out must not alias h/c (the reference allows it).
+    // tmp_Rh is unused.  h_out/c_out may alias h/c.
     void Iterate(
         const hipStream_t& stream,
         const T* W,
@@ -41,7 +41,19 @@ class ForwardPass {
         T* v,
         T* tmp_Rh,
         const float zoneout_prob,
-        const T* zoneout_mask);
+        const T* zoneout_mask) {
+      // `stream` is where the caller produced the inputs and will consume the outputs;
+      // the step itself runs on the stream given to the constructor.
+      void* mine = detail::stream_arg(data_.stream);
+      void* theirs = detail::stream_arg(stream);
+      data_.status = haste_hip_stream_order(theirs, mine);
+      if (data_.status != HASTE_HIP_OK) return;
+      data_.status = haste_hip_lstm_forward_iterate_f32(
+          data_.training, data_.batch_size, data_.input_size, data_.hidden_size,
+          W, R, b, x, h, c, h_out, c_out, v, tmp_Rh, zoneout_prob, zoneout_mask, mine);
+      if (data_.status != HASTE_HIP_OK) return;
+      data_.status = haste_hip_stream_order(mine, theirs);
+    }
 
     // All steps.  W[C,4H] R[H,4H] b[4H] x[T,N,C]; h,c[T+1,N,H] with slot 0 preset by the
     // caller; v[T,N,4H]; tmp_Rh[N,4H] unused (may be null); zoneout_mask[T,N,H] or null.
@@ -104,7 +116,18 @@ class BackwardPass {
         T* dh,
         T* dc,
         T* v,
-        const T* zoneout_mask);
+        const T* zoneout_mask) {
+      void* mine = detail::stream_arg(data_.stream);
+      void* theirs = detail::stream_arg(stream);
+      data_.status = haste_hip_stream_order(theirs, mine);
+      if (data_.status != HASTE_HIP_OK) return;
+      data_.status = haste_hip_lstm_backward_iterate_f32(
+          data_.batch_size, data_.input_size, data_.hidden_size,
+          W_t, R_t, b, x_t, h, c, c_new, dh_new, dc_new, dx, dW, dR, db, dh, dc, v, zoneout_mask,
+          mine);
+      if (data_.status != HASTE_HIP_OK) return;
+      data_.status = haste_hip_stream_order(mine, theirs);
+    }
 
     // W_t[4H,C] R_t[4H,H] b[4H] x_t[C,T,N] h,c[T+1,N,H] dh_new,dc_new[T+1,N,H];
     // dx[T,N,C] assigned; dW[C,4H] dR[H,4H] db[4H] accumulated into; dh,dc[N,H] zero on

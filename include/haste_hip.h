@@ -44,6 +44,12 @@ int haste_hip_max_hidden_size(int gates, int batch_size);
  * device memory; the caller must have synchronized the streams that used them). */
 int haste_hip_release_workspaces(void);
 
+/* Makes everything enqueued on `then` after this call wait for everything enqueued on
+ * `first` before it (an event recorded on `first`, waited for on `then`); no-op when both
+ * name the same stream.  Counterpart of the event hand-over around the reference's
+ * lstm::ForwardPass::Iterate(stream, ...) (lib/lstm_forward_gpu.cu.cc:171-175,203-206). */
+int haste_hip_stream_order(void* first, void* then);
+
 /* Per-kernel timing, off by default.  While enabled, every kernel the library
  * launches is bracketed by a pair of HIP events recorded on the stream the kernel
  * runs on.  haste_hip_profile_read waits for those events and returns, for the kernel
@@ -98,6 +104,29 @@ int haste_hip_lstm_backward_f32(int steps, int batch_size, int input_size, int h
                                 float* dh, float* dc, float* v,
                                 const float* zoneout_mask, void* stream);
 
+/* Single-step variants: reference lib/haste/lstm.h:73-86 (ForwardPass::Iterate,
+ * lib/lstm_forward_gpu.cu.cc:140-208) and lib/haste/lstm.h:201-219 (BackwardPass::Iterate,
+ * lib/lstm_backward_gpu.cu.cc:143-244).  Shapes are those of the all-steps entry points
+ * with T = 1, except that the states before and after the step are separate [N,H]
+ * buffers: x[N,C] h,c[N,H] -> h_out,c_out[N,H] (h_out may alias h, c_out may alias c),
+ * v[N,4H], zoneout_mask[N,H] or NULL.  Backward: x_t[C,N], h,c = states before the step,
+ * c_new = cell state after it, dh_new,dc_new[N,H] upstream gradients of the states the
+ * step produced, dx[N,C] assigned, dW,dR,db accumulated, dh,dc[N,H] in/out, v in/out. */
+int haste_hip_lstm_forward_iterate_f32(int training, int batch_size, int input_size,
+                                       int hidden_size,
+                                       const float* W, const float* R, const float* b,
+                                       const float* x, const float* h, const float* c,
+                                       float* h_out, float* c_out, float* v, float* tmp_Rh,
+                                       float zoneout_prob, const float* zoneout_mask,
+                                       void* stream);
+int haste_hip_lstm_backward_iterate_f32(int batch_size, int input_size, int hidden_size,
+                                        const float* W_t, const float* R_t, const float* b,
+                                        const float* x_t, const float* h, const float* c,
+                                        const float* c_new, const float* dh_new,
+                                        const float* dc_new, float* dx, float* dW, float* dR,
+                                        float* db, float* dh, float* dc, float* v,
+                                        const float* zoneout_mask, void* stream);
+
 /* ---- GRU -------------------------------------------------------------------
  * reference lib/haste/gru.h:86-98, lib/gru_forward_gpu.cu.cc:314-371.
  * W[C,3H] R[H,3H] bx,br[3H] x[T,N,C] h[T+1,N,H] v[T,N,4H] = (z,r,g,Rh_g+br_g)
@@ -126,6 +155,25 @@ int haste_hip_gru_backward_f32(int steps, int batch_size, int input_size, int hi
                                const float* dh_new, float* dx, float* dW, float* dR,
                                float* dbx, float* dbr, float* dh, float* dp, float* dq,
                                const float* zoneout_mask, void* stream);
+
+/* Single-step variants: reference lib/haste/gru.h:72-84 (ForwardPass::Iterate,
+ * lib/gru_forward_gpu.cu.cc:159-212) and lib/haste/gru.h:172-189 (BackwardPass::Iterate,
+ * lib/gru_backward_gpu.cu.cc:167-250).  x[N,C] h[N,H] -> h_out[N,H] (may alias h),
+ * v[N,4H], tmp_Wx[N,3H].  Backward: x_t[C,N], h = state before the step, v[N,4H],
+ * dh_new[N,H] upstream gradient of the state the step produced, dp,dq[N,3H]. */
+int haste_hip_gru_forward_iterate_f32(int training, int batch_size, int input_size,
+                                      int hidden_size,
+                                      const float* W, const float* R, const float* bx,
+                                      const float* br, const float* x, const float* h,
+                                      float* h_out, float* v, float* tmp_Wx, float* tmp_Rh,
+                                      float zoneout_prob, const float* zoneout_mask,
+                                      void* stream);
+int haste_hip_gru_backward_iterate_f32(int batch_size, int input_size, int hidden_size,
+                                       const float* W_t, const float* R_t, const float* bx,
+                                       const float* br, const float* x_t, const float* h,
+                                       const float* v, const float* dh_new, float* dx, float* dW,
+                                       float* dR, float* dbx, float* dbr, float* dh, float* dp,
+                                       float* dq, const float* zoneout_mask, void* stream);
 
 /* ---- Layer norm --------------------------------------------------------------
  * reference lib/haste/layer_norm.h:30-49, lib/layer_norm_forward_gpu.cu.cc:96-150.

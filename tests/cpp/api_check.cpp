@@ -97,8 +97,15 @@ int main(int argc, char** argv) {
   const size_t TN = (size_t)T * N, NH = (size_t)N * H;
   const bool has_mask = zoneout > 0.f;
 
-  if (cell == "lstm" || cell == "layer_norm_lstm") {
+  // The *_iterate cells run the same problems one step at a time through Iterate()
+  // (cf. reference examples/lstm.cc:252,309), handing each step a second stream as the
+  // one the caller works on.
+  hipStream_t caller_stream;
+  CHECK_HIP(hipStreamCreate(&caller_stream));
+
+  if (cell == "lstm" || cell == "layer_norm_lstm" || cell == "lstm_iterate") {
     const bool ln = cell == "layer_norm_lstm";
+    const bool iter = cell == "lstm_iterate";
     const int G = 4;
     std::vector<float> W = read_tensor((size_t)C * G * H), R = read_tensor((size_t)H * G * H),
                        b = read_tensor((size_t)G * H), x = read_tensor(TN * C), h0 = read_tensor(NH),
@@ -118,7 +125,16 @@ int main(int argc, char** argv) {
     DeviceBuf dgamma(gamma), dgamma_h(gamma_h), dbeta_h(beta_h);
     const float* maskp = has_mask ? dmask.p : nullptr;
 
-    if (!ln) {
+    if (iter) {
+      lstm::ForwardPass<float> fwd(true, N, C, H, blas, stream);
+      for (int t = 0; t < T; ++t) {
+        fwd.Iterate(caller_stream, dW_.p, dR_.p, db_.p, dx_.p + (size_t)t * N * C, h.p + t * NH,
+                    c.p + t * NH, h.p + (t + 1) * NH, c.p + (t + 1) * NH, v.p + (size_t)t * N * G * H,
+                    tmp_Rh.p, zoneout, has_mask ? maskp + t * NH : nullptr);
+        require_ok(fwd.last_status(), "lstm forward iterate");
+      }
+      CHECK_HIP(hipStreamSynchronize(caller_stream));
+    } else if (!ln) {
       lstm::ForwardPass<float> fwd(true, N, C, H, blas, stream);
       fwd.Run(T, dW_.p, dR_.p, db_.p, dx_.p, h.p, c.p, v.p, tmp_Rh.p, zoneout, maskp);
       require_ok(fwd.last_status(), "lstm forward");
@@ -139,7 +155,25 @@ int main(int argc, char** argv) {
         R_t(transpose(R, H, (size_t)G * H)), ddh_new(dh_new), ddc_new(dc_new);
     DeviceBuf gdx(TN * C), gdW((size_t)C * G * H), gdR((size_t)H * G * H), gdb((size_t)G * H), gdh(NH),
         gdc(NH), gdgamma(ln ? (size_t)2 * G * H : 0), gdgamma_h(ln ? H : 0), gdbeta_h(ln ? H : 0);
-    if (!ln) {
+    if (iter) {
+      // per-step transposes of x: step t is [C,N]
+      std::vector<float> xs(TN * C);
+      for (int t = 0; t < T; ++t) {
+        std::vector<float> one(x.begin() + (size_t)t * N * C, x.begin() + (size_t)(t + 1) * N * C);
+        one = transpose(one, N, C);
+        std::memcpy(xs.data() + (size_t)t * N * C, one.data(), one.size() * sizeof(float));
+      }
+      DeviceBuf x_steps(xs);
+      lstm::BackwardPass<float> bwd(N, C, H, blas, stream);
+      for (int t = T - 1; t >= 0; --t) {
+        bwd.Iterate(caller_stream, W_t.p, R_t.p, db_.p, x_steps.p + (size_t)t * N * C, h.p + t * NH,
+                    c.p + t * NH, c.p + (t + 1) * NH, ddh_new.p + (t + 1) * NH,
+                    ddc_new.p + (t + 1) * NH, gdx.p + (size_t)t * N * C, gdW.p, gdR.p, gdb.p, gdh.p,
+                    gdc.p, v.p + (size_t)t * N * G * H, has_mask ? maskp + t * NH : nullptr);
+        require_ok(bwd.last_status(), "lstm backward iterate");
+      }
+      CHECK_HIP(hipStreamSynchronize(caller_stream));
+    } else if (!ln) {
       lstm::BackwardPass<float> bwd(N, C, H, blas, stream);
       bwd.Run(T, W_t.p, R_t.p, db_.p, x_t.p, h.p, c.p, ddh_new.p, ddc_new.p, gdx.p, gdW.p, gdR.p,
               gdb.p, gdh.p, gdc.p, v.p, maskp);
@@ -159,8 +193,9 @@ int main(int argc, char** argv) {
     write_tensor(gdx); write_tensor(gdW); write_tensor(gdR); write_tensor(gdb);
     write_tensor(gdh); write_tensor(gdc);
     if (ln) { write_tensor(gdgamma); write_tensor(gdgamma_h); write_tensor(gdbeta_h); }
-  } else if (cell == "gru" || cell == "layer_norm_gru") {
+  } else if (cell == "gru" || cell == "layer_norm_gru" || cell == "gru_iterate") {
     const bool ln = cell == "layer_norm_gru";
+    const bool iter = cell == "gru_iterate";
     const int G = 3;
     std::vector<float> W = read_tensor((size_t)C * G * H), R = read_tensor((size_t)H * G * H),
                        bx = read_tensor((size_t)G * H), br = read_tensor((size_t)G * H),
@@ -176,7 +211,15 @@ int main(int argc, char** argv) {
     DeviceBuf act_Wx(ln ? TN * G * H : 0), act_Rh(ln ? TN * G * H : 0), cache1(ln ? TN * 2 : 0),
         cache2(ln ? TN * 2 : 0);
     const float* maskp = has_mask ? dmask.p : nullptr;
-    if (!ln) {
+    if (iter) {
+      gru::ForwardPass<float> fwd(true, N, C, H, blas, stream);
+      for (int t = 0; t < T; ++t) {
+        fwd.Iterate(dW_.p, dR_.p, dbx_.p, dbr_.p, dx_.p + (size_t)t * N * C, h.p + t * NH,
+                    h.p + (t + 1) * NH, v.p + (size_t)t * N * 4 * H, tmp_Wx.p, tmp_Rh.p, zoneout,
+                    has_mask ? maskp + t * NH : nullptr);
+        require_ok(fwd.last_status(), "gru forward iterate");
+      }
+    } else if (!ln) {
       gru::ForwardPass<float> fwd(true, N, C, H, blas, stream);
       fwd.Run(T, dW_.p, dR_.p, dbx_.p, dbr_.p, dx_.p, h.p, v.p, tmp_Wx.p, tmp_Rh.p, zoneout, maskp);
       require_ok(fwd.last_status(), "gru forward");
@@ -195,7 +238,23 @@ int main(int argc, char** argv) {
         R_t(transpose(R, H, (size_t)G * H)), ddh_new(dh_new);
     DeviceBuf gdx(TN * C), gdW((size_t)C * G * H), gdR((size_t)H * G * H), gdbx((size_t)G * H),
         gdbr((size_t)G * H), gdh(NH), dp(TN * G * H), dq(TN * G * H), gdgamma(ln ? (size_t)2 * G * H : 0);
-    if (!ln) {
+    if (iter) {
+      std::vector<float> xs(TN * C);
+      for (int t = 0; t < T; ++t) {
+        std::vector<float> one(x.begin() + (size_t)t * N * C, x.begin() + (size_t)(t + 1) * N * C);
+        one = transpose(one, N, C);
+        std::memcpy(xs.data() + (size_t)t * N * C, one.data(), one.size() * sizeof(float));
+      }
+      DeviceBuf x_steps(xs);
+      gru::BackwardPass<float> bwd(N, C, H, blas, stream);
+      for (int t = T - 1; t >= 0; --t) {
+        bwd.Iterate(W_t.p, R_t.p, dbx_.p, dbr_.p, x_steps.p + (size_t)t * N * C, h.p + t * NH,
+                    v.p + (size_t)t * N * 4 * H, ddh_new.p + (t + 1) * NH, gdx.p + (size_t)t * N * C,
+                    gdW.p, gdR.p, gdbx.p, gdbr.p, gdh.p, dp.p, dq.p,
+                    has_mask ? maskp + t * NH : nullptr);
+        require_ok(bwd.last_status(), "gru backward iterate");
+      }
+    } else if (!ln) {
       gru::BackwardPass<float> bwd(N, C, H, blas, stream);
       bwd.Run(T, W_t.p, R_t.p, dbx_.p, dbr_.p, x_t.p, h.p, v.p, ddh_new.p, gdx.p, gdW.p, gdR.p,
               gdbx.p, gdbr.p, gdh.p, dp.p, dq.p, maskp);

@@ -42,13 +42,13 @@ CASES = [(5, 3, 7, 12, 0.0), (9, 20, 24, 64, 0.3)]
 
 
 @pytest.mark.parametrize("T,N,C,H,zoneout", CASES)
-@pytest.mark.parametrize("ln", [False, True])
+@pytest.mark.parametrize("ln", [False, True, "iterate"])
 def test_cpp_lstm(T, N, C, H, zoneout, ln):
     p = problem(700 + T + H, T, N, C, H, 4, zoneout)
     mask = [p["mask"]] if zoneout else []
     base = [p["W"], p["R"], p["b"], p["x"], p["h0"], p["c0"], p["dh_new"], p["dc_new"]]
     shapes = [(T + 1, N, H), (T + 1, N, H), (T, N, C), (C, 4 * H), (H, 4 * H), (4 * H,), (N, H), (N, H)]
-    if ln:
+    if ln is True:
         outs = _run("layer_norm_lstm", T, N, C, H, zoneout,
                     base + [p["gamma"], p["gamma_h"], p["beta_h"]] + mask,
                     shapes + [(2, 4 * H), (H,), (H,)])
@@ -59,7 +59,8 @@ def test_cpp_lstm(T, N, C, H, zoneout, ln):
         ref = [fwd["h"], fwd["c"], g["dx"], g["dW"], g["dR"], g["db"], g["dh0"], g["dc0"],
                g["dgamma"], g["dgamma_h"], g["dbeta_h"]]
     else:
-        outs = _run("lstm", T, N, C, H, zoneout, base + mask, shapes)
+        # "iterate": the same problem one step at a time through Iterate()
+        outs = _run("lstm_iterate" if ln else "lstm", T, N, C, H, zoneout, base + mask, shapes)
         h, c, v = O.lstm_forward(p["W"], p["R"], p["b"], p["x"], p["h0"], p["c0"], True, zoneout, p["mask"])
         dx, dW, dR, db, dh0, dc0, _ = O.lstm_backward(p["W"], p["R"], p["b"], p["x"], h, c, v,
                                                       p["dh_new"], p["dc_new"], p["mask"])
@@ -69,13 +70,13 @@ def test_cpp_lstm(T, N, C, H, zoneout, ln):
 
 
 @pytest.mark.parametrize("T,N,C,H,zoneout", CASES)
-@pytest.mark.parametrize("ln", [False, True])
+@pytest.mark.parametrize("ln", [False, True, "iterate"])
 def test_cpp_gru(T, N, C, H, zoneout, ln):
     p = problem(710 + T + H, T, N, C, H, 3, zoneout)
     mask = [p["mask"]] if zoneout else []
     base = [p["W"], p["R"], p["b"], p["b2"], p["x"], p["h0"], p["dh_new"]]
     shapes = [(T + 1, N, H), (T, N, C), (C, 3 * H), (H, 3 * H), (3 * H,), (3 * H,), (N, H)]
-    if ln:
+    if ln is True:
         outs = _run("layer_norm_gru", T, N, C, H, zoneout, base + [p["gamma"]] + mask,
                     shapes + [(2, 3 * H)])
         fwd = O.layer_norm_gru_forward(p["W"], p["R"], p["b"], p["b2"], p["gamma"], p["x"], p["h0"],
@@ -84,7 +85,7 @@ def test_cpp_gru(T, N, C, H, zoneout, ln):
                                       p["dh_new"], p["mask"])
         ref = [fwd["h"], g["dx"], g["dW"], g["dR"], g["dbx"], g["dbr"], g["dh0"], g["dgamma"]]
     else:
-        outs = _run("gru", T, N, C, H, zoneout, base + mask, shapes)
+        outs = _run("gru_iterate" if ln else "gru", T, N, C, H, zoneout, base + mask, shapes)
         h, v = O.gru_forward(p["W"], p["R"], p["b"], p["b2"], p["x"], p["h0"], True, zoneout, p["mask"])
         dx, dW, dR, dbx, dbr, dh0, _, _ = O.gru_backward(p["W"], p["R"], p["b"], p["b2"], p["x"], h, v,
                                                          p["dh_new"], p["mask"])
