@@ -1,0 +1,215 @@
+"""The torch.nn layers on the GPU: outputs and parameter gradients against torch.nn.LSTM /
+torch.nn.GRU on the CPU (through the native-weight maps, as the reference's
+validation/pytorch.py:60-89 does) and against the fp64 oracle for the options torch.nn
+lacks (zoneout, DropConnect, layer norm, IndRNN); batch_first, lengths and
+return_state_sequence handling."""
+import numpy as np
+import pytest
+import torch
+
+import haste_amd
+from oracle import haste_oracle as O
+from util import TOL, relerr
+
+pytestmark = pytest.mark.gpu
+
+
+def npy(t):
+    return t.detach().cpu().double().numpy()
+
+
+def test_lstm_layer_matches_torch_nn():
+    T, N, C, H = 12, 9, 20, 32
+    torch.manual_seed(0)
+    layer = haste_amd.LSTM(C, H, batch_first=True).cuda()
+    ref = torch.nn.LSTM(C, H, batch_first=True).double()
+    for name, w in zip(("weight_ih_l0", "weight_hh_l0", "bias_ih_l0", "bias_hh_l0"), layer.to_native_weights()):
+        setattr(ref, name, torch.nn.Parameter(w.detach().cpu().double()))
+    x = torch.randn(N, T, C)
+    h0, c0 = torch.randn(1, N, H) * 0.5, torch.randn(1, N, H) * 0.5
+    xg = x.cuda().requires_grad_()
+    y, (hn, cn) = layer(xg, (h0.cuda(), c0.cuda()))
+    xr = x.double().requires_grad_()
+    yr, (hr, cr) = ref(xr, (h0.double(), c0.double()))
+    assert tuple(y.shape) == (N, T, H) and tuple(hn.shape) == (1, N, H)
+    assert relerr(npy(y), npy(yr)) < TOL and relerr(npy(hn), npy(hr)) < TOL and relerr(npy(cn), npy(cr)) < TOL
+    dy = torch.randn(N, T, H)
+    dcn = torch.randn(1, N, H)
+    ((y * dy.cuda()).sum() + (cn * dcn.cuda()).sum()).backward()
+    ((yr * dy.double()).sum() + (cr * dcn.double()).sum()).backward()
+    assert relerr(npy(xg.grad), npy(xr.grad)) < TOL
+    # gradients of the native-layout weights, mapped back to the haste layout
+    back = haste_amd.LSTM(C, H).double()
+    back.from_native_weights(ref.weight_ih_l0.grad, ref.weight_hh_l0.grad, ref.bias_ih_l0.grad,
+                             torch.zeros_like(ref.bias_hh_l0.grad))
+    assert relerr(npy(layer.kernel.grad), npy(back.kernel)) < TOL
+    assert relerr(npy(layer.recurrent_kernel.grad), npy(back.recurrent_kernel)) < TOL
+    assert relerr(npy(layer.bias.grad), npy(back.bias)) < TOL
+    with pytest.raises(RuntimeError, match="twice"):
+        layer.zero_grad()
+        y2, _ = layer(xg)
+        y2.sum().backward(retain_graph=True)
+        y2.sum().backward()
+
+
+def test_gru_layer_matches_torch_nn():
+    T, N, C, H = 10, 7, 16, 24
+    torch.manual_seed(1)
+    layer = haste_amd.GRU(C, H).cuda()
+    with torch.no_grad():
+        layer.bias.normal_(0, 0.1)
+        layer.recurrent_bias.normal_(0, 0.1)
+    ref = torch.nn.GRU(C, H).double()
+    for name, w in zip(("weight_ih_l0", "weight_hh_l0", "bias_ih_l0", "bias_hh_l0"), layer.to_native_weights()):
+        setattr(ref, name, torch.nn.Parameter(w.detach().cpu().double()))
+    x = torch.randn(T, N, C)
+    xg = x.cuda().requires_grad_()
+    y, hn = layer(xg)
+    xr = x.double().requires_grad_()
+    yr, hr = ref(xr)
+    assert relerr(npy(y), npy(yr)) < TOL and relerr(npy(hn), npy(hr)) < TOL
+    dy = torch.randn(T, N, H)
+    (y * dy.cuda()).sum().backward()
+    (yr * dy.double()).sum().backward()
+    assert relerr(npy(xg.grad), npy(xr.grad)) < TOL
+    back = haste_amd.GRU(C, H).double()
+    back.from_native_weights(ref.weight_ih_l0.grad, ref.weight_hh_l0.grad, ref.bias_ih_l0.grad,
+                             ref.bias_hh_l0.grad)
+    for name in ("kernel", "recurrent_kernel", "bias", "recurrent_bias"):
+        assert relerr(npy(getattr(layer, name).grad), npy(getattr(back, name))) < TOL, name
+
+
+def _drawn_masks(layer, T, N, seed):
+    """The DropConnect and zoneout masks the layer will draw after torch.manual_seed(seed):
+    it draws the DropConnect mask first, then the zoneout mask."""
+    torch.manual_seed(seed)
+    dmask, dscale = None, 1.0
+    if getattr(layer, "dropout", 0.0) and layer.training:
+        dmask = torch.empty_like(layer.recurrent_kernel).bernoulli_(1.0 - layer.dropout)
+        dscale = 1.0 / (1.0 - layer.dropout)
+    zmask = None
+    if layer.zoneout:
+        zmask = torch.empty(T, N, layer.hidden_size, device="cuda").bernoulli_(1.0 - layer.zoneout)
+    return dmask, dscale, zmask
+
+
+def test_lstm_layer_zoneout_dropconnect_vs_oracle():
+    T, N, C, H = 7, 5, 12, 16
+    torch.manual_seed(2)
+    layer = haste_amd.LSTM(C, H, dropout=0.2, zoneout=0.3).cuda()
+    x = torch.randn(T, N, C, device="cuda", requires_grad=True)
+    dmask, dscale, zmask = _drawn_masks(layer, T, N, 77)
+    torch.manual_seed(77)
+    y, (hn, cn) = layer(x)
+    dy = torch.randn(T, N, H, device="cuda")
+    (y * dy).sum().backward()
+    W, R, b = npy(layer.kernel), npy(layer.recurrent_kernel), npy(layer.bias)
+    Reff = R * npy(dmask) * np.float64(np.float32(dscale))
+    m = npy(zmask)
+    h, c, v = O.lstm_forward(W, Reff, b, npy(x), np.zeros((N, H)), np.zeros((N, H)), True, 0.3, m)
+    assert relerr(npy(y), h[1:]) < TOL and relerr(npy(cn[0]), c[-1]) < TOL
+    dh_new = np.concatenate([np.zeros((1, N, H)), npy(dy)], 0)
+    dx, dW, dR, db, _, _, _ = O.lstm_backward(W, Reff, b, npy(x), h, c, v, dh_new, np.zeros_like(dh_new), m)
+    assert relerr(npy(x.grad), dx) < TOL and relerr(npy(layer.kernel.grad), dW) < TOL
+    assert relerr(npy(layer.bias.grad), db) < TOL
+    assert relerr(npy(layer.recurrent_kernel.grad), dR * npy(dmask) * dscale) < TOL
+    # evaluation mode: no DropConnect, zoneout becomes the deterministic blend
+    layer.eval()
+    with torch.no_grad():
+        ye, _ = layer(x)
+    he, _, _ = O.lstm_forward(W, R, b, npy(x), np.zeros((N, H)), np.zeros((N, H)), False, 0.3, m)
+    assert relerr(npy(ye), he[1:]) < TOL
+    with pytest.raises(RuntimeError, match="training mode"):
+        ye2, _ = layer(x)
+        ye2.sum().backward()
+
+
+def test_gru_layer_zoneout_dropconnect_vs_oracle():
+    T, N, C, H = 6, 4, 10, 16
+    torch.manual_seed(3)
+    layer = haste_amd.GRU(C, H, dropout=0.25, zoneout=0.2).cuda()
+    x = torch.randn(T, N, C, device="cuda", requires_grad=True)
+    dmask, dscale, zmask = _drawn_masks(layer, T, N, 78)
+    torch.manual_seed(78)
+    y, hn = layer(x)
+    dy = torch.randn(T, N, H, device="cuda")
+    (y * dy).sum().backward()
+    W, R, bx, br = (npy(layer.kernel), npy(layer.recurrent_kernel), npy(layer.bias), npy(layer.recurrent_bias))
+    Reff = R * npy(dmask) * np.float64(np.float32(dscale))
+    m = npy(zmask)
+    h, v = O.gru_forward(W, Reff, bx, br, npy(x), np.zeros((N, H)), True, 0.2, m)
+    assert relerr(npy(y), h[1:]) < TOL
+    dh_new = np.concatenate([np.zeros((1, N, H)), npy(dy)], 0)
+    dx, dW, dR, dbx, dbr, _, _, _ = O.gru_backward(W, Reff, bx, br, npy(x), h, v, dh_new, m)
+    assert relerr(npy(x.grad), dx) < TOL and relerr(npy(layer.kernel.grad), dW) < TOL
+    assert relerr(npy(layer.bias.grad), dbx) < TOL and relerr(npy(layer.recurrent_bias.grad), dbr) < TOL
+    assert relerr(npy(layer.recurrent_kernel.grad), dR * npy(dmask) * dscale) < TOL
+
+
+def test_layer_norm_layers_vs_oracle():
+    T, N, C, H = 6, 5, 10, 16
+    torch.manual_seed(4)
+    x = torch.randn(T, N, C, device="cuda", requires_grad=True)
+    dy = torch.randn(T, N, H, device="cuda")
+    z = np.zeros((N, H))
+    dh_new = np.concatenate([np.zeros((1, N, H)), npy(dy)], 0)
+
+    layer = haste_amd.LayerNormLSTM(C, H, zoneout=0.2).cuda()
+    with torch.no_grad():
+        layer.gamma.uniform_(0.5, 1.5), layer.gamma_h.uniform_(0.5, 1.5), layer.beta_h.uniform_(-0.5, 0.5)
+    _, _, zmask = _drawn_masks(layer, T, N, 79)
+    torch.manual_seed(79)
+    y, _ = layer(x)
+    (y * dy).sum().backward()
+    P = {k: npy(v) for k, v in layer.named_parameters()}
+    fwd = O.layer_norm_lstm_forward(P["kernel"], P["recurrent_kernel"], P["bias"], P["gamma"], P["gamma_h"],
+                                    P["beta_h"], npy(x), z, z, True, 0.2, npy(zmask))
+    g = O.layer_norm_lstm_backward(P["kernel"], P["recurrent_kernel"], P["bias"], P["gamma"], P["gamma_h"],
+                                   P["beta_h"], npy(x), fwd, dh_new, np.zeros_like(dh_new), npy(zmask))
+    assert relerr(npy(y), fwd["h"][1:]) < TOL and relerr(npy(x.grad), g["dx"]) < TOL
+    for name, key in (("kernel", "dW"), ("recurrent_kernel", "dR"), ("bias", "db"), ("gamma", "dgamma"),
+                      ("gamma_h", "dgamma_h"), ("beta_h", "dbeta_h")):
+        assert relerr(npy(getattr(layer, name).grad), g[key]) < TOL, name
+
+    x.grad = None
+    layer = haste_amd.LayerNormGRU(C, H).cuda()
+    with torch.no_grad():
+        layer.gamma.uniform_(0.5, 1.5)
+    y, _ = layer(x)
+    (y * dy).sum().backward()
+    P = {k: npy(v) for k, v in layer.named_parameters()}
+    fwd = O.layer_norm_gru_forward(P["kernel"], P["recurrent_kernel"], P["bias"], P["recurrent_bias"],
+                                   P["gamma"], npy(x), z)
+    g = O.layer_norm_gru_backward(P["kernel"], P["recurrent_kernel"], P["bias"], P["recurrent_bias"],
+                                  P["gamma"], npy(x), fwd, dh_new)
+    assert relerr(npy(y), fwd["h"][1:]) < TOL and relerr(npy(x.grad), g["dx"]) < TOL
+    for name, key in (("kernel", "dW"), ("recurrent_kernel", "dR"), ("bias", "dbx"),
+                      ("recurrent_bias", "dbr"), ("gamma", "dgamma")):
+        assert relerr(npy(getattr(layer, name).grad), g[key]) < TOL, name
+
+    for cls, use_gamma in ((haste_amd.IndRNN, False), (haste_amd.LayerNormIndRNN, True)):
+        x.grad = None
+        layer = cls(C, H).cuda()
+        y, _ = layer(x)
+        (y * dy).sum().backward()
+        P = {k: npy(v) for k, v in layer.named_parameters()}
+        gam = P["gamma"] if use_gamma else None
+        fwd = O.indrnn_forward(P["kernel"], P["recurrent_scale"], P["bias"], npy(x), z, True, 0.0, None, gam)
+        g = O.indrnn_backward(P["kernel"], P["recurrent_scale"], P["bias"], npy(x), fwd, dh_new, None, gam)
+        assert relerr(npy(y), fwd["h"][1:]) < TOL and relerr(npy(x.grad), g["dx"]) < TOL
+        for name, key in (("kernel", "dW"), ("recurrent_scale", "du"), ("bias", "db")):
+            assert relerr(npy(getattr(layer, name).grad), g[key]) < TOL, name
+
+
+def test_lengths_and_state_sequence():
+    T, N, C, H = 8, 4, 6, 8
+    torch.manual_seed(5)
+    layer = haste_amd.GRU(C, H).cuda()
+    x = torch.randn(T, N, C, device="cuda")
+    lengths = torch.tensor([8, 3, 5, 1])
+    y, hn = layer(x, lengths=lengths)
+    for n, L in enumerate(lengths.tolist()):
+        assert torch.equal(hn[0, n], y[L - 1, n])
+    layer.return_state_sequence = True
+    y2, hs = layer(x)
+    assert tuple(hs.shape) == (1, T, N, H) and torch.equal(hs[0], y2)
