@@ -80,9 +80,11 @@ def run_metric(args, torch, lib, ops, dev):
 
     def step():
         h, c, cache = ops.lstm_forward(True, 0.0, xd, h0, c0, Wd, Rd, bd, no_mask)
-        x_t = xd.permute(2, 0, 1).contiguous()
-        W_t = Wd.t().contiguous()
-        R_t = Rd.t().contiguous()
+        # the caller-side transposes the backward API asks for, with the library's helper
+        # (the reference's benchmark uses cublasSgeam, benchmarks/benchmark_lstm.cc:417-445)
+        x_t = ops.transpose(xd)
+        W_t = ops.transpose(Wd)
+        R_t = ops.transpose(Rd)
         return ops.lstm_backward(x_t, W_t, R_t, bd, no_mask, h, c, cache, dh_new, dc_new)
 
     for _ in range(args.warmup):

@@ -8,11 +8,15 @@
 // quadrant = 2x2 v_mfma_f32_32x32x2_f32 tiles), K consumed 16 at a time through a
 // double-buffered LDS stage.  Both operand tiles sit in LDS k-major, so a wavefront
 // reads the 32 consecutive floats of one k for each half of its lanes, which is the
-// operand layout of the 32x32x2 instruction and is bank-conflict free.  Small
-// outputs with a long K (dW, dR: K = T*N) are split along K over several workgroups
-// that park partial tiles; a second, bandwidth-bound kernel adds the splits in index
-// order, so results do not depend on scheduling.  Workgroup ids are remapped so that
-// each XCD (one L2) works on a contiguous run of tiles.
+// operand layout of the 32x32x2 instruction and is bank-conflict free.
+//
+// Work distribution: output tiles are handed out in rounds of one tile per CU for as
+// long as whole rounds remain; the tiles of the last, partial round (all tiles, when
+// there are fewer tiles than CUs: dW, dR with K = T*N) are cut along K into pieces so
+// that the pieces again fill the chip evenly.  Pieces park partial tiles; a second,
+// bandwidth-bound kernel adds the pieces of a tile in index order, so results do not
+// depend on scheduling.  Whole tiles are numbered so that each XCD (one L2) works on a
+// contiguous run of them; the pieces follow, dealt round-robin over the XCDs.
 #include "common.h"
 
 namespace haste_hip {
@@ -48,7 +52,7 @@ void gemm_f32_kernel(int M, int N, int K,
                      const float* __restrict__ A, int lda,
                      const float* __restrict__ B, int ldb,
                      float* __restrict__ C, int ldc, int accumulate,
-                     int tiles_n, int total_blocks, int splits, int k_per_split,
+                     int tiles_n, int whole_tiles, int splits, int k_per_split,
                      int a_vec_ok, int b_vec_ok,
                      float* __restrict__ partial) {
   // A tile k-major in LDS: leading dimension BM+2 when it is written with transposing
@@ -61,18 +65,28 @@ void gemm_f32_kernel(int M, int N, int K,
   float* As = smem;
   float* Bs = smem + 2 * A_STAGE;
 
-  // Workgroup ids are handed to the XCDs round-robin; give XCD x the x-th contiguous
-  // chunk of the tile list so that neighbours in the list share an L2.
+  // Workgroups [0, whole_tiles) compute one whole tile each.  Ids are handed to the XCDs
+  // round-robin; XCD x gets the x-th contiguous chunk of the tile list so that neighbours
+  // in the list share an L2.  Workgroups from whole_tiles on compute one K piece of one of
+  // the remaining tiles: piece j = id - whole_tiles is split j % splits of tile
+  // whole_tiles + j / splits, and parks its result at partial + j * BM * BN.
   const int id = blockIdx.x;
-  const int q = total_blocks / kXcds, r = total_blocks % kXcds;
-  const int xcd = id % kXcds, local = id / kXcds;
-  const int nid = xcd * q + (xcd < r ? xcd : r) + local;
-  const int split = nid % splits;
-  const int tile = nid / splits;
+  int tile, k_begin, k_end;
+  const bool piece = id >= whole_tiles;
+  if (!piece) {
+    const int q = whole_tiles / kXcds, r = whole_tiles % kXcds;
+    const int xcd = id % kXcds, local = id / kXcds;
+    tile = xcd * q + (xcd < r ? xcd : r) + local;
+    k_begin = 0;
+    k_end = K;
+  } else {
+    const int j = id - whole_tiles;
+    tile = whole_tiles + j / splits;
+    k_begin = (j % splits) * k_per_split;
+    k_end = (k_begin + k_per_split < K) ? (k_begin + k_per_split) : K;
+  }
   const int tm = tile / tiles_n, tn = tile % tiles_n;
   const int m0 = tm * BM, n0 = tn * BN;
-  const int k_begin = split * k_per_split;
-  const int k_end = (k_begin + k_per_split < K) ? (k_begin + k_per_split) : K;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -181,7 +195,7 @@ void gemm_f32_kernel(int M, int N, int K,
   // col = lane % 32, row = 8*(e/4) + 4*(lane/32) + e%4.
   const int col_in = lane & 31;
   const int row_in = (lane >> 5) * 4;
-  if (splits == 1) {
+  if (!piece) {
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
@@ -199,45 +213,48 @@ void gemm_f32_kernel(int M, int N, int K,
     return;
   }
 
-  // Split-K: park the partial tile in [split][M][N] layout; a second, bandwidth-bound
-  // kernel adds the splits in order (the kernel boundary makes the partials visible, so
-  // no cache-wide fence is needed here).
-  float* part = partial + (size_t)split * M * N;
+  // A K piece: park the whole [BM][BN] partial tile (rows and columns beyond the problem
+  // hold zeros); a second, bandwidth-bound kernel adds a tile's pieces in order (the kernel
+  // boundary makes them visible, so no cache-wide fence is needed here).
+  float* part = partial + (size_t)(id - whole_tiles) * BM * BN;
 #pragma unroll
   for (int i = 0; i < MI; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int col = n0 + wn + 32 * j + col_in;
+      const int col = wn + 32 * j + col_in;
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const int row = m0 + wm + 32 * i + 8 * (e >> 2) + row_in + (e & 3);
-        if (row < M && col < N) part[(size_t)row * N + col] = acc[i][j][e];
+        const int row = wm + 32 * i + 8 * (e >> 2) + row_in + (e & 3);
+        part[row * BN + col] = acc[i][j][e];
       }
     }
 }
 
-// C (+)= sum over splits of partial[split][M][N], splits added in index order.
+// For the split tiles (tile index whole_tiles + blockIdx.x): C tile (+)= sum over its
+// `splits` pieces of partial[(blockIdx.x * splits + piece)][BM][BN], pieces added in index
+// order.  blockIdx.y selects 8 of the tile's rows; a thread owns 4 consecutive columns.
+template <int BM>
 __global__ __launch_bounds__(256)
-void splitk_reduce_kernel(int M, int N, int splits, const float* __restrict__ partial,
-                          float* __restrict__ C, int ldc, int accumulate, int vec_ok) {
-  const size_t MN = (size_t)M * N;
-  const size_t stride = (size_t)gridDim.x * 256;
-  if (vec_ok) {
-    for (size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4; i < MN; i += stride * 4) {
-      float4_t s = *reinterpret_cast<const float4_t*>(partial + i);
-      for (int sp = 1; sp < splits; ++sp) s += *reinterpret_cast<const float4_t*>(partial + sp * MN + i);
-      const size_t row = i / N, col = i % N;
-      float4_t* p = reinterpret_cast<float4_t*>(C + row * ldc + col);
-      *p = accumulate ? (*p + s) : s;
-    }
+void split_reduce_kernel(int M, int N, int splits, int tiles_n, int whole_tiles,
+                         const float* __restrict__ partial, float* __restrict__ C, int ldc,
+                         int accumulate, int vec_ok) {
+  const int tile = whole_tiles + blockIdx.x;
+  const int tm = tile / tiles_n, tn = tile % tiles_n;
+  const int r = blockIdx.y * 8 + (threadIdx.x >> 5);
+  const int c = (threadIdx.x & 31) * 4;
+  const int row = tm * BM + r, col = tn * BN + c;
+  if (r >= BM || row >= M || col >= N) return;
+  const float* p = partial + ((size_t)blockIdx.x * splits) * BM * BN + r * BN + c;
+  float4_t s = *reinterpret_cast<const float4_t*>(p);
+  for (int sp = 1; sp < splits; ++sp)
+    s += *reinterpret_cast<const float4_t*>(p + (size_t)sp * BM * BN);
+  float* out = C + (size_t)row * ldc + col;
+  if (vec_ok && col + 3 < N) {
+    float4_t* o = reinterpret_cast<float4_t*>(out);
+    *o = accumulate ? (*o + s) : s;
   } else {
-    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < MN; i += stride) {
-      float s = partial[i];
-      for (int sp = 1; sp < splits; ++sp) s += partial[sp * MN + i];
-      const size_t row = i / N, col = i % N;
-      float* p = C + row * ldc + col;
-      *p = accumulate ? (*p + s) : s;
-    }
+    const float v[4] = {s.x, s.y, s.z, s.w};
+    for (int i = 0; i < 4 && col + i < N; ++i) out[i] = accumulate ? (out[i] + v[i]) : v[i];
   }
 }
 
@@ -254,55 +271,77 @@ int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
   const int tiles_n = (N + BN - 1) / BN;
   const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
 
-  // Tile height: 64 rows only when the output has no more than that.  K splits: when the
-  // output tiles alone leave CUs without two workgroups each, K is cut into the smallest
-  // power-of-two number of pieces that does, as long as a piece keeps at least 256 of K
-  // (measured on the backward shapes: dW/dR 51 -> 91-99 TFLOP/s, dx 73 -> 82 TFLOP/s).
-  // The choice depends on the shape only, so results are reproducible.
+  // Tile height: 64 rows only when the output has no more than that.
   const int bm = M <= 64 ? 64 : 128;
-  int splits = 1;
-  {
-    const long long t = (long long)((M + bm - 1) / bm) * tiles_n;
-    while (t * splits < 2LL * cus && K / (splits * 2) >= 256 && splits < 32) splits *= 2;
-  }
   const int tiles_m = (M + bm - 1) / bm;
   const long long tiles = (long long)tiles_m * tiles_n;
-  HASTE_HIP_REQUIRE(tiles < (1ll << 28));
+  HASTE_HIP_REQUIRE(tiles < (1ll << 26));
+
+  // Whole rounds of one tile per CU run unsplit; the `rest` tiles of the last round are each
+  // cut into `splits` K pieces.  In units of the time one CU needs for one whole tile, s
+  // pieces per tile cost ceil(rest*s/CUs)/s for the arithmetic plus 0.25*rest*s/K for
+  // writing and re-reading the partial tiles (128 KiB per piece at the chip's memory rate
+  // against 2*128*128*K flops at one CU's MFMA rate); a launch that consists of fewer than
+  // two pieces per CU pays 12 % more (a lone workgroup cannot hide its own load latency).
+  // The cheapest s is taken, a piece keeping at least 64 of K.  The choice depends on the
+  // shape only, so results are reproducible.
+  const long long whole = tiles >= cus ? tiles / cus * cus : 0;
+  const int rest = (int)(tiles - whole);
+  int splits = 1;
+  if (rest > 0) {
+    const int k_iters = (K + BK - 1) / BK;
+    int s_max = k_iters / 4;
+    if (s_max > 64) s_max = 64;
+    auto cost = [&](int s) {
+      const long long pieces = (long long)rest * s;
+      double c = (double)((pieces + cus - 1) / cus) / s;
+      if (whole == 0 && pieces < 2LL * cus) c *= 1.12;
+      if (s > 1) c += 0.25 * (double)rest * s / K;
+      return c;
+    };
+    double best = cost(1);
+    for (int s = 2; s <= s_max; ++s)
+      if (cost(s) < best - 1e-9) { best = cost(s); splits = s; }
+  }
   int k_per_split = (K + splits - 1) / splits;
   k_per_split = (k_per_split + BK - 1) / BK * BK;
   splits = (K + k_per_split - 1) / k_per_split;
+  const bool split = splits > 1;
+  // Unsplit "rest" tiles are ordinary whole tiles.
+  const int whole_tiles = split ? (int)whole : (int)tiles;
+  const int pieces = split ? rest * splits : 0;
 
   Workspace ws;
   float* partial = nullptr;
-  if (splits > 1) {
-    const size_t bytes = (size_t)splits * M * N * sizeof(float);
+  if (split) {
+    const size_t bytes = (size_t)pieces * bm * BN * sizeof(float);
     HASTE_HIP_PROPAGATE(get_workspace(stream, bytes, &ws));
     partial = ws.scratch;
   }
   const int a_vec_ok = aligned16(A) && (lda % 4 == 0) && (k_per_split % 4 == 0);
   const int b_vec_ok = aligned16(B) && (ldb % 4 == 0);
-  const int total = (int)(tiles * splits);
-  dim3 grid((unsigned)total), block(256);
+  dim3 grid((unsigned)(whole_tiles + pieces)), block(256);
   ScopedKernelTimer timer("gemm_f32", stream);
 #define HASTE_GEMM_LAUNCH(TA_, BM_)                                                          \
   if (trans_a == TA_ && bm == BM_)                                                           \
     gemm_f32_kernel<TA_, BM_><<<grid, block, 0, stream>>>(                                   \
-        M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, tiles_n, total, splits,         \
+        M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, tiles_n, whole_tiles, splits,   \
         k_per_split, a_vec_ok, b_vec_ok, partial);
   HASTE_GEMM_LAUNCH(false, 128) HASTE_GEMM_LAUNCH(false, 64)
   HASTE_GEMM_LAUNCH(true, 128) HASTE_GEMM_LAUNCH(true, 64)
 #undef HASTE_GEMM_LAUNCH
   HASTE_HIP_TRY(hipGetLastError());
-  if (splits > 1) {
-    const size_t MN = (size_t)M * N;
-    const int vec = (N % 4 == 0) && (ldc % 4 == 0) && aligned16(C) && aligned16(partial);
-    size_t blocks = (MN / (vec ? 4 : 1) + 255) / 256;
-    if (blocks > (size_t)cus * 8) blocks = (size_t)cus * 8;
-    if (blocks < 1) blocks = 1;
-    splitk_reduce_kernel<<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
-        M, N, splits, partial, C, ldc, accumulate ? 1 : 0, vec);
+  if (split) {
+    const int vec = (ldc % 4 == 0) && aligned16(C);
+    const dim3 rgrid((unsigned)rest, (unsigned)(bm / 8));
+    if (bm == 128)
+      split_reduce_kernel<128><<<rgrid, dim3(256), 0, stream>>>(
+          M, N, splits, tiles_n, whole_tiles, partial, C, ldc, accumulate ? 1 : 0, vec);
+    else
+      split_reduce_kernel<64><<<rgrid, dim3(256), 0, stream>>>(
+          M, N, splits, tiles_n, whole_tiles, partial, C, ldc, accumulate ? 1 : 0, vec);
+    HASTE_HIP_TRY(hipGetLastError());
   }
-  HASTE_HIP_TRY(hipGetLastError());
   return HASTE_HIP_OK;
 }
 

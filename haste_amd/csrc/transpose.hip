@@ -1,0 +1,53 @@
+// out[cols, rows] = in[rows, cols]: the layout change the backward passes ask their
+// callers for (x[T*N, C] -> x_t[C, T*N], W -> W_t, R -> R_t; reference
+// frameworks/pytorch/lstm.py:84-86, and cublasSgeam in benchmarks/benchmark_lstm.cc:417-445).
+//
+// Bound: HBM.  Algorithmic bytes 2 * rows * cols * 4.  A workgroup moves a 64 x 64 tile
+// through LDS: rows of the tile are read as 256-byte segments, the transposed rows are
+// written as 256-byte segments; the 65-float row pitch keeps both LDS phases conflict free.
+#include "common.h"
+
+namespace haste_hip {
+namespace {
+
+constexpr int TT = 64;
+
+__global__ __launch_bounds__(256)
+void transpose_f32_kernel(int rows, int cols, const float* __restrict__ in,
+                          float* __restrict__ out, int tiles_c) {
+  __shared__ float tile[TT][TT + 1];
+  const int tr = blockIdx.x / tiles_c, tc = blockIdx.x % tiles_c;
+  const int r0 = tr * TT, c0 = tc * TT;
+  const int lx = threadIdx.x & 63, ly = threadIdx.x >> 6;
+  float v[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int r = r0 + ly + 4 * i, c = c0 + lx;
+    v[i] = (r < rows && c < cols) ? in[(size_t)r * cols + c] : 0.f;
+  }
+#pragma unroll
+  for (int i = 0; i < 16; ++i) tile[ly + 4 * i][lx] = v[i];
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int c = c0 + ly + 4 * i, r = r0 + lx;
+    if (c < cols && r < rows) out[(size_t)c * rows + r] = tile[lx][ly + 4 * i];
+  }
+}
+
+}  // namespace
+}  // namespace haste_hip
+
+extern "C" int haste_hip_transpose_f32(int rows, int cols, const float* in, float* out,
+                                       void* stream) {
+  HASTE_HIP_REQUIRE(rows > 0 && cols > 0 && in != nullptr && out != nullptr && in != out);
+  const long long tiles_r = (rows + haste_hip::TT - 1) / haste_hip::TT;
+  const long long tiles_c = (cols + haste_hip::TT - 1) / haste_hip::TT;
+  HASTE_HIP_REQUIRE(tiles_r * tiles_c < (1ll << 31));
+  haste_hip::ScopedKernelTimer timer("transpose_f32", haste_hip::as_stream(stream));
+  haste_hip::transpose_f32_kernel<<<dim3((unsigned)(tiles_r * tiles_c)), dim3(256), 0,
+                                    haste_hip::as_stream(stream)>>>(rows, cols, in, out,
+                                                                    (int)tiles_c);
+  HASTE_HIP_TRY(hipGetLastError());
+  return HASTE_HIP_OK;
+}

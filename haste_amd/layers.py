@@ -21,11 +21,11 @@ __all__ = ["LSTM", "GRU", "IndRNN", "LayerNormLSTM", "LayerNormGRU", "LayerNormI
 
 def _time_major_t(x):
     """[T,N,C] -> [C,T,N], the layout the backward passes take x in."""
-    return x.permute(2, 0, 1).contiguous()
+    return ops.transpose(x) if x.is_cuda else x.permute(2, 0, 1).contiguous()
 
 
 def _t(w):
-    return w.t().contiguous()
+    return ops.transpose(w) if w.is_cuda and w.is_contiguous() else w.t().contiguous()
 
 
 def _single_shot(ctx, name):

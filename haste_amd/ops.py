@@ -39,6 +39,18 @@ def gemm(a, b, out=None, trans_a=False, accumulate=False):
     return out
 
 
+def transpose(a, out=None):
+    """[rows, cols] -> [cols, rows] (a contiguous copy); leading dimensions of `a` beyond
+    the last are folded into rows, so x[T,N,C] gives x_t[C,T,N]."""
+    _check(a)
+    cols = a.shape[-1]
+    rows = a.numel() // cols
+    if out is None:
+        out = torch.empty((cols,) + tuple(a.shape[:-1]), device=a.device, dtype=a.dtype)
+    lib.call("haste_hip_transpose_f32", rows, cols, a, out)
+    return out
+
+
 # ---- LSTM (reference frameworks/pytorch/lstm.cc:31-157) ---------------------
 def lstm_forward(training, zoneout_prob, x, h0, c0, kernel, recurrent_kernel, bias, zoneout_mask,
                  dropconnect_mask=None, dropconnect_scale=1.0):

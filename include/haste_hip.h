@@ -69,6 +69,12 @@ int haste_hip_gemm_f32(int trans_a, int M, int N, int K,
                        const float* A, int lda, const float* B, int ldb,
                        float* C, int ldc, int accumulate, void* stream);
 
+/* out[cols,rows] = in[rows,cols] (in != out).  The backward entry points take x, W and R
+ * transposed by the caller (x_t[C,T*N], W_t, R_t), as the reference's do
+ * (lib/haste/lstm.h:230-247); its benchmark produces them with cublasSgeam inside the timed
+ * region (benchmarks/benchmark_lstm.cc:417-445).  This is that helper. */
+int haste_hip_transpose_f32(int rows, int cols, const float* in, float* out, void* stream);
+
 /* ---- LSTM ----------------------------------------------------------------
  * reference lib/haste/lstm.h:118-129 (ForwardPass::Run), lib/lstm_forward_gpu.cu.cc:313-366.
  * W[C,4H] R[H,4H] b[4H] x[T,N,C] h,c[T+1,N,H] (slot 0 preset by the caller)

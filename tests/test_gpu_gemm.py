@@ -48,3 +48,13 @@ def test_gemm_split_k_is_run_to_run_identical():
     o2 = ops.gemm(a, b)
     torch.cuda.synchronize()
     assert torch.equal(o1, o2)
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (3, 5), (64, 64), (65, 63), (100, 7, 33), (6400, 512), (512, 2048)])
+def test_transpose(shape):
+    import torch
+    from haste_amd import ops
+    a = torch.randn(*shape, device="cuda")
+    out = ops.transpose(a)
+    ref = a.reshape(-1, shape[-1]).t().contiguous().reshape((shape[-1],) + tuple(shape[:-1]))
+    assert out.shape == ref.shape and torch.equal(out, ref)
