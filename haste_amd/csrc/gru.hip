@@ -23,7 +23,7 @@ struct GruFwdParams {
   const float* zoneout_mask;
   const float* dc_mask;  // DropConnect mask [H,3H] or null
   float dc_scale;
-  float* xh;             // exchange tiles of h: [batch tiles][2][Kpad/4][NB][4]
+  float* xh;             // polled exchange tiles of h: [batch tiles][4][Kpad/4][NB][4]
   LaunchShape ls;
 };
 
@@ -53,15 +53,16 @@ void gru_forward_kernel(GruFwdParams p) {
   const size_t NH = (size_t)N * H;
 
   const int tile_floats = Kpad * NB;
-  float* xh = p.xh + (size_t)role.bt * 2 * tile_floats;
-  const TileBuffer xhb = make_tile_buffer(xh, 2 * tile_floats);
+  float* xh = p.xh + (size_t)role.bt * kPolledTiles * tile_floats;
+  const TileBuffer xhb = make_tile_buffer(xh, kPolledTiles * tile_floats);
 
   GroupSync gs;
   group_sync_init(gs, p.ls, role);
 
-  // Own k range of the exchange tiles (the last workgroup also owns the padding).
+  // Own k range of the exchange tiles (the last workgroup also owns the padding): rows and
+  // k beyond the problem stay zero for the whole launch.
   zero_tile_share(gs, xh, tile_floats, NB, j0 / 4,
-                  (role.cw == p.ls.gx - 1 ? Kpad - j0 : HS) / 4);
+                  (role.cw == p.ls.gx - 1 ? Kpad - j0 : HS) / 4, kPolledTiles);
 
   {
     const bool fast = H % 4 == 0 && ((reinterpret_cast<uintptr_t>(p.R) |
@@ -96,32 +97,51 @@ void gru_forward_kernel(GruFwdParams p) {
     }
   }
   const bool zoneout = p.zoneout_prob != 0.f && p.zoneout_mask != nullptr;
+  // Tile 0 receives h[0]; the elements of the other tiles that steps will publish start out
+  // unwritten.  One real barrier: nobody polls a tile before all of its owners have set it up.
 #pragma unroll
   for (int pp = 0; pp < PP; ++pp)
-    if (act[pp]) store_exchanged(gs, &xh[xchg_index(pj[pp], pl[pp], NB)], h_prev[pp]);
-  group_arrive(gs);  // h[0] is published; the slice is complete in LDS
+    if (act[pp]) {
+      float* e = &xh[xchg_index(pj[pp], pl[pp], NB)];
+      store_exchanged(gs, e, publishable(h_prev[pp]));
+      for (int b = 1; b < kPolledTiles; ++b) store_exchanged(gs, e + (size_t)b * tile_floats, unwritten_value());
+    }
+  group_arrive(gs);  // also: the slice is complete in LDS
+  group_wait(gs);
+
+  // Inputs of a step that do not depend on the recurrence (x*W, the zoneout mask) are
+  // fetched one step ahead.
+  float wx_next[PP][3], mk_next[PP];
+  auto fetch = [&](int t) {
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      mk_next[pp] = 1.f;
+#pragma unroll
+      for (int g = 0; g < 3; ++g) wx_next[pp][g] = 0.f;
+      if (act[pp] && t < T) {
+        const float* wt = p.Wx + ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 3; ++g) wx_next[pp][g] = wt[g * H];
+        if (zoneout && p.training) mk_next[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
+      }
+    }
+  };
+  fetch(0);
 
   for (int t = 0; t < T; ++t) {
     float wx[PP][3], mk[PP];
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
-      mk[pp] = 1.f;
+      mk[pp] = mk_next[pp];
 #pragma unroll
-      for (int g = 0; g < 3; ++g) wx[pp][g] = 0.f;
-      if (act[pp]) {
-        const float* wt = p.Wx + ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
-#pragma unroll
-        for (int g = 0; g < 3; ++g) wx[pp][g] = wt[g * H];
-        if (zoneout && p.training) mk[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
-      }
+      for (int g = 0; g < 3; ++g) wx[pp][g] = wx_next[pp][g];
     }
-    group_wait(gs);  // h[t] complete for this batch tile
-
-    tile_product<NB, CT, false>(xhb, (t & 1) * tile_floats, Kpad, w_lds, red);
+    // The operand loads wait for h[t] themselves (polled tile t % 4).
+    tile_product<NB, CT, false, true>(xhb, (t & 3) * tile_floats, Kpad, w_lds, red, &gs);
     __syncthreads();
 
     float saved[PP][4];  // z, r, g, q of the step for the caller's cache
-    float* xh_next = xh + ((t + 1) & 1) * tile_floats;
+    float h_pub[PP];
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
       if (act[pp]) {
@@ -141,12 +161,27 @@ void gru_forward_kernel(GruFwdParams p) {
           if (p.training) h_new = (h_new - h_prev[pp]) * mk[pp] + h_prev[pp];
           else h_new = p.zoneout_prob * h_prev[pp] + (1.0f - p.zoneout_prob) * h_new;
         }
-        if (t + 1 < T) store_exchanged(gs, &xh_next[xchg_index(pj[pp], pl[pp], NB)], h_new);
         h_prev[pp] = h_new;
       }
+      h_pub[pp] = publishable(h_prev[pp]);
     }
-    if (t + 1 < T) group_arrive(gs);  // publishes h[t+1]; also fences `red` reuse
-    // The caller's copies are written behind the barrier: nobody in the launch waits for them.
+    // Everything this wavefront stored during the previous step (its resets among it) has
+    // landed before h[t+1] becomes visible.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (t + 1 < T) {
+      float* xh_next = xh + ((t + 1) & 3) * tile_floats;
+      float* xh_done = xh + ((t + 3) & 3) * tile_floats;  // read at step t-1: nobody needs it any more
+#pragma unroll
+      for (int pp = 0; pp < PP; ++pp)
+        if (act[pp]) {
+          const int e = xchg_index(pj[pp], pl[pp], NB);
+          store_exchanged(gs, &xh_next[e], h_pub[pp]);
+          if (t + 3 < T) store_exchanged(gs, &xh_done[e], unwritten_value());
+        }
+    }
+    fetch(t + 1);
+    __syncthreads();  // `red` may be overwritten by the next step's product
+    // The caller's copies are written last: nobody in the launch waits for them.
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
       if (act[pp]) {
@@ -210,8 +245,8 @@ void gru_backward_kernel(GruBwdParams p) {
   const size_t NH = (size_t)N * H;
 
   const int tile_floats = Kpad * NB;
-  float* xdq = p.xdq + (size_t)role.bt * 2 * tile_floats;
-  const TileBuffer xdqb = make_tile_buffer(xdq, 2 * tile_floats);
+  float* xdq = p.xdq + (size_t)role.bt * kPolledTiles * tile_floats;
+  const TileBuffer xdqb = make_tile_buffer(xdq, kPolledTiles * tile_floats);
 
   GroupSync gs;
   group_sync_init(gs, p.ls, role);
@@ -219,7 +254,7 @@ void gru_backward_kernel(GruBwdParams p) {
   // Own k range of the exchange tiles (the last workgroup also owns the padding); only
   // rows and units of the problem are written afterwards.
   zero_tile_share(gs, xdq, tile_floats, NB, 12 * role.cw,
-                  (role.cw == p.ls.gx - 1 ? Kpad - 48 * role.cw : 48) / 4);
+                  (role.cw == p.ls.gx - 1 ? Kpad - 48 * role.cw : 48) / 4, kPolledTiles);
 
   {
     const bool fast = H % 4 == 0 && (reinterpret_cast<uintptr_t>(p.R_t) & 15u) == 0;
@@ -245,7 +280,18 @@ void gru_backward_kernel(GruBwdParams p) {
     for (int g = 0; g < 6; ++g) dbacc[pp][g] = 0.f;
   }
   const bool zoneout = p.zoneout_mask != nullptr;
-  __syncthreads();
+  // The elements that steps will publish start out unwritten (rows and units beyond the
+  // problem stay zero).  One real barrier: nobody polls a tile before its owners have set
+  // it up.
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp)
+    if (act[pp])
+      for (int b = 0; b < kPolledTiles; ++b)
+        for (int g = 0; g < 3; ++g)
+          store_exchanged(gs, xdq + (size_t)b * tile_floats + xchg_index(3 * pj[pp] + g, pl[pp], NB),
+                          unwritten_value());
+  group_arrive(gs);  // also: the slice is complete in LDS
+  group_wait(gs);
 
   struct StepIn { float vt[4], h0, dhn, m; };
   StepIn nxt[PP];
@@ -269,7 +315,9 @@ void gru_backward_kernel(GruBwdParams p) {
 
   for (int t = T - 1; t >= 0; --t) {
     float dh_keep[PP], dpv[PP][3], dqv[PP];
-    float* xdq_t = xdq + (t & 1) * tile_floats;
+    const int done = T - 1 - t;  // steps done so far; this step uses polled tile done % 4
+    float* xdq_t = xdq + (done & 3) * tile_floats;
+    float* xdq_done = xdq + ((done + 2) & 3) * tile_floats;  // read two steps ago
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
       dh_keep[pp] = 0.f;
@@ -291,10 +339,6 @@ void gru_backward_kernel(GruBwdParams p) {
         const float dr = dp_g * qg;
         const float dp_r = d_sigmoid_f(r) * dr;
         const float dp_z = d_sigmoid_f(z) * dz;
-        float* xq = xdq_t + xchg_index(3 * pj[pp], pl[pp], NB);
-        store_exchanged(gs, xq, dp_z);
-        store_exchanged(gs, xdq_t + xchg_index(3 * pj[pp] + 1, pl[pp], NB), dp_r);
-        store_exchanged(gs, xdq_t + xchg_index(3 * pj[pp] + 2, pl[pp], NB), dq_g);
         dpv[pp][0] = dp_z;
         dpv[pp][1] = dp_r;
         dpv[pp][2] = dp_g;
@@ -307,8 +351,21 @@ void gru_backward_kernel(GruBwdParams p) {
         dbacc[pp][5] += dq_g;
       }
     }
-    group_arrive(gs);  // dq_t of this workgroup's units is published
-    // The caller's copies are written behind the barrier: nobody in the launch waits for them.
+    // What this wavefront stored during the previous step (its resets among it) has landed
+    // before the gate gradients of this step become visible.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp)
+      if (act[pp]) {
+        const float q[3] = {dpv[pp][0], dpv[pp][1], dqv[pp]};
+#pragma unroll
+        for (int g = 0; g < 3; ++g) {
+          const int e = xchg_index(3 * pj[pp] + g, pl[pp], NB);
+          store_exchanged(gs, xdq_t + e, publishable(q[g]));
+          if (done + 2 < T) store_exchanged(gs, xdq_done + e, unwritten_value());
+        }
+      }
+    // The caller's copies: nobody in the launch waits for them.
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
       if (act[pp]) {
@@ -322,13 +379,13 @@ void gru_backward_kernel(GruBwdParams p) {
       }
     }
     fetch(t - 1);
-    group_wait(gs);    // dq_t of every unit is complete for this batch tile
-
-    tile_product<NB, 1, true>(xdqb, (t & 1) * tile_floats, Kpad, w_lds, red);
+    // The operand loads wait for dq_t of every unit themselves.
+    tile_product<NB, 1, true, true>(xdqb, (done & 3) * tile_floats, Kpad, w_lds, red, &gs);
     __syncthreads();
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp)
       if (tid + 256 * pp < NB * HSB) dh[pp] = dh_keep[pp] + sum_product<NB, 1>(red, pl[pp], pc[pp]);
+    __syncthreads();  // `red` may be overwritten by the next step's product
   }
 
 #pragma unroll
@@ -376,7 +433,8 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
 
   // Taken after the GEMM, which may replace the stream's scratch buffer with a larger one.
   Workspace ws;
-  HASTE_HIP_PROPAGATE(get_workspace(stream, exchange_floats(H, tile.nb, tile.gy) * sizeof(float), &ws));
+  HASTE_HIP_PROPAGATE(get_workspace(
+      stream, exchange_floats(H, tile.nb, tile.gy, kPolledTiles) * sizeof(float), &ws));
   HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 
   GruFwdParams p;
@@ -415,7 +473,7 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
 
   Workspace ws;
   const size_t db_floats = ((size_t)tile.gy * 6 * H + 3) / 4 * 4;
-  const size_t xdq_floats = exchange_floats(gru_backward_k(H), tile.nb, tile.gy);
+  const size_t xdq_floats = exchange_floats(gru_backward_k(H), tile.nb, tile.gy, kPolledTiles);
   HASTE_HIP_PROPAGATE(get_workspace(stream, (db_floats + xdq_floats) * sizeof(float), &ws));
   HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 

@@ -23,7 +23,7 @@ struct LstmFwdParams {
   const float* zoneout_mask;   // [T,N,H] or null
   const float* dc_mask;        // DropConnect mask [H,4H] or null
   float dc_scale;
-  float* xh;                   // exchange tiles of h: [batch tiles][2][Kpad/4][NB][4]
+  float* xh;                   // polled exchange tiles of h: [batch tiles][4][Kpad/4][NB][4]
   LaunchShape ls;
 };
 
@@ -52,16 +52,17 @@ void lstm_forward_kernel(LstmFwdParams p) {
   const size_t NH = (size_t)N * H;
 
   const int tile_floats = Kpad * NB;
-  float* xh = p.xh + (size_t)role.bt * 2 * tile_floats;
+  float* xh = p.xh + (size_t)role.bt * kPolledTiles * tile_floats;
 
-  const TileBuffer xhb = make_tile_buffer(xh, 2 * tile_floats);
+  const TileBuffer xhb = make_tile_buffer(xh, kPolledTiles * tile_floats);
 
   GroupSync gs;
   group_sync_init(gs, p.ls, role);
 
-  // Own k range of the exchange tiles (the last workgroup also owns the padding).
+  // Own k range of the exchange tiles (the last workgroup also owns the padding): rows and
+  // k beyond the problem stay zero for the whole launch.
   zero_tile_share(gs, xh, tile_floats, NB, j0 / 4,
-                  (role.cw == p.ls.gx - 1 ? Kpad - j0 : HS) / 4);
+                  (role.cw == p.ls.gx - 1 ? Kpad - j0 : HS) / 4, kPolledTiles);
 
   // Resident slice: column c of the slice is gate c/HS, hidden unit j0 + c%HS.
   {
@@ -97,33 +98,50 @@ void lstm_forward_kernel(LstmFwdParams p) {
     }
   }
   const bool zoneout = p.zoneout_prob != 0.f && p.zoneout_mask != nullptr;
+  // Tile 0 receives h[0]; the elements of the other tiles that steps will publish start out
+  // unwritten.  One real barrier: nobody polls a tile before all of its owners have set it up.
 #pragma unroll
   for (int pp = 0; pp < PP; ++pp)
-    if (act[pp]) store_exchanged(gs, &xh[xchg_index(pj[pp], pl[pp], NB)], h_prev[pp]);
-  group_arrive(gs);  // h[0] is published; the slice is complete in LDS
+    if (act[pp]) {
+      float* e = &xh[xchg_index(pj[pp], pl[pp], NB)];
+      store_exchanged(gs, e, publishable(h_prev[pp]));
+      for (int b = 1; b < kPolledTiles; ++b) store_exchanged(gs, e + (size_t)b * tile_floats, unwritten_value());
+    }
+  group_arrive(gs);  // also: the slice is complete in LDS
+  group_wait(gs);
+
+  // Inputs of a step that do not depend on the recurrence (x*W, the zoneout mask) are
+  // fetched one step ahead, while the matrix units work on the step before.
+  float wx_next[PP][4], mk_next[PP];
+  auto fetch = [&](int t) {
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      mk_next[pp] = 1.f;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) wx_next[pp][g] = 0.f;
+      if (act[pp] && t < T) {
+        const float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) wx_next[pp][g] = vt[g * H];
+        if (zoneout && p.training) mk_next[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
+      }
+    }
+  };
+  fetch(0);
 
   for (int t = 0; t < T; ++t) {
-    // Inputs of this step that do not depend on the recurrence: issue before waiting.
     float wx[PP][4], mk[PP];
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
-      mk[pp] = 1.f;
+      mk[pp] = mk_next[pp];
 #pragma unroll
-      for (int g = 0; g < 4; ++g) wx[pp][g] = 0.f;
-      if (act[pp]) {
-        const float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
-#pragma unroll
-        for (int g = 0; g < 4; ++g) wx[pp][g] = vt[g * H];
-        if (zoneout && p.training) mk[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
-      }
+      for (int g = 0; g < 4; ++g) wx[pp][g] = wx_next[pp][g];
     }
-    group_wait(gs);  // h[t] complete for this batch tile
-
-    tile_product<NB, CT, false>(xhb, (t & 1) * tile_floats, Kpad, w_lds, red);
+    // The operand loads wait for h[t] themselves (polled tile t % 4).
+    tile_product<NB, CT, false, true>(xhb, (t & 3) * tile_floats, Kpad, w_lds, red, &gs);
     __syncthreads();
 
-    float gate[PP][4];
-    float* xh_next = xh + ((t + 1) & 1) * tile_floats;
+    float gate[PP][4], h_pub[PP];
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
       if (act[pp]) {
@@ -141,13 +159,28 @@ void lstm_forward_kernel(LstmFwdParams p) {
           if (p.training) h_new = (h_new - h_prev[pp]) * mk[pp] + h_prev[pp];
           else h_new = p.zoneout_prob * h_prev[pp] + (1.0f - p.zoneout_prob) * h_new;
         }
-        if (t + 1 < T) store_exchanged(gs, &xh_next[xchg_index(pj[pp], pl[pp], NB)], h_new);
         c_prev[pp] = c_new;
         h_prev[pp] = h_new;
       }
+      h_pub[pp] = publishable(h_prev[pp]);
     }
-    if (t + 1 < T) group_arrive(gs);  // publishes h[t+1]; also fences `red` reuse
-    // The caller's copies are written behind the barrier: nobody in the launch waits for them.
+    // Everything this wavefront stored during the previous step (its resets among it) has
+    // landed before h[t+1] becomes visible.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (t + 1 < T) {
+      float* xh_next = xh + ((t + 1) & 3) * tile_floats;
+      float* xh_done = xh + ((t + 3) & 3) * tile_floats;  // read at step t-1: nobody needs it any more
+#pragma unroll
+      for (int pp = 0; pp < PP; ++pp)
+        if (act[pp]) {
+          const int e = xchg_index(pj[pp], pl[pp], NB);
+          store_exchanged(gs, &xh_next[e], h_pub[pp]);
+          if (t + 3 < T) store_exchanged(gs, &xh_done[e], unwritten_value());
+        }
+    }
+    fetch(t + 1);
+    __syncthreads();  // `red` may be overwritten by the next step's product
+    // The caller's copies are written last: nobody in the launch waits for them.
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
       if (act[pp]) {
@@ -177,7 +210,7 @@ struct LstmBwdParams {
   float* v;             // [T,N,4H] in: activations, out: gate gradients
   const float* zoneout_mask;
   float* db_partial;    // [batch tiles, 4H] scratch
-  float* xdv;           // exchange tiles of the gate gradients: [batch tiles][2][Kpad/4][NB][4]
+  float* xdv;           // polled exchange tiles of the gate gradients: [batch tiles][4][Kpad/4][NB][4]
   LaunchShape ls;
 };
 
@@ -212,8 +245,8 @@ void lstm_backward_kernel(LstmBwdParams p) {
   group_sync_init(gs, p.ls, role);
 
   const int tile_floats = Kpad * NB;
-  float* xdv = p.xdv + (size_t)role.bt * 2 * tile_floats;
-  const TileBuffer xdvb = make_tile_buffer(xdv, 2 * tile_floats);
+  float* xdv = p.xdv + (size_t)role.bt * kPolledTiles * tile_floats;
+  const TileBuffer xdvb = make_tile_buffer(xdv, kPolledTiles * tile_floats);
 
   {
     const bool fast = H % 4 == 0 && (reinterpret_cast<uintptr_t>(p.R_t) & 15u) == 0;
@@ -240,7 +273,18 @@ void lstm_backward_kernel(LstmBwdParams p) {
     for (int g = 0; g < 4; ++g) dbacc[pp][g] = 0.f;
   }
   const bool zoneout = p.zoneout_mask != nullptr;
-  __syncthreads();
+  // Every element of the polled tiles belongs to the thread that publishes it (rows and
+  // units beyond the problem are published as zeros); all start out unwritten.  One real
+  // barrier: nobody polls a tile before all of its owners have set it up.
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp)
+    if (tid + 256 * pp < NB * HSB) {
+      const float u = unwritten_value();
+      for (int b = 0; b < kPolledTiles; ++b)
+        store_exchanged4(gs, xdv + (size_t)b * tile_floats + ((size_t)pj[pp] * NB + pl[pp]) * 4, u, u, u, u);
+    }
+  group_arrive(gs);  // also: the slice is complete in LDS
+  group_wait(gs);
 
   // Step inputs that do not depend on the recurrence, fetched one step ahead.
   struct StepIn { float vt[4], c0, c1, dhn, dcn, m; };
@@ -267,7 +311,9 @@ void lstm_backward_kernel(LstmBwdParams p) {
 
   for (int t = T - 1; t >= 0; --t) {
     float dh_keep[PP], dv[PP][4];
-    float* xdv_t = xdv + (t & 1) * tile_floats;
+    const int done = T - 1 - t;  // steps done so far; this step uses polled tile done % 4
+    float* xdv_t = xdv + (done & 3) * tile_floats;
+    float* xdv_done = xdv + ((done + 2) & 3) * tile_floats;  // read two steps ago
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
       dh_keep[pp] = 0.f;
@@ -301,13 +347,24 @@ void lstm_backward_kernel(LstmBwdParams p) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) dbacc[pp][g] += dv[pp][g];
       }
-      // rows and units beyond the problem are published as zeros
-      if (tid + 256 * pp < NB * HSB)
-        store_exchanged4(gs, xdv_t + ((size_t)pj[pp] * NB + pl[pp]) * 4, dv[pp][0], dv[pp][1],
-                         dv[pp][2], dv[pp][3]);
     }
-    group_arrive(gs);   // dv_t of this workgroup's units is published
-    // The caller's copy is written behind the barrier: nobody in the launch waits for it.
+    // What this wavefront stored during the previous step (its resets among it) has landed
+    // before the gate gradients of this step become visible.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      // rows and units beyond the problem are published as zeros
+      if (tid + 256 * pp < NB * HSB) {
+        const size_t e = ((size_t)pj[pp] * NB + pl[pp]) * 4;
+        store_exchanged4(gs, xdv_t + e, publishable(dv[pp][0]), publishable(dv[pp][1]),
+                         publishable(dv[pp][2]), publishable(dv[pp][3]));
+        if (done + 2 < T) {
+          const float u = unwritten_value();
+          store_exchanged4(gs, xdv_done + e, u, u, u, u);
+        }
+      }
+    }
+    // The caller's copy: nobody in the launch waits for it.
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
       if (act[pp]) {
@@ -316,15 +373,15 @@ void lstm_backward_kernel(LstmBwdParams p) {
         for (int g = 0; g < 4; ++g) vt[g * H] = dv[pp][g];
       }
     }
-    fetch(t - 1);       // overlap next step's loads with the wait
-    group_wait(gs);     // dv_t of every unit is complete for this batch tile
-
-    tile_product<NB, 1, true>(xdvb, (t & 1) * tile_floats, Kpad, w_lds, red);
+    // The operand loads wait for dv_t of every unit themselves; the next step's inputs are
+    // requested once the first operands are in.
+    fetch(t - 1);
+    tile_product<NB, 1, true, true>(xdvb, (done & 3) * tile_floats, Kpad, w_lds, red, &gs);
     __syncthreads();
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp)
       if (tid + 256 * pp < NB * HSB) dh[pp] = dh_keep[pp] + sum_product<NB, 1>(red, pl[pp], pc[pp]);
-    // `red` is next written after the __syncthreads inside the next group_arrive.
+    __syncthreads();  // `red` may be overwritten by the next step's product
   }
 
 #pragma unroll
@@ -376,7 +433,8 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
 
   // Taken after the GEMM, which may replace the stream's scratch buffer with a larger one.
   Workspace ws;
-  HASTE_HIP_PROPAGATE(get_workspace(stream, exchange_floats(H, tile.nb, tile.gy) * sizeof(float), &ws));
+  HASTE_HIP_PROPAGATE(get_workspace(
+      stream, exchange_floats(H, tile.nb, tile.gy, kPolledTiles) * sizeof(float), &ws));
   HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 
   LstmFwdParams p;
@@ -417,7 +475,7 @@ int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
 
   Workspace ws;
   const size_t db_floats = (size_t)tile.gy * 4 * H;
-  const size_t xdv_floats = exchange_floats(64 * tile.gx, tile.nb, tile.gy);
+  const size_t xdv_floats = exchange_floats(64 * tile.gx, tile.nb, tile.gy, kPolledTiles);
   HASTE_HIP_PROPAGATE(get_workspace(stream, ((db_floats + 3) / 4 * 4 + xdv_floats) * sizeof(float), &ws));
   HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 

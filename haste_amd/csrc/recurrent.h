@@ -514,6 +514,67 @@ __device__ __forceinline__ float4_t load_tile4(const TileBuffer& b, int float_in
                   __uint_as_float(v.w)};
 }
 
+// ---- polled exchange tiles -------------------------------------------------------------
+// The step barrier costs a store acknowledgement (the producer may only raise its flag
+// once its data has landed), a flag round trip and then the operand load itself.  Polled
+// tiles drop the flags: an element that has not been published yet holds a bit pattern no
+// producer ever stores (all ones, a NaN that publishable() maps to the canonical NaN), and
+// the consumers' operand loads are themselves the wait: a wavefront re-issues the loads of
+// a chunk until none of its elements is unwritten.  What a consumer has seen of step s
+// therefore tells it that every producer of those elements had finished step s-1.
+//
+// kPolledTiles tiles rotate.  The tile read at step s is reset to "unwritten" by its
+// owners during step s+1 (once their workgroup has seen all of step s+1's data, nobody can
+// still be reading step s), and is written again at the earliest two steps later, behind an
+// s_waitcnt vmcnt(0) that the reset has long satisfied: a consumer that has seen what an
+// owner published at that point is guaranteed to see the reset as well, so a stale value
+// of four steps ago can never pass for new data.
+constexpr unsigned int kUnwrittenBits = 0xffffffffu;
+constexpr int kPolledTiles = 4;
+
+__device__ __forceinline__ float unwritten_value() { return __uint_as_float(kUnwrittenBits); }
+__device__ __forceinline__ float publishable(float v) {
+  return __float_as_uint(v) == kUnwrittenBits ? __uint_as_float(0x7fc00000u) : v;
+}
+
+// True (in every lane) when no lane of the wavefront holds an unwritten element.
+template <int A, int B>
+__device__ __forceinline__ bool all_written(const float4_t (&av)[A][B]) {
+  unsigned int m = 0u;
+#pragma unroll
+  for (int a = 0; a < A; ++a)
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+      const unsigned int x = __float_as_uint(av[a][b].x), y = __float_as_uint(av[a][b].y);
+      const unsigned int z = __float_as_uint(av[a][b].z), w = __float_as_uint(av[a][b].w);
+      const unsigned int xy = x > y ? x : y, zw = z > w ? z : w;
+      const unsigned int q = xy > zw ? xy : zw;
+      m = m > q ? m : q;
+    }
+  return __all(m != kUnwrittenBits) != 0;
+}
+
+// Re-issues `load()` until `written()`; gives up (abort flag, host status) after the launch's
+// spin limit or when another workgroup has given up, so that every wavefront still reaches
+// the end of the kernel.
+template <class LoadFn, class WrittenFn>
+__device__ __forceinline__ void poll_until_written(const GroupSync& g, LoadFn&& load, WrittenFn&& written) {
+  unsigned int spins = 0;
+  while (!written()) {
+    ++spins;
+    if ((spins & 255u) == 0u) {
+      const unsigned int ab = __hip_atomic_load(g.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (spins >= g.spin_limit && (threadIdx.x & 63) == 0) {
+        __hip_atomic_store(g.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(g.host_status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      }
+      if (ab != 0u || spins >= g.spin_limit) break;
+    }
+    asm volatile("" ::: "memory");  // the loads must really be issued again
+    load();
+  }
+}
+
 // 16x16x4 path: A operands of k-groups [g_abs, g_abs+CHUNK) from an exchange tile of
 // 16*RT rows.  Lane l holds row l%16 (of each 16-row block) and k = 16 g + 4 (l/16) .. +3.
 template <int RT, int CHUNK>
@@ -535,9 +596,10 @@ __device__ __forceinline__ void load_tile_chunk(const TileBuffer& xb, int tile_o
   }
 }
 
-template <int RT, int CT, int CHUNK>
+template <int RT, int CT, int CHUNK, bool POLLED>
 __device__ __forceinline__ void tall_tile_product(const TileBuffer& xb, int tile_off, int Kpad,
-                                                  const float* w_lds, float* red) {
+                                                  const float* w_lds, float* red,
+                                                  const GroupSync* gs) {
   const int wave = threadIdx.x >> 6;
   const int groups = Kpad >> 6;  // k-groups of 16 per wavefront
   const int full = groups / CHUNK;
@@ -554,6 +616,9 @@ __device__ __forceinline__ void tall_tile_product(const TileBuffer& xb, int tile
     load_tile_chunk<RT, CHUNK>(xb, tile_off, g, g_end, cur);
     for (int c = 0; c < full; ++c) {
       if (c + 1 < full) load_tile_chunk<RT, CHUNK>(xb, tile_off, g + CHUNK, g_end, nxt);
+      if constexpr (POLLED)
+        poll_until_written(*gs, [&] { load_tile_chunk<RT, CHUNK>(xb, tile_off, g, g_end, cur); },
+                           [&] { return all_written(cur); });
       mfma_chunk<RT, CT, CHUNK>(w_lds, g, cur, acc, acc1);
 #pragma unroll
       for (int gi = 0; gi < CHUNK; ++gi)
@@ -565,6 +630,9 @@ __device__ __forceinline__ void tall_tile_product(const TileBuffer& xb, int tile
   for (; g < g_end; ++g) {
     float4_t one[1][RT];
     load_tile_chunk<RT, 1>(xb, tile_off, g, g_end, one);
+    if constexpr (POLLED)
+      poll_until_written(*gs, [&] { load_tile_chunk<RT, 1>(xb, tile_off, g, g_end, one); },
+                         [&] { return all_written(one); });
     mfma_chunk<RT, CT, 1>(w_lds, g, one, acc, acc1);
   }
 #pragma unroll
@@ -660,9 +728,10 @@ __device__ __forceinline__ void mfma_tile_rows4(const float* w_lds, int s,
 // 4*rb + r, column ct*MC + l%MC, partial g = l/MC).  The operand
 // loads of chunk c+1 (CH super-groups) are issued before the MFMAs of chunk c; the two
 // register buffers alternate so that nothing is copied.
-template <int RB, int CT, int CH>
+template <int RB, int CT, int CH, bool POLLED>
 __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int tile_off, int Kpad,
-                                                       const float* w_lds, float* red) {
+                                                       const float* w_lds, float* red,
+                                                       const GroupSync* gs) {
   using S = ShortTileShape<CT>;
   constexpr int NB = 4 * RB;
   const int lane = threadIdx.x & 63;
@@ -683,10 +752,16 @@ __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int
     int c = 0;
     for (;;) {
       if (c + 1 < chunks) load_tile_rows4<RB, CT, CH>(xb, tile_off, s + 4 * CH, buf1);
+      if constexpr (POLLED)
+        poll_until_written(*gs, [&] { load_tile_rows4<RB, CT, CH>(xb, tile_off, s, buf0); },
+                           [&] { return all_written(buf0); });
       mfma_tile_rows4<RB, CT, CH>(w_lds, s, buf0, acc0, acc1);
       s += 4 * CH;
       if (++c == chunks) break;
       if (c + 1 < chunks) load_tile_rows4<RB, CT, CH>(xb, tile_off, s + 4 * CH, buf0);
+      if constexpr (POLLED)
+        poll_until_written(*gs, [&] { load_tile_rows4<RB, CT, CH>(xb, tile_off, s, buf1); },
+                           [&] { return all_written(buf1); });
       mfma_tile_rows4<RB, CT, CH>(w_lds, s, buf1, acc0, acc1);
       s += 4 * CH;
       if (++c == chunks) break;
@@ -695,6 +770,9 @@ __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int
   for (; s < s_end; s += 4) {
     float4_t one[1][RB];
     load_tile_rows4<RB, CT, 1>(xb, tile_off, s, one);
+    if constexpr (POLLED)
+      poll_until_written(*gs, [&] { load_tile_rows4<RB, CT, 1>(xb, tile_off, s, one); },
+                         [&] { return all_written(one); });
     mfma_tile_rows4<RB, CT, 1>(w_lds, s, one, acc0, acc1);
   }
 
@@ -715,27 +793,29 @@ __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int
 // red <- partial tiles of tile[NB rows, Kpad] * slice[Kpad, 16*CT]; the exchange tile
 // starts at float `tile_off` of `xb`.  LONG_K selects deeper prefetch for contractions much
 // longer than the hidden size (the backward passes).
-template <int NB, int CT, bool LONG_K>
+// POLLED: the tile is a polled exchange tile (see above) and `gs` supplies the bounds of the
+// wait; otherwise the caller has waited at the group's step barrier and `gs` is unused.
+template <int NB, int CT, bool LONG_K, bool POLLED = false>
 __device__ __forceinline__ void tile_product(const TileBuffer& xb, int tile_off, int Kpad,
-                                             const float* w_lds, float* red) {
+                                             const float* w_lds, float* red,
+                                             const GroupSync* gs = nullptr) {
   if constexpr (ProductTile<NB, CT>::kShort) {
-    short_exchange_product<NB / 4, CT, LONG_K ? 4 : 2>(xb, tile_off, Kpad, w_lds, red);
+    short_exchange_product<NB / 4, CT, LONG_K ? 4 : 2, POLLED>(xb, tile_off, Kpad, w_lds, red, gs);
   } else {
     constexpr int RT = NB / 16;
     constexpr int CHUNK = LONG_K ? (RT == 1 ? 8 : (RT == 2 ? 4 : 2)) : (RT >= 4 ? 2 : 4);
-    tall_tile_product<RT, CT, CHUNK>(xb, tile_off, Kpad, w_lds, red);
+    tall_tile_product<RT, CT, CHUNK, POLLED>(xb, tile_off, Kpad, w_lds, red, gs);
   }
 }
 
-// Zeroes this workgroup's share of its group's two exchange tiles: float4 rows
-// [first4, first4 + count4) of [Kpad/4][NB][4], both parities.  The stores have completed
+// Zeroes this workgroup's share of its group's exchange tiles: float4 rows
+// [first4, first4 + count4) of [Kpad/4][NB][4], in each of the n_tiles tiles.  The stores have completed
 // when it returns.  Called by all threads.
 __device__ __forceinline__ void zero_tile_share(const GroupSync& g, float* tiles, int tile_floats,
-                                                int nb, int first4, int count4) {
+                                                int nb, int first4, int count4, int n_tiles = 2) {
   for (int i = threadIdx.x; i < count4 * nb; i += 256) {
     float* q = tiles + ((size_t)first4 * nb + i) * 4;
-    store_exchanged4(g, q, 0.f, 0.f, 0.f, 0.f);
-    store_exchanged4(g, q + tile_floats, 0.f, 0.f, 0.f, 0.f);
+    for (int b = 0; b < n_tiles; ++b) store_exchanged4(g, q + (size_t)b * tile_floats, 0.f, 0.f, 0.f, 0.f);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
@@ -846,10 +926,11 @@ int launch_persistent(const char* name, KernelT kernel, const LaunchPlan& plan, 
 
 constexpr size_t kMaxLdsBytes = 160 * 1024;  // LDS per workgroup on gfx950
 
-// Floats of the two exchange tiles of every group (batch tile) for contraction length K.
-inline size_t exchange_floats(int K, int nb, int gy) {
+// Floats of the exchange tiles (2 behind a step barrier, kPolledTiles when polled) of every
+// group (batch tile) for contraction length K.
+inline size_t exchange_floats(int K, int nb, int gy, int n_tiles = 2) {
   const size_t Kpad = (size_t)(K + 63) / 64 * 64;
-  return 2 * Kpad * nb * gy;
+  return (size_t)n_tiles * Kpad * nb * gy;
 }
 
 // Geometry of a forward recurrence: nb batch rows and hs hidden units per workgroup
