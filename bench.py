@@ -22,9 +22,9 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch at the metric workload, from two rocprofv3 --pmc runs (FETCH_SIZE, then
 # WRITE_SIZE) scaled by what the same counters read for a 1 GiB device copy (--workload copy):
 # one FETCH_SIZE unit = 2.000 KiB, one WRITE_SIZE unit = 1.000 KiB.  A GEMM "launch" is the mean
-# of the step's four products, each with its share of the split-K reduce.
-MEASURED_TRAFFIC_BYTES = {"gemm_f32": 250.0e6, "lstm_forward_recurrence": 167.0e6,
-                          "lstm_backward_recurrence": 181.9e6}
+# of the step's four products, each with its split reduce.
+MEASURED_TRAFFIC_BYTES = {"gemm_f32": 208.3e6, "lstm_forward_recurrence": 166.8e6,
+                          "lstm_backward_recurrence": 183.0e6}
 
 
 def parse():
@@ -34,7 +34,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget", type=float, default=15.0)
-    ap.add_argument("--workload", choices=["all", "metric", "streaming", "copy"], default="all",
+    ap.add_argument("--workload", choices=["all", "metric", "streaming", "copy", "configs"], default="all",
                     help="restrict the run to one workload (for profiling); the JSON line is "
                          "only complete with 'all'.  'copy' runs a plain device copy of known "
                          "size, the yardstick for the FETCH_SIZE / WRITE_SIZE counters")
@@ -175,6 +175,83 @@ def run_streaming(args, torch, lib, ops, dev):
     return out, (W1, R1, b1, x1)
 
 
+def run_configs(args, torch, lib, ops, dev):
+    """The other BASELINE.json configurations (parity-test cases; timed here for the record):
+    forward (+ backward with the caller-side transposes) in ms per call."""
+    def timed(fn, reps):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return round(e0.elapsed_time(e1) / reps, 4)
+
+    g = torch.Generator(device="cpu").manual_seed(0)
+
+    def rnd(*shape, scale=1.0):
+        return (torch.randn(*shape, generator=g) * scale).to(dev)
+
+    def uni(k, *shape):
+        return ((torch.rand(*shape, generator=g) * 2 - 1) * k).to(dev)
+    no_mask = torch.empty(0, 0, 0, device=dev)
+    out = {}
+
+    T, N, C, H = 100, 16, 128, 256  # config 1: LSTM forward inference
+    k = H ** -0.5
+    x, W, R, b = rnd(T, N, C), uni(k, C, 4 * H), uni(k, H, 4 * H), torch.zeros(4 * H, device=dev)
+    z = torch.zeros(N, H, device=dev)
+    out["lstm_inference_N16_T100_C128_H256_ms"] = timed(
+        lambda: ops.lstm_forward(False, 0.0, x, z, z, W, R, b, no_mask), 50)
+
+    T, N, C, H = 100, 64, 512, 512  # config 2: GRU training, zoneout 0.1, DropConnect 0.05
+    k = H ** -0.5
+    x, W, R = rnd(T, N, C), uni(k, C, 3 * H), uni(k, H, 3 * H)
+    bx, br, z = uni(k, 3 * H), uni(k, 3 * H), torch.zeros(N, H, device=dev)
+    zm = (torch.rand(T, N, H, generator=g) >= 0.1).float().to(dev)
+    dm = (torch.rand(H, 3 * H, generator=g) >= 0.05).float().to(dev)
+    dh_new = rnd(T + 1, N, H)
+
+    def gru_step():
+        h, cache = ops.gru_forward(True, 0.1, x, z, W, R, bx, br, zm, dm, 1.0 / 0.95)
+        Reff_t = ops.transpose(R * dm * (1.0 / 0.95))
+        return ops.gru_backward(ops.transpose(x), ops.transpose(W), Reff_t, bx, br, zm, h, cache, dh_new)
+    out["gru_fwd_bwd_N64_T100_H512_zoneout_dropconnect_ms"] = timed(gru_step, 30)
+
+    T, N, C, H = 100, 128, 512, 512  # config 3: LSTM training, N=128
+    x, W, R = rnd(T, N, C), uni(k, C, 4 * H), uni(k, H, 4 * H)
+    b = torch.zeros(4 * H, device=dev)
+    b[2 * H:3 * H] = 1.0
+    z = torch.zeros(N, H, device=dev)
+    dh_new, dc_new = rnd(T + 1, N, H), rnd(T + 1, N, H)
+
+    def lstm_step():
+        h, c, cache = ops.lstm_forward(True, 0.0, x, z, z, W, R, b, no_mask)
+        return ops.lstm_backward(ops.transpose(x), ops.transpose(W), ops.transpose(R), b, no_mask, h, c,
+                                 cache, dh_new, dc_new)
+    out["lstm_fwd_bwd_N128_T100_H512_ms"] = timed(lstm_step, 30)
+
+    T, N, C, H = 500, 32, 256, 256  # config 4: LayerNormLSTM training, zoneout 0.1
+    k = H ** -0.5
+    x, W, R = rnd(T, N, C), uni(k, C, 4 * H), uni(k, H, 4 * H)
+    b = torch.zeros(4 * H, device=dev)
+    b[2 * H:3 * H] = 1.0
+    gamma, gamma_h, beta_h = torch.ones(2, 4 * H, device=dev), torch.ones(H, device=dev), torch.zeros(H, device=dev)
+    z = torch.zeros(N, H, device=dev)
+    zm = (torch.rand(T, N, H, generator=g) >= 0.1).float().to(dev)
+    dh_new, dc_new = rnd(T + 1, N, H), rnd(T + 1, N, H)
+
+    def ln_lstm_step():
+        fwd = ops.layer_norm_lstm_forward(True, 0.1, x, z, z, W, R, b, gamma, gamma_h, beta_h, zm)
+        return ops.layer_norm_lstm_backward(ops.transpose(x), ops.transpose(W), ops.transpose(R), b, gamma,
+                                            gamma_h, beta_h, zm, *fwd, dh_new, dc_new)
+    out["layer_norm_lstm_fwd_bwd_N32_T500_H256_zoneout_ms"] = timed(ln_lstm_step, 10)
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -204,6 +281,9 @@ def main():
         m = run_metric(args, torch, lib, ops, dev)
         print(json.dumps({"workload": "metric", "ms_per_step": round(m["ms_per_step"], 4),
                           "kernels": m["kernels"]}))
+        return
+    if args.workload == "configs":
+        print(json.dumps(run_configs(args, torch, lib, ops, dev)))
         return
     if args.workload == "streaming":
         s, _ = run_streaming(args, torch, lib, ops, dev)
