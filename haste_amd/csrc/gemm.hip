@@ -31,16 +31,31 @@ constexpr int LDB = BN + 4;
 constexpr int B_STAGE = BK * LDB;
 constexpr int kXcds = 8;
 
-__device__ __forceinline__ float4_t load4_guarded(const float* p, int valid, bool vec_ok) {
-  float4_t v = {0.f, 0.f, 0.f, 0.f};
-  if (valid >= 4 && vec_ok) {
-    v = *reinterpret_cast<const float4_t*>(p);
-  } else {
-    if (valid > 0) v.x = p[0];
-    if (valid > 1) v.y = p[1];
-    if (valid > 2) v.z = p[2];
-    if (valid > 3) v.w = p[3];
-  }
+// Operand panels are read through buffer resources: a 16-byte load at any 4-byte aligned
+// offset, elements beyond the resource's range read as zero and never fault.  That keeps the
+// K loop free of branches (the compiler can then overlap the loads of the next step with the
+// MFMAs of this one); `valid` (how many of the four elements belong to the problem) is applied
+// with selects.
+typedef unsigned int uint4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_panel(const float* base, long long floats) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, (int)(floats * 4), 0x00020000);
+}
+
+// The load is issued here; `valid` is applied by masked4() when the data is used, so that
+// nothing waits for the load in between.
+__device__ __forceinline__ uint4_t load4_raw(__amdgpu_buffer_rsrc_t panel, long long float_offset,
+                                             int valid) {
+  const unsigned int off = valid > 0 ? (unsigned int)(float_offset * 4) : 0x7ffffff0u;
+  return __builtin_amdgcn_raw_buffer_load_b128(panel, off, 0, 0);
+}
+
+__device__ __forceinline__ float4_t masked4(uint4_t u, int valid) {
+  float4_t v;
+  v.x = valid > 0 ? __uint_as_float(u.x) : 0.f;
+  v.y = valid > 1 ? __uint_as_float(u.y) : 0.f;
+  v.z = valid > 2 ? __uint_as_float(u.z) : 0.f;
+  v.w = valid > 3 ? __uint_as_float(u.w) : 0.f;
   return v;
 }
 
@@ -53,7 +68,6 @@ void gemm_f32_kernel(int M, int N, int K,
                      const float* __restrict__ B, int ldb,
                      float* __restrict__ C, int ldc, int accumulate,
                      int tiles_n, int whole_tiles, int splits, int k_per_split,
-                     int a_vec_ok, int b_vec_ok,
                      float* __restrict__ partial) {
   // A tile k-major in LDS: leading dimension BM+2 when it is written with transposing
   // scalar stores (bank-conflict free), BM+4 when written with 16-byte stores.
@@ -102,10 +116,20 @@ void gemm_f32_kernel(int M, int N, int K,
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  float4_t a_reg[A_PASSES], b_reg[2];
+  uint4_t a_raw[A_PASSES], b_raw[2];
+  int a_valid[A_PASSES], b_valid[2];
   // A tile stored [K][M] in memory: one pass covers (256*4/BM) k-rows of BM columns.
   constexpr int TA_ROWS = 1024 / BM;
   constexpr int TA_COLS = BM / 4;
+
+  // This workgroup's operand panels: its BM rows (TRANS_A: columns) of A and its 128 columns
+  // of B, all of K.  Offsets below are in floats from the panel's first element.
+  const int rows_here = (M - m0) < BM ? (M - m0) : BM;
+  const int cols_here = (N - n0) < BN ? (N - n0) : BN;
+  const __amdgpu_buffer_rsrc_t a_panel =
+      TRANS_A ? make_panel(A + m0, (long long)(K - 1) * lda + rows_here)
+              : make_panel(A + (size_t)m0 * lda, (long long)(rows_here - 1) * lda + K);
+  const __amdgpu_buffer_rsrc_t b_panel = make_panel(B + n0, (long long)(K - 1) * ldb + cols_here);
 
   auto load_global = [&](int kk) {
 #pragma unroll
@@ -113,24 +137,24 @@ void gemm_f32_kernel(int M, int N, int K,
       if (TRANS_A) {
         const int ak = (tid / TA_COLS) + TA_ROWS * i;
         const int am = (tid % TA_COLS) * 4;
-        const int k = kk + ak, m = m0 + am;
-        const int valid = (k < k_end) ? (M - m) : 0;
-        a_reg[i] = load4_guarded(A + (size_t)k * lda + m, valid, a_vec_ok);
+        const int k = kk + ak;
+        a_valid[i] = (k < k_end) ? (rows_here - am) : 0;
+        a_raw[i] = load4_raw(a_panel, (long long)k * lda + am, a_valid[i]);
       } else {
         const int arow = (tid >> 2) + 64 * i;
         const int ak = (tid & 3) * 4;
-        const int m = m0 + arow, k = kk + ak;
-        const int valid = (m < M) ? (k_end - k) : 0;
-        a_reg[i] = load4_guarded(A + (size_t)m * lda + k, valid, a_vec_ok);
+        const int k = kk + ak;
+        a_valid[i] = (arow < rows_here) ? (k_end - k) : 0;
+        a_raw[i] = load4_raw(a_panel, (long long)arow * lda + k, a_valid[i]);
       }
     }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int bk = (tid >> 5) + 8 * i;
       const int bn = (tid & 31) * 4;
-      const int k = kk + bk, n = n0 + bn;
-      const int valid = (k < k_end) ? (N - n) : 0;
-      b_reg[i] = load4_guarded(B + (size_t)k * ldb + n, valid, b_vec_ok);
+      const int k = kk + bk;
+      b_valid[i] = (k < k_end) ? (cols_here - bn) : 0;
+      b_raw[i] = load4_raw(b_panel, (long long)k * ldb + bn, b_valid[i]);
     }
   };
 
@@ -139,39 +163,55 @@ void gemm_f32_kernel(int M, int N, int K,
     float* bs = Bs + buf * B_STAGE;
 #pragma unroll
     for (int i = 0; i < A_PASSES; ++i) {
+      const float4_t a = masked4(a_raw[i], a_valid[i]);
       if (TRANS_A) {
         const int ak = (tid / TA_COLS) + TA_ROWS * i;
         const int am = (tid % TA_COLS) * 4;
-        *reinterpret_cast<float4_t*>(as + ak * LDA + am) = a_reg[i];
+        *reinterpret_cast<float4_t*>(as + ak * LDA + am) = a;
       } else {
         const int arow = (tid >> 2) + 64 * i;
         const int ak = (tid & 3) * 4;
-        as[(ak + 0) * LDA + arow] = a_reg[i].x;
-        as[(ak + 1) * LDA + arow] = a_reg[i].y;
-        as[(ak + 2) * LDA + arow] = a_reg[i].z;
-        as[(ak + 3) * LDA + arow] = a_reg[i].w;
+        as[(ak + 0) * LDA + arow] = a.x;
+        as[(ak + 1) * LDA + arow] = a.y;
+        as[(ak + 2) * LDA + arow] = a.z;
+        as[(ak + 3) * LDA + arow] = a.w;
       }
     }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int bk = (tid >> 5) + 8 * i;
       const int bn = (tid & 31) * 4;
-      *reinterpret_cast<float4_t*>(bs + bk * LDB + bn) = b_reg[i];
+      *reinterpret_cast<float4_t*>(bs + bk * LDB + bn) = masked4(b_raw[i], b_valid[i]);
     }
   };
 
   auto compute = [&](int buf) {
     const float* as = As + buf * A_STAGE + (lane >> 5) * LDA + wm + (lane & 31);
     const float* bs = Bs + buf * B_STAGE + (lane >> 5) * LDB + wn + (lane & 31);
+    // The LDS reads of K pair k2+2 are issued before the MFMAs of pair k2.
+    float b_nxt[2], a_nxt[MI];
+    b_nxt[0] = bs[0];
+    b_nxt[1] = bs[32];
+#pragma unroll
+    for (int i = 0; i < MI; ++i) a_nxt[i] = as[32 * i];
 #pragma unroll
     for (int k2 = 0; k2 < BK; k2 += 2) {
-      const float b0 = bs[k2 * LDB];
-      const float b1 = bs[k2 * LDB + 32];
+      const float b0 = b_nxt[0], b1 = b_nxt[1];
+      float av[MI];
+#pragma unroll
+      for (int i = 0; i < MI; ++i) av[i] = a_nxt[i];
+      if (k2 + 2 < BK) {
+        b_nxt[0] = bs[(k2 + 2) * LDB];
+        b_nxt[1] = bs[(k2 + 2) * LDB + 32];
+#pragma unroll
+        for (int i = 0; i < MI; ++i) a_nxt[i] = as[(k2 + 2) * LDA + 32 * i];
+        // keep the reads here: the scheduler would otherwise sink them to just before their use
+        __builtin_amdgcn_sched_barrier(0);
+      }
 #pragma unroll
       for (int i = 0; i < MI; ++i) {
-        const float av = as[k2 * LDA + 32 * i];
-        acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b0, acc[i][0], 0, 0, 0);
-        acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b1, acc[i][1], 0, 0, 0);
+        acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], b0, acc[i][0], 0, 0, 0);
+        acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], b1, acc[i][1], 0, 0, 0);
       }
     }
   };
@@ -318,15 +358,17 @@ int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
     HASTE_HIP_PROPAGATE(get_workspace(stream, bytes, &ws));
     partial = ws.scratch;
   }
-  const int a_vec_ok = aligned16(A) && (lda % 4 == 0) && (k_per_split % 4 == 0);
-  const int b_vec_ok = aligned16(B) && (ldb % 4 == 0);
+  // A workgroup addresses its operand panels (its rows of A, its columns of B, all of K)
+  // with 32-bit byte offsets.
+  HASTE_HIP_REQUIRE(((long long)(trans_a ? K : bm) * lda + (trans_a ? bm : K)) * 4 < (1ll << 31));
+  HASTE_HIP_REQUIRE(((long long)K * ldb + BN) * 4 < (1ll << 31));
   dim3 grid((unsigned)(whole_tiles + pieces)), block(256);
   ScopedKernelTimer timer("gemm_f32", stream);
 #define HASTE_GEMM_LAUNCH(TA_, BM_)                                                          \
   if (trans_a == TA_ && bm == BM_)                                                           \
     gemm_f32_kernel<TA_, BM_><<<grid, block, 0, stream>>>(                                   \
         M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, tiles_n, whole_tiles, splits,   \
-        k_per_split, a_vec_ok, b_vec_ok, partial);
+        k_per_split, partial);
   HASTE_GEMM_LAUNCH(false, 128) HASTE_GEMM_LAUNCH(false, 64)
   HASTE_GEMM_LAUNCH(true, 128) HASTE_GEMM_LAUNCH(true, 64)
 #undef HASTE_GEMM_LAUNCH

@@ -373,8 +373,8 @@ void lstm_backward_kernel(LstmBwdParams p) {
         for (int g = 0; g < 4; ++g) vt[g * H] = dv[pp][g];
       }
     }
-    // The operand loads wait for dv_t of every unit themselves; the next step's inputs are
-    // requested once the first operands are in.
+    // The next step's inputs are requested now; the operand loads of the product wait for
+    // dv_t of every unit themselves.
     fetch(t - 1);
     tile_product<NB, 1, true, true>(xdvb, (done & 3) * tile_floats, Kpad, w_lds, red, &gs);
     __syncthreads();
