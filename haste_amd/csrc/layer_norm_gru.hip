@@ -25,7 +25,7 @@ struct LnGruFwdParams {
   float* cache2;         // [T*N,2] or null
   float zoneout_prob;
   const float* zoneout_mask;
-  float* part2;          // exchange [groups][gx][NB][2]
+  unsigned long long* part2;  // tagged row exchange [groups][2][gx][NB] slots: moments of h*R
   float* xh;             // exchange tiles of h: [batch tiles][2][Kpad/4][NB][4]
   LaunchShape ls;
 };
@@ -56,17 +56,21 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
   const size_t NH = (size_t)N * H;
   const int own_units = (H - j0) < HS ? (H - j0) : HS;
   const int last_units = H - (gx - 1) * HS;
-  float* part2 = p.part2 + (size_t)role.bt * gx * NB * 2;
+  const size_t row_words = tagged_row_words(gx, NB, 2);
+  unsigned long long* part2 = p.part2 + (size_t)role.bt * 2 * row_words;
 
   const int tile_floats = Kpad * NB;
-  float* xh = p.xh + (size_t)role.bt * 2 * tile_floats;
-  const TileBuffer xhb = make_tile_buffer(xh, 2 * tile_floats);
+  float* xh = p.xh + (size_t)role.bt * kPolledTiles * tile_floats;
+  const TileBuffer xhb = make_tile_buffer(xh, kPolledTiles * tile_floats);
 
   GroupSync gs;
   group_sync_init(gs, p.ls, role);
 
-  // Own k range of the exchange tiles (the last workgroup also owns the padding).
-  zero_tile_share(gs, xh, tile_floats, NB, j0 / 4, (role.cw == gx - 1 ? Kpad - j0 : HS) / 4);
+  // Own k range of the exchange tiles (the last workgroup also owns the padding): rows and
+  // k beyond the problem stay zero for the whole launch.
+  zero_tile_share(gs, xh, tile_floats, NB, j0 / 4, (role.cw == gx - 1 ? Kpad - j0 : HS) / 4,
+                  kPolledTiles);
+  clear_row_words(gs, part2, gx, role.cw, NB, 2);
 
   {
     const bool fast = H % 4 == 0 && (reinterpret_cast<uintptr_t>(p.R) & 15u) == 0;
@@ -97,28 +101,49 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
     }
   }
   const bool zoneout = p.zoneout_prob != 0.f && p.zoneout_mask != nullptr;
+  // Tile 0 receives h[0]; the elements of the other tiles that steps will publish start out
+  // unwritten.  One real barrier: nobody polls before every owner has set its share up.
 #pragma unroll
   for (int pp = 0; pp < PP; ++pp)
-    if (act[pp]) store_exchanged(gs, &xh[xchg_index(pj[pp], pl[pp], NB)], h_prev[pp]);
-  group_arrive(gs);  // h[0] is published; the slice is complete in LDS
+    if (act[pp]) {
+      float* e = &xh[xchg_index(pj[pp], pl[pp], NB)];
+      store_exchanged(gs, e, publishable(h_prev[pp]));
+      for (int b = 1; b < kPolledTiles; ++b) store_exchanged(gs, e + (size_t)b * tile_floats, unwritten_value());
+    }
+  group_arrive(gs);  // also: the slice is complete in LDS
+  group_wait(gs);
+
+  // Inputs of a step that do not depend on the recurrence, fetched one step ahead.
+  float wx_next[PP][3], mk_next[PP];
+  auto fetch = [&](int t) {
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      mk_next[pp] = 1.f;
+#pragma unroll
+      for (int g = 0; g < 3; ++g) wx_next[pp][g] = 0.f;
+      if (act[pp] && t < T) {
+        const float* wt = p.Wxn + ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 3; ++g) wx_next[pp][g] = wt[g * H];
+        if (zoneout && p.training) mk_next[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
+      }
+    }
+  };
+  fetch(0);
 
   for (int t = 0; t < T; ++t) {
     float wx[PP][3], mk[PP];
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
-      mk[pp] = 1.f;
+      mk[pp] = mk_next[pp];
 #pragma unroll
-      for (int g = 0; g < 3; ++g) wx[pp][g] = 0.f;
-      if (act[pp]) {
-        const float* wt = p.Wxn + ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
-#pragma unroll
-        for (int g = 0; g < 3; ++g) wx[pp][g] = wt[g * H];
-        if (zoneout && p.training) mk[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
-      }
+      for (int g = 0; g < 3; ++g) wx[pp][g] = wx_next[pp][g];
     }
-    group_wait(gs);  // h[t]
+    const unsigned int tag = gs.epoch + 2u + (unsigned int)t;  // names this step's row exchange
+    unsigned long long* ex2 = part2 + (size_t)(t & 1) * row_words;
 
-    tile_product<NB, CT, false>(xhb, (t & 1) * tile_floats, Kpad, w_lds, red);
+    // The operand loads wait for h[t] themselves (polled tile t % 4).
+    tile_product<NB, CT, false, true>(xhb, (t & 3) * tile_floats, Kpad, w_lds, red, &gs);
     __syncthreads();
 
     float rh[PP][3];
@@ -130,11 +155,6 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
         rh[pp][g] = colok[pp] ? sum_product<NB, CT>(red, pl[pp], g * HS + pc[pp]) : 0.f;
         s += rh[pp][g];
       }
-      if (act[pp]) {
-        float* ar = p.act_Rh + ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
-#pragma unroll
-        for (int g = 0; g < 3; ++g) ar[g * H] = rh[pp][g];
-      }
       const float mean = segment_sum<HS>(s) / (3.0f * (float)own_units);
       float q = 0.f;
 #pragma unroll
@@ -143,49 +163,77 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
         q += colok[pp] ? d * d : 0.f;
       }
       q = segment_sum<HS>(q);
-      if (pc[pp] == 0 && tid + 256 * pp < NB * HS)
-        store_exchanged2(gs, part2 + ((size_t)role.cw * NB + pl[pp]) * 2, mean, q);
+      if (pc[pp] == 0 && tid + 256 * pp < NB * HS) {
+        const float mq[2] = {mean, q};
+        publish_row<2>(gs, ex2, NB, role.cw, pl[pp], mq, tag);
+      }
     }
-    group_arrive(gs);
-    group_wait(gs);
-    merge_row_moments<NB>(part2, gx, 3.0f * HS, 3.0f * last_units, 3.0f * H, stat);
+    merge_row_moments_polled<NB>(gs, ex2, gx, tag, 3.0f * HS, 3.0f * last_units, 3.0f * H, stat);
     __syncthreads();
 
+    float saved[PP][4], mu2[PP], is2[PP], h_pub[PP];
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
+      mu2[pp] = stat[pl[pp] * 2];
+      is2[pp] = stat[pl[pp] * 2 + 1];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) saved[pp][g] = 0.f;
       if (act[pp]) {
-        const float mu = stat[pl[pp] * 2], is = stat[pl[pp] * 2 + 1];
         float rn[3];
 #pragma unroll
-        for (int g = 0; g < 3; ++g) rn[g] = (rh[pp][g] - mu) * is * g2[pp][g];
+        for (int g = 0; g < 3; ++g) rn[g] = (rh[pp][g] - mu2[pp]) * is2[pp] * g2[pp][g];
         const float z = sigmoid_f(wx[pp][0] + rn[0] + bxv[pp][0] + brv[pp][0]);
         const float r = sigmoid_f(wx[pp][1] + rn[1] + bxv[pp][1] + brv[pp][1]);
         const float qg = rn[2] + brv[pp][2];
         const float g = tanh_f(wx[pp][2] + r * qg + bxv[pp][2]);
-        if (p.training) {
-          float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
-          vt[0] = z;
-          vt[H] = r;
-          vt[2 * H] = g;
-          vt[3 * H] = qg;
-        }
+        saved[pp][0] = z;
+        saved[pp][1] = r;
+        saved[pp][2] = g;
+        saved[pp][3] = qg;
         float h_new = z * h_prev[pp] + (1.0f - z) * g;
         if (zoneout) {
           if (p.training) h_new = (h_new - h_prev[pp]) * mk[pp] + h_prev[pp];
           else h_new = p.zoneout_prob * h_prev[pp] + (1.0f - p.zoneout_prob) * h_new;
         }
-        p.h[(size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp]] = h_new;
-        if (t + 1 < T)
-          store_exchanged(gs, &xh[((t + 1) & 1) * tile_floats + xchg_index(pj[pp], pl[pp], NB)], h_new);
         h_prev[pp] = h_new;
+      }
+      h_pub[pp] = publishable(h_prev[pp]);
+    }
+    // Everything this wavefront stored during the previous step (its resets among it) has
+    // landed before h[t+1] becomes visible.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (t + 1 < T) {
+      float* xh_next = xh + ((t + 1) & 3) * tile_floats;
+      float* xh_done = xh + ((t + 3) & 3) * tile_floats;  // read at step t-1: nobody needs it any more
+#pragma unroll
+      for (int pp = 0; pp < PP; ++pp)
+        if (act[pp]) {
+          const int e = xchg_index(pj[pp], pl[pp], NB);
+          store_exchanged(gs, &xh_next[e], h_pub[pp]);
+          if (t + 3 < T) store_exchanged(gs, &xh_done[e], unwritten_value());
+        }
+    }
+    fetch(t + 1);
+    __syncthreads();  // red and stat may be overwritten by the next step
+    // The caller's copies are written last: nobody in the launch waits for them.
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      if (act[pp]) {
+        float* ar = p.act_Rh + ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 3; ++g) ar[g * H] = rh[pp][g];
+        if (p.training) {
+          float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+#pragma unroll
+          for (int g = 0; g < 4; ++g) vt[g * H] = saved[pp][g];
+        }
+        p.h[(size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp]] = h_prev[pp];
         if (role.cw == 0 && pc[pp] == 0 && p.cache2 != nullptr) {
-          p.cache2[((size_t)t * N + pn[pp]) * 2 + 0] = mu;
-          p.cache2[((size_t)t * N + pn[pp]) * 2 + 1] = is;
+          p.cache2[((size_t)t * N + pn[pp]) * 2 + 0] = mu2[pp];
+          p.cache2[((size_t)t * N + pn[pp]) * 2 + 1] = is2[pp];
         }
       }
     }
-    if (t + 1 < T) group_arrive(gs);
-    else __syncthreads();
   }
 }
 
@@ -205,9 +253,9 @@ struct LnGruBwdParams {
   float* dgamma2;        // [3H]
   const float* cache2;   // [T*N,2]
   const float* zoneout_mask;
-  float* part;           // exchange [groups][gx][NB][4]
+  unsigned long long* part;  // tagged row exchange [groups][2][gx][NB] slots: h*R norm sums
   float* col_partial;    // [batch tiles][9][H]
-  float* xdq;            // exchange tiles of dq: [batch tiles][2][Kpad/4][NB][4]
+  float* xdq;            // polled exchange tiles of dq: [batch tiles][4][Kpad/4][NB][4]
   LaunchShape ls;
 };
 
@@ -243,19 +291,21 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
   const int n0 = role.bt * p.ls.tile_rows;
   const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
-  float* part = p.part + (size_t)role.bt * gx * NB * 4;
+  const size_t row_words = tagged_row_words(gx, NB, 3);
+  unsigned long long* part = p.part + (size_t)role.bt * 2 * row_words;
 
   const int tile_floats = Kpad * NB;
-  float* xdq = p.xdq + (size_t)role.bt * 2 * tile_floats;
-  const TileBuffer xdqb = make_tile_buffer(xdq, 2 * tile_floats);
+  float* xdq = p.xdq + (size_t)role.bt * kPolledTiles * tile_floats;
+  const TileBuffer xdqb = make_tile_buffer(xdq, kPolledTiles * tile_floats);
 
   GroupSync gs;
   group_sync_init(gs, p.ls, role);
 
   // Own k range of the exchange tiles (the last workgroup also owns the padding); only
-  // rows and units of the problem are written afterwards.
+  // rows and units of the problem are written afterwards, the rest stays zero.
   zero_tile_share(gs, xdq, tile_floats, NB, 12 * role.cw,
-                  (role.cw == gx - 1 ? Kpad - 48 * role.cw : 48) / 4);
+                  (role.cw == gx - 1 ? Kpad - 48 * role.cw : 48) / 4, kPolledTiles);
+  clear_row_words(gs, part, gx, role.cw, NB, 3);
 
   {
     const bool fast = H % 4 == 0 && (reinterpret_cast<uintptr_t>(p.R_t) & 15u) == 0;
@@ -284,7 +334,17 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
     for (int a = 0; a < NACC; ++a) accs[pp][a] = 0.f;
   }
   const bool zoneout = p.zoneout_mask != nullptr;
-  __syncthreads();
+  // The elements that steps will publish start out unwritten.  One real barrier: nobody
+  // polls before every owner has set its share up.
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp)
+    if (act[pp])
+      for (int b = 0; b < kPolledTiles; ++b)
+        for (int k = 0; k < 3; ++k)
+          store_exchanged(gs, xdq + (size_t)b * tile_floats + xchg_index(3 * pj[pp] + k, pl[pp], NB),
+                          unwritten_value());
+  group_arrive(gs);  // also: the slice is complete in LDS
+  group_wait(gs);
 
   struct StepIn { float vt[4], rh[3], h0, dhn, m, mu2, is2; };
   StepIn nxt[PP];
@@ -314,11 +374,16 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
   const float inv3H = 1.0f / (float)(3 * H);
   for (int t = T - 1; t >= 0; --t) {
     StepIn s[PP];
-    float dh_keep[PP], xc[PP][3], gd[PP][3];
+    float dh_keep[PP], xc[PP][3], gd[PP][3], dps[PP][3], dqs[PP][3];
+    const int done = T - 1 - t;  // steps done so far
+    const unsigned int tag = gs.epoch + 2u + (unsigned int)done;  // names this step's row exchange
+    unsigned long long* ex = part + (size_t)(done & 1) * row_words;
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
       s[pp] = nxt[pp];
       dh_keep[pp] = 0.f;
+#pragma unroll
+      for (int k = 0; k < 3; ++k) dps[pp][k] = dqs[pp][k] = 0.f;
       float t0 = 0.f, t1 = 0.f, t2 = 0.f;
 #pragma unroll
       for (int g = 0; g < 3; ++g) xc[pp][g] = gd[pp][g] = 0.f;
@@ -339,10 +404,9 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
         const float dr = dp_g * qg;
         const float dp_r = d_sigmoid_f(r) * dr;
         const float dp_z = d_sigmoid_f(z) * dz;
-        const size_t o3 = ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
-        p.dp[o3] = dp_z;
-        p.dp[o3 + H] = dp_r;
-        p.dp[o3 + 2 * H] = dp_g;
+        dps[pp][0] = dp_z;
+        dps[pp][1] = dp_r;
+        dps[pp][2] = dp_g;
         const float dqv[3] = {dp_z, dp_r, dq_g};
         accs[pp][0] += dp_z;
         accs[pp][1] += dp_r;
@@ -361,12 +425,12 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
       t0 = segment_sum<HSB>(t0);
       t1 = segment_sum<HSB>(t1);
       t2 = segment_sum<HSB>(t2);
-      if (pc[pp] == 0 && own[pp])
-        store_exchanged4(gs, part + ((size_t)role.cw * NB + pl[pp]) * 4, t0, t1, t2, 0.f);
+      if (pc[pp] == 0 && own[pp]) {
+        const float v3[3] = {t0, t1, t2};
+        publish_row<3>(gs, ex, NB, role.cw, pl[pp], v3, tag);
+      }
     }
-    group_arrive(gs);
-    group_wait(gs);
-    sum_row_partials<NB>(part, gx, sums);
+    sum_row_partials_polled<NB>(gs, ex, gx, tag, sums);
     __syncthreads();
 
 #pragma unroll
@@ -375,24 +439,47 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
         const float is2 = s[pp].is2;
         const float dsigma = -0.5f * sums[pl[pp] * 4 + 0] * is2 * is2 * is2;
         const float dmu = (-2.0f * sums[pl[pp] * 4 + 1] * dsigma * inv3H) - (sums[pl[pp] * 4 + 2] * is2);
-        float* dqt = p.dq + ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
 #pragma unroll
-        for (int k = 0; k < 3; ++k) {
-          const float d = (2.0f * xc[pp][k] * dsigma * inv3H) + (is2 * gd[pp][k]) + (dmu * inv3H);
-          store_exchanged(gs, xdq + (t & 1) * tile_floats + xchg_index(3 * pj[pp] + k, pl[pp], NB), d);
-          dqt[(size_t)k * H] = d;
-        }
+        for (int k = 0; k < 3; ++k)
+          dqs[pp][k] = (2.0f * xc[pp][k] * dsigma * inv3H) + (is2 * gd[pp][k]) + (dmu * inv3H);
       }
     }
-    group_arrive(gs);
+    // What this wavefront stored during the previous step (its resets among it) has landed
+    // before the gradients of this step become visible.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    {
+      float* xdq_t = xdq + (done & 3) * tile_floats;
+      float* xdq_done = xdq + ((done + 2) & 3) * tile_floats;  // read two steps ago
+#pragma unroll
+      for (int pp = 0; pp < PP; ++pp)
+        if (act[pp]) {
+#pragma unroll
+          for (int k = 0; k < 3; ++k) {
+            const int e = xchg_index(3 * pj[pp] + k, pl[pp], NB);
+            store_exchanged(gs, xdq_t + e, publishable(dqs[pp][k]));
+            if (done + 2 < T) store_exchanged(gs, xdq_done + e, unwritten_value());
+          }
+        }
+    }
+    // The caller's copies: nobody in the launch waits for them.
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp)
+      if (act[pp]) {
+        const size_t o3 = ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+          p.dp[o3 + (size_t)k * H] = dps[pp][k];
+          p.dq[o3 + (size_t)k * H] = dqs[pp][k];
+        }
+      }
     fetch(t - 1);
-    group_wait(gs);  // dq_t of every unit is complete for this batch tile
-
-    tile_product<NB, 1, true>(xdqb, (t & 1) * tile_floats, Kpad, w_lds, red);
+    // The operand loads wait for dq_t of every unit themselves.
+    tile_product<NB, 1, true, true>(xdqb, (done & 3) * tile_floats, Kpad, w_lds, red, &gs);
     __syncthreads();
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp)
       dh[pp] = dh_keep[pp] + sum_product<NB, 1>(red, pl[pp], pc[pp]);
+    __syncthreads();  // sums (and red) may be overwritten by the next step
   }
 
 #pragma unroll
@@ -449,14 +536,15 @@ int haste_hip_layer_norm_gru_forward_f32(int training, int steps, int batch_size
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const int gx = tile.gx, gy = tile.gy;
   const int NB = tile.nb;
-  const size_t part_floats = (size_t)gy * gx * NB * 2;
+  // the tagged row exchange: [groups][2] buffers of 8-byte words, counted in floats
+  const size_t part_floats = (size_t)gy * 2 * tagged_row_words(gx, NB, 2) * 2;
 
   HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 3 * H, C, x, C, W, 3 * H, act_Wx, 3 * H, false));
   HASTE_HIP_PROPAGATE(layer_norm_forward(stream, T * N, 3 * H, gamma1, nullptr, act_Wx, tmp_Wx_norm, cache1));
 
   // Taken after the GEMM, which may replace the stream's scratch buffer with a larger one.
   Workspace ws;
-  const size_t xh_floats = exchange_floats(H, NB, gy);
+  const size_t xh_floats = exchange_floats(H, NB, gy, kPolledTiles);
   HASTE_HIP_PROPAGATE(get_workspace(stream, (part_floats + xh_floats) * sizeof(float), &ws));
   HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 
@@ -465,7 +553,7 @@ int haste_hip_layer_norm_gru_forward_f32(int training, int steps, int batch_size
   p.R = R; p.bx = bx; p.br = br; p.h = h; p.v = v; p.Wxn = tmp_Wx_norm; p.act_Rh = act_Rh;
   p.gamma2 = gamma2; p.cache2 = cache2;
   p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
-  p.part2 = ws.scratch;
+  p.part2 = reinterpret_cast<unsigned long long*>(ws.scratch);
   p.xh = ws.scratch + part_floats;
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes, 2u * (unsigned)T + 1, &plan));
@@ -506,9 +594,10 @@ int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_s
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const int gx = tile.gx, gy = tile.gy;
   const int NB = tile.nb;
-  const size_t part_floats = (size_t)gy * gx * NB * 4;
+  // the tagged row exchange: [groups][2] buffers of 8-byte words, counted in floats
+  const size_t part_floats = (size_t)gy * 2 * tagged_row_words(gx, NB, 3) * 2;
   const size_t col_floats = ((size_t)gy * 9 * H + 3) / 4 * 4;
-  const size_t xdq_floats = exchange_floats(ln_gru_backward_k(H), NB, gy);
+  const size_t xdq_floats = exchange_floats(ln_gru_backward_k(H), NB, gy, kPolledTiles);
 
   Workspace ws;
   HASTE_HIP_PROPAGATE(get_workspace(stream, (part_floats + col_floats + xdq_floats) * sizeof(float), &ws));
@@ -520,7 +609,8 @@ int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_s
   p.dbx = dbx; p.dbr = dbr; p.dh = dh; p.dp = dp; p.dq = dq;
   p.act_Rh = act_Rh; p.gamma2 = gamma2; p.dgamma2 = dgamma2; p.cache2 = cache2;
   p.zoneout_mask = zoneout_mask;
-  p.part = ws.scratch; p.col_partial = ws.scratch + part_floats;
+  p.part = reinterpret_cast<unsigned long long*>(ws.scratch);
+  p.col_partial = ws.scratch + part_floats;
   p.xdq = ws.scratch + part_floats + col_floats;
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes, 2u * (unsigned)T + 1, &plan));

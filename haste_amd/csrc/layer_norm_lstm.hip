@@ -32,9 +32,9 @@ struct LnLstmFwdParams {
   float* act_c_norm;      // [T,N,H] out
   float zoneout_prob;
   const float* zoneout_mask;
-  float* part2;           // exchange [groups][gx][NB][2]
-  float* part3;           // exchange [groups][gx][NB][2]
-  float* xh;              // exchange tiles of h: [batch tiles][2][Kpad/4][NB][4]
+  unsigned long long* part2;  // tagged row exchange [groups][2][gx][NB][2] words: moments of h*R
+  unsigned long long* part3;  // tagged row exchange [groups][2][gx][NB][2] words: moments of c
+  float* xh;              // polled exchange tiles of h: [batch tiles][4][Kpad/4][NB][4]
   LaunchShape ls;
 };
 
@@ -54,7 +54,8 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
   const int Kpad = round_up(H, 64);
   float* w_lds = lds;
   float* red = lds + Kpad * NCOLS;
-  float* stat = red + ProductTile<NB, CT>::kRedFloats;  // [NB][2]
+  float* stat2 = red + ProductTile<NB, CT>::kRedFloats;  // [NB][2] statistics of h*R
+  float* stat3 = stat2 + 2 * NB;                          // [NB][2] statistics of c
 
   const int tid = threadIdx.x;
   const int gx = p.ls.gx;
@@ -64,18 +65,23 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
   const size_t NH = (size_t)N * H;
   const int own_units = (H - j0) < HS ? (H - j0) : HS;     // valid hidden units here
   const int last_units = H - (gx - 1) * HS;                 // ... in the last workgroup
-  float* part2 = p.part2 + (size_t)role.bt * gx * NB * 2;
-  float* part3 = p.part3 + (size_t)role.bt * gx * NB * 2;
+  const size_t row_words = tagged_row_words(gx, NB, 2);
+  unsigned long long* part2 = p.part2 + (size_t)role.bt * 2 * row_words;
+  unsigned long long* part3 = p.part3 + (size_t)role.bt * 2 * row_words;
 
   const int tile_floats = Kpad * NB;
-  float* xh = p.xh + (size_t)role.bt * 2 * tile_floats;
-  const TileBuffer xhb = make_tile_buffer(xh, 2 * tile_floats);
+  float* xh = p.xh + (size_t)role.bt * kPolledTiles * tile_floats;
+  const TileBuffer xhb = make_tile_buffer(xh, kPolledTiles * tile_floats);
 
   GroupSync gs;
   group_sync_init(gs, p.ls, role);
 
-  // Own k range of the exchange tiles (the last workgroup also owns the padding).
-  zero_tile_share(gs, xh, tile_floats, NB, j0 / 4, (role.cw == gx - 1 ? Kpad - j0 : HS) / 4);
+  // Own k range of the exchange tiles (the last workgroup also owns the padding): rows and
+  // k beyond the problem stay zero for the whole launch.
+  zero_tile_share(gs, xh, tile_floats, NB, j0 / 4, (role.cw == gx - 1 ? Kpad - j0 : HS) / 4,
+                  kPolledTiles);
+  clear_row_words(gs, part2, gx, role.cw, NB, 2);
+  clear_row_words(gs, part3, gx, role.cw, NB, 2);
 
   {
     const bool fast = H % 4 == 0 && (reinterpret_cast<uintptr_t>(p.R) & 15u) == 0;
@@ -115,28 +121,50 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
     }
   }
   const bool zoneout = p.zoneout_prob != 0.f && p.zoneout_mask != nullptr;
+  // Tile 0 receives h[0]; the elements of the other tiles that steps will publish start out
+  // unwritten.  One real barrier: nobody polls before every owner has set its share up.
 #pragma unroll
   for (int pp = 0; pp < PP; ++pp)
-    if (act[pp]) store_exchanged(gs, &xh[xchg_index(pj[pp], pl[pp], NB)], h_prev[pp]);
-  group_arrive(gs);  // h[0] is published; the slice is complete in LDS
+    if (act[pp]) {
+      float* e = &xh[xchg_index(pj[pp], pl[pp], NB)];
+      store_exchanged(gs, e, publishable(h_prev[pp]));
+      for (int b = 1; b < kPolledTiles; ++b) store_exchanged(gs, e + (size_t)b * tile_floats, unwritten_value());
+    }
+  group_arrive(gs);  // also: the slice is complete in LDS
+  group_wait(gs);
+
+  // Inputs of a step that do not depend on the recurrence, fetched one step ahead.
+  float wx_next[PP][4], mk_next[PP];
+  auto fetch = [&](int t) {
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      mk_next[pp] = 1.f;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) wx_next[pp][g] = 0.f;
+      if (act[pp] && t < T) {
+        const float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) wx_next[pp][g] = vt[g * H];
+        if (zoneout && p.training) mk_next[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
+      }
+    }
+  };
+  fetch(0);
 
   for (int t = 0; t < T; ++t) {
     float wx[PP][4], mk[PP];
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
-      mk[pp] = 1.f;
+      mk[pp] = mk_next[pp];
 #pragma unroll
-      for (int g = 0; g < 4; ++g) wx[pp][g] = 0.f;
-      if (act[pp]) {
-        const float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
-#pragma unroll
-        for (int g = 0; g < 4; ++g) wx[pp][g] = vt[g * H];
-        if (zoneout && p.training) mk[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
-      }
+      for (int g = 0; g < 4; ++g) wx[pp][g] = wx_next[pp][g];
     }
-    group_wait(gs);  // h[t]
+    const unsigned int tag = gs.epoch + 2u + (unsigned int)t;  // names this step's row exchanges
+    unsigned long long* ex2 = part2 + (size_t)(t & 1) * row_words;
+    unsigned long long* ex3 = part3 + (size_t)(t & 1) * row_words;
 
-    tile_product<NB, CT, false>(xhb, (t & 1) * tile_floats, Kpad, w_lds, red);
+    // The operand loads wait for h[t] themselves (polled tile t % 4).
+    tile_product<NB, CT, false, true>(xhb, (t & 3) * tile_floats, Kpad, w_lds, red, &gs);
     __syncthreads();
 
     // h*R of the owned columns; moments of those columns per row, published.
@@ -149,11 +177,6 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
         rh[pp][g] = colok[pp] ? sum_product<NB, CT>(red, pl[pp], g * HS + pc[pp]) : 0.f;
         s += rh[pp][g];
       }
-      if (act[pp]) {
-        float* ar = p.act_Rh + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
-#pragma unroll
-        for (int g = 0; g < 4; ++g) ar[g * H] = rh[pp][g];
-      }
       const float cnt = 4.0f * (float)own_units;
       const float mean = segment_sum<HS>(s) / cnt;
       float q = 0.f;
@@ -163,81 +186,108 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
         q += colok[pp] ? d * d : 0.f;
       }
       q = segment_sum<HS>(q);
-      if (pc[pp] == 0 && tid + 256 * pp < NB * HS)
-        store_exchanged2(gs, part2 + ((size_t)role.cw * NB + pl[pp]) * 2, mean, q);
+      if (pc[pp] == 0 && tid + 256 * pp < NB * HS) {
+        const float mq[2] = {mean, q};
+        publish_row<2>(gs, ex2, NB, role.cw, pl[pp], mq, tag);
+      }
     }
-    group_arrive(gs);
-    group_wait(gs);  // every workgroup's moments of h*R
-    merge_row_moments<NB>(part2, gx, 4.0f * HS, 4.0f * last_units, 4.0f * H, stat);
+    merge_row_moments_polled<NB>(gs, ex2, gx, tag, 4.0f * HS, 4.0f * last_units, 4.0f * H, stat2);
     __syncthreads();
 
-    float go[PP], c_new[PP];
+    float gate[PP][4], c_new[PP], mu2[PP], is2[PP];
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
-      const float mu = stat[pl[pp] * 2], is = stat[pl[pp] * 2 + 1];
-      go[pp] = 0.f;
+      mu2[pp] = stat2[pl[pp] * 2];
+      is2[pp] = stat2[pl[pp] * 2 + 1];
       c_new[pp] = 0.f;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) gate[pp][g] = 0.f;
       if (act[pp]) {
         float a[4];
 #pragma unroll
         for (int g = 0; g < 4; ++g)
-          a[g] = wx[pp][g] + (rh[pp][g] - mu) * is * g2[pp][g] + bias[pp][g];
-        const float gi = sigmoid_f(a[0]);
-        const float gg = tanh_f(a[1]);
-        const float gf = sigmoid_f(a[2]);
-        go[pp] = sigmoid_f(a[3]);
-        if (p.training) {
-          float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
-          vt[0] = gi;
-          vt[H] = gg;
-          vt[2 * H] = gf;
-          vt[3 * H] = go[pp];
-        }
-        c_new[pp] = gf * c_prev[pp] + gi * gg;
-        p.c[(size_t)(t + 1) * NH + (size_t)pn[pp] * H + pj[pp]] = c_new[pp];
+          a[g] = wx[pp][g] + (rh[pp][g] - mu2[pp]) * is2[pp] * g2[pp][g] + bias[pp][g];
+        gate[pp][0] = sigmoid_f(a[0]);
+        gate[pp][1] = tanh_f(a[1]);
+        gate[pp][2] = sigmoid_f(a[2]);
+        gate[pp][3] = sigmoid_f(a[3]);
+        c_new[pp] = gate[pp][2] * c_prev[pp] + gate[pp][0] * gate[pp][1];
         c_prev[pp] = c_new[pp];
-        if (role.cw == 0 && pc[pp] == 0 && p.cache2 != nullptr) {
-          p.cache2[((size_t)t * N + pn[pp]) * 2 + 0] = mu;
-          p.cache2[((size_t)t * N + pn[pp]) * 2 + 1] = is;
-        }
       }
       // moments of the new cell state over the owned hidden units
       const float cv = colok[pp] ? c_new[pp] : 0.f;
       const float mean = segment_sum<HS>(cv) / (float)own_units;
       const float d = cv - mean;
       const float q = segment_sum<HS>(colok[pp] ? d * d : 0.f);
-      if (pc[pp] == 0 && tid + 256 * pp < NB * HS)
-        store_exchanged2(gs, part3 + ((size_t)role.cw * NB + pl[pp]) * 2, mean, q);
+      if (pc[pp] == 0 && tid + 256 * pp < NB * HS) {
+        const float mq[2] = {mean, q};
+        publish_row<2>(gs, ex3, NB, role.cw, pl[pp], mq, tag);
+      }
     }
-    group_arrive(gs);
-    group_wait(gs);  // every workgroup's moments of c
-    merge_row_moments<NB>(part3, gx, (float)HS, (float)last_units, (float)H, stat);
+    merge_row_moments_polled<NB>(gs, ex3, gx, tag, (float)HS, (float)last_units, (float)H, stat3);
     __syncthreads();
 
+    float cn[PP], mu3[PP], is3[PP], h_pub[PP];
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
+      mu3[pp] = stat3[pl[pp] * 2];
+      is3[pp] = stat3[pl[pp] * 2 + 1];
+      cn[pp] = 0.f;
       if (act[pp]) {
-        const float mu = stat[pl[pp] * 2], is = stat[pl[pp] * 2 + 1];
-        const float cn = (c_new[pp] - mu) * is * gh[pp] + bh[pp];
-        const size_t e = (size_t)pn[pp] * H + pj[pp];
-        p.act_c_norm[(size_t)t * NH + e] = cn;
-        float h_new = go[pp] * tanh_f(cn);
+        cn[pp] = (c_new[pp] - mu3[pp]) * is3[pp] * gh[pp] + bh[pp];
+        float h_new = gate[pp][3] * tanh_f(cn[pp]);
         if (zoneout) {
           if (p.training) h_new = (h_new - h_prev[pp]) * mk[pp] + h_prev[pp];
           else h_new = p.zoneout_prob * h_prev[pp] + (1.0f - p.zoneout_prob) * h_new;
         }
-        p.h[(size_t)(t + 1) * NH + e] = h_new;
-        if (t + 1 < T)
-          store_exchanged(gs, &xh[((t + 1) & 1) * tile_floats + xchg_index(pj[pp], pl[pp], NB)], h_new);
         h_prev[pp] = h_new;
-        if (role.cw == 0 && pc[pp] == 0 && p.cache3 != nullptr) {
-          p.cache3[((size_t)t * N + pn[pp]) * 2 + 0] = mu;
-          p.cache3[((size_t)t * N + pn[pp]) * 2 + 1] = is;
+      }
+      h_pub[pp] = publishable(h_prev[pp]);
+    }
+    // Everything this wavefront stored during the previous step (its resets among it) has
+    // landed before h[t+1] becomes visible.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (t + 1 < T) {
+      float* xh_next = xh + ((t + 1) & 3) * tile_floats;
+      float* xh_done = xh + ((t + 3) & 3) * tile_floats;  // read at step t-1: nobody needs it any more
+#pragma unroll
+      for (int pp = 0; pp < PP; ++pp)
+        if (act[pp]) {
+          const int e = xchg_index(pj[pp], pl[pp], NB);
+          store_exchanged(gs, &xh_next[e], h_pub[pp]);
+          if (t + 3 < T) store_exchanged(gs, &xh_done[e], unwritten_value());
+        }
+    }
+    fetch(t + 1);
+    __syncthreads();  // red, stat2 and stat3 may be overwritten by the next step
+    // The caller's copies are written last: nobody in the launch waits for them.
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      if (act[pp]) {
+        const size_t e4 = ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+        const size_t e = (size_t)pn[pp] * H + pj[pp];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) p.act_Rh[e4 + (size_t)g * H] = rh[pp][g];
+        if (p.training) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) p.v[e4 + (size_t)g * H] = gate[pp][g];
+        }
+        p.c[(size_t)(t + 1) * NH + e] = c_new[pp];
+        p.act_c_norm[(size_t)t * NH + e] = cn[pp];
+        p.h[(size_t)(t + 1) * NH + e] = h_prev[pp];
+        if (role.cw == 0 && pc[pp] == 0) {
+          const size_t r = ((size_t)t * N + pn[pp]) * 2;
+          if (p.cache2 != nullptr) {
+            p.cache2[r] = mu2[pp];
+            p.cache2[r + 1] = is2[pp];
+          }
+          if (p.cache3 != nullptr) {
+            p.cache3[r] = mu3[pp];
+            p.cache3[r + 1] = is3[pp];
+          }
         }
       }
     }
-    if (t + 1 < T) group_arrive(gs);  // publishes h[t+1]; also orders reuse of red/stat
-    else __syncthreads();
   }
 }
 
@@ -261,10 +311,10 @@ struct LnLstmBwdParams {
   const float* cache3;     // [T*N,2]
   const float* act_c_norm; // [T,N,H]
   const float* zoneout_mask;
-  float* part_a;           // exchange [groups][gx][NB][4]
-  float* part_b;           // exchange [groups][gx][NB][4]
+  unsigned long long* part_a;  // tagged row exchange [groups][2][gx][NB][3] words: cell-state norm sums
+  unsigned long long* part_b;  // tagged row exchange [groups][2][gx][NB][3] words: h*R norm sums
   float* col_partial;      // [batch tiles][10][H]
-  float* xd;               // exchange tiles of the gradient w.r.t. h*R: [batch tiles][2][Kpad/4][NB][4]
+  float* xd;               // polled exchange tiles of the gradient w.r.t. h*R: [batch tiles][4][Kpad/4][NB][4]
   LaunchShape ls;
 };
 
@@ -287,7 +337,8 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   const int Kpad = 64 * p.ls.gx;  // k = 4*unit + gate over the 16 units of every workgroup
   float* w_lds = lds;
   float* red = lds + Kpad * NCOLS;  // the partial tiles, reused for the column sums
-  float* sums = red + RED;           // [NB][4]
+  float* sums_a = red + RED;         // [NB][4] row sums of the cell-state norm
+  float* sums_b = sums_a + 4 * NB;   // [NB][4] row sums of the h*R norm
 
   const int tid = threadIdx.x;
   const int gx = p.ls.gx;
@@ -295,15 +346,18 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   const int n0 = role.bt * p.ls.tile_rows;
   const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
-  float* part_a = p.part_a + (size_t)role.bt * gx * NB * 4;
-  float* part_b = p.part_b + (size_t)role.bt * gx * NB * 4;
+  const size_t row_words = tagged_row_words(gx, NB, 3);
+  unsigned long long* part_a = p.part_a + (size_t)role.bt * 2 * row_words;
+  unsigned long long* part_b = p.part_b + (size_t)role.bt * 2 * row_words;
 
   const int tile_floats = Kpad * NB;
-  float* xd = p.xd + (size_t)role.bt * 2 * tile_floats;
-  const TileBuffer xdb = make_tile_buffer(xd, 2 * tile_floats);
+  float* xd = p.xd + (size_t)role.bt * kPolledTiles * tile_floats;
+  const TileBuffer xdb = make_tile_buffer(xd, kPolledTiles * tile_floats);
 
   GroupSync gs;
   group_sync_init(gs, p.ls, role);
+  clear_row_words(gs, part_a, gx, role.cw, NB, 3);
+  clear_row_words(gs, part_b, gx, role.cw, NB, 3);
 
   {
     const bool fast = H % 4 == 0 && (reinterpret_cast<uintptr_t>(p.R_t) & 15u) == 0;
@@ -334,7 +388,18 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
     for (int a = 0; a < NACC; ++a) accs[pp][a] = 0.f;
   }
   const bool zoneout = p.zoneout_mask != nullptr;
-  __syncthreads();
+  // Every element of the polled tiles belongs to the thread that publishes it (rows and
+  // units beyond the problem are published as zeros); all start out unwritten.  One real
+  // barrier: nobody polls before every owner has set its share up.
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp)
+    if (own[pp]) {
+      const float u = unwritten_value();
+      for (int b = 0; b < kPolledTiles; ++b)
+        store_exchanged4(gs, xd + (size_t)b * tile_floats + ((size_t)pj[pp] * NB + pl[pp]) * 4, u, u, u, u);
+    }
+  group_arrive(gs);  // also: the slice is complete in LDS
+  group_wait(gs);
 
   struct StepIn { float vt[4], rh[4], c0, c1, dhn, dcn, m, cn, mu2, is2, mu3, is3; };
   StepIn nxt[PP];
@@ -373,6 +438,10 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   for (int t = T - 1; t >= 0; --t) {
     StepIn s[PP];
     float dh_keep[PP], dv_o[PP], xc3[PP], gd3[PP];
+    const int done = T - 1 - t;  // steps done so far
+    const unsigned int tag = gs.epoch + 2u + (unsigned int)done;  // names this step's row exchanges
+    unsigned long long* ex_a = part_a + (size_t)(done & 1) * row_words;
+    unsigned long long* ex_b = part_b + (size_t)(done & 1) * row_words;
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
       s[pp] = nxt[pp];
@@ -396,24 +465,24 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
       const float s0 = segment_sum<HSB>(xc3[pp] * gd3[pp]);
       const float s1 = segment_sum<HSB>(xc3[pp]);
       const float s2 = segment_sum<HSB>(gd3[pp]);
-      if (pc[pp] == 0 && own[pp])
-        store_exchanged4(gs, part_a + ((size_t)role.cw * NB + pl[pp]) * 4, s0, s1, s2, 0.f);
+      if (pc[pp] == 0 && own[pp]) {
+        const float v3[3] = {s0, s1, s2};
+        publish_row<3>(gs, ex_a, NB, role.cw, pl[pp], v3, tag);
+      }
     }
-    group_arrive(gs);
-    group_wait(gs);  // row sums of the cell-state norm
-    sum_row_partials<NB>(part_a, gx, sums);
+    sum_row_partials_polled<NB>(gs, ex_a, gx, tag, sums_a);  // row sums of the cell-state norm
     __syncthreads();
 
-    float xc2[PP][4], gd2[PP][4];
+    float xc2[PP][4], gd2[PP][4], dvs[PP][4];
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
       float t0 = 0.f, t1 = 0.f, t2 = 0.f;
 #pragma unroll
-      for (int g = 0; g < 4; ++g) xc2[pp][g] = gd2[pp][g] = 0.f;
+      for (int g = 0; g < 4; ++g) xc2[pp][g] = gd2[pp][g] = dvs[pp][g] = 0.f;
       if (act[pp]) {
         const float is3 = s[pp].is3;
-        const float dsigma = -0.5f * sums[pl[pp] * 4 + 0] * is3 * is3 * is3;
-        const float dmu = (-2.0f * sums[pl[pp] * 4 + 1] * dsigma * invH) - (sums[pl[pp] * 4 + 2] * is3);
+        const float dsigma = -0.5f * sums_a[pl[pp] * 4 + 0] * is3 * is3 * is3;
+        const float dmu = (-2.0f * sums_a[pl[pp] * 4 + 1] * dsigma * invH) - (sums_a[pl[pp] * 4 + 2] * is3);
         const float dc_ln = (2.0f * xc3[pp] * dsigma * invH) + (is3 * gd3[pp]) + (dmu * invH);
         const float gi = s[pp].vt[0], gg = s[pp].vt[1], gf = s[pp].vt[2];
         const float dc_total = s[pp].dcn + dc[pp] + dc_ln;
@@ -426,10 +495,9 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
         dv[1] = d_tanh_f(gg) * dg;
         dv[2] = d_sigmoid_f(gf) * df;
         dv[3] = dv_o[pp];
-        float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          vt[(size_t)g * H] = dv[g];
+          dvs[pp][g] = dv[g];
           accs[pp][g] += dv[g];
           xc2[pp][g] = s[pp].rh[g] - s[pp].mu2;
           gd2[pp][g] = g2[pp][g] * dv[g];
@@ -442,12 +510,12 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
       t0 = segment_sum<HSB>(t0);
       t1 = segment_sum<HSB>(t1);
       t2 = segment_sum<HSB>(t2);
-      if (pc[pp] == 0 && own[pp])
-        store_exchanged4(gs, part_b + ((size_t)role.cw * NB + pl[pp]) * 4, t0, t1, t2, 0.f);
+      if (pc[pp] == 0 && own[pp]) {
+        const float v3[3] = {t0, t1, t2};
+        publish_row<3>(gs, ex_b, NB, role.cw, pl[pp], v3, tag);
+      }
     }
-    group_arrive(gs);
-    group_wait(gs);  // row sums of the h*R norm
-    sum_row_partials<NB>(part_b, gx, sums);
+    sum_row_partials_polled<NB>(gs, ex_b, gx, tag, sums_b);  // row sums of the h*R norm
     __syncthreads();
 
     float dr[PP][4];
@@ -457,31 +525,47 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
       for (int g = 0; g < 4; ++g) dr[pp][g] = 0.f;
       if (act[pp]) {
         const float is2 = s[pp].is2;
-        const float dsigma = -0.5f * sums[pl[pp] * 4 + 0] * is2 * is2 * is2;
-        const float dmu = (-2.0f * sums[pl[pp] * 4 + 1] * dsigma * inv4H) - (sums[pl[pp] * 4 + 2] * is2);
+        const float dsigma = -0.5f * sums_b[pl[pp] * 4 + 0] * is2 * is2 * is2;
+        const float dmu = (-2.0f * sums_b[pl[pp] * 4 + 1] * dsigma * inv4H) - (sums_b[pl[pp] * 4 + 2] * is2);
 #pragma unroll
         for (int g = 0; g < 4; ++g)
           dr[pp][g] = (2.0f * xc2[pp][g] * dsigma * inv4H) + (is2 * gd2[pp][g]) + (dmu * inv4H);
       }
-      // rows and units beyond the problem are published as zeros
-      if (own[pp])
-        store_exchanged4(gs, xd + (t & 1) * tile_floats + ((size_t)pj[pp] * NB + pl[pp]) * 4,
-                         dr[pp][0], dr[pp][1], dr[pp][2], dr[pp][3]);
     }
-    group_arrive(gs);
-    // The caller's copy is written behind the barrier: nobody in the launch waits for it.
+    // What this wavefront stored during the previous step (its resets among it) has landed
+    // before the gradients of this step become visible.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    {
+      float* xd_t = xd + (done & 3) * tile_floats;
+      float* xd_done = xd + ((done + 2) & 3) * tile_floats;  // read two steps ago
+#pragma unroll
+      for (int pp = 0; pp < PP; ++pp)
+        // rows and units beyond the problem are published as zeros
+        if (own[pp]) {
+          const size_t e = ((size_t)pj[pp] * NB + pl[pp]) * 4;
+          store_exchanged4(gs, xd_t + e, publishable(dr[pp][0]), publishable(dr[pp][1]),
+                           publishable(dr[pp][2]), publishable(dr[pp][3]));
+          if (done + 2 < T) {
+            const float u = unwritten_value();
+            store_exchanged4(gs, xd_done + e, u, u, u, u);
+          }
+        }
+    }
+    // The caller's copies: nobody in the launch waits for them.
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
       if (act[pp]) {
-        float* ar = p.act_Rh + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+        const size_t e4 = ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
 #pragma unroll
-        for (int g = 0; g < 4; ++g) ar[(size_t)g * H] = dr[pp][g];
+        for (int g = 0; g < 4; ++g) {
+          p.v[e4 + (size_t)g * H] = dvs[pp][g];
+          p.act_Rh[e4 + (size_t)g * H] = dr[pp][g];
+        }
       }
     }
     fetch(t - 1);
-    group_wait(gs);  // gradient w.r.t. h*R complete for this batch tile
-
-    tile_product<NB, 1, true>(xdb, (t & 1) * tile_floats, Kpad, w_lds, red);
+    // The operand loads wait for the gradient w.r.t. h*R of every unit themselves.
+    tile_product<NB, 1, true, true>(xdb, (done & 3) * tile_floats, Kpad, w_lds, red, &gs);
     __syncthreads();
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp)
@@ -547,18 +631,19 @@ int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_siz
   HASTE_HIP_REQUIRE(W && R && b && x && h && c && act_Wx && gamma1 && act_Wx_norm && act_Rh);
   HASTE_HIP_REQUIRE(gamma2 && gamma_h && beta_h && act_c_norm);
   hipStream_t stream = as_stream(stream_);
-  const ForwardTile tile = pick_forward_tile(4, N, H, 2 * sizeof(float));
+  const ForwardTile tile = pick_forward_tile(4, N, H, 4 * sizeof(float));
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const int gx = tile.gx, gy = tile.gy;
   const int NB = tile.nb;
-  const size_t part_floats = (size_t)gy * gx * NB * 2;
+  // one tagged row exchange: [groups][2] buffers of 8-byte words, counted in floats
+  const size_t part_floats = (size_t)gy * 2 * tagged_row_words(gx, NB, 2) * 2;
 
   HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 4 * H, C, x, C, W, 4 * H, act_Wx, 4 * H, false));
   HASTE_HIP_PROPAGATE(layer_norm_forward(stream, T * N, 4 * H, gamma1, nullptr, act_Wx, act_Wx_norm, cache1));
 
   // Taken after the GEMM, which may replace the stream's scratch buffer with a larger one.
   Workspace ws;
-  const size_t xh_floats = exchange_floats(H, NB, gy);
+  const size_t xh_floats = exchange_floats(H, NB, gy, kPolledTiles);
   HASTE_HIP_PROPAGATE(get_workspace(stream, (2 * part_floats + xh_floats) * sizeof(float), &ws));
   HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 
@@ -567,7 +652,8 @@ int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_siz
   p.R = R; p.b = b; p.h = h; p.c = c; p.v = act_Wx_norm; p.act_Rh = act_Rh;
   p.gamma2 = gamma2; p.cache2 = cache2; p.gamma_h = gamma_h; p.beta_h = beta_h; p.cache3 = cache3;
   p.act_c_norm = act_c_norm; p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
-  p.part2 = ws.scratch; p.part3 = ws.scratch + part_floats;
+  p.part2 = reinterpret_cast<unsigned long long*>(ws.scratch);
+  p.part3 = reinterpret_cast<unsigned long long*>(ws.scratch + part_floats);
   p.xh = ws.scratch + 2 * part_floats;
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes, 3u * (unsigned)T + 1, &plan));
@@ -611,16 +697,17 @@ int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_
   HASTE_HIP_REQUIRE(dgamma_h && dbeta_h && cache3 && act_c_norm);
   hipStream_t stream = as_stream(stream_);
   // per row: 10 column-sum accumulators of 16 floats (or the partial tiles, whichever is more) + 4 sums
-  const BackwardTile tile = pick_backward_tile(4 * H, N, H, 10 * 16, 4);
+  const BackwardTile tile = pick_backward_tile(4 * H, N, H, 10 * 16, 8);
   if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const int gx = tile.gx, gy = tile.gy;
   const int NB = tile.nb;
-  const size_t part_floats = (size_t)gy * gx * NB * 4;
+  // one tagged row exchange: [groups][2] buffers of 8-byte words, counted in floats
+  const size_t part_floats = (size_t)gy * 2 * tagged_row_words(gx, NB, 3) * 2;
   const size_t col_floats = (size_t)gy * 10 * H;
   const size_t col_floats4 = (col_floats + 3) / 4 * 4;
 
   Workspace ws;
-  const size_t xd_floats = exchange_floats(64 * gx, NB, gy);
+  const size_t xd_floats = exchange_floats(64 * gx, NB, gy, kPolledTiles);
   HASTE_HIP_PROPAGATE(get_workspace(stream, (2 * part_floats + col_floats4 + xd_floats) * sizeof(float), &ws));
   HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 
@@ -631,7 +718,8 @@ int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_
   p.gamma2 = gamma2; p.dgamma2 = dgamma2; p.cache2 = cache2;
   p.gamma_h = gamma_h; p.dgamma_h = dgamma_h; p.dbeta_h = dbeta_h; p.cache3 = cache3;
   p.act_c_norm = act_c_norm; p.zoneout_mask = zoneout_mask;
-  p.part_a = ws.scratch; p.part_b = ws.scratch + part_floats;
+  p.part_a = reinterpret_cast<unsigned long long*>(ws.scratch);
+  p.part_b = reinterpret_cast<unsigned long long*>(ws.scratch + part_floats);
   p.col_partial = ws.scratch + 2 * part_floats;
   p.xd = ws.scratch + 2 * part_floats + col_floats4;
   LaunchPlan plan;

@@ -18,12 +18,36 @@ namespace haste_hip {
 
 constexpr float kLnEps = 1e-5f;
 
-// Sum over the W consecutive lanes (W a power of two, segment aligned to W).
+// Cross-lane moves inside a row of 16 lanes on the data-parallel-primitive path of the
+// VALU (a few cycles; a shuffle through the LDS crossbar costs over a hundred).
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+
+// Sum over the W consecutive lanes (W a power of two up to 16, segment aligned to W); every
+// lane of the segment receives it.  Pairs are formed by quad permutes (lane^1, lane^2), then
+// by mirroring the half row and the row: once the lanes of a quad (half row) agree, lane i and
+// lane 7-i (15-i) hold the sums of the two halves.
 template <int W>
 __device__ __forceinline__ float segment_sum(float v) {
-#pragma unroll
-  for (int off = W / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  static_assert(W == 1 || W == 2 || W == 4 || W == 8 || W == 16, "segment within a row of 16 lanes");
+  if (W >= 2) v += dpp_move<0xB1>(v);    // quad_perm [1,0,3,2]
+  if (W >= 4) v += dpp_move<0x4E>(v);    // quad_perm [2,3,0,1]
+  if (W >= 8) v += dpp_move<0x141>(v);   // row_half_mirror
+  if (W >= 16) v += dpp_move<0x140>(v);  // row_mirror
   return v;
+}
+
+// Sum over all 64 lanes, the same value in every lane: rows of 16 as above, then the four
+// row sums in lane order.
+__device__ __forceinline__ float wave_sum(float v) {
+  v = segment_sum<16>(v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0)) +
+         __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16)) +
+         __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32)) +
+         __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
 }
 
 __device__ __forceinline__ void load_exchanged2(const float* p, float& a, float& b) {
@@ -76,6 +100,162 @@ __device__ __forceinline__ void merge_row_moments(const float* part, int gx, flo
     if (lane == 0) {
       out[row * 2 + 0] = acc.mean;
       out[row * 2 + 1] = 1.0f / sqrtf(acc.m2 / D + kLnEps);
+    }
+  }
+}
+
+// ---- tagged row exchange ---------------------------------------------------------------
+// The same exchanges without a step barrier.  Every float travels in an 8-byte word next to
+// a 32-bit tag that names the use (launch epoch + running count), so a reader knows from the
+// word itself whether it has been published: it re-issues its loads until every tag matches.
+// Two buffers alternate by use parity: a workgroup publishes use u+2 only after it has read
+// every contribution to use u+1, and those were published after their authors had read use u,
+// so nobody can still be reading the words that use u+2 overwrites.  Layout of one buffer:
+// [gx][NB] slots of WS = 2 or 4 words (W values, padded to a 16-byte multiple so that a slot
+// is written and read with 16-byte accesses); a workgroup's slots share lines with nobody.
+template <int W> struct RowSlot { static constexpr int kWords = W <= 2 ? 2 : 4; };
+
+__host__ __device__ __forceinline__ size_t tagged_row_words(int gx, int nb, int w) {
+  return (size_t)gx * nb * (w <= 2 ? 2 : 4);
+}
+
+typedef unsigned int uint4_row_t __attribute__((ext_vector_type(4)));
+
+template <int W>
+__device__ __forceinline__ void publish_row(const GroupSync& g, unsigned long long* buffer, int nb,
+                                            int cw, int row, const float (&v)[W], unsigned int tag) {
+  constexpr int WS = RowSlot<W>::kWords;
+  unsigned long long* q = buffer + ((size_t)cw * nb + row) * WS;
+#pragma unroll
+  for (int i = 0; i < WS; i += 2) {
+    uint4_row_t u;
+    u.x = __float_as_uint(v[i]);
+    u.y = tag;
+    u.z = i + 1 < W ? __float_as_uint(v[i + 1 < W ? i + 1 : i]) : 0u;
+    u.w = tag;
+    if (g.same_xcd) {
+      *reinterpret_cast<volatile uint4_row_t*>(q + i) = u;
+    } else {
+      __hip_atomic_store(q + i, (unsigned long long)u.x | ((unsigned long long)u.y << 32),
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(q + i + 1, (unsigned long long)u.z | ((unsigned long long)u.w << 32),
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+// Zeroes this workgroup's slots of both buffers (a tag of zero is never expected); called
+// before the launch's initial barrier.
+__device__ __forceinline__ void clear_row_words(const GroupSync& g, unsigned long long* both, int gx,
+                                                int cw, int nb, int w) {
+  const int ws = w <= 2 ? 2 : 4;
+  for (int i = threadIdx.x; i < 2 * nb * ws; i += 256) {
+    unsigned long long* q = both + (size_t)(i / (nb * ws)) * tagged_row_words(gx, nb, w) +
+                            (size_t)cw * nb * ws + i % (nb * ws);
+    if (g.same_xcd) *reinterpret_cast<volatile unsigned long long*>(q) = 0ull;
+    else __hip_atomic_store(q, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+// Loads the slot of (cw, row) until all of its words carry `tag` (`have` false: nothing to
+// load).  `slots` is a buffer resource over the buffer (16-byte agent-scope loads, never
+// served by this CU's L1).  The whole wavefront polls together, backing off briefly between
+// attempts (all workgroups of the group poll the same few lines); bounded like every wait of
+// the launch.
+template <int W>
+__device__ __forceinline__ void load_row_polled(const GroupSync& g, const TileBuffer& slots, int nb,
+                                                int cw, int row, bool have, unsigned int tag,
+                                                float (&v)[W]) {
+  constexpr int WS = RowSlot<W>::kWords;
+  const int word = ((have ? cw : 0) * nb + row) * WS;
+  bool ok = !have;
+  auto load = [&] {
+    bool all = true;
+#pragma unroll
+    for (int i = 0; i < WS; i += 2) {
+      const uint4_t u = __builtin_amdgcn_raw_buffer_load_b128(slots.rsrc, (word + i) * 8, 0, 16);
+      v[i] = __uint_as_float(u.x);
+      if (i + 1 < W) v[i + 1 < W ? i + 1 : i] = __uint_as_float(u.z);
+      all = all && u.y == tag && u.w == tag;
+    }
+    ok = !have || all;
+  };
+  if (have) load();
+    poll_until_written(g, [&] { __builtin_amdgcn_s_sleep(1); load(); }, [&] { return __all(ok) != 0; });
+}
+
+// Row statistics from a tagged buffer ([gx][NB][2] words holding each workgroup's (mean, m2)
+// of its `full_count` columns, `last_count` for the last one): the merged mean is the weighted
+// mean of the means, the merged m2 the sum of m2_i + n_i (mean_i - mean)^2 -- the pairwise
+// update of merge_moments written out for all parts at once, as two plain sums.  Writes
+// (mean, 1/sqrt(var + eps)) of the whole row (D columns) to out[row*2 .. +1] in LDS; the
+// caller synchronises the workgroup before reading `out`.  Called by all 256 threads.
+template <int NB>
+__device__ __forceinline__ void merge_row_moments_polled(const GroupSync& g,
+                                                         unsigned long long* buffer, int gx,
+                                                         unsigned int tag, float full_count,
+                                                         float last_count, float D, float* out) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const TileBuffer slots = make_tile_buffer(reinterpret_cast<float*>(buffer),
+                                            (int)tagged_row_words(gx, NB, 2) * 2);
+  for (int row = wave; row < NB; row += 4) {
+    float first[2] = {0.f, 0.f};
+    float s1 = 0.f;
+    for (int c0 = 0; c0 < gx; c0 += 64) {
+      const int cw = c0 + lane;
+      float v[2];
+      load_row_polled<2>(g, slots, NB, cw, row, cw < gx, tag, v);
+      if (cw < gx) s1 += ((cw == gx - 1) ? last_count : full_count) * v[0];
+      if (c0 == 0) { first[0] = v[0]; first[1] = v[1]; }
+    }
+    const float mean = wave_sum(s1) / D;
+    float s2 = 0.f;
+    for (int c0 = 0; c0 < gx; c0 += 64) {
+      const int cw = c0 + lane;
+      float v[2] = {first[0], first[1]};
+      if (c0 != 0) load_row_polled<2>(g, slots, NB, cw, row, cw < gx, tag, v);  // seen before
+      if (cw < gx) {
+        const float d = v[0] - mean;
+        s2 += v[1] + ((cw == gx - 1) ? last_count : full_count) * d * d;
+      }
+    }
+    const float m2 = wave_sum(s2);
+    if (lane == 0) {
+      out[row * 2 + 0] = mean;
+      out[row * 2 + 1] = 1.0f / sqrtf(m2 / D + kLnEps);
+    }
+  }
+}
+
+// sum_row_partials over a tagged buffer (slots holding (s0, s1, s2)).
+template <int NB>
+__device__ __forceinline__ void sum_row_partials_polled(const GroupSync& g,
+                                                        unsigned long long* buffer, int gx,
+                                                        unsigned int tag, float* out) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const TileBuffer slots = make_tile_buffer(reinterpret_cast<float*>(buffer),
+                                            (int)tagged_row_words(gx, NB, 3) * 2);
+  for (int row = wave; row < NB; row += 4) {
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f;
+    for (int c0 = 0; c0 < gx; c0 += 64) {
+      const int cw = c0 + lane;
+      float v[3];
+      load_row_polled<3>(g, slots, NB, cw, row, cw < gx, tag, v);
+      if (cw < gx) {
+        s0 += v[0];
+        s1 += v[1];
+        s2 += v[2];
+      }
+    }
+    s0 = wave_sum(s0);
+    s1 = wave_sum(s1);
+    s2 = wave_sum(s2);
+    if (lane == 0) {
+      out[row * 4 + 0] = s0;
+      out[row * 4 + 1] = s1;
+      out[row * 4 + 2] = s2;
     }
   }
 }
