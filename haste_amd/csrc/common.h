@@ -90,10 +90,39 @@ int order_persistent_launches(hipStream_t stream, bool before);
 // cross-XCD exchange path; for experiments).
 bool xcd_local_enabled();
 
-// C[M,N] = op(A)*B (+C): fp32 MFMA GEMM on `stream`. `ws` supplies split-K scratch.
+// C[M,N] = op(A)*B (+C): fp32 MFMA GEMM on `stream`.  The partial tiles of a split product
+// are kept `scratch_offset` bytes (a multiple of 16) into the stream's scratch buffer.
 int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
              const float* A, int lda, const float* B, int ldb,
-             float* C, int ldc, bool accumulate);
+             float* C, int ldc, bool accumulate, size_t scratch_offset = 0);
+
+// Bytes of scratch gemm_f32 uses for this shape (0 when nothing is split).
+size_t gemm_f32_scratch_bytes(int M, int N, int K);
+
+// LSTM / GRU with the recurrent matrix streamed from HBM every step (per-step GEMM +
+// pointwise kernel): for hidden sizes whose slices of R do not fit on chip.  Arguments as
+// the persistent implementations in lstm.hip / gru.hip.
+int lstm_forward_streamed(hipStream_t stream, int training, int T, int N, int C, int H,
+                          const float* W, const float* R, const float* b, const float* x,
+                          const float* h, const float* c, float* h_out, float* c_out, float* v,
+                          float zoneout_prob, const float* zoneout_mask, const float* dc_mask,
+                          float dc_scale);
+int lstm_backward_streamed(hipStream_t stream, int T, int N, int C, int H,
+                           const float* W_t, const float* R_t, const float* x_t,
+                           const float* h, const float* c, const float* c_next,
+                           const float* dh_next, const float* dc_next,
+                           float* dx, float* dW, float* dR, float* db, float* dh, float* dc, float* v,
+                           const float* zoneout_mask);
+int gru_forward_streamed(hipStream_t stream, int training, int T, int N, int C, int H,
+                         const float* W, const float* R, const float* bx, const float* br,
+                         const float* x, const float* h, float* h_out, float* v, float* tmp_Wx,
+                         float zoneout_prob, const float* zoneout_mask, const float* dc_mask,
+                         float dc_scale);
+int gru_backward_streamed(hipStream_t stream, int T, int N, int C, int H,
+                          const float* W_t, const float* R_t, const float* x_t, const float* h,
+                          const float* v, const float* dh_next, float* dx, float* dW, float* dR,
+                          float* dbx, float* dbr, float* dh, float* dp, float* dq,
+                          const float* zoneout_mask);
 
 // Row-wise layer norm kernels (rows x dim), used stand-alone and by the LN cells.
 int layer_norm_forward(hipStream_t stream, int rows, int dim, const float* gamma,

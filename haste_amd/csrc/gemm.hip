@@ -300,22 +300,21 @@ void split_reduce_kernel(int M, int N, int splits, int tiles_n, int whole_tiles,
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-}  // namespace
+// How a product is cut into workgroups (depends on the shape only).
+struct GemmPlan {
+  int bm, tiles_n, whole_tiles, rest, splits, k_per_split, pieces;
+  size_t scratch_bytes;
+};
 
-int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
-             const float* A, int lda, const float* B, int ldb,
-             float* C, int ldc, bool accumulate) {
-  HASTE_HIP_REQUIRE(M > 0 && N > 0 && K > 0);
-  HASTE_HIP_REQUIRE(A != nullptr && B != nullptr && C != nullptr);
-  HASTE_HIP_REQUIRE(lda >= (trans_a ? M : K) && ldb >= N && ldc >= N);
-  const int tiles_n = (N + BN - 1) / BN;
+GemmPlan plan_gemm(int M, int N, int K) {
+  GemmPlan g;
+  g.tiles_n = (N + BN - 1) / BN;
   const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
 
   // Tile height: 64 rows only when the output has no more than that.
-  const int bm = M <= 64 ? 64 : 128;
-  const int tiles_m = (M + bm - 1) / bm;
-  const long long tiles = (long long)tiles_m * tiles_n;
-  HASTE_HIP_REQUIRE(tiles < (1ll << 26));
+  g.bm = M <= 64 ? 64 : 128;
+  const int tiles_m = (M + g.bm - 1) / g.bm;
+  const long long tiles = (long long)tiles_m * g.tiles_n;
 
   // Whole rounds of one tile per CU run unsplit; the `rest` tiles of the last round are each
   // cut into `splits` K pieces.  In units of the time one CU needs for one whole tile, s
@@ -326,37 +325,60 @@ int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
   // The cheapest s is taken, a piece keeping at least 64 of K.  The choice depends on the
   // shape only, so results are reproducible.
   const long long whole = tiles >= cus ? tiles / cus * cus : 0;
-  const int rest = (int)(tiles - whole);
+  g.rest = (int)(tiles - whole);
   int splits = 1;
-  if (rest > 0) {
+  if (g.rest > 0) {
     const int k_iters = (K + BK - 1) / BK;
     int s_max = k_iters / 4;
     if (s_max > 64) s_max = 64;
     auto cost = [&](int s) {
-      const long long pieces = (long long)rest * s;
+      const long long pieces = (long long)g.rest * s;
       double c = (double)((pieces + cus - 1) / cus) / s;
       if (whole == 0 && pieces < 2LL * cus) c *= 1.12;
-      if (s > 1) c += 0.25 * (double)rest * s / K;
+      if (s > 1) c += 0.25 * (double)g.rest * s / K;
       return c;
     };
     double best = cost(1);
     for (int s = 2; s <= s_max; ++s)
       if (cost(s) < best - 1e-9) { best = cost(s); splits = s; }
   }
-  int k_per_split = (K + splits - 1) / splits;
-  k_per_split = (k_per_split + BK - 1) / BK * BK;
-  splits = (K + k_per_split - 1) / k_per_split;
-  const bool split = splits > 1;
+  g.k_per_split = (K + splits - 1) / splits;
+  g.k_per_split = (g.k_per_split + BK - 1) / BK * BK;
+  g.splits = (K + g.k_per_split - 1) / g.k_per_split;
+  const bool split = g.splits > 1;
   // Unsplit "rest" tiles are ordinary whole tiles.
-  const int whole_tiles = split ? (int)whole : (int)tiles;
-  const int pieces = split ? rest * splits : 0;
+  g.whole_tiles = split ? (int)whole : (int)tiles;
+  g.pieces = split ? g.rest * g.splits : 0;
+  g.scratch_bytes = (size_t)g.pieces * g.bm * BN * sizeof(float);
+  return g;
+}
 
+}  // namespace
+
+size_t gemm_f32_scratch_bytes(int M, int N, int K) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  return plan_gemm(M, N, K).scratch_bytes;
+}
+
+int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
+             const float* A, int lda, const float* B, int ldb,
+             float* C, int ldc, bool accumulate, size_t scratch_offset) {
+  HASTE_HIP_REQUIRE(M > 0 && N > 0 && K > 0);
+  HASTE_HIP_REQUIRE(A != nullptr && B != nullptr && C != nullptr);
+  HASTE_HIP_REQUIRE(lda >= (trans_a ? M : K) && ldb >= N && ldc >= N);
+  HASTE_HIP_REQUIRE((long long)((M + 63) / 64) * ((N + BN - 1) / BN) < (1ll << 26));
+  const GemmPlan g = plan_gemm(M, N, K);
+  const int bm = g.bm, tiles_n = g.tiles_n, whole_tiles = g.whole_tiles, rest = g.rest;
+  const int splits = g.splits, k_per_split = g.k_per_split, pieces = g.pieces;
+  const bool split = splits > 1;
+
+  // The partial tiles live `scratch_offset` bytes (a multiple of 16) into the stream's
+  // scratch buffer; callers that keep data of their own in front of them say so.
   Workspace ws;
   float* partial = nullptr;
   if (split) {
-    const size_t bytes = (size_t)pieces * bm * BN * sizeof(float);
-    HASTE_HIP_PROPAGATE(get_workspace(stream, bytes, &ws));
-    partial = ws.scratch;
+    HASTE_HIP_PROPAGATE(get_workspace(stream, scratch_offset + g.scratch_bytes, &ws));
+    partial = ws.scratch + scratch_offset / sizeof(float);
   }
   // A workgroup addresses its operand panels (its rows of A, its columns of B, all of K)
   // with 32-bit byte offsets.

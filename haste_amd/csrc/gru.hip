@@ -428,7 +428,10 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
   HASTE_HIP_REQUIRE(W && R && bx && br && x && h && h_out && tmp_Wx);
   HASTE_HIP_REQUIRE(!training || v != nullptr);
   const ForwardTile tile = pick_forward_tile(3, N, H, 0);
-  if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  // No slice of R fits a CU: stream R from HBM every step instead.
+  if (!tile.ok)
+    return gru_forward_streamed(stream, training, T, N, C, H, W, R, bx, br, x, h, h_out, v, tmp_Wx,
+                                zoneout_prob, zoneout_mask, dc_mask, dc_scale);
   HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 3 * H, C, x, C, W, 3 * H, tmp_Wx, 3 * H, false));
 
   // Taken after the GEMM, which may replace the stream's scratch buffer with a larger one.
@@ -469,7 +472,9 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   HASTE_HIP_REQUIRE(dx && dW && dR && dbx && dbr && dh && dp && dq);
   // per row: the partial tiles or the 6 bias-gradient columns of 16 floats
   const BackwardTile tile = pick_backward_tile(gru_backward_k(H), N, H, 6 * 16, 0);
-  if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  if (!tile.ok)
+    return gru_backward_streamed(stream, T, N, C, H, W_t, R_t, x_t, h, v, dh_next, dx, dW, dR, dbx,
+                                 dbr, dh, dp, dq, zoneout_mask);
 
   Workspace ws;
   const size_t db_floats = ((size_t)tile.gy * 6 * H + 3) / 4 * 4;

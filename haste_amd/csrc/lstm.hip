@@ -427,7 +427,10 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
   HASTE_HIP_REQUIRE(W && R && b && x && h && c && h_out && c_out && v);
   const ForwardTile tile = pick_forward_tile(4, N, H, 0);
-  if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  // No slice of R fits a CU: stream R from HBM every step instead.
+  if (!tile.ok)
+    return lstm_forward_streamed(stream, training, T, N, C, H, W, R, b, x, h, c, h_out, c_out, v,
+                                 zoneout_prob, zoneout_mask, dc_mask, dc_scale);
   // v = x * W for all steps at once.
   HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 4 * H, C, x, C, W, 4 * H, v, 4 * H, false));
 
@@ -471,7 +474,9 @@ int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && c && c_next && dh_next && dc_next);
   HASTE_HIP_REQUIRE(dx && dW && dR && db && dh && dc && v);
   const BackwardTile tile = pick_backward_tile(4 * H, N, H, 4 * 16, 0);
-  if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  if (!tile.ok)
+    return lstm_backward_streamed(stream, T, N, C, H, W_t, R_t, x_t, h, c, c_next, dh_next, dc_next,
+                                  dx, dW, dR, db, dh, dc, v, zoneout_mask);
 
   Workspace ws;
   const size_t db_floats = (size_t)tile.gy * 4 * H;

@@ -37,7 +37,10 @@ const char* haste_hip_last_runtime_error(void);
 
 /* Largest hidden size whose recurrent weight slice the persistent kernels can keep
  * on chip for `gates` gate blocks (4 LSTM, 3 GRU) and `batch_size` rows on the
- * current device; 0 if none. */
+ * current device; 0 if none.  LSTM and GRU accept larger hidden sizes as well: they then
+ * stream the recurrent matrix from HBM every step (one GEMM and one pointwise kernel per
+ * step, as the reference does); the layer-norm cells return
+ * HASTE_HIP_ERROR_UNSUPPORTED_SIZE beyond it. */
 int haste_hip_max_hidden_size(int gates, int batch_size);
 
 /* Drops this thread's cached per-stream workspaces on the current device (frees

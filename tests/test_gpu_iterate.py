@@ -8,7 +8,8 @@ from util import TOL, dev, host, problem, relerr
 
 pytestmark = pytest.mark.gpu
 
-SHAPES = [(3, 2, 3, 4), (4, 5, 7, 20), (5, 16, 32, 64), (3, 64, 48, 128), (4, 1, 128, 512)]
+SHAPES = [(3, 2, 3, 4), (4, 5, 7, 20), (5, 16, 32, 64), (3, 64, 48, 128), (4, 1, 128, 512),
+          (2, 3, 16, 1536)]  # the last one streams R
 
 
 @pytest.mark.parametrize("zoneout", [0.0, 0.3])

@@ -10,7 +10,9 @@ pytestmark = pytest.mark.gpu
 # (T, N, C, H): tiny, ragged (sizes that are not multiples of any tile), and config-like
 SHAPES = [(1, 1, 1, 1), (3, 2, 3, 4), (5, 3, 7, 5), (6, 17, 20, 36), (4, 16, 32, 64),
           (10, 33, 48, 128), (8, 64, 64, 256), (12, 16, 128, 256), (6, 128, 96, 512),
-          (3, 200, 16, 64), (2, 300, 8, 48), (2, 520, 8, 32)]
+          (3, 200, 16, 64), (2, 300, 8, 48), (2, 520, 8, 32),
+          # hidden sizes beyond what stays on chip: the backward pass, then both passes, stream R
+          (3, 5, 40, 640), (3, 4, 32, 1536), (2, 70, 24, 1300)]
 
 
 def run_lstm(p, training, zoneout_prob, T, N, C, H):
@@ -89,3 +91,21 @@ def test_lstm_accumulates_into_weight_gradients_and_is_deterministic():
     torch.cuda.synchronize()
     for a, b in zip(*outs):
         assert torch.equal(a, b)
+
+
+def test_lstm_streamed_dropconnect_and_inference():
+    """DropConnect and the inference-mode zoneout blend on the path that streams R (H = 1536)."""
+    from haste_amd import ops
+    import torch
+    T, N, C, H = 3, 6, 16, 1536
+    p = problem(12, T, N, C, H, 4, 0.25)
+    m = (np.random.default_rng(4).uniform(size=p["R"].shape) >= 0.1).astype(np.float64)
+    scale = np.float64(np.float32(1.0 / 0.9))
+    h, c, v = ops.lstm_forward(False, 0.25, dev(p["x"]), dev(p["h0"]), dev(p["c0"]), dev(p["W"]),
+                               dev(p["R"]), dev(p["b"]), dev(p["mask"]), dropconnect_mask=dev(m),
+                               dropconnect_scale=float(scale))
+    torch.cuda.synchronize()
+    ho, co, _ = O.lstm_forward(p["W"], p["R"] * m * scale, p["b"], p["x"], p["h0"], p["c0"], False, 0.25,
+                               p["mask"])
+    assert relerr(host(h), ho) < TOL
+    assert relerr(host(c), co) < TOL
