@@ -924,7 +924,10 @@ int launch_persistent(const char* name, KernelT kernel, const LaunchPlan& plan, 
   return HASTE_HIP_OK;
 }
 
-constexpr size_t kMaxLdsBytes = 160 * 1024;  // LDS per workgroup on gfx950
+// Dynamic LDS a persistent kernel may ask for: the 160 KiB of a gfx950 workgroup less room
+// for the kernels' few statically allocated words (role, flag), which count against the
+// same limit.
+constexpr size_t kMaxLdsBytes = 160 * 1024 - 256;
 
 // Floats of the exchange tiles (2 behind a step barrier, kPolledTiles when polled) of every
 // group (batch tile) for contraction length K.

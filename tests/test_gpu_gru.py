@@ -11,7 +11,7 @@ SHAPES = [(1, 1, 1, 1), (3, 2, 3, 4), (5, 3, 7, 5), (6, 17, 20, 36), (4, 16, 32,
           (10, 33, 48, 128), (8, 64, 64, 256), (6, 128, 96, 512),
           (3, 200, 16, 64), (2, 300, 8, 48), (2, 520, 8, 32),
           # hidden sizes beyond what stays on chip: the backward pass, then both passes, stream R
-          (3, 5, 40, 704), (3, 4, 32, 1536), (2, 70, 24, 1700)]
+          (3, 5, 40, 704), (3, 4, 32, 1536), (2, 70, 24, 1700), (2, 128, 16, 1024)]
 
 
 @pytest.mark.parametrize("zoneout", [0.0, 0.3])
