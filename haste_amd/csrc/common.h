@@ -99,9 +99,10 @@ int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
 // Bytes of scratch gemm_f32 uses for this shape (0 when nothing is split).
 size_t gemm_f32_scratch_bytes(int M, int N, int K);
 
-// LSTM / GRU with the recurrent matrix streamed from HBM every step (per-step GEMM +
-// pointwise kernel): for hidden sizes whose slices of R do not fit on chip.  Arguments as
-// the persistent implementations in lstm.hip / gru.hip.
+// The cells in step-wise form, the recurrent matrix streamed from HBM every step (per-step
+// GEMM + row-wise norms + pointwise kernels): for hidden sizes whose slices of R do not fit
+// on chip.  Arguments as the persistent implementations in lstm.hip / gru.hip /
+// layer_norm_lstm.hip / layer_norm_gru.hip.
 int lstm_forward_streamed(hipStream_t stream, int training, int T, int N, int C, int H,
                           const float* W, const float* R, const float* b, const float* x,
                           const float* h, const float* c, float* h_out, float* c_out, float* v,
@@ -123,6 +124,37 @@ int gru_backward_streamed(hipStream_t stream, int T, int N, int C, int H,
                           const float* v, const float* dh_next, float* dx, float* dW, float* dR,
                           float* dbx, float* dbr, float* dh, float* dp, float* dq,
                           const float* zoneout_mask);
+int layer_norm_lstm_forward_streamed(hipStream_t stream, int training, int T, int N, int C, int H,
+                                     const float* W, const float* R, const float* b, const float* x,
+                                     float* h, float* c, float* act_Wx, const float* gamma1,
+                                     float* cache1, float* act_Wx_norm, float* act_Rh,
+                                     const float* gamma2, float* cache2, const float* gamma_h,
+                                     const float* beta_h, float* cache3, float* act_c_norm,
+                                     float zoneout_prob, const float* zoneout_mask);
+int layer_norm_lstm_backward_streamed(hipStream_t stream, int T, int N, int C, int H,
+                                      const float* W_t, const float* R_t, const float* x_t,
+                                      const float* h, const float* c, const float* dh_new,
+                                      const float* dc_new, float* dx, float* dW, float* dR, float* db,
+                                      float* dh, float* dc, float* act_Wx, const float* gamma1,
+                                      float* dgamma1, float* act_Wx_norm, float* act_Rh,
+                                      const float* gamma2, float* dgamma2, const float* cache2,
+                                      const float* gamma_h, float* dgamma_h, float* dbeta_h,
+                                      const float* cache3, float* act_c_norm,
+                                      const float* zoneout_mask);
+int layer_norm_gru_forward_streamed(hipStream_t stream, int training, int T, int N, int C, int H,
+                                    const float* W, const float* R, const float* bx, const float* br,
+                                    const float* x, float* h, float* v, float* act_Wx,
+                                    const float* gamma1, float* cache1, float* tmp_Wx_norm,
+                                    float* act_Rh, const float* gamma2, float* cache2,
+                                    float zoneout_prob, const float* zoneout_mask);
+int layer_norm_gru_backward_streamed(hipStream_t stream, int T, int N, int C, int H,
+                                     const float* W_t, const float* R_t, const float* x_t,
+                                     const float* h, const float* v, const float* dh_new, float* dx,
+                                     float* dW, float* dR, float* dbx, float* dbr, float* dh,
+                                     float* dp, float* dq, const float* act_Wx, const float* gamma1,
+                                     float* dgamma1, const float* act_Rh, const float* gamma2,
+                                     float* dgamma2, const float* cache2,
+                                     const float* zoneout_mask);
 
 // Row-wise layer norm kernels (rows x dim), used stand-alone and by the LN cells.
 int layer_norm_forward(hipStream_t stream, int rows, int dim, const float* gamma,

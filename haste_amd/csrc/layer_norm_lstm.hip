@@ -632,7 +632,11 @@ int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_siz
   HASTE_HIP_REQUIRE(gamma2 && gamma_h && beta_h && act_c_norm);
   hipStream_t stream = as_stream(stream_);
   const ForwardTile tile = pick_forward_tile(4, N, H, 4 * sizeof(float));
-  if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  if (!tile.ok)
+    return layer_norm_lstm_forward_streamed(stream, training, T, N, C, H, W, R, b, x, h, c, act_Wx,
+                                            gamma1, cache1, act_Wx_norm, act_Rh, gamma2, cache2,
+                                            gamma_h, beta_h, cache3, act_c_norm, zoneout_prob,
+                                            zoneout_mask);
   const int gx = tile.gx, gy = tile.gy;
   const int NB = tile.nb;
   // one tagged row exchange: [groups][2] buffers of 8-byte words, counted in floats
@@ -698,7 +702,11 @@ int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_
   hipStream_t stream = as_stream(stream_);
   // per row: 10 column-sum accumulators of 16 floats (or the partial tiles, whichever is more) + 4 sums
   const BackwardTile tile = pick_backward_tile(4 * H, N, H, 10 * 16, 8);
-  if (!tile.ok) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  if (!tile.ok)
+    return layer_norm_lstm_backward_streamed(stream, T, N, C, H, W_t, R_t, x_t, h, c, dh_new, dc_new,
+                                             dx, dW, dR, db, dh, dc, act_Wx, gamma1, dgamma1,
+                                             act_Wx_norm, act_Rh, gamma2, dgamma2, cache2, gamma_h,
+                                             dgamma_h, dbeta_h, cache3, act_c_norm, zoneout_mask);
   const int gx = tile.gx, gy = tile.gy;
   const int NB = tile.nb;
   // one tagged row exchange: [groups][2] buffers of 8-byte words, counted in floats

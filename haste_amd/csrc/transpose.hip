@@ -12,18 +12,19 @@ namespace {
 
 constexpr int TT = 64;
 
+template <typename T>
 __global__ __launch_bounds__(256)
-void transpose_f32_kernel(int rows, int cols, const float* __restrict__ in,
-                          float* __restrict__ out, int tiles_c) {
-  __shared__ float tile[TT][TT + 1];
+void transpose_kernel(int rows, int cols, const T* __restrict__ in, T* __restrict__ out,
+                      int tiles_c) {
+  __shared__ T tile[TT][TT + 1];
   const int tr = blockIdx.x / tiles_c, tc = blockIdx.x % tiles_c;
   const int r0 = tr * TT, c0 = tc * TT;
   const int lx = threadIdx.x & 63, ly = threadIdx.x >> 6;
-  float v[16];
+  T v[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
     const int r = r0 + ly + 4 * i, c = c0 + lx;
-    v[i] = (r < rows && c < cols) ? in[(size_t)r * cols + c] : 0.f;
+    v[i] = (r < rows && c < cols) ? in[(size_t)r * cols + c] : T(0);
   }
 #pragma unroll
   for (int i = 0; i < 16; ++i) tile[ly + 4 * i][lx] = v[i];
@@ -35,19 +36,28 @@ void transpose_f32_kernel(int rows, int cols, const float* __restrict__ in,
   }
 }
 
+template <typename T>
+int transpose(const char* name, int rows, int cols, const T* in, T* out, hipStream_t stream) {
+  HASTE_HIP_REQUIRE(rows > 0 && cols > 0 && in != nullptr && out != nullptr && in != out);
+  const long long tiles_r = (rows + TT - 1) / TT;
+  const long long tiles_c = (cols + TT - 1) / TT;
+  HASTE_HIP_REQUIRE(tiles_r * tiles_c < (1ll << 31));
+  ScopedKernelTimer timer(name, stream);
+  transpose_kernel<T><<<dim3((unsigned)(tiles_r * tiles_c)), dim3(256), 0, stream>>>(
+      rows, cols, in, out, (int)tiles_c);
+  HASTE_HIP_TRY(hipGetLastError());
+  return HASTE_HIP_OK;
+}
+
 }  // namespace
 }  // namespace haste_hip
 
 extern "C" int haste_hip_transpose_f32(int rows, int cols, const float* in, float* out,
                                        void* stream) {
-  HASTE_HIP_REQUIRE(rows > 0 && cols > 0 && in != nullptr && out != nullptr && in != out);
-  const long long tiles_r = (rows + haste_hip::TT - 1) / haste_hip::TT;
-  const long long tiles_c = (cols + haste_hip::TT - 1) / haste_hip::TT;
-  HASTE_HIP_REQUIRE(tiles_r * tiles_c < (1ll << 31));
-  haste_hip::ScopedKernelTimer timer("transpose_f32", haste_hip::as_stream(stream));
-  haste_hip::transpose_f32_kernel<<<dim3((unsigned)(tiles_r * tiles_c)), dim3(256), 0,
-                                    haste_hip::as_stream(stream)>>>(rows, cols, in, out,
-                                                                    (int)tiles_c);
-  HASTE_HIP_TRY(hipGetLastError());
-  return HASTE_HIP_OK;
+  return haste_hip::transpose("transpose_f32", rows, cols, in, out, haste_hip::as_stream(stream));
+}
+
+extern "C" int haste_hip_transpose_f64(int rows, int cols, const double* in, double* out,
+                                       void* stream) {
+  return haste_hip::transpose("transpose_f64", rows, cols, in, out, haste_hip::as_stream(stream));
 }

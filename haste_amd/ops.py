@@ -2,8 +2,9 @@
 (`haste_pytorch_lib.<cell>_forward / <cell>_backward`, reference
 frameworks/pytorch/{lstm,gru,indrnn,layer_norm_lstm,layer_norm_gru,layer_norm_indrnn}.cc),
 with the same argument order, allocation protocol and return tuples, implemented by
-calls into libhaste_hip.so.  Tensors are float32, contiguous, on the GPU; torch is
-used only to allocate device memory and to name the current stream.
+calls into libhaste_hip.so.  Tensors are float32 or float64 (all tensors of a call alike),
+contiguous, on the GPU; torch is used only to allocate device memory and to name the
+current stream.
 """
 import torch
 
@@ -17,8 +18,21 @@ def _check(*tensors):
             raise ValueError("tensor must be a GPU tensor")
         if not t.is_contiguous():
             raise ValueError("tensor must be contiguous")
-        if t.dtype != torch.float32:
-            raise ValueError("only float32 is implemented")
+        if t.numel() and t.dtype not in _SUFFIX:
+            raise ValueError("only float32 and float64 are implemented")
+
+
+_SUFFIX = {torch.float32: "_f32", torch.float64: "_f64"}
+
+
+def _call(entry, *args):
+    """Calls `entry` + "_f32" / "_f64" according to the tensors among `args`, which must all
+    have one dtype (the reference's bindings dispatch the same way, AT_DISPATCH_FLOATING_TYPES,
+    frameworks/pytorch/lstm.cc:65)."""
+    dtypes = {a.dtype for a in args if isinstance(a, torch.Tensor) and a.numel()}
+    if len(dtypes) != 1:
+        raise ValueError("all tensors of a call must have the same dtype, got %s" % sorted(map(str, dtypes)))
+    lib.call(entry + _SUFFIX[dtypes.pop()], *args)
 
 
 def _mask_or_none(has_zoneout, zoneout_mask):
@@ -34,7 +48,7 @@ def gemm(a, b, out=None, trans_a=False, accumulate=False):
     if out is None:
         assert not accumulate
         out = torch.empty(M, N, device=a.device, dtype=a.dtype)
-    lib.call("haste_hip_gemm_f32", int(trans_a), M, N, K, a, a.stride(0), b, b.stride(0),
+    _call("haste_hip_gemm", int(trans_a), M, N, K, a, a.stride(0), b, b.stride(0),
              out, out.stride(0), int(accumulate))
     return out
 
@@ -47,7 +61,7 @@ def transpose(a, out=None):
     rows = a.numel() // cols
     if out is None:
         out = torch.empty((cols,) + tuple(a.shape[:-1]), device=a.device, dtype=a.dtype)
-    lib.call("haste_hip_transpose_f32", rows, cols, a, out)
+    _call("haste_hip_transpose", rows, cols, a, out)
     return out
 
 
@@ -67,11 +81,11 @@ def lstm_forward(training, zoneout_prob, x, h0, c0, kernel, recurrent_kernel, bi
     zp = float(zoneout_prob) if has_zoneout else 0.0
     mask = _mask_or_none(has_zoneout, zoneout_mask)
     if dropconnect_mask is None:
-        lib.call("haste_hip_lstm_forward_f32", bool(training), T, N, C, H, kernel, recurrent_kernel,
+        _call("haste_hip_lstm_forward", bool(training), T, N, C, H, kernel, recurrent_kernel,
                  bias, x, output, output_state, cache, None, zp, mask)
     else:
         _check(dropconnect_mask)
-        lib.call("haste_hip_lstm_forward_dropconnect_f32", bool(training), T, N, C, H, kernel,
+        _call("haste_hip_lstm_forward_dropconnect", bool(training), T, N, C, H, kernel,
                  recurrent_kernel, bias, x, output, output_state, cache, zp, mask,
                  dropconnect_mask, float(dropconnect_scale))
     return output, output_state, cache
@@ -89,7 +103,7 @@ def lstm_backward(x_t, kernel_t, recurrent_kernel_t, bias, zoneout_mask, h, c, c
     db = torch.zeros(4 * H, **opts)
     dh = torch.zeros(N, H, **opts)
     dc = torch.zeros(N, H, **opts)
-    lib.call("haste_hip_lstm_backward_f32", T, N, C, H, kernel_t, recurrent_kernel_t, bias, x_t,
+    _call("haste_hip_lstm_backward", T, N, C, H, kernel_t, recurrent_kernel_t, bias, x_t,
              h, c, dh_new, dc_new, dx, dW, dR, db, dh, dc, cache,
              _mask_or_none(has_zoneout, zoneout_mask))
     return dx, dh, dc, dW, dR, db
@@ -107,7 +121,7 @@ def lstm_forward_iterate(training, zoneout_prob, x, h, c, kernel, recurrent_kern
     c_out = torch.empty_like(c) if c_out is None else c_out
     v = torch.empty(N, 4 * H, device=x.device, dtype=x.dtype)
     has_zoneout = bool(zoneout_prob) and zoneout_mask is not None and zoneout_mask.numel() > 0
-    lib.call("haste_hip_lstm_forward_iterate_f32", bool(training), N, C, H, kernel, recurrent_kernel,
+    _call("haste_hip_lstm_forward_iterate", bool(training), N, C, H, kernel, recurrent_kernel,
              bias, x, h, c, h_out, c_out, v, None, float(zoneout_prob) if has_zoneout else 0.0,
              zoneout_mask if has_zoneout else None)
     return h_out, c_out, v
@@ -122,7 +136,7 @@ def lstm_backward_iterate(x_t, kernel_t, recurrent_kernel_t, bias, h, c, c_new, 
     _check(x_t, kernel_t, recurrent_kernel_t, bias, h, c, c_new, dh_new, dc_new, v, dW, dR, db, dh, dc)
     dx = torch.empty(N, C, device=x_t.device, dtype=x_t.dtype)
     has_zoneout = zoneout_mask is not None and zoneout_mask.numel() > 0
-    lib.call("haste_hip_lstm_backward_iterate_f32", N, C, H, kernel_t, recurrent_kernel_t, bias, x_t,
+    _call("haste_hip_lstm_backward_iterate", N, C, H, kernel_t, recurrent_kernel_t, bias, x_t,
              h, c, c_new, dh_new, dc_new, dx, dW, dR, db, dh, dc, v,
              zoneout_mask if has_zoneout else None)
     return dx
@@ -138,7 +152,7 @@ def gru_forward_iterate(training, zoneout_prob, x, h, kernel, recurrent_kernel, 
     v = torch.empty(N, 4 * H, device=x.device, dtype=x.dtype)
     tmp_Wx = torch.empty(N, 3 * H, device=x.device, dtype=x.dtype)
     has_zoneout = bool(zoneout_prob) and zoneout_mask is not None and zoneout_mask.numel() > 0
-    lib.call("haste_hip_gru_forward_iterate_f32", bool(training), N, C, H, kernel, recurrent_kernel,
+    _call("haste_hip_gru_forward_iterate", bool(training), N, C, H, kernel, recurrent_kernel,
              bias, recurrent_bias, x, h, h_out, v, tmp_Wx, None,
              float(zoneout_prob) if has_zoneout else 0.0, zoneout_mask if has_zoneout else None)
     return h_out, v
@@ -154,7 +168,7 @@ def gru_backward_iterate(x_t, kernel_t, recurrent_kernel_t, bias, recurrent_bias
     dp = torch.empty(N, 3 * H, **opts)
     dq = torch.empty(N, 3 * H, **opts)
     has_zoneout = zoneout_mask is not None and zoneout_mask.numel() > 0
-    lib.call("haste_hip_gru_backward_iterate_f32", N, C, H, kernel_t, recurrent_kernel_t, bias,
+    _call("haste_hip_gru_backward_iterate", N, C, H, kernel_t, recurrent_kernel_t, bias,
              recurrent_bias, x_t, h, v, dh_new, dx, dW, dR, dbx, dbr, dh, dp, dq,
              zoneout_mask if has_zoneout else None)
     return dx
@@ -175,11 +189,11 @@ def gru_forward(training, zoneout_prob, x, h0, kernel, recurrent_kernel, bias, r
     zp = float(zoneout_prob) if has_zoneout else 0.0
     mask = _mask_or_none(has_zoneout, zoneout_mask)
     if dropconnect_mask is None:
-        lib.call("haste_hip_gru_forward_f32", bool(training), T, N, C, H, kernel, recurrent_kernel,
+        _call("haste_hip_gru_forward", bool(training), T, N, C, H, kernel, recurrent_kernel,
                  bias, recurrent_bias, x, output, cache if training else None, tmp_Wx, None, zp, mask)
     else:
         _check(dropconnect_mask)
-        lib.call("haste_hip_gru_forward_dropconnect_f32", bool(training), T, N, C, H, kernel,
+        _call("haste_hip_gru_forward_dropconnect", bool(training), T, N, C, H, kernel,
                  recurrent_kernel, bias, recurrent_bias, x, output, cache if training else None,
                  tmp_Wx, zp, mask, dropconnect_mask, float(dropconnect_scale))
     return output, cache
@@ -200,7 +214,7 @@ def gru_backward(x_t, kernel_t, recurrent_kernel_t, bias, recurrent_bias, zoneou
     dh = torch.zeros(N, H, **opts)
     dp = torch.empty(T, N, 3 * H, **opts)
     dq = torch.empty(T, N, 3 * H, **opts)
-    lib.call("haste_hip_gru_backward_f32", T, N, C, H, kernel_t, recurrent_kernel_t, bias,
+    _call("haste_hip_gru_backward", T, N, C, H, kernel_t, recurrent_kernel_t, bias,
              recurrent_bias, x_t, h, cache, dh_new, dx, dW, dR, dbx, dbr, dh, dp, dq,
              _mask_or_none(has_zoneout, zoneout_mask))
     return dx, dh, dW, dR, dbx, dbr
@@ -212,7 +226,7 @@ def layer_norm_forward(x, gamma, beta=None):
     rows, dim = x.numel() // x.shape[-1], x.shape[-1]
     y = torch.empty_like(x)
     cache = torch.empty(rows, 2, device=x.device, dtype=x.dtype)
-    lib.call("haste_hip_layer_norm_forward_f32", rows, dim, gamma, beta, x, y, cache)
+    _call("haste_hip_layer_norm_forward", rows, dim, gamma, beta, x, y, cache)
     return y, cache
 
 
@@ -222,7 +236,7 @@ def layer_norm_backward(x, gamma, dy, cache=None, with_beta=True, in_place=False
     dx = dy if in_place else torch.empty_like(x)
     dgamma = torch.zeros_like(gamma)
     dbeta = torch.zeros_like(gamma) if with_beta else None
-    lib.call("haste_hip_layer_norm_backward_f32", rows, dim, gamma, x, dy, dx, dgamma, dbeta, cache)
+    _call("haste_hip_layer_norm_backward", rows, dim, gamma, x, dy, dx, dgamma, dbeta, cache)
     return dx, dgamma, dbeta
 
 
@@ -236,7 +250,7 @@ def indrnn_forward(training, zoneout_prob, x, h0, kernel, recurrent_scale, bias,
     output = torch.empty(T + 1, N, H, **opts)
     workspace = torch.empty(T, N, H, **opts)
     output[0] = h0
-    lib.call("haste_hip_indrnn_forward_f32", bool(training), T, N, C, H, kernel, recurrent_scale,
+    _call("haste_hip_indrnn_forward", bool(training), T, N, C, H, kernel, recurrent_scale,
              bias, x, output, workspace, float(zoneout_prob) if has_zoneout else 0.0,
              _mask_or_none(has_zoneout, zoneout_mask))
     return output
@@ -254,7 +268,7 @@ def indrnn_backward(x_t, kernel_t, recurrent_scale, bias, zoneout_mask, h, dh_ne
     db = torch.zeros_like(bias)
     dh = torch.zeros(N, H, **opts)
     workspace = torch.empty(T, N, H, **opts)
-    lib.call("haste_hip_indrnn_backward_f32", T, N, C, H, kernel_t, recurrent_scale, bias, x_t, h,
+    _call("haste_hip_indrnn_backward", T, N, C, H, kernel_t, recurrent_scale, bias, x_t, h,
              dh_new, dx, dW, du, db, dh, workspace, _mask_or_none(has_zoneout, zoneout_mask))
     return dx, dh, dW, du, db
 
@@ -272,7 +286,7 @@ def layer_norm_indrnn_forward(training, zoneout_prob, x, h0, kernel, recurrent_s
     act_Wx = torch.empty(T, N, H, **opts)
     act_Wx_norm_cache = torch.empty(T, N, 2, **opts)
     output[0] = h0
-    lib.call("haste_hip_layer_norm_indrnn_forward_f32", bool(training), T, N, C, H, kernel,
+    _call("haste_hip_layer_norm_indrnn_forward", bool(training), T, N, C, H, kernel,
              recurrent_scale, bias, x, output, workspace, act_Wx, gamma[0], act_Wx_norm_cache,
              float(zoneout_prob) if has_zoneout else 0.0, _mask_or_none(has_zoneout, zoneout_mask))
     return output, act_Wx, act_Wx_norm_cache
@@ -292,7 +306,7 @@ def layer_norm_indrnn_backward(x_t, kernel_t, recurrent_scale, bias, gamma, zone
     dh = torch.zeros(N, H, **opts)
     workspace = torch.empty(T, N, H, **opts)
     dgamma = torch.zeros_like(gamma)
-    lib.call("haste_hip_layer_norm_indrnn_backward_f32", T, N, C, H, kernel_t, recurrent_scale, bias,
+    _call("haste_hip_layer_norm_indrnn_backward", T, N, C, H, kernel_t, recurrent_scale, bias,
              x_t, h, dh_new, dx, dW, du, db, dh, workspace, act_Wx, gamma[0], dgamma[0],
              _mask_or_none(has_zoneout, zoneout_mask))
     return dx, dh, dW, du, db, dgamma
@@ -317,7 +331,7 @@ def layer_norm_lstm_forward(training, zoneout_prob, x, h0, c0, kernel, recurrent
     act_c_norm_cache = torch.empty(T, N, 2, **opts)
     output[0] = h0
     output_state[0] = c0
-    lib.call("haste_hip_layer_norm_lstm_forward_f32", bool(training), T, N, C, H, kernel,
+    _call("haste_hip_layer_norm_lstm_forward", bool(training), T, N, C, H, kernel,
              recurrent_kernel, bias, x, output, output_state, act_Wx, None,
              gamma[0], act_Wx_norm_cache, act_Wx_norm, act_Rh, gamma[1], act_Rh_norm_cache,
              gamma_h, beta_h, act_c_norm_cache, act_c_norm,
@@ -345,7 +359,7 @@ def layer_norm_lstm_backward(x_t, kernel_t, recurrent_kernel_t, bias, gamma, gam
     dbeta_h = torch.zeros_like(beta_h)
     dh = torch.zeros(N, H, **opts)
     dc = torch.zeros(N, H, **opts)
-    lib.call("haste_hip_layer_norm_lstm_backward_f32", T, N, C, H, kernel_t, recurrent_kernel_t,
+    _call("haste_hip_layer_norm_lstm_backward", T, N, C, H, kernel_t, recurrent_kernel_t,
              bias, x_t, h, c, dh_new, dc_new, dx, dW, dR, db, dh, dc,
              act_Wx, gamma[0], dgamma[0], act_Wx_norm, act_Rh, gamma[1], dgamma[1],
              act_Rh_norm_cache, gamma_h, beta_h, dgamma_h, dbeta_h, act_c_norm_cache, act_c_norm,
@@ -369,7 +383,7 @@ def layer_norm_gru_forward(training, zoneout_prob, x, h0, kernel, recurrent_kern
     act_Rh = torch.empty(T, N, 3 * H, **opts)
     act_Rh_norm_cache = torch.empty(T, N, 2, **opts)
     output[0] = h0
-    lib.call("haste_hip_layer_norm_gru_forward_f32", bool(training), T, N, C, H, kernel,
+    _call("haste_hip_layer_norm_gru_forward", bool(training), T, N, C, H, kernel,
              recurrent_kernel, bias, recurrent_bias, x, output, cache if training else None,
              act_Wx, gamma[0], act_Wx_norm_cache, tmp_Wx_norm, act_Rh, gamma[1], act_Rh_norm_cache,
              None, float(zoneout_prob) if has_zoneout else 0.0,
@@ -395,7 +409,7 @@ def layer_norm_gru_backward(x_t, kernel_t, recurrent_kernel_t, bias, recurrent_b
     dp = torch.empty(T, N, 3 * H, **opts)
     dq = torch.empty(T, N, 3 * H, **opts)
     dgamma = torch.zeros_like(gamma)
-    lib.call("haste_hip_layer_norm_gru_backward_f32", T, N, C, H, kernel_t, recurrent_kernel_t, bias,
+    _call("haste_hip_layer_norm_gru_backward", T, N, C, H, kernel_t, recurrent_kernel_t, bias,
              recurrent_bias, x_t, h, cache, dh_new, dx, dW, dR, dbx, dbr, dh, dp, dq,
              act_Wx, gamma[0], dgamma[0], act_Rh, gamma[1], dgamma[1], act_Rh_norm_cache,
              _mask_or_none(has_zoneout, zoneout_mask))

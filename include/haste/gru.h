@@ -38,7 +38,7 @@ class ForwardPass {
         T* tmp_Rh,
         const float zoneout_prob,
         const T* zoneout_mask) {
-      data_.status = haste_hip_gru_forward_iterate_f32(
+      data_.status = detail::Abi<T>::gru_forward_iterate(
           data_.training, data_.batch_size, data_.input_size, data_.hidden_size,
           W, R, bx, br, x, h, h_out, v, tmp_Wx, tmp_Rh, zoneout_prob, zoneout_mask,
           detail::stream_arg(data_.stream));
@@ -60,7 +60,7 @@ class ForwardPass {
         T* tmp_Rh,
         const float zoneout_prob,
         const T* zoneout_mask) {
-      data_.status = haste_hip_gru_forward_f32(
+      data_.status = detail::Abi<T>::gru_forward(
           data_.training, steps, data_.batch_size, data_.input_size, data_.hidden_size,
           W, R, bx, br, x, h, v, tmp_Wx, tmp_Rh, zoneout_prob, zoneout_mask,
           detail::stream_arg(data_.stream));
@@ -105,7 +105,7 @@ class BackwardPass {
         T* dp,
         T* dq,
         const T* zoneout_mask) {
-      data_.status = haste_hip_gru_backward_iterate_f32(
+      data_.status = detail::Abi<T>::gru_backward_iterate(
           data_.batch_size, data_.input_size, data_.hidden_size,
           W_t, R_t, bx, br, x_t, h, v, dh_new, dx, dW, dR, dbx, dbr, dh, dp, dq, zoneout_mask,
           detail::stream_arg(data_.stream));
@@ -133,7 +133,7 @@ class BackwardPass {
         T* dp,
         T* dq,
         const T* zoneout_mask) {
-      data_.status = haste_hip_gru_backward_f32(
+      data_.status = detail::Abi<T>::gru_backward(
           steps, data_.batch_size, data_.input_size, data_.hidden_size,
           W_t, R_t, bx, br, x_t, h, v, dh_new, dx, dW, dR, dbx, dbr, dh, dp, dq, zoneout_mask,
           detail::stream_arg(data_.stream));

@@ -34,7 +34,7 @@ class ForwardPass {
         T* workspace,
         const float zoneout_prob,
         const T* zoneout_mask) {
-      data_.status = haste_hip_indrnn_forward_f32(
+      data_.status = detail::Abi<T>::indrnn_forward(
           data_.training, steps, data_.batch_size, data_.input_size, data_.hidden_size,
           W, u, b, x, h, workspace, zoneout_prob, zoneout_mask, detail::stream_arg(data_.stream));
     }
@@ -77,7 +77,7 @@ class BackwardPass {
         T* dh,
         T* workspace,
         const T* zoneout_mask) {
-      data_.status = haste_hip_indrnn_backward_f32(
+      data_.status = detail::Abi<T>::indrnn_backward(
           steps, data_.batch_size, data_.input_size, data_.hidden_size,
           W_t, u, b, x_t, h, dh_new, dx, dW, du, db, dh, workspace, zoneout_mask,
           detail::stream_arg(data_.stream));

@@ -36,7 +36,7 @@ class ForwardPass {
         const T* x,
         T* y) {
       assert(partial_ + minibatch <= batch_size_);
-      status_ = haste_hip_layer_norm_forward_f32(
+      status_ = detail::Abi<T>::layer_norm_forward(
           minibatch, hidden_size_, gamma_, beta_, x, y, cache_ ? cache_ + partial_ * 2 : nullptr,
           detail::stream_arg(stream));
       partial_ += minibatch;
@@ -93,7 +93,7 @@ class BackwardPass {
         T* dx) {
       assert(partial_ - minibatch >= 0);
       const int first = partial_ - minibatch;
-      status_ = haste_hip_layer_norm_backward_f32(
+      status_ = detail::Abi<T>::layer_norm_backward(
           minibatch, hidden_size_, gamma_, x_ + static_cast<long long>(first) * hidden_size_, dy,
           dx, dgamma_, (beta_ && dbeta_) ? dbeta_ : nullptr, cache_ ? cache_ + first * 2 : nullptr,
           detail::stream_arg(stream));

@@ -44,7 +44,7 @@ class ForwardPass {
         T* tmp_Rh_norm,
         const float zoneout_prob,
         const T* zoneout_mask) {
-      data_.status = haste_hip_layer_norm_gru_forward_f32(
+      data_.status = detail::Abi<T>::layer_norm_gru_forward(
           data_.training, steps, data_.batch_size, data_.input_size, data_.hidden_size,
           W, R, bx, br, x, h, v, act_Wx, layer_norm1.gamma(), layer_norm1.cache(), tmp_Wx_norm,
           act_Rh, layer_norm2.gamma(), layer_norm2.cache(), tmp_Rh_norm,
@@ -96,7 +96,7 @@ class BackwardPass {
         layer_norm::BackwardPass<T>& layer_norm1,
         layer_norm::BackwardPass<T>& layer_norm2,
         const T* zoneout_mask) {
-      data_.status = haste_hip_layer_norm_gru_backward_f32(
+      data_.status = detail::Abi<T>::layer_norm_gru_backward(
           steps, data_.batch_size, data_.input_size, data_.hidden_size,
           W_t, R_t, bx, br, x_t, h, v, dh_new, dx, dW, dR, dbx, dbr, dh, dp, dq,
           layer_norm1.x(), layer_norm1.gamma(), layer_norm1.dgamma(),

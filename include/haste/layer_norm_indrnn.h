@@ -38,7 +38,7 @@ class ForwardPass {
         layer_norm::ForwardPass<T>& layer_norm1,
         const float zoneout_prob,
         const T* zoneout_mask) {
-      data_.status = haste_hip_layer_norm_indrnn_forward_f32(
+      data_.status = detail::Abi<T>::layer_norm_indrnn_forward(
           data_.training, steps, data_.batch_size, data_.input_size, data_.hidden_size,
           W, u, b, x, h, workspace, act_Wx, layer_norm1.gamma(), layer_norm1.cache(),
           zoneout_prob, zoneout_mask, detail::stream_arg(data_.stream));
@@ -82,7 +82,7 @@ class BackwardPass {
         T* workspace,
         layer_norm::BackwardPass<T>& layer_norm1,
         const T* zoneout_mask) {
-      data_.status = haste_hip_layer_norm_indrnn_backward_f32(
+      data_.status = detail::Abi<T>::layer_norm_indrnn_backward(
           steps, data_.batch_size, data_.input_size, data_.hidden_size,
           W_t, u, b, x_t, h, dh_new, dx, dW, du, db, dh, workspace,
           layer_norm1.x(), layer_norm1.gamma(), layer_norm1.dgamma(), zoneout_mask,

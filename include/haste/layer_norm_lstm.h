@@ -48,7 +48,7 @@ class ForwardPass {
         T* act_c_norm,
         const float zoneout_prob,
         const T* zoneout_mask) {
-      data_.status = haste_hip_layer_norm_lstm_forward_f32(
+      data_.status = detail::Abi<T>::layer_norm_lstm_forward(
           data_.training, steps, data_.batch_size, data_.input_size, data_.hidden_size,
           W, R, b, x, h, c, act_Wx, tmp_Rh,
           layer_norm1.gamma(), layer_norm1.cache(), act_Wx_norm, act_Rh,
@@ -105,7 +105,7 @@ class BackwardPass {
         layer_norm::BackwardPass<T>& layer_norm3,
         T* act_c_norm,
         const T* zoneout_mask) {
-      data_.status = haste_hip_layer_norm_lstm_backward_f32(
+      data_.status = detail::Abi<T>::layer_norm_lstm_backward(
           steps, data_.batch_size, data_.input_size, data_.hidden_size,
           W_t, R_t, b, x_t, h, c, dh_new, dc_new, dx, dW, dR, db, dh, dc,
           act_Wx, layer_norm1.gamma(), layer_norm1.dgamma(), act_Wx_norm, act_Rh,

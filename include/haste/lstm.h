@@ -48,7 +48,7 @@ class ForwardPass {
       void* theirs = detail::stream_arg(stream);
       data_.status = haste_hip_stream_order(theirs, mine);
       if (data_.status != HASTE_HIP_OK) return;
-      data_.status = haste_hip_lstm_forward_iterate_f32(
+      data_.status = detail::Abi<T>::lstm_forward_iterate(
           data_.training, data_.batch_size, data_.input_size, data_.hidden_size,
           W, R, b, x, h, c, h_out, c_out, v, tmp_Rh, zoneout_prob, zoneout_mask, mine);
       if (data_.status != HASTE_HIP_OK) return;
@@ -69,7 +69,7 @@ class ForwardPass {
         T* tmp_Rh,
         const float zoneout_prob,
         const T* zoneout_mask) {
-      data_.status = haste_hip_lstm_forward_f32(
+      data_.status = detail::Abi<T>::lstm_forward(
           data_.training, steps, data_.batch_size, data_.input_size, data_.hidden_size,
           W, R, b, x, h, c, v, tmp_Rh, zoneout_prob, zoneout_mask,
           detail::stream_arg(data_.stream));
@@ -121,7 +121,7 @@ class BackwardPass {
       void* theirs = detail::stream_arg(stream);
       data_.status = haste_hip_stream_order(theirs, mine);
       if (data_.status != HASTE_HIP_OK) return;
-      data_.status = haste_hip_lstm_backward_iterate_f32(
+      data_.status = detail::Abi<T>::lstm_backward_iterate(
           data_.batch_size, data_.input_size, data_.hidden_size,
           W_t, R_t, b, x_t, h, c, c_new, dh_new, dc_new, dx, dW, dR, db, dh, dc, v, zoneout_mask,
           mine);
@@ -150,7 +150,7 @@ class BackwardPass {
         T* dc,
         T* v,
         const T* zoneout_mask) {
-      data_.status = haste_hip_lstm_backward_f32(
+      data_.status = detail::Abi<T>::lstm_backward(
           steps, data_.batch_size, data_.input_size, data_.hidden_size,
           W_t, R_t, b, x_t, h, c, dh_new, dc_new, dx, dW, dR, db, dh, dc, v, zoneout_mask,
           detail::stream_arg(data_.stream));

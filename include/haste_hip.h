@@ -37,10 +37,9 @@ const char* haste_hip_last_runtime_error(void);
 
 /* Largest hidden size whose recurrent weight slice the persistent kernels can keep
  * on chip for `gates` gate blocks (4 LSTM, 3 GRU) and `batch_size` rows on the
- * current device; 0 if none.  LSTM and GRU accept larger hidden sizes as well: they then
- * stream the recurrent matrix from HBM every step (one GEMM and one pointwise kernel per
- * step, as the reference does); the layer-norm cells return
- * HASTE_HIP_ERROR_UNSUPPORTED_SIZE beyond it. */
+ * current device; 0 if none.  Larger hidden sizes are accepted as well: the cells then
+ * stream the recurrent matrix from HBM every step (one GEMM plus row-wise norm and pointwise
+ * kernels per step, as the reference does). */
 int haste_hip_max_hidden_size(int gates, int batch_size);
 
 /* Drops this thread's cached per-stream workspaces on the current device (frees
@@ -306,6 +305,165 @@ int haste_hip_layer_norm_indrnn_backward_f32(int steps, int batch_size, int inpu
                                              const float* act_Wx, const float* gamma1,
                                              float* dgamma1,
                                              const float* zoneout_mask, void* stream);
+
+/* ---- double precision -------------------------------------------------------------
+ * The reference instantiates every class for double as well (e.g.
+ * lib/lstm_forward_gpu.cu.cc:368-369, lib/gru_forward_gpu.cu.cc:374-375,
+ * lib/layer_norm_forward_gpu.cu.cc:152-153, lib/indrnn_forward_gpu.cu.cc:212-213).  These are
+ * what haste::v0::<cell>::ForwardPass<double>::Run / BackwardPass<double>::Run (and Iterate)
+ * bind to: same arguments, shapes and semantics as the *_f32 entry points above, tensors in
+ * double; zoneout_prob and dropconnect_scale stay float as in the reference's signatures.
+ * Every step is a GEMM on the fp64 matrix cores plus row-wise / pointwise kernels, for any
+ * hidden size. */
+int haste_hip_gemm_f64(int trans_a, int M, int N, int K,
+                       const double* A, int lda, const double* B, int ldb,
+                       double* C, int ldc, int accumulate, void* stream);
+int haste_hip_transpose_f64(int rows, int cols, const double* in, double* out, void* stream);
+int haste_hip_lstm_forward_f64(int training, int steps, int batch_size, int input_size,
+                               int hidden_size,
+                               const double* W, const double* R, const double* b, const double* x,
+                               double* h, double* c, double* v, double* tmp_Rh,
+                               float zoneout_prob, const double* zoneout_mask, void* stream);
+int haste_hip_lstm_forward_dropconnect_f64(int training, int steps, int batch_size,
+                                           int input_size, int hidden_size,
+                                           const double* W, const double* R, const double* b,
+                                           const double* x, double* h, double* c, double* v,
+                                           float zoneout_prob, const double* zoneout_mask,
+                                           const double* dropconnect_mask, float dropconnect_scale,
+                                           void* stream);
+int haste_hip_lstm_backward_f64(int steps, int batch_size, int input_size, int hidden_size,
+                                const double* W_t, const double* R_t, const double* b,
+                                const double* x_t, const double* h, const double* c,
+                                const double* dh_new, const double* dc_new,
+                                double* dx, double* dW, double* dR, double* db,
+                                double* dh, double* dc, double* v,
+                                const double* zoneout_mask, void* stream);
+int haste_hip_lstm_forward_iterate_f64(int training, int batch_size, int input_size,
+                                       int hidden_size,
+                                       const double* W, const double* R, const double* b,
+                                       const double* x, const double* h, const double* c,
+                                       double* h_out, double* c_out, double* v, double* tmp_Rh,
+                                       float zoneout_prob, const double* zoneout_mask,
+                                       void* stream);
+int haste_hip_lstm_backward_iterate_f64(int batch_size, int input_size, int hidden_size,
+                                        const double* W_t, const double* R_t, const double* b,
+                                        const double* x_t, const double* h, const double* c,
+                                        const double* c_new, const double* dh_new,
+                                        const double* dc_new, double* dx, double* dW, double* dR,
+                                        double* db, double* dh, double* dc, double* v,
+                                        const double* zoneout_mask, void* stream);
+int haste_hip_gru_forward_f64(int training, int steps, int batch_size, int input_size,
+                              int hidden_size,
+                              const double* W, const double* R, const double* bx, const double* br,
+                              const double* x, double* h, double* v, double* tmp_Wx, double* tmp_Rh,
+                              float zoneout_prob, const double* zoneout_mask, void* stream);
+int haste_hip_gru_forward_dropconnect_f64(int training, int steps, int batch_size,
+                                          int input_size, int hidden_size,
+                                          const double* W, const double* R, const double* bx,
+                                          const double* br, const double* x, double* h, double* v,
+                                          double* tmp_Wx, float zoneout_prob,
+                                          const double* zoneout_mask,
+                                          const double* dropconnect_mask, float dropconnect_scale,
+                                          void* stream);
+int haste_hip_gru_backward_f64(int steps, int batch_size, int input_size, int hidden_size,
+                               const double* W_t, const double* R_t, const double* bx,
+                               const double* br, const double* x_t, const double* h, const double* v,
+                               const double* dh_new, double* dx, double* dW, double* dR,
+                               double* dbx, double* dbr, double* dh, double* dp, double* dq,
+                               const double* zoneout_mask, void* stream);
+int haste_hip_gru_forward_iterate_f64(int training, int batch_size, int input_size,
+                                      int hidden_size,
+                                      const double* W, const double* R, const double* bx,
+                                      const double* br, const double* x, const double* h,
+                                      double* h_out, double* v, double* tmp_Wx, double* tmp_Rh,
+                                      float zoneout_prob, const double* zoneout_mask,
+                                      void* stream);
+int haste_hip_gru_backward_iterate_f64(int batch_size, int input_size, int hidden_size,
+                                       const double* W_t, const double* R_t, const double* bx,
+                                       const double* br, const double* x_t, const double* h,
+                                       const double* v, const double* dh_new, double* dx, double* dW,
+                                       double* dR, double* dbx, double* dbr, double* dh, double* dp,
+                                       double* dq, const double* zoneout_mask, void* stream);
+int haste_hip_layer_norm_forward_f64(int rows, int dim, const double* gamma, const double* beta,
+                                     const double* x, double* y, double* cache, void* stream);
+int haste_hip_layer_norm_backward_f64(int rows, int dim, const double* gamma, const double* x,
+                                      const double* dy, double* dx, double* dgamma, double* dbeta,
+                                      const double* cache, void* stream);
+int haste_hip_layer_norm_lstm_forward_f64(int training, int steps, int batch_size,
+                                          int input_size, int hidden_size,
+                                          const double* W, const double* R, const double* b,
+                                          const double* x, double* h, double* c,
+                                          double* act_Wx, double* tmp_Rh,
+                                          const double* gamma1, double* cache1,
+                                          double* act_Wx_norm, double* act_Rh,
+                                          const double* gamma2, double* cache2,
+                                          const double* gamma_h, const double* beta_h, double* cache3,
+                                          double* act_c_norm,
+                                          float zoneout_prob, const double* zoneout_mask,
+                                          void* stream);
+int haste_hip_layer_norm_lstm_backward_f64(int steps, int batch_size, int input_size,
+                                           int hidden_size,
+                                           const double* W_t, const double* R_t, const double* b,
+                                           const double* x_t, const double* h, const double* c,
+                                           const double* dh_new, const double* dc_new,
+                                           double* dx, double* dW, double* dR, double* db,
+                                           double* dh, double* dc,
+                                           double* act_Wx, const double* gamma1, double* dgamma1,
+                                           double* act_Wx_norm, double* act_Rh,
+                                           const double* gamma2, double* dgamma2,
+                                           const double* cache2,
+                                           const double* gamma_h, const double* beta_h,
+                                           double* dgamma_h, double* dbeta_h,
+                                           const double* cache3,
+                                           double* act_c_norm,
+                                           const double* zoneout_mask, void* stream);
+int haste_hip_layer_norm_gru_forward_f64(int training, int steps, int batch_size,
+                                         int input_size, int hidden_size,
+                                         const double* W, const double* R, const double* bx,
+                                         const double* br, const double* x, double* h, double* v,
+                                         double* act_Wx, const double* gamma1, double* cache1,
+                                         double* tmp_Wx_norm, double* act_Rh,
+                                         const double* gamma2, double* cache2, double* tmp_Rh_norm,
+                                         float zoneout_prob, const double* zoneout_mask,
+                                         void* stream);
+int haste_hip_layer_norm_gru_backward_f64(int steps, int batch_size, int input_size,
+                                          int hidden_size,
+                                          const double* W_t, const double* R_t, const double* bx,
+                                          const double* br, const double* x_t, const double* h,
+                                          const double* v, const double* dh_new,
+                                          double* dx, double* dW, double* dR, double* dbx, double* dbr,
+                                          double* dh, double* dp, double* dq,
+                                          const double* act_Wx, const double* gamma1, double* dgamma1,
+                                          const double* act_Rh, const double* gamma2, double* dgamma2,
+                                          const double* cache2,
+                                          const double* zoneout_mask, void* stream);
+int haste_hip_indrnn_forward_f64(int training, int steps, int batch_size, int input_size,
+                                 int hidden_size,
+                                 const double* W, const double* u, const double* b, const double* x,
+                                 double* h, double* workspace,
+                                 float zoneout_prob, const double* zoneout_mask, void* stream);
+int haste_hip_indrnn_backward_f64(int steps, int batch_size, int input_size, int hidden_size,
+                                  const double* W_t, const double* u, const double* b,
+                                  const double* x_t, const double* h, const double* dh_new,
+                                  double* dx, double* dW, double* du, double* db, double* dh,
+                                  double* workspace, const double* zoneout_mask, void* stream);
+int haste_hip_layer_norm_indrnn_forward_f64(int training, int steps, int batch_size,
+                                            int input_size, int hidden_size,
+                                            const double* W, const double* u, const double* b,
+                                            const double* x, double* h, double* workspace,
+                                            double* act_Wx, const double* gamma1, double* cache1,
+                                            float zoneout_prob, const double* zoneout_mask,
+                                            void* stream);
+int haste_hip_layer_norm_indrnn_backward_f64(int steps, int batch_size, int input_size,
+                                             int hidden_size,
+                                             const double* W_t, const double* u, const double* b,
+                                             const double* x_t, const double* h,
+                                             const double* dh_new,
+                                             double* dx, double* dW, double* du, double* db, double* dh,
+                                             double* workspace,
+                                             const double* act_Wx, const double* gamma1,
+                                             double* dgamma1,
+                                             const double* zoneout_mask, void* stream);
 
 #ifdef __cplusplus
 }

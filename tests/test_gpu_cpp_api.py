@@ -14,6 +14,7 @@ pytestmark = pytest.mark.gpu
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 BIN = os.path.join(HERE, "cpp", "api_check")
+DTYPE = np.float32  # np.float64 runs the classes instantiated for double ("f64:<cell>")
 
 
 def _run(cell, T, N, C, H, zoneout, inputs, out_shapes):
@@ -23,12 +24,12 @@ def _run(cell, T, N, C, H, zoneout, inputs, out_shapes):
         fin, fout = os.path.join(d, "in.bin"), os.path.join(d, "out.bin")
         with open(fin, "wb") as f:
             for a in inputs:
-                f.write(np.ascontiguousarray(a, dtype=np.float32).tobytes())
+                f.write(np.ascontiguousarray(a, dtype=DTYPE).tobytes())
         print("api_check", cell, T, N, C, H, zoneout, flush=True)
-        res = subprocess.run([BIN, cell, str(T), str(N), str(C), str(H), str(zoneout), fin, fout],
+        res = subprocess.run([BIN, ("f64:" if DTYPE is np.float64 else "") + cell, str(T), str(N), str(C), str(H), str(zoneout), fin, fout],
                              capture_output=True, text=True, timeout=100)
         assert res.returncode == 0, res.stdout + res.stderr
-        raw = np.fromfile(fout, dtype=np.float32).astype(np.float64)
+        raw = np.fromfile(fout, dtype=DTYPE).astype(np.float64)
     outs, off = [], 0
     for shp in out_shapes:
         n = int(np.prod(shp))

@@ -41,7 +41,7 @@ def test_lstm_iterate(T, N, C, H, zoneout):
     assert relerr(host(ci), cio[-1]) < TOL
 
     W_t, R_t = W.t().contiguous(), R.t().contiguous()
-    opts = dict(device="cuda", dtype=torch.float32)
+    opts = dict(device="cuda", dtype=W.dtype)
     dW, dR, db = torch.zeros(C, 4 * H, **opts), torch.zeros(H, 4 * H, **opts), torch.zeros(4 * H, **opts)
     dh, dc = torch.zeros(N, H, **opts), torch.zeros(N, H, **opts)
     dh_new, dc_new = dev(p["dh_new"]), dev(p["dc_new"])
@@ -77,7 +77,7 @@ def test_gru_iterate(T, N, C, H, zoneout):
     assert relerr(host(torch.stack(vs)), vo) < TOL
 
     W_t, R_t = W.t().contiguous(), R.t().contiguous()
-    opts = dict(device="cuda", dtype=torch.float32)
+    opts = dict(device="cuda", dtype=W.dtype)
     dW, dR = torch.zeros(C, 3 * H, **opts), torch.zeros(H, 3 * H, **opts)
     dbx, dbr, dh = torch.zeros(3 * H, **opts), torch.zeros(3 * H, **opts), torch.zeros(N, H, **opts)
     dh_new = dev(p["dh_new"])
