@@ -26,6 +26,8 @@ namespace haste_hip {
 
 int gemm_f64(hipStream_t stream, bool trans_a, int M, int N, int K, const double* A, int lda,
              const double* B, int ldb, double* C, int ldc, bool accumulate);
+int gemm_f16(hipStream_t stream, bool trans_a, int M, int N, int K, const void* A, int lda,
+             const void* B, int ldb, void* C, int ldc, bool accumulate);
 
 namespace {
 
@@ -36,6 +38,11 @@ constexpr int kThreads = 256;
 inline dim3 blocks_for(size_t n) { return dim3((unsigned)((n + kThreads - 1) / kThreads)); }
 
 // ---- scalar math ------------------------------------------------------------------
+// Storage type T, arithmetic type Acc<T>::type: half tensors (GRU only) are computed in float.
+typedef _Float16 half_t;
+template <typename T> struct Acc { using type = T; };
+template <> struct Acc<half_t> { using type = float; };
+
 template <typename T> struct Fn;
 template <> struct Fn<float> {
   static __device__ __forceinline__ float sigmoid(float x) { return sigmoid_f(x); }
@@ -59,9 +66,14 @@ inline int gemm(hipStream_t s, bool ta, int M, int N, int K, const double* A, in
                 const double* B, int ldb, double* C, int ldc, bool acc, size_t) {
   return gemm_f64(s, ta, M, N, K, A, lda, B, ldb, C, ldc, acc);
 }
+inline int gemm(hipStream_t s, bool ta, int M, int N, int K, const half_t* A, int lda,
+                const half_t* B, int ldb, half_t* C, int ldc, bool acc, size_t) {
+  return gemm_f16(s, ta, M, N, K, A, lda, B, ldb, C, ldc, acc);
+}
 template <typename T> size_t gemm_room(int M, int N, int K);
 template <> size_t gemm_room<float>(int M, int N, int K) { return gemm_f32_scratch_bytes(M, N, K); }
 template <> size_t gemm_room<double>(int, int, int) { return 0; }
+template <> size_t gemm_room<half_t>(int, int, int) { return 0; }
 
 // Scratch of a call: buffers of its own in front, the float GEMM's partial tiles behind
 // them.  Everything is sized before the first launch so that the buffer never moves while
@@ -91,44 +103,47 @@ int open_scratch(hipStream_t stream, size_t own_bytes, size_t gemm_bytes, Scratc
 // R_eff = R * mask * scale (DropConnect), materialised once per call.
 template <typename T>
 __global__ __launch_bounds__(kThreads)
-void scale_mask_kernel(size_t n, const T* __restrict__ w, const T* __restrict__ mask, T scale,
-                       T* __restrict__ out) {
+void scale_mask_kernel(size_t n, const T* __restrict__ w, const T* __restrict__ mask,
+                       typename Acc<T>::type scale, T* __restrict__ out) {
+  using A = typename Acc<T>::type;
   const size_t i = blockIdx.x * (size_t)kThreads + threadIdx.x;
-  if (i < n) out[i] = w[i] * mask[i] * scale;
+  if (i < n) out[i] = T(A(w[i]) * A(mask[i]) * scale);
 }
 
 // Column sums over rows in two deterministic stages.  MODE 0: a[r][col]; MODE 1: the gain
 // gradient of a layer norm, (x[r][col] - mean_r) * invstd_r * a[r][col] with (mean, invstd)
 // from cache[r].  Stage one: one thread per (column, chunk of rows); stage two adds the
-// chunks in index order into out (accumulating).  With one chunk stage one adds directly.
+// chunks in index order into out (accumulating).  Sums are kept in the arithmetic type.
 template <typename T, int MODE>
 __global__ __launch_bounds__(kThreads)
 void column_partial_kernel(size_t rows, int cols, size_t rows_per_chunk, const T* __restrict__ a,
                            const T* __restrict__ x, const T* __restrict__ cache,
-                           T* __restrict__ partial, int add_into) {
+                           typename Acc<T>::type* __restrict__ partial) {
+  using A = typename Acc<T>::type;
   const int col = blockIdx.x * kThreads + threadIdx.x;
   if (col >= cols) return;
   const size_t r0 = blockIdx.y * rows_per_chunk;
   size_t r1 = r0 + rows_per_chunk;
   if (r1 > rows) r1 = rows;
-  T s = T(0);
+  A s = A(0);
   for (size_t r = r0; r < r1; ++r) {
     const size_t at = r * cols + col;
-    if (MODE == 0) s += a[at];
-    else s += (x[at] - cache[2 * r]) * cache[2 * r + 1] * a[at];
+    if (MODE == 0) s += A(a[at]);
+    else s += (A(x[at]) - A(cache[2 * r])) * A(cache[2 * r + 1]) * A(a[at]);
   }
-  T* dst = partial + (size_t)blockIdx.y * cols + col;
-  *dst = add_into ? *dst + s : s;
+  partial[(size_t)blockIdx.y * cols + col] = s;
 }
 
 template <typename T>
 __global__ __launch_bounds__(kThreads)
-void column_finish_kernel(int chunks, int cols, const T* __restrict__ partial, T* __restrict__ out) {
+void column_finish_kernel(int chunks, int cols, const typename Acc<T>::type* __restrict__ partial,
+                          T* __restrict__ out) {
+  using A = typename Acc<T>::type;
   const int col = blockIdx.x * kThreads + threadIdx.x;
   if (col >= cols) return;
-  T s = T(0);
+  A s = A(0);
   for (int k = 0; k < chunks; ++k) s += partial[(size_t)k * cols + col];
-  out[col] += s;
+  out[col] = T(A(out[col]) + s);
 }
 
 inline int column_chunks(size_t rows, size_t* rows_per_chunk) {
@@ -140,8 +155,7 @@ inline int column_chunks(size_t rows, size_t* rows_per_chunk) {
 template <typename T>
 size_t column_sum_bytes(size_t rows, int cols) {
   size_t rpc;
-  const int chunks = column_chunks(rows, &rpc);
-  return chunks > 1 ? padded((size_t)chunks * cols * sizeof(T)) : 0;
+  return padded((size_t)column_chunks(rows, &rpc) * cols * sizeof(typename Acc<T>::type));
 }
 // Room for sums over all rows of a call and over the rows of one step.
 template <typename T>
@@ -151,19 +165,15 @@ size_t column_sum_bytes(size_t all_rows, size_t step_rows, int cols) {
 }
 
 // out[col] += column sum (MODE 0) or gain gradient (MODE 1); `partial` holds
-// column_sum_bytes() bytes when more than one chunk is needed.
+// column_sum_bytes() bytes.
 template <typename T, int MODE>
 int column_sum(hipStream_t stream, size_t rows, int cols, const T* a, const T* x, const T* cache,
-               T* partial, T* out) {
+               void* partial_, T* out) {
+  typename Acc<T>::type* partial = static_cast<typename Acc<T>::type*>(partial_);
   size_t rpc;
   const int chunks = column_chunks(rows, &rpc);
   const dim3 grid((unsigned)((cols + kThreads - 1) / kThreads), (unsigned)chunks);
-  if (chunks == 1) {
-    column_partial_kernel<T, MODE><<<grid, dim3(kThreads), 0, stream>>>(rows, cols, rpc, a, x, cache, out, 1);
-    HASTE_LAUNCHED();
-    return HASTE_HIP_OK;
-  }
-  column_partial_kernel<T, MODE><<<grid, dim3(kThreads), 0, stream>>>(rows, cols, rpc, a, x, cache, partial, 0);
+  column_partial_kernel<T, MODE><<<grid, dim3(kThreads), 0, stream>>>(rows, cols, rpc, a, x, cache, partial);
   HASTE_LAUNCHED();
   column_finish_kernel<T><<<dim3(grid.x), dim3(kThreads), 0, stream>>>(chunks, cols, partial, out);
   HASTE_LAUNCHED();
@@ -269,7 +279,7 @@ int ln_forward_rows(hipStream_t stream, size_t rows, int D, const T* gamma, cons
 // `partial` as for column_sum.
 template <typename T>
 int ln_backward_rows(hipStream_t stream, size_t rows, int D, const T* gamma, const T* x,
-                     const T* dy, T* dx, T* dgamma, T* dbeta, const T* cache, T* partial) {
+                     const T* dy, T* dx, T* dgamma, T* dbeta, const T* cache, void* partial) {
   HASTE_HIP_PROPAGATE((column_sum<T, 1>(stream, rows, D, dy, x, cache, partial, dgamma)));
   if (dbeta != nullptr)
     HASTE_HIP_PROPAGATE((column_sum<T, 0>(stream, rows, D, dy, nullptr, nullptr, partial, dbeta)));
@@ -355,28 +365,29 @@ void gru_forward_pointwise(int training, int N, int H, const T* __restrict__ wx,
                            const T* __restrict__ br, const T* __restrict__ h,
                            T* __restrict__ h_out, T* __restrict__ v_t, float zoneout_prob,
                            const T* __restrict__ mask_t) {
+  using A = typename Acc<T>::type;
   const size_t idx = blockIdx.x * (size_t)kThreads + threadIdx.x;
   if (idx >= (size_t)N * H) return;
   const int n = (int)(idx / H), j = (int)(idx % H);
   const size_t g0 = (size_t)n * 3 * H + j;
-  const T z = Fn<T>::sigmoid(wx[g0] + rh[g0] + bx[j] + br[j]);
-  const T r = Fn<T>::sigmoid(wx[g0 + H] + rh[g0 + H] + bx[H + j] + br[H + j]);
-  const T qg = rh[g0 + 2 * (size_t)H] + br[2 * H + j];
-  const T g = Fn<T>::tanh_(wx[g0 + 2 * (size_t)H] + r * qg + bx[2 * H + j]);
+  const A z = Fn<A>::sigmoid(A(wx[g0]) + A(rh[g0]) + A(bx[j]) + A(br[j]));
+  const A r = Fn<A>::sigmoid(A(wx[g0 + H]) + A(rh[g0 + H]) + A(bx[H + j]) + A(br[H + j]));
+  const A qg = A(rh[g0 + 2 * (size_t)H]) + A(br[2 * H + j]);
+  const A g = Fn<A>::tanh_(A(wx[g0 + 2 * (size_t)H]) + r * qg + A(bx[2 * H + j]));
   if (training) {
     const size_t v0 = (size_t)n * 4 * H + j;
-    v_t[v0] = z;
-    v_t[v0 + H] = r;
-    v_t[v0 + 2 * (size_t)H] = g;
-    v_t[v0 + 3 * (size_t)H] = qg;
+    v_t[v0] = T(z);
+    v_t[v0 + H] = T(r);
+    v_t[v0 + 2 * (size_t)H] = T(g);
+    v_t[v0 + 3 * (size_t)H] = T(qg);
   }
-  const T h_old = h[idx];
-  T h_new = z * h_old + (T(1) - z) * g;
+  const A h_old = A(h[idx]);
+  A h_new = z * h_old + (A(1) - z) * g;
   if (zoneout_prob != 0.f && mask_t != nullptr) {
-    if (training) h_new = (h_new - h_old) * mask_t[idx] + h_old;
-    else h_new = T(zoneout_prob) * h_old + (T(1) - T(zoneout_prob)) * h_new;
+    if (training) h_new = (h_new - h_old) * A(mask_t[idx]) + h_old;
+    else h_new = A(zoneout_prob) * h_old + (A(1) - A(zoneout_prob)) * h_new;
   }
-  h_out[idx] = h_new;
+  h_out[idx] = T(h_new);
 }
 
 template <typename T>
@@ -385,35 +396,37 @@ void gru_backward_pointwise(int N, int H, const T* __restrict__ h, const T* __re
                             const T* __restrict__ dh_next, T* __restrict__ dh,
                             T* __restrict__ dp_t, T* __restrict__ dq_t,
                             const T* __restrict__ mask_t) {
+  using A = typename Acc<T>::type;
   const size_t idx = blockIdx.x * (size_t)kThreads + threadIdx.x;
   if (idx >= (size_t)N * H) return;
   const int n = (int)(idx / H), j = (int)(idx % H);
   const size_t v0 = (size_t)n * 4 * H + j, g0 = (size_t)n * 3 * H + j;
-  const T z = v_t[v0], r = v_t[v0 + H], g = v_t[v0 + 2 * (size_t)H], qg = v_t[v0 + 3 * (size_t)H];
-  T dh_total = dh_next[idx] + dh[idx];
-  T dh_keep;
+  const A z = A(v_t[v0]), r = A(v_t[v0 + H]), g = A(v_t[v0 + 2 * (size_t)H]),
+          qg = A(v_t[v0 + 3 * (size_t)H]);
+  A dh_total = A(dh_next[idx]) + A(dh[idx]);
+  A dh_keep;
   if (mask_t != nullptr) {
-    const T m = mask_t[idx];
-    dh_keep = (T(1) - m) * dh_total;
+    const A m = A(mask_t[idx]);
+    dh_keep = (A(1) - m) * dh_total;
     dh_total = m * dh_total;
     dh_keep += z * dh_total;
   } else {
     dh_keep = z * dh_total;
   }
-  const T dg = (T(1) - z) * dh_total;
-  const T dz = (h[idx] - g) * dh_total;
-  const T dp_g = d_tanh(g) * dg;
-  const T dq_g = dp_g * r;
-  const T dr = dp_g * qg;
-  const T dp_r = d_sigmoid(r) * dr;
-  const T dp_z = d_sigmoid(z) * dz;
-  dh[idx] = dh_keep;
-  dp_t[g0] = dp_z;
-  dp_t[g0 + H] = dp_r;
-  dp_t[g0 + 2 * (size_t)H] = dp_g;
-  dq_t[g0] = dp_z;
-  dq_t[g0 + H] = dp_r;
-  dq_t[g0 + 2 * (size_t)H] = dq_g;
+  const A dg = (A(1) - z) * dh_total;
+  const A dz = (A(h[idx]) - g) * dh_total;
+  const A dp_g = d_tanh(g) * dg;
+  const A dq_g = dp_g * r;
+  const A dr = dp_g * qg;
+  const A dp_r = d_sigmoid(r) * dr;
+  const A dp_z = d_sigmoid(z) * dz;
+  dh[idx] = T(dh_keep);
+  dp_t[g0] = T(dp_z);
+  dp_t[g0 + H] = T(dp_r);
+  dp_t[g0 + 2 * (size_t)H] = T(dp_g);
+  dq_t[g0] = T(dp_z);
+  dq_t[g0 + H] = T(dp_r);
+  dq_t[g0 + 2 * (size_t)H] = T(dq_g);
 }
 
 // ---- layer-norm LSTM pointwise ------------------------------------------------------------
@@ -565,7 +578,7 @@ int effective_r(hipStream_t stream, size_t n, const T* R, const T* dc_mask, floa
                 T* r_eff, const T** out) {
   *out = R;
   if (dc_mask == nullptr) return HASTE_HIP_OK;
-  scale_mask_kernel<T><<<blocks_for(n), dim3(kThreads), 0, stream>>>(n, R, dc_mask, T(dc_scale), r_eff);
+  scale_mask_kernel<T><<<blocks_for(n), dim3(kThreads), 0, stream>>>(n, R, dc_mask, typename Acc<T>::type(dc_scale), r_eff);
   HASTE_LAUNCHED();
   *out = r_eff;
   return HASTE_HIP_OK;
@@ -611,7 +624,7 @@ int lstm_backward_steps(hipStream_t stream, int steps, int N, int C, int H, cons
   room = max2(room, max2(gemm_room<T>(H, 4 * H, TN), gemm_room<T>(TN, C, 4 * H)));
   Scratch sc;
   HASTE_HIP_PROPAGATE(open_scratch(stream, own, room, &sc));
-  T* partial = sc.take<T>(own / sizeof(T));
+  void* partial = sc.take<char>(own);
   {
     ScopedKernelTimer timer("lstm_backward_steps", stream);
     for (int t = steps - 1; t >= 0; --t) {
@@ -668,7 +681,7 @@ int gru_backward_steps(hipStream_t stream, int steps, int N, int C, int H, const
   room = max2(room, max2(gemm_room<T>(H, 3 * H, TN), gemm_room<T>(TN, C, 3 * H)));
   Scratch sc;
   HASTE_HIP_PROPAGATE(open_scratch(stream, own, room, &sc));
-  T* partial = sc.take<T>(own / sizeof(T));
+  void* partial = sc.take<char>(own);
   {
     ScopedKernelTimer timer("gru_backward_steps", stream);
     for (int t = steps - 1; t >= 0; --t) {
@@ -738,7 +751,7 @@ int ln_lstm_backward_steps(hipStream_t stream, int steps, int N, int C, int H, c
   room = max2(room, max2(gemm_room<T>(H, 4 * H, TN), gemm_room<T>(TN, C, 4 * H)));
   Scratch sc;
   HASTE_HIP_PROPAGATE(open_scratch(stream, own, room, &sc));
-  T* partial = sc.take<T>(part_bytes / sizeof(T));
+  void* partial = sc.take<char>(part_bytes);
   T* stats1 = sc.take<T>((size_t)TN * 2);
   {
     ScopedKernelTimer timer("layer_norm_lstm_backward_steps", stream);
@@ -814,7 +827,7 @@ int ln_gru_backward_steps(hipStream_t stream, int steps, int N, int C, int H, co
   room = max2(room, max2(gemm_room<T>(H, 3 * H, TN), gemm_room<T>(TN, C, 3 * H)));
   Scratch sc;
   HASTE_HIP_PROPAGATE(open_scratch(stream, own, room, &sc));
-  T* partial = sc.take<T>(part_bytes / sizeof(T));
+  void* partial = sc.take<char>(part_bytes);
   T* stats1 = sc.take<T>((size_t)TN * 2);
   {
     ScopedKernelTimer timer("layer_norm_gru_backward_steps", stream);
@@ -870,7 +883,7 @@ int indrnn_backward_steps(hipStream_t stream, int steps, int N, int C, int H, co
   const size_t own = part_bytes + 2 * padded(NH * sizeof(T)) + padded((size_t)TN * 2 * sizeof(T));
   Scratch sc;
   HASTE_HIP_PROPAGATE(open_scratch(stream, own, max2(gemm_room<T>(C, H, TN), gemm_room<T>(TN, C, H)), &sc));
-  T* partial = sc.take<T>(part_bytes / sizeof(T));
+  void* partial = sc.take<char>(part_bytes);
   T* du_rows = sc.take<T>(NH);
   T* db_rows = sc.take<T>(NH);
   T* stats1 = sc.take<T>((size_t)TN * 2);
@@ -1145,7 +1158,7 @@ int haste_hip_layer_norm_backward_f64(int rows, int dim, const double* gamma, co
   const size_t part_bytes = column_sum_bytes<double>((size_t)rows, dim);
   Scratch sc;
   HASTE_HIP_PROPAGATE(open_scratch(stream, part_bytes + padded((size_t)rows * 2 * sizeof(double)), 0, &sc));
-  double* partial = sc.take<double>(part_bytes / sizeof(double));
+  void* partial = sc.take<char>(part_bytes);
   double* stats = sc.take<double>((size_t)rows * 2);
   ScopedKernelTimer timer("layer_norm_backward_f64", stream);
   HASTE_HIP_PROPAGATE(ln_forward_rows<double>(stream, (size_t)rows, dim, gamma, nullptr, x, nullptr, stats));
@@ -1286,6 +1299,89 @@ int haste_hip_layer_norm_indrnn_backward_f64(int steps, int batch_size, int inpu
   return indrnn_backward_steps<double>(as_stream(stream), steps, batch_size, input_size, hidden_size,
                                        W_t, u, x_t, h, dh_new, dx, dW, du, db, dh, workspace, act_Wx,
                                        gamma1, dgamma1, zoneout_mask);
+}
+
+// ---- half (GRU only, as in the reference: lib/gru_forward_gpu.cu.cc:373,
+// lib/gru_backward_gpu.cu.cc:411).  Tensors are IEEE binary16 passed as void*; products are
+// accumulated and the pointwise math is done in float, results rounded to half.
+static inline const half_t* hp(const void* p) { return static_cast<const half_t*>(p); }
+static inline half_t* hp(void* p) { return static_cast<half_t*>(p); }
+
+int haste_hip_gru_forward_f16(int training, int steps, int batch_size, int input_size,
+                              int hidden_size, const void* W, const void* R, const void* bx,
+                              const void* br, const void* x, void* h, void* v, void* tmp_Wx,
+                              void* tmp_Rh, float zoneout_prob, const void* zoneout_mask,
+                              void* stream) {
+  (void)tmp_Rh;
+  HASTE_HIP_REQUIRE(steps > 0 && batch_size > 0 && input_size > 0 && hidden_size > 0);
+  HASTE_HIP_REQUIRE(W && R && bx && br && x && h && tmp_Wx && (v || !training));
+  const size_t NH = (size_t)batch_size * hidden_size;
+  return gru_forward_steps<half_t>(as_stream(stream), training, steps, batch_size, input_size,
+                                   hidden_size, hp(W), hp(R), hp(bx), hp(br), hp(x), hp(h),
+                                   hp(h) + NH, hp(v), hp(tmp_Wx), zoneout_prob, hp(zoneout_mask),
+                                   nullptr, 1.f);
+}
+
+int haste_hip_gru_forward_dropconnect_f16(int training, int steps, int batch_size, int input_size,
+                                          int hidden_size, const void* W, const void* R,
+                                          const void* bx, const void* br, const void* x, void* h,
+                                          void* v, void* tmp_Wx, float zoneout_prob,
+                                          const void* zoneout_mask, const void* dropconnect_mask,
+                                          float dropconnect_scale, void* stream) {
+  HASTE_HIP_REQUIRE(steps > 0 && batch_size > 0 && input_size > 0 && hidden_size > 0);
+  HASTE_HIP_REQUIRE(W && R && bx && br && x && h && tmp_Wx && (v || !training));
+  const size_t NH = (size_t)batch_size * hidden_size;
+  return gru_forward_steps<half_t>(as_stream(stream), training, steps, batch_size, input_size,
+                                   hidden_size, hp(W), hp(R), hp(bx), hp(br), hp(x), hp(h),
+                                   hp(h) + NH, hp(v), hp(tmp_Wx), zoneout_prob, hp(zoneout_mask),
+                                   hp(dropconnect_mask), dropconnect_scale);
+}
+
+int haste_hip_gru_backward_f16(int steps, int batch_size, int input_size, int hidden_size,
+                               const void* W_t, const void* R_t, const void* bx, const void* br,
+                               const void* x_t, const void* h, const void* v, const void* dh_new,
+                               void* dx, void* dW, void* dR, void* dbx, void* dbr, void* dh, void* dp,
+                               void* dq, const void* zoneout_mask, void* stream) {
+  (void)bx;
+  (void)br;
+  HASTE_HIP_REQUIRE(steps > 0 && batch_size > 0 && input_size > 0 && hidden_size > 0);
+  HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && v && dh_new);
+  HASTE_HIP_REQUIRE(dx && dW && dR && dbx && dbr && dh && dp && dq);
+  const size_t NH = (size_t)batch_size * hidden_size;
+  return gru_backward_steps<half_t>(as_stream(stream), steps, batch_size, input_size, hidden_size,
+                                    hp(W_t), hp(R_t), hp(x_t), hp(h), hp(v), hp(dh_new) + NH, hp(dx),
+                                    hp(dW), hp(dR), hp(dbx), hp(dbr), hp(dh), hp(dp), hp(dq),
+                                    hp(zoneout_mask));
+}
+
+int haste_hip_gru_forward_iterate_f16(int training, int batch_size, int input_size, int hidden_size,
+                                      const void* W, const void* R, const void* bx, const void* br,
+                                      const void* x, const void* h, void* h_out, void* v,
+                                      void* tmp_Wx, void* tmp_Rh, float zoneout_prob,
+                                      const void* zoneout_mask, void* stream) {
+  (void)tmp_Rh;
+  HASTE_HIP_REQUIRE(batch_size > 0 && input_size > 0 && hidden_size > 0);
+  HASTE_HIP_REQUIRE(W && R && bx && br && x && h && h_out && tmp_Wx && (v || !training));
+  return gru_forward_steps<half_t>(as_stream(stream), training, 1, batch_size, input_size,
+                                   hidden_size, hp(W), hp(R), hp(bx), hp(br), hp(x), hp(h), hp(h_out),
+                                   hp(v), hp(tmp_Wx), zoneout_prob, hp(zoneout_mask), nullptr, 1.f);
+}
+
+int haste_hip_gru_backward_iterate_f16(int batch_size, int input_size, int hidden_size,
+                                       const void* W_t, const void* R_t, const void* bx,
+                                       const void* br, const void* x_t, const void* h, const void* v,
+                                       const void* dh_new, void* dx, void* dW, void* dR, void* dbx,
+                                       void* dbr, void* dh, void* dp, void* dq,
+                                       const void* zoneout_mask, void* stream) {
+  (void)bx;
+  (void)br;
+  HASTE_HIP_REQUIRE(batch_size > 0 && input_size > 0 && hidden_size > 0);
+  HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && v && dh_new);
+  HASTE_HIP_REQUIRE(dx && dW && dR && dbx && dbr && dh && dp && dq);
+  return gru_backward_steps<half_t>(as_stream(stream), 1, batch_size, input_size, hidden_size,
+                                    hp(W_t), hp(R_t), hp(x_t), hp(h), hp(v), hp(dh_new), hp(dx),
+                                    hp(dW), hp(dR), hp(dbx), hp(dbr), hp(dh), hp(dp), hp(dq),
+                                    hp(zoneout_mask));
 }
 
 }  // extern "C"

@@ -61,3 +61,9 @@ extern "C" int haste_hip_transpose_f64(int rows, int cols, const double* in, dou
                                        void* stream) {
   return haste_hip::transpose("transpose_f64", rows, cols, in, out, haste_hip::as_stream(stream));
 }
+
+// IEEE binary16 elements, passed as void*.
+extern "C" int haste_hip_transpose_f16(int rows, int cols, const void* in, void* out, void* stream) {
+  return haste_hip::transpose("transpose_f16", rows, cols, static_cast<const _Float16*>(in),
+                              static_cast<_Float16*>(out), haste_hip::as_stream(stream));
+}

@@ -254,9 +254,9 @@ class _RNNBase(nn.Module):
         if not all(t.is_cuda for t in tensors):
             raise RuntimeError(
                 "%s: parameters and input must be GPU tensors; haste_amd has no CPU path" % self._name)
-        if x.dtype not in (torch.float32, torch.float64) or any(t.dtype != x.dtype for t in tensors):
+        if x.dtype not in (torch.float32, torch.float64, torch.float16) or any(t.dtype != x.dtype for t in tensors):
             raise RuntimeError(
-                "%s: parameters and input must all be float32 or all float64" % self._name)
+                "%s: parameters and input must all have one dtype: float32, float64 or (GRU) float16" % self._name)
 
 
 def _init_gates(kernel, recurrent_kernel, hidden_size, gates):

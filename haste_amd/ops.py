@@ -2,7 +2,7 @@
 (`haste_pytorch_lib.<cell>_forward / <cell>_backward`, reference
 frameworks/pytorch/{lstm,gru,indrnn,layer_norm_lstm,layer_norm_gru,layer_norm_indrnn}.cc),
 with the same argument order, allocation protocol and return tuples, implemented by
-calls into libhaste_hip.so.  Tensors are float32 or float64 (all tensors of a call alike),
+calls into libhaste_hip.so.  Tensors are float32 or float64, for the GRU also float16 (all tensors of a call alike),
 contiguous, on the GPU; torch is used only to allocate device memory and to name the
 current stream.
 """
@@ -19,10 +19,10 @@ def _check(*tensors):
         if not t.is_contiguous():
             raise ValueError("tensor must be contiguous")
         if t.numel() and t.dtype not in _SUFFIX:
-            raise ValueError("only float32 and float64 are implemented")
+            raise ValueError("only float32, float64 and (GRU) float16 are implemented")
 
 
-_SUFFIX = {torch.float32: "_f32", torch.float64: "_f64"}
+_SUFFIX = {torch.float32: "_f32", torch.float64: "_f64", torch.float16: "_f16"}
 
 
 def _call(entry, *args):
@@ -32,7 +32,11 @@ def _call(entry, *args):
     dtypes = {a.dtype for a in args if isinstance(a, torch.Tensor) and a.numel()}
     if len(dtypes) != 1:
         raise ValueError("all tensors of a call must have the same dtype, got %s" % sorted(map(str, dtypes)))
-    lib.call(entry + _SUFFIX[dtypes.pop()], *args)
+    name = entry + _SUFFIX[dtypes.pop()]
+    if not hasattr(lib.load(), name):
+        # as in the reference, half exists for the GRU only (lib/gru_forward_gpu.cu.cc:373)
+        raise ValueError("%s is not implemented" % name)
+    lib.call(name, *args)
 
 
 def _mask_or_none(has_zoneout, zoneout_mask):

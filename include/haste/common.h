@@ -2,6 +2,7 @@
 #pragma once
 
 #include <hip/hip_runtime_api.h>
+#include <hip/hip_fp16.h>
 
 #if __has_include(<hipblas/hipblas.h>)
 #include <hipblas/hipblas.h>
@@ -30,7 +31,8 @@ inline void* stream_arg(hipStream_t s) { return reinterpret_cast<void*>(s); }
 
 // The C entry points behind a class instantiated for T.  As in the reference, only the
 // types the library is built for can be used (float and double, e.g.
-// lib/lstm_forward_gpu.cu.cc:368-369); any other T fails to compile here.
+// lib/lstm_forward_gpu.cu.cc:368-369, and __half for the GRU, lib/gru_forward_gpu.cu.cc:373);
+// any other T fails to compile here.
 template<typename T> struct Abi;
 template<> struct Abi<float> {
   static constexpr auto lstm_forward = &haste_hip_lstm_forward_f32;
@@ -71,6 +73,13 @@ template<> struct Abi<double> {
   static constexpr auto indrnn_backward = &haste_hip_indrnn_backward_f64;
   static constexpr auto layer_norm_indrnn_forward = &haste_hip_layer_norm_indrnn_forward_f64;
   static constexpr auto layer_norm_indrnn_backward = &haste_hip_layer_norm_indrnn_backward_f64;
+};
+
+template<> struct Abi<__half> {
+  static constexpr auto gru_forward = &haste_hip_gru_forward_f16;
+  static constexpr auto gru_backward = &haste_hip_gru_backward_f16;
+  static constexpr auto gru_forward_iterate = &haste_hip_gru_forward_iterate_f16;
+  static constexpr auto gru_backward_iterate = &haste_hip_gru_backward_iterate_f16;
 };
 
 }  // namespace detail

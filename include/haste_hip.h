@@ -465,6 +465,44 @@ int haste_hip_layer_norm_indrnn_backward_f64(int steps, int batch_size, int inpu
                                              double* dgamma1,
                                              const double* zoneout_mask, void* stream);
 
+/* ---- half precision (GRU only) ------------------------------------------------------
+ * The reference instantiates gru::ForwardPass / BackwardPass for half as well
+ * (lib/gru_forward_gpu.cu.cc:373, lib/gru_backward_gpu.cu.cc:411).  Same arguments, shapes and
+ * semantics as the GRU *_f32 entry points; every tensor holds IEEE binary16 values and is
+ * passed as void* (C has no portable half type).  Products are accumulated in fp32 on the
+ * matrix cores and the pointwise math is done in float; results are rounded to half, so
+ * accumulated outputs (dh over the steps, dW, dR, dbx, dbr) carry half rounding per update. */
+int haste_hip_gemm_f16(int trans_a, int M, int N, int K, const void* A, int lda, const void* B,
+                       int ldb, void* C, int ldc, int accumulate, void* stream);
+int haste_hip_transpose_f16(int rows, int cols, const void* in, void* out, void* stream);
+int haste_hip_gru_forward_f16(int training, int steps, int batch_size, int input_size,
+                              int hidden_size, const void* W, const void* R, const void* bx,
+                              const void* br, const void* x, void* h, void* v, void* tmp_Wx,
+                              void* tmp_Rh, float zoneout_prob, const void* zoneout_mask,
+                              void* stream);
+int haste_hip_gru_forward_dropconnect_f16(int training, int steps, int batch_size, int input_size,
+                                          int hidden_size, const void* W, const void* R,
+                                          const void* bx, const void* br, const void* x, void* h,
+                                          void* v, void* tmp_Wx, float zoneout_prob,
+                                          const void* zoneout_mask, const void* dropconnect_mask,
+                                          float dropconnect_scale, void* stream);
+int haste_hip_gru_backward_f16(int steps, int batch_size, int input_size, int hidden_size,
+                               const void* W_t, const void* R_t, const void* bx, const void* br,
+                               const void* x_t, const void* h, const void* v, const void* dh_new,
+                               void* dx, void* dW, void* dR, void* dbx, void* dbr, void* dh, void* dp,
+                               void* dq, const void* zoneout_mask, void* stream);
+int haste_hip_gru_forward_iterate_f16(int training, int batch_size, int input_size, int hidden_size,
+                                      const void* W, const void* R, const void* bx, const void* br,
+                                      const void* x, const void* h, void* h_out, void* v,
+                                      void* tmp_Wx, void* tmp_Rh, float zoneout_prob,
+                                      const void* zoneout_mask, void* stream);
+int haste_hip_gru_backward_iterate_f16(int batch_size, int input_size, int hidden_size,
+                                       const void* W_t, const void* R_t, const void* bx,
+                                       const void* br, const void* x_t, const void* h, const void* v,
+                                       const void* dh_new, void* dx, void* dW, void* dR, void* dbx,
+                                       void* dbr, void* dh, void* dp, void* dq,
+                                       const void* zoneout_mask, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -84,6 +84,11 @@ static void require_ok(int status, const char* what) {
   }
 }
 
+// The GRU classes also exist for half, as in the reference (lib/gru_forward_gpu.cu.cc:373):
+// instantiating every member checks that they bind to the *_f16 entry points.
+template class haste::v0::gru::ForwardPass<__half>;
+template class haste::v0::gru::BackwardPass<__half>;
+
 // The problem in precision S (the files hold S as well).
 template <typename S>
 static int run(const std::string& cell, int T, int N, int C, int H, float zoneout) {

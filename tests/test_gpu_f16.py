@@ -1,0 +1,102 @@
+"""The half-precision GRU (haste_hip_gru_*_f16, what gru::ForwardPass<__half> /
+BackwardPass<__half> bind to) against the fp64 oracle on half-representable inputs.
+
+Tolerance 2e-2 (max-norm relative, per tensor): every stored tensor is rounded to half
+(2^-11 relative) and the states / carried gradients are rounded once per step; products are
+accumulated in fp32.  The reference's own half instantiation computes in half throughout."""
+import numpy as np
+import pytest
+
+from oracle import haste_oracle as O
+from util import host, problem, relerr
+
+pytestmark = pytest.mark.gpu
+
+TOL16 = 2e-2
+SHAPES = [(3, 2, 3, 4), (4, 5, 7, 20), (6, 16, 32, 64), (8, 33, 48, 128), (3, 70, 24, 300)]
+
+
+def dev16(a):
+    import torch
+    if a is None:
+        return torch.empty(0, 0, 0, dtype=torch.float16, device="cuda")
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float16)).cuda()
+
+
+def half_problem(seed, T, N, C, H, zoneout):
+    p = problem(seed, T, N, C, H, 3, zoneout)
+    return {k: (v.astype(np.float16).astype(np.float64) if v is not None else None) for k, v in p.items()}
+
+
+@pytest.mark.parametrize("zoneout", [0.0, 0.3])
+@pytest.mark.parametrize("T,N,C,H", SHAPES)
+def test_f16_gru_training_forward_backward(T, N, C, H, zoneout):
+    from haste_amd import ops
+    import torch
+    print("gru f16", T, N, C, H, zoneout, flush=True)
+    p = half_problem(900 + T + N + C + H, T, N, C, H, zoneout)
+    mask = dev16(p["mask"])
+    h, cache = ops.gru_forward(True, zoneout, dev16(p["x"]), dev16(p["h0"]), dev16(p["W"]), dev16(p["R"]),
+                               dev16(p["b"]), dev16(p["b2"]), mask)
+    torch.cuda.synchronize()
+    assert h.dtype == torch.float16 and cache.dtype == torch.float16
+    ho, vo = O.gru_forward(p["W"], p["R"], p["b"], p["b2"], p["x"], p["h0"], True, zoneout, p["mask"])
+    assert relerr(host(h), ho) < TOL16
+    assert relerr(host(cache), vo) < TOL16
+    grads = ops.gru_backward(ops.transpose(dev16(p["x"])), ops.transpose(dev16(p["W"])),
+                             ops.transpose(dev16(p["R"])), dev16(p["b"]), dev16(p["b2"]), mask, h, cache,
+                             dev16(p["dh_new"]))
+    torch.cuda.synchronize()
+    # the oracle's backward from the GPU's own (half) activations: what the kernels were given
+    ref = O.gru_backward(p["W"], p["R"], p["b"], p["b2"], p["x"], host(h), host(cache), p["dh_new"], p["mask"])
+    for name, ours, theirs in zip(("dx", "dh0", "dW", "dR", "dbx", "dbr"), grads,
+                                  (ref[0], ref[5], ref[1], ref[2], ref[3], ref[4])):
+        assert ours.dtype == torch.float16
+        assert relerr(host(ours), theirs) < TOL16, name
+
+
+def test_f16_gru_inference_and_iterate():
+    from haste_amd import ops
+    import torch
+    T, N, C, H = 6, 9, 16, 40
+    p = half_problem(17, T, N, C, H, 0.25)
+    W, R, bx, br, x = (dev16(p[k]) for k in ("W", "R", "b", "b2", "x"))
+    h, _ = ops.gru_forward(False, 0.25, x, dev16(p["h0"]), W, R, bx, br, dev16(p["mask"]))
+    ho, _ = O.gru_forward(p["W"], p["R"], p["b"], p["b2"], p["x"], p["h0"], False, 0.25, p["mask"])
+    assert relerr(host(h), ho) < TOL16
+    # one step at a time gives the same bits as all steps at once
+    hs = [dev16(p["h0"])]
+    for t in range(T):
+        h1, _ = ops.gru_forward_iterate(False, 0.25, x[t].contiguous(), hs[t], W, R, bx, br,
+                                        dev16(p["mask"])[t].contiguous())
+        hs.append(h1)
+    torch.cuda.synchronize()
+    assert torch.equal(torch.stack(hs), h)
+
+
+def test_f16_lstm_is_refused():
+    """As in the reference, half exists for the GRU only."""
+    from haste_amd import ops
+    p = {k: v for k, v in problem(1, 2, 2, 3, 4, 4).items()}
+    with pytest.raises(ValueError):
+        ops.lstm_forward(True, 0.0, dev16(p["x"]), dev16(p["h0"]), dev16(p["c0"]), dev16(p["W"]),
+                         dev16(p["R"]), dev16(p["b"]), dev16(None))
+
+
+@pytest.mark.parametrize("trans_a,M,N,K", [(False, 1, 1, 1), (False, 37, 53, 29), (False, 128, 192, 64),
+                                           (True, 70, 130, 45), (True, 5, 20, 33), (False, 300, 100, 1000)])
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_f16_gemm_and_transpose(trans_a, M, N, K, accumulate):
+    from haste_amd import ops
+    import torch
+    r = np.random.default_rng(M * 7 + N * 3 + K)
+    h16 = lambda a: a.astype(np.float16).astype(np.float64)
+    a = h16(r.standard_normal((K, M) if trans_a else (M, K)))
+    b = h16(r.standard_normal((K, N)))
+    c0 = h16(r.standard_normal((M, N)))
+    out = dev16(c0)
+    ops.gemm(dev16(a), dev16(b), out=out, trans_a=trans_a, accumulate=accumulate)
+    ref = (a.T if trans_a else a) @ b + (c0 if accumulate else 0.0)
+    assert relerr(host(out), ref) < 2e-3  # one rounding to half of an fp32-accumulated product
+    t = ops.transpose(dev16(a))
+    assert torch.equal(t, dev16(a).t().contiguous())
