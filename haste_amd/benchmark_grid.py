@@ -116,6 +116,9 @@ def main():
     ap.add_argument("--impl", choices=["haste_amd", "torch_nn"], default="haste_amd")
     ap.add_argument("--sample_size", type=int, default=10)
     ap.add_argument("--time_steps", type=int, default=50)
+    ap.add_argument("--batch_sizes", type=int, nargs="+", default=list(BATCH_SIZES))
+    ap.add_argument("--hidden_sizes", type=int, nargs="+", default=list(HIDDEN_SIZES))
+    ap.add_argument("--input_sizes", type=int, nargs="+", default=list(INPUT_SIZES))
     ap.add_argument("--compare", nargs=2, metavar=("A.csv", "B.csv"))
     args = ap.parse_args()
     if args.compare:
@@ -131,9 +134,9 @@ def main():
     print("#   Time steps: %d" % args.time_steps)
     print("#")
     print("# batch_size,hidden_size,input_size,time_ms")
-    for N in BATCH_SIZES:
-        for H in HIDDEN_SIZES:
-            for C in INPUT_SIZES:
+    for N in args.batch_sizes:
+        for H in args.hidden_sizes:
+            for C in args.input_sizes:
                 if args.impl == "haste_amd":
                     fn = haste_sample(torch, ops, args.cell, training, args.time_steps, N, C, H)
                 else:

@@ -96,8 +96,18 @@ int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
              const float* A, int lda, const float* B, int ldb,
              float* C, int ldc, bool accumulate, size_t scratch_offset = 0);
 
-// Bytes of scratch gemm_f32 uses for this shape (0 when nothing is split).
+// Bytes of scratch gemm_f32 may use for this shape (0 when nothing is split).
 size_t gemm_f32_scratch_bytes(int M, int N, int K);
+
+// The product for M <= 32 with B streamed from HBM straight into the MFMA operands
+// (gemm_skinny.hip); gemm_f32 hands such shapes over when the operands are 16-byte aligned.
+bool gemm_f32_skinny_shape(bool trans_a, int M, int N, int K);
+bool gemm_f32_skinny_applies(bool trans_a, int M, int N, int K, const float* A, int lda,
+                             const float* B, int ldb, const float* C, int ldc);
+size_t gemm_f32_skinny_scratch_bytes(int M, int N, int K);
+int gemm_f32_skinny(hipStream_t stream, int M, int N, int K, const float* A, int lda,
+                    const float* B, int ldb, float* C, int ldc, bool accumulate,
+                    size_t scratch_offset);
 
 // The cells in step-wise form, the recurrent matrix streamed from HBM every step (per-step
 // GEMM + row-wise norms + pointwise kernels): for hidden sizes whose slices of R do not fit

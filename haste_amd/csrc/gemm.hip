@@ -357,7 +357,10 @@ GemmPlan plan_gemm(int M, int N, int K) {
 
 size_t gemm_f32_scratch_bytes(int M, int N, int K) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
-  return plan_gemm(M, N, K).scratch_bytes;
+  // Which kernel runs also depends on the operands' alignment: room for either.
+  const size_t tiled = plan_gemm(M, N, K).scratch_bytes;
+  const size_t skinny = gemm_f32_skinny_shape(false, M, N, K) ? gemm_f32_skinny_scratch_bytes(M, N, K) : 0;
+  return tiled > skinny ? tiled : skinny;
 }
 
 int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
@@ -367,6 +370,8 @@ int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
   HASTE_HIP_REQUIRE(A != nullptr && B != nullptr && C != nullptr);
   HASTE_HIP_REQUIRE(lda >= (trans_a ? M : K) && ldb >= N && ldc >= N);
   HASTE_HIP_REQUIRE((long long)((M + 63) / 64) * ((N + BN - 1) / BN) < (1ll << 26));
+  if (gemm_f32_skinny_applies(trans_a, M, N, K, A, lda, B, ldb, C, ldc))
+    return gemm_f32_skinny(stream, M, N, K, A, lda, B, ldb, C, ldc, accumulate, scratch_offset);
   const GemmPlan g = plan_gemm(M, N, K);
   const int bm = g.bm, tiles_n = g.tiles_n, whole_tiles = g.whole_tiles, rest = g.rest;
   const int splits = g.splits, k_per_split = g.k_per_split, pieces = g.pieces;

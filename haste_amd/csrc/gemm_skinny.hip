@@ -1,0 +1,221 @@
+// C[M,N] (+)= A[M,K] * B[K,N] for M <= 32: the recurrent product of one step (h_t * R,
+// delta_t * R^T) when R is streamed from HBM every step (stepwise.hip) and the batch is
+// small.  Replaces the per-step cublasSgemm of the reference
+// (lib/lstm_forward_gpu.cu.cc:232-242, lib/lstm_backward_gpu.cu.cc:281-291).
+//
+// Bound: HBM.  Algorithmic bytes 4*K*N (B is read exactly once; A and C are M rows).  The
+// 128 x 128 tile kernel of gemm.hip gives such a product a handful of tiles and pushes B
+// through LDS; here B goes from HBM straight into the MFMA operand registers: a lane loads 16
+// bytes (four consecutive columns of one k row), a wavefront 1 KiB of whole 256- or 512-byte
+// row segments, and the four components feed four MFMAs whose output columns are therefore
+// interleaved by 4 -- which is exactly a 16-byte store per lane in the epilogue.  M <= 16
+// uses v_mfma_f32_16x16x4_f32 (4 k rows x 64 columns per load), M <= 32 v_mfma_f32_32x32x2_f32
+// (2 k rows x 128 columns); the matrix cores then need 128 / 256 cycles per KiB of B, below
+// the 330 cycles a CU's share of 8 TB/s allows.  The four wavefronts of a workgroup split the
+// workgroup's k range and add their tiles through LDS in wavefront order; workgroups split K
+// further (enough of them to keep every CU's memory pipeline full) and a second small kernel
+// adds their tiles in chunk order: deterministic, no atomics.
+#include "common.h"
+
+namespace haste_hip {
+namespace {
+
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+template <int MT> struct SkinnyShape;
+template <> struct SkinnyShape<16> {
+  static constexpr int kStep = 4, kCols = 64;
+  typedef float4_t Acc;
+  static __device__ __forceinline__ Acc mfma(float a, float b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+  }
+  // row of accumulator element e held by `lane`
+  static __device__ __forceinline__ int row(int lane, int e) { return 4 * (lane >> 4) + e; }
+  static constexpr int kAccElems = 4;
+};
+template <> struct SkinnyShape<32> {
+  static constexpr int kStep = 2, kCols = 128;
+  typedef float16_t Acc;
+  static __device__ __forceinline__ Acc mfma(float a, float b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ int row(int lane, int e) {
+    return 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+  }
+  static constexpr int kAccElems = 16;
+};
+
+constexpr int kUnroll = 8;  // load instructions in flight per wavefront and operand
+
+template <int MT>
+__global__ __launch_bounds__(256)
+void skinny_kernel(int M, int N, int K, const float* __restrict__ A, int lda,
+                   const float* __restrict__ B, int ldb, float* __restrict__ C, int ldc,
+                   int accumulate, int k_per_wg, float* __restrict__ partial) {
+  typedef SkinnyShape<MT> S;
+  typedef typename S::Acc Acc;
+  __shared__ __attribute__((aligned(16))) float red[3][MT][S::kCols];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n0 = blockIdx.x * S::kCols;
+  const int chunk = blockIdx.y;
+  const int kb_wg = chunk * k_per_wg;
+  const int ke_wg = kb_wg + k_per_wg < K ? kb_wg + k_per_wg : K;
+  const int k_per_wave = ((k_per_wg + 3) / 4 + 7) / 8 * 8;
+  const int kb = kb_wg + wave * k_per_wave;
+  const int ke = kb + k_per_wave < ke_wg ? kb + k_per_wave : ke_wg;
+
+  const int i = lane % MT, kq = lane / MT;
+  const int col = n0 + 4 * (lane % MT);
+  const bool col_ok = col < N, row_ok = i < M;
+  // Out-of-range lanes load from a valid address and drop the value.
+  const float* ap = A + (size_t)(row_ok ? i : 0) * lda;
+  const float* bp = B + (col_ok ? col : 0);
+
+  Acc acc[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+#pragma unroll
+    for (int e = 0; e < S::kAccElems; ++e) acc[c][e] = 0.f;
+
+  // A batch is kUnroll MFMA steps.  Which k a lane contributes at which step is free as long
+  // as both operands agree: lane group kq takes the run of kUnroll consecutive k starting at
+  // k + kUnroll*kq, one per step, so its A values are two 16-byte loads of consecutive k and
+  // every B load instruction still covers whole row segments.
+  for (int k = kb; k < ke; k += S::kStep * kUnroll) {
+    const int k_mine = k + kUnroll * kq;
+    float4_t b[kUnroll];
+    float4_t a4[kUnroll / 4];
+#pragma unroll
+    for (int j = 0; j < kUnroll / 4; ++j) {
+      const int g = k_mine + 4 * j;
+      const bool ok = g < ke;
+      const float4_t av = *reinterpret_cast<const float4_t*>(ap + (ok ? g : kb));
+      a4[j] = (ok && row_ok) ? av : float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int r = k_mine + u;
+      const bool ok = r < ke;
+      const float4_t bv = *reinterpret_cast<const float4_t*>(bp + (size_t)(ok ? r : kb) * ldb);
+      b[u] = (ok && col_ok) ? bv : float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const float a = a4[u / 4][u % 4];
+      acc[0] = S::mfma(a, b[u].x, acc[0]);
+      acc[1] = S::mfma(a, b[u].y, acc[1]);
+      acc[2] = S::mfma(a, b[u].z, acc[2]);
+      acc[3] = S::mfma(a, b[u].w, acc[3]);
+    }
+  }
+
+  // Element e of the four accumulators = four consecutive columns of one row.
+  const int cslot = 4 * (lane % MT);
+  if (wave > 0) {
+#pragma unroll
+    for (int e = 0; e < S::kAccElems; ++e)
+      *reinterpret_cast<float4_t*>(&red[wave - 1][S::row(lane, e)][cslot]) =
+          float4_t{acc[0][e], acc[1][e], acc[2][e], acc[3][e]};
+  }
+  __syncthreads();
+  if (wave > 0 || !col_ok) return;
+#pragma unroll
+  for (int e = 0; e < S::kAccElems; ++e) {
+    const int row = S::row(lane, e);
+    if (row >= M) continue;
+    float4_t s = float4_t{acc[0][e], acc[1][e], acc[2][e], acc[3][e]};
+    s += *reinterpret_cast<const float4_t*>(&red[0][row][cslot]);
+    s += *reinterpret_cast<const float4_t*>(&red[1][row][cslot]);
+    s += *reinterpret_cast<const float4_t*>(&red[2][row][cslot]);
+    if (partial != nullptr) {
+      *reinterpret_cast<float4_t*>(partial + ((size_t)chunk * M + row) * N + col) = s;
+    } else {
+      float4_t* o = reinterpret_cast<float4_t*>(C + (size_t)row * ldc + col);
+      *o = accumulate ? (*o + s) : s;
+    }
+  }
+}
+
+// C (+)= sum over chunks of partial[chunk][M][N], chunks added in index order.
+__global__ __launch_bounds__(256)
+void skinny_reduce_kernel(int M, int N, int chunks, const float* __restrict__ partial,
+                          float* __restrict__ C, int ldc, int accumulate) {
+  const size_t q = blockIdx.x * (size_t)256 + threadIdx.x;  // index of a group of 4 columns
+  const size_t per_row = (size_t)N / 4;
+  if (q >= per_row * M) return;
+  const size_t row = q / per_row, col = (q % per_row) * 4;
+  float4_t s = float4_t{0.f, 0.f, 0.f, 0.f};
+  for (int k = 0; k < chunks; ++k)
+    s += *reinterpret_cast<const float4_t*>(partial + ((size_t)k * M + row) * N + col);
+  float4_t* o = reinterpret_cast<float4_t*>(C + row * ldc + col);
+  *o = accumulate ? (*o + s) : s;
+}
+
+struct SkinnyPlan {
+  int mt, col_blocks, chunks, k_per_wg;
+};
+
+SkinnyPlan plan_skinny(int M, int N, int K) {
+  SkinnyPlan p;
+  p.mt = M <= 16 ? 16 : 32;
+  const int cols = 4 * p.mt;
+  p.col_blocks = (N + cols - 1) / cols;
+  // Enough workgroups for about four per CU, a workgroup keeping at least 128 of K.
+  const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
+  int chunks = (4 * cus + p.col_blocks - 1) / p.col_blocks;
+  const int most = (K + 127) / 128;
+  if (chunks > most) chunks = most;
+  if (chunks < 1) chunks = 1;
+  p.k_per_wg = (K + chunks - 1) / chunks;
+  p.k_per_wg = (p.k_per_wg + 31) / 32 * 32;  // four wavefronts x a multiple of 8
+  p.chunks = (K + p.k_per_wg - 1) / p.k_per_wg;
+  return p;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace
+
+bool gemm_f32_skinny_shape(bool trans_a, int M, int N, int K) {
+  return !trans_a && M <= 32 && N % 4 == 0 && K % 4 == 0 && K >= 64 && (long long)K * N >= (1ll << 16);
+}
+
+size_t gemm_f32_skinny_scratch_bytes(int M, int N, int K) {
+  const SkinnyPlan p = plan_skinny(M, N, K);
+  return p.chunks > 1 ? (size_t)p.chunks * M * N * sizeof(float) : 0;
+}
+
+bool gemm_f32_skinny_applies(bool trans_a, int M, int N, int K, const float* A, int lda,
+                             const float* B, int ldb, const float* C, int ldc) {
+  return gemm_f32_skinny_shape(trans_a, M, N, K) && lda % 4 == 0 && ldb % 4 == 0 && ldc % 4 == 0 &&
+         aligned16(A) && aligned16(B) && aligned16(C);
+}
+
+int gemm_f32_skinny(hipStream_t stream, int M, int N, int K, const float* A, int lda,
+                    const float* B, int ldb, float* C, int ldc, bool accumulate,
+                    size_t scratch_offset) {
+  const SkinnyPlan p = plan_skinny(M, N, K);
+  float* partial = nullptr;
+  if (p.chunks > 1) {
+    Workspace ws;
+    HASTE_HIP_PROPAGATE(get_workspace(stream, scratch_offset + gemm_f32_skinny_scratch_bytes(M, N, K), &ws));
+    partial = ws.scratch + scratch_offset / sizeof(float);
+  }
+  const dim3 grid((unsigned)p.col_blocks, (unsigned)p.chunks);
+  ScopedKernelTimer timer("gemm_f32_skinny", stream);
+  if (p.mt == 16)
+    skinny_kernel<16><<<grid, dim3(256), 0, stream>>>(M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, p.k_per_wg, partial);
+  else
+    skinny_kernel<32><<<grid, dim3(256), 0, stream>>>(M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, p.k_per_wg, partial);
+  HASTE_HIP_TRY(hipGetLastError());
+  if (partial != nullptr) {
+    const size_t groups = (size_t)M * (N / 4);
+    skinny_reduce_kernel<<<dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, stream>>>(
+        M, N, p.chunks, partial, C, ldc, accumulate ? 1 : 0);
+    HASTE_HIP_TRY(hipGetLastError());
+  }
+  return HASTE_HIP_OK;
+}
+
+}  // namespace haste_hip
