@@ -23,8 +23,11 @@ PEAK_HBM_GBS = 8000.0
 # WRITE_SIZE) scaled by what the same counters read for a 1 GiB device copy (--workload copy):
 # one FETCH_SIZE unit = 2.000 KiB, one WRITE_SIZE unit = 1.000 KiB.  A GEMM "launch" is the mean
 # of the step's four products, each with its split reduce.
-MEASURED_TRAFFIC_BYTES = {"gemm_f32": 208.3e6, "lstm_forward_recurrence": 166.8e6,
-                          "lstm_backward_recurrence": 183.0e6}
+MEASURED_TRAFFIC_BYTES = {"gemm_f32": 205.6e6, "lstm_forward_recurrence": 166.8e6,
+                          "lstm_backward_recurrence": 183.0e6,
+                          # at N=1 C=512 H=4096 (--workload stepwise): 131168.5 FETCH_SIZE units
+                          # + 256 WRITE_SIZE units per launch of the streaming kernel
+                          "gemm_f32_skinny": 268.9e6}
 
 
 def parse():
@@ -34,7 +37,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget", type=float, default=15.0)
-    ap.add_argument("--workload", choices=["all", "metric", "streaming", "copy", "configs"], default="all",
+    ap.add_argument("--workload", choices=["all", "metric", "streaming", "stepwise", "copy", "configs"], default="all",
                     help="restrict the run to one workload (for profiling); the JSON line is "
                          "only complete with 'all'.  'copy' runs a plain device copy of known "
                          "size, the yardstick for the FETCH_SIZE / WRITE_SIZE counters")
@@ -175,6 +178,53 @@ def run_streaming(args, torch, lib, ops, dev):
     return out, (W1, R1, b1, x1)
 
 
+def run_stepwise(args, torch, lib, ops, dev):
+    """LSTM inference N=1 T=50 C=512 H=4096 (the largest hidden size of the reference's
+    benchmark grid): R does not fit on chip and is streamed from HBM by every step's product."""
+    T, N, C, H = 50, 1, 512, 4096
+    g = torch.Generator(device="cpu").manual_seed(2)
+    k = H ** -0.5
+    W = ((torch.rand(C, 4 * H, generator=g) * 2 - 1) * k).to(dev)
+    R = ((torch.rand(H, 4 * H, generator=g) * 2 - 1) * k).to(dev)
+    b = torch.zeros(4 * H, device=dev)
+    x = torch.randn(T, N, C, generator=g).to(dev)
+    h0, c0 = torch.zeros(N, H, device=dev), torch.zeros(N, H, device=dev)
+    no_mask = torch.empty(0, 0, 0, device=dev)
+
+    def step():
+        return ops.lstm_forward(False, 0.0, x, h0, c0, W, R, b, no_mask)
+
+    for _ in range(3):
+        step()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    reps = 10
+    ev0.record()
+    for _ in range(reps):
+        step()
+    ev1.record()
+    torch.cuda.synchronize()
+    us_total = ev0.elapsed_time(ev1) * 1e3 / reps / T
+    # again with per-kernel event timing switched on in the library
+    lib.haste_hip_profile_reset()
+    lib.haste_hip_profile_enable(1)
+    for _ in range(reps):
+        step()
+    torch.cuda.synchronize()
+    lib.haste_hip_profile_enable(0)
+    ms, n = profile_read(lib, "gemm_f32_skinny")
+    lib.haste_hip_profile_reset()
+    us_product = ms * 1e3 / max(n, 1)
+    b_product = 4.0 * H * 4 * H  # R, read once per step
+    gbs = b_product / (us_product * 1e-6) / 1e9
+    return {"workload": "LSTM inference N=1 T=50 C=512 H=4096 fp32",
+            "us_per_timestep": round(us_total, 3),
+            "roofline": {"kernel": "gemm_f32_skinny", "bound": "hbm", "achieved": round(gbs, 1),
+                         "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4),
+                         "us_per_launch": round(us_product, 2), "bytes_per_launch": b_product,
+                         "traffic": MEASURED_TRAFFIC_BYTES.get("gemm_f32_skinny")}}
+
+
 def run_configs(args, torch, lib, ops, dev):
     """The other BASELINE.json configurations (parity-test cases; timed here for the record):
     forward (+ backward with the caller-side transposes) in ms per call."""
@@ -289,9 +339,13 @@ def main():
         s, _ = run_streaming(args, torch, lib, ops, dev)
         print(json.dumps(s))
         return
+    if args.workload == "stepwise":
+        print(json.dumps(run_stepwise(args, torch, lib, ops, dev)))
+        return
 
     m = run_metric(args, torch, lib, ops, dev)
     streaming, host1 = run_streaming(args, torch, lib, ops, dev)
+    stepwise = run_stepwise(args, torch, lib, ops, dev)
 
     # CPU baseline: torch.nn.LSTM fwd+bwd on the host cores (bounded sample).
     cpu = None
@@ -321,6 +375,7 @@ def main():
         "roofline": m["roofline"],
         "kernels": m["kernels"],
         "streaming_n1": streaming,
+        "stepwise_n1_h4096": stepwise,
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))

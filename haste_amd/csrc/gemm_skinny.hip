@@ -203,13 +203,16 @@ int gemm_f32_skinny(hipStream_t stream, int M, int N, int K, const float* A, int
     partial = ws.scratch + scratch_offset / sizeof(float);
   }
   const dim3 grid((unsigned)p.col_blocks, (unsigned)p.chunks);
-  ScopedKernelTimer timer("gemm_f32_skinny", stream);
-  if (p.mt == 16)
-    skinny_kernel<16><<<grid, dim3(256), 0, stream>>>(M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, p.k_per_wg, partial);
-  else
-    skinny_kernel<32><<<grid, dim3(256), 0, stream>>>(M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, p.k_per_wg, partial);
-  HASTE_HIP_TRY(hipGetLastError());
+  {
+    ScopedKernelTimer timer("gemm_f32_skinny", stream);
+    if (p.mt == 16)
+      skinny_kernel<16><<<grid, dim3(256), 0, stream>>>(M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, p.k_per_wg, partial);
+    else
+      skinny_kernel<32><<<grid, dim3(256), 0, stream>>>(M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, p.k_per_wg, partial);
+    HASTE_HIP_TRY(hipGetLastError());
+  }
   if (partial != nullptr) {
+    ScopedKernelTimer timer("gemm_f32_skinny_reduce", stream);
     const size_t groups = (size_t)M * (N / 4);
     skinny_reduce_kernel<<<dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, stream>>>(
         M, N, p.chunks, partial, C, ldc, accumulate ? 1 : 0);
