@@ -108,6 +108,9 @@ size_t gemm_f32_skinny_scratch_bytes(int M, int N, int K);
 int gemm_f32_skinny(hipStream_t stream, int M, int N, int K, const float* A, int lda,
                     const float* B, int ldb, float* C, int ldc, bool accumulate,
                     size_t scratch_offset);
+int gemm_f32_skinny_chunks(hipStream_t stream, int M, int N, int K, const float* A, int lda,
+                           const float* B, int ldb, size_t scratch_offset, const float** partial,
+                           int* chunks);
 
 // The cells in step-wise form, the recurrent matrix streamed from HBM every step (per-step
 // GEMM + row-wise norms + pointwise kernels): for hidden sizes whose slices of R do not fit

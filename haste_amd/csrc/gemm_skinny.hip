@@ -13,8 +13,9 @@
 // (2 k rows x 128 columns); the matrix cores then need 128 / 256 cycles per KiB of B, below
 // the 330 cycles a CU's share of 8 TB/s allows.  The four wavefronts of a workgroup split the
 // workgroup's k range and add their tiles through LDS in wavefront order; workgroups split K
-// further (enough of them to keep every CU's memory pipeline full) and a second small kernel
-// adds their tiles in chunk order: deterministic, no atomics.
+// further (enough of them to keep every CU's memory pipeline full); their tiles are added in
+// chunk order by a second small kernel, or by the consumer of the product itself
+// (gemm_f32_skinny_chunks): deterministic, no atomics.
 #include "common.h"
 
 namespace haste_hip {
@@ -161,9 +162,10 @@ SkinnyPlan plan_skinny(int M, int N, int K) {
   p.mt = M <= 16 ? 16 : 32;
   const int cols = 4 * p.mt;
   p.col_blocks = (N + cols - 1) / cols;
-  // Enough workgroups for about four per CU, a workgroup keeping at least 128 of K.
+  // Enough workgroups for about three per CU (measured: four is no faster at 268 MB of B and
+  // slower when B fits the memory-side cache), a workgroup keeping at least 128 of K.
   const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
-  int chunks = (4 * cus + p.col_blocks - 1) / p.col_blocks;
+  int chunks = (3 * cus + p.col_blocks - 1) / p.col_blocks;
   const int most = (K + 127) / 128;
   if (chunks > most) chunks = most;
   if (chunks < 1) chunks = 1;
@@ -182,14 +184,35 @@ bool gemm_f32_skinny_shape(bool trans_a, int M, int N, int K) {
 }
 
 size_t gemm_f32_skinny_scratch_bytes(int M, int N, int K) {
-  const SkinnyPlan p = plan_skinny(M, N, K);
-  return p.chunks > 1 ? (size_t)p.chunks * M * N * sizeof(float) : 0;
+  return (size_t)plan_skinny(M, N, K).chunks * M * N * sizeof(float);
 }
 
 bool gemm_f32_skinny_applies(bool trans_a, int M, int N, int K, const float* A, int lda,
                              const float* B, int ldb, const float* C, int ldc) {
   return gemm_f32_skinny_shape(trans_a, M, N, K) && lda % 4 == 0 && ldb % 4 == 0 && ldc % 4 == 0 &&
          aligned16(A) && aligned16(B) && aligned16(C);
+}
+
+// The streaming kernel alone: leaves `*chunks` partial results [chunk][M][N] at `*partial`
+// (in the stream's scratch buffer, valid until the next product on the stream) for a consumer
+// that adds them itself, in chunk order.
+int gemm_f32_skinny_chunks(hipStream_t stream, int M, int N, int K, const float* A, int lda,
+                           const float* B, int ldb, size_t scratch_offset, const float** partial,
+                           int* chunks) {
+  const SkinnyPlan p = plan_skinny(M, N, K);
+  Workspace ws;
+  HASTE_HIP_PROPAGATE(get_workspace(stream, scratch_offset + (size_t)p.chunks * M * N * sizeof(float), &ws));
+  float* part = ws.scratch + scratch_offset / sizeof(float);
+  const dim3 grid((unsigned)p.col_blocks, (unsigned)p.chunks);
+  ScopedKernelTimer timer("gemm_f32_skinny", stream);
+  if (p.mt == 16)
+    skinny_kernel<16><<<grid, dim3(256), 0, stream>>>(M, N, K, A, lda, B, ldb, nullptr, 0, 0, p.k_per_wg, part);
+  else
+    skinny_kernel<32><<<grid, dim3(256), 0, stream>>>(M, N, K, A, lda, B, ldb, nullptr, 0, 0, p.k_per_wg, part);
+  HASTE_HIP_TRY(hipGetLastError());
+  *partial = part;
+  *chunks = p.chunks;
+  return HASTE_HIP_OK;
 }
 
 int gemm_f32_skinny(hipStream_t stream, int M, int N, int K, const float* A, int lda,

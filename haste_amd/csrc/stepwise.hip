@@ -75,6 +75,111 @@ template <> size_t gemm_room<float>(int M, int N, int K) { return gemm_f32_scrat
 template <> size_t gemm_room<double>(int, int, int) { return 0; }
 template <> size_t gemm_room<half_t>(int, int, int) { return 0; }
 
+// A step's product as its consumer reads it: either one finished matrix (chunks == 1,
+// stride == 0) or the K chunks of the small-batch streaming kernel, which the consumer adds in
+// chunk order itself -- one launch per step less than reducing them first, which is what
+// bounds the step at small batch and moderate hidden size.  chunks == 0: nothing pending.
+template <typename T>
+struct StepProduct {
+  const T* base = nullptr;
+  int chunks = 0;
+  size_t stride = 0;
+  // out[g] = the product at idx + g * gate_stride, g < G.  Chunks are added in index order;
+  // the loads of two chunks and all G gates are issued together.
+  template <int G>
+  __device__ __forceinline__ void at(size_t idx, size_t gate_stride, typename Acc<T>::type (&out)[G]) const {
+    typedef typename Acc<T>::type A;
+#pragma unroll
+    for (int g = 0; g < G; ++g) out[g] = A(0);
+    int k = 0;
+    for (; k + 2 <= chunks; k += 2) {
+      A v0[G], v1[G];
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        v0[g] = (A)base[k * stride + idx + g * gate_stride];
+        v1[g] = (A)base[(k + 1) * stride + idx + g * gate_stride];
+      }
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        out[g] += v0[g];
+        out[g] += v1[g];
+      }
+    }
+    if (k < chunks) {
+#pragma unroll
+      for (int g = 0; g < G; ++g) out[g] += (A)base[k * stride + idx + g * gate_stride];
+    }
+  }
+  __device__ __forceinline__ typename Acc<T>::type at(size_t idx) const {
+    typename Acc<T>::type out[1];
+    at<1>(idx, 0, out);
+    return out[0];
+  }
+};
+
+// C[M,N] = A[M,K] * B[K,N] for one step, for a consumer kernel: into `out` (then the product
+// reads as one matrix), or left as chunks.
+template <typename T>
+int step_product(hipStream_t s, int M, int N, int K, const T* A, const T* B, T* out,
+                 size_t scratch_offset, StepProduct<T>* p) {
+  HASTE_HIP_PROPAGATE(gemm(s, false, M, N, K, A, K, B, N, out, N, false, scratch_offset));
+  p->base = out;
+  p->chunks = 1;
+  p->stride = 0;
+  return HASTE_HIP_OK;
+}
+template <>
+int step_product<float>(hipStream_t s, int M, int N, int K, const float* A, const float* B,
+                        float* out, size_t scratch_offset, StepProduct<float>* p) {
+  if (gemm_f32_skinny_applies(false, M, N, K, A, K, B, N, out, N)) {
+    HASTE_HIP_PROPAGATE(gemm_f32_skinny_chunks(s, M, N, K, A, K, B, N, scratch_offset, &p->base, &p->chunks));
+    p->stride = (size_t)M * N;
+    return HASTE_HIP_OK;
+  }
+  HASTE_HIP_PROPAGATE(gemm_f32(s, false, M, N, K, A, K, B, N, out, N, false, scratch_offset));
+  p->base = out;
+  p->chunks = 1;
+  p->stride = 0;
+  return HASTE_HIP_OK;
+}
+
+// dh += (pending chunks): the recurrent contribution a reverse step leaves for the next
+// step's pointwise kernel, added for real after the last step.
+template <typename T>
+__global__ __launch_bounds__(kThreads)
+void add_pending_kernel(size_t n, StepProduct<T> pend, T* __restrict__ dh) {
+  const size_t i = blockIdx.x * (size_t)kThreads + threadIdx.x;
+  if (i < n) dh[i] = T((typename Acc<T>::type)dh[i] + pend.at(i));
+}
+
+// The recurrent product of a reverse step, dh += dv_t[M,K] * R_t[K,N]: accumulated into dh
+// (nothing pending), or left as chunks for the next consumer of dh.
+template <typename T>
+int reverse_product(hipStream_t s, int M, int N, int K, const T* A, const T* B, T* dh,
+                    size_t scratch_offset, StepProduct<T>* pend) {
+  pend->chunks = 0;
+  return gemm(s, false, M, N, K, A, K, B, N, dh, N, true, scratch_offset);
+}
+template <>
+int reverse_product<float>(hipStream_t s, int M, int N, int K, const float* A, const float* B,
+                           float* dh, size_t scratch_offset, StepProduct<float>* pend) {
+  pend->chunks = 0;
+  if (gemm_f32_skinny_applies(false, M, N, K, A, K, B, N, dh, N)) {
+    HASTE_HIP_PROPAGATE(gemm_f32_skinny_chunks(s, M, N, K, A, K, B, N, scratch_offset, &pend->base, &pend->chunks));
+    pend->stride = (size_t)M * N;
+    return HASTE_HIP_OK;
+  }
+  return gemm_f32(s, false, M, N, K, A, K, B, N, dh, N, true, scratch_offset);
+}
+
+template <typename T>
+int flush_pending(hipStream_t s, size_t n, const StepProduct<T>& pend, T* dh) {
+  if (pend.chunks == 0) return HASTE_HIP_OK;
+  add_pending_kernel<T><<<blocks_for(n), dim3(kThreads), 0, s>>>(n, pend, dh);
+  HASTE_LAUNCHED();
+  return HASTE_HIP_OK;
+}
+
 // Scratch of a call: buffers of its own in front, the float GEMM's partial tiles behind
 // them.  Everything is sized before the first launch so that the buffer never moves while
 // it is in use.
@@ -292,7 +397,7 @@ int ln_backward_rows(hipStream_t stream, size_t rows, int D, const T* gamma, con
 // v_t: in x*W of the step, out (training) the gate activations; rh = h*R of the step.
 template <typename T>
 __global__ __launch_bounds__(kThreads)
-void lstm_forward_pointwise(int training, int N, int H, const T* __restrict__ rh,
+void lstm_forward_pointwise(int training, int N, int H, StepProduct<T> rh,
                             const T* __restrict__ b, const T* __restrict__ h,
                             const T* __restrict__ c, T* __restrict__ h_out, T* __restrict__ c_out,
                             T* __restrict__ v_t, float zoneout_prob, const T* __restrict__ mask_t) {
@@ -301,8 +406,9 @@ void lstm_forward_pointwise(int training, int N, int H, const T* __restrict__ rh
   const int n = (int)(idx / H), j = (int)(idx % H);
   const size_t g0 = (size_t)n * 4 * H + j;
   T a[4];
+  rh.template at<4>(g0, (size_t)H, a);
 #pragma unroll
-  for (int g = 0; g < 4; ++g) a[g] = v_t[g0 + (size_t)g * H] + rh[g0 + (size_t)g * H] + b[g * H + j];
+  for (int g = 0; g < 4; ++g) a[g] = v_t[g0 + (size_t)g * H] + a[g] + b[g * H + j];
   const T gi = Fn<T>::sigmoid(a[0]), gg = Fn<T>::tanh_(a[1]), gf = Fn<T>::sigmoid(a[2]),
           go = Fn<T>::sigmoid(a[3]);
   if (training) {
@@ -328,15 +434,15 @@ template <typename T>
 __global__ __launch_bounds__(kThreads)
 void lstm_backward_pointwise(int N, int H, const T* __restrict__ c, const T* __restrict__ c_next,
                              const T* __restrict__ dh_next, const T* __restrict__ dc_next,
-                             T* __restrict__ dh, T* __restrict__ dc, T* __restrict__ v_t,
-                             const T* __restrict__ mask_t) {
+                             T* __restrict__ dh, StepProduct<T> pend, T* __restrict__ dc,
+                             T* __restrict__ v_t, const T* __restrict__ mask_t) {
   const size_t idx = blockIdx.x * (size_t)kThreads + threadIdx.x;
   if (idx >= (size_t)N * H) return;
   const int n = (int)(idx / H), j = (int)(idx % H);
   const size_t g0 = (size_t)n * 4 * H + j;
   const T gi = v_t[g0], gg = v_t[g0 + H], gf = v_t[g0 + 2 * (size_t)H], go = v_t[g0 + 3 * (size_t)H];
   T dc_total = dc_next[idx] + dc[idx];
-  T dh_total = dh_next[idx] + dh[idx];
+  T dh_total = dh_next[idx] + (dh[idx] + pend.at(idx));
   const T c_tanh = Fn<T>::tanh_(c_next[idx]);
   T dh_keep = T(0);
   if (mask_t != nullptr) {
@@ -361,7 +467,7 @@ void lstm_backward_pointwise(int N, int H, const T* __restrict__ c, const T* __r
 template <typename T>
 __global__ __launch_bounds__(kThreads)
 void gru_forward_pointwise(int training, int N, int H, const T* __restrict__ wx,
-                           const T* __restrict__ rh, const T* __restrict__ bx,
+                           StepProduct<T> rh, const T* __restrict__ bx,
                            const T* __restrict__ br, const T* __restrict__ h,
                            T* __restrict__ h_out, T* __restrict__ v_t, float zoneout_prob,
                            const T* __restrict__ mask_t) {
@@ -370,9 +476,11 @@ void gru_forward_pointwise(int training, int N, int H, const T* __restrict__ wx,
   if (idx >= (size_t)N * H) return;
   const int n = (int)(idx / H), j = (int)(idx % H);
   const size_t g0 = (size_t)n * 3 * H + j;
-  const A z = Fn<A>::sigmoid(A(wx[g0]) + A(rh[g0]) + A(bx[j]) + A(br[j]));
-  const A r = Fn<A>::sigmoid(A(wx[g0 + H]) + A(rh[g0 + H]) + A(bx[H + j]) + A(br[H + j]));
-  const A qg = A(rh[g0 + 2 * (size_t)H]) + A(br[2 * H + j]);
+  A q[3];
+  rh.template at<3>(g0, (size_t)H, q);
+  const A z = Fn<A>::sigmoid(A(wx[g0]) + q[0] + A(bx[j]) + A(br[j]));
+  const A r = Fn<A>::sigmoid(A(wx[g0 + H]) + q[1] + A(bx[H + j]) + A(br[H + j]));
+  const A qg = q[2] + A(br[2 * H + j]);
   const A g = Fn<A>::tanh_(A(wx[g0 + 2 * (size_t)H]) + r * qg + A(bx[2 * H + j]));
   if (training) {
     const size_t v0 = (size_t)n * 4 * H + j;
@@ -394,7 +502,7 @@ template <typename T>
 __global__ __launch_bounds__(kThreads)
 void gru_backward_pointwise(int N, int H, const T* __restrict__ h, const T* __restrict__ v_t,
                             const T* __restrict__ dh_next, T* __restrict__ dh,
-                            T* __restrict__ dp_t, T* __restrict__ dq_t,
+                            StepProduct<T> pend, T* __restrict__ dp_t, T* __restrict__ dq_t,
                             const T* __restrict__ mask_t) {
   using A = typename Acc<T>::type;
   const size_t idx = blockIdx.x * (size_t)kThreads + threadIdx.x;
@@ -403,7 +511,7 @@ void gru_backward_pointwise(int N, int H, const T* __restrict__ h, const T* __re
   const size_t v0 = (size_t)n * 4 * H + j, g0 = (size_t)n * 3 * H + j;
   const A z = A(v_t[v0]), r = A(v_t[v0 + H]), g = A(v_t[v0 + 2 * (size_t)H]),
           qg = A(v_t[v0 + 3 * (size_t)H]);
-  A dh_total = A(dh_next[idx]) + A(dh[idx]);
+  A dh_total = A(dh_next[idx]) + (A(dh[idx]) + pend.at(idx));
   A dh_keep;
   if (mask_t != nullptr) {
     const A m = A(mask_t[idx]);
@@ -480,13 +588,13 @@ void ln_lstm_cell_output(int training, int N, int H, const T* __restrict__ rhn,
 template <typename T>
 __global__ __launch_bounds__(kThreads)
 void ln_lstm_output_grad(int N, int H, const T* __restrict__ dh_next, T* __restrict__ dh,
-                         const T* __restrict__ mask_t, T* __restrict__ c_norm_t, T* __restrict__ v_t) {
+                         StepProduct<T> pend, const T* __restrict__ mask_t, T* __restrict__ c_norm_t, T* __restrict__ v_t) {
   const size_t idx = blockIdx.x * (size_t)kThreads + threadIdx.x;
   if (idx >= (size_t)N * H) return;
   const int n = (int)(idx / H), j = (int)(idx % H);
   const size_t o_at = (size_t)n * 4 * H + 3 * (size_t)H + j;
   const T go = v_t[o_at];
-  T dh_total = dh_next[idx] + dh[idx];
+  T dh_total = dh_next[idx] + (dh[idx] + pend.at(idx));
   T dh_keep = T(0);
   if (mask_t != nullptr) {
     const T m = mask_t[idx];
@@ -603,9 +711,10 @@ int lstm_forward_steps(hipStream_t stream, int training, int steps, int N, int C
   for (int t = 0; t < steps; ++t) {
     const T* h_t = t == 0 ? h : h_out + (size_t)(t - 1) * NH;
     const T* c_t = t == 0 ? c : c_out + (size_t)(t - 1) * NH;
-    HASTE_HIP_PROPAGATE(gemm(stream, false, N, 4 * H, H, h_t, H, Ruse, 4 * H, rh, 4 * H, false, sc.gemm_offset()));
+    StepProduct<T> prod;
+    HASTE_HIP_PROPAGATE(step_product<T>(stream, N, 4 * H, H, h_t, Ruse, rh, sc.gemm_offset(), &prod));
     lstm_forward_pointwise<T><<<blocks_for(NH), dim3(kThreads), 0, stream>>>(
-        training, N, H, rh, b, h_t, c_t, h_out + (size_t)t * NH, c_out + (size_t)t * NH,
+        training, N, H, prod, b, h_t, c_t, h_out + (size_t)t * NH, c_out + (size_t)t * NH,
         v + (size_t)t * N4H, zoneout_prob, zoneout_mask ? zoneout_mask + (size_t)t * NH : nullptr);
     HASTE_LAUNCHED();
   }
@@ -627,15 +736,17 @@ int lstm_backward_steps(hipStream_t stream, int steps, int N, int C, int H, cons
   void* partial = sc.take<char>(own);
   {
     ScopedKernelTimer timer("lstm_backward_steps", stream);
+    StepProduct<T> pend;
     for (int t = steps - 1; t >= 0; --t) {
       lstm_backward_pointwise<T><<<blocks_for(NH), dim3(kThreads), 0, stream>>>(
           N, H, c + (size_t)t * NH, c_next + (size_t)t * NH, dh_next + (size_t)t * NH,
-          dc_next + (size_t)t * NH, dh, dc, v + (size_t)t * N4H,
+          dc_next + (size_t)t * NH, dh, pend, dc, v + (size_t)t * N4H,
           zoneout_mask ? zoneout_mask + (size_t)t * NH : nullptr);
       HASTE_LAUNCHED();
       // dh += dv_t * R^T
-      HASTE_HIP_PROPAGATE(gemm(stream, false, N, H, 4 * H, v + (size_t)t * N4H, 4 * H, R_t, H, dh, H, true, sc.gemm_offset()));
+      HASTE_HIP_PROPAGATE(reverse_product<T>(stream, N, H, 4 * H, v + (size_t)t * N4H, R_t, dh, sc.gemm_offset(), &pend));
     }
+    HASTE_HIP_PROPAGATE(flush_pending<T>(stream, NH, pend, dh));
   }
   HASTE_HIP_PROPAGATE((column_sum<T, 0>(stream, (size_t)TN, 4 * H, v, nullptr, nullptr, partial, db)));
   HASTE_HIP_PROPAGATE(gemm(stream, false, C, 4 * H, TN, x_t, TN, v, 4 * H, dW, 4 * H, true, sc.gemm_offset()));
@@ -660,9 +771,10 @@ int gru_forward_steps(hipStream_t stream, int training, int steps, int N, int C,
   ScopedKernelTimer timer("gru_forward_steps", stream);
   for (int t = 0; t < steps; ++t) {
     const T* h_t = t == 0 ? h : h_out + (size_t)(t - 1) * NH;
-    HASTE_HIP_PROPAGATE(gemm(stream, false, N, 3 * H, H, h_t, H, Ruse, 3 * H, rh, 3 * H, false, sc.gemm_offset()));
+    StepProduct<T> prod;
+    HASTE_HIP_PROPAGATE(step_product<T>(stream, N, 3 * H, H, h_t, Ruse, rh, sc.gemm_offset(), &prod));
     gru_forward_pointwise<T><<<blocks_for(NH), dim3(kThreads), 0, stream>>>(
-        training, N, H, tmp_Wx + (size_t)t * N3H, rh, bx, br, h_t, h_out + (size_t)t * NH,
+        training, N, H, tmp_Wx + (size_t)t * N3H, prod, bx, br, h_t, h_out + (size_t)t * NH,
         v ? v + (size_t)t * N4H : nullptr, zoneout_prob,
         zoneout_mask ? zoneout_mask + (size_t)t * NH : nullptr);
     HASTE_LAUNCHED();
@@ -684,15 +796,17 @@ int gru_backward_steps(hipStream_t stream, int steps, int N, int C, int H, const
   void* partial = sc.take<char>(own);
   {
     ScopedKernelTimer timer("gru_backward_steps", stream);
+    StepProduct<T> pend;
     for (int t = steps - 1; t >= 0; --t) {
       gru_backward_pointwise<T><<<blocks_for(NH), dim3(kThreads), 0, stream>>>(
-          N, H, h + (size_t)t * NH, v + (size_t)t * N4H, dh_next + (size_t)t * NH, dh,
+          N, H, h + (size_t)t * NH, v + (size_t)t * N4H, dh_next + (size_t)t * NH, dh, pend,
           dp + (size_t)t * N3H, dq + (size_t)t * N3H,
           zoneout_mask ? zoneout_mask + (size_t)t * NH : nullptr);
       HASTE_LAUNCHED();
       // dh += dq_t * R^T
-      HASTE_HIP_PROPAGATE(gemm(stream, false, N, H, 3 * H, dq + (size_t)t * N3H, 3 * H, R_t, H, dh, H, true, sc.gemm_offset()));
+      HASTE_HIP_PROPAGATE(reverse_product<T>(stream, N, H, 3 * H, dq + (size_t)t * N3H, R_t, dh, sc.gemm_offset(), &pend));
     }
+    HASTE_HIP_PROPAGATE(flush_pending<T>(stream, NH, pend, dh));
   }
   HASTE_HIP_PROPAGATE((column_sum<T, 0>(stream, (size_t)TN, 3 * H, dp, nullptr, nullptr, partial, dbx)));
   HASTE_HIP_PROPAGATE((column_sum<T, 0>(stream, (size_t)TN, 3 * H, dq, nullptr, nullptr, partial, dbr)));
@@ -755,13 +869,14 @@ int ln_lstm_backward_steps(hipStream_t stream, int steps, int N, int C, int H, c
   T* stats1 = sc.take<T>((size_t)TN * 2);
   {
     ScopedKernelTimer timer("layer_norm_lstm_backward_steps", stream);
+    StepProduct<T> pend;
     for (int t = steps - 1; t >= 0; --t) {
       T* v_t = v + (size_t)t * N4H;
       T* cn_t = act_c_norm + (size_t)t * NH;
       T* rh_t = act_Rh + (size_t)t * N4H;
       const T* mask_t = zoneout_mask ? zoneout_mask + (size_t)t * NH : nullptr;
       ln_lstm_output_grad<T><<<blocks_for(NH), dim3(kThreads), 0, stream>>>(
-          N, H, dh_new + (size_t)(t + 1) * NH, dh, mask_t, cn_t, v_t);
+          N, H, dh_new + (size_t)(t + 1) * NH, dh, pend, mask_t, cn_t, v_t);
       HASTE_LAUNCHED();
       // through the norm of the cell state, in place over act_c_norm[t]
       HASTE_HIP_PROPAGATE(ln_backward_rows<T>(stream, (size_t)N, H, gamma_h, c + (size_t)(t + 1) * NH, cn_t, cn_t,
@@ -772,8 +887,9 @@ int ln_lstm_backward_steps(hipStream_t stream, int steps, int N, int C, int H, c
       // through the norm of h*R, in place over act_Rh[t]
       HASTE_HIP_PROPAGATE(ln_backward_rows<T>(stream, (size_t)N, 4 * H, gamma2, rh_t, v_t, rh_t, dgamma2,
                                               nullptr, cache2 + (size_t)t * N * 2, partial));
-      HASTE_HIP_PROPAGATE(gemm(stream, false, N, H, 4 * H, rh_t, 4 * H, R_t, H, dh, H, true, sc.gemm_offset()));
+      HASTE_HIP_PROPAGATE(reverse_product<T>(stream, N, H, 4 * H, rh_t, R_t, dh, sc.gemm_offset(), &pend));
     }
+    HASTE_HIP_PROPAGATE(flush_pending<T>(stream, NH, pend, dh));
   }
   HASTE_HIP_PROPAGATE((column_sum<T, 0>(stream, (size_t)TN, 4 * H, v, nullptr, nullptr, partial, db)));
   // through the norm of x*W, in place over act_Wx
@@ -804,8 +920,11 @@ int ln_gru_forward_steps(hipStream_t stream, int training, int steps, int N, int
     HASTE_HIP_PROPAGATE(gemm(stream, false, N, 3 * H, H, h_t, H, R, 3 * H, rh_t, 3 * H, false, sc.gemm_offset()));
     HASTE_HIP_PROPAGATE(ln_forward_rows<T>(stream, (size_t)N, 3 * H, gamma2, nullptr, rh_t, rhn,
                                            cache2 ? cache2 + (size_t)t * N * 2 : nullptr));
+    StepProduct<T> normed;
+    normed.base = rhn;
+    normed.chunks = 1;
     gru_forward_pointwise<T><<<blocks_for(NH), dim3(kThreads), 0, stream>>>(
-        training, N, H, tmp_Wx_norm + (size_t)t * N3H, rhn, bx, br, h_t, h + (size_t)(t + 1) * NH,
+        training, N, H, tmp_Wx_norm + (size_t)t * N3H, normed, bx, br, h_t, h + (size_t)(t + 1) * NH,
         v ? v + (size_t)t * N4H : nullptr, zoneout_prob,
         zoneout_mask ? zoneout_mask + (size_t)t * NH : nullptr);
     HASTE_LAUNCHED();
@@ -831,18 +950,20 @@ int ln_gru_backward_steps(hipStream_t stream, int steps, int N, int C, int H, co
   T* stats1 = sc.take<T>((size_t)TN * 2);
   {
     ScopedKernelTimer timer("layer_norm_gru_backward_steps", stream);
+    StepProduct<T> pend;
     for (int t = steps - 1; t >= 0; --t) {
       T* dq_t = dq + (size_t)t * N3H;
       gru_backward_pointwise<T><<<blocks_for(NH), dim3(kThreads), 0, stream>>>(
-          N, H, h + (size_t)t * NH, v + (size_t)t * N4H, dh_new + (size_t)(t + 1) * NH, dh,
+          N, H, h + (size_t)t * NH, v + (size_t)t * N4H, dh_new + (size_t)(t + 1) * NH, dh, pend,
           dp + (size_t)t * N3H, dq_t, zoneout_mask ? zoneout_mask + (size_t)t * NH : nullptr);
       HASTE_LAUNCHED();
       // the recurrent bias sees dq before the norm; then through the norm of h*R, in place
       HASTE_HIP_PROPAGATE((column_sum<T, 0>(stream, (size_t)N, 3 * H, dq_t, nullptr, nullptr, partial, dbr)));
       HASTE_HIP_PROPAGATE(ln_backward_rows<T>(stream, (size_t)N, 3 * H, gamma2, act_Rh + (size_t)t * N3H, dq_t, dq_t,
                                               dgamma2, nullptr, cache2 + (size_t)t * N * 2, partial));
-      HASTE_HIP_PROPAGATE(gemm(stream, false, N, H, 3 * H, dq_t, 3 * H, R_t, H, dh, H, true, sc.gemm_offset()));
+      HASTE_HIP_PROPAGATE(reverse_product<T>(stream, N, H, 3 * H, dq_t, R_t, dh, sc.gemm_offset(), &pend));
     }
+    HASTE_HIP_PROPAGATE(flush_pending<T>(stream, NH, pend, dh));
   }
   HASTE_HIP_PROPAGATE((column_sum<T, 0>(stream, (size_t)TN, 3 * H, dp, nullptr, nullptr, partial, dbx)));
   HASTE_HIP_PROPAGATE(ln_forward_rows<T>(stream, (size_t)TN, 3 * H, gamma1, nullptr, act_Wx, nullptr, stats1));
