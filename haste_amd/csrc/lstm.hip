@@ -36,14 +36,15 @@ void lstm_forward_kernel(LstmFwdParams p) {
   constexpr int NCOLS = 16 * CT;
   constexpr int PP = (NB * HS + 255) / 256;
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  __shared__ unsigned int s_role;
-  const Role role = take_role(p.ls, &s_role);
-  if (!role.active) return;
-
   const int H = p.H, N = p.N, T = p.T;
   const int Kpad = round_up(H, 64);
   float* w_lds = lds;
   float* red = lds + Kpad * NCOLS;
+  // The role is handed round through a word of the partial-tile area, which nothing else
+  // uses before the first step: the kernel has no static LDS, so that a slice and its
+  // partial tiles may fill the workgroup's 160 KiB exactly (N = 128, H = 1024).
+  const Role role = take_role(p.ls, reinterpret_cast<unsigned int*>(red));
+  if (!role.active) return;
 
   const int tid = threadIdx.x;
   const int j0 = role.cw * HS;
@@ -426,7 +427,7 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
                       float dc_scale) {
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
   HASTE_HIP_REQUIRE(W && R && b && x && h && c && h_out && c_out && v);
-  const ForwardTile tile = pick_forward_tile(4, N, H, 0);
+  const ForwardTile tile = pick_forward_tile(4, N, H, 0, kWorkgroupLdsBytes);
   // No slice of R fits a CU: stream R from HBM every step instead.
   if (!tile.ok)
     return lstm_forward_streamed(stream, training, T, N, C, H, W, R, b, x, h, c, h_out, c_out, v,

@@ -1,13 +1,14 @@
 // Device-side building blocks of the persistent recurrence kernels.
 //
-// A recurrence kernel is one cooperative launch that runs all T steps.  The grid is
-// (column workgroups) x (batch tiles): a workgroup owns `HS` hidden units (all of
-// their gate columns) for the 16*RT batch rows of its tile, keeps its slice of the
-// recurrent weight matrix in LDS for the whole launch, and per step multiplies the
-// tile's rows of the exchanged activation (h_t forward, the gate gradients backward)
-// with that slice on the MFMA units.  Workgroups that share a batch tile form a
-// group and synchronise once per exchange through a counter in device memory;
-// different batch tiles never wait for each other.
+// A recurrence kernel is one launch that runs all T steps (an ordinary launch whose grid
+// is checked against what the chip can hold at once).  The grid is (column workgroups) x
+// (batch tiles): a workgroup owns `HS` hidden units (all of their gate columns) for the NB
+// batch rows of its tile, keeps its slice of the recurrent weight matrix in LDS for the
+// whole launch, and per step multiplies the tile's rows of the exchanged activation (h_t
+// forward, the gate gradients backward) with that slice on the MFMA units.  Workgroups that
+// share a batch tile form a group and hand each step's activations to each other through
+// tiles in device memory whose consumers poll for the data itself (or, at set-up, through
+// per-workgroup flag words); different batch tiles never wait for each other.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -926,8 +927,9 @@ int launch_persistent(const char* name, KernelT kernel, const LaunchPlan& plan, 
 
 // Dynamic LDS a persistent kernel may ask for: the 160 KiB of a gfx950 workgroup less room
 // for the kernels' few statically allocated words (role, flag), which count against the
-// same limit.
-constexpr size_t kMaxLdsBytes = 160 * 1024 - 256;
+// same limit.  A kernel without static LDS may ask for all of it.
+constexpr size_t kWorkgroupLdsBytes = 160 * 1024;
+constexpr size_t kMaxLdsBytes = kWorkgroupLdsBytes - 256;
 
 // Floats of the exchange tiles (2 behind a step barrier, kPolledTiles when polled) of every
 // group (batch tile) for contraction length K.
@@ -950,7 +952,8 @@ constexpr int kTileHeights[] = {4, 8, 16, 32, 64};
 // spreads a small batch over the most XCDs; then the most column workgroups), else the
 // cross-XCD geometry with the most parallelism that fits the chip.  `extra_lds_per_row` is
 // what the cell needs in LDS per batch row beyond the slice and the partial tiles.
-inline ForwardTile pick_forward_tile(int gates, int N, int H, size_t extra_lds_per_row) {
+inline ForwardTile pick_forward_tile(int gates, int N, int H, size_t extra_lds_per_row,
+                                     size_t lds_limit = kMaxLdsBytes) {
   const int cus = device_cu_count();
   ForwardTile best;
   best.ok = false;
@@ -963,7 +966,7 @@ inline ForwardTile pick_forward_tile(int gates, int N, int H, size_t extra_lds_p
         const int ct = (gates * hs + 15) / 16;
         const int gx = (H + hs - 1) / hs, gy = (N + nb - 1) / nb;
         const size_t lds = fwd_lds_bytes(H, nb, ct) + extra_lds_per_row * nb;
-        if (lds > kMaxLdsBytes || gy > kMaxGroups || gx * gy > kMaxWorkgroups) continue;
+        if (lds > lds_limit || gy > kMaxGroups || gx * gy > kMaxWorkgroups) continue;
         if (pass == 0 ? !xcd_local_fits(gx, gy) : (long long)gx * gy > cus) continue;
         best = ForwardTile{nb, ct, hs, gx, gy, lds, true};
       }

@@ -1,5 +1,5 @@
 // Library runtime: version, error text, and the per-(device, stream) workspace cache.
-#include "common.h"
+#include "recurrent.h"
 
 #include <cstdio>
 #include <cstdlib>
@@ -228,27 +228,14 @@ int haste_hip_stream_order(void* first, void* then) {
 
 int haste_hip_max_hidden_size(int gates, int batch_size) {
   if (gates < 1 || gates > 4 || batch_size < 1) return 0;
-  const int cus = haste_hip::device_cu_count();
-  if (cus <= 0) return 0;
-  const long long lds_limit = 160 * 1024;
+  if (haste_hip::device_cu_count() <= 0) return 0;
+  // The geometry search of the LSTM (4 gates) / GRU (3 gates) entry points themselves: the
+  // largest hidden size for which both the forward and the backward recurrence find a tile.
   auto fits = [&](int H) {
-    bool fwd = false, bwd = false;
-    for (int rt : {1, 2, 4}) {
-      const int gy = (batch_size + 16 * rt - 1) / (16 * rt);
-      if (gy > haste_hip::kMaxGroups) continue;
-      for (int hs : {4, 8, 16}) {
-        const int ct = (gates * hs + 15) / 16;
-        const long long kpad = (H + 63) / 64 * 64;
-        const long long lds = (kpad * 16 * ct + 4LL * 16 * rt * 16 * ct + 32LL * rt) * 4;
-        const long long gx = (H + hs - 1) / hs;
-        if (lds <= lds_limit && gx * gy <= cus) fwd = true;
-      }
-      const long long kpad = ((long long)gates * H + 63) / 64 * 64;
-      const long long lds = (kpad * 16 + 16LL * rt * 10 * 16 + 64LL * rt) * 4;
-      const long long gx = (H + 15) / 16;
-      if (lds <= lds_limit && gx * gy <= cus) bwd = true;
-    }
-    return fwd && bwd;
+    const int k_back = gates == 3 ? 48 * ((H + 15) / 16) : gates * H;
+    const size_t reduce_floats = gates == 3 ? 6 * 16 : (size_t)gates * 16;
+    return haste_hip::pick_forward_tile(gates, batch_size, H, 0, haste_hip::kWorkgroupLdsBytes).ok &&
+           haste_hip::pick_backward_tile(k_back, batch_size, H, reduce_floats, 0).ok;
   };
   int best = 0;
   for (int H = 16; H <= 8192; H += 16)
