@@ -39,6 +39,18 @@ def _call(entry, *args):
     lib.call(name, *args)
 
 
+def _zeros(opts, *shapes):
+    """Zero tensors of the given shapes carved out of one allocation: one fill kernel for all
+    the accumulated outputs of a backward pass (each starts on a 256-byte boundary)."""
+    sizes = [int(torch.Size(shp).numel()) for shp in shapes]
+    starts, total = [], 0
+    for n in sizes:
+        starts.append(total)
+        total += (n + 63) // 64 * 64
+    flat = torch.zeros(total, **opts)
+    return [flat[a:a + n].view(shp) for a, n, shp in zip(starts, sizes, shapes)]
+
+
 def _mask_or_none(has_zoneout, zoneout_mask):
     return zoneout_mask if has_zoneout else None
 
@@ -80,8 +92,7 @@ def lstm_forward(training, zoneout_prob, x, h0, c0, kernel, recurrent_kernel, bi
     output = torch.empty(T + 1, N, H, **opts)
     output_state = torch.empty(T + 1, N, H, **opts)
     cache = torch.empty(T, N, 4 * H, **opts)
-    output[0] = h0
-    output_state[0] = c0
+    torch._foreach_copy_([output[0], output_state[0]], [h0, c0])  # one kernel for both
     zp = float(zoneout_prob) if has_zoneout else 0.0
     mask = _mask_or_none(has_zoneout, zoneout_mask)
     if dropconnect_mask is None:
@@ -102,11 +113,7 @@ def lstm_backward(x_t, kernel_t, recurrent_kernel_t, bias, zoneout_mask, h, c, c
     _check(x_t, kernel_t, recurrent_kernel_t, bias, zoneout_mask, h, c, cache, dh_new, dc_new)
     opts = dict(device=x_t.device, dtype=x_t.dtype)
     dx = torch.empty(T, N, C, **opts)
-    dW = torch.zeros(C, 4 * H, **opts)
-    dR = torch.zeros(H, 4 * H, **opts)
-    db = torch.zeros(4 * H, **opts)
-    dh = torch.zeros(N, H, **opts)
-    dc = torch.zeros(N, H, **opts)
+    dW, dR, db, dh, dc = _zeros(opts, (C, 4 * H), (H, 4 * H), (4 * H,), (N, H), (N, H))
     _call("haste_hip_lstm_backward", T, N, C, H, kernel_t, recurrent_kernel_t, bias, x_t,
              h, c, dh_new, dc_new, dx, dW, dR, db, dh, dc, cache,
              _mask_or_none(has_zoneout, zoneout_mask))
@@ -211,11 +218,7 @@ def gru_backward(x_t, kernel_t, recurrent_kernel_t, bias, recurrent_bias, zoneou
     _check(x_t, kernel_t, recurrent_kernel_t, bias, recurrent_bias, zoneout_mask, h, cache, dh_new)
     opts = dict(device=x_t.device, dtype=x_t.dtype)
     dx = torch.empty(T, N, C, **opts)
-    dW = torch.zeros(C, 3 * H, **opts)
-    dR = torch.zeros(H, 3 * H, **opts)
-    dbx = torch.zeros(3 * H, **opts)
-    dbr = torch.zeros(3 * H, **opts)
-    dh = torch.zeros(N, H, **opts)
+    dW, dR, dbx, dbr, dh = _zeros(opts, (C, 3 * H), (H, 3 * H), (3 * H,), (3 * H,), (N, H))
     dp = torch.empty(T, N, 3 * H, **opts)
     dq = torch.empty(T, N, 3 * H, **opts)
     _call("haste_hip_gru_backward", T, N, C, H, kernel_t, recurrent_kernel_t, bias,
@@ -267,10 +270,7 @@ def indrnn_backward(x_t, kernel_t, recurrent_scale, bias, zoneout_mask, h, dh_ne
     _check(x_t, kernel_t, recurrent_scale, bias, zoneout_mask, h, dh_new)
     opts = dict(device=x_t.device, dtype=x_t.dtype)
     dx = torch.empty(T, N, C, **opts)
-    dW = torch.zeros(C, H, **opts)
-    du = torch.zeros(H, **opts)
-    db = torch.zeros_like(bias)
-    dh = torch.zeros(N, H, **opts)
+    dW, du, db, dh = _zeros(opts, (C, H), (H,), (H,), (N, H))
     workspace = torch.empty(T, N, H, **opts)
     _call("haste_hip_indrnn_backward", T, N, C, H, kernel_t, recurrent_scale, bias, x_t, h,
              dh_new, dx, dW, du, db, dh, workspace, _mask_or_none(has_zoneout, zoneout_mask))
@@ -304,10 +304,7 @@ def layer_norm_indrnn_backward(x_t, kernel_t, recurrent_scale, bias, gamma, zone
     _check(x_t, kernel_t, recurrent_scale, bias, gamma, zoneout_mask, h, act_Wx, dh_new)
     opts = dict(device=x_t.device, dtype=x_t.dtype)
     dx = torch.empty(T, N, C, **opts)
-    dW = torch.zeros(C, H, **opts)
-    du = torch.zeros(H, **opts)
-    db = torch.zeros_like(bias)
-    dh = torch.zeros(N, H, **opts)
+    dW, du, db, dh = _zeros(opts, (C, H), (H,), (H,), (N, H))
     workspace = torch.empty(T, N, H, **opts)
     dgamma = torch.zeros_like(gamma)
     _call("haste_hip_layer_norm_indrnn_backward", T, N, C, H, kernel_t, recurrent_scale, bias,
@@ -324,8 +321,8 @@ def layer_norm_lstm_forward(training, zoneout_prob, x, h0, c0, kernel, recurrent
     has_zoneout = bool(zoneout_prob) and zoneout_mask.numel() > 0
     _check(x, h0, c0, kernel, recurrent_kernel, bias, gamma, gamma_h, beta_h, zoneout_mask)
     opts = dict(device=x.device, dtype=x.dtype)
-    output = torch.zeros(T + 1, N, H, **opts)
-    output_state = torch.zeros(T + 1, N, H, **opts)
+    output = torch.empty(T + 1, N, H, **opts)
+    output_state = torch.empty(T + 1, N, H, **opts)
     act_Wx = torch.empty(T, N, 4 * H, **opts)
     act_Wx_norm = torch.empty(T, N, 4 * H, **opts)
     act_Wx_norm_cache = torch.empty(T, N, 2, **opts)
@@ -355,14 +352,8 @@ def layer_norm_lstm_backward(x_t, kernel_t, recurrent_kernel_t, bias, gamma, gam
            act_c_norm_cache, dh_new, dc_new)
     opts = dict(device=x_t.device, dtype=x_t.dtype)
     dx = torch.empty(T, N, C, **opts)
-    dW = torch.zeros(C, 4 * H, **opts)
-    dR = torch.zeros(H, 4 * H, **opts)
-    db = torch.zeros(4 * H, **opts)
-    dgamma = torch.zeros_like(gamma)
-    dgamma_h = torch.zeros_like(gamma_h)
-    dbeta_h = torch.zeros_like(beta_h)
-    dh = torch.zeros(N, H, **opts)
-    dc = torch.zeros(N, H, **opts)
+    dW, dR, db, dgamma, dgamma_h, dbeta_h, dh, dc = _zeros(
+        opts, (C, 4 * H), (H, 4 * H), (4 * H,), tuple(gamma.shape), (H,), (H,), (N, H), (N, H))
     _call("haste_hip_layer_norm_lstm_backward", T, N, C, H, kernel_t, recurrent_kernel_t,
              bias, x_t, h, c, dh_new, dc_new, dx, dW, dR, db, dh, dc,
              act_Wx, gamma[0], dgamma[0], act_Wx_norm, act_Rh, gamma[1], dgamma[1],
@@ -405,14 +396,10 @@ def layer_norm_gru_backward(x_t, kernel_t, recurrent_kernel_t, bias, recurrent_b
            act_Wx, act_Wx_norm_cache, act_Rh, act_Rh_norm_cache, dh_new)
     opts = dict(device=x_t.device, dtype=x_t.dtype)
     dx = torch.empty(T, N, C, **opts)
-    dW = torch.zeros(C, 3 * H, **opts)
-    dR = torch.zeros(H, 3 * H, **opts)
-    dbx = torch.zeros(3 * H, **opts)
-    dbr = torch.zeros(3 * H, **opts)
-    dh = torch.zeros(N, H, **opts)
+    dW, dR, dbx, dbr, dh, dgamma = _zeros(opts, (C, 3 * H), (H, 3 * H), (3 * H,), (3 * H,), (N, H),
+                                          tuple(gamma.shape))
     dp = torch.empty(T, N, 3 * H, **opts)
     dq = torch.empty(T, N, 3 * H, **opts)
-    dgamma = torch.zeros_like(gamma)
     _call("haste_hip_layer_norm_gru_backward", T, N, C, H, kernel_t, recurrent_kernel_t, bias,
              recurrent_bias, x_t, h, cache, dh_new, dx, dW, dR, dbx, dbr, dh, dp, dq,
              act_Wx, gamma[0], dgamma[0], act_Rh, gamma[1], dgamma[1], act_Rh_norm_cache,
