@@ -37,7 +37,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget", type=float, default=15.0)
-    ap.add_argument("--workload", choices=["all", "metric", "streaming", "stepwise", "copy", "configs"], default="all",
+    ap.add_argument("--workload", choices=["all", "metric", "streaming", "stepwise", "hbm_kernels", "copy", "configs"],
+                    default="all",
                     help="restrict the run to one workload (for profiling); the JSON line is "
                          "only complete with 'all'.  'copy' runs a plain device copy of known "
                          "size, the yardstick for the FETCH_SIZE / WRITE_SIZE counters")
@@ -225,6 +226,71 @@ def run_stepwise(args, torch, lib, ops, dev):
                          "traffic": MEASURED_TRAFFIC_BYTES.get("gemm_f32_skinny")}}
 
 
+def run_hbm_kernels(args, torch, lib, ops, dev):
+    """The HBM-bound kernels of the path against the 8 TB/s roof: stand-alone layer norm
+    (rows = T*N of BASELINE configuration 4, D = 4H), IndRNN recurrences and the transpose
+    helper.  Algorithmic bytes: each distinct tensor element read or written once."""
+    out = {}
+
+    def timed(names, fn, reps=20):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        lib.haste_hip_profile_reset()
+        lib.haste_hip_profile_enable(1)
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        lib.haste_hip_profile_enable(0)
+        res = {}
+        for name in names:
+            ms, n = profile_read(lib, name)
+            res[name] = ms / max(n, 1)
+        lib.haste_hip_profile_reset()
+        return res
+
+    def entry(ms, nbytes):
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        return {"us": round(ms * 1e3, 2), "bytes": nbytes, "bound": "hbm", "achieved": round(gbs, 1),
+                "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4)}
+
+    rows, D = 500 * 32, 1024
+    x = torch.randn(rows, D, device=dev)
+    dy = torch.randn(rows, D, device=dev)
+    gamma = torch.rand(D, device=dev) + 0.5
+    cache = [None]
+
+    def ln():
+        y, cache[0] = ops.layer_norm_forward(x, gamma, None)
+        ops.layer_norm_backward(x, gamma, dy, cache[0], False)
+    t = timed(("layer_norm_forward", "layer_norm_backward"), ln)
+    out["layer_norm_forward_16000x1024"] = entry(t["layer_norm_forward"], 4.0 * (2 * rows * D + 2 * rows))
+    out["layer_norm_backward_16000x1024"] = entry(t["layer_norm_backward"], 4.0 * 3 * rows * D)
+
+    T, N, C, H = 100, 64, 512, 512
+    xs = torch.randn(T, N, C, device=dev)
+    W = (torch.rand(C, H, device=dev) - 0.5) * H ** -0.5
+    u = torch.rand(H, device=dev) - 0.5
+    b = torch.zeros(H, device=dev)
+    h0 = torch.zeros(N, H, device=dev)
+    dh_new = torch.randn(T + 1, N, H, device=dev)
+    no_mask = torch.empty(0, 0, 0, device=dev)
+    x_t, W_t = ops.transpose(xs), ops.transpose(W)
+
+    def ind():
+        h = ops.indrnn_forward(True, 0.0, xs, h0, W, u, b, no_mask)
+        ops.indrnn_backward(x_t, W_t, u, b, no_mask, h, dh_new)
+    t = timed(("indrnn_forward_recurrence", "indrnn_backward_recurrence"), ind)
+    # forward: x*W in, h out; backward: h (twice: h_t, h_{t+1} are the same tensor) and
+    # dh_new in, the gradient w.r.t. x*W out
+    out["indrnn_forward_N64_T100_H512"] = entry(t["indrnn_forward_recurrence"], 4.0 * 2 * T * N * H)
+    out["indrnn_backward_N64_T100_H512"] = entry(t["indrnn_backward_recurrence"], 4.0 * 3 * T * N * H)
+
+    t = timed(("transpose_f32",), lambda: ops.transpose(xs))
+    out["transpose_6400x512"] = entry(t["transpose_f32"], 4.0 * 2 * T * N * C)
+    return out
+
+
 def run_configs(args, torch, lib, ops, dev):
     """The other BASELINE.json configurations (parity-test cases; timed here for the record):
     forward (+ backward with the caller-side transposes) in ms per call."""
@@ -342,10 +408,14 @@ def main():
     if args.workload == "stepwise":
         print(json.dumps(run_stepwise(args, torch, lib, ops, dev)))
         return
+    if args.workload == "hbm_kernels":
+        print(json.dumps(run_hbm_kernels(args, torch, lib, ops, dev)))
+        return
 
     m = run_metric(args, torch, lib, ops, dev)
     streaming, host1 = run_streaming(args, torch, lib, ops, dev)
     stepwise = run_stepwise(args, torch, lib, ops, dev)
+    hbm_kernels = run_hbm_kernels(args, torch, lib, ops, dev)
 
     # CPU baseline: torch.nn.LSTM fwd+bwd on the host cores (bounded sample).
     cpu = None
@@ -376,6 +446,7 @@ def main():
         "kernels": m["kernels"],
         "streaming_n1": streaming,
         "stepwise_n1_h4096": stepwise,
+        "hbm_kernels": hbm_kernels,
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))

@@ -118,9 +118,7 @@ template <int E, bool VEC>
 __global__ __launch_bounds__(256)
 void layer_norm_backward_kernel(int rows, int D, const float* __restrict__ gamma,
                                 const float* x, const float* dy, float* dx,
-                                float* __restrict__ dgamma, float* __restrict__ dbeta,
-                                float* __restrict__ partial, ControlBlock* cb) {
-  __shared__ unsigned int s_flag;
+                                float* __restrict__ partial) {
   extern __shared__ __attribute__((aligned(16))) float lds[];  // [4][2][E*64]
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -177,13 +175,35 @@ void layer_norm_backward_kernel(int rows, int D, const float* __restrict__ gamma
       part[which * D + c] = s;
     }
   }
-  if (grid_last_arrival(cb, gridDim.x, &s_flag)) {
-    for (int c = threadIdx.x; c < 2 * D; c += 256) {
-      float s = 0.f;
-      for (int b = 0; b < (int)gridDim.x; ++b) s += partial[(size_t)b * 2 * D + c];
-      if (c < D) dgamma[c] += s;
-      else if (dbeta != nullptr) dbeta[c - D] += s;
+}
+
+// dgamma (and dbeta) += the workgroups' column sums, added in workgroup order.  A thread owns
+// one column and every fourth workgroup; the four partial sums of a column are then combined
+// in a fixed order, so the result does not depend on timing.
+__global__ __launch_bounds__(256)
+void layer_norm_reduce_kernel(int parts, int D, const float* __restrict__ partial,
+                              float* __restrict__ dgamma, float* __restrict__ dbeta) {
+  __shared__ float sums[4][64];
+  const int c = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int q = threadIdx.x >> 6;
+  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  if (c < 2 * D) {
+    int b = q;
+    for (; b + 12 < parts; b += 16) {  // four loads in flight
+      s0 += partial[(size_t)b * 2 * D + c];
+      s1 += partial[(size_t)(b + 4) * 2 * D + c];
+      s2 += partial[(size_t)(b + 8) * 2 * D + c];
+      s3 += partial[(size_t)(b + 12) * 2 * D + c];
     }
+    for (; b < parts; b += 4) s0 += partial[(size_t)b * 2 * D + c];
+  }
+  sums[q][threadIdx.x & 63] = (s0 + s1) + (s2 + s3);
+  __syncthreads();
+  if (q == 0 && c < 2 * D) {
+    const int l = threadIdx.x & 63;
+    const float s = (sums[0][l] + sums[1][l]) + (sums[2][l] + sums[3][l]);
+    if (c < D) dgamma[c] += s;
+    else if (dbeta != nullptr) dbeta[c - D] += s;
   }
 }
 
@@ -243,13 +263,16 @@ int layer_norm_backward(hipStream_t stream, int rows, int dim, const float* gamm
         reinterpret_cast<const void*>(layer_norm_backward_kernel<E_, VEC_>),              \
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                           \
     layer_norm_backward_kernel<E_, VEC_><<<dim3(grid), dim3(256), lds, stream>>>(         \
-        rows, dim, gamma, x, dy, dx, dgamma, dbeta, ws.scratch, ws.control);              \
+        rows, dim, gamma, x, dy, dx, ws.scratch);                                          \
   }
   HASTE_LN_BWD(4, true) HASTE_LN_BWD(8, true) HASTE_LN_BWD(16, true) HASTE_LN_BWD(32, true)
   HASTE_LN_BWD(64, true)
   HASTE_LN_BWD(1, false) HASTE_LN_BWD(2, false) HASTE_LN_BWD(4, false) HASTE_LN_BWD(8, false)
   HASTE_LN_BWD(16, false)
 #undef HASTE_LN_BWD
+  HASTE_HIP_TRY(hipGetLastError());
+  layer_norm_reduce_kernel<<<dim3((unsigned)((2 * dim + 63) / 64)), dim3(256), 0, stream>>>(
+      grid, dim, ws.scratch, dgamma, dbeta);
   HASTE_HIP_TRY(hipGetLastError());
   return HASTE_HIP_OK;
 }
