@@ -897,6 +897,12 @@ inline int plan_launch(hipStream_t stream, const Workspace& ws, int gx, int gy, 
   return HASTE_HIP_OK;
 }
 
+// Dynamic LDS a persistent kernel may ask for: the 160 KiB of a gfx950 workgroup less room
+// for the kernels' few statically allocated words (role, flag), which count against the
+// same limit.  A kernel without static LDS may ask for all of it.
+constexpr size_t kWorkgroupLdsBytes = 160 * 1024;
+constexpr size_t kMaxLdsBytes = kWorkgroupLdsBytes - 256;
+
 // Launches a persistent kernel whose workgroups wait for each other, so all of them must
 // be resident at once: the grid is checked against what the chip can hold.  It is an
 // ordinary launch, not hipLaunchCooperativeKernel: the cooperative queue can be held by only
@@ -908,11 +914,26 @@ inline int plan_launch(hipStream_t stream, const Workspace& ws, int gx, int gy, 
 template <typename KernelT, typename ParamsT>
 int launch_persistent(const char* name, KernelT kernel, const LaunchPlan& plan, ParamsT& params,
                       hipStream_t stream) {
-  HASTE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)plan.lds_bytes));
-  int per_cu = 0;
-  HASTE_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, plan.lds_bytes));
+  // The attribute and the occupancy of (kernel, LDS request) are looked up once per thread
+  // and device: single-step callers (Iterate) launch the same kernel over and over.
+  struct Known { const void* kernel; size_t lds; int device; int per_cu; };
+  thread_local Known known[8] = {};
+  thread_local int next_slot = 0;
+  int device = 0;
+  HASTE_HIP_TRY(hipGetDevice(&device));
+  const void* fn = reinterpret_cast<const void*>(kernel);
+  int per_cu = -1;
+  for (const Known& k : known)
+    if (k.kernel == fn && k.lds == plan.lds_bytes && k.device == device) per_cu = k.per_cu;
+  if (per_cu < 0) {
+    // The limit is a property of the kernel, not of the launch: it is only ever raised (a
+    // later launch with a smaller, already known request must not find it lowered).
+    const size_t limit = plan.lds_bytes > kMaxLdsBytes ? plan.lds_bytes : kMaxLdsBytes;
+    HASTE_HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)limit));
+    HASTE_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, plan.lds_bytes));
+    known[next_slot] = Known{fn, plan.lds_bytes, device, per_cu};
+    next_slot = (next_slot + 1) % 8;
+  }
   const long long capacity = (long long)per_cu * device_cu_count();
   if ((long long)plan.grid.x * plan.grid.y > capacity) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   HASTE_HIP_PROPAGATE(order_persistent_launches(stream, true));
@@ -925,11 +946,6 @@ int launch_persistent(const char* name, KernelT kernel, const LaunchPlan& plan, 
   return HASTE_HIP_OK;
 }
 
-// Dynamic LDS a persistent kernel may ask for: the 160 KiB of a gfx950 workgroup less room
-// for the kernels' few statically allocated words (role, flag), which count against the
-// same limit.  A kernel without static LDS may ask for all of it.
-constexpr size_t kWorkgroupLdsBytes = 160 * 1024;
-constexpr size_t kMaxLdsBytes = kWorkgroupLdsBytes - 256;
 
 // Floats of the exchange tiles (2 behind a step barrier, kPolledTiles when polled) of every
 // group (batch tile) for contraction length K.
