@@ -66,6 +66,25 @@ def test_null_pointers_and_bad_dimensions_are_rejected_on_the_host(lib):
     assert _call(lib, "haste_hip_layer_norm_gru_forward_f32", 1, 3, 2, 2, 2, *([None] * 15), 0.0, None, None) == INVALID
 
 
+def test_double_and_half_entry_points_reject_bad_arguments_too(lib):
+    INVALID = 1
+    for sfx in ("_f64", "_f16"):
+        assert _call(lib, "haste_hip_gemm" + sfx, 0, 4, 4, 4, None, 4, None, 4, None, 4, 0, None) == INVALID
+        assert _call(lib, "haste_hip_transpose" + sfx, 4, 4, None, None, None) == INVALID
+        assert _call(lib, "haste_hip_gru_forward" + sfx, 1, 0, 1, 1, 1, *([None] * 9), 0.0, None, None) == INVALID
+        assert _call(lib, "haste_hip_gru_forward" + sfx, 1, 3, 2, 2, 2, *([None] * 9), 0.0, None, None) == INVALID
+        assert _call(lib, "haste_hip_gru_backward" + sfx, 3, 2, 2, 2, *([None] * 17), None) == INVALID
+    assert _call(lib, "haste_hip_lstm_forward_f64", 1, 3, 2, 2, 2, *([None] * 8), 0.0, None, None) == INVALID
+    assert _call(lib, "haste_hip_lstm_backward_f64", 3, 2, 2, 2, *([None] * 16), None) == INVALID
+    assert _call(lib, "haste_hip_layer_norm_forward_f64", 4, 8, *([None] * 5), None) == INVALID
+    assert _call(lib, "haste_hip_layer_norm_backward_f64", 4, 8, *([None] * 7), None) == INVALID
+    assert _call(lib, "haste_hip_indrnn_forward_f64", 1, 3, 2, 2, 2, *([None] * 6), 0.0, None, None) == INVALID
+    assert _call(lib, "haste_hip_layer_norm_lstm_forward_f64", 1, 3, 2, 2, 2, *([None] * 18), 0.0, None, None) == INVALID
+    assert _call(lib, "haste_hip_layer_norm_gru_forward_f64", 1, 3, 2, 2, 2, *([None] * 15), 0.0, None, None) == INVALID
+    # as in the reference, half exists for the GRU only
+    assert not hasattr(lib, "haste_hip_lstm_forward_f16")
+
+
 def test_cpp_headers_declare_the_reference_class_surface():
     """include/haste/*.h keeps the reference's namespaces and class names."""
     for ns in ("lstm", "gru", "indrnn", "layer_norm", "layer_norm_lstm", "layer_norm_gru",
