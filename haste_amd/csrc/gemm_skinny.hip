@@ -1,4 +1,4 @@
-// C[M,N] (+)= A[M,K] * B[K,N] for M <= 32: the recurrent product of one step (h_t * R,
+// C[M,N] (+)= A[M,K] * B[K,N] for M <= 64: the recurrent product of one step (h_t * R,
 // delta_t * R^T) when R is streamed from HBM every step (stepwise.hip) and the batch is
 // small.  Replaces the per-step cublasSgemm of the reference
 // (lib/lstm_forward_gpu.cu.cc:232-242, lib/lstm_backward_gpu.cu.cc:281-291).
@@ -11,7 +11,8 @@
 // interleaved by 4 -- which is exactly a 16-byte store per lane in the epilogue.  M <= 16
 // uses v_mfma_f32_16x16x4_f32 (4 k rows x 64 columns per load), M <= 32 v_mfma_f32_32x32x2_f32
 // (2 k rows x 128 columns); the matrix cores then need 128 / 256 cycles per KiB of B, below
-// the 330 cycles a CU's share of 8 TB/s allows.  The four wavefronts of a workgroup split the
+// the 330 cycles a CU's share of 8 TB/s allows.  M <= 64 carries two blocks of 32 rows on the
+// same B registers: bound by the matrix cores, but still without LDS traffic or tile pieces.  The four wavefronts of a workgroup split the
 // workgroup's k range and add their tiles through LDS in wavefront order; workgroups split K
 // further (enough of them to keep every CU's memory pipeline full); their tiles are added in
 // chunk order by a second small kernel, or by the consumer of the product itself
@@ -49,7 +50,9 @@ template <> struct SkinnyShape<32> {
 
 constexpr int kUnroll = 8;  // load instructions in flight per wavefront and operand
 
-template <int MT>
+// MT: rows of one MFMA tile (16 or 32); RB: row blocks of MT rows a wavefront carries (the
+// B registers are shared between them), so a workgroup covers MT*RB rows of A.
+template <int MT, int RB>
 __global__ __launch_bounds__(256)
 void skinny_kernel(int M, int N, int K, const float* __restrict__ A, int lda,
                    const float* __restrict__ B, int ldb, float* __restrict__ C, int ldc,
@@ -68,16 +71,24 @@ void skinny_kernel(int M, int N, int K, const float* __restrict__ A, int lda,
 
   const int i = lane % MT, kq = lane / MT;
   const int col = n0 + 4 * (lane % MT);
-  const bool col_ok = col < N, row_ok = i < M;
+  const bool col_ok = col < N;
   // Out-of-range lanes load from a valid address and drop the value.
-  const float* ap = A + (size_t)(row_ok ? i : 0) * lda;
+  bool row_ok[RB];
+  const float* ap[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    row_ok[rb] = rb * MT + i < M;
+    ap[rb] = A + (size_t)(row_ok[rb] ? rb * MT + i : 0) * lda;
+  }
   const float* bp = B + (col_ok ? col : 0);
 
-  Acc acc[4];
+  Acc acc[RB][4];
 #pragma unroll
-  for (int c = 0; c < 4; ++c)
+  for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-    for (int e = 0; e < S::kAccElems; ++e) acc[c][e] = 0.f;
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+      for (int e = 0; e < S::kAccElems; ++e) acc[rb][c][e] = 0.f;
 
   // A batch is kUnroll MFMA steps.  Which k a lane contributes at which step is free as long
   // as both operands agree: lane group kq takes the run of kUnroll consecutive k starting at
@@ -86,14 +97,16 @@ void skinny_kernel(int M, int N, int K, const float* __restrict__ A, int lda,
   for (int k = kb; k < ke; k += S::kStep * kUnroll) {
     const int k_mine = k + kUnroll * kq;
     float4_t b[kUnroll];
-    float4_t a4[kUnroll / 4];
+    float4_t a4[RB][kUnroll / 4];
 #pragma unroll
-    for (int j = 0; j < kUnroll / 4; ++j) {
-      const int g = k_mine + 4 * j;
-      const bool ok = g < ke;
-      const float4_t av = *reinterpret_cast<const float4_t*>(ap + (ok ? g : kb));
-      a4[j] = (ok && row_ok) ? av : float4_t{0.f, 0.f, 0.f, 0.f};
-    }
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int j = 0; j < kUnroll / 4; ++j) {
+        const int g = k_mine + 4 * j;
+        const bool ok = g < ke;
+        const float4_t av = *reinterpret_cast<const float4_t*>(ap[rb] + (ok ? g : kb));
+        a4[rb][j] = (ok && row_ok[rb]) ? av : float4_t{0.f, 0.f, 0.f, 0.f};
+      }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       const int r = k_mine + u;
@@ -102,38 +115,47 @@ void skinny_kernel(int M, int N, int K, const float* __restrict__ A, int lda,
       b[u] = (ok && col_ok) ? bv : float4_t{0.f, 0.f, 0.f, 0.f};
     }
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const float a = a4[u / 4][u % 4];
-      acc[0] = S::mfma(a, b[u].x, acc[0]);
-      acc[1] = S::mfma(a, b[u].y, acc[1]);
-      acc[2] = S::mfma(a, b[u].z, acc[2]);
-      acc[3] = S::mfma(a, b[u].w, acc[3]);
-    }
+    for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const float a = a4[rb][u / 4][u % 4];
+        acc[rb][0] = S::mfma(a, b[u].x, acc[rb][0]);
+        acc[rb][1] = S::mfma(a, b[u].y, acc[rb][1]);
+        acc[rb][2] = S::mfma(a, b[u].z, acc[rb][2]);
+        acc[rb][3] = S::mfma(a, b[u].w, acc[rb][3]);
+      }
   }
 
-  // Element e of the four accumulators = four consecutive columns of one row.
+  // Element e of the four accumulators = four consecutive columns of one row.  The
+  // wavefronts' tiles are added through LDS, one row block at a time.
   const int cslot = 4 * (lane % MT);
-  if (wave > 0) {
 #pragma unroll
-    for (int e = 0; e < S::kAccElems; ++e)
-      *reinterpret_cast<float4_t*>(&red[wave - 1][S::row(lane, e)][cslot]) =
-          float4_t{acc[0][e], acc[1][e], acc[2][e], acc[3][e]};
-  }
-  __syncthreads();
-  if (wave > 0 || !col_ok) return;
+  for (int rb = 0; rb < RB; ++rb) {
+    if (rb > 0) __syncthreads();  // wavefront 0 has read the previous block's tiles
+    if (wave > 0) {
 #pragma unroll
-  for (int e = 0; e < S::kAccElems; ++e) {
-    const int row = S::row(lane, e);
-    if (row >= M) continue;
-    float4_t s = float4_t{acc[0][e], acc[1][e], acc[2][e], acc[3][e]};
-    s += *reinterpret_cast<const float4_t*>(&red[0][row][cslot]);
-    s += *reinterpret_cast<const float4_t*>(&red[1][row][cslot]);
-    s += *reinterpret_cast<const float4_t*>(&red[2][row][cslot]);
-    if (partial != nullptr) {
-      *reinterpret_cast<float4_t*>(partial + ((size_t)chunk * M + row) * N + col) = s;
-    } else {
-      float4_t* o = reinterpret_cast<float4_t*>(C + (size_t)row * ldc + col);
-      *o = accumulate ? (*o + s) : s;
+      for (int e = 0; e < S::kAccElems; ++e)
+        *reinterpret_cast<float4_t*>(&red[wave - 1][S::row(lane, e)][cslot]) =
+            float4_t{acc[rb][0][e], acc[rb][1][e], acc[rb][2][e], acc[rb][3][e]};
+    }
+    __syncthreads();
+    if (wave == 0 && col_ok) {
+#pragma unroll
+      for (int e = 0; e < S::kAccElems; ++e) {
+        const int in_block = S::row(lane, e);
+        const int row = rb * MT + in_block;
+        if (row >= M) continue;
+        float4_t s = float4_t{acc[rb][0][e], acc[rb][1][e], acc[rb][2][e], acc[rb][3][e]};
+        s += *reinterpret_cast<const float4_t*>(&red[0][in_block][cslot]);
+        s += *reinterpret_cast<const float4_t*>(&red[1][in_block][cslot]);
+        s += *reinterpret_cast<const float4_t*>(&red[2][in_block][cslot]);
+        if (partial != nullptr) {
+          *reinterpret_cast<float4_t*>(partial + ((size_t)chunk * M + row) * N + col) = s;
+        } else {
+          float4_t* o = reinterpret_cast<float4_t*>(C + (size_t)row * ldc + col);
+          *o = accumulate ? (*o + s) : s;
+        }
+      }
     }
   }
 }
@@ -154,12 +176,13 @@ void skinny_reduce_kernel(int M, int N, int chunks, const float* __restrict__ pa
 }
 
 struct SkinnyPlan {
-  int mt, col_blocks, chunks, k_per_wg;
+  int mt, rb, col_blocks, chunks, k_per_wg;  // MFMA tile rows, row blocks
 };
 
 SkinnyPlan plan_skinny(int M, int N, int K) {
   SkinnyPlan p;
   p.mt = M <= 16 ? 16 : 32;
+  p.rb = M <= 32 ? 1 : 2;
   const int cols = 4 * p.mt;
   p.col_blocks = (N + cols - 1) / cols;
   // Enough workgroups for about three per CU (measured: four is no faster at 268 MB of B and
@@ -177,10 +200,25 @@ SkinnyPlan plan_skinny(int M, int N, int K) {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+void launch_skinny(const SkinnyPlan& p, dim3 grid, hipStream_t stream, int M, int N, int K,
+                   const float* A, int lda, const float* B, int ldb, float* C, int ldc,
+                   int accumulate, float* partial) {
+  if (p.mt == 16)
+    skinny_kernel<16, 1><<<grid, dim3(256), 0, stream>>>(M, N, K, A, lda, B, ldb, C, ldc, accumulate, p.k_per_wg, partial);
+  else if (p.rb == 1)
+    skinny_kernel<32, 1><<<grid, dim3(256), 0, stream>>>(M, N, K, A, lda, B, ldb, C, ldc, accumulate, p.k_per_wg, partial);
+  else
+    skinny_kernel<32, 2><<<grid, dim3(256), 0, stream>>>(M, N, K, A, lda, B, ldb, C, ldc, accumulate, p.k_per_wg, partial);
+}
+
 }  // namespace
 
 bool gemm_f32_skinny_shape(bool trans_a, int M, int N, int K) {
-  return !trans_a && M <= 32 && N % 4 == 0 && K % 4 == 0 && K >= 64 && (long long)K * N >= (1ll << 16);
+  if (trans_a || M > 64 || N % 4 != 0 || K % 4 != 0 || K < 64 || (long long)K * N < (1ll << 16)) return false;
+  // 33..64 rows are bound by the matrix cores; measured against the tile kernel they win while
+  // B is small (the tile kernel then has too few tiles and pays for its pieces): up to 6 Mi
+  // elements, e.g. the reverse step of H = 1024 (4096 x 1024).
+  return M <= 32 || (long long)K * N <= 6ll * (1 << 20);
 }
 
 size_t gemm_f32_skinny_scratch_bytes(int M, int N, int K) {
@@ -205,10 +243,7 @@ int gemm_f32_skinny_chunks(hipStream_t stream, int M, int N, int K, const float*
   float* part = ws.scratch + scratch_offset / sizeof(float);
   const dim3 grid((unsigned)p.col_blocks, (unsigned)p.chunks);
   ScopedKernelTimer timer("gemm_f32_skinny", stream);
-  if (p.mt == 16)
-    skinny_kernel<16><<<grid, dim3(256), 0, stream>>>(M, N, K, A, lda, B, ldb, nullptr, 0, 0, p.k_per_wg, part);
-  else
-    skinny_kernel<32><<<grid, dim3(256), 0, stream>>>(M, N, K, A, lda, B, ldb, nullptr, 0, 0, p.k_per_wg, part);
+  launch_skinny(p, grid, stream, M, N, K, A, lda, B, ldb, nullptr, 0, 0, part);
   HASTE_HIP_TRY(hipGetLastError());
   *partial = part;
   *chunks = p.chunks;
@@ -228,10 +263,7 @@ int gemm_f32_skinny(hipStream_t stream, int M, int N, int K, const float* A, int
   const dim3 grid((unsigned)p.col_blocks, (unsigned)p.chunks);
   {
     ScopedKernelTimer timer("gemm_f32_skinny", stream);
-    if (p.mt == 16)
-      skinny_kernel<16><<<grid, dim3(256), 0, stream>>>(M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, p.k_per_wg, partial);
-    else
-      skinny_kernel<32><<<grid, dim3(256), 0, stream>>>(M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, p.k_per_wg, partial);
+    launch_skinny(p, grid, stream, M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, partial);
     HASTE_HIP_TRY(hipGetLastError());
   }
   if (partial != nullptr) {
