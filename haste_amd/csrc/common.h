@@ -99,7 +99,7 @@ int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
 // Bytes of scratch gemm_f32 may use for this shape (0 when nothing is split).
 size_t gemm_f32_scratch_bytes(int M, int N, int K);
 
-// The product for M <= 64 with B streamed from HBM straight into the MFMA operands
+// The product for M <= 128 with B streamed from HBM straight into the MFMA operands
 // (gemm_skinny.hip); gemm_f32 hands such shapes over when the operands are 16-byte aligned.
 bool gemm_f32_skinny_shape(bool trans_a, int M, int N, int K);
 bool gemm_f32_skinny_applies(bool trans_a, int M, int N, int K, const float* A, int lda,

@@ -1,4 +1,4 @@
-// C[M,N] (+)= A[M,K] * B[K,N] for M <= 64: the recurrent product of one step (h_t * R,
+// C[M,N] (+)= A[M,K] * B[K,N] for M <= 128: the recurrent product of one step (h_t * R,
 // delta_t * R^T) when R is streamed from HBM every step (stepwise.hip) and the batch is
 // small.  Replaces the per-step cublasSgemm of the reference
 // (lib/lstm_forward_gpu.cu.cc:232-242, lib/lstm_backward_gpu.cu.cc:281-291).
@@ -70,6 +70,7 @@ void skinny_kernel(int M, int N, int K, const float* __restrict__ A, int lda,
   const int ke = kb + k_per_wave < ke_wg ? kb + k_per_wave : ke_wg;
 
   const int i = lane % MT, kq = lane / MT;
+  const int m0 = blockIdx.z * (MT * RB);  // more than MT*RB rows: one grid layer per group of rows
   const int col = n0 + 4 * (lane % MT);
   const bool col_ok = col < N;
   // Out-of-range lanes load from a valid address and drop the value.
@@ -77,8 +78,8 @@ void skinny_kernel(int M, int N, int K, const float* __restrict__ A, int lda,
   const float* ap[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    row_ok[rb] = rb * MT + i < M;
-    ap[rb] = A + (size_t)(row_ok[rb] ? rb * MT + i : 0) * lda;
+    row_ok[rb] = m0 + rb * MT + i < M;
+    ap[rb] = A + (size_t)(row_ok[rb] ? m0 + rb * MT + i : 0) * lda;
   }
   const float* bp = B + (col_ok ? col : 0);
 
@@ -143,7 +144,7 @@ void skinny_kernel(int M, int N, int K, const float* __restrict__ A, int lda,
 #pragma unroll
       for (int e = 0; e < S::kAccElems; ++e) {
         const int in_block = S::row(lane, e);
-        const int row = rb * MT + in_block;
+        const int row = m0 + rb * MT + in_block;
         if (row >= M) continue;
         float4_t s = float4_t{acc[rb][0][e], acc[rb][1][e], acc[rb][2][e], acc[rb][3][e]};
         s += *reinterpret_cast<const float4_t*>(&red[0][in_block][cslot]);
@@ -176,19 +177,20 @@ void skinny_reduce_kernel(int M, int N, int chunks, const float* __restrict__ pa
 }
 
 struct SkinnyPlan {
-  int mt, rb, col_blocks, chunks, k_per_wg;  // MFMA tile rows, row blocks
+  int mt, rb, row_groups, col_blocks, chunks, k_per_wg;  // MFMA tile rows, row blocks, grid layers
 };
 
 SkinnyPlan plan_skinny(int M, int N, int K) {
   SkinnyPlan p;
   p.mt = M <= 16 ? 16 : 32;
   p.rb = M <= 32 ? 1 : 2;
+  p.row_groups = (M + p.mt * p.rb - 1) / (p.mt * p.rb);
   const int cols = 4 * p.mt;
   p.col_blocks = (N + cols - 1) / cols;
   // Enough workgroups for about three per CU (measured: four is no faster at 268 MB of B and
   // slower when B fits the memory-side cache), a workgroup keeping at least 128 of K.
   const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
-  int chunks = (3 * cus + p.col_blocks - 1) / p.col_blocks;
+  int chunks = (3 * cus + p.col_blocks * p.row_groups - 1) / (p.col_blocks * p.row_groups);
   const int most = (K + 127) / 128;
   if (chunks > most) chunks = most;
   if (chunks < 1) chunks = 1;
@@ -214,9 +216,9 @@ void launch_skinny(const SkinnyPlan& p, dim3 grid, hipStream_t stream, int M, in
 }  // namespace
 
 bool gemm_f32_skinny_shape(bool trans_a, int M, int N, int K) {
-  if (trans_a || M > 64 || N % 4 != 0 || K % 4 != 0 || K < 64 || (long long)K * N < (1ll << 16)) return false;
-  // 33..64 rows are bound by the matrix cores; measured against the tile kernel they win while
-  // B is small (the tile kernel then has too few tiles and pays for its pieces): up to 6 Mi
+  if (trans_a || M > 128 || N % 4 != 0 || K % 4 != 0 || K < 64 || (long long)K * N < (1ll << 16)) return false;
+  // 33..128 rows (65 and up as two grid layers of 64) are bound by the matrix cores; measured
+  // against the tile kernel they win while B is small (the tile kernel then has too few tiles and pays for its pieces): up to 6 Mi
   // elements, e.g. the reverse step of H = 1024 (4096 x 1024).
   return M <= 32 || (long long)K * N <= 6ll * (1 << 20);
 }
@@ -241,7 +243,7 @@ int gemm_f32_skinny_chunks(hipStream_t stream, int M, int N, int K, const float*
   Workspace ws;
   HASTE_HIP_PROPAGATE(get_workspace(stream, scratch_offset + (size_t)p.chunks * M * N * sizeof(float), &ws));
   float* part = ws.scratch + scratch_offset / sizeof(float);
-  const dim3 grid((unsigned)p.col_blocks, (unsigned)p.chunks);
+  const dim3 grid((unsigned)p.col_blocks, (unsigned)p.chunks, (unsigned)p.row_groups);
   ScopedKernelTimer timer("gemm_f32_skinny", stream);
   launch_skinny(p, grid, stream, M, N, K, A, lda, B, ldb, nullptr, 0, 0, part);
   HASTE_HIP_TRY(hipGetLastError());
@@ -260,7 +262,7 @@ int gemm_f32_skinny(hipStream_t stream, int M, int N, int K, const float* A, int
     HASTE_HIP_PROPAGATE(get_workspace(stream, scratch_offset + gemm_f32_skinny_scratch_bytes(M, N, K), &ws));
     partial = ws.scratch + scratch_offset / sizeof(float);
   }
-  const dim3 grid((unsigned)p.col_blocks, (unsigned)p.chunks);
+  const dim3 grid((unsigned)p.col_blocks, (unsigned)p.chunks, (unsigned)p.row_groups);
   {
     ScopedKernelTimer timer("gemm_f32_skinny", stream);
     launch_skinny(p, grid, stream, M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, partial);

@@ -16,7 +16,8 @@ SHAPES = [
     (False, 6400, 512, 2048),   # dx
     (False, 96, 96, 5000),      # split-K with ragged tiles
     # M <= 64 with a long enough K: the kernel that streams B into the MFMA operands
-    (False, 64, 1024, 4096), (False, 47, 6144, 1536), (False, 33, 772, 3000),
+    (False, 64, 1024, 4096), (False, 47, 6144, 1536), (False, 33, 772, 3000), (False, 128, 1024, 4096),
+    (False, 100, 768, 3072),
     (False, 1, 2048, 512), (False, 16, 6144, 1536), (False, 5, 1300, 5200), (False, 32, 768, 3072),
     (False, 17, 4100, 332), (False, 3, 64, 1024), (False, 32, 16384, 1000),
 ]
