@@ -321,7 +321,8 @@ GemmPlan plan_gemm(int M, int N, int K) {
   // pieces per tile cost ceil(rest*s/CUs)/s for the arithmetic plus 0.25*rest*s/K for
   // writing and re-reading the partial tiles (128 KiB per piece at the chip's memory rate
   // against 2*128*128*K flops at one CU's MFMA rate); a launch that consists of fewer than
-  // two pieces per CU pays 12 % more (a lone workgroup cannot hide its own load latency).
+  // two pieces per CU pays 20 % more (a lone workgroup cannot hide its own load latency;
+  // measured 5-9 % between 1 and 2 pieces per CU at 128 x 8192 x 2048 with the traffic term).
   // The cheapest s is taken, a piece keeping at least 64 of K.  The choice depends on the
   // shape only, so results are reproducible.
   const long long whole = tiles >= cus ? tiles / cus * cus : 0;
@@ -334,7 +335,7 @@ GemmPlan plan_gemm(int M, int N, int K) {
     auto cost = [&](int s) {
       const long long pieces = (long long)g.rest * s;
       double c = (double)((pieces + cus - 1) / cus) / s;
-      if (whole == 0 && pieces < 2LL * cus) c *= 1.12;
+      if (whole == 0 && pieces < 2LL * cus) c *= 1.2;
       if (s > 1) c += 0.25 * (double)g.rest * s / K;
       return c;
     };
