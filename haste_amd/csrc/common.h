@@ -96,6 +96,12 @@ int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
              const float* A, int lda, const float* B, int ldb,
              float* C, int ldc, bool accumulate, size_t scratch_offset = 0);
 
+// The product left as the K pieces of the tile kernel for a consumer that adds them itself;
+// *splits == 0 (and nothing launched) when the shape is not cut that way.  See gemm.hip.
+int gemm_f32_pieces(hipStream_t stream, int M, int N, int K, const float* A, int lda,
+                    const float* B, int ldb, size_t scratch_offset, const float** partial,
+                    int* splits, int* bm);
+
 // Bytes of scratch gemm_f32 may use for this shape (0 when nothing is split).
 size_t gemm_f32_scratch_bytes(int M, int N, int K);
 

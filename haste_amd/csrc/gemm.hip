@@ -415,6 +415,39 @@ int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
   return HASTE_HIP_OK;
 }
 
+// The product as its K pieces, for a consumer that adds them itself (in piece order): only the
+// tile kernel is launched.  Possible when every tile of the product is cut into pieces and
+// the output is one tile high; *splits == 0 otherwise (nothing launched).  Element (row, col)
+// of piece s lies at partial[((col / 128 * splits + s) * bm + row) * 128 + col % 128]; valid
+// until the next product on the stream.
+int gemm_f32_pieces(hipStream_t stream, int M, int N, int K, const float* A, int lda,
+                    const float* B, int ldb, size_t scratch_offset, const float** partial,
+                    int* splits, int* bm) {
+  *splits = 0;
+  HASTE_HIP_REQUIRE(M > 0 && N > 0 && K > 0 && A != nullptr && B != nullptr);
+  HASTE_HIP_REQUIRE(lda >= K && ldb >= N);
+  const GemmPlan g = plan_gemm(M, N, K);
+  if (g.splits <= 1 || g.whole_tiles != 0 || M > g.bm) return HASTE_HIP_OK;
+  if (((long long)g.bm * lda + K) * 4 >= (1ll << 31) || ((long long)K * ldb + BN) * 4 >= (1ll << 31))
+    return HASTE_HIP_OK;
+  Workspace ws;
+  HASTE_HIP_PROPAGATE(get_workspace(stream, scratch_offset + g.scratch_bytes, &ws));
+  float* part = ws.scratch + scratch_offset / sizeof(float);
+  dim3 grid((unsigned)g.pieces), block(256);
+  ScopedKernelTimer timer("gemm_f32", stream);
+  if (g.bm == 128)
+    gemm_f32_kernel<false, 128><<<grid, block, 0, stream>>>(M, N, K, A, lda, B, ldb, nullptr, 0, 0, g.tiles_n,
+                                                            0, g.splits, g.k_per_split, part);
+  else
+    gemm_f32_kernel<false, 64><<<grid, block, 0, stream>>>(M, N, K, A, lda, B, ldb, nullptr, 0, 0, g.tiles_n,
+                                                           0, g.splits, g.k_per_split, part);
+  HASTE_HIP_TRY(hipGetLastError());
+  *partial = part;
+  *splits = g.splits;
+  *bm = g.bm;
+  return HASTE_HIP_OK;
+}
+
 }  // namespace haste_hip
 
 extern "C" int haste_hip_gemm_f32(int trans_a, int M, int N, int K,

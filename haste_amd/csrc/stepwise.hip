@@ -84,20 +84,38 @@ struct StepProduct {
   const T* base = nullptr;
   int chunks = 0;
   size_t stride = 0;
+  // tile_rows != 0: the chunks are the K pieces of the tile kernel (gemm_f32_pieces), element
+  // (row, col) of piece k at base[((col / 128 * chunks + k) * tile_rows + row) * 128 + col % 128].
+  int tile_rows = 0;
+  int row_len = 0;
+
+  __device__ __forceinline__ size_t first(size_t idx) const {
+    if (tile_rows == 0) return idx;
+    const size_t row = idx / row_len, col = idx % row_len;
+    return ((col / 128 * chunks) * tile_rows + row) * 128 + col % 128;
+  }
+  __device__ __forceinline__ size_t step() const {
+    return tile_rows == 0 ? stride : (size_t)tile_rows * 128;
+  }
   // out[g] = the product at idx + g * gate_stride, g < G.  Chunks are added in index order;
   // the loads of two chunks and all G gates are issued together.
   template <int G>
   __device__ __forceinline__ void at(size_t idx, size_t gate_stride, typename Acc<T>::type (&out)[G]) const {
     typedef typename Acc<T>::type A;
+    size_t at0[G];
 #pragma unroll
-    for (int g = 0; g < G; ++g) out[g] = A(0);
+    for (int g = 0; g < G; ++g) {
+      out[g] = A(0);
+      at0[g] = first(idx + g * gate_stride);
+    }
+    const size_t st = step();
     int k = 0;
     for (; k + 2 <= chunks; k += 2) {
       A v0[G], v1[G];
 #pragma unroll
       for (int g = 0; g < G; ++g) {
-        v0[g] = (A)base[k * stride + idx + g * gate_stride];
-        v1[g] = (A)base[(k + 1) * stride + idx + g * gate_stride];
+        v0[g] = (A)base[at0[g] + k * st];
+        v1[g] = (A)base[at0[g] + (k + 1) * st];
       }
 #pragma unroll
       for (int g = 0; g < G; ++g) {
@@ -107,7 +125,7 @@ struct StepProduct {
     }
     if (k < chunks) {
 #pragma unroll
-      for (int g = 0; g < G; ++g) out[g] += (A)base[k * stride + idx + g * gate_stride];
+      for (int g = 0; g < G; ++g) out[g] += (A)base[at0[g] + k * st];
     }
   }
   __device__ __forceinline__ typename Acc<T>::type at(size_t idx) const {
@@ -134,6 +152,14 @@ int step_product<float>(hipStream_t s, int M, int N, int K, const float* A, cons
   if (gemm_f32_skinny_applies(false, M, N, K, A, K, B, N, out, N)) {
     HASTE_HIP_PROPAGATE(gemm_f32_skinny_chunks(s, M, N, K, A, K, B, N, scratch_offset, &p->base, &p->chunks));
     p->stride = (size_t)M * N;
+    return HASTE_HIP_OK;
+  }
+  int splits = 0, bm = 0;
+  HASTE_HIP_PROPAGATE(gemm_f32_pieces(s, M, N, K, A, K, B, N, scratch_offset, &p->base, &splits, &bm));
+  if (splits > 0) {
+    p->chunks = splits;
+    p->tile_rows = bm;
+    p->row_len = N;
     return HASTE_HIP_OK;
   }
   HASTE_HIP_PROPAGATE(gemm_f32(s, false, M, N, K, A, K, B, N, out, N, false, scratch_offset));
@@ -163,10 +189,18 @@ int reverse_product(hipStream_t s, int M, int N, int K, const T* A, const T* B, 
 template <>
 int reverse_product<float>(hipStream_t s, int M, int N, int K, const float* A, const float* B,
                            float* dh, size_t scratch_offset, StepProduct<float>* pend) {
-  pend->chunks = 0;
+  *pend = StepProduct<float>();
   if (gemm_f32_skinny_applies(false, M, N, K, A, K, B, N, dh, N)) {
     HASTE_HIP_PROPAGATE(gemm_f32_skinny_chunks(s, M, N, K, A, K, B, N, scratch_offset, &pend->base, &pend->chunks));
     pend->stride = (size_t)M * N;
+    return HASTE_HIP_OK;
+  }
+  int splits = 0, bm = 0;
+  HASTE_HIP_PROPAGATE(gemm_f32_pieces(s, M, N, K, A, K, B, N, scratch_offset, &pend->base, &splits, &bm));
+  if (splits > 0) {
+    pend->chunks = splits;
+    pend->tile_rows = bm;
+    pend->row_len = N;
     return HASTE_HIP_OK;
   }
   return gemm_f32(s, false, M, N, K, A, K, B, N, dh, N, true, scratch_offset);
