@@ -43,7 +43,7 @@ constexpr int kMaxWorkgroups = 2048;  // workgroups a persistent kernel may have
 constexpr int kCounterStride = 32;    // uint32 slots between counters (128 B apart)
 struct ControlBlock {
   unsigned int step_flags[kMaxWorkgroups];                 // per-workgroup arrival counts
-  unsigned int grid_exit_counter[kCounterStride];          // all workgroups of a launch
+  unsigned int grid_exit_counter[kCounterStride];          // unused (kept for the layout)
   unsigned int tile_counter[4096];                         // arrivals per column block at the end of a launch
   unsigned int xcd_ticket[16 * kCounterStride];            // per-XCD role tickets (only ever grow)
   unsigned int abort_flag[kCounterStride];                 // set when a barrier wait gives up
@@ -181,6 +181,12 @@ int layer_norm_forward(hipStream_t stream, int rows, int dim, const float* gamma
 int layer_norm_backward(hipStream_t stream, int rows, int dim, const float* gamma,
                         const float* x, const float* dy, float* dx, float* dgamma,
                         float* dbeta);
+
+// first[c] += sum over b < parts of partial[b][c], second[c] += ... of partial[b][D + c]
+// (partial is [parts][2][D]; second may be null), parts added in index order by a small
+// parallel kernel: the deterministic finish of column sums parked by many workgroups.
+int add_column_partials(hipStream_t stream, int parts, int D, const float* partial, float* first,
+                        float* second);
 
 // Brackets the launches made during its lifetime with a pair of events on `stream`
 // when profiling has been switched on (haste_hip_profile_enable); otherwise does

@@ -64,12 +64,9 @@ template <bool ZONEOUT>
 __global__ __launch_bounds__(256)
 void indrnn_backward_kernel(int T, int N, int H, const float* __restrict__ u,
                             const float* __restrict__ h, const float* __restrict__ dh_new,
-                            float* __restrict__ du, float* __restrict__ db,
                             float* __restrict__ dh, float* __restrict__ dk,
-                            const float* __restrict__ mask, float* __restrict__ partial,
-                            ControlBlock* cb) {
+                            const float* __restrict__ mask, float* __restrict__ partial) {
   __shared__ float red[2][4][64];
-  __shared__ unsigned int s_flag;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int j = blockIdx.x * 64 + lane;
   const int n = blockIdx.y * 4 + w;
@@ -130,15 +127,6 @@ void indrnn_backward_kernel(int T, int N, int H, const float* __restrict__ u,
     const float s = (red[which][0][lane] + red[which][1][lane]) + (red[which][2][lane] + red[which][3][lane]);
     if (j < H) partial[((size_t)blockIdx.y * 2 + which) * H + j] = s;
   }
-  if (grid_last_arrival(cb, gridDim.x * gridDim.y, &s_flag)) {
-    for (int c = threadIdx.x; c < 2 * H; c += 256) {
-      const int which = c / H, col = c % H;
-      float s = 0.f;
-      for (int by = 0; by < (int)gridDim.y; ++by) s += partial[((size_t)by * 2 + which) * H + col];
-      if (which == 0) du[col] += s;
-      else db[col] += s;
-    }
-  }
 }
 
 int run_forward_recurrence(hipStream_t stream, int training, int T, int N, int H, const float* Wx,
@@ -167,12 +155,12 @@ int run_backward_recurrence(hipStream_t stream, int T, int N, int H, const float
   HASTE_HIP_PROPAGATE(get_workspace(stream, (size_t)grid.y * 2 * H * sizeof(float), &ws));
   ScopedKernelTimer timer("indrnn_backward_recurrence", stream);
   if (mask != nullptr)
-    indrnn_backward_kernel<true><<<grid, block, 0, stream>>>(T, N, H, u, h, dh_new, du, db, dh, dk,
-                                                              mask, ws.scratch, ws.control);
+    indrnn_backward_kernel<true><<<grid, block, 0, stream>>>(T, N, H, u, h, dh_new, dh, dk, mask, ws.scratch);
   else
-    indrnn_backward_kernel<false><<<grid, block, 0, stream>>>(T, N, H, u, h, dh_new, du, db, dh, dk,
-                                                               nullptr, ws.scratch, ws.control);
+    indrnn_backward_kernel<false><<<grid, block, 0, stream>>>(T, N, H, u, h, dh_new, dh, dk, nullptr, ws.scratch);
   HASTE_HIP_TRY(hipGetLastError());
+  // du, db += the workgroups' column sums, in workgroup order
+  HASTE_HIP_PROPAGATE(add_column_partials(stream, (int)grid.y, H, ws.scratch, du, db));
   return HASTE_HIP_OK;
 }
 

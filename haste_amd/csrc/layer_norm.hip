@@ -219,6 +219,14 @@ int elements_per_lane(int D, bool vec) {
 
 }  // namespace
 
+int add_column_partials(hipStream_t stream, int parts, int D, const float* partial, float* first,
+                        float* second) {
+  layer_norm_reduce_kernel<<<dim3((unsigned)((2 * D + 63) / 64)), dim3(256), 0, stream>>>(
+      parts, D, partial, first, second);
+  HASTE_HIP_TRY(hipGetLastError());
+  return HASTE_HIP_OK;
+}
+
 int layer_norm_forward(hipStream_t stream, int rows, int dim, const float* gamma,
                        const float* beta, const float* x, float* y, float* cache) {
   HASTE_HIP_REQUIRE(rows > 0 && dim > 0 && gamma && x && y);
@@ -271,10 +279,7 @@ int layer_norm_backward(hipStream_t stream, int rows, int dim, const float* gamm
   HASTE_LN_BWD(16, false)
 #undef HASTE_LN_BWD
   HASTE_HIP_TRY(hipGetLastError());
-  layer_norm_reduce_kernel<<<dim3((unsigned)((2 * dim + 63) / 64)), dim3(256), 0, stream>>>(
-      grid, dim, ws.scratch, dgamma, dbeta);
-  HASTE_HIP_TRY(hipGetLastError());
-  return HASTE_HIP_OK;
+  return add_column_partials(stream, grid, dim, ws.scratch, dgamma, dbeta);
 }
 
 }  // namespace haste_hip

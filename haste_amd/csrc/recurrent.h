@@ -233,30 +233,9 @@ __device__ __forceinline__ void group_wait(GroupSync& g) {
   __syncthreads();
 }
 
-// True in exactly one workgroup of the launch: the last to call it.  Stores made by
-// the other workgroups before their call are visible to that workgroup afterwards.
-// `flag` is a word of LDS.  Called by all threads.
-__device__ __forceinline__ bool grid_last_arrival(ControlBlock* cb, unsigned int total_workgroups,
-                                                  unsigned int* flag) {
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-    const unsigned int old = __hip_atomic_fetch_add(&cb->grid_exit_counter[0], 1u, __ATOMIC_RELAXED,
-                                                    __HIP_MEMORY_SCOPE_AGENT);
-    const bool last = old == total_workgroups - 1;
-    if (last) {
-      __hip_atomic_store(&cb->grid_exit_counter[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-    }
-    *flag = last ? 1u : 0u;
-  }
-  __syncthreads();
-  return *flag != 0u;
-}
-
 // Publishing without cache-wide fences: agent-scope stores (store_agent) before an arrival,
-// agent-scope loads (load_exchanged) after it.  The release/acquire fences of
-// grid_last_arrival write back and invalidate whole caches instead.
+// agent-scope loads (load_exchanged) after it (release / acquire fences at agent scope would
+// write back and invalidate whole caches instead).
 __device__ __forceinline__ void store_agent(float* p, float v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
