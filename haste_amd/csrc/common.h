@@ -175,6 +175,13 @@ int layer_norm_gru_backward_streamed(hipStream_t stream, int T, int N, int C, in
                                      float* dgamma2, const float* cache2,
                                      const float* zoneout_mask);
 
+// The same for rows too wide for layer_norm.hip's row-in-registers kernels (stepwise.hip).
+int layer_norm_forward_wide(hipStream_t stream, int rows, int dim, const float* gamma,
+                            const float* beta, const float* x, float* y, float* cache);
+int layer_norm_backward_wide(hipStream_t stream, int rows, int dim, const float* gamma,
+                             const float* x, const float* dy, float* dx, float* dgamma,
+                             float* dbeta);
+
 // Row-wise layer norm kernels (rows x dim), used stand-alone and by the LN cells.
 int layer_norm_forward(hipStream_t stream, int rows, int dim, const float* gamma,
                        const float* beta, const float* x, float* y, float* cache);

@@ -233,7 +233,7 @@ int layer_norm_forward(hipStream_t stream, int rows, int dim, const float* gamma
   const bool vec = dim % 4 == 0 && aligned16(gamma) && aligned16(x) && aligned16(y) &&
                    (beta == nullptr || aligned16(beta));
   const int E = elements_per_lane(dim, vec);
-  if (E == 0) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  if (E == 0) return layer_norm_forward_wide(stream, rows, dim, gamma, beta, x, y, cache);
   const int cus = device_cu_count();
   int grid = (rows + 3) / 4;
   if (grid > 16 * cus) grid = 16 * cus;
@@ -257,7 +257,7 @@ int layer_norm_backward(hipStream_t stream, int rows, int dim, const float* gamm
   HASTE_HIP_REQUIRE(rows > 0 && dim > 0 && gamma && x && dy && dx && dgamma);
   const bool vec = dim % 4 == 0 && aligned16(gamma) && aligned16(x) && aligned16(dy) && aligned16(dx);
   const int E = elements_per_lane(dim, vec);
-  if (E == 0) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  if (E == 0) return layer_norm_backward_wide(stream, rows, dim, gamma, x, dy, dx, dgamma, dbeta);
   const int cus = device_cu_count();
   int grid = (rows + 3) / 4;
   if (grid > 2 * cus) grid = 2 * cus;

@@ -1094,6 +1094,24 @@ int gru_backward_streamed(hipStream_t stream, int T, int N, int C, int H, const 
   return gru_backward_steps<float>(stream, T, N, C, H, W_t, R_t, x_t, h, v, dh_next, dx, dW, dR, dbx,
                                    dbr, dh, dp, dq, zoneout_mask);
 }
+// Row-wise layer norm of any width (one workgroup per row): what layer_norm.hip hands rows
+// to that do not fit a wavefront's registers.
+int layer_norm_forward_wide(hipStream_t stream, int rows, int dim, const float* gamma,
+                            const float* beta, const float* x, float* y, float* cache) {
+  return ln_forward_rows<float>(stream, (size_t)rows, dim, gamma, beta, x, y, cache);
+}
+int layer_norm_backward_wide(hipStream_t stream, int rows, int dim, const float* gamma,
+                             const float* x, const float* dy, float* dx, float* dgamma,
+                             float* dbeta) {
+  const size_t part_bytes = column_sum_bytes<float>((size_t)rows, dim);
+  Scratch sc;
+  HASTE_HIP_PROPAGATE(open_scratch(stream, part_bytes + padded((size_t)rows * 2 * sizeof(float)), 0, &sc));
+  void* partial = sc.take<char>(part_bytes);
+  float* stats = sc.take<float>((size_t)rows * 2);
+  HASTE_HIP_PROPAGATE(ln_forward_rows<float>(stream, (size_t)rows, dim, gamma, nullptr, x, nullptr, stats));
+  return ln_backward_rows<float>(stream, (size_t)rows, dim, gamma, x, dy, dx, dgamma, dbeta, stats, partial);
+}
+
 int layer_norm_lstm_forward_streamed(hipStream_t stream, int training, int T, int N, int C, int H,
                                      const float* W, const float* R, const float* b, const float* x,
                                      float* h, float* c, float* act_Wx, const float* gamma1,

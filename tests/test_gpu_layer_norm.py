@@ -8,7 +8,9 @@ from util import TOL, dev, host, relerr
 pytestmark = pytest.mark.gpu
 
 SHAPES = [(1, 1), (3, 5), (7, 33), (64, 64), (100, 256), (37, 1000), (3200, 1024), (500, 2048),
-          (33, 4096), (9, 1023)]
+          (33, 4096), (9, 1023),
+          # wider than a wavefront keeps in registers: the row-per-workgroup kernels
+          (5, 5000), (3, 4101), (40, 8192)]
 
 
 @pytest.mark.parametrize("with_beta", [False, True])

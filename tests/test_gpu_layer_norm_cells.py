@@ -15,7 +15,9 @@ SHAPES = [(1, 1, 3, 4), (3, 2, 3, 4), (5, 3, 7, 5), (6, 17, 20, 36), (4, 16, 32,
           (3, 200, 16, 64), (2, 300, 8, 48), (2, 520, 8, 32),
           # hidden sizes beyond what stays on chip: the backward pass, then both passes, run
           # step by step (GEMM + row-wise norms + pointwise kernels)
-          (3, 5, 24, 640), (2, 6, 16, 1536), (2, 130, 8, 1100)]
+          (3, 5, 24, 640), (2, 6, 16, 1536), (2, 130, 8, 1100),
+          # resident forward whose norm of x*W is wider than 4096 columns
+          (2, 3, 8, 1028)]
 
 
 @pytest.mark.parametrize("zoneout", [0.0, 0.3])
