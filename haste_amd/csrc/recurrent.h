@@ -13,6 +13,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <map>
+#include <mutex>
 #include <utility>
 
 #include "common.h"
@@ -893,26 +895,29 @@ constexpr size_t kMaxLdsBytes = kWorkgroupLdsBytes - 256;
 template <typename KernelT, typename ParamsT>
 int launch_persistent(const char* name, KernelT kernel, const LaunchPlan& plan, ParamsT& params,
                       hipStream_t stream) {
-  // The attribute and the occupancy of (kernel, LDS request) are looked up once per thread
-  // and device: single-step callers (Iterate) launch the same kernel over and over.
-  struct Known { const void* kernel; size_t lds; int device; int per_cu; };
-  thread_local Known known[8] = {};
-  thread_local int next_slot = 0;
+  // The kernel's LDS limit and its occupancy at this request are looked up once per process
+  // and device: single-step callers (Iterate) launch the same kernel over and over.  The
+  // limit is a property of the kernel, not of the launch, and is only ever raised.
+  struct Known { size_t limit = 0; std::map<size_t, int> per_cu; };
+  static std::mutex known_mutex;
+  static std::map<std::pair<const void*, int>, Known> known;
   int device = 0;
   HASTE_HIP_TRY(hipGetDevice(&device));
   const void* fn = reinterpret_cast<const void*>(kernel);
-  int per_cu = -1;
-  for (const Known& k : known)
-    if (k.kernel == fn && k.lds == plan.lds_bytes && k.device == device) per_cu = k.per_cu;
-  if (per_cu < 0) {
-    // The limit is a property of the kernel, not of the launch: it is only ever raised (a
-    // later launch with a smaller, already known request must not find it lowered).
+  std::lock_guard<std::mutex> lock(known_mutex);
+  Known& k = known[std::make_pair(fn, device)];
+  if (k.limit < plan.lds_bytes) {
     const size_t limit = plan.lds_bytes > kMaxLdsBytes ? plan.lds_bytes : kMaxLdsBytes;
     HASTE_HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)limit));
-    HASTE_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, plan.lds_bytes));
-    known[next_slot] = Known{fn, plan.lds_bytes, device, per_cu};
-    next_slot = (next_slot + 1) % 8;
+    k.limit = limit;
   }
+  auto found = k.per_cu.find(plan.lds_bytes);
+  if (found == k.per_cu.end()) {
+    int blocks = 0;
+    HASTE_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, kernel, 256, plan.lds_bytes));
+    found = k.per_cu.emplace(plan.lds_bytes, blocks).first;
+  }
+  const int per_cu = found->second;
   const long long capacity = (long long)per_cu * device_cu_count();
   if ((long long)plan.grid.x * plan.grid.y > capacity) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   HASTE_HIP_PROPAGATE(order_persistent_launches(stream, true));
