@@ -96,6 +96,12 @@ int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
              const float* A, int lda, const float* B, int ldb,
              float* C, int ldc, bool accumulate, size_t scratch_offset = 0);
 
+// Two products with the same N and K, the second with A stored transposed, in one launch when
+// that halves their K pieces (gemm.hip): dW and dR of a backward pass.
+int gemm_f32_pair(hipStream_t stream, int M1, int M2, int N, int K, const float* A1, int lda1,
+                  const float* B1, int ldb1, float* C1, int ldc1, const float* A2, int lda2,
+                  const float* B2, int ldb2, float* C2, int ldc2, bool accumulate);
+
 // The product left as the K pieces of the tile kernel for a consumer that adds them itself;
 // *splits == 0 (and nothing launched) when the shape is not cut that way.  See gemm.hip.
 int gemm_f32_pieces(hipStream_t stream, int M, int N, int K, const float* A, int lda,
@@ -200,7 +206,8 @@ int add_column_partials(hipStream_t stream, int parts, int D, const float* parti
 // nothing.  `name` must be a string literal.
 class ScopedKernelTimer {
  public:
-  ScopedKernelTimer(const char* name, hipStream_t stream);
+  // `products`: how many launches of `name` the bracket counts as (a fused pair counts 2).
+  ScopedKernelTimer(const char* name, hipStream_t stream, int products = 1);
   ~ScopedKernelTimer();
  private:
   hipStream_t stream_;

@@ -59,47 +59,25 @@ __device__ __forceinline__ float4_t masked4(uint4_t u, int valid) {
   return v;
 }
 
-// BM x 128 output tile; BM = 128 (each wavefront a 64x64 quadrant) or 64 (each a 32x64
-// quadrant) for outputs too small to fill the chip with 128-row tiles.
+// One BM x 128 output tile over the K range [k_begin, k_end): BM = 128 (each wavefront a
+// 64x64 quadrant) or 64 (each a 32x64 quadrant) for outputs too small to fill the chip with
+// 128-row tiles.  part == null: the tile goes to C (+= when accumulate); otherwise the whole
+// [BM][BN] partial tile is parked at `part`.  `smem`: 2 * (BK * (BM + 4) + B_STAGE) floats.
 template <bool TRANS_A, int BM>
-__global__ __launch_bounds__(256, 2)
-void gemm_f32_kernel(int M, int N, int K,
-                     const float* __restrict__ A, int lda,
-                     const float* __restrict__ B, int ldb,
-                     float* __restrict__ C, int ldc, int accumulate,
-                     int tiles_n, int whole_tiles, int splits, int k_per_split,
-                     float* __restrict__ partial) {
+__device__ __forceinline__ void gemm_tile(int M, int N, int K,
+                                          const float* __restrict__ A, int lda,
+                                          const float* __restrict__ B, int ldb,
+                                          float* __restrict__ C, int ldc, int accumulate,
+                                          int tm, int tn, int k_begin, int k_end,
+                                          float* __restrict__ part, float* smem) {
   // A tile k-major in LDS: leading dimension BM+2 when it is written with transposing
   // scalar stores (bank-conflict free), BM+4 when written with 16-byte stores.
   constexpr int LDA = TRANS_A ? BM + 4 : BM + 2;
   constexpr int A_STAGE = BK * (BM + 4);
   constexpr int MI = BM / 64;       // 32x32 MFMA tiles per wavefront along M
   constexpr int A_PASSES = BM / 64; // passes of 256 threads to load the A tile
-  __shared__ __attribute__((aligned(16))) float smem[2 * A_STAGE + 2 * B_STAGE];
   float* As = smem;
   float* Bs = smem + 2 * A_STAGE;
-
-  // Workgroups [0, whole_tiles) compute one whole tile each.  Ids are handed to the XCDs
-  // round-robin; XCD x gets the x-th contiguous chunk of the tile list so that neighbours
-  // in the list share an L2.  Workgroups from whole_tiles on compute one K piece of one of
-  // the remaining tiles: piece j = id - whole_tiles is split j % splits of tile
-  // whole_tiles + j / splits, and parks its result at partial + j * BM * BN.
-  const int id = blockIdx.x;
-  int tile, k_begin, k_end;
-  const bool piece = id >= whole_tiles;
-  if (!piece) {
-    const int q = whole_tiles / kXcds, r = whole_tiles % kXcds;
-    const int xcd = id % kXcds, local = id / kXcds;
-    tile = xcd * q + (xcd < r ? xcd : r) + local;
-    k_begin = 0;
-    k_end = K;
-  } else {
-    const int j = id - whole_tiles;
-    tile = whole_tiles + j / splits;
-    k_begin = (j % splits) * k_per_split;
-    k_end = (k_begin + k_per_split < K) ? (k_begin + k_per_split) : K;
-  }
-  const int tm = tile / tiles_n, tn = tile % tiles_n;
   const int m0 = tm * BM, n0 = tn * BN;
 
   const int tid = threadIdx.x;
@@ -235,7 +213,7 @@ void gemm_f32_kernel(int M, int N, int K,
   // col = lane % 32, row = 8*(e/4) + 4*(lane/32) + e%4.
   const int col_in = lane & 31;
   const int row_in = (lane >> 5) * 4;
-  if (!piece) {
+  if (part == nullptr) {
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
@@ -256,7 +234,6 @@ void gemm_f32_kernel(int M, int N, int K,
   // A K piece: park the whole [BM][BN] partial tile (rows and columns beyond the problem
   // hold zeros); a second, bandwidth-bound kernel adds a tile's pieces in order (the kernel
   // boundary makes them visible, so no cache-wide fence is needed here).
-  float* part = partial + (size_t)(id - whole_tiles) * BM * BN;
 #pragma unroll
   for (int i = 0; i < MI; ++i)
 #pragma unroll
@@ -270,6 +247,71 @@ void gemm_f32_kernel(int M, int N, int K,
     }
 }
 
+template <bool TRANS_A, int BM>
+__global__ __launch_bounds__(256, 2)
+void gemm_f32_kernel(int M, int N, int K,
+                     const float* __restrict__ A, int lda,
+                     const float* __restrict__ B, int ldb,
+                     float* __restrict__ C, int ldc, int accumulate,
+                     int tiles_n, int whole_tiles, int splits, int k_per_split,
+                     float* __restrict__ partial) {
+  __shared__ __attribute__((aligned(16))) float smem[2 * BK * (BM + 4) + 2 * B_STAGE];
+  // Workgroups [0, whole_tiles) compute one whole tile each.  Ids are handed to the XCDs
+  // round-robin; XCD x gets the x-th contiguous chunk of the tile list so that neighbours
+  // in the list share an L2.  Workgroups from whole_tiles on compute one K piece of one of
+  // the remaining tiles: piece j = id - whole_tiles is split j % splits of tile
+  // whole_tiles + j / splits, and parks its result at partial + j * BM * BN.
+  const int id = blockIdx.x;
+  int tile, k_begin, k_end;
+  float* part = nullptr;
+  if (id < whole_tiles) {
+    const int q = whole_tiles / kXcds, r = whole_tiles % kXcds;
+    const int xcd = id % kXcds, local = id / kXcds;
+    tile = xcd * q + (xcd < r ? xcd : r) + local;
+    k_begin = 0;
+    k_end = K;
+  } else {
+    const int j = id - whole_tiles;
+    tile = whole_tiles + j / splits;
+    k_begin = (j % splits) * k_per_split;
+    k_end = (k_begin + k_per_split < K) ? (k_begin + k_per_split) : K;
+    part = partial + (size_t)j * BM * BN;
+  }
+  gemm_tile<TRANS_A, BM>(M, N, K, A, lda, B, ldb, C, ldc, accumulate, tile / tiles_n, tile % tiles_n,
+                         k_begin, k_end, part, smem);
+}
+
+// Two products with the same N and K in one launch (dW = x^T dv and dR = h^T dv of a backward
+// pass): A1 row-major [M1,K], A2 stored transposed [K,M2].  Their tiles form one list, every
+// tile cut into `splits` K pieces (splits == 1: whole tiles); piece j of the list parks its
+// result at partial + j * BM * BN.  One launch of twice the tiles needs half the pieces per
+// tile to fill the chip, i.e. half the partial-tile traffic.
+struct GemmPair {
+  int M1, M2, N, K;
+  const float* A1; int lda1; const float* B1; int ldb1; float* C1; int ldc1;
+  const float* A2; int lda2; const float* B2; int ldb2; float* C2; int ldc2;
+  int accumulate, tiles_n, tiles_m1, splits, k_per_split;
+  float* partial;
+};
+
+template <int BM>
+__global__ __launch_bounds__(256, 2)
+void gemm_f32_pair_kernel(GemmPair p) {
+  __shared__ __attribute__((aligned(16))) float smem[2 * BK * (BM + 4) + 2 * B_STAGE];
+  const int j = blockIdx.x;
+  const int tile = j / p.splits;
+  const int k_begin = (j % p.splits) * p.k_per_split;
+  const int k_end = (k_begin + p.k_per_split < p.K) ? (k_begin + p.k_per_split) : p.K;
+  float* part = p.splits > 1 ? p.partial + (size_t)j * BM * BN : nullptr;
+  const int tm = tile / p.tiles_n, tn = tile % p.tiles_n;
+  if (tm < p.tiles_m1)
+    gemm_tile<false, BM>(p.M1, p.N, p.K, p.A1, p.lda1, p.B1, p.ldb1, p.C1, p.ldc1, p.accumulate, tm, tn,
+                         k_begin, k_end, part, smem);
+  else
+    gemm_tile<true, BM>(p.M2, p.N, p.K, p.A2, p.lda2, p.B2, p.ldb2, p.C2, p.ldc2, p.accumulate,
+                        tm - p.tiles_m1, tn, k_begin, k_end, part, smem);
+}
+
 // For the split tiles (tile index whole_tiles + blockIdx.x): C tile (+)= sum over its
 // `splits` pieces of partial[(blockIdx.x * splits + piece)][BM][BN], pieces added in index
 // order.  blockIdx.y selects 8 of the tile's rows; a thread owns 4 consecutive columns.
@@ -280,6 +322,39 @@ void split_reduce_kernel(int M, int N, int splits, int tiles_n, int whole_tiles,
                          int accumulate, int vec_ok) {
   const int tile = whole_tiles + blockIdx.x;
   const int tm = tile / tiles_n, tn = tile % tiles_n;
+  const int r = blockIdx.y * 8 + (threadIdx.x >> 5);
+  const int c = (threadIdx.x & 31) * 4;
+  const int row = tm * BM + r, col = tn * BN + c;
+  if (r >= BM || row >= M || col >= N) return;
+  const float* p = partial + ((size_t)blockIdx.x * splits) * BM * BN + r * BN + c;
+  float4_t s = *reinterpret_cast<const float4_t*>(p);
+  for (int sp = 1; sp < splits; ++sp)
+    s += *reinterpret_cast<const float4_t*>(p + (size_t)sp * BM * BN);
+  float* out = C + (size_t)row * ldc + col;
+  if (vec_ok && col + 3 < N) {
+    float4_t* o = reinterpret_cast<float4_t*>(out);
+    *o = accumulate ? (*o + s) : s;
+  } else {
+    const float v[4] = {s.x, s.y, s.z, s.w};
+    for (int i = 0; i < 4 && col + i < N; ++i) out[i] = accumulate ? (out[i] + v[i]) : v[i];
+  }
+}
+
+// The same for the tile list of gemm_f32_pair_kernel: tile rows below tiles_m1 belong to the
+// first product.
+template <int BM>
+__global__ __launch_bounds__(256)
+void split_reduce_pair_kernel(int M1, int M2, int N, int splits, int tiles_n, int tiles_m1,
+                              const float* __restrict__ partial, float* __restrict__ C1, int ldc1,
+                              float* __restrict__ C2, int ldc2, int accumulate, int vec_ok) {
+  const int tile = blockIdx.x;
+  int tm = tile / tiles_n;
+  const int tn = tile % tiles_n;
+  const bool second = tm >= tiles_m1;
+  if (second) tm -= tiles_m1;
+  const int M = second ? M2 : M1;
+  float* C = second ? C2 : C1;
+  const int ldc = second ? ldc2 : ldc1;
   const int r = blockIdx.y * 8 + (threadIdx.x >> 5);
   const int c = (threadIdx.x & 31) * 4;
   const int row = tm * BM + r, col = tn * BN + c;
@@ -410,6 +485,67 @@ int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
     else
       split_reduce_kernel<64><<<rgrid, dim3(256), 0, stream>>>(
           M, N, splits, tiles_n, whole_tiles, partial, C, ldc, accumulate ? 1 : 0, vec);
+    HASTE_HIP_TRY(hipGetLastError());
+  }
+  return HASTE_HIP_OK;
+}
+
+// C1[M1,N] (+)= A1[M1,K] * B1 and C2[M2,N] (+)= A2^T * B2 (A2 stored [K,M2]) in one launch when
+// together they have fewer tiles than the chip has CUs (then each alone would be cut into
+// twice the pieces); otherwise two ordinary products.  `products` of the timer: 2.
+int gemm_f32_pair(hipStream_t stream, int M1, int M2, int N, int K, const float* A1, int lda1,
+                  const float* B1, int ldb1, float* C1, int ldc1, const float* A2, int lda2,
+                  const float* B2, int ldb2, float* C2, int ldc2, bool accumulate) {
+  HASTE_HIP_REQUIRE(M1 > 0 && M2 > 0 && N > 0 && K > 0 && A1 && B1 && C1 && A2 && B2 && C2);
+  HASTE_HIP_REQUIRE(lda1 >= K && lda2 >= M2 && ldb1 >= N && ldb2 >= N && ldc1 >= N && ldc2 >= N);
+  const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
+  const int tiles_n = (N + BN - 1) / BN;
+  const int tiles_m1 = (M1 + 127) / 128, tiles_m2 = (M2 + 127) / 128;
+  const long long tiles = (long long)(tiles_m1 + tiles_m2) * tiles_n;
+  const bool panels_ok = ((long long)128 * lda1 + K) * 4 < (1ll << 31) && ((long long)K * lda2 + 128) * 4 < (1ll << 31) &&
+                         ((long long)K * ldb1 + BN) * 4 < (1ll << 31) && ((long long)K * ldb2 + BN) * 4 < (1ll << 31);
+  if (tiles >= cus || M1 <= 64 || M2 <= 64 || !panels_ok) {
+    HASTE_HIP_PROPAGATE(gemm_f32(stream, false, M1, N, K, A1, lda1, B1, ldb1, C1, ldc1, accumulate));
+    return gemm_f32(stream, true, M2, N, K, A2, lda2, B2, ldb2, C2, ldc2, accumulate);
+  }
+  // The cost model of plan_gemm for a list in which every tile is cut.
+  const int k_iters = (K + BK - 1) / BK;
+  int s_max = k_iters / 4;
+  if (s_max > 64) s_max = 64;
+  auto cost = [&](int s) {
+    const long long pieces = tiles * s;
+    double c = (double)((pieces + cus - 1) / cus) / s;
+    if (pieces < 2LL * cus) c *= 1.2;
+    if (s > 1) c += 0.25 * (double)tiles * s / K;
+    return c;
+  };
+  int splits = 1;
+  double best = cost(1);
+  for (int s = 2; s <= s_max; ++s)
+    if (cost(s) < best - 1e-9) { best = cost(s); splits = s; }
+  int k_per_split = (K + splits - 1) / splits;
+  k_per_split = (k_per_split + BK - 1) / BK * BK;
+  splits = (K + k_per_split - 1) / k_per_split;
+
+  GemmPair p;
+  p.M1 = M1; p.M2 = M2; p.N = N; p.K = K;
+  p.A1 = A1; p.lda1 = lda1; p.B1 = B1; p.ldb1 = ldb1; p.C1 = C1; p.ldc1 = ldc1;
+  p.A2 = A2; p.lda2 = lda2; p.B2 = B2; p.ldb2 = ldb2; p.C2 = C2; p.ldc2 = ldc2;
+  p.accumulate = accumulate ? 1 : 0;
+  p.tiles_n = tiles_n; p.tiles_m1 = tiles_m1; p.splits = splits; p.k_per_split = k_per_split;
+  p.partial = nullptr;
+  if (splits > 1) {
+    Workspace ws;
+    HASTE_HIP_PROPAGATE(get_workspace(stream, (size_t)tiles * splits * 128 * BN * sizeof(float), &ws));
+    p.partial = ws.scratch;
+  }
+  ScopedKernelTimer timer("gemm_f32", stream, 2);
+  gemm_f32_pair_kernel<128><<<dim3((unsigned)(tiles * splits)), dim3(256), 0, stream>>>(p);
+  HASTE_HIP_TRY(hipGetLastError());
+  if (splits > 1) {
+    const int vec = (ldc1 % 4 == 0) && (ldc2 % 4 == 0) && aligned16(C1) && aligned16(C2);
+    split_reduce_pair_kernel<128><<<dim3((unsigned)tiles, 16), dim3(256), 0, stream>>>(
+        M1, M2, N, splits, tiles_n, tiles_m1, p.partial, C1, ldc1, C2, ldc2, p.accumulate, vec);
     HASTE_HIP_TRY(hipGetLastError());
   }
   return HASTE_HIP_OK;

@@ -633,8 +633,9 @@ int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_s
   const int TN = T * N;
   HASTE_HIP_PROPAGATE(layer_norm_backward(stream, TN, 3 * H, gamma1, act_Wx, dp, dp, dgamma1, nullptr));
   HASTE_HIP_PROPAGATE(gemm_f32(stream, false, TN, C, 3 * H, dp, 3 * H, W_t, C, dx, C, false));
-  HASTE_HIP_PROPAGATE(gemm_f32(stream, true, H, 3 * H, TN, h, H, dq, 3 * H, dR, 3 * H, true));
-  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, C, 3 * H, TN, x_t, TN, dp, 3 * H, dW, 3 * H, true));
+  // dW += x^T dp and dR += h^T dq: one launch when that halves their K pieces
+  HASTE_HIP_PROPAGATE(gemm_f32_pair(stream, C, H, 3 * H, TN, x_t, TN, dp, 3 * H, dW, 3 * H,
+                                    h, H, dq, 3 * H, dR, 3 * H, true));
   return HASTE_HIP_OK;
 }
 

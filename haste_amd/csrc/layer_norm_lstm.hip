@@ -746,8 +746,8 @@ int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_
   const int TN = T * N;
   HASTE_HIP_PROPAGATE(layer_norm_backward(stream, TN, 4 * H, gamma1, act_Wx, act_Wx_norm, act_Wx,
                                           dgamma1, nullptr));
-  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, C, 4 * H, TN, x_t, TN, act_Wx, 4 * H, dW, 4 * H, true));
-  HASTE_HIP_PROPAGATE(gemm_f32(stream, true, H, 4 * H, TN, h, H, act_Rh, 4 * H, dR, 4 * H, true));
+  HASTE_HIP_PROPAGATE(gemm_f32_pair(stream, C, H, 4 * H, TN, x_t, TN, act_Wx, 4 * H, dW, 4 * H,
+                                    h, H, act_Rh, 4 * H, dR, 4 * H, true));
   HASTE_HIP_PROPAGATE(gemm_f32(stream, false, TN, C, 4 * H, act_Wx, 4 * H, W_t, C, dx, C, false));
   return HASTE_HIP_OK;
 }

@@ -505,8 +505,9 @@ int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
 
   // dW += x^T dv ; dR += h[0:T]^T dv ; dx = dv W^T  (dv now lives in v).
   const int TN = T * N;
-  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, C, 4 * H, TN, x_t, TN, v, 4 * H, dW, 4 * H, true));
-  HASTE_HIP_PROPAGATE(gemm_f32(stream, true, H, 4 * H, TN, h, H, v, 4 * H, dR, 4 * H, true));
+  // dW += x^T dv and dR += h^T dv: one launch when that halves their K pieces
+  HASTE_HIP_PROPAGATE(gemm_f32_pair(stream, C, H, 4 * H, TN, x_t, TN, v, 4 * H, dW, 4 * H,
+                                    h, H, v, 4 * H, dR, 4 * H, true));
   HASTE_HIP_PROPAGATE(gemm_f32(stream, false, TN, C, 4 * H, v, 4 * H, W_t, C, dx, C, false));
   return HASTE_HIP_OK;
 }

@@ -38,17 +38,19 @@ __global__ void fill_zero_kernel(unsigned int* p, size_t n) {
 struct TimedLaunch {
   const char* name;
   hipEvent_t start, stop;
+  int products;
 };
 bool g_profile_on = false;
 std::vector<TimedLaunch> g_timed;
 
 }  // namespace
 
-ScopedKernelTimer::ScopedKernelTimer(const char* name, hipStream_t stream)
+ScopedKernelTimer::ScopedKernelTimer(const char* name, hipStream_t stream, int products)
     : stream_(stream), slot_(-1) {
   if (!g_profile_on) return;
   TimedLaunch t;
   t.name = name;
+  t.products = products;
   if (hipEventCreate(&t.start) != hipSuccess) return;
   if (hipEventCreate(&t.stop) != hipSuccess) { (void)hipEventDestroy(t.start); return; }
   (void)hipEventRecord(t.start, stream);
@@ -272,7 +274,7 @@ int haste_hip_profile_read(const char* name, double* total_ms, int* launches) {
     float ms = 0.f;
     if (hipEventElapsedTime(&ms, t.start, t.stop) != hipSuccess) return HASTE_HIP_ERROR_RUNTIME;
     total += ms;
-    ++count;
+    count += t.products;
   }
   *total_ms = total;
   *launches = count;

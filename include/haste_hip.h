@@ -56,7 +56,8 @@ int haste_hip_stream_order(void* first, void* then);
  * launches is bracketed by a pair of HIP events recorded on the stream the kernel
  * runs on.  haste_hip_profile_read waits for those events and returns, for the kernel
  * called `name` ("gemm_f32", "lstm_forward_recurrence", "lstm_backward_recurrence", ...),
- * the summed duration in milliseconds and the number of launches since the last reset.
+ * the summed duration in milliseconds and the number of launches since the last reset (a
+ * launch that fuses two products, dW and dR of the LSTM backward pass, counts as two).
  * The reference has only cudaEvent timers in its benchmarks
  * (benchmarks/benchmark_lstm.cc:49-63); this is their in-library counterpart. */
 int haste_hip_profile_enable(int on);
