@@ -90,6 +90,10 @@ int order_persistent_launches(hipStream_t stream, bool before);
 // cross-XCD exchange path; for experiments).
 bool xcd_local_enabled();
 
+// False when the environment variable HASTE_HIP_PAIRED_SETS is set to 0: 8- and 16-row
+// batch tiles then run as one tile instead of two sets of half the rows (for experiments).
+bool paired_sets_enabled();
+
 // C[M,N] = op(A)*B (+C): fp32 MFMA GEMM on `stream`.  The partial tiles of a split product
 // are kept `scratch_offset` bytes (a multiple of 16) into the stream's scratch buffer.
 int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,

@@ -73,6 +73,21 @@ __device__ __forceinline__ float4_t load_exchanged4(const float* p) {
   return v;
 }
 
+// A workgroup of 512 threads (SETS == 2) holds two sets of 256 threads (four wavefronts) that
+// work on batch tiles of their own.  The sets take the workgroup's wavefronts alternately:
+// wavefronts land on the CU's four SIMDs round-robin, so each set gets two SIMDs of its own
+// and the products of one set never delay the pointwise work of the other (measured: sets
+// of four consecutive wavefronts, which share all four SIMDs, are 12 % slower per step).
+// set_thread: thread index inside the set (0..255); set_wave: wavefront inside the set.
+template <int SETS>
+__device__ __forceinline__ int set_index() { return SETS == 1 ? 0 : (int)((threadIdx.x >> 6) & 1); }
+template <int SETS>
+__device__ __forceinline__ int set_wave() { return (int)(threadIdx.x >> (SETS == 1 ? 6 : 7)); }
+template <int SETS>
+__device__ __forceinline__ int set_thread() {
+  return SETS == 1 ? (int)threadIdx.x : (int)(((threadIdx.x >> 7) << 6) | (threadIdx.x & 63));
+}
+
 // What the host tells a persistent kernel about its launch.
 struct LaunchShape {
   ControlBlock* cb;
@@ -300,8 +315,9 @@ __device__ __forceinline__ void fill_slice(float* w_lds, int Kpad, const float* 
                                            const float* __restrict__ mask, float scale, bool fast,
                                            OffsetFn offset) {
   const int tid = threadIdx.x;
+  const int nthreads = blockDim.x;
   if (!fast) {
-    for (int idx = tid; idx < Kpad * NCOLS; idx += 256) {
+    for (int idx = tid; idx < Kpad * NCOLS; idx += nthreads) {
       const int k = idx / NCOLS, col = idx % NCOLS;
       const long long off = offset(k, col);
       float w = 0.f;
@@ -317,11 +333,11 @@ __device__ __forceinline__ void fill_slice(float* w_lds, int Kpad, const float* 
   constexpr int UNROLL = 4;
   const int items = (Kpad / 4) * QUADS;
   const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
-  for (int base = tid; base < items; base += 256 * UNROLL) {
+  for (int base = tid; base < items; base += nthreads * UNROLL) {
     float4_t v[UNROLL][4];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int item = base + 256 * u;
+      const int item = base + nthreads * u;
       const int k4 = item / QUADS, col = (item % QUADS) * 4;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -336,7 +352,7 @@ __device__ __forceinline__ void fill_slice(float* w_lds, int Kpad, const float* 
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int item = base + 256 * u;
+      const int item = base + nthreads * u;
       if (item < items) {
         const int k4 = item / QUADS, col = (item % QUADS) * 4;
         float* dst = w_lds + ((size_t)k4 * NCOLS + col) * 4;
@@ -709,17 +725,22 @@ __device__ __forceinline__ void mfma_tile_rows4(const float* w_lds, int s,
 // partial tile of lane group g (accumulator element r of acc[rb][ct] in lane l is row
 // 4*rb + r, column ct*MC + l%MC, partial g = l/MC).  The operand
 // loads of chunk c+1 (CH super-groups) are issued before the MFMAs of chunk c; the two
-// register buffers alternate so that nothing is copied.
-template <int RB, int CT, int CH, bool POLLED>
+// register buffers alternate so that nothing is copied.  The four wavefronts are those of one
+// 256-thread set of the workgroup.  TAGGED: the partial tiles are themselves polled by their
+// readers (take_product), so no element may carry the "unwritten" pattern.
+template <int RB, int CT, int CH, bool POLLED, bool TAGGED = false>
 __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int tile_off, int Kpad,
                                                        const float* w_lds, float* red,
                                                        const GroupSync* gs) {
   using S = ShortTileShape<CT>;
   constexpr int NB = 4 * RB;
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = set_wave<TAGGED ? 2 : 1>();  // polled partial tiles: two sets
   const int s_end = Kpad >> 6;
   const int mine = (s_end - wave + 3) >> 2;  // super-groups wave, wave+4, ...
+  // A wavefront without a share of k waits for nobody, so nothing would keep it from running
+  // steps ahead of the readers of its partial tile: it leaves no partial tile at all.
+  if (TAGGED && mine == 0) return;
   const int chunks = mine / CH;
   float4_t acc0[RB][S::CTN], acc1[RB][S::CTN];
 #pragma unroll
@@ -763,7 +784,8 @@ __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int
   for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
     for (int ct = 0; ct < S::CTN; ++ct) {
-      const float4_t v = acc0[rb][ct] + acc1[rb][ct];
+      float4_t v = acc0[rb][ct] + acc1[rb][ct];
+      if constexpr (TAGGED) v = float4_t{publishable(v.x), publishable(v.y), publishable(v.z), publishable(v.w)};
       float* q = base + (4 * rb) * S::NCOLS + ct * S::MC;
       q[0] = v.x;
       q[S::NCOLS] = v.y;
@@ -777,13 +799,14 @@ __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int
 // longer than the hidden size (the backward passes).
 // POLLED: the tile is a polled exchange tile (see above) and `gs` supplies the bounds of the
 // wait; otherwise the caller has waited at the group's step barrier and `gs` is unused.
-template <int NB, int CT, bool LONG_K, bool POLLED = false>
+template <int NB, int CT, bool LONG_K, bool POLLED = false, bool TAGGED = false>
 __device__ __forceinline__ void tile_product(const TileBuffer& xb, int tile_off, int Kpad,
                                              const float* w_lds, float* red,
                                              const GroupSync* gs = nullptr) {
   if constexpr (ProductTile<NB, CT>::kShort) {
-    short_exchange_product<NB / 4, CT, LONG_K ? 4 : 2, POLLED>(xb, tile_off, Kpad, w_lds, red, gs);
+    short_exchange_product<NB / 4, CT, LONG_K ? 4 : 2, POLLED, TAGGED>(xb, tile_off, Kpad, w_lds, red, gs);
   } else {
+    static_assert(!TAGGED, "polled partial tiles exist for short tiles only");
     constexpr int RT = NB / 16;
     constexpr int CHUNK = LONG_K ? (RT == 1 ? 8 : (RT == 2 ? 4 : 2)) : (RT >= 4 ? 2 : 4);
     tall_tile_product<RT, CT, CHUNK, POLLED>(xb, tile_off, Kpad, w_lds, red, gs);
@@ -792,10 +815,12 @@ __device__ __forceinline__ void tile_product(const TileBuffer& xb, int tile_off,
 
 // Zeroes this workgroup's share of its group's exchange tiles: float4 rows
 // [first4, first4 + count4) of [Kpad/4][NB][4], in each of the n_tiles tiles.  The stores have completed
-// when it returns.  Called by all threads.
+// when it returns.  Called by all threads of the workgroup.
+template <int SETS = 1>
 __device__ __forceinline__ void zero_tile_share(const GroupSync& g, float* tiles, int tile_floats,
                                                 int nb, int first4, int count4, int n_tiles = 2) {
-  for (int i = threadIdx.x; i < count4 * nb; i += 256) {
+  // the threads of one set share the work (two sets: each has tiles of its own)
+  for (int i = set_thread<SETS>(); i < count4 * nb; i += 256) {
     float* q = tiles + ((size_t)first4 * nb + i) * 4;
     for (int b = 0; b < n_tiles; ++b) store_exchanged4(g, q + (size_t)b * tile_floats, 0.f, 0.f, 0.f, 0.f);
   }
@@ -820,6 +845,88 @@ __device__ __forceinline__ float sum_product(const float* red, int row, int col)
   return v[0];
 }
 
+// ---- polled partial tiles -------------------------------------------------------------
+// A workgroup may hold two independent batch tiles: two 256-thread sets that share the
+// resident slice and are at different points of their steps, so that one set's product
+// runs while the other waits for its exchange.  Such a set cannot use the workgroup barrier
+// between its product and the threads that consume it.  Its partial tiles are polled
+// instead, like the exchange tiles: every element starts out unwritten, the product stores
+// publishable values (TAGGED), and the one thread that consumes an element re-reads it
+// until it is written and resets it afterwards.  Two such areas alternate by step: a
+// wavefront can only get to the product of step s+2 once every workgroup has finished step
+// s+1, for which the consumers of this set had to publish the results of step s -- after
+// their resets (LDS operations of a wavefront complete in order, and the reset is waited
+// for here).
+//
+// Partial tiles that a TAGGED product of contraction length Kpad writes: those of the
+// wavefronts that have a share of k.
+template <int CT>
+__device__ __forceinline__ int live_partials(int Kpad) {
+  const int waves = (Kpad >> 6) < 4 ? (Kpad >> 6) : 4;
+  return waves * ShortTileShape<CT>::KS;
+}
+
+// out[g] = element (row, col0 + g * col_stride) of the product, partials added in
+// sum_product's order.  Called by whole wavefronts; lanes with !mine take no part.  Only the
+// first `live` partial tiles are ever written (live_partials()): the others hold zeros.
+template <int NB, int CT, int G>
+__device__ __forceinline__ void take_product(const GroupSync& gs, float* red, int row, int col0,
+                                             int col_stride, bool mine, int live, float (&out)[G]) {
+  using P = ProductTile<NB, CT>;
+  constexpr int STRIDE = NB * P::NCOLS;
+  float* p = red + row * P::NCOLS + col0;
+  // Every lane reads (lanes that take no part: some valid address) and the reads carry no
+  // conditions, so that all of them are in flight at once.
+  const float* q = mine ? p : red;
+  float v[G][P::kPartials];
+  auto load = [&] {
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int i = 0; i < P::kPartials; ++i) v[g][i] = q[g * col_stride + i * STRIDE];
+  };
+  auto written = [&] {
+    unsigned int m = 0u;
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int i = 0; i < P::kPartials; ++i) {
+        const unsigned int x = __float_as_uint(v[g][i]);
+        m = m > x ? m : x;
+      }
+    return __all(!mine || m != kUnwrittenBits) != 0;
+  };
+  load();
+  poll_until_written(gs, [&] { __builtin_amdgcn_s_sleep(1); load(); }, written);
+  if (mine) {
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int i = 0; i < P::kPartials; ++i)
+        p[g * col_stride + i * STRIDE] = i < live ? unwritten_value() : 0.f;
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+#pragma unroll
+    for (int w = P::kPartials / 2; w > 0; w >>= 1)
+#pragma unroll
+      for (int i = 0; i < w; ++i) v[g][i] = v[g][2 * i] + v[g][2 * i + 1];
+    out[g] = v[g][0];
+  }
+}
+
+// Sets up the two polled areas of partial tiles of one set: the tiles that products write
+// start out unwritten, the others hold zeros for good.  A workgroup barrier must follow
+// before the first product.
+template <int NB, int CT>
+__device__ __forceinline__ void reset_partials(float* red, int live) {
+  using P = ProductTile<NB, CT>;
+  constexpr int TILE = NB * P::NCOLS;
+  for (int i = set_thread<2>(); i < 2 * P::kRedFloats; i += 256)
+    red[i] = (i % P::kRedFloats) / TILE < live ? unwritten_value() : 0.f;
+}
+
 // ---- host side ---------------------------------------------------------------------
 // Partial tiles slice_product leaves in LDS (ProductTile<nb, ct>::kPartials).
 inline int product_partials(int nb, int ct) {
@@ -842,6 +949,7 @@ struct LaunchPlan {
   dim3 grid;
   size_t lds_bytes;
   LaunchShape shape;
+  int threads = 256;  // 512: two 256-thread sets per workgroup
 };
 
 constexpr int kXcdCount = 8;
@@ -914,7 +1022,7 @@ int launch_persistent(const char* name, KernelT kernel, const LaunchPlan& plan, 
   auto found = k.per_cu.find(plan.lds_bytes);
   if (found == k.per_cu.end()) {
     int blocks = 0;
-    HASTE_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, kernel, 256, plan.lds_bytes));
+    HASTE_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, kernel, plan.threads, plan.lds_bytes));
     found = k.per_cu.emplace(plan.lds_bytes, blocks).first;
   }
   const int per_cu = found->second;
@@ -923,7 +1031,7 @@ int launch_persistent(const char* name, KernelT kernel, const LaunchPlan& plan, 
   HASTE_HIP_PROPAGATE(order_persistent_launches(stream, true));
   {
     ScopedKernelTimer timer(name, stream);
-    kernel<<<plan.grid, dim3(256), plan.lds_bytes, stream>>>(params);
+    kernel<<<plan.grid, dim3((unsigned)plan.threads), plan.lds_bytes, stream>>>(params);
     HASTE_HIP_TRY(hipGetLastError());
   }
   HASTE_HIP_PROPAGATE(order_persistent_launches(stream, false));

@@ -105,6 +105,14 @@ bool xcd_local_enabled() {
   return enabled;
 }
 
+bool paired_sets_enabled() {
+  static const bool enabled = [] {
+    const char* v = std::getenv("HASTE_HIP_PAIRED_SETS");
+    return v == nullptr || v[0] != '0';
+  }();
+  return enabled;
+}
+
 int device_cu_count() {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
