@@ -29,32 +29,40 @@ struct GruFwdParams {
 
 // HS hidden units per workgroup; their 3 gate columns occupy 3*HS of the 16*CT slice
 // columns (the rest are zero padding).
-// NB batch rows per workgroup.
-template <int NB, int CT, int HS>
-__global__ __launch_bounds__(256, 1)
+// SETS sets of 256 threads, each with a batch tile of NB rows of its own.  Two sets share
+// the resident slice but nothing else: while one waits for its exchange the other computes,
+// which a single tile of 2*NB rows cannot do.
+template <int NB, int CT, int HS, int SETS>
+__global__ __launch_bounds__(256 * SETS, 1)
 void gru_forward_kernel(GruFwdParams p) {
   static_assert(3 * HS <= 16 * CT, "slice too narrow");
+  static_assert(SETS == 1 || (SETS == 2 && NB < 16), "two sets: short tiles only");
   constexpr int NCOLS = 16 * CT;
   constexpr int PP = (NB * HS + 255) / 256;
+  constexpr int RED = ProductTile<NB, CT>::kRedFloats;
+  constexpr bool kPolledPartials = SETS == 2;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int H = p.H, N = p.N, T = p.T;
   const int Kpad = round_up(H, 64);
+  const int set = set_index<SETS>();
   float* w_lds = lds;
-  float* red = lds + Kpad * NCOLS;
+  // one set: one area of partial tiles behind workgroup barriers; two sets: two polled
+  // areas each, alternating by step
+  float* red = lds + Kpad * NCOLS + (SETS == 1 ? 0 : set * 2 * RED);
   // The role is handed round through a word of the partial-tile area, which nothing else
   // uses before the first step: the kernel has no static LDS, so that a slice and its
   // partial tiles may fill the workgroup's 160 KiB exactly (N = 128, H = 1024).
-  const Role role = take_role(p.ls, reinterpret_cast<unsigned int*>(red));
+  const Role role = take_role(p.ls, reinterpret_cast<unsigned int*>(lds + Kpad * NCOLS));
   if (!role.active) return;
 
-  const int tid = threadIdx.x;
+  const int tid = set_thread<SETS>();
   const int j0 = role.cw * HS;
-  const int n0 = role.bt * p.ls.tile_rows;
-  const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
+  const int n0 = (role.bt * SETS + set) * NB;
+  const int rows_here = (N - n0) < NB ? (N - n0) : NB;  // <= 0: a set without rows
   const size_t NH = (size_t)N * H;
 
   const int tile_floats = Kpad * NB;
-  float* xh = p.xh + (size_t)role.bt * kPolledTiles * tile_floats;
+  float* xh = p.xh + (size_t)(role.bt * SETS + set) * kPolledTiles * tile_floats;
   const TileBuffer xhb = make_tile_buffer(xh, kPolledTiles * tile_floats);
 
   GroupSync gs;
@@ -62,8 +70,8 @@ void gru_forward_kernel(GruFwdParams p) {
 
   // Own k range of the exchange tiles (the last workgroup also owns the padding): rows and
   // k beyond the problem stay zero for the whole launch.
-  zero_tile_share(gs, xh, tile_floats, NB, j0 / 4,
-                  (role.cw == p.ls.gx - 1 ? Kpad - j0 : HS) / 4, kPolledTiles);
+  zero_tile_share<SETS>(gs, xh, tile_floats, NB, j0 / 4,
+                        (role.cw == p.ls.gx - 1 ? Kpad - j0 : HS) / 4, kPolledTiles);
 
   {
     const bool fast = H % 4 == 0 && ((reinterpret_cast<uintptr_t>(p.R) |
@@ -107,8 +115,10 @@ void gru_forward_kernel(GruFwdParams p) {
       store_exchanged(gs, e, publishable(h_prev[pp]));
       for (int b = 1; b < kPolledTiles; ++b) store_exchanged(gs, e + (size_t)b * tile_floats, unwritten_value());
     }
+  if constexpr (SETS == 2) reset_partials<NB, CT>(red, live_partials<CT>(Kpad));
   group_arrive(gs);  // also: the slice is complete in LDS
   group_wait(gs);
+  if (SETS == 2 && rows_here <= 0) return;  // no workgroup barrier from here on
 
   // Inputs of a step that do not depend on the recurrence (x*W, the zoneout mask) are
   // fetched one step ahead.
@@ -138,17 +148,25 @@ void gru_forward_kernel(GruFwdParams p) {
       for (int g = 0; g < 3; ++g) wx[pp][g] = wx_next[pp][g];
     }
     // The operand loads wait for h[t] themselves (polled tile t % 4).
-    tile_product<NB, CT, false, true>(xhb, (t & 3) * tile_floats, Kpad, w_lds, red, &gs);
-    __syncthreads();
+    float* red_t = !kPolledPartials ? red : red + (t & 1) * RED;
+    tile_product<NB, CT, false, true, kPolledPartials>(xhb, (t & 3) * tile_floats, Kpad, w_lds, red_t, &gs);
+    if constexpr (!kPolledPartials) __syncthreads();
 
     float saved[PP][4];  // z, r, g, q of the step for the caller's cache
     float h_pub[PP];
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
-      if (act[pp]) {
-        float rh[3];
+      float rh[3] = {0.f, 0.f, 0.f};
+      if constexpr (kPolledPartials) {
+        // whole wavefronts: the wait is a wavefront-wide vote
+        if (((tid + 256 * pp) & ~63) < NB * HS)
+          take_product<NB, CT, 3>(gs, red_t, pl[pp], pc[pp], HS, tid + 256 * pp < NB * HS,
+                                  live_partials<CT>(Kpad), rh);
+      } else if (act[pp]) {
 #pragma unroll
         for (int g = 0; g < 3; ++g) rh[g] = sum_product<NB, CT>(red, pl[pp], g * HS + pc[pp]);
+      }
+      if (act[pp]) {
         const float z = sigmoid_f(wx[pp][0] + rh[0] + bxv[pp][0] + brv[pp][0]);
         const float r = sigmoid_f(wx[pp][1] + rh[1] + bxv[pp][1] + brv[pp][1]);
         const float qg = rh[2] + brv[pp][2];
@@ -181,7 +199,7 @@ void gru_forward_kernel(GruFwdParams p) {
         }
     }
     fetch(t + 1);
-    __syncthreads();  // `red` may be overwritten by the next step's product
+    if constexpr (!kPolledPartials) __syncthreads();  // `red` may be overwritten by the next step's product
     // The caller's copies are written last: nobody in the launch waits for them.
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
@@ -221,13 +239,17 @@ inline int gru_backward_k(int H) { return 48 * ((H + 15) / 16); }
 
 // A workgroup owns 16 hidden units for NB batch rows; its slice of R_t is [3H x 16].
 // Inside the launch the contraction index runs unit-major (k = 3*unit + gate), so every
-// workgroup publishes one contiguous k range of the exchange tile.
-template <int NB>
-__global__ __launch_bounds__(256, 1)
+// workgroup publishes one contiguous k range of the exchange tile.  SETS sets of 256 threads,
+// each with a batch tile of NB rows of its own (see gru_forward_kernel).
+template <int NB, int SETS>
+__global__ __launch_bounds__(256 * SETS, 1)
 void gru_backward_kernel(GruBwdParams p) {
+  static_assert(SETS == 1 || (SETS == 2 && NB < 16), "two sets: short tiles only");
   constexpr int HSB = 16;
   constexpr int NCOLS = 16;
   constexpr int PP = (NB * HSB + 255) / 256;
+  constexpr int RED = ProductTile<NB, 1>::kRedFloats;
+  constexpr bool kPolledPartials = SETS == 2;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   __shared__ unsigned int s_role;
   const Role role = take_role(p.ls, &s_role);
@@ -236,17 +258,21 @@ void gru_backward_kernel(GruBwdParams p) {
 
   const int H = p.H, N = p.N, T = p.T;
   const int Kpad = round_up(48 * p.ls.gx, 64);
+  const int set = set_index<SETS>();
   float* w_lds = lds;
-  float* red = lds + Kpad * NCOLS;  // the partial tiles or NB*6*16 floats, whichever is more
+  // the partial tiles or NB*6*16 floats, whichever is more (two sets: two polled areas of
+  // partial tiles each, alternating by step)
+  float* red = lds + Kpad * NCOLS + (SETS == 1 ? 0 : set * 2 * RED);
 
-  const int tid = threadIdx.x;
+  const int tid = set_thread<SETS>();
   const int j0 = role.cw * HSB;
-  const int n0 = role.bt * p.ls.tile_rows;
-  const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
+  const int bt = role.bt * SETS + set;  // this set's batch tile
+  const int n0 = bt * NB;
+  const int rows_here = (N - n0) < NB ? (N - n0) : NB;  // <= 0: a set without rows
   const size_t NH = (size_t)N * H;
 
   const int tile_floats = Kpad * NB;
-  float* xdq = p.xdq + (size_t)role.bt * kPolledTiles * tile_floats;
+  float* xdq = p.xdq + (size_t)bt * kPolledTiles * tile_floats;
   const TileBuffer xdqb = make_tile_buffer(xdq, kPolledTiles * tile_floats);
 
   GroupSync gs;
@@ -254,8 +280,8 @@ void gru_backward_kernel(GruBwdParams p) {
 
   // Own k range of the exchange tiles (the last workgroup also owns the padding); only
   // rows and units of the problem are written afterwards.
-  zero_tile_share(gs, xdq, tile_floats, NB, 12 * role.cw,
-                  (role.cw == p.ls.gx - 1 ? Kpad - 48 * role.cw : 48) / 4, kPolledTiles);
+  zero_tile_share<SETS>(gs, xdq, tile_floats, NB, 12 * role.cw,
+                        (role.cw == p.ls.gx - 1 ? Kpad - 48 * role.cw : 48) / 4, kPolledTiles);
 
   {
     const bool fast = H % 4 == 0 && (reinterpret_cast<uintptr_t>(p.R_t) & 15u) == 0;
@@ -291,6 +317,7 @@ void gru_backward_kernel(GruBwdParams p) {
         for (int g = 0; g < 3; ++g)
           store_exchanged(gs, xdq + (size_t)b * tile_floats + xchg_index(3 * pj[pp] + g, pl[pp], NB),
                           unwritten_value());
+  if constexpr (SETS == 2) reset_partials<NB, 1>(red, live_partials<1>(Kpad));
   group_arrive(gs);  // also: the slice is complete in LDS
   group_wait(gs);
 
@@ -314,7 +341,8 @@ void gru_backward_kernel(GruBwdParams p) {
   };
   fetch(T - 1);
 
-  for (int t = T - 1; t >= 0; --t) {
+  // A set without rows skips the steps (two sets: no workgroup barrier inside them).
+  for (int t = (SETS == 2 && rows_here <= 0) ? -1 : T - 1; t >= 0; --t) {
     float dh_keep[PP], dpv[PP][3], dqv[PP];
     const int done = T - 1 - t;  // steps done so far; this step uses polled tile done % 4
     float* xdq_t = xdq + (done & 3) * tile_floats;
@@ -381,12 +409,24 @@ void gru_backward_kernel(GruBwdParams p) {
     }
     fetch(t - 1);
     // The operand loads wait for dq_t of every unit themselves.
-    tile_product<NB, 1, true, true>(xdqb, (done & 3) * tile_floats, Kpad, w_lds, red, &gs);
-    __syncthreads();
+    float* red_t = !kPolledPartials ? red : red + (done & 1) * RED;
+    tile_product<NB, 1, true, true, kPolledPartials>(xdqb, (done & 3) * tile_floats, Kpad, w_lds, red_t, &gs);
+    if constexpr (kPolledPartials) {
 #pragma unroll
-    for (int pp = 0; pp < PP; ++pp)
-      if (tid + 256 * pp < NB * HSB) dh[pp] = dh_keep[pp] + sum_product<NB, 1>(red, pl[pp], pc[pp]);
-    __syncthreads();  // `red` may be overwritten by the next step's product
+      for (int pp = 0; pp < PP; ++pp)
+        if (((tid + 256 * pp) & ~63) < NB * HSB) {  // whole wavefronts: the wait is a vote
+          float rdq[1];
+          take_product<NB, 1, 1>(gs, red_t, pl[pp], pc[pp], 0, tid + 256 * pp < NB * HSB,
+                                 live_partials<1>(Kpad), rdq);
+          if (tid + 256 * pp < NB * HSB) dh[pp] = dh_keep[pp] + rdq[0];
+        }
+    } else {
+      __syncthreads();
+#pragma unroll
+      for (int pp = 0; pp < PP; ++pp)
+        if (tid + 256 * pp < NB * HSB) dh[pp] = dh_keep[pp] + sum_product<NB, 1>(red, pl[pp], pc[pp]);
+      __syncthreads();  // `red` may be overwritten by the next step's product
+    }
   }
 
 #pragma unroll
@@ -405,12 +445,12 @@ void gru_backward_kernel(GruBwdParams p) {
     const int g = tid / HSB, jj = tid % HSB;
     float s = 0.f;
     for (int r = 0; r < NB; ++r) s += red[(r * 6 + g) * HSB + jj];
-    if (j0 + jj < H) store_agent(&p.db_partial[(size_t)role.bt * 6 * H + g * H + j0 + jj], s);
+    if (j0 + jj < H) store_agent(&p.db_partial[(size_t)bt * 6 * H + g * H + j0 + jj], s);
   }
   if (column_last_arrival(p.ls.cb, role.cw, (unsigned)p.ls.gy, &s_flag)) {
-    if (tid < 6 * HSB && j0 + tid % HSB < H) {
+    if (set == 0 && tid < 6 * HSB && j0 + tid % HSB < H) {
       const int col = (tid / HSB) * H + j0 + tid % HSB;
-      const float s = sum_over_tiles(p.db_partial + col, (size_t)6 * H, p.ls.gy);
+      const float s = sum_over_tiles(p.db_partial + col, (size_t)6 * H, p.ls.gy * SETS);
       if (col < 3 * H) p.dbx[col] += s;
       else p.dbr[col - 3 * H] += s;
     }
@@ -435,6 +475,11 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
                                 zoneout_prob, zoneout_mask, dc_mask, dc_scale);
   HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 3 * H, C, x, C, W, 3 * H, tmp_Wx, 3 * H, false));
 
+  // An 8-row tile is run as two sets of 4 rows when the partial tiles of both fit beside the
+  // slice (exchange tiles: one per set, together as large as the tile's).
+  const size_t paired_lds = paired_lds_bytes((H + 63) / 64 * 64, tile.ct);
+  const bool paired = tile.nb == 8 && paired_lds <= kWorkgroupLdsBytes && paired_sets_enabled();
+
   // Taken after the GEMM, which may replace the stream's scratch buffer with a larger one.
   Workspace ws;
   HASTE_HIP_PROPAGATE(get_workspace(
@@ -448,11 +493,19 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
   p.dc_mask = dc_mask; p.dc_scale = dc_scale;
   p.xh = ws.scratch;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.nb, tile.lds_bytes, (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.nb,
+                                  paired ? paired_lds : tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;
+  if (paired) plan.threads = 512;
+#define HASTE_LAUNCH_FWD_PAIRED(CT_, HS_)                                                     \
+  if (paired && tile.hs == HS_)                                                               \
+    return launch_persistent("gru_forward_recurrence", gru_forward_kernel<4, CT_, HS_, 2>,    \
+                             plan, p, stream);
+  HASTE_LAUNCH_FWD_PAIRED(1, 4) HASTE_LAUNCH_FWD_PAIRED(2, 8) HASTE_LAUNCH_FWD_PAIRED(3, 16)
+#undef HASTE_LAUNCH_FWD_PAIRED
 #define HASTE_LAUNCH_FWD(NB_, CT_, HS_)                                                       \
   if (tile.nb == NB_ && tile.hs == HS_)                                                       \
-    return launch_persistent("gru_forward_recurrence", gru_forward_kernel<NB_, CT_, HS_>,     \
+    return launch_persistent("gru_forward_recurrence", gru_forward_kernel<NB_, CT_, HS_, 1>,  \
                              plan, p, stream);
   HASTE_LAUNCH_FWD(4, 1, 4) HASTE_LAUNCH_FWD(4, 2, 8) HASTE_LAUNCH_FWD(4, 3, 16)
   HASTE_LAUNCH_FWD(8, 1, 4) HASTE_LAUNCH_FWD(8, 2, 8) HASTE_LAUNCH_FWD(8, 3, 16)
@@ -477,8 +530,13 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
     return gru_backward_streamed(stream, T, N, C, H, W_t, R_t, x_t, h, v, dh_next, dx, dW, dR, dbx,
                                  dbr, dh, dp, dq, zoneout_mask);
 
+  // An 8-row tile is run as two sets of 4 rows (see gru_forward_impl).
+  const size_t paired_lds = paired_lds_bytes((gru_backward_k(H) + 63) / 64 * 64, 1);
+  const bool paired = tile.nb == 8 && paired_lds <= kMaxLdsBytes && paired_sets_enabled();
+  const int sets = paired ? 2 : 1;
+
   Workspace ws;
-  const size_t db_floats = ((size_t)tile.gy * 6 * H + 3) / 4 * 4;
+  const size_t db_floats = ((size_t)tile.gy * sets * 6 * H + 3) / 4 * 4;
   const size_t xdq_floats = exchange_floats(gru_backward_k(H), tile.nb, tile.gy, kPolledTiles);
   HASTE_HIP_PROPAGATE(get_workspace(stream, (db_floats + xdq_floats) * sizeof(float), &ws));
   HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
@@ -490,15 +548,18 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   p.db_partial = ws.scratch;
   p.xdq = ws.scratch + db_floats;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.nb, tile.lds_bytes, (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.nb,
+                                  paired ? paired_lds : tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;
+  if (paired) plan.threads = 512;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const char* name = "gru_backward_recurrence";
-  if (tile.nb == 4) rc = launch_persistent(name, gru_backward_kernel<4>, plan, p, stream);
-  if (tile.nb == 8) rc = launch_persistent(name, gru_backward_kernel<8>, plan, p, stream);
-  if (tile.nb == 16) rc = launch_persistent(name, gru_backward_kernel<16>, plan, p, stream);
-  if (tile.nb == 32) rc = launch_persistent(name, gru_backward_kernel<32>, plan, p, stream);
-  if (tile.nb == 64) rc = launch_persistent(name, gru_backward_kernel<64>, plan, p, stream);
+  if (paired) rc = launch_persistent(name, gru_backward_kernel<4, 2>, plan, p, stream);
+  else if (tile.nb == 4) rc = launch_persistent(name, gru_backward_kernel<4, 1>, plan, p, stream);
+  else if (tile.nb == 8) rc = launch_persistent(name, gru_backward_kernel<8, 1>, plan, p, stream);
+  else if (tile.nb == 16) rc = launch_persistent(name, gru_backward_kernel<16, 1>, plan, p, stream);
+  else if (tile.nb == 32) rc = launch_persistent(name, gru_backward_kernel<32, 1>, plan, p, stream);
+  else if (tile.nb == 64) rc = launch_persistent(name, gru_backward_kernel<64, 1>, plan, p, stream);
   HASTE_HIP_PROPAGATE(rc);
 
   const int TN = T * N;

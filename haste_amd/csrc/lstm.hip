@@ -480,9 +480,7 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
   // An 8-row tile is run as two sets of 4 rows when the partial tiles of both fit beside the
   // slice (exchange tiles: one per set, together as large as the tile's).  Measured at
   // H = 512: 6 % faster per step; two sets of 8 rows instead of a 16-row tile: 6 % slower.
-  const int half = tile.nb / 2;
-  const size_t paired_lds = fwd_lds_bytes(H, half, tile.ct) +
-      3 * (size_t)product_partials(half, tile.ct) * half * 16 * tile.ct * sizeof(float);
+  const size_t paired_lds = paired_lds_bytes((H + 63) / 64 * 64, tile.ct);
   const bool paired = tile.nb == 8 && paired_lds <= kWorkgroupLdsBytes && paired_sets_enabled();
 
   // Taken after the GEMM, which may replace the stream's scratch buffer with a larger one.
@@ -502,11 +500,11 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
                                   paired ? paired_lds : tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;
   if (paired) plan.threads = 512;
-#define HASTE_LAUNCH_FWD_PAIRED(NB_, CT_)                                                  \
-  if (paired && half == NB_ && tile.ct == CT_)                                             \
-    return launch_persistent("lstm_forward_recurrence", lstm_forward_kernel<NB_, CT_, 2>, plan, p, \
+#define HASTE_LAUNCH_FWD_PAIRED(CT_)                                                       \
+  if (paired && tile.ct == CT_)                                                            \
+    return launch_persistent("lstm_forward_recurrence", lstm_forward_kernel<4, CT_, 2>, plan, p, \
                              stream);
-  HASTE_LAUNCH_FWD_PAIRED(4, 1) HASTE_LAUNCH_FWD_PAIRED(4, 2) HASTE_LAUNCH_FWD_PAIRED(4, 4)
+  HASTE_LAUNCH_FWD_PAIRED(1) HASTE_LAUNCH_FWD_PAIRED(2) HASTE_LAUNCH_FWD_PAIRED(4)
 #undef HASTE_LAUNCH_FWD_PAIRED
 #define HASTE_LAUNCH_FWD(NB_, CT_)                                                         \
   if (tile.nb == NB_ && tile.ct == CT_)                                                    \
@@ -539,8 +537,7 @@ int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
 
   // An 8-row tile is run as two sets of 4 rows (see lstm_forward_impl): four polled areas of
   // partial tiles beside the slice.
-  const size_t paired_lds =
-      ((size_t)64 * tile.gx * 16 + 4 * (size_t)product_partials(4, 1) * 4 * 16) * sizeof(float);
+  const size_t paired_lds = paired_lds_bytes(64 * tile.gx, 1);
   const bool paired = tile.nb == 8 && paired_lds <= kMaxLdsBytes && paired_sets_enabled();
   const int sets = paired ? 2 : 1;
 

@@ -941,6 +941,12 @@ inline size_t fwd_lds_bytes(int H, int nb, int ct) {
   return ((size_t)Kpad * 16 * ct + (size_t)product_partials(nb, ct) * nb * 16 * ct) * sizeof(float);
 }
 
+// LDS bytes of a kernel that runs an 8-row tile as two sets of 4 rows: the slice
+// [Kpad x 16*ct] and, per set, two polled areas of partial tiles.
+inline size_t paired_lds_bytes(int Kpad, int ct) {
+  return ((size_t)Kpad * 16 * ct + 4 * (size_t)product_partials(4, ct) * 4 * 16 * ct) * sizeof(float);
+}
+
 // Host-side plan of a persistent launch: fills `shape` and the grid for (gx, gy).
 // An XCD-local launch is used when every group fits on one XCD (gx <= CUs per XCD,
 // gy <= XCDs); it fills the chip with one workgroup per CU (the LDS request is raised so
