@@ -1,0 +1,83 @@
+"""LSTM / GRU recurrences: an 8-row batch tile run as two 4-row sets per workgroup gives the
+same bits as one tile per workgroup.
+
+The split only changes which wavefronts work on which rows and how they wait for each other;
+every element is still the same sum in the same order -- except the bias gradients, whose sum
+over the batch is grouped by tile (4 rows at a time instead of 8) and so differs by rounding.
+The one-tile variant is selected by an environment variable that the library reads once, so it
+runs in a child process."""
+import os
+import subprocess
+import sys
+import tempfile
+
+import numpy as np
+import pytest
+
+from util import dev, host, problem, relerr
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+# (T, N, C, H): 8-row tiles with a ragged last set / a set without rows / full sets
+SHAPES = [(6, 41, 24, 512), (5, 64, 32, 256), (4, 36, 8, 72)]
+BATCH_SUMS = ("lstm_db", "gru_5", "gru_6")  # db; dbx, dbr
+
+
+def run_cells(T, N, C, H):
+    """LSTM and GRU forward + backward with zoneout; every output as float64 arrays."""
+    import torch
+    from haste_amd import ops
+    out = {}
+    p = problem(900 + T + N + C + H, T, N, C, H, 4, 0.2)
+    mask = dev(p["mask"])
+    h, c, cache = ops.lstm_forward(True, 0.2, dev(p["x"]), dev(p["h0"]), dev(p["c0"]),
+                                   dev(p["W"]), dev(p["R"]), dev(p["b"]), mask)
+    x_t = dev(p["x"]).permute(2, 0, 1).contiguous()
+    grads = ops.lstm_backward(x_t, dev(p["W"]).t().contiguous(), dev(p["R"]).t().contiguous(),
+                              dev(p["b"]), mask, h, c, cache, dev(p["dh_new"]), dev(p["dc_new"]))
+    for name, t in zip(("h", "c", "dx", "dh", "dc", "dW", "dR", "db", "dv"), (h, c) + tuple(grads) + (cache,)):
+        out["lstm_" + name] = host(t)
+
+    p = problem(901 + T + N + C + H, T, N, C, H, 3, 0.2)
+    mask = dev(p["mask"])
+    W, R, bx, br = dev(p["W"]), dev(p["R"]), dev(p["b"]), dev(p["b2"])
+    h, cache = ops.gru_forward(True, 0.2, dev(p["x"]), dev(p["h0"]), W, R, bx, br, mask)
+    x_t = dev(p["x"]).permute(2, 0, 1).contiguous()
+    grads = ops.gru_backward(x_t, W.t().contiguous(), R.t().contiguous(), bx, br, mask, h, cache,
+                             dev(p["dh_new"]))
+    for i, t in enumerate((h,) + tuple(grads)):
+        out["gru_%d" % i] = host(t)
+    torch.cuda.synchronize()
+    return out
+
+
+def child(path):
+    arrays = {}
+    for shape in SHAPES:
+        for k, v in run_cells(*shape).items():
+            arrays["%d_%d_%d_%d_%s" % (shape + (k,))] = v
+    np.savez(path, **arrays)
+
+
+def test_two_sets_match_one_tile_bit_for_bit():
+    with tempfile.TemporaryDirectory() as d:
+        path = os.path.join(d, "one_tile.npz")
+        env = dict(os.environ, HASTE_HIP_PAIRED_SETS="0",
+                   PYTHONPATH=os.pathsep.join([ROOT, os.path.join(ROOT, "tests")]))
+        res = subprocess.run([sys.executable, os.path.abspath(__file__), path], env=env,
+                             capture_output=True, text=True, timeout=110)
+        assert res.returncode == 0, res.stdout + res.stderr
+        one_tile = np.load(path)
+        for shape in SHAPES:
+            print("paired sets vs one tile", shape, flush=True)
+            for k, v in run_cells(*shape).items():
+                ref = one_tile["%d_%d_%d_%d_%s" % (shape + (k,))]
+                if k in BATCH_SUMS:
+                    assert relerr(v, ref) < 2e-6, (shape, k)
+                else:
+                    assert np.array_equal(v, ref), (shape, k)
+
+
+if __name__ == "__main__":
+    child(sys.argv[1])
