@@ -177,33 +177,47 @@ void layer_norm_backward_kernel(int rows, int D, const float* __restrict__ gamma
   }
 }
 
-// dgamma (and dbeta) += the workgroups' column sums, added in workgroup order.  A thread owns
-// one column and every fourth workgroup; the four partial sums of a column are then combined
-// in a fixed order, so the result does not depend on timing.
-__global__ __launch_bounds__(256)
+// dgamma (and dbeta) += the workgroups' column sums.  A workgroup of 1024 threads owns 64
+// columns; a thread adds every sixteenth partial row of one column (eight loads in flight),
+// and the sixteen sums of a column are then combined pairwise in a fixed order, so the result
+// does not depend on timing.
+constexpr int kReduceGroups = 16;
+
+__global__ __launch_bounds__(64 * kReduceGroups)
 void layer_norm_reduce_kernel(int parts, int D, const float* __restrict__ partial,
                               float* __restrict__ dgamma, float* __restrict__ dbeta) {
-  __shared__ float sums[4][64];
-  const int c = blockIdx.x * 64 + (threadIdx.x & 63);
+  __shared__ float sums[kReduceGroups][64];
+  const int l = threadIdx.x & 63;
+  const int c = blockIdx.x * 64 + l;
   const int q = threadIdx.x >> 6;
-  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  constexpr int U = 8;
+  float s[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) s[u] = 0.f;
   if (c < 2 * D) {
+    const size_t row = (size_t)2 * D;
     int b = q;
-    for (; b + 12 < parts; b += 16) {  // four loads in flight
-      s0 += partial[(size_t)b * 2 * D + c];
-      s1 += partial[(size_t)(b + 4) * 2 * D + c];
-      s2 += partial[(size_t)(b + 8) * 2 * D + c];
-      s3 += partial[(size_t)(b + 12) * 2 * D + c];
+    for (; b + (U - 1) * kReduceGroups < parts; b += U * kReduceGroups) {
+      float v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = partial[(size_t)(b + u * kReduceGroups) * row + c];
+#pragma unroll
+      for (int u = 0; u < U; ++u) s[u] += v[u];
     }
-    for (; b < parts; b += 4) s0 += partial[(size_t)b * 2 * D + c];
+    for (; b < parts; b += kReduceGroups) s[0] += partial[(size_t)b * row + c];
   }
-  sums[q][threadIdx.x & 63] = (s0 + s1) + (s2 + s3);
+  sums[q][l] = ((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]));
   __syncthreads();
   if (q == 0 && c < 2 * D) {
-    const int l = threadIdx.x & 63;
-    const float s = (sums[0][l] + sums[1][l]) + (sums[2][l] + sums[3][l]);
-    if (c < D) dgamma[c] += s;
-    else if (dbeta != nullptr) dbeta[c - D] += s;
+    float t[kReduceGroups];
+#pragma unroll
+    for (int g = 0; g < kReduceGroups; ++g) t[g] = sums[g][l];
+#pragma unroll
+    for (int w = kReduceGroups / 2; w > 0; w >>= 1)
+#pragma unroll
+      for (int g = 0; g < w; ++g) t[g] = t[2 * g] + t[2 * g + 1];
+    if (c < D) dgamma[c] += t[0];
+    else if (dbeta != nullptr) dbeta[c - D] += t[0];
   }
 }
 
@@ -221,7 +235,7 @@ int elements_per_lane(int D, bool vec) {
 
 int add_column_partials(hipStream_t stream, int parts, int D, const float* partial, float* first,
                         float* second) {
-  layer_norm_reduce_kernel<<<dim3((unsigned)((2 * D + 63) / 64)), dim3(256), 0, stream>>>(
+  layer_norm_reduce_kernel<<<dim3((unsigned)((2 * D + 63) / 64)), dim3(64 * kReduceGroups), 0, stream>>>(
       parts, D, partial, first, second);
   HASTE_HIP_TRY(hipGetLastError());
   return HASTE_HIP_OK;
@@ -260,7 +274,7 @@ int layer_norm_backward(hipStream_t stream, int rows, int dim, const float* gamm
   if (E == 0) return layer_norm_backward_wide(stream, rows, dim, gamma, x, dy, dx, dgamma, dbeta);
   const int cus = device_cu_count();
   int grid = (rows + 3) / 4;
-  if (grid > 2 * cus) grid = 2 * cus;
+  if (grid > 2 * cus) grid = 2 * cus;  // measured: 3, 4 and 6 per CU are no faster
   Workspace ws;
   HASTE_HIP_PROPAGATE(get_workspace(stream, (size_t)grid * 2 * dim * sizeof(float), &ws));
   const size_t lds = (size_t)4 * 2 * E * 64 * sizeof(float);
