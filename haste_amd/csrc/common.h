@@ -94,6 +94,11 @@ bool xcd_local_enabled();
 // batch tiles then run as one tile instead of two sets of half the rows (for experiments).
 bool paired_sets_enabled();
 
+// False when the environment variable HASTE_HIP_SINGLE_ROW is set to 0: an LSTM forward pass
+// with one batch row then runs as a 4-row tile instead of the kernel that keeps the recurrent
+// weights in registers (for experiments).
+bool single_row_enabled();
+
 // C[M,N] = op(A)*B (+C): fp32 MFMA GEMM on `stream`.  The partial tiles of a split product
 // are kept `scratch_offset` bytes (a multiple of 16) into the stream's scratch buffer.
 int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,

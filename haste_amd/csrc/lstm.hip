@@ -218,6 +218,164 @@ void lstm_forward_kernel(LstmFwdParams p) {
   }
 }
 
+// ---- batch of one -----------------------------------------------------------------------
+// With a single batch row the step's product is a matrix-vector product.  The 4-row MFMA tile
+// spends three quarters of the matrix unit's time on padding and, like any tile, reads the
+// whole slice from LDS every step (128 KiB at H = 512: 0.45 us at the LDS's rate).  Here the
+// slice lives in REGISTERS: a thread owns one of the 64 slice columns (16 hidden units x 4
+// gates) and a quarter of k, i.e. up to 128 weights, and a step is up to 128 FMAs per thread
+// against h, which the wavefront polls from the exchange tile, parks in LDS and reads back as
+// broadcast 16-byte reads.  KW: the k range of a wavefront (Kpad / 4, at most the template's).
+template <int KW_MAX>
+__global__ __launch_bounds__(256, 1)
+void lstm_forward_single_row_kernel(LstmFwdParams p) {
+  constexpr int HS = 16, NCOLS = 64;
+  // No static LDS (launch_persistent sizes the dynamic limit for kernels without any):
+  // [4][KW_MAX] a wavefront's share of h, [2][4][NCOLS] partial sums by step parity and
+  // wavefront, one word for the role.
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  float (*h_lds)[KW_MAX] = reinterpret_cast<float (*)[KW_MAX]>(lds);
+  float (*red)[4][NCOLS] = reinterpret_cast<float (*)[4][NCOLS]>(lds + 4 * KW_MAX);
+  const int H = p.H, T = p.T;
+  const int Kpad = round_up(H, 64);
+  const int KW = Kpad / 4;  // multiple of 16
+  const Role role = take_role(p.ls, reinterpret_cast<unsigned int*>(lds + 4 * KW_MAX + 2 * 4 * NCOLS));
+  if (!role.active) return;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int j0 = role.cw * HS;
+  float* xh = p.xh;  // one batch tile: [4 polled tiles][Kpad]
+  const TileBuffer xhb = make_tile_buffer(xh, kPolledTiles * Kpad);
+
+  GroupSync gs;
+  group_sync_init(gs, p.ls, role);
+  // Own k range of the exchange tiles (the last workgroup also owns the padding).
+  zero_tile_share(gs, xh, Kpad, 1, j0 / 4, (role.cw == p.ls.gx - 1 ? Kpad - j0 : HS) / 4, kPolledTiles);
+
+  // The thread's weights: column `lane` (gate lane/16, unit j0 + lane%16), k = wave*KW + i.
+  float w[KW_MAX];
+  {
+    const int gate = lane / HS, j = j0 + lane % HS;
+#pragma unroll
+    for (int i = 0; i < KW_MAX; ++i) {
+      const int k = wave * KW + i;
+      float v = 0.f;
+      if (i < KW && k < H && j < H) {
+        const size_t o = (size_t)k * 4 * H + gate * H + j;
+        v = p.R[o];
+        if (p.dc_mask != nullptr) v = v * p.dc_mask[o] * p.dc_scale;
+      }
+      w[i] = v;
+    }
+  }
+
+  for (int i = tid; i < 4 * KW_MAX; i += 256) (&h_lds[0][0])[i] = 0.f;  // ordered by group_arrive's barrier
+
+  // Pointwise ownership: thread u < 16 handles hidden unit j0 + u.
+  const int pj = j0 + tid;
+  const bool act = tid < HS && pj < H;
+  float c_prev = 0.f, h_prev = 0.f, bias[4] = {0.f, 0.f, 0.f, 0.f};
+  if (act) {
+    c_prev = p.c[pj];
+    h_prev = p.h[pj];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) bias[g] = p.b[g * H + pj];
+  }
+  const bool zoneout = p.zoneout_prob != 0.f && p.zoneout_mask != nullptr;
+  // Tile 0 receives h[0]; the elements of the other tiles that steps will publish start out
+  // unwritten.  One real barrier: nobody polls a tile before all of its owners have set it up.
+  if (act) {
+    store_exchanged(gs, &xh[pj], publishable(h_prev));
+    for (int b = 1; b < kPolledTiles; ++b) store_exchanged(gs, &xh[b * Kpad + pj], unwritten_value());
+  }
+  group_arrive(gs);
+  group_wait(gs);
+
+  float wx_next[4], mk_next;
+  auto fetch = [&](int t) {
+    mk_next = 1.f;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) wx_next[g] = 0.f;
+    if (act && t < T) {
+      const float* vt = p.v + (size_t)t * 4 * H + pj;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) wx_next[g] = vt[g * H];
+      if (zoneout && p.training) mk_next = p.zoneout_mask[(size_t)t * H + pj];
+    }
+  };
+  fetch(0);
+
+  for (int t = 0; t < T; ++t) {
+    float wx[4];
+    const float mk = mk_next;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) wx[g] = wx_next[g];
+
+    // The wavefront's share of h[t]: lanes 0 .. KW/4-1 poll four k each (polled tile t % 4).
+    const int off = (t & 3) * Kpad + wave * KW + 4 * lane;
+    const bool loads = 4 * lane < KW;
+    float4_t hv[1][1];
+    auto load = [&] { hv[0][0] = loads ? load_tile4(xhb, off) : float4_t{0.f, 0.f, 0.f, 0.f}; };
+    load();
+    poll_until_written(gs, load, [&] { return all_written(hv); });
+    if (loads) *reinterpret_cast<float4_t*>(&h_lds[wave][4 * lane]) = hv[0][0];
+    // LDS operations of a wavefront complete in order: the reads below see the store above.
+    float acc0 = 0.f, acc1 = 0.f;
+    // (k beyond KW: the weights and the parked h are zero, so no step of the loop is conditional)
+#pragma unroll
+    for (int i = 0; i < KW_MAX; i += 4) {
+      const float4_t h4 = *reinterpret_cast<const float4_t*>(&h_lds[wave][i]);
+      acc0 = fmaf(w[i], h4.x, acc0);
+      acc1 = fmaf(w[i + 1], h4.y, acc1);
+      acc0 = fmaf(w[i + 2], h4.z, acc0);
+      acc1 = fmaf(w[i + 3], h4.w, acc1);
+    }
+    red[t & 1][wave][lane] = acc0 + acc1;
+    __syncthreads();
+
+    float gate[4] = {0.f, 0.f, 0.f, 0.f};
+    if (act) {
+      float a[4];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const float* r = &red[t & 1][0][g * HS + tid];
+        a[g] = wx[g] + ((r[0] + r[NCOLS]) + (r[2 * NCOLS] + r[3 * NCOLS])) + bias[g];
+      }
+      gate[0] = sigmoid_f(a[0]);
+      gate[1] = tanh_f(a[1]);
+      gate[2] = sigmoid_f(a[2]);
+      gate[3] = sigmoid_f(a[3]);
+      const float c_new = gate[2] * c_prev + gate[0] * gate[1];
+      float h_new = gate[3] * tanh_f(c_new);
+      if (zoneout) {
+        if (p.training) h_new = (h_new - h_prev) * mk + h_prev;
+        else h_new = p.zoneout_prob * h_prev + (1.0f - p.zoneout_prob) * h_new;
+      }
+      c_prev = c_new;
+      h_prev = h_new;
+    }
+    // Everything this wavefront stored during the previous step (its resets among it) has
+    // landed before h[t+1] becomes visible.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (act && t + 1 < T) {
+      store_exchanged(gs, &xh[((t + 1) & 3) * Kpad + pj], publishable(h_prev));
+      // the tile read at step t-1: nobody needs it any more
+      if (t + 3 < T) store_exchanged(gs, &xh[((t + 3) & 3) * Kpad + pj], unwritten_value());
+    }
+    fetch(t + 1);
+    // The caller's copies are written last: nobody in the launch waits for them.
+    if (act) {
+      if (p.training) {
+        float* vt = p.v + (size_t)t * 4 * H + pj;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) vt[g * H] = gate[g];
+      }
+      p.c_out[(size_t)t * H + pj] = c_prev;
+      p.h_out[(size_t)t * H + pj] = h_prev;
+    }
+  }
+}
+
 struct LstmBwdParams {
   int T, N, H;
   const float* R_t;     // [4H,H]
@@ -461,6 +619,35 @@ void lstm_backward_kernel(LstmBwdParams p) {
 
 }  // namespace
 
+// The forward pass of a single batch row with H <= 512: the recurrent weights live in the
+// registers of the 16-unit workgroups of one XCD (lstm_forward_single_row_kernel).
+int lstm_forward_single_row(hipStream_t stream, int training, int T, int C, int H,
+                            const float* W, const float* R, const float* b, const float* x,
+                            const float* h, const float* c, float* h_out, float* c_out, float* v,
+                            float zoneout_prob, const float* zoneout_mask, const float* dc_mask,
+                            float dc_scale) {
+  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T, 4 * H, C, x, C, W, 4 * H, v, 4 * H, false));
+  const int Kpad = (H + 63) / 64 * 64;
+  Workspace ws;
+  HASTE_HIP_PROPAGATE(get_workspace(stream, (size_t)kPolledTiles * Kpad * sizeof(float), &ws));
+  HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
+  LstmFwdParams p;
+  p.training = training; p.T = T; p.N = 1; p.H = H;
+  p.R = R; p.b = b; p.h = h; p.c = c; p.h_out = h_out; p.c_out = c_out; p.v = v;
+  p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
+  p.dc_mask = dc_mask; p.dc_scale = dc_scale;
+  p.xh = ws.scratch;
+  LaunchPlan plan;
+  const int kw_max = Kpad <= 128 ? 32 : (Kpad <= 256 ? 64 : 128);
+  const size_t lds_bytes = ((size_t)4 * kw_max + 2 * 4 * 64 + 4) * sizeof(float);
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, (H + 15) / 16, 1, 1, lds_bytes, (unsigned)T + 1, &plan));
+  p.ls = plan.shape;
+  const char* name = "lstm_forward_recurrence";
+  if (Kpad <= 128) return launch_persistent(name, lstm_forward_single_row_kernel<32>, plan, p, stream);
+  if (Kpad <= 256) return launch_persistent(name, lstm_forward_single_row_kernel<64>, plan, p, stream);
+  return launch_persistent(name, lstm_forward_single_row_kernel<128>, plan, p, stream);
+}
+
 // h, c: [N,H] state before the first step; h_out, c_out: [T,N,H] states after each step.
 int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int H,
                       const float* W, const float* R, const float* b, const float* x,
@@ -469,6 +656,9 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
                       float dc_scale) {
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
   HASTE_HIP_REQUIRE(W && R && b && x && h && c && h_out && c_out && v);
+  if (N == 1 && H <= 512 && xcd_local_fits((H + 15) / 16, 1) && single_row_enabled())
+    return lstm_forward_single_row(stream, training, T, C, H, W, R, b, x, h, c, h_out, c_out, v,
+                                   zoneout_prob, zoneout_mask, dc_mask, dc_scale);
   const ForwardTile tile = pick_forward_tile(4, N, H, 0, kWorkgroupLdsBytes);
   // No slice of R fits a CU: stream R from HBM every step instead.
   if (!tile.ok)

@@ -113,6 +113,14 @@ bool paired_sets_enabled() {
   return enabled;
 }
 
+bool single_row_enabled() {
+  static const bool enabled = [] {
+    const char* v = std::getenv("HASTE_HIP_SINGLE_ROW");
+    return v == nullptr || v[0] != '0';
+  }();
+  return enabled;
+}
+
 int device_cu_count() {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;

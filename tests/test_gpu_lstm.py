@@ -15,6 +15,8 @@ SHAPES = [(1, 1, 1, 1), (3, 2, 3, 4), (5, 3, 7, 5), (6, 17, 20, 36), (4, 16, 32,
           # hidden sizes that are not multiples of the 16 units of a workgroup
           (7, 41, 24, 512), (5, 57, 16, 200), (4, 36, 8, 72),
           (1, 40, 8, 128), (2, 64, 8, 64), (3, 50, 8, 16),
+          # one batch row: the forward pass keeps the recurrent weights in registers (H <= 512)
+          (9, 1, 7, 100), (6, 1, 16, 512), (5, 1, 8, 300), (4, 1, 8, 48), (7, 1, 5, 17),
           # hidden sizes beyond what stays on chip: the backward pass, then both passes, stream R
           (3, 5, 40, 640), (3, 4, 32, 1536), (2, 70, 24, 1300), (2, 128, 16, 1024)]
 
