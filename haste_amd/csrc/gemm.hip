@@ -63,7 +63,7 @@ __device__ __forceinline__ float4_t masked4(uint4_t u, int valid) {
 // 64x64 quadrant) or 64 (each a 32x64 quadrant) for outputs too small to fill the chip with
 // 128-row tiles.  part == null: the tile goes to C (+= when accumulate); otherwise the whole
 // [BM][BN] partial tile is parked at `part`.  `smem`: 2 * (BK * (BM + 4) + B_STAGE) floats.
-template <bool TRANS_A, int BM>
+template <bool TRANS_A, int BM, bool INTERIOR = false>
 __device__ __forceinline__ void gemm_tile(int M, int N, int K,
                                           const float* __restrict__ A, int lda,
                                           const float* __restrict__ B, int ldb,
@@ -109,20 +109,47 @@ __device__ __forceinline__ void gemm_tile(int M, int N, int K,
               : make_panel(A + (size_t)m0 * lda, (long long)(rows_here - 1) * lda + K);
   const __amdgpu_buffer_rsrc_t b_panel = make_panel(B + n0, (long long)(K - 1) * ldb + cols_here);
 
+  // INTERIOR (every tile whole, K and the K pieces multiples of BK): a thread's offsets into
+  // the panels are fixed and the step enters as the instruction's scalar offset, so that a
+  // step's loads cost no vector instruction besides themselves (everything the vector units
+  // do in this loop is time the matrix units stand still).
+  unsigned int a_voff[A_PASSES], b_voff[2];
+#pragma unroll
+  for (int i = 0; i < A_PASSES; ++i)
+    a_voff[i] = TRANS_A ? (unsigned int)((((tid / TA_COLS) + TA_ROWS * i) * lda + (tid % TA_COLS) * 4) * 4)
+                        : (unsigned int)((((tid >> 2) + 64 * i) * lda + (tid & 3) * 4) * 4);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) b_voff[i] = (unsigned int)((((tid >> 5) + 8 * i) * ldb + (tid & 31) * 4) * 4);
+
   auto load_global = [&](int kk) {
+    if constexpr (INTERIOR) {
+      const int a_soff = TRANS_A ? kk * lda * 4 : kk * 4;
+      const int b_soff = kk * ldb * 4;
+#pragma unroll
+      for (int i = 0; i < A_PASSES; ++i) {
+        a_valid[i] = 4;
+        a_raw[i] = __builtin_amdgcn_raw_buffer_load_b128(a_panel, a_voff[i], a_soff, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        b_valid[i] = 4;
+        b_raw[i] = __builtin_amdgcn_raw_buffer_load_b128(b_panel, b_voff[i], b_soff, 0);
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < A_PASSES; ++i) {
       if (TRANS_A) {
         const int ak = (tid / TA_COLS) + TA_ROWS * i;
         const int am = (tid % TA_COLS) * 4;
         const int k = kk + ak;
-        a_valid[i] = (k < k_end) ? (rows_here - am) : 0;
+        a_valid[i] = INTERIOR ? 4 : ((k < k_end) ? (rows_here - am) : 0);
         a_raw[i] = load4_raw(a_panel, (long long)k * lda + am, a_valid[i]);
       } else {
         const int arow = (tid >> 2) + 64 * i;
         const int ak = (tid & 3) * 4;
         const int k = kk + ak;
-        a_valid[i] = (arow < rows_here) ? (k_end - k) : 0;
+        a_valid[i] = INTERIOR ? 4 : ((arow < rows_here) ? (k_end - k) : 0);
         a_raw[i] = load4_raw(a_panel, (long long)arow * lda + k, a_valid[i]);
       }
     }
@@ -131,7 +158,7 @@ __device__ __forceinline__ void gemm_tile(int M, int N, int K,
       const int bk = (tid >> 5) + 8 * i;
       const int bn = (tid & 31) * 4;
       const int k = kk + bk;
-      b_valid[i] = (k < k_end) ? (cols_here - bn) : 0;
+      b_valid[i] = INTERIOR ? 4 : ((k < k_end) ? (cols_here - bn) : 0);
       b_raw[i] = load4_raw(b_panel, (long long)k * ldb + bn, b_valid[i]);
     }
   };
@@ -247,7 +274,7 @@ __device__ __forceinline__ void gemm_tile(int M, int N, int K,
     }
 }
 
-template <bool TRANS_A, int BM>
+template <bool TRANS_A, int BM, bool INTERIOR = false>
 __global__ __launch_bounds__(256, 2)
 void gemm_f32_kernel(int M, int N, int K,
                      const float* __restrict__ A, int lda,
@@ -277,7 +304,7 @@ void gemm_f32_kernel(int M, int N, int K,
     k_end = (k_begin + k_per_split < K) ? (k_begin + k_per_split) : K;
     part = partial + (size_t)j * BM * BN;
   }
-  gemm_tile<TRANS_A, BM>(M, N, K, A, lda, B, ldb, C, ldc, accumulate, tile / tiles_n, tile % tiles_n,
+  gemm_tile<TRANS_A, BM, INTERIOR>(M, N, K, A, lda, B, ldb, C, ldc, accumulate, tile / tiles_n, tile % tiles_n,
                          k_begin, k_end, part, smem);
 }
 
@@ -294,7 +321,7 @@ struct GemmPair {
   float* partial;
 };
 
-template <int BM>
+template <int BM, bool INTERIOR>
 __global__ __launch_bounds__(256, 2)
 void gemm_f32_pair_kernel(GemmPair p) {
   __shared__ __attribute__((aligned(16))) float smem[2 * BK * (BM + 4) + 2 * B_STAGE];
@@ -305,11 +332,11 @@ void gemm_f32_pair_kernel(GemmPair p) {
   float* part = p.splits > 1 ? p.partial + (size_t)j * BM * BN : nullptr;
   const int tm = tile / p.tiles_n, tn = tile % p.tiles_n;
   if (tm < p.tiles_m1)
-    gemm_tile<false, BM>(p.M1, p.N, p.K, p.A1, p.lda1, p.B1, p.ldb1, p.C1, p.ldc1, p.accumulate, tm, tn,
-                         k_begin, k_end, part, smem);
+    gemm_tile<false, BM, INTERIOR>(p.M1, p.N, p.K, p.A1, p.lda1, p.B1, p.ldb1, p.C1, p.ldc1, p.accumulate,
+                                   tm, tn, k_begin, k_end, part, smem);
   else
-    gemm_tile<true, BM>(p.M2, p.N, p.K, p.A2, p.lda2, p.B2, p.ldb2, p.C2, p.ldc2, p.accumulate,
-                        tm - p.tiles_m1, tn, k_begin, k_end, part, smem);
+    gemm_tile<true, BM, INTERIOR>(p.M2, p.N, p.K, p.A2, p.lda2, p.B2, p.ldb2, p.C2, p.ldc2, p.accumulate,
+                                  tm - p.tiles_m1, tn, k_begin, k_end, part, smem);
 }
 
 // For the split tiles (tile index whole_tiles + blockIdx.x): C tile (+)= sum over its
@@ -467,13 +494,16 @@ int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
   HASTE_HIP_REQUIRE(((long long)K * ldb + BN) * 4 < (1ll << 31));
   dim3 grid((unsigned)(whole_tiles + pieces)), block(256);
   ScopedKernelTimer timer("gemm_f32", stream);
-#define HASTE_GEMM_LAUNCH(TA_, BM_)                                                          \
-  if (trans_a == TA_ && bm == BM_)                                                           \
-    gemm_f32_kernel<TA_, BM_><<<grid, block, 0, stream>>>(                                   \
+  const bool interior = M % bm == 0 && N % BN == 0 && K % BK == 0 && k_per_split % BK == 0;
+#define HASTE_GEMM_LAUNCH(TA_, BM_, IN_)                                                     \
+  if (trans_a == TA_ && bm == BM_ && interior == IN_)                                        \
+    gemm_f32_kernel<TA_, BM_, IN_><<<grid, block, 0, stream>>>(                              \
         M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, tiles_n, whole_tiles, splits,   \
         k_per_split, partial);
-  HASTE_GEMM_LAUNCH(false, 128) HASTE_GEMM_LAUNCH(false, 64)
-  HASTE_GEMM_LAUNCH(true, 128) HASTE_GEMM_LAUNCH(true, 64)
+  HASTE_GEMM_LAUNCH(false, 128, false) HASTE_GEMM_LAUNCH(false, 64, false)
+  HASTE_GEMM_LAUNCH(true, 128, false) HASTE_GEMM_LAUNCH(true, 64, false)
+  HASTE_GEMM_LAUNCH(false, 128, true) HASTE_GEMM_LAUNCH(false, 64, true)
+  HASTE_GEMM_LAUNCH(true, 128, true) HASTE_GEMM_LAUNCH(true, 64, true)
 #undef HASTE_GEMM_LAUNCH
   HASTE_HIP_TRY(hipGetLastError());
   if (split) {
@@ -540,7 +570,10 @@ int gemm_f32_pair(hipStream_t stream, int M1, int M2, int N, int K, const float*
     p.partial = ws.scratch;
   }
   ScopedKernelTimer timer("gemm_f32", stream, 2);
-  gemm_f32_pair_kernel<128><<<dim3((unsigned)(tiles * splits)), dim3(256), 0, stream>>>(p);
+  if (M1 % 128 == 0 && M2 % 128 == 0 && N % BN == 0 && K % BK == 0 && k_per_split % BK == 0)
+    gemm_f32_pair_kernel<128, true><<<dim3((unsigned)(tiles * splits)), dim3(256), 0, stream>>>(p);
+  else
+    gemm_f32_pair_kernel<128, false><<<dim3((unsigned)(tiles * splits)), dim3(256), 0, stream>>>(p);
   HASTE_HIP_TRY(hipGetLastError());
   if (splits > 1) {
     const int vec = (ldc1 % 4 == 0) && (ldc2 % 4 == 0) && aligned16(C1) && aligned16(C2);
