@@ -604,12 +604,14 @@ int gemm_f32_pieces(hipStream_t stream, int M, int N, int K, const float* A, int
   float* part = ws.scratch + scratch_offset / sizeof(float);
   dim3 grid((unsigned)g.pieces), block(256);
   ScopedKernelTimer timer("gemm_f32", stream);
-  if (g.bm == 128)
-    gemm_f32_kernel<false, 128><<<grid, block, 0, stream>>>(M, N, K, A, lda, B, ldb, nullptr, 0, 0, g.tiles_n,
-                                                            0, g.splits, g.k_per_split, part);
-  else
-    gemm_f32_kernel<false, 64><<<grid, block, 0, stream>>>(M, N, K, A, lda, B, ldb, nullptr, 0, 0, g.tiles_n,
-                                                           0, g.splits, g.k_per_split, part);
+  const bool interior = M % g.bm == 0 && N % BN == 0 && K % BK == 0 && g.k_per_split % BK == 0;
+#define HASTE_GEMM_LAUNCH(BM_, IN_)                                                          \
+  if (g.bm == BM_ && interior == IN_)                                                        \
+    gemm_f32_kernel<false, BM_, IN_><<<grid, block, 0, stream>>>(                            \
+        M, N, K, A, lda, B, ldb, nullptr, 0, 0, g.tiles_n, 0, g.splits, g.k_per_split, part);
+  HASTE_GEMM_LAUNCH(128, false) HASTE_GEMM_LAUNCH(64, false)
+  HASTE_GEMM_LAUNCH(128, true) HASTE_GEMM_LAUNCH(64, true)
+#undef HASTE_GEMM_LAUNCH
   HASTE_HIP_TRY(hipGetLastError());
   *partial = part;
   *splits = g.splits;
