@@ -274,7 +274,23 @@ __device__ __forceinline__ void gemm_tile(int M, int N, int K,
     }
 }
 
-template <bool TRANS_A, int BM, bool INTERIOR = false>
+// Runs one tile (or K piece of a tile) with the loop that fits it: whole tiles whose K range
+// is a multiple of BK need no masks (gemm_tile's INTERIOR), the tiles on the edges of a ragged
+// problem do.
+template <bool TRANS_A, int BM>
+__device__ __forceinline__ void gemm_any_tile(int M, int N, int K, const float* __restrict__ A, int lda,
+                                              const float* __restrict__ B, int ldb,
+                                              float* __restrict__ C, int ldc, int accumulate,
+                                              int tm, int tn, int k_begin, int k_end,
+                                              float* __restrict__ part, float* smem) {
+  const bool whole = M - tm * BM >= BM && N - tn * BN >= BN && (k_end - k_begin) % BK == 0;
+  if (whole)
+    gemm_tile<TRANS_A, BM, true>(M, N, K, A, lda, B, ldb, C, ldc, accumulate, tm, tn, k_begin, k_end, part, smem);
+  else
+    gemm_tile<TRANS_A, BM, false>(M, N, K, A, lda, B, ldb, C, ldc, accumulate, tm, tn, k_begin, k_end, part, smem);
+}
+
+template <bool TRANS_A, int BM>
 __global__ __launch_bounds__(256, 2)
 void gemm_f32_kernel(int M, int N, int K,
                      const float* __restrict__ A, int lda,
@@ -304,8 +320,8 @@ void gemm_f32_kernel(int M, int N, int K,
     k_end = (k_begin + k_per_split < K) ? (k_begin + k_per_split) : K;
     part = partial + (size_t)j * BM * BN;
   }
-  gemm_tile<TRANS_A, BM, INTERIOR>(M, N, K, A, lda, B, ldb, C, ldc, accumulate, tile / tiles_n, tile % tiles_n,
-                         k_begin, k_end, part, smem);
+  gemm_any_tile<TRANS_A, BM>(M, N, K, A, lda, B, ldb, C, ldc, accumulate, tile / tiles_n, tile % tiles_n,
+                             k_begin, k_end, part, smem);
 }
 
 // Two products with the same N and K in one launch (dW = x^T dv and dR = h^T dv of a backward
@@ -321,7 +337,7 @@ struct GemmPair {
   float* partial;
 };
 
-template <int BM, bool INTERIOR>
+template <int BM>
 __global__ __launch_bounds__(256, 2)
 void gemm_f32_pair_kernel(GemmPair p) {
   __shared__ __attribute__((aligned(16))) float smem[2 * BK * (BM + 4) + 2 * B_STAGE];
@@ -332,11 +348,11 @@ void gemm_f32_pair_kernel(GemmPair p) {
   float* part = p.splits > 1 ? p.partial + (size_t)j * BM * BN : nullptr;
   const int tm = tile / p.tiles_n, tn = tile % p.tiles_n;
   if (tm < p.tiles_m1)
-    gemm_tile<false, BM, INTERIOR>(p.M1, p.N, p.K, p.A1, p.lda1, p.B1, p.ldb1, p.C1, p.ldc1, p.accumulate,
-                                   tm, tn, k_begin, k_end, part, smem);
+    gemm_any_tile<false, BM>(p.M1, p.N, p.K, p.A1, p.lda1, p.B1, p.ldb1, p.C1, p.ldc1, p.accumulate,
+                             tm, tn, k_begin, k_end, part, smem);
   else
-    gemm_tile<true, BM, INTERIOR>(p.M2, p.N, p.K, p.A2, p.lda2, p.B2, p.ldb2, p.C2, p.ldc2, p.accumulate,
-                                  tm - p.tiles_m1, tn, k_begin, k_end, part, smem);
+    gemm_any_tile<true, BM>(p.M2, p.N, p.K, p.A2, p.lda2, p.B2, p.ldb2, p.C2, p.ldc2, p.accumulate,
+                            tm - p.tiles_m1, tn, k_begin, k_end, part, smem);
 }
 
 // For the split tiles (tile index whole_tiles + blockIdx.x): C tile (+)= sum over its
@@ -494,16 +510,13 @@ int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
   HASTE_HIP_REQUIRE(((long long)K * ldb + BN) * 4 < (1ll << 31));
   dim3 grid((unsigned)(whole_tiles + pieces)), block(256);
   ScopedKernelTimer timer("gemm_f32", stream);
-  const bool interior = M % bm == 0 && N % BN == 0 && K % BK == 0 && k_per_split % BK == 0;
-#define HASTE_GEMM_LAUNCH(TA_, BM_, IN_)                                                     \
-  if (trans_a == TA_ && bm == BM_ && interior == IN_)                                        \
-    gemm_f32_kernel<TA_, BM_, IN_><<<grid, block, 0, stream>>>(                              \
+#define HASTE_GEMM_LAUNCH(TA_, BM_)                                                          \
+  if (trans_a == TA_ && bm == BM_)                                                           \
+    gemm_f32_kernel<TA_, BM_><<<grid, block, 0, stream>>>(                                   \
         M, N, K, A, lda, B, ldb, C, ldc, accumulate ? 1 : 0, tiles_n, whole_tiles, splits,   \
         k_per_split, partial);
-  HASTE_GEMM_LAUNCH(false, 128, false) HASTE_GEMM_LAUNCH(false, 64, false)
-  HASTE_GEMM_LAUNCH(true, 128, false) HASTE_GEMM_LAUNCH(true, 64, false)
-  HASTE_GEMM_LAUNCH(false, 128, true) HASTE_GEMM_LAUNCH(false, 64, true)
-  HASTE_GEMM_LAUNCH(true, 128, true) HASTE_GEMM_LAUNCH(true, 64, true)
+  HASTE_GEMM_LAUNCH(false, 128) HASTE_GEMM_LAUNCH(false, 64)
+  HASTE_GEMM_LAUNCH(true, 128) HASTE_GEMM_LAUNCH(true, 64)
 #undef HASTE_GEMM_LAUNCH
   HASTE_HIP_TRY(hipGetLastError());
   if (split) {
@@ -570,10 +583,7 @@ int gemm_f32_pair(hipStream_t stream, int M1, int M2, int N, int K, const float*
     p.partial = ws.scratch;
   }
   ScopedKernelTimer timer("gemm_f32", stream, 2);
-  if (M1 % 128 == 0 && M2 % 128 == 0 && N % BN == 0 && K % BK == 0 && k_per_split % BK == 0)
-    gemm_f32_pair_kernel<128, true><<<dim3((unsigned)(tiles * splits)), dim3(256), 0, stream>>>(p);
-  else
-    gemm_f32_pair_kernel<128, false><<<dim3((unsigned)(tiles * splits)), dim3(256), 0, stream>>>(p);
+  gemm_f32_pair_kernel<128><<<dim3((unsigned)(tiles * splits)), dim3(256), 0, stream>>>(p);
   HASTE_HIP_TRY(hipGetLastError());
   if (splits > 1) {
     const int vec = (ldc1 % 4 == 0) && (ldc2 % 4 == 0) && aligned16(C1) && aligned16(C2);
@@ -604,14 +614,12 @@ int gemm_f32_pieces(hipStream_t stream, int M, int N, int K, const float* A, int
   float* part = ws.scratch + scratch_offset / sizeof(float);
   dim3 grid((unsigned)g.pieces), block(256);
   ScopedKernelTimer timer("gemm_f32", stream);
-  const bool interior = M % g.bm == 0 && N % BN == 0 && K % BK == 0 && g.k_per_split % BK == 0;
-#define HASTE_GEMM_LAUNCH(BM_, IN_)                                                          \
-  if (g.bm == BM_ && interior == IN_)                                                        \
-    gemm_f32_kernel<false, BM_, IN_><<<grid, block, 0, stream>>>(                            \
-        M, N, K, A, lda, B, ldb, nullptr, 0, 0, g.tiles_n, 0, g.splits, g.k_per_split, part);
-  HASTE_GEMM_LAUNCH(128, false) HASTE_GEMM_LAUNCH(64, false)
-  HASTE_GEMM_LAUNCH(128, true) HASTE_GEMM_LAUNCH(64, true)
-#undef HASTE_GEMM_LAUNCH
+  if (g.bm == 128)
+    gemm_f32_kernel<false, 128><<<grid, block, 0, stream>>>(M, N, K, A, lda, B, ldb, nullptr, 0, 0, g.tiles_n,
+                                                            0, g.splits, g.k_per_split, part);
+  else
+    gemm_f32_kernel<false, 64><<<grid, block, 0, stream>>>(M, N, K, A, lda, B, ldb, nullptr, 0, 0, g.tiles_n,
+                                                           0, g.splits, g.k_per_split, part);
   HASTE_HIP_TRY(hipGetLastError());
   *partial = part;
   *splits = g.splits;
