@@ -24,7 +24,7 @@ PEAK_HBM_GBS = 8000.0
 # one FETCH_SIZE unit = 2.000 KiB, one WRITE_SIZE unit = 1.000 KiB.  A GEMM "launch" is the mean
 # of the step's four products (dW and dR share a launch that counts as two), each with its
 # split reduce.
-MEASURED_TRAFFIC_BYTES = {"gemm_f32": 180.0e6, "lstm_forward_recurrence": 166.8e6,
+MEASURED_TRAFFIC_BYTES = {"gemm_f32": 180.2e6, "lstm_forward_recurrence": 166.8e6,
                           "lstm_backward_recurrence": 183.0e6,
                           # at N=1 C=512 H=4096 (--workload stepwise): 131558.5 FETCH_SIZE units
                           # + 192 WRITE_SIZE units per launch of the streaming kernel
