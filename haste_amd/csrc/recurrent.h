@@ -808,7 +808,11 @@ __device__ __forceinline__ void tile_product(const TileBuffer& xb, int tile_off,
   } else {
     static_assert(!TAGGED, "polled partial tiles exist for short tiles only");
     constexpr int RT = NB / 16;
-    constexpr int CHUNK = LONG_K ? (RT == 1 ? 8 : (RT == 2 ? 4 : 2)) : (RT >= 4 ? 2 : 4);
+    // k-groups of operands per load (two loads in flight).  Measured at H = 512: a forward share
+    // (8 groups per wavefront) in one piece, a backward share (32 groups) in two, are 9-10 %
+    // faster per step than pieces of 4 / 8 at 16 rows, pieces of 8 than 4 at 32 rows; twice
+    // that is slower again.
+    constexpr int CHUNK = LONG_K ? (RT == 1 ? 16 : (RT == 2 ? 8 : 2)) : (RT >= 4 ? 2 : 8);
     tall_tile_product<RT, CT, CHUNK, POLLED>(xb, tile_off, Kpad, w_lds, red, gs);
   }
 }
