@@ -580,18 +580,14 @@ __device__ __forceinline__ void load_tile_chunk(const TileBuffer& xb, int tile_o
                                                 int g_end, float4_t (&av)[CHUNK][RT]) {
   constexpr int NB = 16 * RT;
   const int lane = threadIdx.x & 63;
-  const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
-  const int base = tile_off + ((lane >> 4) * NB + (lane & 15)) * 4;
+  // Every caller stays inside its wavefront's share (g_abs + CHUNK <= g_end), so the loads
+  // carry no conditions: selects among the MFMAs would be time the matrix unit stands still.
+  (void)g_end;
+  const int base = tile_off + ((lane >> 4) * NB + (lane & 15)) * 4 + g_abs * 16 * NB;
 #pragma unroll
-  for (int gi = 0; gi < CHUNK; ++gi) {
-    const bool ok = g_abs + gi < g_end;
-    const int g = ok ? g_abs + gi : g_abs;
+  for (int gi = 0; gi < CHUNK; ++gi)
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      const float4_t v = load_tile4(xb, base + (g * 4 * NB + rt * 16) * 4);
-      av[gi][rt] = ok ? v : zero4;
-    }
-  }
+    for (int rt = 0; rt < RT; ++rt) av[gi][rt] = load_tile4(xb, base + (gi * 4 * NB + rt * 16) * 4);
 }
 
 template <int RT, int CT, int CHUNK, bool POLLED>
