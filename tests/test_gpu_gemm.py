@@ -20,6 +20,10 @@ SHAPES = [
     (False, 100, 768, 3072),
     (False, 1, 2048, 512), (False, 16, 6144, 1536), (False, 5, 1300, 5200), (False, 32, 768, 3072),
     (False, 17, 4100, 332), (False, 3, 64, 1024), (False, 32, 16384, 1000),
+    # whole tiles beside edge tiles, K pieces that are and are not multiples of 16: the unmasked
+    # and the masked loop in one launch
+    (False, 300, 260, 250), (True, 384, 1000, 1600), (False, 640, 192, 2048), (True, 800, 512, 1000),
+    (False, 1024, 1024, 17),
 ]
 
 
@@ -41,6 +45,25 @@ def test_gemm_matches_numpy(trans_a, M, N, K, accumulate):
     if accumulate:
         ref = ref + c0
     assert relerr(host(out), ref) < 1e-5  # fp32 accumulation over K up to 6400
+
+
+@pytest.mark.parametrize("trans_a,M,N,K,pad_a,pad_b", [(False, 256, 256, 128, 4, 4), (True, 384, 128, 96, 3, 1),
+                                                        (False, 130, 100, 64, 3, 4), (True, 128, 256, 2048, 4, 0)])
+def test_gemm_padded_leading_dimensions(trans_a, M, N, K, pad_a, pad_b):
+    """Operands that are column ranges of wider arrays (lda > K, ldb > N), aligned and not."""
+    import torch
+    from haste_amd import lib as hlib
+    g = torch.Generator().manual_seed(M + N + K)
+    a_full = torch.randn((K, M + pad_a) if trans_a else (M, K + pad_a), generator=g).cuda()
+    b_full = torch.randn(K, N + pad_b, generator=g).cuda()
+    a = a_full[:, :M] if trans_a else a_full[:, :K]
+    out = torch.zeros(M, N, device="cuda")
+    print("gemm padded", trans_a, M, N, K, pad_a, pad_b, flush=True)
+    hlib.call("haste_hip_gemm_f32", int(trans_a), M, N, K, a_full, a_full.stride(0), b_full, b_full.stride(0),
+              out, out.stride(0), 0)
+    torch.cuda.synchronize()
+    ref = (a.double().t() if trans_a else a.double()) @ b_full[:, :N].double()
+    assert relerr(host(out), host(ref)) < 1e-5
 
 
 def test_gemm_split_k_is_run_to_run_identical():
