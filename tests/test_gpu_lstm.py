@@ -57,8 +57,9 @@ def test_lstm_training_forward_backward(T, N, C, H, zoneout):
 
 
 @pytest.mark.parametrize("zoneout", [0.0, 0.25])
-def test_lstm_inference_forward(zoneout):
-    T, N, C, H = 20, 16, 128, 256
+@pytest.mark.parametrize("T,N,C,H", [(20, 16, 128, 256), (12, 1, 32, 512), (9, 1, 8, 130), (8, 50, 16, 512)])
+def test_lstm_inference_forward(zoneout, T, N, C, H):
+    """Inference (zoneout as the convex blend) through the tile, single-row and two-set kernels."""
     p = problem(7, T, N, C, H, 4, zoneout)
     h, c, _, _ = run_lstm(p, False, zoneout, T, N, C, H)
     ho, co, _ = O.lstm_forward(p["W"], p["R"], p["b"], p["x"], p["h0"], p["c0"], False, zoneout, p["mask"])
@@ -66,10 +67,11 @@ def test_lstm_inference_forward(zoneout):
     assert relerr(host(c), co) < TOL
 
 
-def test_lstm_dropconnect_fused_equals_premasked_weights():
+@pytest.mark.parametrize("T,N,C,H", [(6, 8, 16, 64), (5, 48, 16, 128), (6, 1, 16, 200)])
+def test_lstm_dropconnect_fused_equals_premasked_weights(T, N, C, H):
+    """Bit for bit, in the 4-row tile kernel, the two-set kernel and the single-row kernel."""
     from haste_amd import ops
     import torch
-    T, N, C, H = 6, 8, 16, 64
     p = problem(9, T, N, C, H, 4)
     r = np.random.default_rng(3)
     m = (r.uniform(size=p["R"].shape) >= 0.05).astype(np.float64)
