@@ -44,10 +44,11 @@ def test_gru_training_forward_backward(T, N, C, H, zoneout):
 
 
 @pytest.mark.parametrize("zoneout", [0.0, 0.25])
-def test_gru_inference_forward(zoneout):
+@pytest.mark.parametrize("T,N,C,H", [(20, 16, 128, 256), (8, 50, 16, 512)])
+def test_gru_inference_forward(zoneout, T, N, C, H):
+    """Inference (zoneout as the convex blend) through the tile and the two-set kernels."""
     from haste_amd import ops
     import torch
-    T, N, C, H = 20, 16, 128, 256
     p = problem(8, T, N, C, H, 3, zoneout)
     h, _ = ops.gru_forward(False, zoneout, dev(p["x"]), dev(p["h0"]), dev(p["W"]), dev(p["R"]),
                            dev(p["b"]), dev(p["b2"]), dev(p["mask"]))
@@ -56,10 +57,11 @@ def test_gru_inference_forward(zoneout):
     assert relerr(host(h), ho) < TOL
 
 
-def test_gru_dropconnect_fused_equals_premasked_weights():
+@pytest.mark.parametrize("T,N,C,H", [(6, 8, 16, 64), (5, 48, 16, 128)])
+def test_gru_dropconnect_fused_equals_premasked_weights(T, N, C, H):
+    """Bit for bit, in the 4-row tile kernel and the two-set kernel."""
     from haste_amd import ops
     import torch
-    T, N, C, H = 6, 8, 16, 64
     p = problem(9, T, N, C, H, 3)
     m = (np.random.default_rng(3).uniform(size=p["R"].shape) >= 0.05).astype(np.float64)
     scale = 1.0 / 0.95
