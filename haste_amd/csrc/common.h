@@ -94,9 +94,9 @@ bool xcd_local_enabled();
 // batch tiles then run as one tile instead of two sets of half the rows (for experiments).
 bool paired_sets_enabled();
 
-// False when the environment variable HASTE_HIP_SINGLE_ROW is set to 0: an LSTM forward pass
-// with one batch row then runs as a 4-row tile instead of the kernel that keeps the recurrent
-// weights in registers (for experiments).
+// False when the environment variable HASTE_HIP_SINGLE_ROW is set to 0: an LSTM or GRU forward
+// pass with one batch row then runs as a 4-row tile instead of the kernel that keeps the
+// recurrent weights in registers (for experiments).
 bool single_row_enabled();
 
 // C[M,N] = op(A)*B (+C): fp32 MFMA GEMM on `stream`.  The partial tiles of a split product

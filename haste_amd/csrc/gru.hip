@@ -215,6 +215,128 @@ void gru_forward_kernel(GruFwdParams p) {
   }
 }
 
+// The forward pass of a single batch row (see "one batch row" in recurrent.h): 16 hidden units
+// x 3 gates per workgroup (the fourth 16 columns of the 64 are idle), the recurrent weights in
+// registers.
+template <int KW_MAX>
+__global__ __launch_bounds__(256, 1)
+void gru_forward_single_row_kernel(GruFwdParams p) {
+  constexpr int HS = kSingleRowUnits, NCOLS = kSingleRowCols;
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  float (*h_lds)[KW_MAX] = reinterpret_cast<float (*)[KW_MAX]>(lds);
+  float (*red)[4][NCOLS] = reinterpret_cast<float (*)[4][NCOLS]>(lds + 4 * KW_MAX);
+  const int H = p.H, T = p.T;
+  const int Kpad = round_up(H, 64);
+  const int KW = Kpad / 4;  // multiple of 16
+  const Role role = take_role(p.ls, reinterpret_cast<unsigned int*>(lds + 4 * KW_MAX + 2 * 4 * NCOLS));
+  if (!role.active) return;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int j0 = role.cw * HS;
+  float* xh = p.xh;  // one batch tile: [4 polled tiles][Kpad]
+  const TileBuffer xhb = make_tile_buffer(xh, kPolledTiles * Kpad);
+
+  GroupSync gs;
+  group_sync_init(gs, p.ls, role);
+  // Own k range of the exchange tiles (the last workgroup also owns the padding).
+  zero_tile_share(gs, xh, Kpad, 1, j0 / 4, (role.cw == p.ls.gx - 1 ? Kpad - j0 : HS) / 4, kPolledTiles);
+
+  float w[KW_MAX];
+  single_row_weights<KW_MAX>(w, p.R, p.dc_mask, p.dc_scale, KW, H, 3 * H, (lane / HS) * H + j0 + lane % HS,
+                             lane / HS < 3 && j0 + lane % HS < H);
+  for (int i = tid; i < 4 * KW_MAX; i += 256) (&h_lds[0][0])[i] = 0.f;  // ordered by group_arrive's barrier
+
+  // Pointwise ownership: thread u < 16 handles hidden unit j0 + u.
+  const int pj = j0 + tid;
+  const bool act = tid < HS && pj < H;
+  float h_prev = 0.f, bxv[3] = {0.f, 0.f, 0.f}, brv[3] = {0.f, 0.f, 0.f};
+  if (act) {
+    h_prev = p.h[pj];
+#pragma unroll
+    for (int g = 0; g < 3; ++g) {
+      bxv[g] = p.bx[g * H + pj];
+      brv[g] = p.br[g * H + pj];
+    }
+  }
+  const bool zoneout = p.zoneout_prob != 0.f && p.zoneout_mask != nullptr;
+  // Tile 0 receives h[0]; the elements of the other tiles that steps will publish start out
+  // unwritten.  One real barrier: nobody polls a tile before all of its owners have set it up.
+  if (act) {
+    store_exchanged(gs, &xh[pj], publishable(h_prev));
+    for (int b = 1; b < kPolledTiles; ++b) store_exchanged(gs, &xh[b * Kpad + pj], unwritten_value());
+  }
+  group_arrive(gs);
+  group_wait(gs);
+
+  float wx_next[3], mk_next;
+  auto fetch = [&](int t) {
+    mk_next = 1.f;
+#pragma unroll
+    for (int g = 0; g < 3; ++g) wx_next[g] = 0.f;
+    if (act && t < T) {
+      const float* wt = p.Wx + (size_t)t * 3 * H + pj;
+#pragma unroll
+      for (int g = 0; g < 3; ++g) wx_next[g] = wt[g * H];
+      if (zoneout && p.training) mk_next = p.zoneout_mask[(size_t)t * H + pj];
+    }
+  };
+  fetch(0);
+
+  for (int t = 0; t < T; ++t) {
+    float wx[3];
+    const float mk = mk_next;
+#pragma unroll
+    for (int g = 0; g < 3; ++g) wx[g] = wx_next[g];
+
+    // The wavefront's share of h[t] (polled tile t % 4) against the thread's weights.
+    red[t & 1][wave][lane] =
+        single_row_product<KW_MAX>(gs, xhb, (t & 3) * Kpad + wave * KW, KW, h_lds[wave], w);
+    __syncthreads();
+
+    float saved[4] = {0.f, 0.f, 0.f, 0.f};  // z, r, g, q of the step for the caller's cache
+    if (act) {
+      float rh[3];
+#pragma unroll
+      for (int g = 0; g < 3; ++g) {
+        const float* r = &red[t & 1][0][g * HS + tid];
+        rh[g] = (r[0] + r[NCOLS]) + (r[2 * NCOLS] + r[3 * NCOLS]);
+      }
+      const float z = sigmoid_f(wx[0] + rh[0] + bxv[0] + brv[0]);
+      const float r = sigmoid_f(wx[1] + rh[1] + bxv[1] + brv[1]);
+      const float qg = rh[2] + brv[2];
+      const float g = tanh_f(wx[2] + r * qg + bxv[2]);
+      saved[0] = z;
+      saved[1] = r;
+      saved[2] = g;
+      saved[3] = qg;
+      float h_new = z * h_prev + (1.0f - z) * g;
+      if (zoneout) {
+        if (p.training) h_new = (h_new - h_prev) * mk + h_prev;
+        else h_new = p.zoneout_prob * h_prev + (1.0f - p.zoneout_prob) * h_new;
+      }
+      h_prev = h_new;
+    }
+    // Everything this wavefront stored during the previous step (its resets among it) has
+    // landed before h[t+1] becomes visible.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (act && t + 1 < T) {
+      store_exchanged(gs, &xh[((t + 1) & 3) * Kpad + pj], publishable(h_prev));
+      // the tile read at step t-1: nobody needs it any more
+      if (t + 3 < T) store_exchanged(gs, &xh[((t + 3) & 3) * Kpad + pj], unwritten_value());
+    }
+    fetch(t + 1);
+    // The caller's copies are written last: nobody in the launch waits for them.
+    if (act) {
+      if (p.training) {
+        float* vt = p.v + (size_t)t * 4 * H + pj;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) vt[g * H] = saved[g];
+      }
+      p.h_out[(size_t)t * H + pj] = h_prev;
+    }
+  }
+}
+
 struct GruBwdParams {
   int T, N, H;
   const float* R_t;     // [3H,H]
@@ -459,6 +581,33 @@ void gru_backward_kernel(GruBwdParams p) {
 
 }  // namespace
 
+// The forward pass of a single batch row with H <= 512: the recurrent weights live in the
+// registers of the 16-unit workgroups of one XCD (gru_forward_single_row_kernel).
+int gru_forward_single_row(hipStream_t stream, int training, int T, int C, int H, const float* W,
+                           const float* R, const float* bx, const float* br, const float* x,
+                           const float* h, float* h_out, float* v, float* tmp_Wx, float zoneout_prob,
+                           const float* zoneout_mask, const float* dc_mask, float dc_scale) {
+  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T, 3 * H, C, x, C, W, 3 * H, tmp_Wx, 3 * H, false));
+  const int Kpad = (H + 63) / 64 * 64;
+  Workspace ws;
+  HASTE_HIP_PROPAGATE(get_workspace(stream, (size_t)kPolledTiles * Kpad * sizeof(float), &ws));
+  HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
+  GruFwdParams p;
+  p.training = training; p.T = T; p.N = 1; p.H = H;
+  p.R = R; p.bx = bx; p.br = br; p.h = h; p.h_out = h_out; p.v = v; p.Wx = tmp_Wx;
+  p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
+  p.dc_mask = dc_mask; p.dc_scale = dc_scale;
+  p.xh = ws.scratch;
+  LaunchPlan plan;
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, (H + 15) / 16, 1, 1,
+                                  single_row_lds_bytes(single_row_kw_max(Kpad)), (unsigned)T + 1, &plan));
+  p.ls = plan.shape;
+  const char* name = "gru_forward_recurrence";
+  if (Kpad <= 128) return launch_persistent(name, gru_forward_single_row_kernel<32>, plan, p, stream);
+  if (Kpad <= 256) return launch_persistent(name, gru_forward_single_row_kernel<64>, plan, p, stream);
+  return launch_persistent(name, gru_forward_single_row_kernel<128>, plan, p, stream);
+}
+
 // h: [N,H] state before the first step; h_out: [T,N,H] states after each step.
 int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int H,
                      const float* W, const float* R, const float* bx, const float* br,
@@ -468,6 +617,9 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
   HASTE_HIP_REQUIRE(W && R && bx && br && x && h && h_out && tmp_Wx);
   HASTE_HIP_REQUIRE(!training || v != nullptr);
+  if (N == 1 && H <= 512 && xcd_local_fits((H + 15) / 16, 1) && single_row_enabled())
+    return gru_forward_single_row(stream, training, T, C, H, W, R, bx, br, x, h, h_out, v, tmp_Wx,
+                                  zoneout_prob, zoneout_mask, dc_mask, dc_scale);
   const ForwardTile tile = pick_forward_tile(3, N, H, 0, kWorkgroupLdsBytes);
   // No slice of R fits a CU: stream R from HBM every step instead.
   if (!tile.ok)

@@ -218,21 +218,12 @@ void lstm_forward_kernel(LstmFwdParams p) {
   }
 }
 
-// ---- batch of one -----------------------------------------------------------------------
-// With a single batch row the step's product is a matrix-vector product.  The 4-row MFMA tile
-// spends three quarters of the matrix unit's time on padding and, like any tile, reads the
-// whole slice from LDS every step (128 KiB at H = 512: 0.45 us at the LDS's rate).  Here the
-// slice lives in REGISTERS: a thread owns one of the 64 slice columns (16 hidden units x 4
-// gates) and a quarter of k, i.e. up to 128 weights, and a step is up to 128 FMAs per thread
-// against h, which the wavefront polls from the exchange tile, parks in LDS and reads back as
-// broadcast 16-byte reads.  KW: the k range of a wavefront (Kpad / 4, at most the template's).
+// The forward pass of a single batch row (see "one batch row" in recurrent.h): 16 hidden units
+// x 4 gates per workgroup, the recurrent weights in registers.
 template <int KW_MAX>
 __global__ __launch_bounds__(256, 1)
 void lstm_forward_single_row_kernel(LstmFwdParams p) {
-  constexpr int HS = 16, NCOLS = 64;
-  // No static LDS (launch_persistent sizes the dynamic limit for kernels without any):
-  // [4][KW_MAX] a wavefront's share of h, [2][4][NCOLS] partial sums by step parity and
-  // wavefront, one word for the role.
+  constexpr int HS = kSingleRowUnits, NCOLS = kSingleRowCols;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   float (*h_lds)[KW_MAX] = reinterpret_cast<float (*)[KW_MAX]>(lds);
   float (*red)[4][NCOLS] = reinterpret_cast<float (*)[4][NCOLS]>(lds + 4 * KW_MAX);
@@ -252,23 +243,9 @@ void lstm_forward_single_row_kernel(LstmFwdParams p) {
   // Own k range of the exchange tiles (the last workgroup also owns the padding).
   zero_tile_share(gs, xh, Kpad, 1, j0 / 4, (role.cw == p.ls.gx - 1 ? Kpad - j0 : HS) / 4, kPolledTiles);
 
-  // The thread's weights: column `lane` (gate lane/16, unit j0 + lane%16), k = wave*KW + i.
   float w[KW_MAX];
-  {
-    const int gate = lane / HS, j = j0 + lane % HS;
-#pragma unroll
-    for (int i = 0; i < KW_MAX; ++i) {
-      const int k = wave * KW + i;
-      float v = 0.f;
-      if (i < KW && k < H && j < H) {
-        const size_t o = (size_t)k * 4 * H + gate * H + j;
-        v = p.R[o];
-        if (p.dc_mask != nullptr) v = v * p.dc_mask[o] * p.dc_scale;
-      }
-      w[i] = v;
-    }
-  }
-
+  single_row_weights<KW_MAX>(w, p.R, p.dc_mask, p.dc_scale, KW, H, 4 * H, (lane / HS) * H + j0 + lane % HS,
+                             j0 + lane % HS < H);
   for (int i = tid; i < 4 * KW_MAX; i += 256) (&h_lds[0][0])[i] = 0.f;  // ordered by group_arrive's barrier
 
   // Pointwise ownership: thread u < 16 handles hidden unit j0 + u.
@@ -311,26 +288,9 @@ void lstm_forward_single_row_kernel(LstmFwdParams p) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) wx[g] = wx_next[g];
 
-    // The wavefront's share of h[t]: lanes 0 .. KW/4-1 poll four k each (polled tile t % 4).
-    const int off = (t & 3) * Kpad + wave * KW + 4 * lane;
-    const bool loads = 4 * lane < KW;
-    float4_t hv[1][1];
-    auto load = [&] { hv[0][0] = loads ? load_tile4(xhb, off) : float4_t{0.f, 0.f, 0.f, 0.f}; };
-    load();
-    poll_until_written(gs, load, [&] { return all_written(hv); });
-    if (loads) *reinterpret_cast<float4_t*>(&h_lds[wave][4 * lane]) = hv[0][0];
-    // LDS operations of a wavefront complete in order: the reads below see the store above.
-    float acc0 = 0.f, acc1 = 0.f;
-    // (k beyond KW: the weights and the parked h are zero, so no step of the loop is conditional)
-#pragma unroll
-    for (int i = 0; i < KW_MAX; i += 4) {
-      const float4_t h4 = *reinterpret_cast<const float4_t*>(&h_lds[wave][i]);
-      acc0 = fmaf(w[i], h4.x, acc0);
-      acc1 = fmaf(w[i + 1], h4.y, acc1);
-      acc0 = fmaf(w[i + 2], h4.z, acc0);
-      acc1 = fmaf(w[i + 3], h4.w, acc1);
-    }
-    red[t & 1][wave][lane] = acc0 + acc1;
+    // The wavefront's share of h[t] (polled tile t % 4) against the thread's weights.
+    red[t & 1][wave][lane] =
+        single_row_product<KW_MAX>(gs, xhb, (t & 3) * Kpad + wave * KW, KW, h_lds[wave], w);
     __syncthreads();
 
     float gate[4] = {0.f, 0.f, 0.f, 0.f};
@@ -638,9 +598,8 @@ int lstm_forward_single_row(hipStream_t stream, int training, int T, int C, int 
   p.dc_mask = dc_mask; p.dc_scale = dc_scale;
   p.xh = ws.scratch;
   LaunchPlan plan;
-  const int kw_max = Kpad <= 128 ? 32 : (Kpad <= 256 ? 64 : 128);
-  const size_t lds_bytes = ((size_t)4 * kw_max + 2 * 4 * 64 + 4) * sizeof(float);
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, (H + 15) / 16, 1, 1, lds_bytes, (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, (H + 15) / 16, 1, 1,
+                                  single_row_lds_bytes(single_row_kw_max(Kpad)), (unsigned)T + 1, &plan));
   p.ls = plan.shape;
   const char* name = "lstm_forward_recurrence";
   if (Kpad <= 128) return launch_persistent(name, lstm_forward_single_row_kernel<32>, plan, p, stream);

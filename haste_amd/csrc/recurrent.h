@@ -927,6 +927,73 @@ __device__ __forceinline__ void reset_partials(float* red, int live) {
     red[i] = (i % P::kRedFloats) / TILE < live ? unwritten_value() : 0.f;
 }
 
+// ---- one batch row -----------------------------------------------------------------------
+// With a single batch row the step's product is a matrix-vector product.  The 4-row MFMA tile
+// spends three quarters of the matrix unit's time on padding and, like any tile, reads the
+// whole slice from LDS every step (128 KiB at H = 512: 0.45 us at the LDS's rate).  The
+// single-row kernels keep the slice in REGISTERS instead: 256 threads, a thread owns one of 64
+// slice columns (16 hidden units x up to 4 gates: column c is gate c/16, unit c%16) and a
+// quarter of k (wavefront w: k in [w*KW, (w+1)*KW), KW = Kpad/4 <= KW_MAX), i.e. up to 128
+// weights, and a step is up to 128 FMAs per thread against h, which the wavefront polls from
+// the exchange tile ([4 polled tiles][Kpad] for the one row), parks in LDS and reads back as
+// broadcast 16-byte reads.
+constexpr int kSingleRowUnits = 16;
+constexpr int kSingleRowCols = 64;
+
+// Dynamic LDS of a single-row kernel: [4][KW_MAX] a wavefront's share of h, [2][4][64]
+// partial sums by step parity and wavefront, one word for the role (no static LDS:
+// launch_persistent sizes the dynamic limit for kernels without any).
+inline size_t single_row_lds_bytes(int kw_max) {
+  return ((size_t)4 * kw_max + 2 * 4 * kSingleRowCols + 4) * sizeof(float);
+}
+inline int single_row_kw_max(int Kpad) { return Kpad <= 128 ? 32 : (Kpad <= 256 ? 64 : 128); }
+
+// The thread's weights: column `lane` of the slice, k = wave*KW + i.  `col` is the column's
+// offset inside a row of `src` (row length `row_len`), valid: the column exists.
+template <int KW_MAX>
+__device__ __forceinline__ void single_row_weights(float (&w)[KW_MAX], const float* __restrict__ src,
+                                                   const float* __restrict__ mask, float scale,
+                                                   int KW, int K, int row_len, int col, bool valid) {
+  const int wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int i = 0; i < KW_MAX; ++i) {
+    const int k = wave * KW + i;
+    float v = 0.f;
+    if (i < KW && k < K && valid) {
+      const size_t o = (size_t)k * row_len + col;
+      v = src[o];
+      if (mask != nullptr) v = v * mask[o] * scale;
+    }
+    w[i] = v;
+  }
+}
+
+// This thread's part of the step's product: its column, its wavefront's quarter of k.  The
+// wavefront's share of the polled tile starts at float `off` of `xb`; h_wave: the wavefront's
+// KW_MAX floats of LDS, zero beyond KW (so no step of the loop is conditional).
+template <int KW_MAX>
+__device__ __forceinline__ float single_row_product(const GroupSync& gs, const TileBuffer& xb, int off,
+                                                    int KW, float* h_wave, const float (&w)[KW_MAX]) {
+  const int lane = threadIdx.x & 63;
+  const bool loads = 4 * lane < KW;  // lanes 0 .. KW/4-1 poll four k each
+  float4_t hv[1][1];
+  auto load = [&] { hv[0][0] = loads ? load_tile4(xb, off + 4 * lane) : float4_t{0.f, 0.f, 0.f, 0.f}; };
+  load();
+  poll_until_written(gs, load, [&] { return all_written(hv); });
+  if (loads) *reinterpret_cast<float4_t*>(&h_wave[4 * lane]) = hv[0][0];
+  // LDS operations of a wavefront complete in order: the reads below see the store above.
+  float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+  for (int i = 0; i < KW_MAX; i += 4) {
+    const float4_t h4 = *reinterpret_cast<const float4_t*>(&h_wave[i]);
+    acc0 = fmaf(w[i], h4.x, acc0);
+    acc1 = fmaf(w[i + 1], h4.y, acc1);
+    acc0 = fmaf(w[i + 2], h4.z, acc0);
+    acc1 = fmaf(w[i + 3], h4.w, acc1);
+  }
+  return acc0 + acc1;
+}
+
 // ---- host side ---------------------------------------------------------------------
 // Partial tiles slice_product leaves in LDS (ProductTile<nb, ct>::kPartials).
 inline int product_partials(int nb, int ct) {

@@ -14,6 +14,8 @@ SHAPES = [(1, 1, 1, 1), (3, 2, 3, 4), (5, 3, 7, 5), (6, 17, 20, 36), (4, 16, 32,
           # hidden sizes that are not multiples of the 16 units of a workgroup
           (7, 41, 24, 512), (5, 57, 16, 200), (4, 36, 8, 72),
           (1, 40, 8, 128), (2, 64, 8, 64), (3, 50, 8, 16),
+          # one batch row: the forward pass keeps the recurrent weights in registers (H <= 512)
+          (9, 1, 7, 100), (6, 1, 16, 512), (5, 1, 8, 300), (4, 1, 8, 48), (7, 1, 5, 17),
           # hidden sizes beyond what stays on chip: the backward pass, then both passes, stream R
           (3, 5, 40, 704), (3, 4, 32, 1536), (2, 70, 24, 1700), (2, 128, 16, 1024)]
 
@@ -44,9 +46,9 @@ def test_gru_training_forward_backward(T, N, C, H, zoneout):
 
 
 @pytest.mark.parametrize("zoneout", [0.0, 0.25])
-@pytest.mark.parametrize("T,N,C,H", [(20, 16, 128, 256), (8, 50, 16, 512)])
+@pytest.mark.parametrize("T,N,C,H", [(20, 16, 128, 256), (8, 50, 16, 512), (12, 1, 32, 512), (9, 1, 8, 130)])
 def test_gru_inference_forward(zoneout, T, N, C, H):
-    """Inference (zoneout as the convex blend) through the tile and the two-set kernels."""
+    """Inference (zoneout as the convex blend) through the tile, two-set and single-row kernels."""
     from haste_amd import ops
     import torch
     p = problem(8, T, N, C, H, 3, zoneout)
@@ -57,9 +59,9 @@ def test_gru_inference_forward(zoneout, T, N, C, H):
     assert relerr(host(h), ho) < TOL
 
 
-@pytest.mark.parametrize("T,N,C,H", [(6, 8, 16, 64), (5, 48, 16, 128)])
+@pytest.mark.parametrize("T,N,C,H", [(6, 8, 16, 64), (5, 48, 16, 128), (6, 1, 16, 200)])
 def test_gru_dropconnect_fused_equals_premasked_weights(T, N, C, H):
-    """Bit for bit, in the 4-row tile kernel and the two-set kernel."""
+    """Bit for bit, in the 4-row tile kernel, the two-set kernel and the single-row kernel."""
     from haste_amd import ops
     import torch
     p = problem(9, T, N, C, H, 3)
