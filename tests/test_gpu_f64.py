@@ -61,11 +61,11 @@ def test_f64_indrnn(double_precision, T, N, C, H, zoneout, layer_norm):
 
 def test_f64_inference_dropconnect_determinism(double_precision):
     for zoneout in (0.0, 0.25):
-        test_gpu_lstm.test_lstm_inference_forward(zoneout)
-        test_gpu_gru.test_gru_inference_forward(zoneout)
+        test_gpu_lstm.test_lstm_inference_forward(zoneout, 20, 16, 128, 256)
+        test_gpu_gru.test_gru_inference_forward(zoneout, 20, 16, 128, 256)
     test_gpu_layer_norm_cells.test_layer_norm_lstm_inference_forward()
-    test_gpu_lstm.test_lstm_dropconnect_fused_equals_premasked_weights()
-    test_gpu_gru.test_gru_dropconnect_fused_equals_premasked_weights()
+    test_gpu_lstm.test_lstm_dropconnect_fused_equals_premasked_weights(6, 8, 16, 64)
+    test_gpu_gru.test_gru_dropconnect_fused_equals_premasked_weights(6, 8, 16, 64)
     test_gpu_lstm.test_lstm_accumulates_into_weight_gradients_and_is_deterministic()
 
 
