@@ -629,13 +629,7 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
 
   // An 8-row tile is run as two sets of 4 rows when the partial tiles of both fit beside the
   // slice (exchange tiles: one per set, together as large as the tile's).
-  // Short tiles of 16 units take a 64-column slice (a fourth, empty gate) when it fits: one
-  // MFMA then covers all columns of one k and a product leaves 4 partial tiles instead of the
-  // 16 of a 48-column slice, which more than pays for a third more MFMAs (forward N = 64,
-  // H = 512: 0.264 -> 0.240 ms).
-  const int ct = (tile.hs == 16 && tile.nb <= 8 && fwd_lds_bytes(H, tile.nb, 4) <= kWorkgroupLdsBytes &&
-                  paired_lds_bytes((H + 63) / 64 * 64, 4) <= kWorkgroupLdsBytes) ? 4 : tile.ct;
-  const size_t paired_lds = paired_lds_bytes((H + 63) / 64 * 64, ct);
+  const size_t paired_lds = paired_lds_bytes((H + 63) / 64 * 64, tile.ct);
   const bool paired = tile.nb == 8 && paired_lds <= kWorkgroupLdsBytes && paired_sets_enabled();
 
   // Taken after the GEMM, which may replace the stream's scratch buffer with a larger one.
@@ -652,23 +646,21 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
   p.xh = ws.scratch;
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.nb,
-                                  paired ? paired_lds : fwd_lds_bytes(H, tile.nb, ct),
-                                  (unsigned)T + 1, &plan));
+                                  paired ? paired_lds : tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;
   if (paired) plan.threads = 512;
 #define HASTE_LAUNCH_FWD_PAIRED(CT_, HS_)                                                     \
-  if (paired && tile.hs == HS_ && ct == CT_)                                                  \
+  if (paired && tile.hs == HS_)                                                               \
     return launch_persistent("gru_forward_recurrence", gru_forward_kernel<4, CT_, HS_, 2>,    \
                              plan, p, stream);
   HASTE_LAUNCH_FWD_PAIRED(1, 4) HASTE_LAUNCH_FWD_PAIRED(2, 8) HASTE_LAUNCH_FWD_PAIRED(3, 16)
-  HASTE_LAUNCH_FWD_PAIRED(4, 16)
 #undef HASTE_LAUNCH_FWD_PAIRED
 #define HASTE_LAUNCH_FWD(NB_, CT_, HS_)                                                       \
-  if (tile.nb == NB_ && tile.hs == HS_ && ct == CT_)                                          \
+  if (tile.nb == NB_ && tile.hs == HS_)                                                       \
     return launch_persistent("gru_forward_recurrence", gru_forward_kernel<NB_, CT_, HS_, 1>,  \
                              plan, p, stream);
-  HASTE_LAUNCH_FWD(4, 1, 4) HASTE_LAUNCH_FWD(4, 2, 8) HASTE_LAUNCH_FWD(4, 3, 16) HASTE_LAUNCH_FWD(4, 4, 16)
-  HASTE_LAUNCH_FWD(8, 1, 4) HASTE_LAUNCH_FWD(8, 2, 8) HASTE_LAUNCH_FWD(8, 3, 16) HASTE_LAUNCH_FWD(8, 4, 16)
+  HASTE_LAUNCH_FWD(4, 1, 4) HASTE_LAUNCH_FWD(4, 2, 8) HASTE_LAUNCH_FWD(4, 3, 16)
+  HASTE_LAUNCH_FWD(8, 1, 4) HASTE_LAUNCH_FWD(8, 2, 8) HASTE_LAUNCH_FWD(8, 3, 16)
   HASTE_LAUNCH_FWD(16, 1, 4) HASTE_LAUNCH_FWD(16, 2, 8) HASTE_LAUNCH_FWD(16, 3, 16)
   HASTE_LAUNCH_FWD(32, 1, 4) HASTE_LAUNCH_FWD(32, 2, 8) HASTE_LAUNCH_FWD(32, 3, 16)
   HASTE_LAUNCH_FWD(64, 1, 4) HASTE_LAUNCH_FWD(64, 2, 8) HASTE_LAUNCH_FWD(64, 3, 16)

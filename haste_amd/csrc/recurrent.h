@@ -455,13 +455,25 @@ __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
+// Sums across lane groups.  swap_add16(a, b): lanes of the even 16-lane rows get a(row) +
+// a(row+1), lanes of the odd rows b(row-1) + b(row), each from the lanes at the same position
+// in the two rows.  swap_add32 is the same for the two halves of the wavefront.
+__device__ __forceinline__ float swap_add16(float a, float b) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float swap_add32(float a, float b) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 template <int CT>
 struct ShortTileShape {
   static constexpr int NCOLS = 16 * CT;
   static constexpr int CBSZ = NCOLS % 64 == 0 ? 4 : (NCOLS % 32 == 0 ? 3 : 2);
   static constexpr int NBC = 1 << CBSZ;   // 4-column blocks sharing one A block
   static constexpr int MC = 4 * NBC;      // slice columns per MFMA
-  static constexpr int KS = 16 / NBC;     // k values per MFMA = partial sums per wavefront
+  static constexpr int KS = 16 / NBC;     // k values per MFMA = lane groups with sums of their own
   static constexpr int CTN = NCOLS / MC;  // MFMAs side by side to cover the slice columns
 };
 
@@ -474,7 +486,7 @@ struct ProductTile {
   static_assert(NB == 4 || NB == 8 || NB % 16 == 0, "unsupported tile height");
   static constexpr bool kShort = NB < 16;
   static constexpr int NCOLS = 16 * CT;
-  static constexpr int kPartials = kShort ? 4 * ShortTileShape<CT>::KS : 4;
+  static constexpr int kPartials = 4;  // one per wavefront
   static constexpr int kRedFloats = kPartials * NB * NCOLS;
 };
 
@@ -717,9 +729,9 @@ __device__ __forceinline__ void mfma_tile_rows4(const float* w_lds, int s,
   });
 }
 
-// Product of a short exchange tile: red[wave*KS + g][4*RB][16*CT] <- this wavefront's
-// partial tile of lane group g (accumulator element r of acc[rb][ct] in lane l is row
-// 4*rb + r, column ct*MC + l%MC, partial g = l/MC).  The operand
+// Product of a short exchange tile: red[wave][4*RB][16*CT] <- this wavefront's partial tile
+// (accumulator element r of acc[rb][ct] in lane l is row 4*rb + r, column ct*MC + l%MC, of
+// the k that lane group l/MC took).  The operand
 // loads of chunk c+1 (CH super-groups) are issued before the MFMAs of chunk c; the two
 // register buffers alternate so that nothing is copied.  The four wavefronts are those of one
 // 256-thread set of the workgroup.  TAGGED: the partial tiles are themselves polled by their
@@ -775,18 +787,36 @@ __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int
     mfma_tile_rows4<RB, CT, 1>(w_lds, s, one, acc0, acc1);
   }
 
-  float* base = red + ((wave * S::KS + lane / S::MC) * NB) * S::NCOLS + lane % S::MC;
+  // The KS lane groups hold partial sums of the same elements: they are added here, so that a
+  // wavefront leaves one partial tile, and every lane stores 4/KS of the 4 rows.
+  float* base = red + (wave * NB) * S::NCOLS + lane % S::MC;
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
     for (int ct = 0; ct < S::CTN; ++ct) {
       float4_t v = acc0[rb][ct] + acc1[rb][ct];
-      if constexpr (TAGGED) v = float4_t{publishable(v.x), publishable(v.y), publishable(v.z), publishable(v.w)};
       float* q = base + (4 * rb) * S::NCOLS + ct * S::MC;
-      q[0] = v.x;
-      q[S::NCOLS] = v.y;
-      q[2 * S::NCOLS] = v.z;
-      q[3 * S::NCOLS] = v.w;
+      if constexpr (S::KS == 4) {
+        // lane group 0, 1, 2, 3 ends up with row 0, 2, 1, 3
+        const float xz = swap_add16(v.x, v.z), yw = swap_add16(v.y, v.w);
+        float r = swap_add32(xz, yw);
+        if constexpr (TAGGED) r = publishable(r);
+        const int g = lane >> 4;
+        q[(((g & 1) << 1) | (g >> 1)) * S::NCOLS] = r;
+      } else if constexpr (S::KS == 2) {
+        // lane group 0: rows 0 and 2; lane group 1: rows 1 and 3
+        float r0 = swap_add32(v.x, v.y), r1 = swap_add32(v.z, v.w);
+        if constexpr (TAGGED) { r0 = publishable(r0); r1 = publishable(r1); }
+        const int g = lane >> 5;
+        q[g * S::NCOLS] = r0;
+        q[(g + 2) * S::NCOLS] = r1;
+      } else {
+        if constexpr (TAGGED) v = float4_t{publishable(v.x), publishable(v.y), publishable(v.z), publishable(v.w)};
+        q[0] = v.x;
+        q[S::NCOLS] = v.y;
+        q[2 * S::NCOLS] = v.z;
+        q[3 * S::NCOLS] = v.w;
+      }
     }
 }
 
@@ -862,8 +892,7 @@ __device__ __forceinline__ float sum_product(const float* red, int row, int col)
 // wavefronts that have a share of k.
 template <int CT>
 __device__ __forceinline__ int live_partials(int Kpad) {
-  const int waves = (Kpad >> 6) < 4 ? (Kpad >> 6) : 4;
-  return waves * ShortTileShape<CT>::KS;
+  return (Kpad >> 6) < 4 ? (Kpad >> 6) : 4;
 }
 
 // out[g] = element (row, col0 + g * col_stride) of the product, partials added in
@@ -997,9 +1026,9 @@ __device__ __forceinline__ float single_row_product(const GroupSync& gs, const T
 // ---- host side ---------------------------------------------------------------------
 // Partial tiles slice_product leaves in LDS (ProductTile<nb, ct>::kPartials).
 inline int product_partials(int nb, int ct) {
-  if (nb >= 16) return 4;
-  const int ncols = 16 * ct;
-  return ncols % 64 == 0 ? 4 : (ncols % 32 == 0 ? 8 : 16);
+  (void)nb;
+  (void)ct;
+  return 4;
 }
 
 // LDS bytes of a forward kernel (slice [Kpad x 16*ct] + the partial tiles of nb rows).
