@@ -532,7 +532,7 @@ int haste_hip_layer_norm_gru_forward_f32(int training, int steps, int batch_size
   HASTE_HIP_REQUIRE(W && R && bx && br && x && h && act_Wx && gamma1 && tmp_Wx_norm && act_Rh && gamma2);
   HASTE_HIP_REQUIRE(!training || v != nullptr);
   hipStream_t stream = as_stream(stream_);
-  const ForwardTile tile = pick_forward_tile(3, N, H, 2 * sizeof(float));
+  const ForwardTile tile = pick_forward_tile(3, N, H, 2 * sizeof(float), kMaxLdsBytes, true);
   if (!tile.ok)
     return layer_norm_gru_forward_streamed(stream, training, T, N, C, H, W, R, bx, br, x, h, v, act_Wx,
                                            gamma1, cache1, tmp_Wx_norm, act_Rh, gamma2, cache2,

@@ -631,7 +631,7 @@ int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_siz
   HASTE_HIP_REQUIRE(W && R && b && x && h && c && act_Wx && gamma1 && act_Wx_norm && act_Rh);
   HASTE_HIP_REQUIRE(gamma2 && gamma_h && beta_h && act_c_norm);
   hipStream_t stream = as_stream(stream_);
-  const ForwardTile tile = pick_forward_tile(4, N, H, 4 * sizeof(float));
+  const ForwardTile tile = pick_forward_tile(4, N, H, 4 * sizeof(float), kMaxLdsBytes, true);
   if (!tile.ok)
     return layer_norm_lstm_forward_streamed(stream, training, T, N, C, H, W, R, b, x, h, c, act_Wx,
                                             gamma1, cache1, act_Wx_norm, act_Rh, gamma2, cache2,
