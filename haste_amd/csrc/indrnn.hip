@@ -14,7 +14,9 @@
 namespace haste_hip {
 namespace {
 
-constexpr int U = 8;  // steps of operands kept in flight per thread
+// Steps of operands kept in flight per thread (twice that while the next batch is requested).
+// 16 is 5-14 % faster than 8 (N*H = 8192 .. 131072 chains); 32 no better.
+constexpr int U = 16;
 
 template <bool TRAINING, bool ZONEOUT>
 __global__ __launch_bounds__(256)
