@@ -15,6 +15,9 @@ namespace haste_hip {
 // Records the text of a failed HIP call for haste_hip_last_runtime_error().
 void set_runtime_error(hipError_t err, const char* what);
 
+// Records a plain explanation (a size limit, a refused configuration) for the same query.
+void set_error_text(const char* text);
+
 #define HASTE_HIP_TRY(expr)                                   \
   do {                                                        \
     hipError_t err__ = (expr);                                \

@@ -12,6 +12,8 @@
 // lib/layer_norm_backward_gpu.cu.cc:46-92 (eps 1e-5, biased variance).
 #include "recurrent.h"
 
+#include <mutex>
+
 namespace haste_hip {
 namespace {
 
@@ -265,27 +267,30 @@ int layer_norm_forward(hipStream_t stream, int rows, int dim, const float* gamma
   return HASTE_HIP_OK;
 }
 
-int layer_norm_backward(hipStream_t stream, int rows, int dim, const float* gamma,
-                        const float* x, const float* dy, float* dx, float* dgamma,
-                        float* dbeta) {
-  HASTE_HIP_REQUIRE(rows > 0 && dim > 0 && gamma && x && dy && dx && dgamma);
-  const bool vec = dim % 4 == 0 && aligned16(gamma) && aligned16(x) && aligned16(dy) && aligned16(dx);
-  const int E = elements_per_lane(dim, vec);
-  if (E == 0) return layer_norm_backward_wide(stream, rows, dim, gamma, x, dy, dx, dgamma, dbeta);
+namespace {
+
+// The row kernel's grid: four rows per workgroup pass, at most two workgroups per CU
+// (measured: 3, 4 and 6 per CU are no faster).
+int backward_grid(int rows) {
   const int cus = device_cu_count();
   int grid = (rows + 3) / 4;
-  if (grid > 2 * cus) grid = 2 * cus;  // measured: 3, 4 and 6 per CU are no faster
-  Workspace ws;
-  HASTE_HIP_PROPAGATE(get_workspace(stream, (size_t)grid * 2 * dim * sizeof(float), &ws));
+  if (grid > 2 * cus) grid = 2 * cus;
+  return grid;
+}
+
+// Row kernel + column-sum kernel with the workgroups' partial column sums parked in
+// `partial` ([grid][2][dim] floats of device memory).
+int layer_norm_backward_launch(hipStream_t stream, int rows, int dim, int E, bool vec, int grid,
+                               const float* gamma, const float* x, const float* dy, float* dx,
+                               float* dgamma, float* dbeta, float* partial) {
   const size_t lds = (size_t)4 * 2 * E * 64 * sizeof(float);
-  ScopedKernelTimer timer("layer_norm_backward", stream);
 #define HASTE_LN_BWD(E_, VEC_)                                                            \
   if (E == E_ && vec == VEC_) {                                                           \
     HASTE_HIP_TRY(hipFuncSetAttribute(                                                    \
         reinterpret_cast<const void*>(layer_norm_backward_kernel<E_, VEC_>),              \
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                           \
     layer_norm_backward_kernel<E_, VEC_><<<dim3(grid), dim3(256), lds, stream>>>(         \
-        rows, dim, gamma, x, dy, dx, ws.scratch);                                          \
+        rows, dim, gamma, x, dy, dx, partial);                                             \
   }
   HASTE_LN_BWD(4, true) HASTE_LN_BWD(8, true) HASTE_LN_BWD(16, true) HASTE_LN_BWD(32, true)
   HASTE_LN_BWD(64, true)
@@ -293,7 +298,81 @@ int layer_norm_backward(hipStream_t stream, int rows, int dim, const float* gamm
   HASTE_LN_BWD(16, false)
 #undef HASTE_LN_BWD
   HASTE_HIP_TRY(hipGetLastError());
-  return add_column_partials(stream, grid, dim, ws.scratch, dgamma, dbeta);
+  return add_column_partials(stream, grid, dim, partial, dgamma, dbeta);
+}
+
+}  // namespace
+
+int layer_norm_backward(hipStream_t stream, int rows, int dim, const float* gamma,
+                        const float* x, const float* dy, float* dx, float* dgamma,
+                        float* dbeta) {
+  HASTE_HIP_REQUIRE(rows > 0 && dim > 0 && gamma && x && dy && dx && dgamma);
+  const bool vec = dim % 4 == 0 && aligned16(gamma) && aligned16(x) && aligned16(dy) && aligned16(dx);
+  const int E = elements_per_lane(dim, vec);
+  if (E == 0) return layer_norm_backward_wide(stream, rows, dim, gamma, x, dy, dx, dgamma, dbeta);
+  const int grid = backward_grid(rows);
+  Workspace ws;
+  HASTE_HIP_PROPAGATE(get_workspace(stream, (size_t)grid * 2 * dim * sizeof(float), &ws));
+  ScopedKernelTimer timer("layer_norm_backward", stream);
+  return layer_norm_backward_launch(stream, rows, dim, E, vec, grid, gamma, x, dy, dx, dgamma,
+                                    dbeta, ws.scratch);
+}
+
+// ---- The variant that allocates nothing ------------------------------------------------
+// The partial column sums live in a fixed array in the library's device image instead of the
+// stream's workspace.  Every GPU the library runs on holds its own copy of the array at its own
+// address until the process ends; in host code the array's name is only a stand-in, so its
+// device address is looked up once per device and that pointer is what the kernels are given.
+constexpr size_t kNoAllocScratchFloats = (size_t)4 << 20;  // 16 MiB: 512 workgroups x 2 x 4096
+static __device__ __align__(256) float scratch[kNoAllocScratchFloats];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_noalloc_mutex;
+float* g_noalloc_scratch[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (looked up at the first call on it).
+int noalloc_scratch(float** out) {
+  int dev = 0;
+  HASTE_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  std::lock_guard<std::mutex> lock(g_noalloc_mutex);
+  if (g_noalloc_scratch[dev] == nullptr) {
+    float* ptr = nullptr;
+    HASTE_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)));
+    if (ptr == nullptr) return HASTE_HIP_ERROR_RUNTIME;
+    g_noalloc_scratch[dev] = ptr;
+  }
+  *out = g_noalloc_scratch[dev];
+  return HASTE_HIP_OK;
+}
+}  // namespace
+
+int layer_norm_backward_noalloc(hipStream_t stream, int rows, int dim, const float* gamma,
+                                const float* x, const float* dy, float* dx, float* dgamma,
+                                float* dbeta) {
+  HASTE_HIP_REQUIRE(rows > 0 && dim > 0 && gamma && x && dy && dx && dgamma);
+  const bool vec = dim % 4 == 0 && aligned16(gamma) && aligned16(x) && aligned16(dy) && aligned16(dx);
+  const int E = elements_per_lane(dim, vec);
+  if (E == 0) {
+    set_error_text("layer_norm_backward_noalloc: rows wider than 4096 columns (1024 when a "
+                   "pointer is not 16-byte aligned or the width is not a multiple of 4) are not "
+                   "supported by the entry point that allocates nothing");
+    return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  }
+  const int grid = backward_grid(rows);
+  if (grid <= 0) return HASTE_HIP_ERROR_RUNTIME;
+  if ((size_t)grid * 2 * dim > kNoAllocScratchFloats) {
+    set_error_text("layer_norm_backward_noalloc: workgroups x 2 x dim exceeds the fixed 16 MiB "
+                   "scratch array");
+    return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  }
+  float* partial = nullptr;
+  HASTE_HIP_PROPAGATE(noalloc_scratch(&partial));
+  // Every element of partial[0 .. grid) x [0 .. 2 dim) is written by the row kernel before the
+  // column-sum kernel reads it, so nothing of an earlier call's contents needs clearing.
+  return layer_norm_backward_launch(stream, rows, dim, E, vec, grid, gamma, x, dy, dx, dgamma,
+                                    dbeta, partial);
 }
 
 }  // namespace haste_hip
@@ -312,6 +391,14 @@ int haste_hip_layer_norm_backward_f32(int rows, int dim, const float* gamma, con
   (void)cache;  // statistics are recomputed from x
   return haste_hip::layer_norm_backward(haste_hip::as_stream(stream), rows, dim, gamma, x, dy, dx,
                                         dgamma, dbeta);
+}
+
+int haste_hip_layer_norm_backward_noalloc_f32(int rows, int dim, const float* gamma, const float* x,
+                                              const float* dy, float* dx, float* dgamma,
+                                              float* dbeta, const float* cache, void* stream) {
+  (void)cache;
+  return haste_hip::layer_norm_backward_noalloc(haste_hip::as_stream(stream), rows, dim, gamma, x,
+                                                dy, dx, dgamma, dbeta);
 }
 
 }  // extern "C"

@@ -72,6 +72,8 @@ void set_runtime_error(hipError_t err, const char* what) {
   (void)hipGetLastError();  // do not leave the error for an unrelated later call
 }
 
+void set_error_text(const char* text) { g_last_error = text; }
+
 namespace {
 struct LastPersistent {
   hipEvent_t event = nullptr;

@@ -198,6 +198,21 @@ int haste_hip_layer_norm_backward_f32(int rows, int dim, const float* gamma, con
                                       const float* dy, float* dx, float* dgamma, float* dbeta,
                                       const float* cache, void* stream);
 
+/* The same computation as haste_hip_layer_norm_backward_f32 for callers that cannot allocate
+ * device memory: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  It has no counterpart in the reference.  The workgroups' partial column sums go
+ * to a fixed 16 MiB array inside the library's device image (one copy per GPU, held until the
+ * process ends) instead of the stream's workspace, and the call makes no hipMalloc / hipFree
+ * and creates no events.  Limits: dim <= 4096 (1024 when dim is not a multiple of 4 or a
+ * pointer is not 16-byte aligned) and min(ceil(rows/4), 2 x compute units) x 2 x dim <= 4 Mi
+ * floats; beyond them HASTE_HIP_ERROR_UNSUPPORTED_SIZE with the reason in
+ * haste_hip_last_runtime_error().  All calls on one GPU share the array: calls that overlap
+ * on one GPU (different streams, or threads) race; calls on one stream are ordered. */
+int haste_hip_layer_norm_backward_noalloc_f32(int rows, int dim, const float* gamma,
+                                              const float* x, const float* dy, float* dx,
+                                              float* dgamma, float* dbeta, const float* cache,
+                                              void* stream);
+
 /* ---- LayerNorm LSTM ----------------------------------------------------------
  * reference lib/haste/layer_norm_lstm.h:75-92, lib/layer_norm_lstm_forward_gpu.cu.cc:276-340.
  * The three layer_norm::ForwardPass objects of the reference are passed flattened:
