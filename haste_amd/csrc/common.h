@@ -102,6 +102,11 @@ bool paired_sets_enabled();
 // recurrent weights in registers (for experiments).
 bool single_row_enabled();
 
+// False when the environment variable HASTE_HIP_FUSED_INPUT is set to 0: the forward
+// recurrences then read x * W from a GEMM launched before them instead of computing it beside
+// their waits (for experiments).
+bool fused_input_enabled();
+
 // C[M,N] = op(A)*B (+C): fp32 MFMA GEMM on `stream`.  The partial tiles of a split product
 // are kept `scratch_offset` bytes (a multiple of 16) into the stream's scratch buffer.
 int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,

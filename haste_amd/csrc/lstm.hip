@@ -24,6 +24,10 @@ struct LstmFwdParams {
   const float* dc_mask;        // DropConnect mask [H,4H] or null
   float dc_scale;
   float* xh;                   // polled exchange tiles of h: [batch tiles][4][Kpad/4][NB][4]
+  // kernels that compute the input projection themselves (XSG > 0): v does not hold x*W
+  const float* x;              // [T,N,C]
+  const float* W;              // [C,4H]
+  int C;
   LaunchShape ls;
 };
 
@@ -31,10 +35,15 @@ struct LstmFwdParams {
 // SETS sets of 256 threads, each with a batch tile of NB rows of its own.  Two sets share
 // the resident slice but nothing else: while one waits for its exchange the other computes,
 // which a single tile of 2*NB rows cannot do.
-template <int NB, int CT, int SETS>
+// XSG > 0 (4-row tiles): the kernel also computes the input projection x[t] * W, on the matrix
+// units while its wavefronts wait for h[t] (InputProjection in recurrent.h; a wavefront takes
+// XSG super-groups of 64 input features), instead of reading it from v.
+template <int NB, int CT, int SETS, int XSG = 0>
 __global__ __launch_bounds__(256 * SETS, 1)
 void lstm_forward_kernel(LstmFwdParams p) {
   static_assert(SETS == 1 || (SETS == 2 && NB < 16), "two sets: short tiles only");
+  static_assert(XSG == 0 || NB == 4, "fused input projection: 4-row tiles only");
+  constexpr bool kFusedInput = XSG > 0;
   constexpr int HS = 4 * CT;
   constexpr int NCOLS = 16 * CT;
   constexpr int PP = (NB * HS + 255) / 256;
@@ -72,6 +81,19 @@ void lstm_forward_kernel(LstmFwdParams p) {
   // k beyond the problem stay zero for the whole launch.
   zero_tile_share<SETS>(gs, xh, tile_floats, NB, j0 / 4,
                         (role.cw == p.ls.gx - 1 ? Kpad - j0 : HS) / 4, kPolledTiles);
+
+  // The wavefront's share of W, in registers (requested before the slice, whose loads then
+  // overlap with these).
+  using Projection = std::conditional_t<kFusedInput, InputProjection<CT, kFusedInput ? XSG : 1>, NoSideWork>;
+  Projection proj;
+  if constexpr (kFusedInput) {
+    proj.setup(p.W, p.x, p.C, N, 4 * H, set_wave<SETS>(), n0 < N ? n0 : N - 1, [=](int col) {
+      const int gate = col / HS, j = j0 + col % HS;
+      return j < H ? (long long)gate * H + j : -1ll;
+    });
+    proj.request();
+    proj.settle();
+  }
 
   // Resident slice: column c of the slice is gate c/HS, hidden unit j0 + c%HS.
   {
@@ -131,9 +153,11 @@ void lstm_forward_kernel(LstmFwdParams p) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) wx_next[pp][g] = 0.f;
       if (act[pp] && t < T) {
-        const float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+        if constexpr (!kFusedInput) {
+          const float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
 #pragma unroll
-        for (int g = 0; g < 4; ++g) wx_next[pp][g] = vt[g * H];
+          for (int g = 0; g < 4; ++g) wx_next[pp][g] = vt[g * H];
+        }
         if (zoneout && p.training) mk_next[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
       }
     }
@@ -150,7 +174,13 @@ void lstm_forward_kernel(LstmFwdParams p) {
     }
     // The operand loads wait for h[t] themselves (polled tile t % 4).
     float* red_t = !kPolledPartials ? red : red + (t & 1) * RED;
-    tile_product<NB, CT, false, true, kPolledPartials>(xhb, (t & 3) * tile_floats, Kpad, w_lds, red_t, &gs);
+    if constexpr (kFusedInput) {
+      tile_product<NB, CT, false, true, kPolledPartials, Projection>(xhb, (t & 3) * tile_floats, Kpad,
+                                                                      w_lds, red_t, &gs, &proj);
+      if (t + 1 < T) proj.request();  // x[t+1]: a whole step to arrive
+    } else {
+      tile_product<NB, CT, false, true, kPolledPartials>(xhb, (t & 3) * tile_floats, Kpad, w_lds, red_t, &gs);
+    }
     if constexpr (!kPolledPartials) __syncthreads();
 
     float gate[PP][4], h_pub[PP];
@@ -169,7 +199,8 @@ void lstm_forward_kernel(LstmFwdParams p) {
       if (act[pp]) {
         float a[4];
 #pragma unroll
-        for (int g = 0; g < 4; ++g) a[g] = wx[pp][g] + rh[g] + bias[pp][g];
+        for (int g = 0; g < 4; ++g)
+          a[g] = kFusedInput ? rh[g] + bias[pp][g] : wx[pp][g] + rh[g] + bias[pp][g];
         gate[pp][0] = sigmoid_f(a[0]);
         gate[pp][1] = tanh_f(a[1]);
         gate[pp][2] = sigmoid_f(a[2]);
@@ -187,7 +218,9 @@ void lstm_forward_kernel(LstmFwdParams p) {
     }
     // Everything this wavefront stored during the previous step (its resets among it) has
     // landed before h[t+1] becomes visible.
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // (x[t+1] arrives with the same wait.)
+    if constexpr (kFusedInput) proj.settle();
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     if (t + 1 < T) {
       float* xh_next = xh + ((t + 1) & 3) * tile_floats;
       float* xh_done = xh + ((t + 3) & 3) * tile_floats;  // read at step t-1: nobody needs it any more
@@ -623,14 +656,21 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
   if (!tile.ok)
     return lstm_forward_streamed(stream, training, T, N, C, H, W, R, b, x, h, c, h_out, c_out, v,
                                  zoneout_prob, zoneout_mask, dc_mask, dc_scale);
-  // v = x * W for all steps at once.
-  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 4 * H, C, x, C, W, 4 * H, v, 4 * H, false));
-
   // An 8-row tile is run as two sets of 4 rows when the partial tiles of both fit beside the
   // slice (exchange tiles: one per set, together as large as the tile's).  Measured at
   // H = 512: 6 % faster per step; two sets of 8 rows instead of a 16-row tile: 6 % slower.
   const size_t paired_lds = paired_lds_bytes((H + 63) / 64 * 64, tile.ct);
   const bool paired = tile.nb == 8 && paired_lds <= kWorkgroupLdsBytes && paired_sets_enabled();
+
+  // With 4-row tiles the recurrence computes x * W itself, beside its waits (every wavefront of
+  // a set must have a share of the recurrent product, H > 192, to keep in step with the readers
+  // of its partial tiles; the projection's weights must fit the registers, C <= 512).
+  // Otherwise: v = x * W for all steps at once.
+  const int xsg = (C + 255) / 256;  // super-groups of 64 input features per wavefront
+  const bool fused = (paired || tile.nb == 4) && H > 192 && C <= 512 && C % 4 == 0 &&
+                     (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && fused_input_enabled();
+  if (!fused)
+    HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 4 * H, C, x, C, W, 4 * H, v, 4 * H, false));
 
   // Taken after the GEMM, which may replace the stream's scratch buffer with a larger one.
   Workspace ws;
@@ -644,11 +684,23 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
   p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
   p.dc_mask = dc_mask; p.dc_scale = dc_scale;
   p.xh = ws.scratch;
+  p.x = x; p.W = W; p.C = C;
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.nb,
                                   paired ? paired_lds : tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;
   if (paired) plan.threads = 512;
+#define HASTE_LAUNCH_FWD_FUSED(CT_, XSG_)                                                       \
+  if (fused && tile.ct == CT_ && xsg == XSG_) {                                                  \
+    if (paired)                                                                                  \
+      return launch_persistent("lstm_forward_recurrence", lstm_forward_kernel<4, CT_, 2, XSG_>,  \
+                               plan, p, stream);                                                 \
+    return launch_persistent("lstm_forward_recurrence", lstm_forward_kernel<4, CT_, 1, XSG_>,    \
+                             plan, p, stream);                                                   \
+  }
+  HASTE_LAUNCH_FWD_FUSED(1, 1) HASTE_LAUNCH_FWD_FUSED(2, 1) HASTE_LAUNCH_FWD_FUSED(4, 1)
+  HASTE_LAUNCH_FWD_FUSED(1, 2) HASTE_LAUNCH_FWD_FUSED(2, 2) HASTE_LAUNCH_FWD_FUSED(4, 2)
+#undef HASTE_LAUNCH_FWD_FUSED
 #define HASTE_LAUNCH_FWD_PAIRED(CT_)                                                       \
   if (paired && tile.ct == CT_)                                                            \
     return launch_persistent("lstm_forward_recurrence", lstm_forward_kernel<4, CT_, 2>, plan, p, \

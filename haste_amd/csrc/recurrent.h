@@ -729,6 +729,122 @@ __device__ __forceinline__ void mfma_tile_rows4(const float* w_lds, int s,
   });
 }
 
+// ---- work beside the wait ------------------------------------------------------------
+// A step of a recurrence is a chain (wait for the exchanged operand, product, pointwise math,
+// publish) during most of which the matrix unit of the wavefront's SIMD is idle.  A product
+// that does not depend on the recurrence can be issued while the wavefront waits: the input
+// projection x[t] * W of a forward pass.  Its B operand comes from registers (no LDS reads
+// compete with the resident slice), its MFMAs accumulate into the accumulators the recurrent
+// product continues with -- always all of the projection first, then the recurrent product,
+// so the sums do not depend on timing -- and between batches of them the wavefront looks at
+// the operand loads it is polling.
+struct NoSideWork {
+  static constexpr int kBatches = 0;
+};
+
+// x[t][4 rows of a batch tile][C] * W[C][16*CT slice columns] on the 4x4x1 path, the
+// contraction split over the four wavefronts of a set like the recurrent product's: this
+// wavefront takes the XSG super-groups (64 k each) wave, wave + 4, ...  A lane keeps the weights
+// its MFMAs need in registers for the whole launch: 4 * CT * XSG floats, i.e. 128 for a
+// 64-column slice and C = 512 (two wavefronts per SIMD leave 256 registers per lane).
+template <int CT, int XSG>
+struct InputProjection {
+  using S = ShortTileShape<CT>;
+  static constexpr int kSteps = XSG * S::NBC;   // one step: 4 * CTN MFMAs on one A block
+  static constexpr int kStepsPerBatch = 4;
+  static constexpr int kBatches = (kSteps + kStepsPerBatch - 1) / kStepsPerBatch;
+  float w[XSG][S::NBC][S::CTN][4];
+  float4_t xa[XSG];          // this step's A operands
+  const float* xp[XSG];      // where the lane's operands of the next step to load are
+  bool valid[XSG];           // the lane's k exist (k < C)
+  size_t step_stride;        // floats between consecutive steps of x
+
+  // `wave`: wavefront inside the set.  Column `col` of the slice is column gcol(col) of W
+  // (row length `row_len`), or does not exist (gcol < 0).  Lane l = 4*block + r multiplies
+  // row n0 + r (rows beyond N read row N-1: their results are never used).
+  template <class ColFn>
+  __device__ __forceinline__ void setup(const float* __restrict__ W, const float* __restrict__ x,
+                                        int C, int N, int row_len, int wave, int n0, ColFn gcol) {
+    const int lane = threadIdx.x & 63;
+    const int g = lane / S::MC;
+    step_stride = (size_t)N * C;
+    int row = n0 + (lane & 3);
+    row = row < N ? row : N - 1;
+    const int block = lane >> 2;
+    const int k4 = (block % S::NBC) * S::KS + block / S::NBC;
+#pragma unroll
+    for (int xs = 0; xs < XSG; ++xs) {
+      const int kx = 64 * (wave + 4 * xs) + 4 * k4;
+      valid[xs] = kx < C;
+      xp[xs] = x + (size_t)row * C + (valid[xs] ? kx : 0);
+#pragma unroll
+      for (int a = 0; a < S::NBC; ++a)
+#pragma unroll
+        for (int ct = 0; ct < S::CTN; ++ct) {
+          const long long col = gcol(ct * S::MC + lane % S::MC);
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            // every lane loads (some valid element where its own does not exist), so that the
+            // loads carry no branches and are all in flight at once
+            const int k = 64 * (wave + 4 * xs) + 4 * (a * S::KS + g) + c;
+            const bool exists = k < C && col >= 0;
+            const float loaded = W[exists ? (size_t)k * row_len + col : 0];
+            w[xs][a][ct][c] = exists ? loaded : 0.f;
+          }
+        }
+    }
+  }
+
+  // Requests the operands of the next step (C is a multiple of 4 and x 16-byte aligned).
+  __device__ __forceinline__ void request() {
+#pragma unroll
+    for (int xs = 0; xs < XSG; ++xs) {
+      xa[xs] = *reinterpret_cast<const float4_t*>(xp[xs]);
+      xp[xs] += step_stride;
+    }
+  }
+
+  // Waits until everything this wavefront has requested or stored has completed -- the
+  // operands of the next step among it -- and finishes those (lanes whose k do not exist
+  // contribute zeros: their loads read some valid element).  The operands pass through the
+  // wait as its outputs, and through an empty statement afterwards: left to itself the compiler
+  // touches them, and so waits for them, at the top of the next step, where its wait also covers
+  // whatever was stored since -- the publication, the caller's copies -- with the matrix
+  // units idle (0.6 us per step).
+  __device__ __forceinline__ void settle() {
+#pragma unroll
+    for (int xs = 0; xs < XSG; ++xs) asm volatile("s_waitcnt vmcnt(0)" : "+v"(xa[xs]) : : "memory");
+#pragma unroll
+    for (int xs = 0; xs < XSG; ++xs) {
+      if (!valid[xs]) xa[xs] = float4_t{0.f, 0.f, 0.f, 0.f};
+      asm volatile("" : "+v"(xa[xs]));
+    }
+  }
+
+  template <int B>
+  __device__ __forceinline__ void batch(float4_t (&acc0)[1][S::CTN], float4_t (&acc1)[1][S::CTN]) const {
+    static_for<kStepsPerBatch>([&](auto ic) {
+      constexpr int I = B * kStepsPerBatch + decltype(ic)::value;
+      if constexpr (I < kSteps) {
+        constexpr int XS = I / S::NBC;
+        constexpr int A = I % S::NBC;
+#pragma unroll
+        for (int ct = 0; ct < S::CTN; ++ct)
+          acc0[0][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(xa[XS].x, w[XS][A][ct][0], acc0[0][ct], S::CBSZ, A, 0);
+#pragma unroll
+        for (int ct = 0; ct < S::CTN; ++ct)
+          acc1[0][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(xa[XS].y, w[XS][A][ct][1], acc1[0][ct], S::CBSZ, A, 0);
+#pragma unroll
+        for (int ct = 0; ct < S::CTN; ++ct)
+          acc0[0][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(xa[XS].z, w[XS][A][ct][2], acc0[0][ct], S::CBSZ, A, 0);
+#pragma unroll
+        for (int ct = 0; ct < S::CTN; ++ct)
+          acc1[0][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(xa[XS].w, w[XS][A][ct][3], acc1[0][ct], S::CBSZ, A, 0);
+      }
+    });
+  }
+};
+
 // Product of a short exchange tile: red[wave][4*RB][16*CT] <- this wavefront's partial tile
 // (accumulator element r of acc[rb][ct] in lane l is row 4*rb + r, column ct*MC + l%MC, of
 // the k that lane group l/MC took).  The operand
@@ -736,10 +852,10 @@ __device__ __forceinline__ void mfma_tile_rows4(const float* w_lds, int s,
 // register buffers alternate so that nothing is copied.  The four wavefronts are those of one
 // 256-thread set of the workgroup.  TAGGED: the partial tiles are themselves polled by their
 // readers (take_product), so no element may carry the "unwritten" pattern.
-template <int RB, int CT, int CH, bool POLLED, bool TAGGED = false>
+template <int RB, int CT, int CH, bool POLLED, bool TAGGED = false, class Side = NoSideWork>
 __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int tile_off, int Kpad,
                                                        const float* w_lds, float* red,
-                                                       const GroupSync* gs) {
+                                                       const GroupSync* gs, Side* side = nullptr) {
   using S = ShortTileShape<CT>;
   constexpr int NB = 4 * RB;
   const int lane = threadIdx.x & 63;
@@ -757,9 +873,32 @@ __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int
     for (int ct = 0; ct < S::CTN; ++ct) acc0[rb][ct] = acc1[rb][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
 
   int s = wave;
+  if constexpr (Side::kBatches > 0) {
+    static_assert(RB == 1 && POLLED, "side work: polled 4-row tiles");
+    // no operand chunk to look at between the batches: the side work runs on its own
+    if (chunks == 0)
+      static_for<Side::kBatches>([&](auto b) { side->template batch<decltype(b)::value>(acc0, acc1); });
+  }
   if (chunks > 0) {
     float4_t buf0[CH][RB], buf1[CH][RB];
     load_tile_rows4<RB, CT, CH>(xb, tile_off, s, buf0);
+    if constexpr (Side::kBatches > 0) {
+      // The side work, in batches; after every second one a look at the first chunk's loads
+      // (re-issued while some element is still unwritten).  How often makes no difference
+      // (looks after every batch, every fourth, none: 3.26-3.33 us per step at N = 64,
+      // C = H = 512): with the projection the step is bound by the rate of the 4x4x1 MFMAs.
+      bool seen = false;
+      static_for<Side::kBatches>([&](auto b) {
+        side->template batch<decltype(b)::value>(acc0, acc1);
+        if (decltype(b)::value % 2 == 1 && !seen) {
+          seen = all_written(buf0);
+          if (!seen) {
+            asm volatile("" ::: "memory");
+            load_tile_rows4<RB, CT, CH>(xb, tile_off, s, buf0);
+          }
+        }
+      });
+    }
     int c = 0;
     for (;;) {
       if (c + 1 < chunks) load_tile_rows4<RB, CT, CH>(xb, tile_off, s + 4 * CH, buf1);
@@ -825,14 +964,16 @@ __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int
 // longer than the hidden size (the backward passes).
 // POLLED: the tile is a polled exchange tile (see above) and `gs` supplies the bounds of the
 // wait; otherwise the caller has waited at the group's step barrier and `gs` is unused.
-template <int NB, int CT, bool LONG_K, bool POLLED = false, bool TAGGED = false>
+template <int NB, int CT, bool LONG_K, bool POLLED = false, bool TAGGED = false, class Side = NoSideWork>
 __device__ __forceinline__ void tile_product(const TileBuffer& xb, int tile_off, int Kpad,
                                              const float* w_lds, float* red,
-                                             const GroupSync* gs = nullptr) {
+                                             const GroupSync* gs = nullptr, Side* side = nullptr) {
   if constexpr (ProductTile<NB, CT>::kShort) {
-    short_exchange_product<NB / 4, CT, LONG_K ? 4 : 2, POLLED, TAGGED>(xb, tile_off, Kpad, w_lds, red, gs);
+    short_exchange_product<NB / 4, CT, LONG_K ? 4 : 2, POLLED, TAGGED, Side>(xb, tile_off, Kpad, w_lds,
+                                                                              red, gs, side);
   } else {
     static_assert(!TAGGED, "polled partial tiles exist for short tiles only");
+    static_assert(Side::kBatches == 0, "side work exists for short tiles only");
     constexpr int RT = NB / 16;
     // k-groups of operands per load (two loads in flight).  Measured at H = 512: a forward share
     // (8 groups per wavefront) in one piece, a backward share (32 groups) in two, are 9-10 %

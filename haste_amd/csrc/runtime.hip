@@ -123,6 +123,14 @@ bool single_row_enabled() {
   return enabled;
 }
 
+bool fused_input_enabled() {
+  static const bool enabled = [] {
+    const char* v = std::getenv("HASTE_HIP_FUSED_INPUT");
+    return v == nullptr || v[0] != '0';
+  }();
+  return enabled;
+}
+
 int device_cu_count() {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
