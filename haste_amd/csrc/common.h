@@ -59,14 +59,22 @@ struct Workspace {
   ControlBlock* control = nullptr;   // device
   float* scratch = nullptr;          // device
   size_t scratch_bytes = 0;
+  size_t scratch_high_water = 0;     // most scratch any call on this stream has asked for
   unsigned int epoch = 0;            // step-flag values handed out so far
   unsigned int ticket_base = 0;      // per-XCD tickets handed out so far
   unsigned int* host_status = nullptr;      // pinned host word the kernels report aborts to
   unsigned int* host_status_dev = nullptr;  // the same word as the device addresses it
+  bool self_resetting = false;       // every persistent launch wipes the control block first
+                                     // and numbers its flags and tickets from zero (set once a
+                                     // launch on this stream has been captured into a graph)
+  bool caller_owned = false;         // control and scratch lie in memory the caller lent
+                                     // (haste_hip_set_workspace): never freed or grown here
 };
 
 // Returns the workspace of (current device, stream) with at least `scratch_bytes`
-// of scratch, creating or growing it if needed.
+// of scratch, creating or growing it if needed.  A workspace in memory lent by the caller is
+// never grown: HASTE_HIP_ERROR_UNSUPPORTED_SIZE (and the size needed in the error text) when
+// it is too small.
 int get_workspace(hipStream_t stream, size_t scratch_bytes, Workspace* out);
 
 // Reserves `count` consecutive step-flag values on the workspace of (current device,
@@ -83,15 +91,31 @@ int check_and_clear_abort(hipStream_t stream, Workspace* ws);
 
 int device_cu_count();
 
+// XCDs of the current device on which a launch of one workgroup per CU puts equally many
+// workgroups each -- found by running such a launch once per device (a probe kernel that
+// records where each workgroup ran) -- or 0 when the placement is not that regular (a
+// partition mode or a CU mask the probe does not understand), when HASTE_HIP_XCD_LOCAL=0, or
+// after a launch found more workgroups on an XCD than it had been promised: the persistent
+// kernels then take the cross-XCD path.  xcc_logical_map: 4 bits per hardware XCC id, its
+// index among the XCDs in use.
+int device_xcd_count();
+unsigned long long device_xcc_logical_map();
+
 // Keeps the persistent kernels of this process on one device in a single order even when
 // they are launched on different streams.  before == true: makes `stream` wait for the
 // previous persistent kernel (if it ran on another stream); before == false: records the
 // kernel just enqueued on `stream` as the one to wait for.
 int order_persistent_launches(hipStream_t stream, bool before);
 
-// False when the environment variable HASTE_HIP_XCD_LOCAL is set to 0 (forces the
-// cross-XCD exchange path; for experiments).
-bool xcd_local_enabled();
+// Polls before a bounded wait of a persistent kernel gives up: 2^24 (seconds), or the value of
+// the environment variable HASTE_HIP_SPIN_LIMIT.
+unsigned int spin_limit();
+
+// Number of workgroups every group barrier also waits for although no workgroup plays them: 0,
+// or the value of the environment variable HASTE_HIP_TEST_ABSENT_WORKGROUP.  Only the test of
+// the time-out path sets it, together with a small spin limit: the waits then run out, the
+// kernel reports it and every wavefront still reaches the end of the kernel.
+int test_absent_workgroups();
 
 // False when the environment variable HASTE_HIP_PAIRED_SETS is set to 0: 8- and 16-row
 // batch tiles then run as one tile instead of two sets of half the rows (for experiments).

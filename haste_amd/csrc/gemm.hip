@@ -457,8 +457,10 @@ GemmPlan plan_gemm(int M, int N, int K) {
       if (s > 1) c += 0.25 * (double)g.rest * s / K;
       return c;
     };
+    // At most four pieces per CU: that bounds the partial tiles of any product (64 KiB a
+    // piece) by a size callers who lend the library its scratch memory can plan for.
     double best = cost(1);
-    for (int s = 2; s <= s_max; ++s)
+    for (int s = 2; s <= s_max && (long long)g.rest * s <= 4LL * cus; ++s)
       if (cost(s) < best - 1e-9) { best = cost(s); splits = s; }
   }
   g.k_per_split = (K + splits - 1) / splits;
@@ -564,7 +566,7 @@ int gemm_f32_pair(hipStream_t stream, int M1, int M2, int N, int K, const float*
   };
   int splits = 1;
   double best = cost(1);
-  for (int s = 2; s <= s_max; ++s)
+  for (int s = 2; s <= s_max && tiles * s <= 4LL * cus; ++s)
     if (cost(s) < best - 1e-9) { best = cost(s); splits = s; }
   int k_per_split = (K + splits - 1) / splits;
   k_per_split = (k_per_split + BK - 1) / BK * BK;

@@ -23,7 +23,6 @@ namespace haste_hip {
 
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
-constexpr unsigned int kSpinLimit = 1u << 24;  // polls before a barrier wait gives up
 
 // Gate nonlinearities on the hardware exp2 and reciprocal (about 1 ulp each): absolute
 // error around 1e-7, the size of one fp32 rounding of the result.
@@ -99,6 +98,9 @@ struct LaunchShape {
   int tile_rows;               // batch rows per group (the kernel's NB)
   int xcd_local;               // 1: group g is the set of workgroups running on XCD g
   int per_xcd;                 // workgroups this launch places on every XCD (xcd_local)
+  unsigned long long xcc_map;  // 4 bits per hardware XCC id: which group runs there (xcd_local)
+  int absent;                  // workgroups the barriers wait for although nobody plays them
+                               // (0 except in the test of the time-out path)
 };
 
 // The part of the problem a workgroup works on.
@@ -137,7 +139,7 @@ __device__ __forceinline__ Role take_role(const LaunchShape& ls, unsigned int* w
       __hip_atomic_store(ls.host_status, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
       *word = 0xffffffffu;
     } else {
-      *word = (xcc << 16) | ticket;
+      *word = ((unsigned int)((ls.xcc_map >> (4 * xcc)) & 0xfull) << 16) | ticket;
     }
   }
   __syncthreads();
@@ -168,7 +170,7 @@ __device__ __forceinline__ void group_sync_init(GroupSync& g, const LaunchShape&
   g.flags = &ls.cb->step_flags[r.bt * ls.gx];
   g.abort_flag = &ls.cb->abort_flag[0];
   g.host_status = ls.host_status;
-  g.group_size = (unsigned int)ls.gx;
+  g.group_size = (unsigned int)(ls.gx + ls.absent);
   g.my_index = (unsigned int)r.cw;
   g.epoch = ls.epoch;
   g.arrivals = 0;
@@ -1195,28 +1197,29 @@ struct LaunchPlan {
   int threads = 256;  // 512: two 256-thread sets per workgroup
 };
 
-constexpr int kXcdCount = 8;
-
 inline bool xcd_local_fits(int gx, int gy) {
-  const int cus = device_cu_count();
-  return xcd_local_enabled() && cus % kXcdCount == 0 && gy <= kXcdCount && gx <= cus / kXcdCount;
+  const int cus = device_cu_count(), xcds = device_xcd_count();
+  return xcds > 0 && cus % xcds == 0 && gy <= xcds && gx <= cus / xcds;
 }
 
 inline int plan_launch(hipStream_t stream, const Workspace& ws, int gx, int gy, int tile_rows,
                        size_t lds_bytes, unsigned int epochs, LaunchPlan* plan) {
   plan->shape.cb = ws.control;
   plan->shape.host_status = ws.host_status_dev;
-  plan->shape.spin_limit = kSpinLimit;
+  plan->shape.spin_limit = spin_limit();
+  plan->shape.absent = test_absent_workgroups();
   plan->shape.gx = gx;
   plan->shape.gy = gy;
   plan->shape.tile_rows = tile_rows;
   plan->shape.ticket_base = 0;
   plan->shape.per_xcd = 0;
+  plan->shape.xcc_map = 0;
   HASTE_HIP_PROPAGATE(reserve_epochs(stream, epochs, &plan->shape.epoch));
-  if (xcd_local_fits(gx, gy)) {
-    const int cus = device_cu_count();
+  const int cus = device_cu_count(), xcds = device_xcd_count();
+  if (xcds > 0 && cus % xcds == 0 && gy <= xcds && gx <= cus / xcds) {
     plan->shape.xcd_local = 1;
-    plan->shape.per_xcd = cus / kXcdCount;
+    plan->shape.per_xcd = cus / xcds;
+    plan->shape.xcc_map = device_xcc_logical_map();
     HASTE_HIP_PROPAGATE(reserve_tickets(stream, (unsigned)plan->shape.per_xcd, &plan->shape.ticket_base));
     plan->grid = dim3((unsigned)cus);
     const size_t one_per_cu = 84 * 1024;  // more than half of a CU's LDS

@@ -39,6 +39,67 @@ def _call(entry, *args):
     lib.call(name, *args)
 
 
+def stream_status(stream=None):
+    """After the caller has synchronized `stream` (default: the current stream): raises
+    lib.HasteHipError when a persistent kernel launched on it gave up a bounded wait (its
+    outputs, and those of library kernels queued behind it, are invalid); see
+    haste_hip_stream_status in include/haste_hip.h."""
+    import ctypes
+    handle = lib.load()
+    if stream is None:
+        stream = torch.cuda.current_stream().cuda_stream
+    handle.haste_hip_stream_status.restype = ctypes.c_int
+    rc = handle.haste_hip_stream_status(ctypes.c_void_p(stream))
+    if rc != 0:
+        raise lib.HasteHipError(rc, "haste_hip_stream_status")
+
+
+def workspace_bytes(time_steps, batch_size, input_size, hidden_size):
+    """Upper bound of the scratch memory any cell needs for these sizes on the current device."""
+    import ctypes
+    handle = lib.load()
+    handle.haste_hip_workspace_bytes.restype = ctypes.c_size_t
+    handle.haste_hip_workspace_bytes.argtypes = [ctypes.c_int] * 4
+    return int(handle.haste_hip_workspace_bytes(time_steps, batch_size, input_size, hidden_size))
+
+
+def set_workspace(buffer, stream=None):
+    """Lends the library `buffer` (a contiguous GPU tensor from torch's allocator, which the
+    caller keeps alive and leaves alone) as the scratch memory of `stream` (default: the current
+    stream); None takes it back.  With a lent buffer the ops allocate, free and synchronize
+    nothing themselves, so they can be recorded into a HIP graph."""
+    import ctypes
+    handle = lib.load()
+    if stream is None:
+        stream = torch.cuda.current_stream().cuda_stream
+    handle.haste_hip_set_workspace.restype = ctypes.c_int
+    handle.haste_hip_set_workspace.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]
+    if buffer is None:
+        rc = handle.haste_hip_set_workspace(ctypes.c_void_p(stream), None, 0)
+    else:
+        if not (buffer.is_cuda and buffer.is_contiguous()):
+            raise ValueError("the workspace must be a contiguous GPU tensor")
+        rc = handle.haste_hip_set_workspace(ctypes.c_void_p(stream), ctypes.c_void_p(buffer.data_ptr()),
+                                            buffer.numel() * buffer.element_size())
+    if rc != 0:
+        raise lib.HasteHipError(rc, "haste_hip_set_workspace")
+
+
+def workspace_high_water(stream=None):
+    """Bytes of scratch memory the calls made on `stream` so far have needed (what to lend for
+    a replay of the same calls)."""
+    import ctypes
+    handle = lib.load()
+    if stream is None:
+        stream = torch.cuda.current_stream().cuda_stream
+    out = ctypes.c_size_t(0)
+    handle.haste_hip_workspace_high_water.restype = ctypes.c_int
+    rc = handle.haste_hip_workspace_high_water(ctypes.c_void_p(stream), ctypes.byref(out))
+    if rc != 0:
+        raise lib.HasteHipError(rc, "haste_hip_workspace_high_water")
+    return int(out.value)
+
+
 def _zeros(opts, *shapes):
     """Zero tensors of the given shapes carved out of one allocation: one fill kernel for all
     the accumulated outputs of a backward pass (each starts on a 256-byte boundary)."""

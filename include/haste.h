@@ -9,11 +9,14 @@
 // fastest; every pointer is device memory and non-null unless stated otherwise.
 //
 // Differences a caller can observe:
-//  * only T = float is implemented;
+//  * T = float and T = double for every class, T = __half for the GRU, as in the
+//    reference (the persistent MFMA kernels are float; double and half run step-wise);
 //  * all work is enqueued on the stream given to the constructor (0 = the null
 //    stream) and completes in stream order; destructors never block;
 //  * the BLAS handle is accepted and ignored (the library has its own MFMA GEMM);
 //  * Run() reports failures through last_status() instead of silently ignoring them;
+//    failures inside a kernel (a bounded wait that ran out) are reported by
+//    stream_status(), to be called after synchronizing the stream;
 //  * layer_norm::BackwardPass recomputes the row statistics, its cache is not read
 //    except by the fused LayerNormLSTM/GRU kernels.
 #pragma once

@@ -40,6 +40,9 @@ class ForwardPass {
     }
 
     int last_status() const { return data_.status; }
+    // After the caller has synchronized the stream: HASTE_HIP_OK, or the error of a kernel of
+    // this stream that gave up a bounded wait (see haste_hip_stream_status).
+    int stream_status() const { return haste_hip_stream_status(detail::stream_arg(data_.stream)); }
 
   private:
     detail::PassState data_;
@@ -84,6 +87,9 @@ class BackwardPass {
     }
 
     int last_status() const { return data_.status; }
+    // After the caller has synchronized the stream: HASTE_HIP_OK, or the error of a kernel of
+    // this stream that gave up a bounded wait (see haste_hip_stream_status).
+    int stream_status() const { return haste_hip_stream_status(detail::stream_arg(data_.stream)); }
 
   private:
     detail::PassState data_;

@@ -77,6 +77,9 @@ class ForwardPass {
 
     // HASTE_HIP_OK or the error code of the last Run()/Iterate().
     int last_status() const { return data_.status; }
+    // After the caller has synchronized the stream: HASTE_HIP_OK, or the error of a kernel of
+    // this stream that gave up a bounded wait (see haste_hip_stream_status).
+    int stream_status() const { return haste_hip_stream_status(detail::stream_arg(data_.stream)); }
 
   private:
     detail::PassState data_;
@@ -157,6 +160,9 @@ class BackwardPass {
     }
 
     int last_status() const { return data_.status; }
+    // After the caller has synchronized the stream: HASTE_HIP_OK, or the error of a kernel of
+    // this stream that gave up a bounded wait (see haste_hip_stream_status).
+    int stream_status() const { return haste_hip_stream_status(detail::stream_arg(data_.stream)); }
 
   private:
     detail::PassState data_;

@@ -16,6 +16,8 @@
 #ifndef HASTE_HIP_H_
 #define HASTE_HIP_H_
 
+#include <stddef.h>
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -45,6 +47,41 @@ int haste_hip_max_hidden_size(int gates, int batch_size);
 /* Drops this thread's cached per-stream workspaces on the current device (frees
  * device memory; the caller must have synchronized the streams that used them). */
 int haste_hip_release_workspaces(void);
+
+/* Status of the persistent kernels launched on `stream` so far; call it after synchronizing
+ * the stream.  HASTE_HIP_OK, or HASTE_HIP_ERROR_STEP_BARRIER when one of them gave up (a
+ * bounded wait for another workgroup ran out, or an XCD hosted more workgroups than the launch
+ * had been promised): the outputs of that launch, and of library launches that were already
+ * queued behind it on the device, are invalid, although the calls that enqueued them returned
+ * HASTE_HIP_OK (they return before the kernels run).  Reporting clears the condition (the
+ * control block is wiped in stream order; after an XCD placement failure later launches use
+ * the placement-independent exchange path) and haste_hip_last_runtime_error() says which of
+ * the two it was.  Without this call the condition is reported by the next entry point
+ * called on the stream.  The reference has no error reporting to replace (its Run methods
+ * return void). */
+int haste_hip_stream_status(void* stream);
+
+/* Caller-owned scratch memory.  By default the library keeps one workspace per (device,
+ * stream) that it allocates on first use and grows on demand (hipMalloc, and on growth a
+ * stream synchronization and hipFree, inside Run).  A caller who wants every byte in its
+ * own allocator, or who records calls into a HIP graph, lends the stream a buffer instead:
+ * `memory` is device memory, 256-byte aligned, of `bytes` bytes, which stays valid and is
+ * used by nothing else until it is replaced or taken back (memory == NULL: back to a
+ * library-owned workspace); the call synchronizes `stream` if the stream has a workspace in
+ * use.  With a lent buffer no entry point allocates, frees or synchronizes; a call that needs
+ * more than `bytes` returns HASTE_HIP_ERROR_UNSUPPORTED_SIZE (the size in
+ * haste_hip_last_runtime_error()) before it launches anything that uses the workspace.
+ * The reference's contract being honoured: every buffer, tmp_Rh included, is the caller's
+ * (lib/haste/lstm.h:98-117).
+ *
+ * haste_hip_workspace_bytes: an upper bound of what any cell, direction and scalar type
+ * needs for (T, N, C, H) on the current device (for the stand-alone layer norm: T = 1,
+ * N = rows, C = H = dim): 64 MiB for the partial tiles of split GEMMs plus terms in N*H,
+ * H*H and T*N.  haste_hip_workspace_high_water: what the calls made on `stream` so far
+ * have actually needed (after a rehearsal of the same calls, the exact size to lend). */
+size_t haste_hip_workspace_bytes(int time_steps, int batch_size, int input_size, int hidden_size);
+int haste_hip_set_workspace(void* stream, void* memory, size_t bytes);
+int haste_hip_workspace_high_water(void* stream, size_t* bytes);
 
 /* Makes everything enqueued on `then` after this call wait for everything enqueued on
  * `first` before it (an event recorded on `first`, waited for on `then`); no-op when both
