@@ -484,9 +484,51 @@ size_t gemm_f32_scratch_bytes(int M, int N, int K) {
   return tiled > skinny ? tiled : skinny;
 }
 
+namespace {
+int gemm_f32_once(hipStream_t stream, bool trans_a, int M, int N, int K,
+                  const float* A, int lda, const float* B, int ldb,
+                  float* C, int ldc, bool accumulate, size_t scratch_offset);
+}  // namespace
+
+// A workgroup of the tile kernel addresses its operand panels (its rows of A, its columns of
+// B, all of K) with 32-bit byte offsets, so a panel must stay under 2 GiB.  A longer
+// contraction -- the dW and dR products of a backward pass contract over T*N with rows of 4H
+// floats, 2 GiB from T*N*H = 2^27 on -- is cut into runs of K that fit, each accumulating into
+// C; where the cuts fall depends on the shape only.
 int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
              const float* A, int lda, const float* B, int ldb,
              float* C, int ldc, bool accumulate, size_t scratch_offset) {
+  HASTE_HIP_REQUIRE(M > 0 && N > 0 && K > 0);
+  HASTE_HIP_REQUIRE(A != nullptr && B != nullptr && C != nullptr);
+  HASTE_HIP_REQUIRE(lda >= (trans_a ? M : K) && ldb >= N && ldc >= N);
+  const long long limit = (1ll << 29) - 256;  // floats a panel may span
+  long long run = (limit - BN) / ldb;
+  if (trans_a) {
+    const long long a_run = (limit - 128) / lda;
+    run = a_run < run ? a_run : run;
+  } else if (128ll * lda + K >= limit) {
+    run = 0;  // 128 rows of A alone exceed the limit
+  }
+  if (run >= K) return gemm_f32_once(stream, trans_a, M, N, K, A, lda, B, ldb, C, ldc, accumulate, scratch_offset);
+  run = run / 1024 * 1024;
+  if (run <= 0) {
+    set_error_text("gemm: a row of an operand is too long for the kernel's 32-bit panel offsets "
+                   "(leading dimension of 2^19 floats or more per 1024 rows)");
+    return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  }
+  for (long long k0 = 0; k0 < K; k0 += run) {
+    const int kc = (int)(K - k0 < run ? K - k0 : run);
+    const float* a = trans_a ? A + (size_t)k0 * lda : A + k0;
+    HASTE_HIP_PROPAGATE(gemm_f32_once(stream, trans_a, M, N, kc, a, lda, B + (size_t)k0 * ldb, ldb, C, ldc,
+                                      accumulate || k0 > 0, scratch_offset));
+  }
+  return HASTE_HIP_OK;
+}
+
+namespace {
+int gemm_f32_once(hipStream_t stream, bool trans_a, int M, int N, int K,
+                  const float* A, int lda, const float* B, int ldb,
+                  float* C, int ldc, bool accumulate, size_t scratch_offset) {
   HASTE_HIP_REQUIRE(M > 0 && N > 0 && K > 0);
   HASTE_HIP_REQUIRE(A != nullptr && B != nullptr && C != nullptr);
   HASTE_HIP_REQUIRE(lda >= (trans_a ? M : K) && ldb >= N && ldc >= N);
@@ -534,6 +576,7 @@ int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,
   }
   return HASTE_HIP_OK;
 }
+}  // namespace
 
 // C1[M1,N] (+)= A1[M1,K] * B1 and C2[M2,N] (+)= A2^T * B2 (A2 stored [K,M2]) in one launch when
 // together they have fewer tiles than the chip has CUs (then each alone would be cut into

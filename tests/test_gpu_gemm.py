@@ -86,3 +86,30 @@ def test_transpose(shape):
     out = ops.transpose(a)
     ref = a.reshape(-1, shape[-1]).t().contiguous().reshape((shape[-1],) + tuple(shape[:-1]))
     assert out.shape == ref.shape and torch.equal(out, ref)
+
+
+@pytest.mark.parametrize("trans_a", [True, False])
+def test_gemm_operand_of_more_than_2_gib(trans_a):
+    """B[K, N] of 2.1 GB (the dv of a backward pass with T*N*H = 2^27 and beyond: dW = x^T dv
+    contracts over T*N): the contraction is cut into runs whose panels the kernel can address.
+    Against the float64 product of the same float32 operands, on the GPU (NumPy would take
+    minutes)."""
+    import torch
+    from haste_amd import ops
+    M, N, K = 256, 2048, (1 << 18) + 48
+    g = torch.Generator(device="cuda").manual_seed(5)
+    a = torch.randn((K, M) if trans_a else (M, K), generator=g, device="cuda")
+    b = torch.randn(K, N, generator=g, device="cuda")
+    assert b.numel() * 4 > 1 << 31
+    print("gemm over 2 GiB, trans_a =", trans_a, flush=True)
+    c0 = torch.randn(M, N, generator=g, device="cuda")
+    out = c0.clone()
+    ops.gemm(a, b, out=out, trans_a=trans_a, accumulate=True)
+    torch.cuda.synchronize()
+    ref = c0.double()
+    step = 1 << 15   # float64 copies of the operands, a slab of K at a time
+    for k0 in range(0, K, step):
+        a_slab = (a[k0:k0 + step].double().t() if trans_a else a[:, k0:k0 + step].double())
+        ref += a_slab @ b[k0:k0 + step].double()
+    err = float((out.double() - ref).abs().max() / ref.abs().max())
+    assert err < 1e-5, err
