@@ -38,7 +38,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget", type=float, default=15.0)
-    ap.add_argument("--workload", choices=["all", "metric", "streaming", "stepwise", "hbm_kernels", "copy", "configs"],
+    ap.add_argument("--workload", choices=["all", "metric", "streaming", "stepwise", "hbm_kernels", "copy", "configs",
+                                           "peak", "iterate"],
                     default="all",
                     help="restrict the run to one workload (for profiling); the JSON line is "
                          "only complete with 'all'.  'copy' runs a plain device copy of known "
@@ -147,10 +148,15 @@ def run_metric(args, torch, lib, ops, dev):
         step()
     torch.cuda.synchronize()
     lib.haste_hip_profile_enable(0)
-    f_gemm = 2.0 * T * N * C * 4 * H  # each of the 4 GEMMs (C == H)
-    f_rec = 2.0 * T * N * H * 4 * H
+    f_gemm = 2.0 * T * N * C * 4 * H  # each of the 4 products x*W, dx, dW, dR (C == H)
+    f_rec = 2.0 * T * N * H * 4 * H   # h*R over all steps, forward or backward
+    gemm_ms, gemm_count = profile_read(lib, "gemm_f32")
+    # With 4-row batch tiles the forward recurrence computes x*W itself: the step then has
+    # three GEMM products instead of four and the forward kernel does the flops of two.
+    fused_input = round(gemm_count / args.steps) == 3
     kernels = {}
-    for name, flops in (("gemm_f32", f_gemm), ("lstm_forward_recurrence", f_rec),
+    for name, flops in (("gemm_f32", f_gemm),
+                        ("lstm_forward_recurrence", f_rec + (f_gemm if fused_input else 0.0)),
                         ("lstm_backward_recurrence", f_rec)):
         total_ms, count = profile_read(lib, name)
         avg_ms = total_ms / max(count, 1)
@@ -159,17 +165,80 @@ def run_metric(args, torch, lib, ops, dev):
                          "ms_per_step": round(total_ms / args.steps, 5),
                          "flops_per_launch": flops, "tflops": round(tf, 3),
                          "frac_of_fp32_mfma_peak": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)}
+    if fused_input:
+        kernels["lstm_forward_recurrence"]["computes_input_projection"] = True
     lib.haste_hip_profile_reset()
-    dominant = max(kernels, key=lambda k: kernels[k]["ms_per_step"])
+    # The roofline entry is the kernel with the longest single launch (a recurrence), with the
+    # whole step beside it: all six products of the step, 2*T*N*4H*(3C + 3H) flops, over the
+    # step's wall time.
+    total_flops = 3.0 * (f_gemm + f_rec)
+    tflops_whole = total_flops / (ms_per_step * 1e-3) / 1e12
+    dominant = max(kernels, key=lambda k: kernels[k]["avg_ms"])
     dom = kernels[dominant]
     roofline = {"kernel": dominant, "bound": "mfma", "achieved": dom["tflops"],
                 "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(dom["tflops"] / PEAK_FP32_MFMA_TFLOPS, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES.get(dominant)}
-    total_flops = 3.0 * (f_gemm + f_rec)
+                "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
+                "us_per_launch": round(dom["avg_ms"] * 1e3, 2),
+                "whole_step_tflops": round(tflops_whole, 3),
+                "whole_step_frac": round(tflops_whole / PEAK_FP32_MFMA_TFLOPS, 4)}
     return dict(ms_per_step=ms_per_step, ms_per_ops_step=ms_per_ops_step, kernels=kernels, roofline=roofline,
-                tflops_whole_step=total_flops / (ms_per_step * 1e-3) / 1e12,
-                host=(W, R, b, x, dy))
+                tflops_whole_step=tflops_whole, host=(W, R, b, x, dy))
+
+
+def run_measured_peak(args, torch, lib, ops, dev):
+    """What the fp32 matrix cores deliver on this box on a long, square product (the library's
+    own GEMM at 8192^3), beside the nominal 157.3 TFLOP/s the fractions are quoted against."""
+    n = 8192
+    a = torch.randn(n, n, device=dev)
+    b = torch.randn(n, n, device=dev)
+    out = torch.empty(n, n, device=dev)
+    for _ in range(2):
+        ops.gemm(a, b, out=out)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    reps = 5
+    e0.record()
+    for _ in range(reps):
+        ops.gemm(a, b, out=out)
+    e1.record()
+    torch.cuda.synchronize()
+    tf = 2.0 * n ** 3 / (e0.elapsed_time(e1) / reps * 1e-3) / 1e12
+    return {"workload": "gemm_f32 8192 x 8192 x 8192", "tflops": round(tf, 2),
+            "frac_of_nominal": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)}
+
+
+def run_iterate(args, torch, lib, ops, dev):
+    """Single steps through the Iterate entry points (the reference's autoregressive API,
+    lib/haste/lstm.h:73-86): microseconds per call, N=1, C=H=512, inference, end to end on
+    preallocated buffers (the state ping-pongs between two pairs)."""
+    from haste_amd import lib as hlib
+    N, C, H = 1, 512, 512
+    g = torch.Generator(device="cpu").manual_seed(3)
+    k = H ** -0.5
+    W = ((torch.rand(C, 4 * H, generator=g) * 2 - 1) * k).to(dev)
+    R = ((torch.rand(H, 4 * H, generator=g) * 2 - 1) * k).to(dev)
+    b = torch.zeros(4 * H, device=dev)
+    x = torch.randn(N, C, generator=g).to(dev)
+    hs = [torch.zeros(N, H, device=dev), torch.zeros(N, H, device=dev)]
+    cs = [torch.zeros(N, H, device=dev), torch.zeros(N, H, device=dev)]
+    v = torch.empty(N, 4 * H, device=dev)
+
+    def call(i):
+        hlib.call("haste_hip_lstm_forward_iterate_f32", False, N, C, H, W, R, b, x, hs[i & 1], cs[i & 1],
+                  hs[(i + 1) & 1], cs[(i + 1) & 1], v, None, 0.0, None)
+    for i in range(20):
+        call(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    reps = 400
+    e0.record()
+    for i in range(reps):
+        call(i)
+    e1.record()
+    torch.cuda.synchronize()
+    return {"workload": "LSTM Iterate N=1 C=H=512 fp32 inference, %d calls back to back" % reps,
+            "us_per_call": round(e0.elapsed_time(e1) * 1e3 / reps, 3)}
 
 
 def run_streaming(args, torch, lib, ops, dev):
@@ -445,6 +514,12 @@ def main():
     if args.workload == "stepwise":
         print(json.dumps(run_stepwise(args, torch, lib, ops, dev)))
         return
+    if args.workload == "peak":
+        print(json.dumps(run_measured_peak(args, torch, lib, ops, dev)))
+        return
+    if args.workload == "iterate":
+        print(json.dumps(run_iterate(args, torch, lib, ops, dev)))
+        return
     if args.workload == "hbm_kernels":
         print(json.dumps(run_hbm_kernels(args, torch, lib, ops, dev)))
         return
@@ -453,6 +528,11 @@ def main():
     streaming, host1 = run_streaming(args, torch, lib, ops, dev)
     stepwise = run_stepwise(args, torch, lib, ops, dev)
     hbm_kernels = run_hbm_kernels(args, torch, lib, ops, dev)
+    configs = run_configs(args, torch, lib, ops, dev)
+    measured_peak = run_measured_peak(args, torch, lib, ops, dev)
+    iterate = run_iterate(args, torch, lib, ops, dev)
+    m["roofline"]["measured_peak"] = measured_peak["tflops"]
+    m["roofline"]["frac_of_measured_peak"] = round(m["roofline"]["achieved"] / measured_peak["tflops"], 4)
 
     # CPU baseline: torch.nn.LSTM fwd+bwd on the host cores (bounded sample).
     cpu = None
@@ -461,14 +541,22 @@ def main():
         W, R, b, x, dy = m["host"]
         W1, R1, b1, x1 = host1
         threads = torch.get_num_threads()
-        sec, iters = cpu_baseline.time_lstm_fwd_bwd(W, R, b, x, dy, budget_s=args.cpu_budget)
-        sec1, it1 = cpu_baseline.time_lstm_inference(W1, R1, b1, x1[:500], budget_s=5.0)
-        cpu = {"value": round(sec * 1e3, 3), "unit": "ms/batch", "cores": threads, "kind": "port",
+        t = cpu_baseline.time_lstm_fwd_bwd(W, R, b, x, dy, budget_s=args.cpu_budget)
+        t1 = cpu_baseline.time_lstm_inference(W1, R1, b1, x1[:500], budget_s=4.0)
+        torch.set_num_threads(1)
+        t1_single = cpu_baseline.time_lstm_inference(W1, R1, b1, x1[:500], budget_s=4.0)
+        torch.set_num_threads(threads)
+        cpu = {"value": round(t["median"] * 1e3, 3), "min": round(t["min"] * 1e3, 3), "unit": "ms/batch",
+               "cores": threads, "kind": "port", "cpu_model": cpu_baseline.cpu_model(),
                "sample": "torch.nn.LSTM fwd+bwd fp32 on host CPU, same weights via the native "
-                         "weight map, N=64 T=100 C=H=512, median of %d iterations; "
-                         "os.cpu_count=%d" % (iters, os.cpu_count()),
-               "n1_us_per_timestep": round(sec1 * 1e6 / 500, 3),
-               "n1_sample": "torch.nn.LSTM inference N=1, first 500 of 2000 steps, median of %d" % it1}
+                         "weight map, N=64 T=100 C=H=512, median (and minimum) of %d iterations; "
+                         "os.cpu_count=%d" % (t["iterations"], os.cpu_count()),
+               "n1_us_per_timestep": round(t1["median"] * 1e6 / 500, 3),
+               "n1_us_per_timestep_min": round(t1["min"] * 1e6 / 500, 3),
+               "n1_us_per_timestep_one_thread": round(t1_single["median"] * 1e6 / 500, 3),
+               "n1_us_per_timestep_one_thread_min": round(t1_single["min"] * 1e6 / 500, 3),
+               "n1_sample": "torch.nn.LSTM inference N=1, first 500 of 2000 steps, %d threads: median "
+                            "of %d; one thread: median of %d" % (threads, t1["iterations"], t1_single["iterations"])}
 
     out = {
         "metric": "LSTM fwd+bwd ms/batch (N=64,T=100,H=512 fp32)",
@@ -486,6 +574,9 @@ def main():
         "streaming_n1": streaming,
         "stepwise_n1_h4096": stepwise,
         "hbm_kernels": hbm_kernels,
+        "other_configs_ms": configs,
+        "measured_fp32_mfma_peak": measured_peak,
+        "iterate_n1": iterate,
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))

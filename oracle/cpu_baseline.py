@@ -26,7 +26,7 @@ def native_lstm(W, R, b):
 
 
 def time_lstm_fwd_bwd(W, R, b, x, dy, budget_s=15.0, warmup=2, min_iters=3):
-    """Median seconds of torch.nn.LSTM forward + backward on CPU, fp32."""
+    """Median and minimum seconds of torch.nn.LSTM forward + backward on CPU, fp32."""
     m = native_lstm(W, R, b)
     xt = torch.from_numpy(x.astype(np.float32)).requires_grad_()
     dyt = torch.from_numpy(dy.astype(np.float32))
@@ -47,11 +47,11 @@ def time_lstm_fwd_bwd(W, R, b, x, dy, budget_s=15.0, warmup=2, min_iters=3):
             break
         if len(times) >= 50:
             break
-    return float(np.median(times)), len(times)
+    return {"median": float(np.median(times)), "min": float(np.min(times)), "iterations": len(times)}
 
 
 def time_lstm_inference(W, R, b, x, budget_s=10.0, warmup=1, min_iters=3):
-    """Median seconds of torch.nn.LSTM forward (no grad) on CPU, fp32."""
+    """Median and minimum seconds of torch.nn.LSTM forward (no grad) on CPU, fp32."""
     m = native_lstm(W, R, b)
     xt = torch.from_numpy(x.astype(np.float32))
     times = []
@@ -69,4 +69,17 @@ def time_lstm_inference(W, R, b, x, budget_s=10.0, warmup=1, min_iters=3):
                 break
             if len(times) >= 50:
                 break
-    return float(np.median(times)), len(times)
+    return {"median": float(np.median(times)), "min": float(np.min(times)), "iterations": len(times)}
+
+
+def cpu_model():
+    """Model name of the host CPU (/proc/cpuinfo), or the platform's processor string."""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    import platform
+    return platform.processor() or "unknown"
