@@ -237,8 +237,40 @@ def run_iterate(args, torch, lib, ops, dev):
         call(i)
     e1.record()
     torch.cuda.synchronize()
-    return {"workload": "LSTM Iterate N=1 C=H=512 fp32 inference, %d calls back to back" % reps,
-            "us_per_call": round(e0.elapsed_time(e1) * 1e3 / reps, 3)}
+    out = {"workload": "LSTM Iterate N=1 C=H=512 fp32 inference, %d calls back to back" % reps,
+           "us_per_call": round(e0.elapsed_time(e1) * 1e3 / reps, 3)}
+
+    # The same calls recorded into a HIP graph (the stream's scratch memory lent by the caller,
+    # so that nothing allocates under capture) and replayed: what a decoding loop that replays a
+    # captured chunk of steps pays per step.
+    chunk = 100
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        lent = torch.empty(ops.workspace_bytes(1, N, C, H), dtype=torch.uint8, device=dev)
+        ops.set_workspace(lent)
+        try:
+            for i in range(4):
+                call(i)
+            side.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(chunk):
+                    call(i)
+            graph.replay()
+            side.synchronize()
+            g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            g0.record()
+            for _ in range(10):
+                graph.replay()
+            g1.record()
+            side.synchronize()
+            out["us_per_call_graph_replay"] = round(g0.elapsed_time(g1) * 1e3 / (10 * chunk), 3)
+            out["graph"] = "%d calls per graph, 10 replays" % chunk
+            del graph
+        finally:
+            side.synchronize()
+            ops.set_workspace(None)
+    return out
 
 
 def run_streaming(args, torch, lib, ops, dev):

@@ -222,6 +222,19 @@ int layer_norm_gru_backward_streamed(hipStream_t stream, int T, int N, int C, in
                                      float* dgamma2, const float* cache2,
                                      const float* zoneout_mask);
 
+// One forward step for a batch of at most 8 rows as a single kernel (single_step.hip): what the
+// Iterate entry points and one-step Run calls use.
+bool single_step_applies(int N, int C, int H);
+int lstm_forward_single_step(hipStream_t stream, int training, int N, int C, int H, const float* W,
+                             const float* R, const float* b, const float* x, const float* h,
+                             const float* c, float* h_out, float* c_out, float* v,
+                             float zoneout_prob, const float* zoneout_mask, const float* dc_mask,
+                             float dc_scale);
+int gru_forward_single_step(hipStream_t stream, int training, int N, int C, int H, const float* W,
+                            const float* R, const float* bx, const float* br, const float* x,
+                            const float* h, float* h_out, float* v, float zoneout_prob,
+                            const float* zoneout_mask, const float* dc_mask, float dc_scale);
+
 // The same for rows too wide for layer_norm.hip's row-in-registers kernels (stepwise.hip).
 int layer_norm_forward_wide(hipStream_t stream, int rows, int dim, const float* gamma,
                             const float* beta, const float* x, float* y, float* cache);

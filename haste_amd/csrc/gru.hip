@@ -617,6 +617,11 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
   HASTE_HIP_REQUIRE(W && R && bx && br && x && h && h_out && tmp_Wx);
   HASTE_HIP_REQUIRE(!training || v != nullptr);
+  // A single step of a small batch (Iterate): one kernel, nothing kept on chip (tmp_Wx is
+  // scratch of the other paths and is left alone).
+  if (T == 1 && single_step_applies(N, C, H))
+    return gru_forward_single_step(stream, training, N, C, H, W, R, bx, br, x, h, h_out, v,
+                                   zoneout_prob, zoneout_mask, dc_mask, dc_scale);
   if (N == 1 && H <= 512 && xcd_local_fits((H + 15) / 16, 1) && single_row_enabled())
     return gru_forward_single_row(stream, training, T, C, H, W, R, bx, br, x, h, h_out, v, tmp_Wx,
                                   zoneout_prob, zoneout_mask, dc_mask, dc_scale);

@@ -648,6 +648,10 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
                       float dc_scale) {
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
   HASTE_HIP_REQUIRE(W && R && b && x && h && c && h_out && c_out && v);
+  // A single step of a small batch (Iterate): one kernel, nothing kept on chip.
+  if (T == 1 && single_step_applies(N, C, H))
+    return lstm_forward_single_step(stream, training, N, C, H, W, R, b, x, h, c, h_out, c_out, v,
+                                    zoneout_prob, zoneout_mask, dc_mask, dc_scale);
   if (N == 1 && H <= 512 && xcd_local_fits((H + 15) / 16, 1) && single_row_enabled())
     return lstm_forward_single_row(stream, training, T, C, H, W, R, b, x, h, c, h_out, c_out, v,
                                    zoneout_prob, zoneout_mask, dc_mask, dc_scale);

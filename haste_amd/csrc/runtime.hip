@@ -546,6 +546,9 @@ size_t haste_hip_workspace_bytes(int time_steps, int batch_size, int input_size,
   // buffers; the stand-alone layer norm's column sums (two workgroups per CU, two rows each).
   b += (N * 4 * H + H * 4 * H + 128 * widest + T * N * 2 + 2 * N * H) * 8 + 16 * 256;
   b += 2 * cus * 2 * widest * sizeof(float);
+  // Single forward steps: partial sums of at most 64 runs of the contraction, both sides, for 8
+  // rows and every gate column, and the staged state.
+  b += 64 * 2 * 8 * (H / 16 + 1) * 64 * sizeof(float) + 8 * H * sizeof(float) + 256;
   return kControlBytes + 4096 + (b + 255) / 256 * 256;
 }
 
