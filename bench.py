@@ -22,10 +22,10 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch at the metric workload, from two rocprofv3 --pmc runs (FETCH_SIZE, then
 # WRITE_SIZE) scaled by what the same counters read for a 1 GiB device copy (--workload copy):
 # one FETCH_SIZE unit = 2.000 KiB, one WRITE_SIZE unit = 1.000 KiB.  A GEMM "launch" is the mean
-# of the step's four products (dW and dR share a launch that counts as two), each with its
-# split reduce.
-MEASURED_TRAFFIC_BYTES = {"gemm_f32": 180.2e6, "lstm_forward_recurrence": 166.8e6,
-                          "lstm_backward_recurrence": 183.0e6,
+# of the step's three products (dx; dW and dR, which share a launch that counts as two), each with
+# its split reduce; the forward recurrence includes the input projection it computes itself.
+MEASURED_TRAFFIC_BYTES = {"gemm_f32": 196.6e6, "lstm_forward_recurrence": 161.3e6,
+                          "lstm_backward_recurrence": 183.1e6,
                           # at N=1 C=512 H=4096 (--workload stepwise): 131558.5 FETCH_SIZE units
                           # + 192 WRITE_SIZE units per launch of the streaming kernel
                           "gemm_f32_skinny": 269.6e6}
