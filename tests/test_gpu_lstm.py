@@ -117,3 +117,23 @@ def test_lstm_streamed_dropconnect_and_inference():
                                p["mask"])
     assert relerr(host(h), ho) < TOL
     assert relerr(host(c), co) < TOL
+
+
+# The forward recurrence computes x*W itself for 4-row tiles (N <= 32: one set; 33..64: two sets)
+# when C <= 512 is a multiple of 4 and H > 192: input sizes below, at and between the 64-feature
+# groups a wavefront takes, one and two groups per wavefront, batches that leave rows of the last
+# tile empty, a single step with more than 8 rows.
+FUSED_INPUT_SHAPES = [(3, 4, 4, 196), (5, 7, 36, 200), (2, 31, 64, 256), (4, 32, 100, 300), (3, 33, 128, 260),
+                      (6, 64, 256, 512), (2, 50, 260, 512), (3, 9, 512, 208), (1, 40, 384, 512), (4, 61, 508, 448)]
+
+
+@pytest.mark.parametrize("zoneout", [0.0, 0.3])
+@pytest.mark.parametrize("T,N,C,H", FUSED_INPUT_SHAPES)
+def test_lstm_input_projection_inside_the_recurrence(T, N, C, H, zoneout):
+    test_lstm_training_forward_backward(T, N, C, H, zoneout)
+
+
+@pytest.mark.parametrize("T,N,C,H", [(4, 24, 96, 256), (3, 64, 512, 512)])
+def test_lstm_dropconnect_with_input_projection_inside(T, N, C, H):
+    test_lstm_dropconnect_fused_equals_premasked_weights(T, N, C, H)
+    test_lstm_inference_forward(0.25, T, N, C, H)
