@@ -99,6 +99,12 @@ static int run(const std::string& cell, int T, int N, int C, int H, float zoneou
   CHECK_HIP(hipStreamCreate(&stream));
   hipblasHandle_t blas = nullptr;  // accepted and ignored by the library
   const size_t TN = (size_t)T * N, NH = (size_t)N * H;
+
+  // HASTE_API_CHECK_LENT_WORKSPACE=1: the library's scratch memory for both streams comes from this
+  // caller (the reference's contract: every buffer is the caller's, lib/haste/lstm.h:98-117).
+  const char* lend = std::getenv("HASTE_API_CHECK_LENT_WORKSPACE");
+  const bool lent = lend != nullptr && lend[0] == '1';
+  void* lent_memory[2] = {nullptr, nullptr};
   const bool has_mask = zoneout > 0.f;
 
   // The *_iterate cells run the same problems one step at a time through Iterate()
@@ -106,6 +112,14 @@ static int run(const std::string& cell, int T, int N, int C, int H, float zoneou
   // one the caller works on.
   hipStream_t caller_stream;
   CHECK_HIP(hipStreamCreate(&caller_stream));
+  if (lent) {
+    const size_t bytes = haste_hip_workspace_bytes(T, N, C, H);
+    hipStream_t both[2] = {stream, caller_stream};
+    for (int i = 0; i < 2; ++i) {
+      CHECK_HIP(hipMalloc(&lent_memory[i], bytes));
+      require_ok(haste_hip_set_workspace(both[i], lent_memory[i], bytes), "haste_hip_set_workspace");
+    }
+  }
 
   if (cell == "lstm" || cell == "layer_norm_lstm" || cell == "lstm_iterate") {
     const bool ln = cell == "layer_norm_lstm";
@@ -347,6 +361,16 @@ static int run(const std::string& cell, int T, int N, int C, int H, float zoneou
   } else {
     std::fprintf(stderr, "unknown cell %s\n", cell.c_str());
     return 2;
+  }
+  // Everything has been synchronized by now: no kernel of either stream gave up a wait.
+  require_ok(haste_hip_stream_status(stream), "haste_hip_stream_status");
+  require_ok(haste_hip_stream_status(caller_stream), "haste_hip_stream_status (caller's stream)");
+  if (lent) {
+    hipStream_t both[2] = {stream, caller_stream};
+    for (int i = 0; i < 2; ++i) {
+      require_ok(haste_hip_set_workspace(both[i], nullptr, 0), "haste_hip_set_workspace(null)");
+      CHECK_HIP(hipFree(lent_memory[i]));
+    }
   }
   std::fclose(g_in);
   std::fclose(g_out);

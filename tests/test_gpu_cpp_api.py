@@ -15,6 +15,7 @@ pytestmark = pytest.mark.gpu
 HERE = os.path.dirname(os.path.abspath(__file__))
 BIN = os.path.join(HERE, "cpp", "api_check")
 DTYPE = np.float32  # np.float64 runs the classes instantiated for double ("f64:<cell>")
+LENT_WORKSPACE = "0"  # "1": api_check lends the library its scratch memory (haste_hip_set_workspace)
 
 
 def _run(cell, T, N, C, H, zoneout, inputs, out_shapes):
@@ -27,7 +28,8 @@ def _run(cell, T, N, C, H, zoneout, inputs, out_shapes):
                 f.write(np.ascontiguousarray(a, dtype=DTYPE).tobytes())
         print("api_check", cell, T, N, C, H, zoneout, flush=True)
         res = subprocess.run([BIN, ("f64:" if DTYPE is np.float64 else "") + cell, str(T), str(N), str(C), str(H), str(zoneout), fin, fout],
-                             capture_output=True, text=True, timeout=100)
+                             capture_output=True, text=True, timeout=100,
+                             env=dict(os.environ, HASTE_API_CHECK_LENT_WORKSPACE=LENT_WORKSPACE))
         assert res.returncode == 0, res.stdout + res.stderr
         raw = np.fromfile(fout, dtype=DTYPE).astype(np.float64)
     outs, off = [], 0
@@ -125,3 +127,13 @@ def test_cpp_layer_norm_partial_cursor():
     dx, dgamma, dbeta = O.layer_norm_backward(x, gamma, dy, cache)
     for i, (a, b) in enumerate(zip(outs, [y, cache, dx, dgamma, dbeta])):
         assert relerr(a, b) < TOL, i
+
+
+def test_cpp_classes_with_a_workspace_lent_by_the_caller(monkeypatch):
+    """The same C++ callers with the library's scratch memory lent through haste_hip_set_workspace
+    (sized by haste_hip_workspace_bytes) and haste_hip_stream_status asked at the end."""
+    import sys
+    monkeypatch.setattr(sys.modules[__name__], "LENT_WORKSPACE", "1")
+    test_cpp_lstm(9, 20, 24, 64, 0.3, False)
+    test_cpp_lstm(9, 20, 24, 64, 0.3, True)
+    test_cpp_lstm(5, 3, 7, 12, 0.0, "iterate")
