@@ -131,6 +131,11 @@ bool single_row_enabled();
 // their waits (for experiments).
 bool fused_input_enabled();
 
+// False when the environment variable HASTE_HIP_RESIDENT_ROWS is set to 0: a backward
+// recurrence whose slice of the recurrent weights exceeds LDS then runs step by step instead
+// of keeping part of the slice in registers (for experiments).
+bool resident_rows_enabled();
+
 // C[M,N] = op(A)*B (+C): fp32 MFMA GEMM on `stream`.  The partial tiles of a split product
 // are kept `scratch_offset` bytes (a multiple of 16) into the stream's scratch buffer.
 int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,

@@ -363,10 +363,13 @@ inline int gru_backward_k(int H) { return 48 * ((H + 15) / 16); }
 // Inside the launch the contraction index runs unit-major (k = 3*unit + gate), so every
 // workgroup publishes one contiguous k range of the exchange tile.  SETS sets of 256 threads,
 // each with a batch tile of NB rows of its own (see gru_forward_kernel).
-template <int NB, int SETS>
+// REG > 0: the slice exceeds LDS; every wavefront keeps the first REG k-groups of its share
+// of the contraction in registers (tall_tile_product).
+template <int NB, int SETS, int REG = 0>
 __global__ __launch_bounds__(256 * SETS, 1)
 void gru_backward_kernel(GruBwdParams p) {
   static_assert(SETS == 1 || (SETS == 2 && NB < 16), "two sets: short tiles only");
+  static_assert(REG == 0 || NB >= 16, "register-resident slice rows: tall tiles only");
   constexpr int HSB = 16;
   constexpr int NCOLS = 16;
   constexpr int PP = (NB * HSB + 255) / 256;
@@ -384,7 +387,7 @@ void gru_backward_kernel(GruBwdParams p) {
   float* w_lds = lds;
   // the partial tiles or NB*6*16 floats, whichever is more (two sets: two polled areas of
   // partial tiles each, alternating by step)
-  float* red = lds + Kpad * NCOLS + (SETS == 1 ? 0 : set * 2 * RED);
+  float* red = lds + (Kpad - 64 * REG) * NCOLS + (SETS == 1 ? 0 : set * 2 * RED);
 
   const int tid = set_thread<SETS>();
   const int j0 = role.cw * HSB;
@@ -405,12 +408,22 @@ void gru_backward_kernel(GruBwdParams p) {
   zero_tile_share<SETS>(gs, xdq, tile_floats, NB, 12 * role.cw,
                         (role.cw == p.ls.gx - 1 ? Kpad - 48 * role.cw : 48) / 4, kPolledTiles);
 
+  float4_t breg[REG > 0 ? REG : 1][1];
   {
     const bool fast = H % 4 == 0 && (reinterpret_cast<uintptr_t>(p.R_t) & 15u) == 0;
-    fill_slice<NCOLS>(w_lds, Kpad, p.R_t, nullptr, 1.0f, fast, [=](int k, int col) {
+    auto offset = [=](int k, int col) {
       const int unit = k / 3, gate = k % 3;
       return (unit < H && j0 + col < H) ? ((long long)gate * H + unit) * H + j0 + col : -1ll;
-    });
+    };
+    if constexpr (REG > 0) {
+      const int groups = Kpad >> 6;
+      fill_slice<NCOLS>(w_lds, Kpad - 64 * REG, p.R_t, nullptr, 1.0f, fast, [=](int k, int col) {
+        return offset(resident_split_k(k, groups, REG), col);
+      });
+      load_resident_rows<REG>(breg, groups, p.R_t, offset);
+    } else {
+      fill_slice<NCOLS>(w_lds, Kpad, p.R_t, nullptr, 1.0f, fast, offset);
+    }
   }
 
   int pn[PP], pj[PP], pl[PP], pc[PP];
@@ -532,7 +545,11 @@ void gru_backward_kernel(GruBwdParams p) {
     fetch(t - 1);
     // The operand loads wait for dq_t of every unit themselves.
     float* red_t = !kPolledPartials ? red : red + (done & 1) * RED;
-    tile_product<NB, 1, true, true, kPolledPartials>(xdqb, (done & 3) * tile_floats, Kpad, w_lds, red_t, &gs);
+    if constexpr (REG > 0)
+      tile_product<NB, 1, true, true, false, NoSideWork, REG, float4_t[REG][1]>(
+          xdqb, (done & 3) * tile_floats, Kpad, w_lds, red_t, &gs, nullptr, &breg);
+    else
+      tile_product<NB, 1, true, true, kPolledPartials>(xdqb, (done & 3) * tile_floats, Kpad, w_lds, red_t, &gs);
     if constexpr (kPolledPartials) {
 #pragma unroll
       for (int pp = 0; pp < PP; ++pp)
@@ -682,7 +699,7 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && v && dh_next);
   HASTE_HIP_REQUIRE(dx && dW && dR && dbx && dbr && dh && dp && dq);
   // per row: the partial tiles or the 6 bias-gradient columns of 16 floats
-  const BackwardTile tile = pick_backward_tile(gru_backward_k(H), N, H, 6 * 16, 0);
+  const BackwardTile tile = pick_backward_tile(gru_backward_k(H), N, H, 6 * 16, 0, resident_rows_enabled());
   if (!tile.ok)
     return gru_backward_streamed(stream, T, N, C, H, W_t, R_t, x_t, h, v, dh_next, dx, dW, dR, dbx,
                                  dbr, dh, dp, dq, zoneout_mask);
@@ -711,7 +728,18 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   if (paired) plan.threads = 512;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const char* name = "gru_backward_recurrence";
-  if (paired) rc = launch_persistent(name, gru_backward_kernel<4, 2>, plan, p, stream);
+#define HASTE_LAUNCH_BWD_RESIDENT(NB_)                                                           \
+  (tile.reg_groups == 8    ? launch_persistent(name, gru_backward_kernel<NB_, 1, 8>, plan, p, stream)  \
+   : tile.reg_groups == 16 ? launch_persistent(name, gru_backward_kernel<NB_, 1, 16>, plan, p, stream) \
+   : tile.reg_groups == 24 ? launch_persistent(name, gru_backward_kernel<NB_, 1, 24>, plan, p, stream) \
+                           : launch_persistent(name, gru_backward_kernel<NB_, 1, 32>, plan, p, stream))
+  if (tile.reg_groups > 0) {
+    if (tile.nb == 16) rc = HASTE_LAUNCH_BWD_RESIDENT(16);
+    else if (tile.nb == 32) rc = HASTE_LAUNCH_BWD_RESIDENT(32);
+    else if (tile.nb == 64) rc = HASTE_LAUNCH_BWD_RESIDENT(64);
+  }
+#undef HASTE_LAUNCH_BWD_RESIDENT
+  else if (paired) rc = launch_persistent(name, gru_backward_kernel<4, 2>, plan, p, stream);
   else if (tile.nb == 4) rc = launch_persistent(name, gru_backward_kernel<4, 1>, plan, p, stream);
   else if (tile.nb == 8) rc = launch_persistent(name, gru_backward_kernel<8, 1>, plan, p, stream);
   else if (tile.nb == 16) rc = launch_persistent(name, gru_backward_kernel<16, 1>, plan, p, stream);

@@ -264,7 +264,9 @@ struct LnGruBwdParams {
 inline int ln_gru_backward_k(int H) { return 48 * ((H + 15) / 16); }
 
 
-template <int NB>
+// REG > 0: the slice exceeds LDS; every wavefront keeps the first REG k-groups of its share
+// of the contraction in registers (tall_tile_product).
+template <int NB, int REG = 0>
 __global__ __launch_bounds__(256, 1)
 void ln_gru_backward_kernel(LnGruBwdParams p) {
   constexpr int HSB = 16;
@@ -282,7 +284,7 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
   const int H = p.H, N = p.N, T = p.T;
   const int Kpad = round_up(48 * p.ls.gx, 64);
   float* w_lds = lds;
-  float* red = lds + Kpad * NCOLS;  // the partial tiles, reused for the column sums
+  float* red = lds + (Kpad - 64 * REG) * NCOLS;  // the partial tiles, reused for the column sums
   float* sums = red + RED;           // [NB][4]
 
   const int tid = threadIdx.x;
@@ -307,12 +309,23 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
                   (role.cw == gx - 1 ? Kpad - 48 * role.cw : 48) / 4, kPolledTiles);
   clear_row_words(gs, part, gx, role.cw, NB, 3);
 
+  static_assert(REG == 0 || NB >= 16, "register-resident slice rows: tall tiles only");
+  float4_t breg[REG > 0 ? REG : 1][1];
   {
     const bool fast = H % 4 == 0 && (reinterpret_cast<uintptr_t>(p.R_t) & 15u) == 0;
-    fill_slice<NCOLS>(w_lds, Kpad, p.R_t, nullptr, 1.0f, fast, [=](int k, int col) {
+    auto offset = [=](int k, int col) {
       const int unit = k / 3, gate = k % 3;
       return (unit < H && j0 + col < H) ? ((long long)gate * H + unit) * H + j0 + col : -1ll;
-    });
+    };
+    if constexpr (REG > 0) {
+      const int groups = Kpad >> 6;
+      fill_slice<NCOLS>(w_lds, Kpad - 64 * REG, p.R_t, nullptr, 1.0f, fast, [=](int k, int col) {
+        return offset(resident_split_k(k, groups, REG), col);
+      });
+      load_resident_rows<REG>(breg, groups, p.R_t, offset);
+    } else {
+      fill_slice<NCOLS>(w_lds, Kpad, p.R_t, nullptr, 1.0f, fast, offset);
+    }
   }
 
   int pn[PP], pj[PP], pl[PP], pc[PP];
@@ -474,7 +487,11 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
       }
     fetch(t - 1);
     // The operand loads wait for dq_t of every unit themselves.
-    tile_product<NB, 1, true, true>(xdqb, (done & 3) * tile_floats, Kpad, w_lds, red, &gs);
+    if constexpr (REG > 0)
+      tile_product<NB, 1, true, true, false, NoSideWork, REG, float4_t[REG][1]>(
+          xdqb, (done & 3) * tile_floats, Kpad, w_lds, red, &gs, nullptr, &breg);
+    else
+      tile_product<NB, 1, true, true>(xdqb, (done & 3) * tile_floats, Kpad, w_lds, red, &gs);
     __syncthreads();
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp)
@@ -593,7 +610,7 @@ int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_s
   HASTE_HIP_REQUIRE(dp && dq && act_Wx && gamma1 && dgamma1 && act_Rh && gamma2 && dgamma2 && cache2);
   hipStream_t stream = as_stream(stream_);
   // per row: 9 column-sum accumulators of 16 floats (or the partial tiles, whichever is more) + 4 sums
-  const BackwardTile tile = pick_backward_tile(ln_gru_backward_k(H), N, H, 9 * 16, 4);
+  const BackwardTile tile = pick_backward_tile(ln_gru_backward_k(H), N, H, 9 * 16, 4, resident_rows_enabled());
   if (!tile.ok)
     return layer_norm_gru_backward_streamed(stream, T, N, C, H, W_t, R_t, x_t, h, v, dh_new, dx, dW, dR,
                                             dbx, dbr, dh, dp, dq, act_Wx, gamma1, dgamma1, act_Rh,
@@ -623,11 +640,22 @@ int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_s
   p.ls = plan.shape;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const char* name = "layer_norm_gru_backward_recurrence";
-  if (NB == 4) rc = launch_persistent(name, ln_gru_backward_kernel<4>, plan, p, stream);
-  if (NB == 8) rc = launch_persistent(name, ln_gru_backward_kernel<8>, plan, p, stream);
-  if (NB == 16) rc = launch_persistent(name, ln_gru_backward_kernel<16>, plan, p, stream);
-  if (NB == 32) rc = launch_persistent(name, ln_gru_backward_kernel<32>, plan, p, stream);
-  if (NB == 64) rc = launch_persistent(name, ln_gru_backward_kernel<64>, plan, p, stream);
+#define HASTE_LAUNCH_BWD_RESIDENT(NB_)                                                          \
+  (tile.reg_groups == 8    ? launch_persistent(name, ln_gru_backward_kernel<NB_, 8>, plan, p, stream)  \
+   : tile.reg_groups == 16 ? launch_persistent(name, ln_gru_backward_kernel<NB_, 16>, plan, p, stream) \
+   : tile.reg_groups == 24 ? launch_persistent(name, ln_gru_backward_kernel<NB_, 24>, plan, p, stream) \
+                           : launch_persistent(name, ln_gru_backward_kernel<NB_, 32>, plan, p, stream))
+  if (tile.reg_groups > 0) {
+    if (NB == 16) rc = HASTE_LAUNCH_BWD_RESIDENT(16);
+    else if (NB == 32) rc = HASTE_LAUNCH_BWD_RESIDENT(32);
+    else if (NB == 64) rc = HASTE_LAUNCH_BWD_RESIDENT(64);
+  }
+#undef HASTE_LAUNCH_BWD_RESIDENT
+  else if (NB == 4) rc = launch_persistent(name, ln_gru_backward_kernel<4>, plan, p, stream);
+  else if (NB == 8) rc = launch_persistent(name, ln_gru_backward_kernel<8>, plan, p, stream);
+  else if (NB == 16) rc = launch_persistent(name, ln_gru_backward_kernel<16>, plan, p, stream);
+  else if (NB == 32) rc = launch_persistent(name, ln_gru_backward_kernel<32>, plan, p, stream);
+  else if (NB == 64) rc = launch_persistent(name, ln_gru_backward_kernel<64>, plan, p, stream);
   HASTE_HIP_PROPAGATE(rc);
 
   const int TN = T * N;

@@ -318,7 +318,9 @@ struct LnLstmBwdParams {
   LaunchShape ls;
 };
 
-template <int NB>
+// REG > 0: the slice exceeds LDS; every wavefront keeps the first REG k-groups of its share
+// of the contraction in registers (tall_tile_product).
+template <int NB, int REG = 0>
 __global__ __launch_bounds__(256, 1)
 void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   constexpr int HSB = 16;
@@ -336,7 +338,7 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   const int H = p.H, N = p.N, T = p.T;
   const int Kpad = 64 * p.ls.gx;  // k = 4*unit + gate over the 16 units of every workgroup
   float* w_lds = lds;
-  float* red = lds + Kpad * NCOLS;  // the partial tiles, reused for the column sums
+  float* red = lds + (Kpad - 64 * REG) * NCOLS;  // the partial tiles, reused for the column sums
   float* sums_a = red + RED;         // [NB][4] row sums of the cell-state norm
   float* sums_b = sums_a + 4 * NB;   // [NB][4] row sums of the h*R norm
 
@@ -359,12 +361,23 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   clear_row_words(gs, part_a, gx, role.cw, NB, 3);
   clear_row_words(gs, part_b, gx, role.cw, NB, 3);
 
+  static_assert(REG == 0 || NB >= 16, "register-resident slice rows: tall tiles only");
+  float4_t breg[REG > 0 ? REG : 1][1];
   {
     const bool fast = H % 4 == 0 && (reinterpret_cast<uintptr_t>(p.R_t) & 15u) == 0;
-    fill_slice<NCOLS>(w_lds, Kpad, p.R_t, nullptr, 1.0f, fast, [=](int k, int col) {
+    auto offset = [=](int k, int col) {
       const int unit = k >> 2, gate = k & 3;
       return (unit < H && j0 + col < H) ? ((long long)gate * H + unit) * H + j0 + col : -1ll;
-    });
+    };
+    if constexpr (REG > 0) {
+      const int groups = Kpad >> 6;
+      fill_slice<NCOLS>(w_lds, Kpad - 64 * REG, p.R_t, nullptr, 1.0f, fast, [=](int k, int col) {
+        return offset(resident_split_k(k, groups, REG), col);
+      });
+      load_resident_rows<REG>(breg, groups, p.R_t, offset);
+    } else {
+      fill_slice<NCOLS>(w_lds, Kpad, p.R_t, nullptr, 1.0f, fast, offset);
+    }
   }
 
   int pn[PP], pj[PP], pl[PP], pc[PP];
@@ -565,7 +578,11 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
     }
     fetch(t - 1);
     // The operand loads wait for the gradient w.r.t. h*R of every unit themselves.
-    tile_product<NB, 1, true, true>(xdb, (done & 3) * tile_floats, Kpad, w_lds, red, &gs);
+    if constexpr (REG > 0)
+      tile_product<NB, 1, true, true, false, NoSideWork, REG, float4_t[REG][1]>(
+          xdb, (done & 3) * tile_floats, Kpad, w_lds, red, &gs, nullptr, &breg);
+    else
+      tile_product<NB, 1, true, true>(xdb, (done & 3) * tile_floats, Kpad, w_lds, red, &gs);
     __syncthreads();
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp)
@@ -701,7 +718,7 @@ int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_
   HASTE_HIP_REQUIRE(dgamma_h && dbeta_h && cache3 && act_c_norm);
   hipStream_t stream = as_stream(stream_);
   // per row: 10 column-sum accumulators of 16 floats (or the partial tiles, whichever is more) + 4 sums
-  const BackwardTile tile = pick_backward_tile(4 * H, N, H, 10 * 16, 8);
+  const BackwardTile tile = pick_backward_tile(4 * H, N, H, 10 * 16, 8, resident_rows_enabled());
   if (!tile.ok)
     return layer_norm_lstm_backward_streamed(stream, T, N, C, H, W_t, R_t, x_t, h, c, dh_new, dc_new,
                                              dx, dW, dR, db, dh, dc, act_Wx, gamma1, dgamma1,
@@ -735,11 +752,22 @@ int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_
   p.ls = plan.shape;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const char* name = "layer_norm_lstm_backward_recurrence";
-  if (NB == 4) rc = launch_persistent(name, ln_lstm_backward_kernel<4>, plan, p, stream);
-  if (NB == 8) rc = launch_persistent(name, ln_lstm_backward_kernel<8>, plan, p, stream);
-  if (NB == 16) rc = launch_persistent(name, ln_lstm_backward_kernel<16>, plan, p, stream);
-  if (NB == 32) rc = launch_persistent(name, ln_lstm_backward_kernel<32>, plan, p, stream);
-  if (NB == 64) rc = launch_persistent(name, ln_lstm_backward_kernel<64>, plan, p, stream);
+#define HASTE_LAUNCH_BWD_RESIDENT(NB_)                                                          \
+  (tile.reg_groups == 8    ? launch_persistent(name, ln_lstm_backward_kernel<NB_, 8>, plan, p, stream)  \
+   : tile.reg_groups == 16 ? launch_persistent(name, ln_lstm_backward_kernel<NB_, 16>, plan, p, stream) \
+   : tile.reg_groups == 24 ? launch_persistent(name, ln_lstm_backward_kernel<NB_, 24>, plan, p, stream) \
+                           : launch_persistent(name, ln_lstm_backward_kernel<NB_, 32>, plan, p, stream))
+  if (tile.reg_groups > 0) {
+    if (NB == 16) rc = HASTE_LAUNCH_BWD_RESIDENT(16);
+    else if (NB == 32) rc = HASTE_LAUNCH_BWD_RESIDENT(32);
+    else if (NB == 64) rc = HASTE_LAUNCH_BWD_RESIDENT(64);
+  }
+#undef HASTE_LAUNCH_BWD_RESIDENT
+  else if (NB == 4) rc = launch_persistent(name, ln_lstm_backward_kernel<4>, plan, p, stream);
+  else if (NB == 8) rc = launch_persistent(name, ln_lstm_backward_kernel<8>, plan, p, stream);
+  else if (NB == 16) rc = launch_persistent(name, ln_lstm_backward_kernel<16>, plan, p, stream);
+  else if (NB == 32) rc = launch_persistent(name, ln_lstm_backward_kernel<32>, plan, p, stream);
+  else if (NB == 64) rc = launch_persistent(name, ln_lstm_backward_kernel<64>, plan, p, stream);
   HASTE_HIP_PROPAGATE(rc);
 
   // Gradient through the norm of x*W (in place over act_Wx), then the batched products.

@@ -391,10 +391,13 @@ struct LstmBwdParams {
 // the contraction index runs unit-major (k = 4*unit + gate), so a thread publishes the
 // four gate gradients of its (row, unit) with one 16-byte store.  SETS sets of 256 threads,
 // each with a batch tile of NB rows of its own (see lstm_forward_kernel).
-template <int NB, int SETS>
+// REG > 0: the slice exceeds LDS; every wavefront keeps the first REG k-groups of its share
+// of the contraction in registers (tall_tile_product).
+template <int NB, int SETS, int REG = 0>
 __global__ __launch_bounds__(256 * SETS, 1)
 void lstm_backward_kernel(LstmBwdParams p) {
   static_assert(SETS == 1 || (SETS == 2 && NB < 16), "two sets: short tiles only");
+  static_assert(REG == 0 || NB >= 16, "register-resident slice rows: tall tiles only");
   constexpr int HSB = 16;
   constexpr int NCOLS = 16;
   constexpr int PP = (NB * HSB + 255) / 256;
@@ -412,7 +415,7 @@ void lstm_backward_kernel(LstmBwdParams p) {
   float* w_lds = lds;
   // the partial tiles (two sets: two polled areas each, alternating by step), reused for
   // the db reduction
-  float* red = lds + Kpad * NCOLS + (SETS == 1 ? 0 : set * 2 * RED);
+  float* red = lds + (Kpad - 64 * REG) * NCOLS + (SETS == 1 ? 0 : set * 2 * RED);
 
   const int tid = set_thread<SETS>();
   const int j0 = role.cw * HSB;
@@ -428,12 +431,22 @@ void lstm_backward_kernel(LstmBwdParams p) {
   float* xdv = p.xdv + (size_t)bt * kPolledTiles * tile_floats;
   const TileBuffer xdvb = make_tile_buffer(xdv, kPolledTiles * tile_floats);
 
+  float4_t breg[REG > 0 ? REG : 1][1];
   {
     const bool fast = H % 4 == 0 && (reinterpret_cast<uintptr_t>(p.R_t) & 15u) == 0;
-    fill_slice<NCOLS>(w_lds, Kpad, p.R_t, nullptr, 1.0f, fast, [=](int k, int col) {
+    auto offset = [=](int k, int col) {
       const int unit = k >> 2, gate = k & 3;
       return (unit < H && j0 + col < H) ? ((long long)gate * H + unit) * H + j0 + col : -1ll;
-    });
+    };
+    if constexpr (REG > 0) {
+      const int groups = Kpad >> 6;
+      fill_slice<NCOLS>(w_lds, Kpad - 64 * REG, p.R_t, nullptr, 1.0f, fast, [=](int k, int col) {
+        return offset(resident_split_k(k, groups, REG), col);
+      });
+      load_resident_rows<REG>(breg, groups, p.R_t, offset);
+    } else {
+      fill_slice<NCOLS>(w_lds, Kpad, p.R_t, nullptr, 1.0f, fast, offset);
+    }
   }
 
   int pn[PP], pj[PP], pl[PP], pc[PP];
@@ -559,7 +572,11 @@ void lstm_backward_kernel(LstmBwdParams p) {
     // dv_t of every unit themselves.
     fetch(t - 1);
     float* red_t = !kPolledPartials ? red : red + (done & 1) * RED;
-    tile_product<NB, 1, true, true, kPolledPartials>(xdvb, (done & 3) * tile_floats, Kpad, w_lds, red_t, &gs);
+    if constexpr (REG > 0)
+      tile_product<NB, 1, true, true, false, NoSideWork, REG, float4_t[REG][1]>(
+          xdvb, (done & 3) * tile_floats, Kpad, w_lds, red_t, &gs, nullptr, &breg);
+    else
+      tile_product<NB, 1, true, true, kPolledPartials>(xdvb, (done & 3) * tile_floats, Kpad, w_lds, red_t, &gs);
     if constexpr (kPolledPartials) {
 #pragma unroll
       for (int pp = 0; pp < PP; ++pp)
@@ -735,7 +752,7 @@ int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
   HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && c && c_next && dh_next && dc_next);
   HASTE_HIP_REQUIRE(dx && dW && dR && db && dh && dc && v);
-  const BackwardTile tile = pick_backward_tile(4 * H, N, H, 4 * 16, 0);
+  const BackwardTile tile = pick_backward_tile(4 * H, N, H, 4 * 16, 0, resident_rows_enabled());
   if (!tile.ok)
     return lstm_backward_streamed(stream, T, N, C, H, W_t, R_t, x_t, h, c, c_next, dh_next, dc_next,
                                   dx, dW, dR, db, dh, dc, v, zoneout_mask);
@@ -765,7 +782,18 @@ int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   if (paired) plan.threads = 512;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const char* name = "lstm_backward_recurrence";
-  if (paired) rc = launch_persistent(name, lstm_backward_kernel<4, 2>, plan, p, stream);
+#define HASTE_LAUNCH_BWD_RESIDENT(NB_)                                                            \
+  (tile.reg_groups == 8    ? launch_persistent(name, lstm_backward_kernel<NB_, 1, 8>, plan, p, stream)  \
+   : tile.reg_groups == 16 ? launch_persistent(name, lstm_backward_kernel<NB_, 1, 16>, plan, p, stream) \
+   : tile.reg_groups == 24 ? launch_persistent(name, lstm_backward_kernel<NB_, 1, 24>, plan, p, stream) \
+                           : launch_persistent(name, lstm_backward_kernel<NB_, 1, 32>, plan, p, stream))
+  if (tile.reg_groups > 0) {
+    if (tile.nb == 16) rc = HASTE_LAUNCH_BWD_RESIDENT(16);
+    else if (tile.nb == 32) rc = HASTE_LAUNCH_BWD_RESIDENT(32);
+    else if (tile.nb == 64) rc = HASTE_LAUNCH_BWD_RESIDENT(64);
+  }
+#undef HASTE_LAUNCH_BWD_RESIDENT
+  else if (paired) rc = launch_persistent(name, lstm_backward_kernel<4, 2>, plan, p, stream);
   else if (tile.nb == 4) rc = launch_persistent(name, lstm_backward_kernel<4, 1>, plan, p, stream);
   else if (tile.nb == 8) rc = launch_persistent(name, lstm_backward_kernel<8, 1>, plan, p, stream);
   else if (tile.nb == 16) rc = launch_persistent(name, lstm_backward_kernel<16, 1>, plan, p, stream);

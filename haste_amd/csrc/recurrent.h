@@ -418,6 +418,70 @@ __device__ __forceinline__ void mfma_chunk(const float* w_lds, int g_abs,
   }
 }
 
+// The same MFMAs for k-groups whose slice rows the lanes hold in registers: lane (kq, row)
+// keeps in breg[j][ct] what mfma_chunk reads from the slice in LDS for its wavefront's
+// j-th k-group (see load_resident_rows).
+template <int RT, int CT, int CHUNK, int REG, int FIRST>
+__device__ __forceinline__ void mfma_chunk_resident(const float4_t (&breg)[REG][CT],
+                                                    const float4_t (&av)[CHUNK][RT],
+                                                    float4_t (&acc0)[RT][CT], float4_t (&acc1)[RT][CT]) {
+  static_assert(FIRST + CHUNK <= REG, "chunk beyond the resident rows");
+#pragma unroll
+  for (int gi = 0; gi < CHUNK; ++gi) {
+    float4_t (&acc)[RT][CT] = (gi & 1) ? acc1 : acc0;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+        acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].x, breg[FIRST + gi][ct].x, acc[rt][ct], 0, 0, 0);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+        acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].y, breg[FIRST + gi][ct].y, acc[rt][ct], 0, 0, 0);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+        acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].z, breg[FIRST + gi][ct].z, acc[rt][ct], 0, 0, 0);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+        acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].w, breg[FIRST + gi][ct].w, acc[rt][ct], 0, 0, 0);
+  }
+}
+
+// A slice too large for LDS keeps the first REG k-groups of every wavefront's share in
+// that wavefront's registers and the rest in LDS, compacted: LDS k-group w*(groups-REG) + j
+// is k-group w*groups + REG + j of the contraction (groups = Kpad/64 per wavefront).
+__device__ __forceinline__ int resident_split_k(int k_lds, int groups, int reg_groups) {
+  const int lds_groups = groups - reg_groups;
+  const int gl = k_lds >> 4;
+  return ((gl / lds_groups) * groups + reg_groups + gl % lds_groups) * 16 + (k_lds & 15);
+}
+
+// Loads the register-resident rows of this wavefront: `offset(k, col)` as for fill_slice.
+template <int REG, class OffsetFn>
+__device__ __forceinline__ void load_resident_rows(float4_t (&breg)[REG][1], int groups,
+                                                   const float* __restrict__ src, OffsetFn offset) {
+  const int lane = threadIdx.x & 63;
+  const int wave = (threadIdx.x >> 6) & 3;
+  const int col = lane & 15, kq = lane >> 4;
+#pragma unroll
+  for (int j = 0; j < REG; ++j) {
+    const int k = (wave * groups + j) * 16 + kq * 4;
+    float w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const long long off = offset(k + i, col);
+      w[i] = src[off >= 0 ? off : 0];
+      if (off < 0) w[i] = 0.f;
+    }
+    breg[j][0] = float4_t{w[0], w[1], w[2], w[3]};
+  }
+}
+
 // Writes this wavefront's accumulators to red[wave][16*RT][16*CT] in LDS.
 template <int RT, int CT>
 __device__ __forceinline__ void store_partials(float* red, const float4_t (&acc)[RT][CT]) {
@@ -604,14 +668,22 @@ __device__ __forceinline__ void load_tile_chunk(const TileBuffer& xb, int tile_o
     for (int rt = 0; rt < RT; ++rt) av[gi][rt] = load_tile4(xb, base + (gi * 4 * NB + rt * 16) * 4);
 }
 
-template <int RT, int CT, int CHUNK, bool POLLED>
+struct NoResidentRows {};
+
+// REG > 0: the first REG k-groups of every wavefront's share take their slice rows from
+// `breg` (registers), the others from the compacted slice in LDS (resident_split_k).
+template <int RT, int CT, int CHUNK, bool POLLED, int REG = 0, class Resident = NoResidentRows>
 __device__ __forceinline__ void tall_tile_product(const TileBuffer& xb, int tile_off, int Kpad,
                                                   const float* w_lds, float* red,
-                                                  const GroupSync* gs) {
+                                                  const GroupSync* gs,
+                                                  const Resident* breg = nullptr) {
+  static_assert(REG % CHUNK == 0, "resident rows: whole chunks");
   const int wave = threadIdx.x >> 6;
   const int groups = Kpad >> 6;  // k-groups of 16 per wavefront
-  const int full = groups / CHUNK;
-  int g = wave * groups;
+  const int lds_groups = groups - REG;
+  const int full = lds_groups / CHUNK;
+  int g = wave * groups;         // k-group of the operand tile
+  int gl = wave * lds_groups;    // k-group of the slice in LDS
   const int g_end = g + groups;
   float4_t acc[RT][CT], acc1[RT][CT];
 #pragma unroll
@@ -619,29 +691,45 @@ __device__ __forceinline__ void tall_tile_product(const TileBuffer& xb, int tile
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = acc1[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-  if (full > 0) {
+  if (REG > 0 || full > 0) {
     float4_t cur[CHUNK][RT], nxt[CHUNK][RT];
     load_tile_chunk<RT, CHUNK>(xb, tile_off, g, g_end, cur);
+    if constexpr (REG > 0) {
+      static_for<REG / CHUNK>([&](auto ic) {
+        constexpr int CI = decltype(ic)::value;
+        if (CI + 1 < REG / CHUNK || full > 0) load_tile_chunk<RT, CHUNK>(xb, tile_off, g + CHUNK, g_end, nxt);
+        if constexpr (POLLED)
+          poll_until_written(*gs, [&] { load_tile_chunk<RT, CHUNK>(xb, tile_off, g, g_end, cur); },
+                             [&] { return all_written(cur); });
+        mfma_chunk_resident<RT, CT, CHUNK, REG, CI * CHUNK>(*breg, cur, acc, acc1);
+#pragma unroll
+        for (int gi = 0; gi < CHUNK; ++gi)
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) cur[gi][rt] = nxt[gi][rt];
+        g += CHUNK;
+      });
+    }
     for (int c = 0; c < full; ++c) {
       if (c + 1 < full) load_tile_chunk<RT, CHUNK>(xb, tile_off, g + CHUNK, g_end, nxt);
       if constexpr (POLLED)
         poll_until_written(*gs, [&] { load_tile_chunk<RT, CHUNK>(xb, tile_off, g, g_end, cur); },
                            [&] { return all_written(cur); });
-      mfma_chunk<RT, CT, CHUNK>(w_lds, g, cur, acc, acc1);
+      mfma_chunk<RT, CT, CHUNK>(w_lds, gl, cur, acc, acc1);
 #pragma unroll
       for (int gi = 0; gi < CHUNK; ++gi)
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) cur[gi][rt] = nxt[gi][rt];
       g += CHUNK;
+      gl += CHUNK;
     }
   }
-  for (; g < g_end; ++g) {
+  for (; g < g_end; ++g, ++gl) {
     float4_t one[1][RT];
     load_tile_chunk<RT, 1>(xb, tile_off, g, g_end, one);
     if constexpr (POLLED)
       poll_until_written(*gs, [&] { load_tile_chunk<RT, 1>(xb, tile_off, g, g_end, one); },
                          [&] { return all_written(one); });
-    mfma_chunk<RT, CT, 1>(w_lds, g, one, acc, acc1);
+    mfma_chunk<RT, CT, 1>(w_lds, gl, one, acc, acc1);
   }
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
@@ -966,11 +1054,15 @@ __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int
 // longer than the hidden size (the backward passes).
 // POLLED: the tile is a polled exchange tile (see above) and `gs` supplies the bounds of the
 // wait; otherwise the caller has waited at the group's step barrier and `gs` is unused.
-template <int NB, int CT, bool LONG_K, bool POLLED = false, bool TAGGED = false, class Side = NoSideWork>
+// REG > 0 (tall tiles): the slice is split between registers and LDS, see tall_tile_product.
+template <int NB, int CT, bool LONG_K, bool POLLED = false, bool TAGGED = false, class Side = NoSideWork,
+          int REG = 0, class Resident = NoResidentRows>
 __device__ __forceinline__ void tile_product(const TileBuffer& xb, int tile_off, int Kpad,
                                              const float* w_lds, float* red,
-                                             const GroupSync* gs = nullptr, Side* side = nullptr) {
+                                             const GroupSync* gs = nullptr, Side* side = nullptr,
+                                             const Resident* breg = nullptr) {
   if constexpr (ProductTile<NB, CT>::kShort) {
+    static_assert(REG == 0, "register-resident slice rows exist for tall tiles only");
     short_exchange_product<NB / 4, CT, LONG_K ? 4 : 2, POLLED, TAGGED, Side>(xb, tile_off, Kpad, w_lds,
                                                                               red, gs, side);
   } else {
@@ -981,8 +1073,9 @@ __device__ __forceinline__ void tile_product(const TileBuffer& xb, int tile_off,
     // (8 groups per wavefront) in one piece, a backward share (32 groups) in two, are 9-10 %
     // faster per step than pieces of 4 / 8 at 16 rows, pieces of 8 than 4 at 32 rows; twice
     // that is slower again.
-    constexpr int CHUNK = LONG_K ? (RT == 1 ? 16 : (RT == 2 ? 8 : 2)) : (RT >= 4 ? 2 : 8);
-    tall_tile_product<RT, CT, CHUNK, POLLED>(xb, tile_off, Kpad, w_lds, red, gs);
+    constexpr int CHUNK0 = LONG_K ? (RT == 1 ? 16 : (RT == 2 ? 8 : 2)) : (RT >= 4 ? 2 : 8);
+    constexpr int CHUNK = (REG % CHUNK0 != 0) ? 8 : CHUNK0;  // REG: a multiple of 8
+    tall_tile_product<RT, CT, CHUNK, POLLED, REG, Resident>(xb, tile_off, Kpad, w_lds, red, gs, breg);
   }
 }
 
@@ -1341,15 +1434,23 @@ struct BackwardTile {
   int nb, gx, gy;
   size_t lds_bytes;
   bool ok;
+  int reg_groups;  // k-groups of the slice that every wavefront keeps in registers
 };
+
+// The most k-groups (of 16) of its share of the slice that a wavefront keeps in registers.
+constexpr int kMaxResidentGroups = 32;
 
 // K = gates*H is the contraction length.  Per batch row the kernel needs, beyond the
 // slice, max(`reduce_floats_per_row`, the partial tiles) + `extra_floats_per_row` floats.
+// `resident_rows`: the kernel can keep part of a slice that exceeds LDS in registers (tiles
+// of 16 rows and more; a multiple of 8 k-groups per wavefront, at most kMaxResidentGroups).
 inline BackwardTile pick_backward_tile(int K, int N, int H, size_t reduce_floats_per_row,
-                                       size_t extra_floats_per_row) {
+                                       size_t extra_floats_per_row, bool resident_rows = false) {
   const int cus = device_cu_count();
   const int gx = (H + 15) / 16;
   const int Kpad = (K + 63) / 64 * 64;
+  const int groups = Kpad / 64;                // per wavefront
+  const size_t group_bytes = 4 * 16 * 16 * sizeof(float);  // one k-group of each wavefront
   BackwardTile best;
   best.ok = false;
   for (int pass = 0; pass < 2 && !best.ok; ++pass) {
@@ -1358,10 +1459,18 @@ inline BackwardTile pick_backward_tile(int K, int N, int H, size_t reduce_floats
       size_t per_row = (size_t)product_partials(nb, 1) * 16;
       if (per_row < reduce_floats_per_row) per_row = reduce_floats_per_row;
       per_row += extra_floats_per_row;
-      const size_t lds = ((size_t)Kpad * 16 + per_row * nb) * sizeof(float);
+      const size_t other = per_row * nb * sizeof(float);
+      size_t lds = (size_t)Kpad * 16 * sizeof(float) + other;
+      int reg_groups = 0;
+      if (lds > kMaxLdsBytes && resident_rows && nb >= 16 && other < kMaxLdsBytes) {
+        const int fit = (int)((kMaxLdsBytes - other) / group_bytes);
+        reg_groups = (groups - fit + 7) / 8 * 8;
+        if (reg_groups > kMaxResidentGroups || reg_groups > groups) continue;
+        lds = (size_t)(groups - reg_groups) * group_bytes + other;
+      }
       if (lds > kMaxLdsBytes || gy > kMaxGroups || gx * gy > kMaxWorkgroups) continue;
       if (pass == 0 ? !xcd_local_fits(gx, gy) : (long long)gx * gy > cus) continue;
-      best = BackwardTile{nb, gx, gy, lds, true};
+      best = BackwardTile{nb, gx, gy, lds, true, reg_groups};
       break;
     }
   }

@@ -241,6 +241,14 @@ bool fused_input_enabled() {
   return enabled;
 }
 
+bool resident_rows_enabled() {
+  static const bool enabled = [] {
+    const char* v = std::getenv("HASTE_HIP_RESIDENT_ROWS");
+    return v == nullptr || v[0] != '0';
+  }();
+  return enabled;
+}
+
 int device_cu_count() {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
@@ -454,7 +462,8 @@ int haste_hip_max_hidden_size(int gates, int batch_size) {
     const int k_back = gates == 3 ? 48 * ((H + 15) / 16) : gates * H;
     const size_t reduce_floats = gates == 3 ? 6 * 16 : (size_t)gates * 16;
     return haste_hip::pick_forward_tile(gates, batch_size, H, 0, haste_hip::kWorkgroupLdsBytes).ok &&
-           haste_hip::pick_backward_tile(k_back, batch_size, H, reduce_floats, 0).ok;
+           haste_hip::pick_backward_tile(k_back, batch_size, H, reduce_floats, 0,
+                                         haste_hip::resident_rows_enabled()).ok;
   };
   int best = 0;
   for (int H = 16; H <= 8192; H += 16)

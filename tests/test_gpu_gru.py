@@ -17,7 +17,12 @@ SHAPES = [(1, 1, 1, 1), (3, 2, 3, 4), (5, 3, 7, 5), (6, 17, 20, 36), (4, 16, 32,
           # one batch row: the forward pass keeps the recurrent weights in registers (H <= 512)
           (9, 1, 7, 100), (6, 1, 16, 512), (5, 1, 8, 300), (4, 1, 8, 48), (7, 1, 5, 17),
           # hidden sizes beyond what stays on chip: the backward pass, then both passes, stream R
-          (3, 5, 40, 704), (3, 4, 32, 1536), (2, 70, 24, 1700), (2, 128, 16, 1024)]
+          (3, 5, 40, 704), (3, 4, 32, 1536), (2, 70, 24, 1700), (2, 128, 16, 1024),
+          # 816 < H <= 1488: the backward recurrence keeps part of its slice of R in registers
+          # (8, 16, 24 or 32 k-groups per wavefront; tiles of 16, 32 and 64 rows; hidden sizes
+          # that leave single k-groups and a ragged last workgroup)
+          (4, 64, 32, 1024), (3, 17, 24, 900), (3, 100, 16, 1200), (2, 60, 16, 1400),
+          (5, 16, 8, 1023), (2, 256, 8, 1024), (3, 9, 8, 1488)]
 
 
 @pytest.mark.parametrize("zoneout", [0.0, 0.3])

@@ -17,7 +17,10 @@ SHAPES = [(1, 1, 3, 4), (3, 2, 3, 4), (5, 3, 7, 5), (6, 17, 20, 36), (4, 16, 32,
           # step by step (GEMM + row-wise norms + pointwise kernels)
           (3, 5, 24, 640), (2, 6, 16, 1536), (2, 130, 8, 1100),
           # resident forward whose norm of x*W is wider than 4096 columns
-          (2, 3, 8, 1028)]
+          (2, 3, 8, 1028),
+          # hidden sizes whose backward recurrence keeps part of its slice of R in registers
+          # (LSTM: 592 < H <= 1104, GRU: 784 < H <= 1472), tiles of 16, 32 and 64 rows
+          (3, 20, 16, 768), (3, 64, 24, 1024), (2, 100, 8, 900), (2, 40, 8, 1300), (3, 130, 8, 1000)]
 
 
 @pytest.mark.parametrize("zoneout", [0.0, 0.3])

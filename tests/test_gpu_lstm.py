@@ -18,7 +18,12 @@ SHAPES = [(1, 1, 1, 1), (3, 2, 3, 4), (5, 3, 7, 5), (6, 17, 20, 36), (4, 16, 32,
           # one batch row: the forward pass keeps the recurrent weights in registers (H <= 512)
           (9, 1, 7, 100), (6, 1, 16, 512), (5, 1, 8, 300), (4, 1, 8, 48), (7, 1, 5, 17),
           # hidden sizes beyond what stays on chip: the backward pass, then both passes, stream R
-          (3, 5, 40, 640), (3, 4, 32, 1536), (2, 70, 24, 1300), (2, 128, 16, 1024)]
+          (3, 5, 40, 640), (3, 4, 32, 1536), (2, 70, 24, 1300), (2, 128, 16, 1024),
+          # 608 < H <= 1120: the backward recurrence keeps part of its slice of R in registers
+          # (8, 16, 24 or 32 k-groups per wavefront; tiles of 16, 32 and 64 rows; hidden sizes
+          # that leave single k-groups and a ragged last workgroup)
+          (4, 64, 32, 1024), (3, 17, 24, 768), (3, 100, 16, 896), (2, 200, 16, 1000),
+          (3, 9, 8, 700), (2, 256, 8, 1024), (3, 30, 8, 1120), (5, 16, 8, 1023)]
 
 
 def run_lstm(p, training, zoneout_prob, T, N, C, H):
@@ -137,3 +142,46 @@ def test_lstm_input_projection_inside_the_recurrence(T, N, C, H, zoneout):
 def test_lstm_dropconnect_with_input_projection_inside(T, N, C, H):
     test_lstm_dropconnect_fused_equals_premasked_weights(T, N, C, H)
     test_lstm_inference_forward(0.25, T, N, C, H)
+
+
+def _launch_counts(lib, names):
+    import ctypes
+    out = {}
+    for name in names:
+        total, count = ctypes.c_double(0.0), ctypes.c_int(0)
+        assert lib.haste_hip_profile_read(name.encode(), ctypes.byref(total), ctypes.byref(count)) == 0
+        out[name] = count.value
+    return out
+
+
+@pytest.mark.parametrize("cell", ["lstm", "gru"])
+@pytest.mark.parametrize("N,H", [(5, 640), (64, 768), (64, 1024), (128, 1024)])
+def test_backward_of_mid_sized_hidden_states_is_one_persistent_launch(cell, N, H):
+    """608 < H <= 1024 (GRU: above 816): the backward pass is one launch of the persistent
+    recurrence, not one product and one pointwise launch per step."""
+    from haste_amd import lib as hlib, ops
+    import torch
+    T, C = 3, 16
+    gates = 4 if cell == "lstm" else 3
+    p = problem(7, T, N, C, H, 4, 0.0)
+    lib = hlib.load()
+    none = torch.empty(0, 0, 0, device="cuda:0")
+    x, h0 = dev(p["x"]), dev(p["h0"])
+    W, R, b = dev(p["W"][:, :gates * H]), dev(p["R"][:, :gates * H]), dev(p["b"][:gates * H])
+    x_t, W_t, R_t = ops.transpose(x), ops.transpose(W), ops.transpose(R)
+    lib.haste_hip_profile_reset()
+    lib.haste_hip_profile_enable(1)
+    try:
+        if cell == "lstm":
+            h, c, cache = ops.lstm_forward(True, 0.0, x, h0, dev(p["c0"]), W, R, b, none)
+            ops.lstm_backward(x_t, W_t, R_t, b, none, h, c, cache, dev(p["dh_new"]), dev(p["dc_new"]))
+        else:
+            b2 = dev(p["b2"][:3 * H])
+            h, cache = ops.gru_forward(True, 0.0, x, h0, W, R, b, b2, none)
+            ops.gru_backward(x_t, W_t, R_t, b, b2, none, h, cache, dev(p["dh_new"]))
+        torch.cuda.synchronize()
+    finally:
+        lib.haste_hip_profile_enable(0)
+    n = _launch_counts(lib, [cell + "_backward_recurrence", cell + "_backward_steps"])
+    lib.haste_hip_profile_reset()
+    assert n[cell + "_backward_recurrence"] == 1 and n[cell + "_backward_steps"] == 0, n
