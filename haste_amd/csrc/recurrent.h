@@ -367,55 +367,78 @@ __device__ __forceinline__ void fill_slice(float* w_lds, int Kpad, const float* 
   }
 }
 
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+// f(std::integral_constant<int, i>) for i = 0 .. N-1, unrolled at compile time (MFMA
+// broadcast selectors must be immediates).
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
 // MFMAs of k-groups [g_abs, g_abs+CHUNK): one straight-line block (no branches, so the
-// accumulators stay in the matrix unit's registers); the LDS reads of the slice columns of
-// a k-group are issued before the MFMAs of the k-group ahead of it.  Consecutive MFMAs go to
-// different accumulators (two per output tile, alternating by k-group) so that none
-// waits for the result of the one before it.
+// accumulators stay in the matrix unit's registers).  The LDS reads of the slice columns
+// run kTallLdsAhead blocks ahead of the MFMAs that use them; a scheduling barrier keeps each
+// read where it is issued (the compiler would otherwise sink it to just before its use and
+// the wavefront would wait out the LDS latency once per block).  Consecutive MFMAs go to
+// different accumulators (two per output tile, alternating by k-group): with one output
+// tile per wavefront a block is two k-groups whose MFMAs alternate, so that none waits for
+// the result of the one before it.
+constexpr int kTallLdsAhead = 2;
+
+// Keeps the two MFMAs issued before it ahead of those issued after it (an empty statement
+// the compiler cannot move accumulator updates across): the compiler otherwise lines up the
+// four dependent MFMAs of one k-group, each of which waits for the one before it.
+__device__ __forceinline__ void pin_mfma_pair(float4_t& a, float4_t& b) {
+  asm volatile("" : "+a"(a), "+a"(b));
+}
+
 template <int RT, int CT, int CHUNK>
 __device__ __forceinline__ void mfma_chunk(const float* w_lds, int g_abs,
                                            const float4_t (&av)[CHUNK][RT],
                                            float4_t (&acc0)[RT][CT], float4_t (&acc1)[RT][CT]) {
   constexpr int NCOLS = 16 * CT;
+  constexpr int P = (RT * CT == 1 && CHUNK % 2 == 0) ? 2 : 1;  // k-groups per block
+  constexpr int BLOCKS = CHUNK / P;
+  constexpr int AHEAD = BLOCKS < kTallLdsAhead ? BLOCKS : kTallLdsAhead;
   const int lane = threadIdx.x & 63;
   const int row = lane & 15;
   const int kq = lane >> 4;
   const float* wp0 = w_lds + ((g_abs * 4 + kq) * NCOLS + row) * 4;
-  float4_t bnext[CT];
+  float4_t b[CHUNK][CT];
+  auto read_block = [&](auto bc) {
+    constexpr int B = decltype(bc)::value;
 #pragma unroll
-  for (int ct = 0; ct < CT; ++ct) bnext[ct] = *reinterpret_cast<const float4_t*>(wp0 + ct * 64);
-#pragma unroll
-  for (int gi = 0; gi < CHUNK; ++gi) {
-    float4_t b[CT];
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) b[ct] = bnext[ct];
-    if (gi + 1 < CHUNK) {
+    for (int p = 0; p < P; ++p)
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct)
-        bnext[ct] = *reinterpret_cast<const float4_t*>(wp0 + (gi + 1) * 4 * NCOLS * 4 + ct * 64);
+        b[B * P + p][ct] = *reinterpret_cast<const float4_t*>(wp0 + (B * P + p) * 4 * NCOLS * 4 + ct * 64);
+  };
+  static_for<AHEAD>(read_block);
+  static_for<BLOCKS>([&](auto bc) {
+    constexpr int B = decltype(bc)::value;
+    if constexpr (B + AHEAD < BLOCKS) {
+      read_block(std::integral_constant<int, B + AHEAD>{});
+      __builtin_amdgcn_sched_barrier(0);
     }
-    float4_t (&acc)[RT][CT] = (gi & 1) ? acc1 : acc0;
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
+    for (int c = 0; c < 4; ++c) {
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct)
-        acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].x, b[ct].x, acc[rt][ct], 0, 0, 0);
+      for (int p = 0; p < P; ++p) {
+        constexpr int G0 = B * P;
+        float4_t (&acc)[RT][CT] = ((G0 + p) & 1) ? acc1 : acc0;
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
+        for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct)
-        acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].y, b[ct].y, acc[rt][ct], 0, 0, 0);
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int ct = 0; ct < CT; ++ct)
-        acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].z, b[ct].z, acc[rt][ct], 0, 0, 0);
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int ct = 0; ct < CT; ++ct)
-        acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].w, b[ct].w, acc[rt][ct], 0, 0, 0);
-  }
+          for (int ct = 0; ct < CT; ++ct)
+            acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[G0 + p][rt][c], b[G0 + p][ct][c],
+                                                               acc[rt][ct], 0, 0, 0);
+      }
+      if constexpr (P == 2) pin_mfma_pair(acc0[0][0], acc1[0][0]);
+    }
+  });
 }
 
 // The same MFMAs for k-groups whose slice rows the lanes hold in registers: lane (kq, row)
@@ -426,30 +449,23 @@ __device__ __forceinline__ void mfma_chunk_resident(const float4_t (&breg)[REG][
                                                     const float4_t (&av)[CHUNK][RT],
                                                     float4_t (&acc0)[RT][CT], float4_t (&acc1)[RT][CT]) {
   static_assert(FIRST + CHUNK <= REG, "chunk beyond the resident rows");
+  constexpr int P = (RT * CT == 1 && CHUNK % 2 == 0) ? 2 : 1;  // k-groups whose MFMAs alternate
 #pragma unroll
-  for (int gi = 0; gi < CHUNK; ++gi) {
-    float4_t (&acc)[RT][CT] = (gi & 1) ? acc1 : acc0;
+  for (int g0 = 0; g0 < CHUNK; g0 += P)
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
+    for (int c = 0; c < 4; ++c) {
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct)
-        acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].x, breg[FIRST + gi][ct].x, acc[rt][ct], 0, 0, 0);
+      for (int p = 0; p < P; ++p) {
+        float4_t (&acc)[RT][CT] = ((g0 + p) & 1) ? acc1 : acc0;
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
+        for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct)
-        acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].y, breg[FIRST + gi][ct].y, acc[rt][ct], 0, 0, 0);
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int ct = 0; ct < CT; ++ct)
-        acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].z, breg[FIRST + gi][ct].z, acc[rt][ct], 0, 0, 0);
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int ct = 0; ct < CT; ++ct)
-        acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[gi][rt].w, breg[FIRST + gi][ct].w, acc[rt][ct], 0, 0, 0);
-  }
+          for (int ct = 0; ct < CT; ++ct)
+            acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[g0 + p][rt][c], breg[FIRST + g0 + p][ct][c],
+                                                               acc[rt][ct], 0, 0, 0);
+      }
+      if constexpr (P == 2) pin_mfma_pair(acc0[0][0], acc1[0][0]);
+    }
 }
 
 // A slice too large for LDS keeps the first REG k-groups of every wavefront's share in
@@ -509,17 +525,6 @@ __device__ __forceinline__ void store_partials(float* red, const float4_t (&acc)
 // of blocks (CBSZ/ABID): one instruction multiplies 4 batch rows by MC = 16, 32 or 64
 // slice columns for KS = 4, 2 or 1 values of k (lane group l/MC takes the k-th value),
 // so the matrix unit's time scales with the rows in steps of 4.
-
-template <class F, int... I>
-__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
-  (f(std::integral_constant<int, I>{}), ...);
-}
-// f(std::integral_constant<int, i>) for i = 0 .. N-1, unrolled at compile time (MFMA
-// broadcast selectors must be immediates).
-template <int N, class F>
-__device__ __forceinline__ void static_for(F&& f) {
-  static_for_impl(f, std::make_integer_sequence<int, N>{});
-}
 
 // Sums across lane groups.  swap_add16(a, b): lanes of the even 16-lane rows get a(row) +
 // a(row+1), lanes of the odd rows b(row-1) + b(row), each from the lanes at the same position
@@ -692,36 +697,43 @@ __device__ __forceinline__ void tall_tile_product(const TileBuffer& xb, int tile
     for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = acc1[rt][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
 
   if (REG > 0 || full > 0) {
-    float4_t cur[CHUNK][RT], nxt[CHUNK][RT];
-    load_tile_chunk<RT, CHUNK>(xb, tile_off, g, g_end, cur);
-    if constexpr (REG > 0) {
-      static_for<REG / CHUNK>([&](auto ic) {
-        constexpr int CI = decltype(ic)::value;
-        if (CI + 1 < REG / CHUNK || full > 0) load_tile_chunk<RT, CHUNK>(xb, tile_off, g + CHUNK, g_end, nxt);
-        if constexpr (POLLED)
-          poll_until_written(*gs, [&] { load_tile_chunk<RT, CHUNK>(xb, tile_off, g, g_end, cur); },
-                             [&] { return all_written(cur); });
-        mfma_chunk_resident<RT, CT, CHUNK, REG, CI * CHUNK>(*breg, cur, acc, acc1);
-#pragma unroll
-        for (int gi = 0; gi < CHUNK; ++gi)
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt) cur[gi][rt] = nxt[gi][rt];
-        g += CHUNK;
-      });
-    }
-    for (int c = 0; c < full; ++c) {
-      if (c + 1 < full) load_tile_chunk<RT, CHUNK>(xb, tile_off, g + CHUNK, g_end, nxt);
+    // Two operand buffers that swap roles chunk by chunk (no copies): while the MFMAs of
+    // one run, the loads of the next chunk fill the other.  The poll comes before those
+    // loads are issued: with them in flight the compiler could not tell whether the poll's
+    // re-load had completed and would wait for the oldest of them before the MFMAs.
+    float4_t buf0[CHUNK][RT], buf1[CHUNK][RT];
+    load_tile_chunk<RT, CHUNK>(xb, tile_off, g, g_end, buf0);
+    auto stage = [&](float4_t (&cur)[CHUNK][RT], float4_t (&nxt)[CHUNK][RT], bool more, auto&& mfmas) {
       if constexpr (POLLED)
         poll_until_written(*gs, [&] { load_tile_chunk<RT, CHUNK>(xb, tile_off, g, g_end, cur); },
                            [&] { return all_written(cur); });
-      mfma_chunk<RT, CT, CHUNK>(w_lds, gl, cur, acc, acc1);
-#pragma unroll
-      for (int gi = 0; gi < CHUNK; ++gi)
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) cur[gi][rt] = nxt[gi][rt];
+      if (more) load_tile_chunk<RT, CHUNK>(xb, tile_off, g + CHUNK, g_end, nxt);
+      mfmas(cur);
       g += CHUNK;
-      gl += CHUNK;
+    };
+    constexpr int RC = REG / CHUNK;  // chunks with register-resident slice rows
+    if constexpr (REG > 0) {
+      static_for<RC>([&](auto ic) {
+        constexpr int CI = decltype(ic)::value;
+        auto mfmas = [&](const float4_t (&cur)[CHUNK][RT]) {
+          mfma_chunk_resident<RT, CT, CHUNK, REG, CI * CHUNK>(*breg, cur, acc, acc1);
+        };
+        if constexpr (CI % 2 == 0) stage(buf0, buf1, CI + 1 < RC || full > 0, mfmas);
+        else stage(buf1, buf0, CI + 1 < RC || full > 0, mfmas);
+      });
     }
+    auto lds_mfmas = [&](const float4_t (&cur)[CHUNK][RT]) {
+      mfma_chunk<RT, CT, CHUNK>(w_lds, gl, cur, acc, acc1);
+      gl += CHUNK;
+    };
+    float4_t (&first)[CHUNK][RT] = RC % 2 == 0 ? buf0 : buf1;
+    float4_t (&second)[CHUNK][RT] = RC % 2 == 0 ? buf1 : buf0;
+    int c = 0;
+    for (; c + 1 < full; c += 2) {
+      stage(first, second, true, lds_mfmas);
+      stage(second, first, c + 2 < full, lds_mfmas);
+    }
+    if (c < full) stage(first, second, false, lds_mfmas);
   }
   for (; g < g_end; ++g, ++gl) {
     float4_t one[1][RT];
