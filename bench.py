@@ -24,7 +24,7 @@ PEAK_HBM_GBS = 8000.0
 # one FETCH_SIZE unit = 2.000 KiB, one WRITE_SIZE unit = 1.000 KiB.  A GEMM "launch" is the mean
 # of the step's three products (dx; dW and dR, which share a launch that counts as two), each with
 # its split reduce; the forward recurrence includes the input projection it computes itself.
-MEASURED_TRAFFIC_BYTES = {"gemm_f32": 196.6e6, "lstm_forward_recurrence": 161.3e6,
+MEASURED_TRAFFIC_BYTES = {"gemm_f32": 143.2e6, "lstm_forward_recurrence": 161.3e6,
                           "lstm_backward_recurrence": 183.1e6,
                           # at N=1 C=512 H=4096 (--workload stepwise): 131558.5 FETCH_SIZE units
                           # + 192 WRITE_SIZE units per launch of the streaming kernel
