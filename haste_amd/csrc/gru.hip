@@ -32,11 +32,14 @@ struct GruFwdParams {
 // SETS sets of 256 threads, each with a batch tile of NB rows of its own.  Two sets share
 // the resident slice but nothing else: while one waits for its exchange the other computes,
 // which a single tile of 2*NB rows cannot do.
-template <int NB, int CT, int HS, int SETS>
+// REG > 0 (tiles of 16 rows and more): the slice exceeds LDS; every wavefront keeps the first REG
+// k-groups of its share of the contraction in registers (tall_tile_product).
+template <int NB, int CT, int HS, int SETS, int REG = 0>
 __global__ __launch_bounds__(256 * SETS, 1)
 void gru_forward_kernel(GruFwdParams p) {
   static_assert(3 * HS <= 16 * CT, "slice too narrow");
   static_assert(SETS == 1 || (SETS == 2 && NB < 16), "two sets: short tiles only");
+  static_assert(REG == 0 || (NB >= 16 && SETS == 1), "register-resident slice rows: tall tiles only");
   constexpr int NCOLS = 16 * CT;
   constexpr int PP = (NB * HS + 255) / 256;
   constexpr int RED = ProductTile<NB, CT>::kRedFloats;
@@ -48,11 +51,11 @@ void gru_forward_kernel(GruFwdParams p) {
   float* w_lds = lds;
   // one set: one area of partial tiles behind workgroup barriers; two sets: two polled
   // areas each, alternating by step
-  float* red = lds + Kpad * NCOLS + (SETS == 1 ? 0 : set * 2 * RED);
+  float* red = lds + (Kpad - 64 * REG) * NCOLS + (SETS == 1 ? 0 : set * 2 * RED);
   // The role is handed round through a word of the partial-tile area, which nothing else
   // uses before the first step: the kernel has no static LDS, so that a slice and its
   // partial tiles may fill the workgroup's 160 KiB exactly (N = 128, H = 1024).
-  const Role role = take_role(p.ls, reinterpret_cast<unsigned int*>(lds + Kpad * NCOLS));
+  const Role role = take_role(p.ls, reinterpret_cast<unsigned int*>(lds + (Kpad - 64 * REG) * NCOLS));
   if (!role.active) return;
 
   const int tid = set_thread<SETS>();
@@ -73,13 +76,23 @@ void gru_forward_kernel(GruFwdParams p) {
   zero_tile_share<SETS>(gs, xh, tile_floats, NB, j0 / 4,
                         (role.cw == p.ls.gx - 1 ? Kpad - j0 : HS) / 4, kPolledTiles);
 
+  float4_t breg[REG > 0 ? REG : 1][CT];
   {
     const bool fast = H % 4 == 0 && ((reinterpret_cast<uintptr_t>(p.R) |
                                       reinterpret_cast<uintptr_t>(p.dc_mask)) & 15u) == 0;
-    fill_slice<NCOLS>(w_lds, Kpad, p.R, p.dc_mask, p.dc_scale, fast, [=](int k, int col) {
+    auto offset = [=](int k, int col) {
       const int gate = col / HS, j = j0 + col % HS;
       return (k < H && gate < 3 && j < H) ? (long long)k * 3 * H + gate * H + j : -1ll;
-    });
+    };
+    if constexpr (REG > 0) {
+      const int groups = Kpad >> 6;
+      fill_slice<NCOLS>(w_lds, Kpad - 64 * REG, p.R, p.dc_mask, p.dc_scale, fast, [=](int k, int col) {
+        return offset(resident_split_k(k, groups, REG), col);
+      });
+      load_resident_rows<REG, CT>(breg, groups, p.R, p.dc_mask, p.dc_scale, offset);
+    } else {
+      fill_slice<NCOLS>(w_lds, Kpad, p.R, p.dc_mask, p.dc_scale, fast, offset);
+    }
   }
 
   int pn[PP], pj[PP], pl[PP], pc[PP];
@@ -149,7 +162,11 @@ void gru_forward_kernel(GruFwdParams p) {
     }
     // The operand loads wait for h[t] themselves (polled tile t % 4).
     float* red_t = !kPolledPartials ? red : red + (t & 1) * RED;
-    tile_product<NB, CT, false, true, kPolledPartials>(xhb, (t & 3) * tile_floats, Kpad, w_lds, red_t, &gs);
+    if constexpr (REG > 0)
+      tile_product<NB, CT, false, true, false, NoSideWork, REG, float4_t[REG][CT]>(
+          xhb, (t & 3) * tile_floats, Kpad, w_lds, red_t, &gs, nullptr, &breg);
+    else
+      tile_product<NB, CT, false, true, kPolledPartials>(xhb, (t & 3) * tile_floats, Kpad, w_lds, red_t, &gs);
     if constexpr (!kPolledPartials) __syncthreads();
 
     float saved[PP][4];  // z, r, g, q of the step for the caller's cache
@@ -420,7 +437,7 @@ void gru_backward_kernel(GruBwdParams p) {
       fill_slice<NCOLS>(w_lds, Kpad - 64 * REG, p.R_t, nullptr, 1.0f, fast, [=](int k, int col) {
         return offset(resident_split_k(k, groups, REG), col);
       });
-      load_resident_rows<REG>(breg, groups, p.R_t, offset);
+      load_resident_rows<REG, 1>(breg, groups, p.R_t, nullptr, 1.0f, offset);
     } else {
       fill_slice<NCOLS>(w_lds, Kpad, p.R_t, nullptr, 1.0f, fast, offset);
     }
@@ -642,7 +659,7 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
   if (N == 1 && H <= 512 && xcd_local_fits((H + 15) / 16, 1) && single_row_enabled())
     return gru_forward_single_row(stream, training, T, C, H, W, R, bx, br, x, h, h_out, v, tmp_Wx,
                                   zoneout_prob, zoneout_mask, dc_mask, dc_scale);
-  const ForwardTile tile = pick_forward_tile(3, N, H, 0, kWorkgroupLdsBytes);
+  const ForwardTile tile = pick_forward_tile(3, N, H, 0, kWorkgroupLdsBytes, false, resident_rows_enabled() ? 3 : 0);
   // No slice of R fits a CU: stream R from HBM every step instead.
   if (!tile.ok)
     return gru_forward_streamed(stream, training, T, N, C, H, W, R, bx, br, x, h, h_out, v, tmp_Wx,
@@ -652,7 +669,8 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
   // An 8-row tile is run as two sets of 4 rows when the partial tiles of both fit beside the
   // slice (exchange tiles: one per set, together as large as the tile's).
   const size_t paired_lds = paired_lds_bytes((H + 63) / 64 * 64, tile.ct);
-  const bool paired = tile.nb == 8 && paired_lds <= kWorkgroupLdsBytes && paired_sets_enabled();
+  const bool paired = tile.nb == 8 && paired_lds <= kWorkgroupLdsBytes && paired_sets_enabled() &&
+                      tile.reg_groups == 0;
 
   // Taken after the GEMM, which may replace the stream's scratch buffer with a larger one.
   Workspace ws;
@@ -671,6 +689,15 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
                                   paired ? paired_lds : tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;
   if (paired) plan.threads = 512;
+#define HASTE_LAUNCH_FWD_RESIDENT(NB_, CT_, HS_, REG_)                                              \
+  if (tile.reg_groups == REG_ && tile.nb == NB_ && tile.hs == HS_)                                 \
+    return launch_persistent("gru_forward_recurrence", gru_forward_kernel<NB_, CT_, HS_, 1, REG_>, \
+                             plan, p, stream);
+  HASTE_LAUNCH_FWD_RESIDENT(16, 2, 8, 8) HASTE_LAUNCH_FWD_RESIDENT(32, 2, 8, 8) HASTE_LAUNCH_FWD_RESIDENT(64, 2, 8, 8)
+  HASTE_LAUNCH_FWD_RESIDENT(16, 2, 8, 16) HASTE_LAUNCH_FWD_RESIDENT(32, 2, 8, 16) HASTE_LAUNCH_FWD_RESIDENT(64, 2, 8, 16)
+  HASTE_LAUNCH_FWD_RESIDENT(16, 3, 16, 8) HASTE_LAUNCH_FWD_RESIDENT(32, 3, 16, 8) HASTE_LAUNCH_FWD_RESIDENT(64, 3, 16, 8)
+#undef HASTE_LAUNCH_FWD_RESIDENT
+  if (tile.reg_groups > 0) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 #define HASTE_LAUNCH_FWD_PAIRED(CT_, HS_)                                                     \
   if (paired && tile.hs == HS_)                                                               \
     return launch_persistent("gru_forward_recurrence", gru_forward_kernel<4, CT_, HS_, 2>,    \

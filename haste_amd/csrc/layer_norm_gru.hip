@@ -322,7 +322,7 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
       fill_slice<NCOLS>(w_lds, Kpad - 64 * REG, p.R_t, nullptr, 1.0f, fast, [=](int k, int col) {
         return offset(resident_split_k(k, groups, REG), col);
       });
-      load_resident_rows<REG>(breg, groups, p.R_t, offset);
+      load_resident_rows<REG, 1>(breg, groups, p.R_t, nullptr, 1.0f, offset);
     } else {
       fill_slice<NCOLS>(w_lds, Kpad, p.R_t, nullptr, 1.0f, fast, offset);
     }

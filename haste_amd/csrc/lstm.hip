@@ -38,11 +38,14 @@ struct LstmFwdParams {
 // XSG > 0 (4-row tiles): the kernel also computes the input projection x[t] * W, on the matrix
 // units while its wavefronts wait for h[t] (InputProjection in recurrent.h; a wavefront takes
 // XSG super-groups of 64 input features), instead of reading it from v.
-template <int NB, int CT, int SETS, int XSG = 0>
+// REG > 0 (tiles of 16 rows and more): the slice exceeds LDS; every wavefront keeps the first REG
+// k-groups of its share of the contraction in registers (tall_tile_product).
+template <int NB, int CT, int SETS, int XSG = 0, int REG = 0>
 __global__ __launch_bounds__(256 * SETS, 1)
 void lstm_forward_kernel(LstmFwdParams p) {
   static_assert(SETS == 1 || (SETS == 2 && NB < 16), "two sets: short tiles only");
   static_assert(XSG == 0 || NB == 4, "fused input projection: 4-row tiles only");
+  static_assert(REG == 0 || (NB >= 16 && SETS == 1), "register-resident slice rows: tall tiles only");
   constexpr bool kFusedInput = XSG > 0;
   constexpr int HS = 4 * CT;
   constexpr int NCOLS = 16 * CT;
@@ -56,11 +59,11 @@ void lstm_forward_kernel(LstmFwdParams p) {
   float* w_lds = lds;
   // one set: one area of partial tiles behind workgroup barriers; two sets: two polled
   // areas each, alternating by step
-  float* red = lds + Kpad * NCOLS + (SETS == 1 ? 0 : set * 2 * RED);
+  float* red = lds + (Kpad - 64 * REG) * NCOLS + (SETS == 1 ? 0 : set * 2 * RED);
   // The role is handed round through a word of the partial-tile area, which nothing else
   // uses before the first step: the kernel has no static LDS, so that a slice and its
   // partial tiles may fill the workgroup's 160 KiB exactly (N = 128, H = 1024).
-  const Role role = take_role(p.ls, reinterpret_cast<unsigned int*>(lds + Kpad * NCOLS));
+  const Role role = take_role(p.ls, reinterpret_cast<unsigned int*>(lds + (Kpad - 64 * REG) * NCOLS));
   if (!role.active) return;
 
   const int tid = set_thread<SETS>();
@@ -96,13 +99,23 @@ void lstm_forward_kernel(LstmFwdParams p) {
   }
 
   // Resident slice: column c of the slice is gate c/HS, hidden unit j0 + c%HS.
+  float4_t breg[REG > 0 ? REG : 1][CT];
   {
     const bool fast = H % 4 == 0 && ((reinterpret_cast<uintptr_t>(p.R) |
                                       reinterpret_cast<uintptr_t>(p.dc_mask)) & 15u) == 0;
-    fill_slice<NCOLS>(w_lds, Kpad, p.R, p.dc_mask, p.dc_scale, fast, [=](int k, int col) {
+    auto offset = [=](int k, int col) {
       const int gate = col / HS, j = j0 + col % HS;
       return (k < H && j < H) ? (long long)k * 4 * H + gate * H + j : -1ll;
-    });
+    };
+    if constexpr (REG > 0) {
+      const int groups = Kpad >> 6;
+      fill_slice<NCOLS>(w_lds, Kpad - 64 * REG, p.R, p.dc_mask, p.dc_scale, fast, [=](int k, int col) {
+        return offset(resident_split_k(k, groups, REG), col);
+      });
+      load_resident_rows<REG, CT>(breg, groups, p.R, p.dc_mask, p.dc_scale, offset);
+    } else {
+      fill_slice<NCOLS>(w_lds, Kpad, p.R, p.dc_mask, p.dc_scale, fast, offset);
+    }
   }
 
   // Pointwise ownership: thread slot pp handles batch row n, hidden unit j.
@@ -178,6 +191,9 @@ void lstm_forward_kernel(LstmFwdParams p) {
       tile_product<NB, CT, false, true, kPolledPartials, Projection>(xhb, (t & 3) * tile_floats, Kpad,
                                                                       w_lds, red_t, &gs, &proj);
       if (t + 1 < T) proj.request();  // x[t+1]: a whole step to arrive
+    } else if constexpr (REG > 0) {
+      tile_product<NB, CT, false, true, false, NoSideWork, REG, float4_t[REG][CT]>(
+          xhb, (t & 3) * tile_floats, Kpad, w_lds, red_t, &gs, nullptr, &breg);
     } else {
       tile_product<NB, CT, false, true, kPolledPartials>(xhb, (t & 3) * tile_floats, Kpad, w_lds, red_t, &gs);
     }
@@ -443,7 +459,7 @@ void lstm_backward_kernel(LstmBwdParams p) {
       fill_slice<NCOLS>(w_lds, Kpad - 64 * REG, p.R_t, nullptr, 1.0f, fast, [=](int k, int col) {
         return offset(resident_split_k(k, groups, REG), col);
       });
-      load_resident_rows<REG>(breg, groups, p.R_t, offset);
+      load_resident_rows<REG, 1>(breg, groups, p.R_t, nullptr, 1.0f, offset);
     } else {
       fill_slice<NCOLS>(w_lds, Kpad, p.R_t, nullptr, 1.0f, fast, offset);
     }
@@ -672,7 +688,7 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
   if (N == 1 && H <= 512 && xcd_local_fits((H + 15) / 16, 1) && single_row_enabled())
     return lstm_forward_single_row(stream, training, T, C, H, W, R, b, x, h, c, h_out, c_out, v,
                                    zoneout_prob, zoneout_mask, dc_mask, dc_scale);
-  const ForwardTile tile = pick_forward_tile(4, N, H, 0, kWorkgroupLdsBytes);
+  const ForwardTile tile = pick_forward_tile(4, N, H, 0, kWorkgroupLdsBytes, false, resident_rows_enabled() ? 2 : 0);
   // No slice of R fits a CU: stream R from HBM every step instead.
   if (!tile.ok)
     return lstm_forward_streamed(stream, training, T, N, C, H, W, R, b, x, h, c, h_out, c_out, v,
@@ -681,7 +697,8 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
   // slice (exchange tiles: one per set, together as large as the tile's).  Measured at
   // H = 512: 6 % faster per step; two sets of 8 rows instead of a 16-row tile: 6 % slower.
   const size_t paired_lds = paired_lds_bytes((H + 63) / 64 * 64, tile.ct);
-  const bool paired = tile.nb == 8 && paired_lds <= kWorkgroupLdsBytes && paired_sets_enabled();
+  const bool paired = tile.nb == 8 && paired_lds <= kWorkgroupLdsBytes && paired_sets_enabled() &&
+                      tile.reg_groups == 0;
 
   // With 4-row tiles the recurrence computes x * W itself, beside its waits (every wavefront of
   // a set must have a share of the recurrent product, H > 192, to keep in step with the readers
@@ -711,6 +728,14 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
                                   paired ? paired_lds : tile.lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;
   if (paired) plan.threads = 512;
+#define HASTE_LAUNCH_FWD_RESIDENT(NB_, REG_)                                                     \
+  if (tile.reg_groups == REG_ && tile.nb == NB_ && tile.ct == 2)                                 \
+    return launch_persistent("lstm_forward_recurrence", lstm_forward_kernel<NB_, 2, 1, 0, REG_>, \
+                             plan, p, stream);
+  HASTE_LAUNCH_FWD_RESIDENT(16, 8) HASTE_LAUNCH_FWD_RESIDENT(32, 8) HASTE_LAUNCH_FWD_RESIDENT(64, 8)
+  HASTE_LAUNCH_FWD_RESIDENT(16, 16) HASTE_LAUNCH_FWD_RESIDENT(32, 16) HASTE_LAUNCH_FWD_RESIDENT(64, 16)
+#undef HASTE_LAUNCH_FWD_RESIDENT
+  if (tile.reg_groups > 0) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 #define HASTE_LAUNCH_FWD_FUSED(CT_, XSG_)                                                       \
   if (fused && tile.ct == CT_ && xsg == XSG_) {                                                  \
     if (paired)                                                                                  \

@@ -477,25 +477,31 @@ __device__ __forceinline__ int resident_split_k(int k_lds, int groups, int reg_g
   return ((gl / lds_groups) * groups + reg_groups + gl % lds_groups) * 16 + (k_lds & 15);
 }
 
-// Loads the register-resident rows of this wavefront: `offset(k, col)` as for fill_slice.
-template <int REG, class OffsetFn>
-__device__ __forceinline__ void load_resident_rows(float4_t (&breg)[REG][1], int groups,
-                                                   const float* __restrict__ src, OffsetFn offset) {
+// Loads the register-resident rows of this wavefront: `offset(k, col)` as for fill_slice,
+// `mask` and `scale` likewise (DropConnect).
+template <int REG, int CT, class OffsetFn>
+__device__ __forceinline__ void load_resident_rows(float4_t (&breg)[REG][CT], int groups,
+                                                   const float* __restrict__ src,
+                                                   const float* __restrict__ mask, float scale,
+                                                   OffsetFn offset) {
   const int lane = threadIdx.x & 63;
   const int wave = (threadIdx.x >> 6) & 3;
-  const int col = lane & 15, kq = lane >> 4;
+  const int col0 = lane & 15, kq = lane >> 4;
 #pragma unroll
-  for (int j = 0; j < REG; ++j) {
-    const int k = (wave * groups + j) * 16 + kq * 4;
-    float w[4];
+  for (int j = 0; j < REG; ++j)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const long long off = offset(k + i, col);
-      w[i] = src[off >= 0 ? off : 0];
-      if (off < 0) w[i] = 0.f;
+    for (int ct = 0; ct < CT; ++ct) {
+      const int k = (wave * groups + j) * 16 + kq * 4;
+      float w[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const long long off = offset(k + i, ct * 16 + col0);
+        w[i] = src[off >= 0 ? off : 0];
+        if (mask != nullptr) w[i] = w[i] * mask[off >= 0 ? off : 0] * scale;
+        if (off < 0) w[i] = 0.f;
+      }
+      breg[j][ct] = float4_t{w[0], w[1], w[2], w[3]};
     }
-    breg[j][0] = float4_t{w[0], w[1], w[2], w[3]};
-  }
 }
 
 // Writes this wavefront's accumulators to red[wave][16*RT][16*CT] in LDS.
@@ -1403,6 +1409,7 @@ struct ForwardTile {
   int nb, ct, hs, gx, gy;
   size_t lds_bytes;
   bool ok;
+  int reg_groups;  // k-groups of the slice that every wavefront keeps in registers
 };
 
 constexpr int kTileHeights[] = {4, 8, 16, 32, 64};
@@ -1415,11 +1422,17 @@ constexpr int kTileHeights[] = {4, 8, 16, 32, 64};
 // whose steps also exchange row statistics among all workgroups of a group (every workgroup
 // reads every other's slots), are 10-25 % faster per step that way (N <= 32, H = 64 .. 256;
 // with 8-row tiles it depends on H, and the plain cells are 10-20 % slower).
+// `resident_max_ct` > 0: the kernel can keep part of a slice that exceeds LDS in registers
+// (tiles of 16 rows and more, 8 or 16 hidden units per workgroup in at most that many column
+// tiles; a multiple of 8 k-groups per wavefront, at most 128 registers per lane).  Tried when no
+// geometry fits LDS alone.
 inline ForwardTile pick_forward_tile(int gates, int N, int H, size_t extra_lds_per_row,
-                                     size_t lds_limit = kMaxLdsBytes, bool wide_first = false) {
+                                     size_t lds_limit = kMaxLdsBytes, bool wide_first = false,
+                                     int resident_max_ct = 0) {
   const int cus = device_cu_count();
   ForwardTile best;
   best.ok = false;
+  best.reg_groups = 0;
   for (int pass = 0; pass < 2 && !best.ok; ++pass) {
     const int hs_order_local[] = {4, 8, 16};
     const int hs_order_wide[] = {16, 8, 4};
@@ -1433,9 +1446,30 @@ inline ForwardTile pick_forward_tile(int gates, int N, int H, size_t extra_lds_p
         const size_t lds = fwd_lds_bytes(H, nb, ct) + extra_lds_per_row * nb;
         if (lds > lds_limit || gy > kMaxGroups || gx * gy > kMaxWorkgroups) continue;
         if (pass == 0 ? !xcd_local_fits(gx, gy) : (long long)gx * gy > cus) continue;
-        best = ForwardTile{nb, ct, hs, gx, gy, lds, true};
+        best = ForwardTile{nb, ct, hs, gx, gy, lds, true, 0};
       }
       if (best.ok) break;
+    }
+  }
+  if (best.ok || resident_max_ct <= 0) return best;
+  const int groups = (H + 63) / 64;  // k-groups of 16 per wavefront
+  for (int nb : kTileHeights) {
+    if (nb < 16) continue;
+    for (int hs : {8, 16}) {
+      const int ct = (gates * hs + 15) / 16;
+      const int gx = (H + hs - 1) / hs, gy = (N + nb - 1) / nb;
+      if (ct > resident_max_ct || gy > kMaxGroups || (long long)gx * gy > cus) continue;
+      const size_t group_bytes = (size_t)4 * 16 * 16 * ct * sizeof(float);  // one k-group of each wavefront
+      const size_t other = (size_t)product_partials(nb, ct) * nb * 16 * ct * sizeof(float) +
+                           extra_lds_per_row * nb;
+      if (other >= lds_limit) continue;
+      const int fit = (int)((lds_limit - other) / group_bytes);
+      if (fit >= groups) continue;  // fits LDS: the passes above decide
+      const int reg_groups = (groups - fit + 7) / 8 * 8;
+      if (reg_groups * ct > 32 || reg_groups >= groups) continue;
+      best = ForwardTile{nb, ct, hs, gx, gy, (size_t)(groups - reg_groups) * group_bytes + other, true,
+                         reg_groups};
+      return best;
     }
   }
   return best;

@@ -461,7 +461,8 @@ int haste_hip_max_hidden_size(int gates, int batch_size) {
   auto fits = [&](int H) {
     const int k_back = gates == 3 ? 48 * ((H + 15) / 16) : gates * H;
     const size_t reduce_floats = gates == 3 ? 6 * 16 : (size_t)gates * 16;
-    return haste_hip::pick_forward_tile(gates, batch_size, H, 0, haste_hip::kWorkgroupLdsBytes).ok &&
+    const int max_ct = !haste_hip::resident_rows_enabled() ? 0 : (gates == 3 ? 3 : (gates == 4 ? 2 : 0));
+    return haste_hip::pick_forward_tile(gates, batch_size, H, 0, haste_hip::kWorkgroupLdsBytes, false, max_ct).ok &&
            haste_hip::pick_backward_tile(k_back, batch_size, H, reduce_floats, 0,
                                          haste_hip::resident_rows_enabled()).ok;
   };

@@ -22,7 +22,10 @@ SHAPES = [(1, 1, 1, 1), (3, 2, 3, 4), (5, 3, 7, 5), (6, 17, 20, 36), (4, 16, 32,
           # (8, 16, 24 or 32 k-groups per wavefront; tiles of 16, 32 and 64 rows; hidden sizes
           # that leave single k-groups and a ragged last workgroup)
           (4, 64, 32, 1024), (3, 17, 24, 900), (3, 100, 16, 1200), (2, 60, 16, 1400),
-          (5, 16, 8, 1023), (2, 256, 8, 1024), (3, 9, 8, 1488)]
+          (5, 16, 8, 1023), (2, 256, 8, 1024), (3, 9, 8, 1488),
+          # 1024 < H <= 2048 with up to 64 rows: the forward recurrence keeps part of its slice
+          # of R in registers as well (8 hidden units per workgroup, tiles of 16, 32 and 64 rows)
+          (3, 20, 16, 2048), (2, 64, 8, 2048), (3, 9, 24, 1536), (2, 50, 8, 1800), (3, 16, 8, 1290), (2, 256, 8, 1024)]
 
 
 @pytest.mark.parametrize("zoneout", [0.0, 0.3])

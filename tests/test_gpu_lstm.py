@@ -23,7 +23,10 @@ SHAPES = [(1, 1, 1, 1), (3, 2, 3, 4), (5, 3, 7, 5), (6, 17, 20, 36), (4, 16, 32,
           # (8, 16, 24 or 32 k-groups per wavefront; tiles of 16, 32 and 64 rows; hidden sizes
           # that leave single k-groups and a ragged last workgroup)
           (4, 64, 32, 1024), (3, 17, 24, 768), (3, 100, 16, 896), (2, 200, 16, 1000),
-          (3, 9, 8, 700), (2, 256, 8, 1024), (3, 30, 8, 1120), (5, 16, 8, 1023)]
+          (3, 9, 8, 700), (2, 256, 8, 1024), (3, 30, 8, 1120), (5, 16, 8, 1023),
+          # 1024 < H <= 2048 with up to 64 rows: the forward recurrence keeps part of its slice
+          # of R in registers as well (8 hidden units per workgroup, tiles of 16, 32 and 64 rows)
+          (3, 20, 16, 2048), (2, 64, 8, 2048), (3, 9, 24, 1536), (2, 50, 8, 1800), (3, 16, 8, 1290)]
 
 
 def run_lstm(p, training, zoneout_prob, T, N, C, H):
@@ -72,7 +75,7 @@ def test_lstm_inference_forward(zoneout, T, N, C, H):
     assert relerr(host(c), co) < TOL
 
 
-@pytest.mark.parametrize("T,N,C,H", [(6, 8, 16, 64), (5, 48, 16, 128), (6, 1, 16, 200)])
+@pytest.mark.parametrize("T,N,C,H", [(6, 8, 16, 64), (5, 48, 16, 128), (6, 1, 16, 200), (3, 20, 16, 1536)])
 def test_lstm_dropconnect_fused_equals_premasked_weights(T, N, C, H):
     """Bit for bit, in the 4-row tile kernel, the two-set kernel and the single-row kernel."""
     from haste_amd import ops
@@ -185,3 +188,32 @@ def test_backward_of_mid_sized_hidden_states_is_one_persistent_launch(cell, N, H
     n = _launch_counts(lib, [cell + "_backward_recurrence", cell + "_backward_steps"])
     lib.haste_hip_profile_reset()
     assert n[cell + "_backward_recurrence"] == 1 and n[cell + "_backward_steps"] == 0, n
+
+
+@pytest.mark.parametrize("cell", ["lstm", "gru"])
+@pytest.mark.parametrize("N,H", [(1, 1536), (32, 2048), (64, 2048)])
+def test_forward_of_large_hidden_states_is_one_persistent_launch(cell, N, H):
+    """1024 < H <= 2048 with up to 64 rows: the forward pass is one launch of the persistent
+    recurrence (part of the slice of R in registers), not one product per step."""
+    from haste_amd import lib as hlib, ops
+    import torch
+    T, C = 3, 16
+    gates = 4 if cell == "lstm" else 3
+    p = problem(9, T, N, C, H, 4, 0.0)
+    lib = hlib.load()
+    none = torch.empty(0, 0, 0, device="cuda:0")
+    x, h0 = dev(p["x"]), dev(p["h0"])
+    W, R, b = dev(p["W"][:, :gates * H]), dev(p["R"][:, :gates * H]), dev(p["b"][:gates * H])
+    lib.haste_hip_profile_reset()
+    lib.haste_hip_profile_enable(1)
+    try:
+        if cell == "lstm":
+            ops.lstm_forward(False, 0.0, x, h0, dev(p["c0"]), W, R, b, none)
+        else:
+            ops.gru_forward(False, 0.0, x, h0, W, R, b, dev(p["b2"][:3 * H]), none)
+        torch.cuda.synchronize()
+    finally:
+        lib.haste_hip_profile_enable(0)
+    n = _launch_counts(lib, [cell + "_forward_recurrence", cell + "_forward_steps"])
+    lib.haste_hip_profile_reset()
+    assert n[cell + "_forward_recurrence"] == 1 and n[cell + "_forward_steps"] == 0, n
