@@ -107,6 +107,18 @@ unsigned long long device_xcc_logical_map();
 // kernel just enqueued on `stream` as the one to wait for.
 int order_persistent_launches(hipStream_t stream, bool before);
 
+// Holds the process-wide order of persistent launches from before the wait for the previous
+// launch until this launch has been recorded as the last one: two host threads that launch
+// on different streams would otherwise both wait for the launch before theirs and then run
+// side by side.
+class PersistentLaunchOrder {
+ public:
+  PersistentLaunchOrder();
+  ~PersistentLaunchOrder();
+  PersistentLaunchOrder(const PersistentLaunchOrder&) = delete;
+  PersistentLaunchOrder& operator=(const PersistentLaunchOrder&) = delete;
+};
+
 // Polls before a bounded wait of a persistent kernel gives up: 2^24 (seconds), or the value of
 // the environment variable HASTE_HIP_SPIN_LIMIT.
 unsigned int spin_limit();

@@ -1385,6 +1385,8 @@ int launch_persistent(const char* name, KernelT kernel, const LaunchPlan& plan, 
   const int per_cu = found->second;
   const long long capacity = (long long)per_cu * device_cu_count();
   if ((long long)plan.grid.x * plan.grid.y > capacity) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+  // wait for the last launch, launch, become the last launch: as one step among host threads
+  PersistentLaunchOrder in_order;
   HASTE_HIP_PROPAGATE(order_persistent_launches(stream, true));
   {
     ScopedKernelTimer timer(name, stream);

@@ -83,6 +83,13 @@ struct LastPersistent {
 std::map<int, LastPersistent> g_last_persistent;
 }  // namespace
 
+namespace {
+std::mutex g_persistent_order_mutex;
+}  // namespace
+
+PersistentLaunchOrder::PersistentLaunchOrder() { g_persistent_order_mutex.lock(); }
+PersistentLaunchOrder::~PersistentLaunchOrder() { g_persistent_order_mutex.unlock(); }
+
 int order_persistent_launches(hipStream_t stream, bool before) {
   int dev = 0;
   HASTE_HIP_TRY(hipGetDevice(&dev));

@@ -38,8 +38,8 @@ const char* haste_hip_error_string(int code);
 const char* haste_hip_last_runtime_error(void);
 
 /* Largest hidden size whose recurrent weight slice the persistent kernels can keep
- * on chip for `gates` gate blocks (4 LSTM, 3 GRU) and `batch_size` rows on the
- * current device; 0 if none.  Larger hidden sizes are accepted as well: the cells then
+ * on chip (in LDS, or in LDS and registers) in both directions for `gates` gate blocks
+ * (4 LSTM, 3 GRU) and `batch_size` rows on the current device; 0 if none.  Larger hidden sizes are accepted as well: the cells then
  * stream the recurrent matrix from HBM every step (one GEMM plus row-wise norm and pointwise
  * kernels per step, as the reference does). */
 int haste_hip_max_hidden_size(int gates, int batch_size);
