@@ -25,19 +25,23 @@ def _shapes(seed, count, hidden):
 
 
 RESIDENT = _shapes(11, 10, lambda r: r.integers(4, 560))
-# beyond the on-chip limits: backward only (577..1000), both passes (1028 and up), widths that
-# are and are not multiples of 4
+# beyond what LDS alone holds: backward only (577..1000), both passes (1028 and up), widths
+# that are and are not multiples of 4 (part of the slice in registers, or step by step)
 STEPWISE = [(T, min(N, 140), C, H, z) for T, N, C, H, z in
             _shapes(12, 8, lambda r: r.choice([577, 580, 644, 700, 801, 1028, 1100, 1301, 1537]))]
+# any hidden size from the first that needs registers beside LDS to past the last that fits
+# them, at batch sizes that take tiles of 16, 32 and 64 rows or fall back to single steps
+REGISTER_ROWS = [(min(T, 3), min(N, 260), C, H, z) for T, N, C, H, z in
+                 _shapes(13, 14, lambda r: r.integers(580, 2150))]
 
 
-@pytest.mark.parametrize("T,N,C,H,zoneout", RESIDENT + STEPWISE)
+@pytest.mark.parametrize("T,N,C,H,zoneout", RESIDENT + STEPWISE + REGISTER_ROWS)
 def test_random_sizes_lstm_gru(T, N, C, H, zoneout):
     test_gpu_lstm.test_lstm_training_forward_backward(T, N, C, H, zoneout)
     test_gpu_gru.test_gru_training_forward_backward(T, N, C, H, zoneout)
 
 
-@pytest.mark.parametrize("T,N,C,H,zoneout", RESIDENT + STEPWISE[:4])
+@pytest.mark.parametrize("T,N,C,H,zoneout", RESIDENT + STEPWISE[:4] + REGISTER_ROWS[:6])
 def test_random_sizes_layer_norm_cells(T, N, C, H, zoneout):
     test_gpu_layer_norm_cells.test_layer_norm_lstm_training_forward_backward(T, N, C, H, zoneout)
     test_gpu_layer_norm_cells.test_layer_norm_gru_training_forward_backward(T, N, C, H, zoneout)
