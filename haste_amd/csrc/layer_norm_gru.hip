@@ -115,18 +115,24 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
 
   // Inputs of a step that do not depend on the recurrence, fetched one step ahead.
   float wx_next[PP][3], mk_next[PP];
+  // Every thread loads (threads without an element, and the request after the last step, some
+  // valid address: their values are never used) and nothing but the loads writes these
+  // registers inside the loop (see ln_lstm_forward_kernel).
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp) {
+    mk_next[pp] = 1.f;
+#pragma unroll
+    for (int g = 0; g < 3; ++g) wx_next[pp][g] = 0.f;
+  }
   auto fetch = [&](int t) {
+    const int tt = t < T ? t : T - 1;
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
-      mk_next[pp] = 1.f;
+      const size_t row = act[pp] ? (size_t)pn[pp] : 0, unit = act[pp] ? (size_t)pj[pp] : 0;
+      const float* wt = p.Wxn + ((size_t)tt * N + row) * 3 * H + unit;
 #pragma unroll
-      for (int g = 0; g < 3; ++g) wx_next[pp][g] = 0.f;
-      if (act[pp] && t < T) {
-        const float* wt = p.Wxn + ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
-#pragma unroll
-        for (int g = 0; g < 3; ++g) wx_next[pp][g] = wt[g * H];
-        if (zoneout && p.training) mk_next[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
-      }
+      for (int g = 0; g < 3; ++g) wx_next[pp][g] = wt[g * H];
+      if (zoneout && p.training) mk_next[pp] = p.zoneout_mask[(size_t)tt * NH + row * H + unit];
     }
   };
   fetch(0);
@@ -361,25 +367,30 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
 
   struct StepIn { float vt[4], rh[3], h0, dhn, m, mu2, is2; };
   StepIn nxt[PP];
+  // Every thread loads and nothing but the loads writes `nxt` inside the loop (see
+  // ln_lstm_forward_kernel).
+  {
+    const StepIn nxt_init = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f}, 0.f, 0.f, 1.f, 0.f, 0.f};
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) nxt[pp] = nxt_init;
+  }
   auto fetch = [&](int t) {
+    const int tt = t >= 0 ? t : 0;
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
-      StepIn s = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f}, 0.f, 0.f, 1.f, 0.f, 0.f};
-      if (act[pp] && t >= 0) {
-        const size_t e = (size_t)pn[pp] * H + pj[pp];
-        const float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
-        const float* ar = p.act_Rh + ((size_t)t * N + pn[pp]) * 3 * H + pj[pp];
+      const size_t row = act[pp] ? (size_t)pn[pp] : 0, unit = act[pp] ? (size_t)pj[pp] : 0;
+      const size_t e = row * H + unit;
+      const float* vt = p.v + ((size_t)tt * N + row) * 4 * H + unit;
+      const float* ar = p.act_Rh + ((size_t)tt * N + row) * 3 * H + unit;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) s.vt[g] = vt[(size_t)g * H];
+      for (int g = 0; g < 4; ++g) nxt[pp].vt[g] = vt[(size_t)g * H];
 #pragma unroll
-        for (int g = 0; g < 3; ++g) s.rh[g] = ar[(size_t)g * H];
-        s.h0 = p.h[(size_t)t * NH + e];
-        s.dhn = p.dh_new[(size_t)(t + 1) * NH + e];
-        if (zoneout) s.m = p.zoneout_mask[(size_t)t * NH + e];
-        s.mu2 = p.cache2[((size_t)t * N + pn[pp]) * 2];
-        s.is2 = p.cache2[((size_t)t * N + pn[pp]) * 2 + 1];
-      }
-      nxt[pp] = s;
+      for (int g = 0; g < 3; ++g) nxt[pp].rh[g] = ar[(size_t)g * H];
+      nxt[pp].h0 = p.h[(size_t)tt * NH + e];
+      nxt[pp].dhn = p.dh_new[(size_t)(tt + 1) * NH + e];
+      if (zoneout) nxt[pp].m = p.zoneout_mask[(size_t)tt * NH + e];
+      nxt[pp].mu2 = p.cache2[((size_t)tt * N + row) * 2];
+      nxt[pp].is2 = p.cache2[((size_t)tt * N + row) * 2 + 1];
     }
   };
   fetch(T - 1);

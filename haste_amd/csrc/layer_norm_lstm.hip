@@ -135,18 +135,25 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
 
   // Inputs of a step that do not depend on the recurrence, fetched one step ahead.
   float wx_next[PP][4], mk_next[PP];
+  // Every thread loads (threads without an element, and the request after the last step, some
+  // valid address: their values are never used) and nothing but the loads writes these
+  // registers inside the loop: a default written there first would have to wait for loads a
+  // thread skipped waiting for and, the counter being in order, for the step's stores with them.
+#pragma unroll
+  for (int pp = 0; pp < PP; ++pp) {
+    mk_next[pp] = 1.f;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) wx_next[pp][g] = 0.f;
+  }
   auto fetch = [&](int t) {
+    const int tt = t < T ? t : T - 1;
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
-      mk_next[pp] = 1.f;
+      const size_t row = act[pp] ? (size_t)pn[pp] : 0, unit = act[pp] ? (size_t)pj[pp] : 0;
+      const float* vt = p.v + ((size_t)tt * N + row) * 4 * H + unit;
 #pragma unroll
-      for (int g = 0; g < 4; ++g) wx_next[pp][g] = 0.f;
-      if (act[pp] && t < T) {
-        const float* vt = p.v + ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
-#pragma unroll
-        for (int g = 0; g < 4; ++g) wx_next[pp][g] = vt[g * H];
-        if (zoneout && p.training) mk_next[pp] = p.zoneout_mask[(size_t)t * NH + (size_t)pn[pp] * H + pj[pp]];
-      }
+      for (int g = 0; g < 4; ++g) wx_next[pp][g] = vt[g * H];
+      if (zoneout && p.training) mk_next[pp] = p.zoneout_mask[(size_t)tt * NH + row * H + unit];
     }
   };
   fetch(0);
@@ -416,32 +423,37 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
 
   struct StepIn { float vt[4], rh[4], c0, c1, dhn, dcn, m, cn, mu2, is2, mu3, is3; };
   StepIn nxt[PP];
+  // Every thread loads and nothing but the loads writes `nxt` inside the loop (see the
+  // forward kernel).
+  {
+    const StepIn nxt_init = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, 0.f, 0.f, 0.f, 0.f, 1.f, 0.f,
+                             0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) nxt[pp] = nxt_init;
+  }
   auto fetch = [&](int t) {
+    const int tt = t >= 0 ? t : 0;
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
-      StepIn s = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, 0.f, 0.f, 0.f, 0.f, 1.f, 0.f,
-                  0.f, 0.f, 0.f, 0.f};
-      if (act[pp] && t >= 0) {
-        const size_t e = (size_t)pn[pp] * H + pj[pp];
-        const size_t e4 = ((size_t)t * N + pn[pp]) * 4 * H + pj[pp];
+      const size_t row = act[pp] ? (size_t)pn[pp] : 0, unit = act[pp] ? (size_t)pj[pp] : 0;
+      const size_t e = row * H + unit;
+      const size_t e4 = ((size_t)tt * N + row) * 4 * H + unit;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          s.vt[g] = p.v[e4 + (size_t)g * H];
-          s.rh[g] = p.act_Rh[e4 + (size_t)g * H];
-        }
-        s.c0 = p.c[(size_t)t * NH + e];
-        s.c1 = p.c[(size_t)(t + 1) * NH + e];
-        s.dhn = p.dh_new[(size_t)(t + 1) * NH + e];
-        s.dcn = p.dc_new[(size_t)(t + 1) * NH + e];
-        s.cn = p.act_c_norm[(size_t)t * NH + e];
-        if (zoneout) s.m = p.zoneout_mask[(size_t)t * NH + e];
-        const size_t r = ((size_t)t * N + pn[pp]) * 2;
-        s.mu2 = p.cache2[r];
-        s.is2 = p.cache2[r + 1];
-        s.mu3 = p.cache3[r];
-        s.is3 = p.cache3[r + 1];
+      for (int g = 0; g < 4; ++g) {
+        nxt[pp].vt[g] = p.v[e4 + (size_t)g * H];
+        nxt[pp].rh[g] = p.act_Rh[e4 + (size_t)g * H];
       }
-      nxt[pp] = s;
+      nxt[pp].c0 = p.c[(size_t)tt * NH + e];
+      nxt[pp].c1 = p.c[(size_t)(tt + 1) * NH + e];
+      nxt[pp].dhn = p.dh_new[(size_t)(tt + 1) * NH + e];
+      nxt[pp].dcn = p.dc_new[(size_t)(tt + 1) * NH + e];
+      nxt[pp].cn = p.act_c_norm[(size_t)tt * NH + e];
+      if (zoneout) nxt[pp].m = p.zoneout_mask[(size_t)tt * NH + e];
+      const size_t r = ((size_t)tt * N + row) * 2;
+      nxt[pp].mu2 = p.cache2[r];
+      nxt[pp].is2 = p.cache2[r + 1];
+      nxt[pp].mu3 = p.cache3[r];
+      nxt[pp].is3 = p.cache3[r + 1];
     }
   };
   fetch(T - 1);
