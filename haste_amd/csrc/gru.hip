@@ -291,17 +291,17 @@ void gru_forward_single_row_kernel(GruFwdParams p) {
   group_arrive(gs);
   group_wait(gs);
 
-  float wx_next[3], mk_next;
+  // Every thread loads (a thread without an element, and the request after the last step, some
+  // valid address) and nothing but the loads writes these registers inside the loop (see
+  // lstm_forward_kernel).
+  float wx_next[3] = {0.f, 0.f, 0.f}, mk_next = 1.f;
   auto fetch = [&](int t) {
-    mk_next = 1.f;
+    const int tt = t < T ? t : T - 1;
+    const int unit = act ? pj : 0;
+    const float* wt = p.Wx + (size_t)tt * 3 * H + unit;
 #pragma unroll
-    for (int g = 0; g < 3; ++g) wx_next[g] = 0.f;
-    if (act && t < T) {
-      const float* wt = p.Wx + (size_t)t * 3 * H + pj;
-#pragma unroll
-      for (int g = 0; g < 3; ++g) wx_next[g] = wt[g * H];
-      if (zoneout && p.training) mk_next = p.zoneout_mask[(size_t)t * H + pj];
-    }
+    for (int g = 0; g < 3; ++g) wx_next[g] = wt[g * H];
+    if (zoneout && p.training) mk_next = p.zoneout_mask[(size_t)tt * H + unit];
   };
   fetch(0);
 

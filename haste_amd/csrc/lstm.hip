@@ -324,17 +324,17 @@ void lstm_forward_single_row_kernel(LstmFwdParams p) {
   group_arrive(gs);
   group_wait(gs);
 
-  float wx_next[4], mk_next;
+  // Every thread loads (a thread without an element, and the request after the last step, some
+  // valid address) and nothing but the loads writes these registers inside the loop (see
+  // lstm_forward_kernel).
+  float wx_next[4] = {0.f, 0.f, 0.f, 0.f}, mk_next = 1.f;
   auto fetch = [&](int t) {
-    mk_next = 1.f;
+    const int tt = t < T ? t : T - 1;
+    const int unit = act ? pj : 0;
+    const float* vt = p.v + (size_t)tt * 4 * H + unit;
 #pragma unroll
-    for (int g = 0; g < 4; ++g) wx_next[g] = 0.f;
-    if (act && t < T) {
-      const float* vt = p.v + (size_t)t * 4 * H + pj;
-#pragma unroll
-      for (int g = 0; g < 4; ++g) wx_next[g] = vt[g * H];
-      if (zoneout && p.training) mk_next = p.zoneout_mask[(size_t)t * H + pj];
-    }
+    for (int g = 0; g < 4; ++g) wx_next[g] = vt[g * H];
+    if (zoneout && p.training) mk_next = p.zoneout_mask[(size_t)tt * H + unit];
   };
   fetch(0);
 
