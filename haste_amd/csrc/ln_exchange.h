@@ -50,6 +50,12 @@ __device__ __forceinline__ float wave_sum(float v) {
          __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
 }
 
+// Sum over the lanes of a wavefront, valid in lane 0 at least.  `first_row_only`: only the first
+// 16 lanes hold anything that counts, and every one of them receives the sum of those.
+__device__ __forceinline__ float lanes_sum(float v, bool first_row_only) {
+  return first_row_only ? segment_sum<16>(v) : wave_sum(v);
+}
+
 __device__ __forceinline__ void load_exchanged2(const float* p, float& a, float& b) {
   const unsigned long long bits = __hip_atomic_load(
       reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -203,6 +209,8 @@ __device__ __forceinline__ void merge_row_moments_polled(const GroupSync& g,
   const int wave = threadIdx.x >> 6;
   const TileBuffer slots = make_tile_buffer(reinterpret_cast<float*>(buffer),
                                             (int)tagged_row_words(gx, NB, 2) * 2);
+  const bool narrow = gx <= 16;
+  const float inv_D = 1.0f / D;
   for (int row = wave; row < NB; row += 4) {
     float first[2] = {0.f, 0.f};
     float s1 = 0.f;
@@ -213,7 +221,7 @@ __device__ __forceinline__ void merge_row_moments_polled(const GroupSync& g,
       if (cw < gx) s1 += ((cw == gx - 1) ? last_count : full_count) * v[0];
       if (c0 == 0) { first[0] = v[0]; first[1] = v[1]; }
     }
-    const float mean = wave_sum(s1) / D;
+    const float mean = lanes_sum(s1, narrow) * inv_D;
     float s2 = 0.f;
     for (int c0 = 0; c0 < gx; c0 += 64) {
       const int cw = c0 + lane;
@@ -224,10 +232,12 @@ __device__ __forceinline__ void merge_row_moments_polled(const GroupSync& g,
         s2 += v[1] + ((cw == gx - 1) ? last_count : full_count) * d * d;
       }
     }
-    const float m2 = wave_sum(s2);
+    const float m2 = lanes_sum(s2, narrow);
     if (lane == 0) {
       out[row * 2 + 0] = mean;
-      out[row * 2 + 1] = 1.0f / sqrtf(m2 / D + kLnEps);
+      // the hardware's reciprocal square root (1 ulp), as the reference's rsqrt
+      // (lib/layer_norm_forward_gpu.cu.cc:77)
+      out[row * 2 + 1] = __builtin_amdgcn_rsqf(m2 * inv_D + kLnEps);
     }
   }
 }
@@ -253,9 +263,9 @@ __device__ __forceinline__ void sum_row_partials_polled(const GroupSync& g,
         s2 += v[2];
       }
     }
-    s0 = wave_sum(s0);
-    s1 = wave_sum(s1);
-    s2 = wave_sum(s2);
+    s0 = lanes_sum(s0, gx <= 16);
+    s1 = lanes_sum(s1, gx <= 16);
+    s2 = lanes_sum(s2, gx <= 16);
     if (lane == 0) {
       out[row * 4 + 0] = s0;
       out[row * 4 + 1] = s1;
