@@ -5,8 +5,10 @@
 // columns and on the new cell state over H columns) are computed inside the step:
 // each workgroup reduces its own columns, the group exchanges per-row moments, and a
 // step therefore has three group barriers (h_t ready, norm of h*R, norm of c).
-// Backward mirrors it in reverse time (three barriers per step as well), then one
-// stand-alone layer-norm backward over all rows and the three batched GEMMs.
+// Backward mirrors it in reverse time with two waits per step: the row sums of both norms
+// travel in one exchange (those of the h*R norm as coefficients, see the step), then the
+// gradient w.r.t. h*R.  One stand-alone layer-norm backward over all rows and the three
+// batched GEMMs follow.
 //
 // Arithmetic follows reference lib/layer_norm_lstm_forward_gpu.cu.cc:50-71,95-108 and
 // lib/layer_norm_lstm_backward_gpu.cu.cc:44-64,84-117; orchestration replaces
@@ -318,8 +320,7 @@ struct LnLstmBwdParams {
   const float* cache3;     // [T*N,2]
   const float* act_c_norm; // [T,N,H]
   const float* zoneout_mask;
-  unsigned long long* part_a;  // tagged row exchange [groups][2][gx][NB][3] words: cell-state norm sums
-  unsigned long long* part_b;  // tagged row exchange [groups][2][gx][NB][3] words: h*R norm sums
+  unsigned long long* part;    // tagged row exchange [groups][2][gx][NB][10] words: the sums of both norms
   float* col_partial;      // [batch tiles][10][H]
   float* xd;               // polled exchange tiles of the gradient w.r.t. h*R: [batch tiles][4][Kpad/4][NB][4]
   LaunchShape ls;
@@ -334,6 +335,7 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   constexpr int NCOLS = 16;
   constexpr int PP = (NB * HSB + 255) / 256;
   constexpr int NACC = 10;  // db x4, dgamma2 x4, dgamma_h, dbeta_h
+  constexpr int kRowValues = 10;  // floats per row and workgroup in the step's row exchange
   constexpr int RED = NB * NACC * HSB > ProductTile<NB, 1>::kRedFloats
                           ? NB * NACC * HSB : ProductTile<NB, 1>::kRedFloats;
   extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -346,8 +348,7 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   const int Kpad = 64 * p.ls.gx;  // k = 4*unit + gate over the 16 units of every workgroup
   float* w_lds = lds;
   float* red = lds + (Kpad - 64 * REG) * NCOLS;  // the partial tiles, reused for the column sums
-  float* sums_a = red + RED;         // [NB][4] row sums of the cell-state norm
-  float* sums_b = sums_a + 4 * NB;   // [NB][4] row sums of the h*R norm
+  float* sums = red + RED;           // [NB][10] row sums of the two norms (see the step)
 
   const int tid = threadIdx.x;
   const int gx = p.ls.gx;
@@ -355,9 +356,8 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   const int n0 = role.bt * p.ls.tile_rows;
   const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
-  const size_t row_words = tagged_row_words(gx, NB, 3);
-  unsigned long long* part_a = p.part_a + (size_t)role.bt * 2 * row_words;
-  unsigned long long* part_b = p.part_b + (size_t)role.bt * 2 * row_words;
+  const size_t row_words = tagged_row_words(gx, NB, kRowValues);
+  unsigned long long* part = p.part + (size_t)role.bt * 2 * row_words;
 
   const int tile_floats = Kpad * NB;
   float* xd = p.xd + (size_t)role.bt * kPolledTiles * tile_floats;
@@ -365,8 +365,7 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
 
   GroupSync gs;
   group_sync_init(gs, p.ls, role);
-  clear_row_words(gs, part_a, gx, role.cw, NB, 3);
-  clear_row_words(gs, part_b, gx, role.cw, NB, 3);
+  clear_row_words(gs, part, gx, role.cw, NB, kRowValues);
 
   static_assert(REG == 0 || NB >= 16, "register-resident slice rows: tall tiles only");
   float4_t breg[REG > 0 ? REG : 1][1];
@@ -462,15 +461,25 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   const float inv4H = 1.0f / (float)(4 * H);
   for (int t = T - 1; t >= 0; --t) {
     StepIn s[PP];
-    float dh_keep[PP], dv_o[PP], xc3[PP], gd3[PP];
+    float dh_keep[PP], dv_o[PP], xc3[PP], gd3[PP], xc2[PP][4];
     const int done = T - 1 - t;  // steps done so far
-    const unsigned int tag = gs.epoch + 2u + (unsigned int)done;  // names this step's row exchanges
-    unsigned long long* ex_a = part_a + (size_t)(done & 1) * row_words;
-    unsigned long long* ex_b = part_b + (size_t)(done & 1) * row_words;
+    const unsigned int tag = gs.epoch + 2u + (unsigned int)done;  // names this step's row exchange
+    unsigned long long* ex = part + (size_t)(done & 1) * row_words;
+    // One row exchange serves both norms.  The sums of the h*R norm are taken over the gate
+    // gradients dv, and those depend on the row sums of the cell-state norm (through dsigma and
+    // dmu below) -- but linearly: dc_total = base + X * dsigma + dmu / H per unit, dv = k *
+    // dc_total for the gates i, g, f.  So every workgroup publishes, beside its parts of the
+    // cell-state sums, its parts of the h*R sums as coefficients of (1, dsigma, dmu / H), and
+    // every reader puts the totals together once it knows dsigma and dmu.
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
       s[pp] = nxt[pp];
       dh_keep[pp] = dv_o[pp] = xc3[pp] = gd3[pp] = 0.f;
+      float part_sum[kRowValues];
+#pragma unroll
+      for (int i = 0; i < kRowValues; ++i) part_sum[i] = 0.f;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) xc2[pp][g] = 0.f;
       if (act[pp]) {
         float dh_total = s[pp].dhn + dh[pp];
         if (zoneout) {
@@ -486,28 +495,51 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
         gd3[pp] = gh[pp] * dln3;
         accs[pp][8] += xc3[pp] * s[pp].is3 * dln3;
         accs[pp][9] += dln3;
+
+        const float gi = s[pp].vt[0], gg = s[pp].vt[1], gf = s[pp].vt[2];
+        const float base = s[pp].dcn + dc[pp] + s[pp].is3 * gd3[pp];
+        const float X = 2.0f * xc3[pp] * invH;
+        const float k[3] = {d_sigmoid_f(gi) * gg, d_tanh_f(gg) * gi, d_sigmoid_f(gf) * s[pp].c0};
+        float F = 0.f, G = 0.f, x2 = 0.f;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          xc2[pp][g] = s[pp].rh[g] - s[pp].mu2;
+          x2 += xc2[pp][g];
+        }
+#pragma unroll
+        for (int g = 0; g < 3; ++g) {
+          F += xc2[pp][g] * g2[pp][g] * k[g];
+          G += g2[pp][g] * k[g];
+        }
+        const float e2 = g2[pp][3] * dv_o[pp];
+        part_sum[0] = xc3[pp] * gd3[pp];
+        part_sum[1] = xc3[pp];
+        part_sum[2] = gd3[pp];
+        part_sum[3] = xc2[pp][3] * e2 + F * base;
+        part_sum[4] = F * X;
+        part_sum[5] = F;
+        part_sum[6] = x2;
+        part_sum[7] = e2 + G * base;
+        part_sum[8] = G * X;
+        part_sum[9] = G;
       }
-      const float s0 = segment_sum<HSB>(xc3[pp] * gd3[pp]);
-      const float s1 = segment_sum<HSB>(xc3[pp]);
-      const float s2 = segment_sum<HSB>(gd3[pp]);
-      if (pc[pp] == 0 && own[pp]) {
-        const float v3[3] = {s0, s1, s2};
-        publish_row<3>(gs, ex_a, NB, role.cw, pl[pp], v3, tag);
-      }
+#pragma unroll
+      for (int i = 0; i < kRowValues; ++i) part_sum[i] = segment_sum<HSB>(part_sum[i]);
+      if (pc[pp] == 0 && own[pp]) publish_row<kRowValues>(gs, ex, NB, role.cw, pl[pp], part_sum, tag);
     }
-    sum_row_partials_polled<NB>(gs, ex_a, gx, tag, sums_a);  // row sums of the cell-state norm
+    sum_row_values_polled<NB, kRowValues>(gs, ex, gx, tag, sums);
     __syncthreads();
 
-    float xc2[PP][4], gd2[PP][4], dvs[PP][4];
+    float gd2[PP][4], dvs[PP][4], dr[PP][4];
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
-      float t0 = 0.f, t1 = 0.f, t2 = 0.f;
 #pragma unroll
-      for (int g = 0; g < 4; ++g) xc2[pp][g] = gd2[pp][g] = dvs[pp][g] = 0.f;
+      for (int g = 0; g < 4; ++g) gd2[pp][g] = dvs[pp][g] = dr[pp][g] = 0.f;
       if (act[pp]) {
+        const float* rs = sums + pl[pp] * RowSlot<kRowValues>::kWords;
         const float is3 = s[pp].is3;
-        const float dsigma = -0.5f * sums_a[pl[pp] * 4 + 0] * is3 * is3 * is3;
-        const float dmu = (-2.0f * sums_a[pl[pp] * 4 + 1] * dsigma * invH) - (sums_a[pl[pp] * 4 + 2] * is3);
+        const float dsigma = -0.5f * rs[0] * is3 * is3 * is3;
+        const float dmu = (-2.0f * rs[1] * dsigma * invH) - (rs[2] * is3);
         const float dc_ln = (2.0f * xc3[pp] * dsigma * invH) + (is3 * gd3[pp]) + (dmu * invH);
         const float gi = s[pp].vt[0], gg = s[pp].vt[1], gf = s[pp].vt[2];
         const float dc_total = s[pp].dcn + dc[pp] + dc_ln;
@@ -524,37 +556,20 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
         for (int g = 0; g < 4; ++g) {
           dvs[pp][g] = dv[g];
           accs[pp][g] += dv[g];
-          xc2[pp][g] = s[pp].rh[g] - s[pp].mu2;
           gd2[pp][g] = g2[pp][g] * dv[g];
           accs[pp][4 + g] += xc2[pp][g] * s[pp].is2 * dv[g];
-          t0 += xc2[pp][g] * gd2[pp][g];
-          t1 += xc2[pp][g];
-          t2 += gd2[pp][g];
         }
-      }
-      t0 = segment_sum<HSB>(t0);
-      t1 = segment_sum<HSB>(t1);
-      t2 = segment_sum<HSB>(t2);
-      if (pc[pp] == 0 && own[pp]) {
-        const float v3[3] = {t0, t1, t2};
-        publish_row<3>(gs, ex_b, NB, role.cw, pl[pp], v3, tag);
-      }
-    }
-    sum_row_partials_polled<NB>(gs, ex_b, gx, tag, sums_b);  // row sums of the h*R norm
-    __syncthreads();
-
-    float dr[PP][4];
-#pragma unroll
-    for (int pp = 0; pp < PP; ++pp) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) dr[pp][g] = 0.f;
-      if (act[pp]) {
+        // the row sums of the h*R norm from their coefficients
+        const float dmuH = dmu * invH;
+        const float t0 = rs[3] + dsigma * rs[4] + dmuH * rs[5];
+        const float t1 = rs[6];
+        const float t2 = rs[7] + dsigma * rs[8] + dmuH * rs[9];
         const float is2 = s[pp].is2;
-        const float dsigma = -0.5f * sums_b[pl[pp] * 4 + 0] * is2 * is2 * is2;
-        const float dmu = (-2.0f * sums_b[pl[pp] * 4 + 1] * dsigma * inv4H) - (sums_b[pl[pp] * 4 + 2] * is2);
+        const float dsigma2 = -0.5f * t0 * is2 * is2 * is2;
+        const float dmu2 = (-2.0f * t1 * dsigma2 * inv4H) - (t2 * is2);
 #pragma unroll
         for (int g = 0; g < 4; ++g)
-          dr[pp][g] = (2.0f * xc2[pp][g] * dsigma * inv4H) + (is2 * gd2[pp][g]) + (dmu * inv4H);
+          dr[pp][g] = (2.0f * xc2[pp][g] * dsigma2 * inv4H) + (is2 * gd2[pp][g]) + (dmu2 * inv4H);
       }
     }
     // What this wavefront stored during the previous step (its resets among it) has landed
@@ -729,8 +744,8 @@ int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_
   HASTE_HIP_REQUIRE(act_Wx_norm && act_Rh && gamma2 && dgamma2 && cache2 && gamma_h);
   HASTE_HIP_REQUIRE(dgamma_h && dbeta_h && cache3 && act_c_norm);
   hipStream_t stream = as_stream(stream_);
-  // per row: 10 column-sum accumulators of 16 floats (or the partial tiles, whichever is more) + 4 sums
-  const BackwardTile tile = pick_backward_tile(4 * H, N, H, 10 * 16, 8, resident_rows_enabled());
+  // per row: 10 column-sum accumulators of 16 floats (or the partial tiles, whichever is more) + 10 sums
+  const BackwardTile tile = pick_backward_tile(4 * H, N, H, 10 * 16, 10, resident_rows_enabled());
   if (!tile.ok)
     return layer_norm_lstm_backward_streamed(stream, T, N, C, H, W_t, R_t, x_t, h, c, dh_new, dc_new,
                                              dx, dW, dR, db, dh, dc, act_Wx, gamma1, dgamma1,
@@ -739,13 +754,13 @@ int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_
   const int gx = tile.gx, gy = tile.gy;
   const int NB = tile.nb;
   // one tagged row exchange: [groups][2] buffers of 8-byte words, counted in floats
-  const size_t part_floats = (size_t)gy * 2 * tagged_row_words(gx, NB, 3) * 2;
+  const size_t part_floats = (size_t)gy * 2 * tagged_row_words(gx, NB, 10) * 2;
   const size_t col_floats = (size_t)gy * 10 * H;
   const size_t col_floats4 = (col_floats + 3) / 4 * 4;
 
   Workspace ws;
   const size_t xd_floats = exchange_floats(64 * gx, NB, gy, kPolledTiles);
-  HASTE_HIP_PROPAGATE(get_workspace(stream, (2 * part_floats + col_floats4 + xd_floats) * sizeof(float), &ws));
+  HASTE_HIP_PROPAGATE(get_workspace(stream, (part_floats + col_floats4 + xd_floats) * sizeof(float), &ws));
   HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 
   LnLstmBwdParams p;
@@ -755,10 +770,9 @@ int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_
   p.gamma2 = gamma2; p.dgamma2 = dgamma2; p.cache2 = cache2;
   p.gamma_h = gamma_h; p.dgamma_h = dgamma_h; p.dbeta_h = dbeta_h; p.cache3 = cache3;
   p.act_c_norm = act_c_norm; p.zoneout_mask = zoneout_mask;
-  p.part_a = reinterpret_cast<unsigned long long*>(ws.scratch);
-  p.part_b = reinterpret_cast<unsigned long long*>(ws.scratch + part_floats);
-  p.col_partial = ws.scratch + 2 * part_floats;
-  p.xd = ws.scratch + 2 * part_floats + col_floats4;
+  p.part = reinterpret_cast<unsigned long long*>(ws.scratch);
+  p.col_partial = ws.scratch + part_floats;
+  p.xd = ws.scratch + part_floats + col_floats4;
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes, 3u * (unsigned)T + 1, &plan));
   p.ls = plan.shape;

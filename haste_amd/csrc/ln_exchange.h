@@ -50,10 +50,24 @@ __device__ __forceinline__ float wave_sum(float v) {
          __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
 }
 
-// Sum over the lanes of a wavefront, valid in lane 0 at least.  `first_row_only`: only the first
-// 16 lanes hold anything that counts, and every one of them receives the sum of those.
+// Sums over the lanes of a wavefront of W values at once, valid in lane 0 at least.
+// `first_row_only`: only the first 16 lanes hold anything that counts, and every one of them
+// receives the sums of those.  One branch for all values, so that their chains of cross-lane
+// adds interleave instead of each waiting out its own hazards.
+template <int W>
+__device__ __forceinline__ void lanes_sums(float (&v)[W], bool first_row_only) {
+  if (first_row_only) {
+#pragma unroll
+    for (int i = 0; i < W; ++i) v[i] = segment_sum<16>(v[i]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < W; ++i) v[i] = wave_sum(v[i]);
+  }
+}
 __device__ __forceinline__ float lanes_sum(float v, bool first_row_only) {
-  return first_row_only ? segment_sum<16>(v) : wave_sum(v);
+  float one[1] = {v};
+  lanes_sums<1>(one, first_row_only);
+  return one[0];
 }
 
 __device__ __forceinline__ void load_exchanged2(const float* p, float& a, float& b) {
@@ -117,12 +131,12 @@ __device__ __forceinline__ void merge_row_moments(const float* part, int gx, flo
 // Two buffers alternate by use parity: a workgroup publishes use u+2 only after it has read
 // every contribution to use u+1, and those were published after their authors had read use u,
 // so nobody can still be reading the words that use u+2 overwrites.  Layout of one buffer:
-// [gx][NB] slots of WS = 2 or 4 words (W values, padded to a 16-byte multiple so that a slot
+// [gx][NB] slots of WS words (W values, padded to an even count so that a slot
 // is written and read with 16-byte accesses); a workgroup's slots share lines with nobody.
-template <int W> struct RowSlot { static constexpr int kWords = W <= 2 ? 2 : 4; };
+template <int W> struct RowSlot { static constexpr int kWords = (W + 1) / 2 * 2; };
 
 __host__ __device__ __forceinline__ size_t tagged_row_words(int gx, int nb, int w) {
-  return (size_t)gx * nb * (w <= 2 ? 2 : 4);
+  return (size_t)gx * nb * ((w + 1) / 2 * 2);
 }
 
 typedef unsigned int uint4_row_t __attribute__((ext_vector_type(4)));
@@ -158,7 +172,7 @@ __device__ __forceinline__ void publish_row(const GroupSync& g, unsigned long lo
 // before the launch's initial barrier.
 __device__ __forceinline__ void clear_row_words(const GroupSync& g, unsigned long long* both, int gx,
                                                 int cw, int nb, int w) {
-  const int ws = w <= 2 ? 2 : 4;
+  const int ws = (w + 1) / 2 * 2;
   for (int i = threadIdx.x; i < 2 * nb * ws; i += 256) {
     unsigned long long* q = both + (size_t)(i / (nb * ws)) * tagged_row_words(gx, nb, w) +
                             (size_t)cw * nb * ws + i % (nb * ws);
@@ -180,15 +194,20 @@ __device__ __forceinline__ void load_row_polled(const GroupSync& g, const TileBu
   const int word = ((have ? cw : 0) * nb + row) * WS;
   bool ok = !have;
   auto load = [&] {
-    bool all = true;
+    // All of a slot's loads are issued before any tag is looked at, and the tags are combined
+    // without branches: with `&&` the compiler makes a load wait for the previous one's tag.
+    uint4_t u[WS / 2];
+#pragma unroll
+    for (int i = 0; i < WS; i += 2)
+      u[i / 2] = __builtin_amdgcn_raw_buffer_load_b128(slots.rsrc, (word + i) * 8, 0, 16);
+    unsigned int differ = 0u;
 #pragma unroll
     for (int i = 0; i < WS; i += 2) {
-      const uint4_t u = __builtin_amdgcn_raw_buffer_load_b128(slots.rsrc, (word + i) * 8, 0, 16);
-      v[i] = __uint_as_float(u.x);
-      if (i + 1 < W) v[i + 1 < W ? i + 1 : i] = __uint_as_float(u.z);
-      all = all && u.y == tag && u.w == tag;
+      v[i] = __uint_as_float(u[i / 2].x);
+      if (i + 1 < W) v[i + 1 < W ? i + 1 : i] = __uint_as_float(u[i / 2].z);
+      differ |= (u[i / 2].y ^ tag) | (u[i / 2].w ^ tag);
     }
-    ok = !have || all;
+    ok = !have || differ == 0u;
   };
   if (have) load();
     poll_until_written(g, [&] { __builtin_amdgcn_s_sleep(1); load(); }, [&] { return __all(ok) != 0; });
@@ -263,13 +282,43 @@ __device__ __forceinline__ void sum_row_partials_polled(const GroupSync& g,
         s2 += v[2];
       }
     }
-    s0 = lanes_sum(s0, gx <= 16);
-    s1 = lanes_sum(s1, gx <= 16);
-    s2 = lanes_sum(s2, gx <= 16);
+    float s[3] = {s0, s1, s2};
+    lanes_sums<3>(s, gx <= 16);
     if (lane == 0) {
-      out[row * 4 + 0] = s0;
-      out[row * 4 + 1] = s1;
-      out[row * 4 + 2] = s2;
+      out[row * 4 + 0] = s[0];
+      out[row * 4 + 1] = s[1];
+      out[row * 4 + 2] = s[2];
+    }
+  }
+}
+
+// Row sums of W values per slot from a tagged buffer: out[row * RowSlot<W>::kWords + i] in LDS.
+// Same calling rules as sum_row_partials_polled.
+template <int NB, int W>
+__device__ __forceinline__ void sum_row_values_polled(const GroupSync& g, unsigned long long* buffer,
+                                                      int gx, unsigned int tag, float* out) {
+  constexpr int WS = RowSlot<W>::kWords;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const TileBuffer slots = make_tile_buffer(reinterpret_cast<float*>(buffer),
+                                            (int)tagged_row_words(gx, NB, W) * 2);
+  for (int row = wave; row < NB; row += 4) {
+    float s[W];
+#pragma unroll
+    for (int i = 0; i < W; ++i) s[i] = 0.f;
+    for (int c0 = 0; c0 < gx; c0 += 64) {
+      const int cw = c0 + lane;
+      float v[W];
+      load_row_polled<W>(g, slots, NB, cw, row, cw < gx, tag, v);
+      if (cw < gx) {
+#pragma unroll
+        for (int i = 0; i < W; ++i) s[i] += v[i];
+      }
+    }
+    lanes_sums<W>(s, gx <= 16);
+    if (lane == 0) {
+#pragma unroll
+      for (int i = 0; i < W; ++i) out[row * WS + i] = s[i];
     }
   }
 }
