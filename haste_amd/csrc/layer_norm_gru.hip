@@ -46,10 +46,11 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
   const int Kpad = round_up(H, 64);
   float* w_lds = lds;
   float* red = lds + Kpad * NCOLS;
-  float* stat = red + ProductTile<NB, CT>::kRedFloats;
+  float* stat = red + ProductTile<NB, CT>::kRedFloats;  // [NB][2] row statistics (long rows only)
 
   const int tid = threadIdx.x;
   const int gx = p.ls.gx;
+  const bool in_wavefront = row_gather_in_wavefront<HS>(gx);
   const int j0 = role.cw * HS;
   const int n0 = role.bt * p.ls.tile_rows;
   const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
@@ -174,14 +175,23 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
         publish_row<2>(gs, ex2, NB, role.cw, pl[pp], mq, tag);
       }
     }
-    merge_row_moments_polled<NB>(gs, ex2, gx, tag, 3.0f * HS, 3.0f * last_units, 3.0f * H, stat);
-    __syncthreads();
-
     float saved[PP][4], mu2[PP], is2[PP], h_pub[PP];
+    if (in_wavefront) {
+#pragma unroll
+      for (int pp = 0; pp < PP; ++pp)
+        gather_row_moments<HS>(gs, ex2, NB, gx, tag, 3.0f * HS, 3.0f * last_units, 3.0f * H, pl[pp],
+                               tid + 256 * pp < NB * HS, mu2[pp], is2[pp]);
+    } else {
+      merge_row_moments_polled<NB>(gs, ex2, gx, tag, 3.0f * HS, 3.0f * last_units, 3.0f * H, stat);
+      __syncthreads();
+#pragma unroll
+      for (int pp = 0; pp < PP; ++pp) {
+        mu2[pp] = stat[pl[pp] * 2];
+        is2[pp] = stat[pl[pp] * 2 + 1];
+      }
+    }
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
-      mu2[pp] = stat[pl[pp] * 2];
-      is2[pp] = stat[pl[pp] * 2 + 1];
 #pragma unroll
       for (int g = 0; g < 4; ++g) saved[pp][g] = 0.f;
       if (act[pp]) {
@@ -291,7 +301,7 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
   const int Kpad = round_up(48 * p.ls.gx, 64);
   float* w_lds = lds;
   float* red = lds + (Kpad - 64 * REG) * NCOLS;  // the partial tiles, reused for the column sums
-  float* sums = red + RED;           // [NB][4]
+  float* sums = red + RED;           // [NB][4] row sums of the norm (long rows only)
 
   const int tid = threadIdx.x;
   const int gx = p.ls.gx;
@@ -299,6 +309,7 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
   const int n0 = role.bt * p.ls.tile_rows;
   const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
+  const bool in_wavefront = row_gather_in_wavefront<HSB>(gx);
   const size_t row_words = tagged_row_words(gx, NB, 3);
   unsigned long long* part = p.part + (size_t)role.bt * 2 * row_words;
 
@@ -454,15 +465,23 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
         publish_row<3>(gs, ex, NB, role.cw, pl[pp], v3, tag);
       }
     }
-    sum_row_partials_polled<NB>(gs, ex, gx, tag, sums);
-    __syncthreads();
-
+    if (!in_wavefront) {
+      sum_row_partials_polled<NB>(gs, ex, gx, tag, sums);
+      __syncthreads();
+    }
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
+      float rs[3];
+      if (in_wavefront) {
+        gather_row_sums<HSB, 3>(gs, ex, NB, gx, tag, pl[pp], own[pp], rs);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 3; ++i) rs[i] = sums[pl[pp] * 4 + i];
+      }
       if (act[pp]) {
         const float is2 = s[pp].is2;
-        const float dsigma = -0.5f * sums[pl[pp] * 4 + 0] * is2 * is2 * is2;
-        const float dmu = (-2.0f * sums[pl[pp] * 4 + 1] * dsigma * inv3H) - (sums[pl[pp] * 4 + 2] * is2);
+        const float dsigma = -0.5f * rs[0] * is2 * is2 * is2;
+        const float dmu = (-2.0f * rs[1] * dsigma * inv3H) - (rs[2] * is2);
 #pragma unroll
         for (int k = 0; k < 3; ++k)
           dqs[pp][k] = (2.0f * xc[pp][k] * dsigma * inv3H) + (is2 * gd[pp][k]) + (dmu * inv3H);
@@ -507,7 +526,7 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp)
       dh[pp] = dh_keep[pp] + sum_product<NB, 1>(red, pl[pp], pc[pp]);
-    __syncthreads();  // sums (and red) may be overwritten by the next step
+    __syncthreads();  // red may be overwritten by the next step
   }
 
 #pragma unroll

@@ -56,11 +56,11 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
   const int Kpad = round_up(H, 64);
   float* w_lds = lds;
   float* red = lds + Kpad * NCOLS;
-  float* stat2 = red + ProductTile<NB, CT>::kRedFloats;  // [NB][2] statistics of h*R
-  float* stat3 = stat2 + 2 * NB;                          // [NB][2] statistics of c
+  float* stat = red + ProductTile<NB, CT>::kRedFloats;  // [2][NB][2] row statistics (long rows only)
 
   const int tid = threadIdx.x;
   const int gx = p.ls.gx;
+  const bool in_wavefront = row_gather_in_wavefront<HS>(gx);
   const int j0 = role.cw * HS;
   const int n0 = role.bt * p.ls.tile_rows;
   const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
@@ -200,14 +200,23 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
         publish_row<2>(gs, ex2, NB, role.cw, pl[pp], mq, tag);
       }
     }
-    merge_row_moments_polled<NB>(gs, ex2, gx, tag, 4.0f * HS, 4.0f * last_units, 4.0f * H, stat2);
-    __syncthreads();
-
     float gate[PP][4], c_new[PP], mu2[PP], is2[PP];
+    if (in_wavefront) {
+#pragma unroll
+      for (int pp = 0; pp < PP; ++pp)
+        gather_row_moments<HS>(gs, ex2, NB, gx, tag, 4.0f * HS, 4.0f * last_units, 4.0f * H, pl[pp],
+                               tid + 256 * pp < NB * HS, mu2[pp], is2[pp]);
+    } else {
+      merge_row_moments_polled<NB>(gs, ex2, gx, tag, 4.0f * HS, 4.0f * last_units, 4.0f * H, stat);
+      __syncthreads();
+#pragma unroll
+      for (int pp = 0; pp < PP; ++pp) {
+        mu2[pp] = stat[pl[pp] * 2];
+        is2[pp] = stat[pl[pp] * 2 + 1];
+      }
+    }
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
-      mu2[pp] = stat2[pl[pp] * 2];
-      is2[pp] = stat2[pl[pp] * 2 + 1];
       c_new[pp] = 0.f;
 #pragma unroll
       for (int g = 0; g < 4; ++g) gate[pp][g] = 0.f;
@@ -233,14 +242,24 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
         publish_row<2>(gs, ex3, NB, role.cw, pl[pp], mq, tag);
       }
     }
-    merge_row_moments_polled<NB>(gs, ex3, gx, tag, (float)HS, (float)last_units, (float)H, stat3);
-    __syncthreads();
-
     float cn[PP], mu3[PP], is3[PP], h_pub[PP];
+    if (in_wavefront) {
+#pragma unroll
+      for (int pp = 0; pp < PP; ++pp)
+        gather_row_moments<HS>(gs, ex3, NB, gx, tag, (float)HS, (float)last_units, (float)H, pl[pp],
+                               tid + 256 * pp < NB * HS, mu3[pp], is3[pp]);
+    } else {
+      // the second half of `stat`: a fast wavefront may be here while a slow one still reads the first
+      merge_row_moments_polled<NB>(gs, ex3, gx, tag, (float)HS, (float)last_units, (float)H, stat + 2 * NB);
+      __syncthreads();
+#pragma unroll
+      for (int pp = 0; pp < PP; ++pp) {
+        mu3[pp] = stat[2 * NB + pl[pp] * 2];
+        is3[pp] = stat[2 * NB + pl[pp] * 2 + 1];
+      }
+    }
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
-      mu3[pp] = stat3[pl[pp] * 2];
-      is3[pp] = stat3[pl[pp] * 2 + 1];
       cn[pp] = 0.f;
       if (act[pp]) {
         cn[pp] = (c_new[pp] - mu3[pp]) * is3[pp] * gh[pp] + bh[pp];
@@ -268,7 +287,7 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
         }
     }
     fetch(t + 1);
-    __syncthreads();  // red, stat2 and stat3 may be overwritten by the next step
+    __syncthreads();  // red and stat may be overwritten by the next step
     // The caller's copies are written last: nobody in the launch waits for them.
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
@@ -348,7 +367,7 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   const int Kpad = 64 * p.ls.gx;  // k = 4*unit + gate over the 16 units of every workgroup
   float* w_lds = lds;
   float* red = lds + (Kpad - 64 * REG) * NCOLS;  // the partial tiles, reused for the column sums
-  float* sums = red + RED;           // [NB][10] row sums of the two norms (see the step)
+  float* sums = red + RED;           // [NB][10] row sums of the two norms (long rows only)
 
   const int tid = threadIdx.x;
   const int gx = p.ls.gx;
@@ -356,6 +375,7 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
   const int n0 = role.bt * p.ls.tile_rows;
   const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
+  const bool in_wavefront = row_gather_in_wavefront<HSB>(gx);
   const size_t row_words = tagged_row_words(gx, NB, kRowValues);
   unsigned long long* part = p.part + (size_t)role.bt * 2 * row_words;
 
@@ -527,16 +547,23 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
       for (int i = 0; i < kRowValues; ++i) part_sum[i] = segment_sum<HSB>(part_sum[i]);
       if (pc[pp] == 0 && own[pp]) publish_row<kRowValues>(gs, ex, NB, role.cw, pl[pp], part_sum, tag);
     }
-    sum_row_values_polled<NB, kRowValues>(gs, ex, gx, tag, sums);
-    __syncthreads();
-
     float gd2[PP][4], dvs[PP][4], dr[PP][4];
+    if (!in_wavefront) {
+      sum_row_values_polled<NB, kRowValues>(gs, ex, gx, tag, sums);
+      __syncthreads();
+    }
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
+      float rs[kRowValues];
+      if (in_wavefront) {
+        gather_row_sums<HSB, kRowValues>(gs, ex, NB, gx, tag, pl[pp], own[pp], rs);
+      } else {
+#pragma unroll
+        for (int i = 0; i < kRowValues; ++i) rs[i] = sums[pl[pp] * RowSlot<kRowValues>::kWords + i];
+      }
 #pragma unroll
       for (int g = 0; g < 4; ++g) gd2[pp][g] = dvs[pp][g] = dr[pp][g] = 0.f;
       if (act[pp]) {
-        const float* rs = sums + pl[pp] * RowSlot<kRowValues>::kWords;
         const float is3 = s[pp].is3;
         const float dsigma = -0.5f * rs[0] * is3 * is3 * is3;
         const float dmu = (-2.0f * rs[1] * dsigma * invH) - (rs[2] * is3);
@@ -614,6 +641,7 @@ void ln_lstm_backward_kernel(LnLstmBwdParams p) {
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp)
       dh[pp] = dh_keep[pp] + sum_product<NB, 1>(red, pl[pp], pc[pp]);
+    __syncthreads();  // red may be overwritten by the next step
   }
 
 #pragma unroll

@@ -12,6 +12,8 @@
 // Backward: contributions are the three sums of lib/layer_norm_backward_gpu.cu.cc:49-78.
 #pragma once
 
+#include <type_traits>
+
 #include "recurrent.h"
 
 namespace haste_hip {
@@ -290,6 +292,131 @@ __device__ __forceinline__ void sum_row_partials_polled(const GroupSync& g,
       out[row * 4 + 2] = s[2];
     }
   }
+}
+
+// ---- gathers that stay inside the wavefront ---------------------------------------------
+// The threads that work on the elements of a row are HS consecutive lanes (thread / HS is the
+// row, HS a power of two up to 16), and they are the only ones that need the row's statistics.
+// So those lanes gather them: lane c of the segment reads the slots of the column workgroups
+// c, c + HS, ... and the segment adds up with DPP row operations, after which every lane of
+// the segment holds the row's totals -- no LDS, no workgroup barrier, and wavefronts without
+// elements do not take part.  Every workgroup adds in the same order, so all of them obtain
+// bit-identical results.  For rows of at most 4 * HS parts (row_gather_in_wavefront); longer
+// rows take the gathers below, which put all 64 lanes of a wavefront on one row and hand the
+// result over through LDS.
+template <int HS>
+__device__ __forceinline__ bool row_gather_in_wavefront(int gx) { return gx <= 4 * HS; }
+
+// The slots of `row` from the column workgroups cw0, cw0 + step, ... (NCH of them, those beyond
+// gx skipped), all loads in flight together and re-issued until every tag matches.
+template <int W, int NCH>
+__device__ __forceinline__ void load_row_chunks_polled(const GroupSync& g, const TileBuffer& slots,
+                                                       int nb, int cw0, int step, int gx, int row,
+                                                       bool have_row, unsigned int tag,
+                                                       float (&v)[NCH][W]) {
+  constexpr int WS = RowSlot<W>::kWords;
+  bool have[NCH];
+  int word[NCH];
+#pragma unroll
+  for (int ch = 0; ch < NCH; ++ch) {
+    const int cw = cw0 + ch * step;
+    have[ch] = have_row && cw < gx;
+    word[ch] = have[ch] ? (cw * nb + row) * WS : 0;
+  }
+  bool ok = false;
+  auto load = [&] {
+    uint4_t u[NCH][WS / 2];
+#pragma unroll
+    for (int ch = 0; ch < NCH; ++ch)
+#pragma unroll
+      for (int i = 0; i < WS; i += 2)
+        u[ch][i / 2] = __builtin_amdgcn_raw_buffer_load_b128(slots.rsrc, (word[ch] + i) * 8, 0, 16);
+    unsigned int differ = 0u;
+#pragma unroll
+    for (int ch = 0; ch < NCH; ++ch) {
+      unsigned int d = 0u;
+#pragma unroll
+      for (int i = 0; i < WS; i += 2) {
+        v[ch][i] = have[ch] ? __uint_as_float(u[ch][i / 2].x) : 0.f;
+        if (i + 1 < W) v[ch][i + 1 < W ? i + 1 : i] = have[ch] ? __uint_as_float(u[ch][i / 2].z) : 0.f;
+        d |= (u[ch][i / 2].y ^ tag) | (u[ch][i / 2].w ^ tag);
+      }
+      differ |= have[ch] ? d : 0u;
+    }
+    ok = differ == 0u;
+  };
+  load();
+  poll_until_written(g, [&] { __builtin_amdgcn_s_sleep(1); load(); }, [&] { return __all(ok) != 0; });
+}
+
+// Totals of the W values of `row` over all gx column workgroups, in every lane of the row's
+// segment.  have_row: the thread works on an element of the tile (the others get zeros).
+template <int HS, int W>
+__device__ __forceinline__ void gather_row_sums(const GroupSync& g, unsigned long long* buffer, int nb,
+                                                int gx, unsigned int tag, int row, bool have_row,
+                                                float (&sum)[W]) {
+#pragma unroll
+  for (int i = 0; i < W; ++i) sum[i] = 0.f;
+  if (__builtin_amdgcn_ballot_w64(have_row) == 0ull) return;
+  const TileBuffer slots = make_tile_buffer(reinterpret_cast<float*>(buffer),
+                                            (int)tagged_row_words(gx, nb, W) * 2);
+  const int c = (int)threadIdx.x % HS;
+  auto add = [&](auto nch, int cw0) {
+    constexpr int NCH = decltype(nch)::value;
+    float v[NCH][W];
+    load_row_chunks_polled<W, NCH>(g, slots, nb, cw0, HS, gx, row, have_row, tag, v);
+#pragma unroll
+    for (int ch = 0; ch < NCH; ++ch)
+#pragma unroll
+      for (int i = 0; i < W; ++i) sum[i] += v[ch][i];
+  };
+  if (gx <= HS) add(std::integral_constant<int, 1>{}, c);
+  else if (gx <= 2 * HS) add(std::integral_constant<int, 2>{}, c);
+  else add(std::integral_constant<int, 4>{}, c);
+#pragma unroll
+  for (int i = 0; i < W; ++i) sum[i] = segment_sum<HS>(sum[i]);
+}
+
+// Mean and 1/sqrt(var + eps) of `row` (D columns) from the (mean, m2) that the column
+// workgroups published for their `full_count` columns (`last_count` for the last one): the
+// weighted mean of the means first, then the sum of m2_i + n_i (mean_i - mean)^2.
+template <int HS>
+__device__ __forceinline__ void gather_row_moments(const GroupSync& g, unsigned long long* buffer,
+                                                   int nb, int gx, unsigned int tag, float full_count,
+                                                   float last_count, float D, int row, bool have_row,
+                                                   float& mean_out, float& invstd_out) {
+  mean_out = 0.f;
+  invstd_out = 0.f;
+  if (__builtin_amdgcn_ballot_w64(have_row) == 0ull) return;
+  const TileBuffer slots = make_tile_buffer(reinterpret_cast<float*>(buffer),
+                                            (int)tagged_row_words(gx, nb, 2) * 2);
+  const int c = (int)threadIdx.x % HS;
+  const float inv_D = 1.0f / D;
+  auto count = [&](int cw) { return cw < gx ? (cw == gx - 1 ? last_count : full_count) : 0.f; };
+  auto finish = [&](float m2) {
+    // the hardware's reciprocal square root (1 ulp), as the reference's rsqrt
+    // (lib/layer_norm_forward_gpu.cu.cc:77)
+    invstd_out = __builtin_amdgcn_rsqf(m2 * inv_D + kLnEps);
+  };
+  auto both = [&](auto nch) {
+    constexpr int NCH = decltype(nch)::value;
+    float v[NCH][2];
+    load_row_chunks_polled<2, NCH>(g, slots, nb, c, HS, gx, row, have_row, tag, v);
+    float s1 = 0.f;
+#pragma unroll
+    for (int ch = 0; ch < NCH; ++ch) s1 += count(c + ch * HS) * v[ch][0];
+    mean_out = segment_sum<HS>(s1) * inv_D;
+    float s2 = 0.f;
+#pragma unroll
+    for (int ch = 0; ch < NCH; ++ch) {
+      const float d = v[ch][0] - mean_out;
+      s2 += v[ch][1] + count(c + ch * HS) * d * d;   // a skipped chunk: 0 + 0 * d * d
+    }
+    finish(segment_sum<HS>(s2));
+  };
+  if (gx <= HS) both(std::integral_constant<int, 1>{});
+  else if (gx <= 2 * HS) both(std::integral_constant<int, 2>{});
+  else both(std::integral_constant<int, 4>{});
 }
 
 // Row sums of W values per slot from a tagged buffer: out[row * RowSlot<W>::kWords + i] in LDS.
