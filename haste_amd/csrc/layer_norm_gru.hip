@@ -56,6 +56,7 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
   const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
   const int own_units = (H - j0) < HS ? (H - j0) : HS;
+  const float inv_own_columns = 1.0f / (3.0f * (float)own_units);
   const int last_units = H - (gx - 1) * HS;
   const size_t row_words = tagged_row_words(gx, NB, 2);
   unsigned long long* part2 = p.part2 + (size_t)role.bt * 2 * row_words;
@@ -159,10 +160,13 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
       float s = 0.f;
 #pragma unroll
       for (int g = 0; g < 3; ++g) {
-        rh[pp][g] = colok[pp] ? sum_product<NB, CT>(red, pl[pp], g * HS + pc[pp]) : 0.f;
+        // every thread reads (the address is valid for all of them): a read per branch would
+        // wait out the LDS latency once per gate
+        const float sum = sum_product<NB, CT>(red, pl[pp], g * HS + pc[pp]);
+        rh[pp][g] = colok[pp] ? sum : 0.f;
         s += rh[pp][g];
       }
-      const float mean = segment_sum<HS>(s) / (3.0f * (float)own_units);
+      const float mean = segment_sum<HS>(s) * inv_own_columns;
       float q = 0.f;
 #pragma unroll
       for (int g = 0; g < 3; ++g) {

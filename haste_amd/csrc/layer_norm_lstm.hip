@@ -66,6 +66,7 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
   const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
   const int own_units = (H - j0) < HS ? (H - j0) : HS;     // valid hidden units here
+  const float inv_own_units = 1.0f / (float)own_units, inv_own_columns = 1.0f / (4.0f * (float)own_units);
   const int last_units = H - (gx - 1) * HS;                 // ... in the last workgroup
   const size_t row_words = tagged_row_words(gx, NB, 2);
   unsigned long long* part2 = p.part2 + (size_t)role.bt * 2 * row_words;
@@ -183,11 +184,13 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
       float s = 0.f;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        rh[pp][g] = colok[pp] ? sum_product<NB, CT>(red, pl[pp], g * HS + pc[pp]) : 0.f;
+        // every thread reads (the address is valid for all of them): a read per branch would
+        // wait out the LDS latency once per gate
+        const float sum = sum_product<NB, CT>(red, pl[pp], g * HS + pc[pp]);
+        rh[pp][g] = colok[pp] ? sum : 0.f;
         s += rh[pp][g];
       }
-      const float cnt = 4.0f * (float)own_units;
-      const float mean = segment_sum<HS>(s) / cnt;
+      const float mean = segment_sum<HS>(s) * inv_own_columns;
       float q = 0.f;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
@@ -234,7 +237,7 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
       }
       // moments of the new cell state over the owned hidden units
       const float cv = colok[pp] ? c_new[pp] : 0.f;
-      const float mean = segment_sum<HS>(cv) / (float)own_units;
+      const float mean = segment_sum<HS>(cv) * inv_own_units;
       const float d = cv - mean;
       const float q = segment_sum<HS>(colok[pp] ? d * d : 0.f);
       if (pc[pp] == 0 && tid + 256 * pp < NB * HS) {
