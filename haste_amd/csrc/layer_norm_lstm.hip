@@ -40,10 +40,14 @@ struct LnLstmFwdParams {
   LaunchShape ls;
 };
 
-// NB batch rows per workgroup.
-template <int NB, int CT>
+// NB batch rows per workgroup.  PARK (the tile's elements leave the last wavefront idle): that
+// wavefront requests the next step's inputs and parks them in LDS for the owners of the elements,
+// see ln_lstm_backward_kernel.
+constexpr int kLnLstmFwdInputs = 5;  // floats per element and step: LN(x*W) of the four gates, the mask
+template <int NB, int CT, bool PARK = false>
 __global__ __launch_bounds__(256, 1)
 void ln_lstm_forward_kernel(LnLstmFwdParams p) {
+  static_assert(!PARK || NB * 4 * CT <= 192, "parked inputs: the last wavefront owns no element");
   constexpr int HS = 4 * CT;
   constexpr int NCOLS = 16 * CT;
   constexpr int PP = (NB * HS + 255) / 256;
@@ -57,6 +61,7 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
   float* w_lds = lds;
   float* red = lds + Kpad * NCOLS;
   float* stat = red + ProductTile<NB, CT>::kRedFloats;  // [2][NB][2] row statistics (long rows only)
+  float* park = stat + 4 * NB;  // PARK: [2][5][NB * HS] inputs of a step, by step parity
 
   const int tid = threadIdx.x;
   const int gx = p.ls.gx;
@@ -149,6 +154,7 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
     for (int g = 0; g < 4; ++g) wx_next[pp][g] = 0.f;
   }
   auto fetch = [&](int t) {
+    if constexpr (PARK) return;
     const int tt = t < T ? t : T - 1;
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
@@ -160,14 +166,50 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
     }
   };
   fetch(0);
+  // PARK: lane l of the helper wavefront requests the inputs of the elements l, l + 64, ... of
+  // the tile for step t and parks them in the buffer of t's parity.
+  constexpr int kElements = NB * HS;
+  const bool helper = PARK && (tid >> 6) == 3;
+  auto park_inputs = [&](int t) {
+    float* dst = park + (size_t)(t & 1) * kLnLstmFwdInputs * kElements;
+#pragma unroll
+    for (int q = 0; q < (kElements + 63) / 64; ++q) {
+      const int idx = (tid & 63) + 64 * q;
+      const int r_ = idx / HS, u_ = idx % HS;
+      const bool exists = idx < kElements && r_ < rows_here && j0 + u_ < H;
+      const size_t row = exists ? (size_t)(n0 + r_) : 0, unit = exists ? (size_t)(j0 + u_) : 0;
+      const float* vt = p.v + ((size_t)t * N + row) * 4 * H + unit;
+      float in[kLnLstmFwdInputs];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) in[g] = vt[g * H];
+      in[4] = zoneout && p.training ? p.zoneout_mask[(size_t)t * NH + row * H + unit] : 1.f;
+      if (idx < kElements) {
+#pragma unroll
+        for (int i = 0; i < kLnLstmFwdInputs; ++i) dst[i * kElements + idx] = in[i];
+      }
+    }
+  };
+  if constexpr (PARK) {
+    if (helper) park_inputs(0);
+    __syncthreads();
+  }
 
   for (int t = 0; t < T; ++t) {
     float wx[PP][4], mk[PP];
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
-      mk[pp] = mk_next[pp];
+      if constexpr (PARK) {
+        // parked during the previous step, before its closing barrier
+        const float* src = park + (size_t)(t & 1) * kLnLstmFwdInputs * kElements;
+        const int idx = tid + 256 * pp < kElements ? tid + 256 * pp : 0;
 #pragma unroll
-      for (int g = 0; g < 4; ++g) wx[pp][g] = wx_next[pp][g];
+        for (int g = 0; g < 4; ++g) wx[pp][g] = src[g * kElements + idx];
+        mk[pp] = src[4 * kElements + idx];
+      } else {
+        mk[pp] = mk_next[pp];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) wx[pp][g] = wx_next[pp][g];
+      }
     }
     const unsigned int tag = gs.epoch + 2u + (unsigned int)t;  // names this step's row exchanges
     unsigned long long* ex2 = part2 + (size_t)(t & 1) * row_words;
@@ -176,6 +218,11 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
     // The operand loads wait for h[t] themselves (polled tile t % 4).
     tile_product<NB, CT, false, true>(xhb, (t & 3) * tile_floats, Kpad, w_lds, red, &gs);
     __syncthreads();
+    // After its share of the product the helper has nothing to do until the step's closing
+    // barrier: time enough for loads from memory nobody has touched.
+    if constexpr (PARK) {
+      if (helper && t + 1 < T) park_inputs(t + 1);
+    }
 
     // h*R of the owned columns; moments of those columns per row, published.
     float rh[PP][4];
@@ -810,9 +857,22 @@ int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_siz
   p.part2 = reinterpret_cast<unsigned long long*>(ws.scratch);
   p.part3 = reinterpret_cast<unsigned long long*>(ws.scratch + part_floats);
   p.xh = ws.scratch + 2 * part_floats;
+  // Tiles whose elements leave the last wavefront idle park the inputs of a step in LDS when
+  // there is room: [2][5][NB * HS] floats.
+  const size_t park_bytes = (size_t)2 * kLnLstmFwdInputs * NB * tile.hs * sizeof(float);
+  const bool parked = NB * tile.hs <= 192 && NB <= 16 && tile.lds_bytes + park_bytes <= kMaxLdsBytes;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes, 3u * (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes + (parked ? park_bytes : 0),
+                                  3u * (unsigned)T + 1, &plan));
   p.ls = plan.shape;
+#define HASTE_LAUNCH_PARKED(NB_, CT_)                                                        \
+  if (parked && tile.nb == NB_ && tile.ct == CT_)                                            \
+    return launch_persistent("layer_norm_lstm_forward_recurrence",                           \
+                             ln_lstm_forward_kernel<NB_, CT_, true>, plan, p, stream);
+  HASTE_LAUNCH_PARKED(4, 1) HASTE_LAUNCH_PARKED(4, 2) HASTE_LAUNCH_PARKED(4, 4)
+  HASTE_LAUNCH_PARKED(8, 1) HASTE_LAUNCH_PARKED(8, 2) HASTE_LAUNCH_PARKED(8, 4)
+  HASTE_LAUNCH_PARKED(16, 1) HASTE_LAUNCH_PARKED(16, 2)
+#undef HASTE_LAUNCH_PARKED
 #define HASTE_LAUNCH(NB_, CT_)                                                               \
   if (tile.nb == NB_ && tile.ct == CT_)                                                      \
     return launch_persistent("layer_norm_lstm_forward_recurrence",                           \
