@@ -1222,6 +1222,10 @@ __device__ __forceinline__ void reset_partials(float* red, int live) {
 // broadcast 16-byte reads.
 constexpr int kSingleRowUnits = 16;
 constexpr int kSingleRowCols = 64;
+// The LSTM kernel adds a fifth wavefront that parks the next steps' inputs in LDS:
+// [2][5][16] floats behind the role word.
+constexpr int kSingleRowThreads = 320;
+constexpr size_t kSingleRowParkBytes = (size_t)(2 * 5 * kSingleRowUnits + 3) * sizeof(float);
 
 // Dynamic LDS of a single-row kernel: [4][KW_MAX] a wavefront's share of h, [2][4][64]
 // partial sums by step parity and wavefront, one word for the role (no static LDS:
