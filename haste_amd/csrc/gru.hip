@@ -242,12 +242,15 @@ void gru_forward_kernel(GruFwdParams p) {
 // x 3 gates per workgroup (the fourth 16 columns of the 64 are idle), the recurrent weights in
 // registers.
 template <int KW_MAX>
-__global__ __launch_bounds__(256, 1)
+__global__ __launch_bounds__(kSingleRowThreads, 1)
 void gru_forward_single_row_kernel(GruFwdParams p) {
   constexpr int HS = kSingleRowUnits, NCOLS = kSingleRowCols;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   float (*h_lds)[KW_MAX] = reinterpret_cast<float (*)[KW_MAX]>(lds);
   float (*red)[4][NCOLS] = reinterpret_cast<float (*)[4][NCOLS]>(lds + 4 * KW_MAX);
+  // inputs of a step (x*W of the three gates, the mask), parked by the fifth wavefront as in
+  // lstm_forward_single_row_kernel
+  float (*park)[5][HS] = reinterpret_cast<float (*)[5][HS]>(lds + 4 * KW_MAX + 2 * 4 * NCOLS + 4);
   const int H = p.H, T = p.T;
   const int Kpad = round_up(H, 64);
   const int KW = Kpad / 4;  // multiple of 16
@@ -267,7 +270,7 @@ void gru_forward_single_row_kernel(GruFwdParams p) {
   float w[KW_MAX];
   single_row_weights<KW_MAX>(w, p.R, p.dc_mask, p.dc_scale, KW, H, 3 * H, (lane / HS) * H + j0 + lane % HS,
                              lane / HS < 3 && j0 + lane % HS < H);
-  for (int i = tid; i < 4 * KW_MAX; i += 256) (&h_lds[0][0])[i] = 0.f;  // ordered by group_arrive's barrier
+  for (int i = tid; i < 4 * KW_MAX; i += kSingleRowThreads) (&h_lds[0][0])[i] = 0.f;  // ordered by group_arrive's barrier
 
   // Pointwise ownership: thread u < 16 handles hidden unit j0 + u.
   const int pj = j0 + tid;
@@ -288,33 +291,50 @@ void gru_forward_single_row_kernel(GruFwdParams p) {
     store_exchanged(gs, &xh[pj], publishable(h_prev));
     for (int b = 1; b < kPolledTiles; ++b) store_exchanged(gs, &xh[b * Kpad + pj], unwritten_value());
   }
+  // The helper's requests: lane l = 16 g + u asks for x*W of gate g < 3, unit j0 + u; the first
+  // sixteen lanes also for the mask.  Every lane loads (some valid address where its element
+  // does not exist, and the last step again after the end).
+  const bool helper = wave == 4;
+  float in_v = 0.f, in_m = 1.f;
+  auto request = [&](int t) {
+    const int tt = t < T ? t : T - 1;
+    const int unit = j0 + lane % HS < H ? j0 + lane % HS : 0;
+    const int gate = lane / HS < 3 ? lane / HS : 0;
+    in_v = p.Wx[(size_t)tt * 3 * H + (size_t)gate * H + unit];
+    if (zoneout && p.training) in_m = p.zoneout_mask[(size_t)tt * H + unit];
+  };
+  auto park_inputs = [&](int t) {
+    park[t & 1][lane / HS][lane % HS] = in_v;
+    if (lane < HS) park[t & 1][4][lane] = in_m;
+  };
+  if (helper) {
+    request(0);
+    park_inputs(0);
+    request(1);
+    park_inputs(1);
+  }
   group_arrive(gs);
   group_wait(gs);
 
-  // Every thread loads (a thread without an element, and the request after the last step, some
-  // valid address) and nothing but the loads writes these registers inside the loop (see
-  // lstm_forward_kernel).
-  float wx_next[3] = {0.f, 0.f, 0.f}, mk_next = 1.f;
-  auto fetch = [&](int t) {
-    const int tt = t < T ? t : T - 1;
-    const int unit = act ? pj : 0;
-    const float* wt = p.Wx + (size_t)tt * 3 * H + unit;
-#pragma unroll
-    for (int g = 0; g < 3; ++g) wx_next[g] = wt[g * H];
-    if (zoneout && p.training) mk_next = p.zoneout_mask[(size_t)tt * H + unit];
-  };
-  fetch(0);
-
   for (int t = 0; t < T; ++t) {
-    float wx[3];
-    const float mk = mk_next;
+    // parked two steps ago (the first two: before the barrier above)
+    float wx[3] = {0.f, 0.f, 0.f}, mk = 1.f;
+    if (act) {
 #pragma unroll
-    for (int g = 0; g < 3; ++g) wx[g] = wx_next[g];
+      for (int g = 0; g < 3; ++g) wx[g] = park[t & 1][g][tid];
+      mk = park[t & 1][4][tid];
+    }
 
     // The wavefront's share of h[t] (polled tile t % 4) against the thread's weights.
-    red[t & 1][wave][lane] =
-        single_row_product<KW_MAX>(gs, xhb, (t & 3) * Kpad + wave * KW, KW, h_lds[wave], w);
+    if (helper) {
+      request(t + 2);
+    } else {
+      red[t & 1][wave][lane] =
+          single_row_product<KW_MAX>(gs, xhb, (t & 3) * Kpad + wave * KW, KW, h_lds[wave], w);
+    }
     __syncthreads();
+    // The owners have read this parity's inputs before the barrier.
+    if (helper) park_inputs(t + 2);
 
     float saved[4] = {0.f, 0.f, 0.f, 0.f};  // z, r, g, q of the step for the caller's cache
     if (act) {
@@ -347,7 +367,6 @@ void gru_forward_single_row_kernel(GruFwdParams p) {
       // the tile read at step t-1: nobody needs it any more
       if (t + 3 < T) store_exchanged(gs, &xh[((t + 3) & 3) * Kpad + pj], unwritten_value());
     }
-    fetch(t + 1);
     // The caller's copies are written last: nobody in the launch waits for them.
     if (act) {
       if (p.training) {
@@ -646,7 +665,9 @@ int gru_forward_single_row(hipStream_t stream, int training, int T, int C, int H
   p.xh = ws.scratch;
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, (H + 15) / 16, 1, 1,
-                                  single_row_lds_bytes(single_row_kw_max(Kpad)), (unsigned)T + 1, &plan));
+                                  single_row_lds_bytes(single_row_kw_max(Kpad)) + kSingleRowParkBytes,
+                                  (unsigned)T + 1, &plan));
+  plan.threads = kSingleRowThreads;
   p.ls = plan.shape;
   const char* name = "gru_forward_recurrence";
   if (Kpad <= 128) return launch_persistent(name, gru_forward_single_row_kernel<32>, plan, p, stream);

@@ -1222,7 +1222,7 @@ __device__ __forceinline__ void reset_partials(float* red, int live) {
 // broadcast 16-byte reads.
 constexpr int kSingleRowUnits = 16;
 constexpr int kSingleRowCols = 64;
-// The LSTM kernel adds a fifth wavefront that parks the next steps' inputs in LDS:
+// The forward kernels add a fifth wavefront that parks the next steps' inputs in LDS:
 // [2][5][16] floats behind the role word.
 constexpr int kSingleRowThreads = 320;
 constexpr size_t kSingleRowParkBytes = (size_t)(2 * 5 * kSingleRowUnits + 3) * sizeof(float);
