@@ -286,9 +286,13 @@ inline int ln_gru_backward_k(int H) { return 48 * ((H + 15) / 16); }
 
 // REG > 0: the slice exceeds LDS; every wavefront keeps the first REG k-groups of its share
 // of the contraction in registers (tall_tile_product).
-template <int NB, int REG = 0>
+// PARK (tiles of 4 rows): the idle last wavefront requests the inputs of the following step
+// and parks them in LDS for the owners of the elements, see ln_lstm_backward_kernel.
+constexpr int kLnGruBwdInputs = 12;  // floats per element and step, see StepIn
+template <int NB, int REG = 0, bool PARK = false>
 __global__ __launch_bounds__(256, 1)
 void ln_gru_backward_kernel(LnGruBwdParams p) {
+  static_assert(!PARK || (NB == 4 && REG == 0), "parked inputs: 4-row tiles");
   constexpr int HSB = 16;
   constexpr int NCOLS = 16;
   constexpr int PP = (NB * HSB + 255) / 256;
@@ -306,6 +310,7 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
   float* w_lds = lds;
   float* red = lds + (Kpad - 64 * REG) * NCOLS;  // the partial tiles, reused for the column sums
   float* sums = red + RED;           // [NB][4] row sums of the norm (long rows only)
+  float* park = sums + 4 * NB;       // PARK: [2][12][NB * 16] inputs of a step, by step parity
 
   const int tid = threadIdx.x;
   const int gx = p.ls.gx;
@@ -389,7 +394,55 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) nxt[pp] = nxt_init;
   }
+  // PARK: the helper wavefront's side.  Lane l requests the inputs of the elements l, l + 64, ...
+  // of the tile for step t and parks them in the buffer of t's parity.
+  constexpr int kElements = NB * HSB;
+  const bool helper = PARK && (tid >> 6) == 3;
+  auto park_inputs = [&](int t) {
+    float* dst = park + (size_t)(t & 1) * kLnGruBwdInputs * kElements;
+#pragma unroll
+    for (int q = 0; q < (kElements + 63) / 64; ++q) {
+      const int idx = (tid & 63) + 64 * q;
+      const int r_ = idx / HSB, u_ = idx % HSB;
+      const bool exists = idx < kElements && r_ < rows_here && j0 + u_ < H;
+      const size_t row = exists ? (size_t)(n0 + r_) : 0, unit = exists ? (size_t)(j0 + u_) : 0;
+      const size_t e = row * H + unit;
+      const float* vt = p.v + ((size_t)t * N + row) * 4 * H + unit;
+      const float* ar = p.act_Rh + ((size_t)t * N + row) * 3 * H + unit;
+      float in[kLnGruBwdInputs];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) in[g] = vt[(size_t)g * H];
+#pragma unroll
+      for (int g = 0; g < 3; ++g) in[4 + g] = ar[(size_t)g * H];
+      in[7] = p.h[(size_t)t * NH + e];
+      in[8] = p.dh_new[(size_t)(t + 1) * NH + e];
+      in[9] = zoneout ? p.zoneout_mask[(size_t)t * NH + e] : 1.f;
+      in[10] = p.cache2[((size_t)t * N + row) * 2];
+      in[11] = p.cache2[((size_t)t * N + row) * 2 + 1];
+      if (idx < kElements) {
+#pragma unroll
+        for (int i = 0; i < kLnGruBwdInputs; ++i) dst[i * kElements + idx] = in[i];
+      }
+    }
+  };
+  // ... and the owners' side: the inputs of step t from the buffer of its parity.
+  auto take_parked = [&](int t, StepIn (&s)[PP]) {
+    const float* src = park + (size_t)(t & 1) * kLnGruBwdInputs * kElements;
+#pragma unroll
+    for (int pp = 0; pp < PP; ++pp) {
+      const int idx = own[pp] ? tid + 256 * pp : 0;
+      float in[kLnGruBwdInputs];
+#pragma unroll
+      for (int i = 0; i < kLnGruBwdInputs; ++i) in[i] = src[i * kElements + idx];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) s[pp].vt[g] = in[g];
+#pragma unroll
+      for (int g = 0; g < 3; ++g) s[pp].rh[g] = in[4 + g];
+      s[pp].h0 = in[7]; s[pp].dhn = in[8]; s[pp].m = in[9]; s[pp].mu2 = in[10]; s[pp].is2 = in[11];
+    }
+  };
   auto fetch = [&](int t) {
+    if constexpr (PARK) return;
     const int tt = t >= 0 ? t : 0;
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
@@ -409,17 +462,27 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
     }
   };
   fetch(T - 1);
+  if constexpr (PARK) {
+    if (helper) park_inputs(T - 1);
+    __syncthreads();
+  }
 
   const float inv3H = 1.0f / (float)(3 * H);
   for (int t = T - 1; t >= 0; --t) {
     StepIn s[PP];
+    if constexpr (PARK) {
+      // Parked during the previous step, before its product's barrier; the buffer this step's
+      // helper fills was last read a step ago.
+      take_parked(t, s);
+      if (helper && t > 0) park_inputs(t - 1);
+    }
     float dh_keep[PP], xc[PP][3], gd[PP][3], dps[PP][3], dqs[PP][3];
     const int done = T - 1 - t;  // steps done so far
     const unsigned int tag = gs.epoch + 2u + (unsigned int)done;  // names this step's row exchange
     unsigned long long* ex = part + (size_t)(done & 1) * row_words;
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
-      s[pp] = nxt[pp];
+      if constexpr (!PARK) s[pp] = nxt[pp];
       dh_keep[pp] = 0.f;
 #pragma unroll
       for (int k = 0; k < 3; ++k) dps[pp][k] = dqs[pp][k] = 0.f;
@@ -669,8 +732,13 @@ int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_s
   p.part = reinterpret_cast<unsigned long long*>(ws.scratch);
   p.col_partial = ws.scratch + part_floats;
   p.xdq = ws.scratch + part_floats + col_floats;
+  // 4-row tiles park the inputs of a step in LDS when there is room: [2][12][NB * 16] floats
+  // (8-row tiles measured 2.6 % slower with it at N = 64, H = 512).
+  const size_t park_bytes = (size_t)2 * kLnGruBwdInputs * NB * 16 * sizeof(float);
+  const bool parked = NB <= 4 && tile.reg_groups == 0 && tile.lds_bytes + park_bytes <= kMaxLdsBytes;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes, 2u * (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes + (parked ? park_bytes : 0),
+                                  2u * (unsigned)T + 1, &plan));
   p.ls = plan.shape;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const char* name = "layer_norm_gru_backward_recurrence";
@@ -685,6 +753,7 @@ int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_s
     else if (NB == 64) rc = HASTE_LAUNCH_BWD_RESIDENT(64);
   }
 #undef HASTE_LAUNCH_BWD_RESIDENT
+  else if (NB == 4 && parked) rc = launch_persistent(name, ln_gru_backward_kernel<4, 0, true>, plan, p, stream);
   else if (NB == 4) rc = launch_persistent(name, ln_gru_backward_kernel<4>, plan, p, stream);
   else if (NB == 8) rc = launch_persistent(name, ln_gru_backward_kernel<8>, plan, p, stream);
   else if (NB == 16) rc = launch_persistent(name, ln_gru_backward_kernel<16>, plan, p, stream);
