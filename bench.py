@@ -104,9 +104,7 @@ def run_metric(args, torch, lib, ops, dev):
 
     def step():
         hlib.call("haste_hip_lstm_forward_f32", True, T, N, C, H, Wd, Rd, bd, xd, h, c, v, None, 0.0, None)
-        hlib.call("haste_hip_transpose_f32", T * N, C, xd, x_t)
-        hlib.call("haste_hip_transpose_f32", C, 4 * H, Wd, W_t)
-        hlib.call("haste_hip_transpose_f32", H, 4 * H, Rd, R_t)
+        hlib.call("haste_hip_transpose3_f32", T * N, C, xd, x_t, C, 4 * H, Wd, W_t, H, 4 * H, Rd, R_t)
         hlib.call("haste_hip_lstm_backward_f32", T, N, C, H, W_t, R_t, bd, x_t, h, c, dh_new, dc_new,
                   dx, dW, dR, db, dh, dc, v, None)
 
@@ -114,7 +112,7 @@ def run_metric(args, torch, lib, ops, dev):
     # h0 / c0 copied into slot 0, the accumulated gradients zero-filled (reported beside it).
     def ops_step():
         hh, cc, cache = ops.lstm_forward(True, 0.0, xd, h0, c0, Wd, Rd, bd, no_mask)
-        return ops.lstm_backward(ops.transpose(xd), ops.transpose(Wd), ops.transpose(Rd), bd, no_mask,
+        return ops.lstm_backward(*ops.transpose3(xd, Wd, Rd), bd, no_mask,
                                  hh, cc, cache, dh_new, dc_new)
 
     for _ in range(args.warmup):
@@ -483,7 +481,7 @@ def run_configs(args, torch, lib, ops, dev):
 
     def lstm_step():
         h, c, cache = ops.lstm_forward(True, 0.0, x, z, z, W, R, b, no_mask)
-        return ops.lstm_backward(ops.transpose(x), ops.transpose(W), ops.transpose(R), b, no_mask, h, c,
+        return ops.lstm_backward(*ops.transpose3(x, W, R), b, no_mask, h, c,
                                  cache, dh_new, dc_new)
     out["lstm_fwd_bwd_N128_T100_H512_ms"] = timed(lstm_step, 30)
 
@@ -499,7 +497,7 @@ def run_configs(args, torch, lib, ops, dev):
 
     def ln_lstm_step():
         fwd = ops.layer_norm_lstm_forward(True, 0.1, x, z, z, W, R, b, gamma, gamma_h, beta_h, zm)
-        return ops.layer_norm_lstm_backward(ops.transpose(x), ops.transpose(W), ops.transpose(R), b, gamma,
+        return ops.layer_norm_lstm_backward(*ops.transpose3(x, W, R), b, gamma,
                                             gamma_h, beta_h, zm, *fwd, dh_new, dc_new)
     out["layer_norm_lstm_fwd_bwd_N32_T500_H256_zoneout_ms"] = timed(ln_lstm_step, 10)
     return out

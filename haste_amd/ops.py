@@ -142,6 +142,24 @@ def transpose(a, out=None):
     return out
 
 
+def transpose3(a, b, c):
+    """transpose() of three float32 tensors in one launch: the x_t, W_t, R_t a backward pass asks
+    its caller for (reference frameworks/pytorch/lstm.py:84-86)."""
+    outs = []
+    args = []
+    for m in (a, b, c):
+        _check(m)
+        if m.dtype != torch.float32:
+            return transpose(a), transpose(b), transpose(c)
+        cols = m.shape[-1]
+        rows = m.numel() // cols
+        out = torch.empty((cols,) + tuple(m.shape[:-1]), device=m.device, dtype=m.dtype)
+        outs.append(out)
+        args += [rows, cols, m, out]
+    lib.call("haste_hip_transpose3_f32", *args)
+    return tuple(outs)
+
+
 # ---- LSTM (reference frameworks/pytorch/lstm.cc:31-157) ---------------------
 def lstm_forward(training, zoneout_prob, x, h0, c0, kernel, recurrent_kernel, bias, zoneout_mask,
                  dropconnect_mask=None, dropconnect_scale=1.0):

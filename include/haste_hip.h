@@ -115,6 +115,14 @@ int haste_hip_gemm_f32(int trans_a, int M, int N, int K,
  * region (benchmarks/benchmark_lstm.cc:417-445).  This is that helper. */
 int haste_hip_transpose_f32(int rows, int cols, const float* in, float* out, void* stream);
 
+/* The same for three matrices in one launch: a backward pass needs x_t, W_t and R_t together
+ * (lib/haste/lstm.h:230-247), and W and R are small enough that a launch each costs more than
+ * the copy (the reference's benchmark issues one cublasSgeam per matrix,
+ * benchmarks/benchmark_lstm.cc:417-445). */
+int haste_hip_transpose3_f32(int rows0, int cols0, const float* in0, float* out0,
+                             int rows1, int cols1, const float* in1, float* out1,
+                             int rows2, int cols2, const float* in2, float* out2, void* stream);
+
 /* ---- LSTM ----------------------------------------------------------------
  * reference lib/haste/lstm.h:118-129 (ForwardPass::Run), lib/lstm_forward_gpu.cu.cc:313-366.
  * W[C,4H] R[H,4H] b[4H] x[T,N,C] h,c[T+1,N,H] (slot 0 preset by the caller)

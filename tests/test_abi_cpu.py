@@ -58,6 +58,7 @@ def test_null_pointers_and_bad_dimensions_are_rejected_on_the_host(lib):
     assert _call(lib, "haste_hip_lstm_backward_f32", 3, 2, 2, 2, *([None] * 16), None) == INVALID
     assert _call(lib, "haste_hip_gru_forward_f32", 1, 3, 2, 2, 2, *([None] * 9), 0.0, None, None) == INVALID
     assert _call(lib, "haste_hip_gru_backward_f32", 3, 2, 2, 2, *([None] * 17), None) == INVALID
+    assert _call(lib, "haste_hip_transpose3_f32", *([4, 4, None, None] * 3), None) == INVALID
     assert _call(lib, "haste_hip_layer_norm_forward_f32", 4, 8, *([None] * 5), None) == INVALID
     assert _call(lib, "haste_hip_layer_norm_backward_f32", 4, 8, *([None] * 7), None) == INVALID
     assert _call(lib, "haste_hip_indrnn_forward_f32", 1, 3, 2, 2, 2, *([None] * 6), 0.0, None, None) == INVALID

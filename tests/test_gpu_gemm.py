@@ -88,6 +88,17 @@ def test_transpose(shape):
     assert out.shape == ref.shape and torch.equal(out, ref)
 
 
+@pytest.mark.parametrize("shapes", [((1, 1), (3, 5), (65, 63)), ((100, 7, 33), (64, 64), (2, 130)),
+                                    ((6400, 512), (512, 2048), (512, 2048))])
+def test_three_transposes_in_one_launch(shapes):
+    import torch
+    from haste_amd import ops
+    ms = [torch.randn(*s, device="cuda") for s in shapes]
+    outs = ops.transpose3(*ms)
+    for m, out in zip(ms, outs):
+        assert torch.equal(out, ops.transpose(m))
+
+
 @pytest.mark.parametrize("trans_a", [True, False])
 def test_gemm_operand_of_more_than_2_gib(trans_a):
     """B[K, N] of 2.1 GB (the dv of a backward pass with T*N*H = 2^27 and beyond: dW = x^T dv
