@@ -100,3 +100,41 @@ def test_layer_norm_lstm_inference_forward():
                                     p["x"], p["h0"], p["c0"], False, 0.25, p["mask"])
     assert relerr(host(outs[0]), fwd["h"]) < TOL
     assert relerr(host(outs[1]), fwd["c"]) < TOL
+
+
+@pytest.mark.parametrize("T,N,C,H", [(6, 5, 12, 40), (5, 32, 16, 256), (4, 9, 8, 1100)])
+def test_layer_norm_lstm_backward_with_badly_scaled_sums(T, N, C, H):
+    """The backward step sends the row sums of the h*R norm as coefficients of the cell-state
+    norm's dsigma and dmu (one exchange for both norms).  Inputs that make those terms large
+    against their total -- norm scales of both signs and sizes, a cell state with a large
+    common offset, upstream cell gradients with one -- must still give the oracle's gradients."""
+    from haste_amd import ops
+    import torch
+    print("ln_lstm scaled", T, N, C, H, flush=True)
+    p = problem(900 + T + N + C + H, T, N, C, H, 4, 0.2)
+    r = np.random.default_rng(7 + H)
+    f32 = lambda a: a.astype(np.float32).astype(np.float64)
+    p["gamma"] = f32(r.uniform(-3.0, 3.0, p["gamma"].shape))
+    p["gamma_h"] = f32(r.uniform(-2.0, 2.0, p["gamma_h"].shape))
+    p["c0"] = f32(p["c0"] * 4.0 + 10.0)
+    p["dc_new"] = f32(p["dc_new"] + 5.0)
+    p["R"] = f32(p["R"] * 4.0)
+    mask = dev(p["mask"])
+    gam, gh, bh = dev(p["gamma"]), dev(p["gamma_h"]), dev(p["beta_h"])
+    outs = ops.layer_norm_lstm_forward(True, 0.2, dev(p["x"]), dev(p["h0"]), dev(p["c0"]),
+                                       dev(p["W"]), dev(p["R"]), dev(p["b"]), gam, gh, bh, mask)
+    h, c, act_Wx, act_Wx_norm, cache1, act_Rh, cache2, act_c_norm, cache3 = outs
+    fwd = O.layer_norm_lstm_forward(p["W"], p["R"], p["b"], p["gamma"], p["gamma_h"], p["beta_h"],
+                                    p["x"], p["h0"], p["c0"], True, 0.2, p["mask"])
+    assert relerr(host(h), fwd["h"]) < TOL
+    assert relerr(host(c), fwd["c"]) < TOL
+    grads = ops.layer_norm_lstm_backward(
+        dev(p["x"]).permute(2, 0, 1).contiguous(), dev(p["W"]).t().contiguous(),
+        dev(p["R"]).t().contiguous(), dev(p["b"]), gam, gh, bh, mask, h, c, act_Wx, act_Wx_norm,
+        cache1, act_Rh, cache2, act_c_norm, cache3, dev(p["dh_new"]), dev(p["dc_new"]))
+    torch.cuda.synchronize()
+    g = O.layer_norm_lstm_backward(p["W"], p["R"], p["b"], p["gamma"], p["gamma_h"], p["beta_h"],
+                                   p["x"], fwd, p["dh_new"], p["dc_new"], p["mask"])
+    names = ("dx", "dh0", "dc0", "dW", "dR", "db", "dgamma", "dgamma_h", "dbeta_h")
+    for name, ours in zip(names, grads):
+        assert relerr(host(ours), g[name]) < TOL, name
