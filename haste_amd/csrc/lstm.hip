@@ -538,14 +538,16 @@ void lstm_backward_kernel(LstmBwdParams p) {
   for (int pp = 0; pp < PP; ++pp) nxt[pp] = nxt_init;
   // (Two sets per workgroup: measured 1.5 % slower per step that way, 0.2887 -> 0.2931 ms at
   // N = 64, T = 100, H = 512; there only the threads with an element load.)
-  // One set per workgroup: requested two steps ahead, right after a product (`later`).  These
-  // inputs come from memory that is cold in this launch, and a wavefront's loads return in
-  // order -- requested just before a product they keep its polls waiting.  Placed there, the
-  // next loads the wavefront issues are the polls of the following product, a pointwise phase
-  // and a publication later (N = 128, T = 100, H = 512 with 16-row tiles: 1.683 -> 1.660 ms
-  // forward + backward).  Two sets keep the request before the product: 0.289 -> 0.291 ms the
-  // other way.
-  constexpr bool kRequestAfterProduct = SETS == 1;
+  // Tiles of 32 and 64 rows (one set per workgroup, the whole slice in LDS): requested two steps
+  // ahead, right after a product (`later`).  These inputs come from memory that is cold in this
+  // launch, and a wavefront's loads return in order -- requested just before a product they keep
+  // its polls waiting.  Placed there, the next loads the wavefront issues are the polls of the
+  // following product, a pointwise phase and a publication later.  Backward pass, T = 100:
+  // N = 256, H = 256 0.914 -> 0.856 ms, N = 512, H = 128 0.989 -> 0.921; 16-row tiles do not
+  // change (N = 128, H = 512), 4-row tiles lose 2 %, tiles with slice rows in registers up to
+  // 10 % (N = 32, H = 1024: the second set of inputs costs them registers), two sets per
+  // workgroup 1 %: those keep the request before the product.
+  constexpr bool kRequestAfterProduct = SETS == 1 && REG == 0 && NB >= 32;
   StepIn later[PP];
 #pragma unroll
   for (int pp = 0; pp < PP; ++pp) later[pp] = nxt_init;
