@@ -47,7 +47,7 @@ constexpr int kLnLstmFwdInputs = 5;  // floats per element and step: LN(x*W) of 
 template <int NB, int CT, bool PARK = false>
 __global__ __launch_bounds__(256, 1)
 void ln_lstm_forward_kernel(LnLstmFwdParams p) {
-  static_assert(!PARK || NB * 4 * CT <= 192, "parked inputs: the last wavefront owns no element");
+  static_assert(!PARK || NB * 4 * CT <= 64, "parked inputs: one element per lane of the idle last wavefront");
   constexpr int HS = 4 * CT;
   constexpr int NCOLS = 16 * CT;
   constexpr int PP = (NB * HS + 255) / 256;
@@ -857,10 +857,13 @@ int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_siz
   p.part2 = reinterpret_cast<unsigned long long*>(ws.scratch);
   p.part3 = reinterpret_cast<unsigned long long*>(ws.scratch + part_floats);
   p.xh = ws.scratch + 2 * part_floats;
-  // Tiles whose elements leave the last wavefront idle park the inputs of a step in LDS when
-  // there is room: [2][5][NB * HS] floats.
+  // Tiles of at most 64 elements (one per lane of the idle last wavefront) park the inputs of a
+  // step in LDS when there is room: [2][5][NB * HS] floats.  Measured forward, T = 200-500:
+  // N = 32, H = 256 -3.5 %, N = 8, H = 128 -3.5 %, N = 4, H = 512 -5 %; with two elements per
+  // lane +1.3 % (N = 64, H = 512), and with rows too long for the gathers inside a wavefront
+  // +2.5 % (N = 16, H = 1024), so those keep their own requests.
   const size_t park_bytes = (size_t)2 * kLnLstmFwdInputs * NB * tile.hs * sizeof(float);
-  const bool parked = NB * tile.hs <= 192 && NB <= 16 && tile.lds_bytes + park_bytes <= kMaxLdsBytes;
+  const bool parked = NB * tile.hs <= 64 && gx <= 4 * tile.hs && tile.lds_bytes + park_bytes <= kMaxLdsBytes;
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes + (parked ? park_bytes : 0),
                                   3u * (unsigned)T + 1, &plan));
@@ -870,8 +873,7 @@ int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_siz
     return launch_persistent("layer_norm_lstm_forward_recurrence",                           \
                              ln_lstm_forward_kernel<NB_, CT_, true>, plan, p, stream);
   HASTE_LAUNCH_PARKED(4, 1) HASTE_LAUNCH_PARKED(4, 2) HASTE_LAUNCH_PARKED(4, 4)
-  HASTE_LAUNCH_PARKED(8, 1) HASTE_LAUNCH_PARKED(8, 2) HASTE_LAUNCH_PARKED(8, 4)
-  HASTE_LAUNCH_PARKED(16, 1) HASTE_LAUNCH_PARKED(16, 2)
+  HASTE_LAUNCH_PARKED(8, 1) HASTE_LAUNCH_PARKED(8, 2) HASTE_LAUNCH_PARKED(16, 1)
 #undef HASTE_LAUNCH_PARKED
 #define HASTE_LAUNCH(NB_, CT_)                                                               \
   if (tile.nb == NB_ && tile.ct == CT_)                                                      \
