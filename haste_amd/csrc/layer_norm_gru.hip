@@ -318,7 +318,7 @@ void ln_gru_backward_kernel(LnGruBwdParams p) {
   const int n0 = role.bt * p.ls.tile_rows;
   const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;
   const size_t NH = (size_t)N * H;
-  const bool in_wavefront = row_gather_in_wavefront<HSB>(gx);
+  const bool in_wavefront = row_sums_gather_in_wavefront<HSB>(gx, NB);
   const size_t row_words = tagged_row_words(gx, NB, 3);
   unsigned long long* part = p.part + (size_t)role.bt * 2 * row_words;
 

@@ -306,6 +306,15 @@ __device__ __forceinline__ void sum_row_partials_polled(const GroupSync& g,
 // result over through LDS.
 template <int HS>
 __device__ __forceinline__ bool row_gather_in_wavefront(int gx) { return gx <= 4 * HS; }
+// The backward passes, whose slots hold 3 or 10 values: with more than two slots per lane the
+// gather inside the wavefront only pays for tiles of 32 rows and more, where the other form
+// has a wavefront poll for eight or sixteen rows one after the other (LayerNormLSTM backward,
+// T = 100: N = 64, H = 1024 on 16-row tiles 3.27 -> 2.89 ms with the hand-over through LDS,
+// N = 128, H = 640 on 32-row tiles 2.62 -> 2.88).
+template <int HS>
+__device__ __forceinline__ bool row_sums_gather_in_wavefront(int gx, int nb) {
+  return gx <= 2 * HS || (gx <= 4 * HS && nb >= 32);
+}
 
 // The slots of `row` from the column workgroups cw0, cw0 + step, ... (NCH of them, those beyond
 // gx skipped), all loads in flight together and re-issued until every tag matches.
