@@ -44,10 +44,13 @@ struct LnLstmFwdParams {
 // wavefront requests the next step's inputs and parks them in LDS for the owners of the elements,
 // see ln_lstm_backward_kernel.
 constexpr int kLnLstmFwdInputs = 5;  // floats per element and step: LN(x*W) of the four gates, the mask
-template <int NB, int CT, bool PARK = false>
+// REG > 0 (tiles of 16 rows and more): the slice exceeds LDS; every wavefront keeps the first REG
+// k-groups of its share of the contraction in registers (tall_tile_product).
+template <int NB, int CT, bool PARK = false, int REG = 0>
 __global__ __launch_bounds__(256, 1)
 void ln_lstm_forward_kernel(LnLstmFwdParams p) {
   static_assert(!PARK || NB * 4 * CT <= 64, "parked inputs: one element per lane of the idle last wavefront");
+  static_assert(REG == 0 || (NB >= 16 && !PARK), "register-resident slice rows: tall tiles only");
   constexpr int HS = 4 * CT;
   constexpr int NCOLS = 16 * CT;
   constexpr int PP = (NB * HS + 255) / 256;
@@ -59,7 +62,7 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
   const int H = p.H, N = p.N, T = p.T;
   const int Kpad = round_up(H, 64);
   float* w_lds = lds;
-  float* red = lds + Kpad * NCOLS;
+  float* red = lds + (Kpad - 64 * REG) * NCOLS;
   float* stat = red + ProductTile<NB, CT>::kRedFloats;  // [2][NB][2] row statistics (long rows only)
   float* park = stat + 4 * NB;  // PARK: [2][5][NB * HS] inputs of a step, by step parity
 
@@ -91,12 +94,22 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
   clear_row_words(gs, part2, gx, role.cw, NB, 2);
   clear_row_words(gs, part3, gx, role.cw, NB, 2);
 
+  float4_t breg[REG > 0 ? REG : 1][CT];
   {
     const bool fast = H % 4 == 0 && (reinterpret_cast<uintptr_t>(p.R) & 15u) == 0;
-    fill_slice<NCOLS>(w_lds, Kpad, p.R, nullptr, 1.0f, fast, [=](int k, int col) {
+    auto offset = [=](int k, int col) {
       const int gate = col / HS, j = j0 + col % HS;
       return (k < H && j < H) ? (long long)k * 4 * H + gate * H + j : -1ll;
-    });
+    };
+    if constexpr (REG > 0) {
+      const int groups = Kpad >> 6;
+      fill_slice<NCOLS>(w_lds, Kpad - 64 * REG, p.R, nullptr, 1.0f, fast, [=](int k, int col) {
+        return offset(resident_split_k(k, groups, REG), col);
+      });
+      load_resident_rows<REG, CT>(breg, groups, p.R, nullptr, 1.0f, offset);
+    } else {
+      fill_slice<NCOLS>(w_lds, Kpad, p.R, nullptr, 1.0f, fast, offset);
+    }
   }
 
   int pn[PP], pj[PP], pl[PP], pc[PP];
@@ -216,7 +229,11 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
     unsigned long long* ex3 = part3 + (size_t)(t & 1) * row_words;
 
     // The operand loads wait for h[t] themselves (polled tile t % 4).
-    tile_product<NB, CT, false, true>(xhb, (t & 3) * tile_floats, Kpad, w_lds, red, &gs);
+    if constexpr (REG > 0)
+      tile_product<NB, CT, false, true, false, NoSideWork, REG, float4_t[REG][CT]>(
+          xhb, (t & 3) * tile_floats, Kpad, w_lds, red, &gs, nullptr, &breg);
+    else
+      tile_product<NB, CT, false, true>(xhb, (t & 3) * tile_floats, Kpad, w_lds, red, &gs);
     __syncthreads();
     // After its share of the product the helper has nothing to do until the step's closing
     // barrier: time enough for loads from memory nobody has touched.
@@ -829,7 +846,8 @@ int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_siz
   HASTE_HIP_REQUIRE(W && R && b && x && h && c && act_Wx && gamma1 && act_Wx_norm && act_Rh);
   HASTE_HIP_REQUIRE(gamma2 && gamma_h && beta_h && act_c_norm);
   hipStream_t stream = as_stream(stream_);
-  const ForwardTile tile = pick_forward_tile(4, N, H, 4 * sizeof(float), kMaxLdsBytes, true);
+  const ForwardTile tile = pick_forward_tile(4, N, H, 4 * sizeof(float), kMaxLdsBytes, true,
+                                             resident_rows_enabled() ? 2 : 0);
   if (!tile.ok)
     return layer_norm_lstm_forward_streamed(stream, training, T, N, C, H, W, R, b, x, h, c, act_Wx,
                                             gamma1, cache1, act_Wx_norm, act_Rh, gamma2, cache2,
@@ -863,11 +881,20 @@ int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_siz
   // lane +1.3 % (N = 64, H = 512), and with rows too long for the gathers inside a wavefront
   // +2.5 % (N = 16, H = 1024), so those keep their own requests.
   const size_t park_bytes = (size_t)2 * kLnLstmFwdInputs * NB * tile.hs * sizeof(float);
-  const bool parked = NB * tile.hs <= 64 && gx <= 4 * tile.hs && tile.lds_bytes + park_bytes <= kMaxLdsBytes;
+  const bool parked = tile.reg_groups == 0 && NB * tile.hs <= 64 && gx <= 4 * tile.hs &&
+                      tile.lds_bytes + park_bytes <= kMaxLdsBytes;
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes + (parked ? park_bytes : 0),
                                   3u * (unsigned)T + 1, &plan));
   p.ls = plan.shape;
+#define HASTE_LAUNCH_RESIDENT(NB_, REG_)                                                      \
+  if (tile.reg_groups == REG_ && tile.nb == NB_ && tile.ct == 2)                             \
+    return launch_persistent("layer_norm_lstm_forward_recurrence",                           \
+                             ln_lstm_forward_kernel<NB_, 2, false, REG_>, plan, p, stream);
+  HASTE_LAUNCH_RESIDENT(16, 8) HASTE_LAUNCH_RESIDENT(32, 8) HASTE_LAUNCH_RESIDENT(64, 8)
+  HASTE_LAUNCH_RESIDENT(16, 16) HASTE_LAUNCH_RESIDENT(32, 16) HASTE_LAUNCH_RESIDENT(64, 16)
+#undef HASTE_LAUNCH_RESIDENT
+  if (tile.reg_groups > 0) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 #define HASTE_LAUNCH_PARKED(NB_, CT_)                                                        \
   if (parked && tile.nb == NB_ && tile.ct == CT_)                                            \
     return launch_persistent("layer_norm_lstm_forward_recurrence",                           \

@@ -20,7 +20,9 @@ SHAPES = [(1, 1, 3, 4), (3, 2, 3, 4), (5, 3, 7, 5), (6, 17, 20, 36), (4, 16, 32,
           (2, 3, 8, 1028),
           # hidden sizes whose backward recurrence keeps part of its slice of R in registers
           # (LSTM: 592 < H <= 1104, GRU: 784 < H <= 1472), tiles of 16, 32 and 64 rows
-          (3, 20, 16, 768), (3, 64, 24, 1024), (2, 100, 8, 900), (2, 40, 8, 1300), (3, 130, 8, 1000)]
+          (3, 20, 16, 768), (3, 64, 24, 1024), (2, 100, 8, 900), (2, 40, 8, 1300), (3, 130, 8, 1000),
+          # ... and whose forward recurrence does (512 < H <= 2048 at small batches)
+          (4, 16, 8, 640), (3, 7, 8, 2048), (2, 33, 8, 1600)]
 
 
 @pytest.mark.parametrize("zoneout", [0.0, 0.3])
