@@ -68,7 +68,7 @@ void ln_lstm_forward_kernel(LnLstmFwdParams p) {
 
   const int tid = threadIdx.x;
   const int gx = p.ls.gx;
-  const bool in_wavefront = row_gather_in_wavefront<HS>(gx);
+  const bool in_wavefront = row_gather_in_wavefront<HS, NB>(gx);
   const int j0 = role.cw * HS;
   const int n0 = role.bt * p.ls.tile_rows;
   const int rows_here = (N - n0) < p.ls.tile_rows ? (N - n0) : p.ls.tile_rows;

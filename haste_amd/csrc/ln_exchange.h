@@ -406,11 +406,19 @@ __device__ __forceinline__ void sum_row_partials_polled(const GroupSync& g,
 // c, c + HS, ... and the segment adds up with DPP row operations, after which every lane of
 // the segment holds the row's totals -- no LDS, no workgroup barrier, and wavefronts without
 // elements do not take part.  Every workgroup adds in the same order, so all of them obtain
-// bit-identical results.  For rows of at most 4 * HS parts (row_gather_in_wavefront); longer
-// rows take the gathers below, which put all 64 lanes of a wavefront on one row and hand the
-// result over through LDS.
-template <int HS>
-__device__ __forceinline__ bool row_gather_in_wavefront(int gx) { return gx <= 4 * HS; }
+// bit-identical results.  For rows of at most 4 * HS parts, and more for narrow workgroups
+// (row_gather_in_wavefront); longer rows take the gathers further up, which put all 64 lanes of
+// a wavefront on one row and hand the result over through LDS.
+// Workgroups of 8 or 4 units whose tile keeps at least two (8 units) or all four wavefronts
+// busy gather rows of up to 16 * HS parts this way, all of a lane's slots in one poll: their
+// rows are the long ones (H > 512: 72 to 128 parts), and through LDS every wavefront polls
+// for four to sixteen rows.  LayerNormLSTM forward, T = 100: N = 64, H = 768 2.03 -> 1.69 ms,
+// N = 128, H = 1024 3.59 -> 2.99, N = 32, H = 1024 1.66 -> 1.28; tiles that leave more
+// wavefronts idle lose that way (N = 8, H >= 576: +11 %; N = 64, H = 128: +7 %).
+template <int HS, int NB>
+__device__ __forceinline__ bool row_gather_in_wavefront(int gx) {
+  return gx <= 4 * HS || (HS <= 8 && NB * HS >= (HS == 8 ? 128 : 256) && gx <= 16 * HS);
+}
 // The backward passes, whose slots hold 3 or 10 values: with more than two slots per lane the
 // gather inside the wavefront only pays for tiles of 32 rows and more, where the other form
 // has a wavefront poll for eight or sixteen rows one after the other (LayerNormLSTM backward,
@@ -530,7 +538,12 @@ __device__ __forceinline__ void gather_row_moments(const GroupSync& g, unsigned 
   };
   if (gx <= HS) both(std::integral_constant<int, 1>{});
   else if (gx <= 2 * HS) both(std::integral_constant<int, 2>{});
-  else both(std::integral_constant<int, 4>{});
+  else if (HS > 8 || gx <= 4 * HS) both(std::integral_constant<int, 4>{});
+  else if constexpr (HS <= 8) {
+    // narrow workgroups (8 or 4 units): rows of up to 16 * HS parts, all slots of a lane in one poll
+    if (gx <= 8 * HS) both(std::integral_constant<int, 8>{});
+    else both(std::integral_constant<int, 16>{});
+  }
 }
 
 // Row sums of W values per slot from a tagged buffer: out[row * RowSlot<W>::kWords + i] in LDS.
