@@ -30,11 +30,14 @@ struct LnGruFwdParams {
   LaunchShape ls;
 };
 
-// NB batch rows per workgroup.
-template <int NB, int CT, int HS>
+// NB batch rows per workgroup.  REG > 0 (tiles of 16 rows and more): the slice exceeds LDS; every
+// wavefront keeps the first REG k-groups of its share of the contraction in registers
+// (tall_tile_product).
+template <int NB, int CT, int HS, int REG = 0>
 __global__ __launch_bounds__(256, 1)
 void ln_gru_forward_kernel(LnGruFwdParams p) {
   static_assert(3 * HS <= 16 * CT, "slice too narrow");
+  static_assert(REG == 0 || NB >= 16, "register-resident slice rows: tall tiles only");
   constexpr int NCOLS = 16 * CT;
   constexpr int PP = (NB * HS + 255) / 256;
   extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -45,7 +48,7 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
   const int H = p.H, N = p.N, T = p.T;
   const int Kpad = round_up(H, 64);
   float* w_lds = lds;
-  float* red = lds + Kpad * NCOLS;
+  float* red = lds + (Kpad - 64 * REG) * NCOLS;
   float* stat = red + ProductTile<NB, CT>::kRedFloats;  // [NB][2] row statistics (long rows only)
 
   const int tid = threadIdx.x;
@@ -74,12 +77,22 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
                   kPolledTiles);
   clear_row_words(gs, part2, gx, role.cw, NB, 2);
 
+  float4_t breg[REG > 0 ? REG : 1][CT];
   {
     const bool fast = H % 4 == 0 && (reinterpret_cast<uintptr_t>(p.R) & 15u) == 0;
-    fill_slice<NCOLS>(w_lds, Kpad, p.R, nullptr, 1.0f, fast, [=](int k, int col) {
+    auto offset = [=](int k, int col) {
       const int gate = col / HS, j = j0 + col % HS;
       return (k < H && gate < 3 && j < H) ? (long long)k * 3 * H + gate * H + j : -1ll;
-    });
+    };
+    if constexpr (REG > 0) {
+      const int groups = Kpad >> 6;
+      fill_slice<NCOLS>(w_lds, Kpad - 64 * REG, p.R, nullptr, 1.0f, fast, [=](int k, int col) {
+        return offset(resident_split_k(k, groups, REG), col);
+      });
+      load_resident_rows<REG, CT>(breg, groups, p.R, nullptr, 1.0f, offset);
+    } else {
+      fill_slice<NCOLS>(w_lds, Kpad, p.R, nullptr, 1.0f, fast, offset);
+    }
   }
 
   int pn[PP], pj[PP], pl[PP], pc[PP];
@@ -151,7 +164,11 @@ void ln_gru_forward_kernel(LnGruFwdParams p) {
     unsigned long long* ex2 = part2 + (size_t)(t & 1) * row_words;
 
     // The operand loads wait for h[t] themselves (polled tile t % 4).
-    tile_product<NB, CT, false, true>(xhb, (t & 3) * tile_floats, Kpad, w_lds, red, &gs);
+    if constexpr (REG > 0)
+      tile_product<NB, CT, false, true, false, NoSideWork, REG, float4_t[REG][CT]>(
+          xhb, (t & 3) * tile_floats, Kpad, w_lds, red, &gs, nullptr, &breg);
+    else
+      tile_product<NB, CT, false, true>(xhb, (t & 3) * tile_floats, Kpad, w_lds, red, &gs);
     __syncthreads();
 
     float rh[PP][3];
@@ -646,7 +663,8 @@ int haste_hip_layer_norm_gru_forward_f32(int training, int steps, int batch_size
   HASTE_HIP_REQUIRE(W && R && bx && br && x && h && act_Wx && gamma1 && tmp_Wx_norm && act_Rh && gamma2);
   HASTE_HIP_REQUIRE(!training || v != nullptr);
   hipStream_t stream = as_stream(stream_);
-  const ForwardTile tile = pick_forward_tile(3, N, H, 2 * sizeof(float), kMaxLdsBytes, true);
+  const ForwardTile tile = pick_forward_tile(3, N, H, 2 * sizeof(float), kMaxLdsBytes, true,
+                                             resident_rows_enabled() ? 3 : 0);
   if (!tile.ok)
     return layer_norm_gru_forward_streamed(stream, training, T, N, C, H, W, R, bx, br, x, h, v, act_Wx,
                                            gamma1, cache1, tmp_Wx_norm, act_Rh, gamma2, cache2,
@@ -675,6 +693,15 @@ int haste_hip_layer_norm_gru_forward_f32(int training, int steps, int batch_size
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, gx, gy, tile.nb, tile.lds_bytes, 2u * (unsigned)T + 1, &plan));
   p.ls = plan.shape;
+#define HASTE_LAUNCH_RESIDENT(NB_, CT_, HS_, REG_)                                            \
+  if (tile.reg_groups == REG_ && tile.nb == NB_ && tile.hs == HS_)                           \
+    return launch_persistent("layer_norm_gru_forward_recurrence",                            \
+                             ln_gru_forward_kernel<NB_, CT_, HS_, REG_>, plan, p, stream);
+  HASTE_LAUNCH_RESIDENT(16, 2, 8, 8) HASTE_LAUNCH_RESIDENT(32, 2, 8, 8) HASTE_LAUNCH_RESIDENT(64, 2, 8, 8)
+  HASTE_LAUNCH_RESIDENT(16, 2, 8, 16) HASTE_LAUNCH_RESIDENT(32, 2, 8, 16) HASTE_LAUNCH_RESIDENT(64, 2, 8, 16)
+  HASTE_LAUNCH_RESIDENT(16, 3, 16, 8) HASTE_LAUNCH_RESIDENT(32, 3, 16, 8) HASTE_LAUNCH_RESIDENT(64, 3, 16, 8)
+#undef HASTE_LAUNCH_RESIDENT
+  if (tile.reg_groups > 0) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 #define HASTE_LAUNCH(NB_, CT_, HS_)                                                          \
   if (tile.nb == NB_ && tile.hs == HS_)                                                      \
     return launch_persistent("layer_norm_gru_forward_recurrence",                            \
