@@ -204,6 +204,54 @@ def test_many_launches_in_a_row_are_bit_equal_to_the_first():
     print("streaming shape: 200 launches", flush=True)
 
 
+@pytest.mark.parametrize("T,N,C,H,launches", [(50, 32, 32, 256, 400), (20, 64, 16, 768, 150), (30, 8, 16, 128, 200)])
+def test_many_layer_norm_launches_in_a_row_are_bit_equal_to_the_first(T, N, C, H, launches):
+    """The layer-norm cells add tagged row exchanges, gathers inside a wavefront and inputs parked
+    in LDS by a helper wavefront to the lock-free machinery: repeated LayerNormLSTM and LayerNormGRU
+    forward + backward passes (4-row tiles with parked inputs; tall tiles across XCDs; a tile that
+    leaves wavefronts idle) must give the first launch's bits every time.  Stops at the first
+    mismatch."""
+    import torch
+    from haste_amd import ops
+    print("ln soak", T, N, C, H, launches, flush=True)
+    p = problem(77 + H, T, N, C, H, 4, 0.2)
+    mask = dev(p["mask"])
+    x, h0, c0 = dev(p["x"]), dev(p["h0"]), dev(p["c0"])
+    W, R, b = dev(p["W"]), dev(p["R"]), dev(p["b"])
+    gam, gh, bh = dev(p["gamma"]), dev(p["gamma_h"]), dev(p["beta_h"])
+    x_t, W_t, R_t = ops.transpose3(x, W, R)
+    dh_new, dc_new = dev(p["dh_new"]), dev(p["dc_new"])
+
+    def lstm_pass():
+        outs = ops.layer_norm_lstm_forward(True, 0.2, x, h0, c0, W, R, b, gam, gh, bh, mask)
+        h, c, act_Wx, act_Wx_norm, cache1, act_Rh, cache2, act_c_norm, cache3 = outs
+        keep = (h.clone(), c.clone(), act_Rh.clone(), act_c_norm.clone())
+        g = ops.layer_norm_lstm_backward(x_t, W_t, R_t, b, gam, gh, bh, mask, h, c, act_Wx, act_Wx_norm,
+                                         cache1, act_Rh, cache2, act_c_norm, cache3, dh_new, dc_new)
+        return keep + tuple(g)
+
+    W3, R3, b3 = W[:, :3 * H].contiguous(), R[:, :3 * H].contiguous(), b[:3 * H].contiguous()
+    gam3 = gam[:, :3 * H].contiguous()
+    x_t3, W3_t, R3_t = ops.transpose3(x, W3, R3)
+
+    def gru_pass():
+        h, cache, act_Wx, cache1, act_Rh, cache2 = ops.layer_norm_gru_forward(
+            True, 0.2, x, h0, W3, R3, b3, b3, gam3, mask)
+        keep = (h.clone(), act_Rh.clone())
+        g = ops.layer_norm_gru_backward(x_t3, W3_t, R3_t, b3, b3, gam3, mask, h, cache, act_Wx, cache1,
+                                        act_Rh, cache2, dh_new)
+        return keep + tuple(g)
+
+    for name, one_pass in (("LayerNormLSTM", lstm_pass), ("LayerNormGRU", gru_pass)):
+        first = one_pass()
+        torch.cuda.synchronize()
+        for i in range(launches):
+            outs = one_pass()
+            same = all(torch.equal(a, b) for a, b in zip(first, outs))  # synchronizes
+            assert same, "%s launch %d differs from the first" % (name, i + 1)
+        print("%s: %d launches" % (name, launches), flush=True)
+
+
 def test_two_host_threads_on_two_streams_match_the_serial_results():
     """Each thread runs forward + backward passes of its own problem on its own stream; the
     persistent kernels of the two streams are chained by the library.  Results must equal the
