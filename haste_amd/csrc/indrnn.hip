@@ -2,9 +2,8 @@
 //
 // The recurrence h_{t+1} = tanh((xW)_t + u*h_t + b) is elementwise, so there is no
 // exchange between threads: one thread owns one (batch row, hidden unit) pair and
-// walks all T steps.  The only cost is the serial chain of HBM loads, so each thread
-// keeps a block of U future steps' operands in flight while it computes the current
-// block.  Consecutive lanes own consecutive hidden units (coalesced 256-byte rows).
+// walks all T steps.  Each thread keeps a block of U future steps' operands in flight
+// while it computes the current block; what remains is the dependent chain of the steps.  Consecutive lanes own consecutive hidden units (coalesced 256-byte rows).
 //
 // Arithmetic follows reference lib/indrnn_forward_gpu.cu.cc:44-62 and
 // lib/indrnn_backward_gpu.cu.cc:46-73; orchestration replaces :114-210 and :122-207
@@ -15,7 +14,11 @@ namespace haste_hip {
 namespace {
 
 // Steps of operands kept in flight per thread (twice that while the next batch is requested).
-// 16 is 5-14 % faster than 8 (N*H = 8192 .. 131072 chains); 32 no better.
+// 16 is 5-14 % faster than 8 (N*H = 8192 .. 131072 chains); 32 no better, nor are two or three
+// batches in flight beyond the current one: the time is the dependent chain of a step, not the
+// loads.  Whole batches run without a bounds check per step (17 % faster: the check is a scalar
+// compare and a branch in every step of the chain); requests beyond the sequence read its last
+// step again and are never used.
 constexpr int U = 16;
 
 template <bool TRAINING, bool ZONEOUT>
@@ -36,32 +39,37 @@ void indrnn_forward_kernel(int T, int N, int H, const float* __restrict__ Wx,
   auto fetch = [&](int t0, float (&wx)[U], float (&mk)[U]) {
 #pragma unroll
     for (int i = 0; i < U; ++i) {
-      const int t = t0 + i;
-      wx[i] = t < T ? Wx[(size_t)t * NH + idx] : 0.f;
-      mk[i] = (ZONEOUT && TRAINING && t < T) ? mask[(size_t)t * NH + idx] : 1.f;
+      const int t = t0 + i < T ? t0 + i : T - 1;
+      wx[i] = Wx[(size_t)t * NH + idx];
+      mk[i] = (ZONEOUT && TRAINING) ? mask[(size_t)t * NH + idx] : 1.f;
     }
   };
+  auto step = [&](int t, float wx, float mk) {
+    float hn = tanh_f(wx + uj * hv + bj);
+    if (ZONEOUT) {
+      if (TRAINING) hn = (hn - hv) * mk + hv;
+      else hn = zoneout_prob * hv + (1.0f - zoneout_prob) * hn;
+    }
+    h[(size_t)(t + 1) * NH + idx] = hn;
+    hv = hn;
+  };
   fetch(0, wx_cur, mk_cur);
-  for (int t0 = 0; t0 < T; t0 += U) {
+  int t0 = 0;
+  for (; t0 + U <= T; t0 += U) {
     fetch(t0 + U, wx_nxt, mk_nxt);
 #pragma unroll
-    for (int i = 0; i < U; ++i) {
-      const int t = t0 + i;
-      if (t < T) {
-        float hn = tanh_f(wx_cur[i] + uj * hv + bj);
-        if (ZONEOUT) {
-          if (TRAINING) hn = (hn - hv) * mk_cur[i] + hv;
-          else hn = zoneout_prob * hv + (1.0f - zoneout_prob) * hn;
-        }
-        h[(size_t)(t + 1) * NH + idx] = hn;
-        hv = hn;
-      }
-    }
+    for (int i = 0; i < U; ++i) step(t0 + i, wx_cur[i], mk_cur[i]);
 #pragma unroll
     for (int i = 0; i < U; ++i) { wx_cur[i] = wx_nxt[i]; mk_cur[i] = mk_nxt[i]; }
   }
+  // the last, partial batch
+#pragma unroll
+  for (int i = 0; i < U; ++i)
+    if (t0 + i < T) step(t0 + i, wx_cur[i], mk_cur[i]);
 }
 
+// Walks the steps backwards; h[t+1] of a step is h[t] of the step before it in the walk, so
+// every state is loaded once.
 template <bool ZONEOUT>
 __global__ __launch_bounds__(256)
 void indrnn_backward_kernel(int T, int N, int H, const float* __restrict__ u,
@@ -75,50 +83,53 @@ void indrnn_backward_kernel(int T, int N, int H, const float* __restrict__ u,
   const bool live = j < H && n < N;
   const size_t NH = (size_t)N * H;
   const size_t idx = live ? (size_t)n * H + j : 0;
-  const float uj = live ? u[j] : 0.f;
-  float dh_io = live ? dh[idx] : 0.f;
   float du_sum = 0.f, db_sum = 0.f;
 
-  struct In { float hn, hp, d, m; };
-  In cur[U], nxt[U];
-  auto fetch = [&](int t_hi, In (&s)[U]) {
+  if (live) {
+    const float uj = u[j];
+    float dh_io = dh[idx];
+    float hn = h[(size_t)T * NH + idx];
+
+    struct In { float hp, d, m; };
+    In cur[U], nxt[U];
+    auto fetch = [&](int t_hi, In (&s)[U]) {
 #pragma unroll
-    for (int i = 0; i < U; ++i) {
-      const int t = t_hi - i;
-      In v = {0.f, 0.f, 0.f, 1.f};
-      if (live && t >= 0) {
-        v.hn = h[(size_t)(t + 1) * NH + idx];
-        v.hp = h[(size_t)t * NH + idx];
-        v.d = dh_new[(size_t)(t + 1) * NH + idx];
-        if (ZONEOUT) v.m = mask[(size_t)t * NH + idx];
+      for (int i = 0; i < U; ++i) {
+        const int t = t_hi - i > 0 ? t_hi - i : 0;
+        s[i].hp = h[(size_t)t * NH + idx];
+        s[i].d = dh_new[(size_t)(t + 1) * NH + idx];
+        s[i].m = ZONEOUT ? mask[(size_t)t * NH + idx] : 1.f;
       }
-      s[i] = v;
-    }
-  };
-  fetch(T - 1, cur);
-  for (int t_hi = T - 1; t_hi >= 0; t_hi -= U) {
-    fetch(t_hi - U, nxt);
-#pragma unroll
-    for (int i = 0; i < U; ++i) {
-      const int t = t_hi - i;
-      if (live && t >= 0) {
-        float dh_total = cur[i].d + dh_io;
-        float keep = 0.f;
-        if (ZONEOUT) {
-          keep = (1.0f - cur[i].m) * dh_total;
-          dh_total = cur[i].m * dh_total;
-        }
-        const float k = d_tanh_f(cur[i].hn) * dh_total;
-        dk[(size_t)t * NH + idx] = k;
-        dh_io = keep + uj * k;
-        du_sum += cur[i].hp * k;
-        db_sum += k;
+    };
+    auto step = [&](int t, const In& in) {
+      float dh_total = in.d + dh_io;
+      float keep = 0.f;
+      if (ZONEOUT) {
+        keep = (1.0f - in.m) * dh_total;
+        dh_total = in.m * dh_total;
       }
-    }
+      const float k = d_tanh_f(hn) * dh_total;
+      dk[(size_t)t * NH + idx] = k;
+      dh_io = keep + uj * k;
+      du_sum += in.hp * k;
+      db_sum += k;
+      hn = in.hp;
+    };
+    fetch(T - 1, cur);
+    int t_hi = T - 1;
+    for (; t_hi - U + 1 >= 0; t_hi -= U) {
+      fetch(t_hi - U, nxt);
 #pragma unroll
-    for (int i = 0; i < U; ++i) cur[i] = nxt[i];
+      for (int i = 0; i < U; ++i) step(t_hi - i, cur[i]);
+#pragma unroll
+      for (int i = 0; i < U; ++i) cur[i] = nxt[i];
+    }
+    // the last, partial batch
+#pragma unroll
+    for (int i = 0; i < U; ++i)
+      if (t_hi - i >= 0) step(t_hi - i, cur[i]);
+    dh[idx] = dh_io;
   }
-  if (live) dh[idx] = dh_io;
 
   // Column sums over the batch: 4 rows per workgroup in LDS, then workgroups in order.
   red[0][w][lane] = du_sum;
