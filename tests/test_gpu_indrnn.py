@@ -7,8 +7,9 @@ from util import TOL, dev, host, problem, relerr
 
 pytestmark = pytest.mark.gpu
 
-SHAPES = [(1, 1, 1, 1), (3, 2, 3, 4), (9, 3, 7, 5), (17, 5, 20, 70), (30, 16, 32, 256),
-          (50, 64, 64, 512)]
+# T on both sides of the kernels' batches of 16 steps: no whole batch, whole batches only, a tail
+SHAPES = [(1, 1, 1, 1), (3, 2, 3, 4), (9, 3, 7, 5), (15, 2, 3, 6), (16, 3, 5, 70), (17, 5, 20, 70),
+          (30, 16, 32, 256), (32, 2, 4, 33), (33, 2, 4, 33), (50, 64, 64, 512)]
 
 
 @pytest.mark.parametrize("layer_norm", [False, True])
