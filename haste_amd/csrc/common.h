@@ -148,6 +148,11 @@ bool fused_input_enabled();
 // of keeping part of the slice in registers (for experiments).
 bool resident_rows_enabled();
 
+// False when the environment variable HASTE_HIP_SCATTER_BACKWARD is set to 0: the backward
+// recurrences of 4-row tiles then exchange the gate gradients (every workgroup gathers all of
+// them) instead of partial sums of dh (for experiments).
+bool scatter_backward_enabled();
+
 // C[M,N] = op(A)*B (+C): fp32 MFMA GEMM on `stream`.  The partial tiles of a split product
 // are kept `scratch_offset` bytes (a multiple of 16) into the stream's scratch buffer.
 int gemm_f32(hipStream_t stream, bool trans_a, int M, int N, int K,

@@ -1210,6 +1210,154 @@ __device__ __forceinline__ void reset_partials(float* red, int live) {
     red[i] = (i % P::kRedFloats) / TILE < live ? unwritten_value() : 0.f;
 }
 
+// ---- scattered partial sums (backward recurrences, 4-row tiles) --------------------------
+// The backward step dh = dv * R_t contracts over the gate gradients of ALL hidden units.  A
+// workgroup that owns output units must therefore gather the whole of dv (4 gates wide) from
+// every other workgroup before its matrix units can start.  The scattered form turns the
+// ownership round: a workgroup contracts over the gate gradients it has just computed itself
+// -- the G gates of its 16 units, a single MFMA operand register per lane -- against the rows
+// of R_t that belong to those units and ALL H columns, and hands every owner its 4 x 16 piece
+// of the partial sums; the owner adds the pieces of all producers in index order.  What
+// crosses between workgroups is H wide instead of G*H wide, the products wait for nothing
+// remote, and a wavefront's share of R_t (its 64*CTN output columns, the workgroup's 16*G
+// rows) lives in registers for the whole launch, so the step has no LDS traffic to speak of.
+//
+// Pieces: per 4-row batch tile two tiles (alternating by step) of [owner][producer][unit][row]
+// floats (a piece is 64 floats).  Producers are padded to kProducers per owner; the padding
+// holds zeros for good and its tags are not looked at.  A piece is polled like the exchange tiles above
+// -- the owner's loads are themselves the wait -- but what marks an element as written is a
+// TAG in its lowest mantissa bit: the use count of its slot, modulo 2.  A piece written at
+// step d (tile d%2, tag (d/2)%2) is read at step d+1 and written again at step d+2, with the
+// other tag, so what the slot held before can never pass for new data and nothing has to be
+// reset in between (resetting the pieces cost as much L2 write bandwidth as publishing them:
+// 512 KiB per XCD and step each at H = 512, 800 cycles of a 6 400-cycle step).  At step d+2 the
+// producer's workgroup has seen the sums of step d+1, which every producer publishes only after
+// its workgroup has finished reading step d, so the slot is free.  The price is the last bit
+// of each partial sum (a relative 6e-8, below the rounding of the sum of 32 of them); an
+// infinite partial sum tagged 1 reads as NaN, a NaN stays NaN.
+//
+// Agent-scope loads are not combined across lanes: every lane's access is a request of its
+// own to the L2 (a gather of 32 pieces with one float per lane and load took 3 500 cycles,
+// 1.7 per request).  So the pieces are read 16 bytes per lane -- lane 16*g + u the four rows of
+// unit u from the producers 4*i + g -- and by three wavefronts of the set at once (the owner
+// and the two that have no other duties between their publication and the owner's operand),
+// each adding up its share of the producers; the owner adds the three sums, and its four lane
+// groups then add theirs to each other so that each ends up with one row: the pointwise work
+// of the owner runs on lane 16*g + u = (row scatter_row(g), unit u), and the gate gradients
+// go to the lanes of the MFMA operand (lane 4*unit + row) from there.
+template <int CTN>
+struct ScatterShape {
+  static constexpr int kColumns = 64 * CTN;     // output columns of one wavefront
+  static constexpr int kProducers = 16 * CTN;   // producers per owner, padded (H <= 256 * CTN)
+  static constexpr int kPieceFloats = 64;
+  static constexpr int kLoads = kProducers / 4;              // 16-byte loads per lane, all producers
+  static constexpr int kOwnerLoads = 2;                      // ... of which the owner issues these
+  static constexpr int kOtherLoads = (kLoads - kOwnerLoads) / 2;  // ... and two others these each
+};
+
+constexpr int kScatterTiles = 2;
+inline size_t scatter_tile_floats(int gx, int ctn) { return (size_t)gx * 16 * ctn * 64; }
+// LDS of a set: the owner wavefront's operand for the three other wavefronts, by step parity;
+// the sums of the two other gathering wavefronts, by step parity; up to 12 parked inputs per
+// lane of the owner, by step parity; which step each parking area holds.
+constexpr size_t kScatterHandFloats = 2 * 3 * 64 * 4;
+constexpr size_t kScatterPartFloats = 2 * 2 * 64 * 4;
+constexpr size_t kScatterParkFloats = 2 * 12 * 64;
+constexpr size_t kScatterSetFloats = kScatterHandFloats + kScatterPartFloats + kScatterParkFloats + 4;
+
+// The batch row (of the tile's four) that lane group g of the owner ends up with.
+__device__ __forceinline__ int scatter_row(int g) { return ((g & 1) << 1) | (g >> 1); }
+
+// The tag of the pieces published at step d, and a value carrying a tag.
+__device__ __forceinline__ unsigned int scatter_tag(int d) { return ((unsigned int)d >> 1) & 1u; }
+__device__ __forceinline__ float tagged(float v, unsigned int tag) {
+  const unsigned int bits = v != v ? 0x7fc00000u : __float_as_uint(v);  // a NaN stays one
+  return __uint_as_float((bits & ~1u) | tag);
+}
+__device__ __forceinline__ float4_t tagged4(const float4_t& v, unsigned int tag) {
+  return float4_t{tagged(v.x, tag), tagged(v.y, tag), tagged(v.z, tag), tagged(v.w, tag)};
+}
+
+// A wavefront's share of an owner's gather: NLW consecutive groups of four producers, starting
+// with group `first`, of the pieces that start at float `owner_off` of `xb`.  Lane 16*g + u
+// ends up with the four rows of unit u summed over producers 4*i + g of its groups, added in
+// index order, once all of them carry the tag `tag`.  request() issues the loads; finish()
+// waits, polls and adds, so that work that does not depend on the sums can stand in between.
+// `gx`: producers that exist.
+template <int NLW>
+struct PieceGather {
+  float4_t v[NLW];
+  int base;
+  bool real[NLW];
+
+  __device__ __forceinline__ void load(const TileBuffer& xb) {
+#pragma unroll
+    for (int i = 0; i < NLW; ++i) v[i] = load_tile4(xb, base + i * 256);
+  }
+  __device__ __forceinline__ void request(const TileBuffer& xb, int owner_off, int first, int gx) {
+    const int lane = threadIdx.x & 63;
+    base = owner_off + (4 * first + (lane >> 4)) * 64 + (lane & 15) * 4;
+#pragma unroll
+    for (int i = 0; i < NLW; ++i) real[i] = 4 * (first + i) + (lane >> 4) < gx;
+    load(xb);
+  }
+  __device__ __forceinline__ float4_t finish(const GroupSync& gs, const TileBuffer& xb, unsigned int tag) {
+    auto written = [&] {
+      unsigned int m = 0u;
+#pragma unroll
+      for (int i = 0; i < NLW; ++i) {
+        const unsigned int q = (__float_as_uint(v[i].x) ^ tag) | (__float_as_uint(v[i].y) ^ tag) |
+                               (__float_as_uint(v[i].z) ^ tag) | (__float_as_uint(v[i].w) ^ tag);
+        m |= real[i] ? q : 0u;
+      }
+      return __all((m & 1u) == 0u) != 0;
+    };
+    poll_until_written(gs, [&] { load(xb); }, written);
+    float4_t s = v[0];
+#pragma unroll
+    for (int i = 1; i < NLW; ++i) s += v[i];
+    return s;
+  }
+};
+
+// The owner's last step: its four lane groups hold sums over different producers of the same
+// elements; lane groups 0, 1, 2, 3 end up with the totals of rows 0, 2, 1, 3 (scatter_row).
+__device__ __forceinline__ float scatter_lane_groups(const float4_t& s) {
+  return swap_add32(swap_add16(s.x, s.z), swap_add16(s.y, s.w));
+}
+
+// Reads a 16-byte word of LDS that another wavefront publishes (every element written with a
+// publishable value) until it is written, and resets it to "unwritten" for its next use.
+__device__ __forceinline__ float4_t take_lds4(const GroupSync& gs, float4_t* q) {
+  float4_t got[1][1];
+  got[0][0] = *q;
+  poll_until_written(gs, [&] { __builtin_amdgcn_s_sleep(1); got[0][0] = *q; }, [&] { return all_written(got); });
+  const float u = unwritten_value();
+  *q = float4_t{u, u, u, u};
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  return got[0][0];
+}
+
+__device__ __forceinline__ float4_t publishable4(const float4_t& v) {
+  return float4_t{publishable(v.x), publishable(v.y), publishable(v.z), publishable(v.w)};
+}
+
+// acc[c%2][ct] += a[c] (the operand of row l%4, k = 4*(l/4) + c, broadcast block by block)
+// times the lane's weights w[block][c][ct], for the G components in use: 16 * G * CTN MFMAs,
+// consecutive ones on different accumulators.
+template <int G, int CTN>
+__device__ __forceinline__ void scatter_product(const float4_t& a, const float (&w)[16][G][CTN],
+                                                float4_t (&acc)[2][CTN]) {
+  static_for<16>([&](auto bc) {
+    constexpr int A = decltype(bc)::value;
+#pragma unroll
+    for (int c = 0; c < G; ++c)
+#pragma unroll
+      for (int ct = 0; ct < CTN; ++ct)
+        acc[c & 1][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(a[c], w[A][c][ct], acc[c & 1][ct], 4, A, 0);
+  });
+}
+
 // ---- one batch row -----------------------------------------------------------------------
 // With a single batch row the step's product is a matrix-vector product.  The 4-row MFMA tile
 // spends three quarters of the matrix unit's time on padding and, like any tile, reads the

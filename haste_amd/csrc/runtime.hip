@@ -256,6 +256,14 @@ bool resident_rows_enabled() {
   return enabled;
 }
 
+bool scatter_backward_enabled() {
+  static const bool enabled = [] {
+    const char* v = std::getenv("HASTE_HIP_SCATTER_BACKWARD");
+    return v == nullptr || v[0] != '0';
+  }();
+  return enabled;
+}
+
 int device_cu_count() {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
@@ -558,6 +566,9 @@ size_t haste_hip_workspace_bytes(int time_steps, int batch_size, int input_size,
   b += 4 * kpad * rows * sizeof(float);
   b += 64 * 2 * 10 * (H + 4) * sizeof(float);
   b += 2 * 2 * 16 * (H / 4 + 2) * rows * 2 * sizeof(float);
+  // Backward recurrences of 4-row tiles in scattered form (H <= 512): two tiles of pieces per
+  // tile of 4 rows, [owners][up to 32 producers][64].
+  if (H <= 512) b += (N / 4 + 2) * 2 * (H / 16 + 1) * 32 * 64 * sizeof(float);
   // Step-wise regime (any scalar type up to 8 bytes): the step's product [N, 4H], a scaled
   // copy of R, column sums in at most 128 chunks, row statistics of all steps, two [N, H]
   // buffers; the stand-alone layer norm's column sums (two workgroups per CU, two rows each).
