@@ -874,8 +874,11 @@ void lstm_backward_scatter_kernel(LstmBwdParams p) {
   };
   auto all_sums = [&](PieceGather<S::kOwnerLoads>& pieces, int d) {
     float4_t sum = pieces.finish(gs, xpb, scatter_tag(d));
-    sum += take_lds4(gs, reinterpret_cast<float4_t*>(&s_part[d & 1][0][lane * 4]));
-    sum += take_lds4(gs, reinterpret_cast<float4_t*>(&s_part[d & 1][1][lane * 4]));
+    float4_t s2, s3;
+    take_lds4_pair(gs, reinterpret_cast<float4_t*>(&s_part[d & 1][0][lane * 4]),
+                   reinterpret_cast<float4_t*>(&s_part[d & 1][1][lane * 4]), s2, s3);
+    sum += s2;
+    sum += s3;
     return scatter_lane_groups(sum);
   };
   float dh_keep = 0.f;

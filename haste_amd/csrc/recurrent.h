@@ -78,10 +78,18 @@ __device__ __forceinline__ float4_t load_exchanged4(const float* p) {
 // and the products of one set never delay the pointwise work of the other (measured: sets
 // of four consecutive wavefronts, which share all four SIMDs, are 12 % slower per step).
 // set_thread: thread index inside the set (0..255); set_wave: wavefront inside the set.
+// (Both are the same in every lane of a wavefront, which the compiler cannot see from
+// threadIdx: told so, it keeps what is derived from them -- tile addresses, buffer resources
+// -- in scalar registers instead of wrapping every buffer load in a loop over the distinct
+// resources its lanes might hold.)
 template <int SETS>
-__device__ __forceinline__ int set_index() { return SETS == 1 ? 0 : (int)((threadIdx.x >> 6) & 1); }
+__device__ __forceinline__ int set_index() {
+  return SETS == 1 ? 0 : __builtin_amdgcn_readfirstlane((int)((threadIdx.x >> 6) & 1));
+}
 template <int SETS>
-__device__ __forceinline__ int set_wave() { return (int)(threadIdx.x >> (SETS == 1 ? 6 : 7)); }
+__device__ __forceinline__ int set_wave() {
+  return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> (SETS == 1 ? 6 : 7)));
+}
 template <int SETS>
 __device__ __forceinline__ int set_thread() {
   return SETS == 1 ? (int)threadIdx.x : (int)(((threadIdx.x >> 7) << 6) | (threadIdx.x & 63));
@@ -1270,9 +1278,9 @@ __device__ __forceinline__ int scatter_row(int g) { return ((g & 1) << 1) | (g >
 
 // The tag of the pieces published at step d, and a value carrying a tag.
 __device__ __forceinline__ unsigned int scatter_tag(int d) { return ((unsigned int)d >> 1) & 1u; }
+// (A NaN stays one: what arithmetic produces is a quiet NaN, whose top mantissa bit is set.)
 __device__ __forceinline__ float tagged(float v, unsigned int tag) {
-  const unsigned int bits = v != v ? 0x7fc00000u : __float_as_uint(v);  // a NaN stays one
-  return __uint_as_float((bits & ~1u) | tag);
+  return __uint_as_float((__float_as_uint(v) & ~1u) | tag);
 }
 __device__ __forceinline__ float4_t tagged4(const float4_t& v, unsigned int tag) {
   return float4_t{tagged(v.x, tag), tagged(v.y, tag), tagged(v.z, tag), tagged(v.w, tag)};
@@ -1326,16 +1334,31 @@ __device__ __forceinline__ float scatter_lane_groups(const float4_t& s) {
   return swap_add32(swap_add16(s.x, s.z), swap_add16(s.y, s.w));
 }
 
-// Reads a 16-byte word of LDS that another wavefront publishes (every element written with a
-// publishable value) until it is written, and resets it to "unwritten" for its next use.
+// Reads 16-byte words of LDS that other wavefronts publish (every element written with a
+// publishable value) until they are written, and resets them to "unwritten" for their next
+// use.  The reset is not waited for: the LDS operations of a wavefront complete in order, so it
+// has landed before anything this wavefront reads from LDS afterwards, and whoever writes the
+// word again has first seen something this wavefront published after such a read.
 __device__ __forceinline__ float4_t take_lds4(const GroupSync& gs, float4_t* q) {
   float4_t got[1][1];
   got[0][0] = *q;
   poll_until_written(gs, [&] { __builtin_amdgcn_s_sleep(1); got[0][0] = *q; }, [&] { return all_written(got); });
   const float u = unwritten_value();
   *q = float4_t{u, u, u, u};
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   return got[0][0];
+}
+__device__ __forceinline__ void take_lds4_pair(const GroupSync& gs, float4_t* q0, float4_t* q1, float4_t& v0,
+                                               float4_t& v1) {
+  float4_t got[2][1];
+  got[0][0] = *q0;
+  got[1][0] = *q1;
+  poll_until_written(gs, [&] { __builtin_amdgcn_s_sleep(1); got[0][0] = *q0; got[1][0] = *q1; },
+                     [&] { return all_written(got); });
+  const float u = unwritten_value();
+  *q0 = float4_t{u, u, u, u};
+  *q1 = float4_t{u, u, u, u};
+  v0 = got[0][0];
+  v1 = got[1][0];
 }
 
 __device__ __forceinline__ float4_t publishable4(const float4_t& v) {
