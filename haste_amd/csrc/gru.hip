@@ -5,7 +5,7 @@
 //
 // Arithmetic follows reference lib/gru_forward_gpu.cu.cc:46-84 and
 // lib/gru_backward_gpu.cu.cc:45-95; orchestration replaces :314-371 and :321-409.
-#include "recurrent.h"
+#include "scatter_backward.h"
 
 namespace haste_hip {
 namespace {
@@ -393,6 +393,7 @@ struct GruBwdParams {
   const float* zoneout_mask;
   float* db_partial;    // [batch tiles, 6H] scratch
   float* xdq;           // exchange tiles of dq: [batch tiles][2][Kpad/4][NB][4]
+                        // (scattered form: the pieces of partial sums, scatter_backward.h)
   LaunchShape ls;
 };
 
@@ -644,6 +645,85 @@ void gru_backward_kernel(GruBwdParams p) {
   }
 }
 
+// The GRU's pointwise backward step for the scattered form of the recurrence
+// (scatter_backward.h): arithmetic as in gru_backward_kernel.  dh contracts over
+// dq = (dp_z, dp_r, dq_g); the operand's fourth component carries dp_g for the caller's copy.
+struct GruScatterCell {
+  using Params = GruBwdParams;
+  static constexpr int kGates = 3;
+  static constexpr int kInputs = 7;  // v (z, r, g, q_g), h before the step, dh_next, mask
+  static constexpr int kSums = 6;    // dbx (3), dbr (3)
+  float dh, dh_keep;
+  float z, r, g, qg, h0, dhn, m, k_g, k_r, k_z;
+
+  __device__ __forceinline__ static float* pieces(const Params& p) { return p.xdq; }
+  __device__ __forceinline__ static void request(const Params& p, float (&in)[kInputs], size_t e, size_t ve,
+                                                 bool zoneout) {
+    const float* vt = p.v + ve;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) in[i] = vt[i * (size_t)p.H];
+    in[4] = p.h[e];
+    in[5] = p.dh_next[e];
+    if (zoneout) in[6] = p.zoneout_mask[e];
+  }
+  __device__ __forceinline__ void load_state(const Params& p, size_t e, bool mine) {
+    dh = mine ? p.dh[e] : 0.f;
+    dh_keep = 0.f;
+  }
+  __device__ __forceinline__ void store_state(const Params& p, size_t e) const { p.dh[e] = dh; }
+  __device__ __forceinline__ void prepare(const float (&sv)[kInputs]) {
+    z = sv[0]; r = sv[1]; g = sv[2]; qg = sv[3];
+    h0 = sv[4]; dhn = sv[5]; m = sv[6];
+    k_g = d_tanh_f(g);
+    k_r = d_sigmoid_f(r);
+    k_z = d_sigmoid_f(z);
+  }
+  __device__ __forceinline__ void add_gathered(float sum) { dh = dh_keep + sum; }
+  __device__ __forceinline__ float4_t step(bool act, bool zoneout, float (&sums)[kSums]) {
+    float4_t a = {0.f, 0.f, 0.f, 0.f};
+    dh_keep = 0.f;
+    if (act) {
+      float dh_total = dhn + dh;
+      if (zoneout) {
+        dh_keep = (1.0f - m) * dh_total;
+        dh_total = m * dh_total;
+        dh_keep += z * dh_total;
+      } else {
+        dh_keep = z * dh_total;
+      }
+      const float dg = (1.0f - z) * dh_total;
+      const float dz = (h0 - g) * dh_total;
+      const float dp_g = k_g * dg;
+      const float dq_g = dp_g * r;
+      const float dr = dp_g * qg;
+      const float dp_r = k_r * dr;
+      const float dp_z = k_z * dz;
+      a = float4_t{dp_z, dp_r, dq_g, dp_g};
+      sums[0] += dp_z;
+      sums[1] += dp_r;
+      sums[2] += dp_g;
+      sums[3] += dp_z;
+      sums[4] += dp_r;
+      sums[5] += dq_g;
+    }
+    return a;
+  }
+  __device__ __forceinline__ static void store_copy(const Params& p, int t, size_t n, size_t j, const float4_t& a) {
+    const size_t H = p.H;
+    const size_t o3 = ((size_t)t * p.N + n) * 3 * H + j;
+    p.dp[o3] = a[0];
+    p.dp[o3 + H] = a[1];
+    p.dp[o3 + 2 * H] = a[3];
+    p.dq[o3] = a[0];
+    p.dq[o3 + H] = a[1];
+    p.dq[o3 + 2 * H] = a[2];
+  }
+  __device__ __forceinline__ static void add_sums(const Params& p, int col, float s) {
+    if (col < 3 * p.H) p.dbx[col] += s;
+    else p.dbr[col - 3 * p.H] += s;
+  }
+};
+
 }  // namespace
 
 // The forward pass of a single batch row with H <= 512: the recurrent weights live in the
@@ -766,12 +846,19 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
 
   // An 8-row tile is run as two sets of 4 rows (see gru_forward_impl).
   const size_t paired_lds = paired_lds_bytes((gru_backward_k(H) + 63) / 64 * 64, 1);
-  const bool paired = tile.nb == 8 && paired_lds <= kMaxLdsBytes && paired_sets_enabled();
+  // 4-row tiles (8 rows: two sets of 4) with H <= 512 take the scattered form: partial sums of
+  // dh go to their owners instead of the gate gradients to everybody.
+  const bool scatter = scatter_backward_enabled() && tile.reg_groups == 0 && H <= 512 &&
+                       (tile.nb == 4 || tile.nb == 8);
+  const bool paired = scatter ? tile.nb == 8
+                              : tile.nb == 8 && paired_lds <= kMaxLdsBytes && paired_sets_enabled();
   const int sets = paired ? 2 : 1;
 
   Workspace ws;
   const size_t db_floats = ((size_t)tile.gy * sets * 6 * H + 3) / 4 * 4;
-  const size_t xdq_floats = exchange_floats(gru_backward_k(H), tile.nb, tile.gy, kPolledTiles);
+  const size_t xdq_floats =
+      scatter ? (size_t)tile.gy * sets * kScatterTiles * scatter_tile_floats(tile.gx, H <= 256 ? 1 : 2)
+              : exchange_floats(gru_backward_k(H), tile.nb, tile.gy, kPolledTiles);
   HASTE_HIP_PROPAGATE(get_workspace(stream, (db_floats + xdq_floats) * sizeof(float), &ws));
   HASTE_HIP_PROPAGATE(check_and_clear_abort(stream, &ws));
 
@@ -783,11 +870,15 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   p.xdq = ws.scratch + db_floats;
   LaunchPlan plan;
   HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.nb,
-                                  paired ? paired_lds : tile.lds_bytes, (unsigned)T + 1, &plan));
+                                  scatter ? sets * kScatterSetFloats * sizeof(float)
+                                          : (paired ? paired_lds : tile.lds_bytes),
+                                  (unsigned)T + 1, &plan));
   p.ls = plan.shape;
   if (paired) plan.threads = 512;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const char* name = "gru_backward_recurrence";
+  if (scatter) rc = launch_scatter_backward<GruScatterCell>(name, H, sets, plan, p, stream);
+  else
 #define HASTE_LAUNCH_BWD_RESIDENT(NB_)                                                           \
   (tile.reg_groups == 8    ? launch_persistent(name, gru_backward_kernel<NB_, 1, 8>, plan, p, stream)  \
    : tile.reg_groups == 16 ? launch_persistent(name, gru_backward_kernel<NB_, 1, 16>, plan, p, stream) \
