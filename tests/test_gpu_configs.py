@@ -62,6 +62,7 @@ def test_config2_gru_training_zoneout_dropconnect():
     dx, dW, dR, dbx, dbr, dh0, _, _ = O.gru_backward(p["W"], R_eff, p["b"], p["b2"], p["x"], ho, vo,
                                                      p["dh_new"], p["mask"])
     assert relerr(host(h), ho) < TOL
+    assert relerr(host(cache), vo) < TOL
     for name, ours, theirs in zip(("dx", "dh0", "dW", "dR", "dbx", "dbr"), outs,
                                   (dx, dh0, dW, dR, dbx, dbr)):
         assert relerr(host(ours), theirs) < TOL, name
@@ -118,12 +119,17 @@ def test_config4_layer_norm_lstm_training():
     f20 = O.layer_norm_lstm_forward(*args, p["x"][:20], p["h0"], p["c0"], True, 0.1, p["mask"][:20])
     assert relerr(hg[:21], f20["h"]) < TOL and relerr(cg[:21], f20["c"]) < TOL
     # (2) each step from the GPU's own state
-    worst = 0.0
+    # ... the new state and everything the step saves for the backward pass
+    sv = dict(v=host(act_Wx_norm), act_Rh=host(act_Rh), act_c_norm=host(act_c_norm),
+              cache2=host(cache2).reshape(T, N, 2), cache3=host(cache3).reshape(T, N, 2))
+    worst = {}
     for t in range(T):
         one = O.layer_norm_lstm_forward(*args, p["x"][t:t + 1], hg[t], cg[t], True, 0.1,
                                         p["mask"][t:t + 1])
-        worst = max(worst, relerr(hg[t + 1], one["h"][1]), relerr(cg[t + 1], one["c"][1]))
-    assert worst < TOL
+        errs = dict(h=relerr(hg[t + 1], one["h"][1]), c=relerr(cg[t + 1], one["c"][1]))
+        errs.update({k: relerr(a[t], one[k][0]) for k, a in sv.items()})
+        worst = {k: max(worst.get(k, 0.0), e) for k, e in errs.items()}
+    assert max(worst.values()) < TOL, worst
     # (3) backward on the saved activations
     saved = dict(h=hg, c=cg, v=host(act_Wx_norm), act_Wx=host(act_Wx), act_Rh=host(act_Rh),
                  act_c_norm=host(act_c_norm), cache1=host(cache1).reshape(T, N, 2),
