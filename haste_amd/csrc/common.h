@@ -101,6 +101,12 @@ int device_cu_count();
 int device_xcd_count();
 unsigned long long device_xcc_logical_map();
 
+// The look at the device's XCD placement allocates, synchronizes the device and launches on the
+// null stream: it cannot run while `stream` is being captured into a graph.  HASTE_HIP_OK when
+// the device has been looked at (or can be now); HASTE_HIP_ERROR_RUNTIME, with the reason in
+// haste_hip_last_runtime_error(), when it has not and `stream` is capturing.
+int xcd_layout_ready(hipStream_t stream);
+
 // Keeps the persistent kernels of this process on one device in a single order even when
 // they are launched on different streams.  before == true: makes `stream` wait for the
 // previous persistent kernel (if it ran on another stream); before == false: records the
@@ -120,38 +126,21 @@ class PersistentLaunchOrder {
 };
 
 // Polls before a bounded wait of a persistent kernel gives up: 2^24 (seconds), or the value of
-// the environment variable HASTE_HIP_SPIN_LIMIT.
+// the environment variable HASTE_HIP_SPIN_LIMIT (at least 2^16, a few milliseconds: less only
+// together with HASTE_HIP_TEST_HOOKS=1).
 unsigned int spin_limit();
 
 // Number of workgroups every group barrier also waits for although no workgroup plays them: 0,
-// or the value of the environment variable HASTE_HIP_TEST_ABSENT_WORKGROUP.  Only the test of
-// the time-out path sets it, together with a small spin limit: the waits then run out, the
-// kernel reports it and every wavefront still reaches the end of the kernel.
+// or -- only when the environment also has HASTE_HIP_TEST_HOOKS=1 -- the value of
+// HASTE_HIP_TEST_ABSENT_WORKGROUP.  Only the test of the time-out path sets them, together with
+// a small spin limit: the waits then run out, the kernel reports it and every wavefront still
+// reaches the end of the kernel.
 int test_absent_workgroups();
-
-// False when the environment variable HASTE_HIP_PAIRED_SETS is set to 0: 8- and 16-row
-// batch tiles then run as one tile instead of two sets of half the rows (for experiments).
-bool paired_sets_enabled();
-
-// False when the environment variable HASTE_HIP_SINGLE_ROW is set to 0: an LSTM or GRU forward
-// pass with one batch row then runs as a 4-row tile instead of the kernel that keeps the
-// recurrent weights in registers (for experiments).
-bool single_row_enabled();
 
 // False when the environment variable HASTE_HIP_FUSED_INPUT is set to 0: the forward
 // recurrences then read x * W from a GEMM launched before them instead of computing it beside
 // their waits (for experiments).
 bool fused_input_enabled();
-
-// False when the environment variable HASTE_HIP_RESIDENT_ROWS is set to 0: a backward
-// recurrence whose slice of the recurrent weights exceeds LDS then runs step by step instead
-// of keeping part of the slice in registers (for experiments).
-bool resident_rows_enabled();
-
-// False when the environment variable HASTE_HIP_SCATTER_BACKWARD is set to 0: the backward
-// recurrences of 4-row tiles then exchange the gate gradients (every workgroup gathers all of
-// them) instead of partial sums of dh (for experiments).
-bool scatter_backward_enabled();
 
 // C[M,N] = op(A)*B (+C): fp32 MFMA GEMM on `stream`.  The partial tiles of a split product
 // are kept `scratch_offset` bytes (a multiple of 16) into the stream's scratch buffer.

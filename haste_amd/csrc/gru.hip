@@ -769,10 +769,10 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
   if (T == 1 && single_step_applies(N, C, H))
     return gru_forward_single_step(stream, training, N, C, H, W, R, bx, br, x, h, h_out, v,
                                    zoneout_prob, zoneout_mask, dc_mask, dc_scale);
-  if (N == 1 && H <= 512 && xcd_local_fits((H + 15) / 16, 1) && single_row_enabled())
+  if (N == 1 && H <= 512 && xcd_local_fits((H + 15) / 16, 1))
     return gru_forward_single_row(stream, training, T, C, H, W, R, bx, br, x, h, h_out, v, tmp_Wx,
                                   zoneout_prob, zoneout_mask, dc_mask, dc_scale);
-  const ForwardTile tile = pick_forward_tile(3, N, H, 0, kWorkgroupLdsBytes, false, resident_rows_enabled() ? 3 : 0);
+  const ForwardTile tile = pick_forward_tile(3, N, H, 0, kWorkgroupLdsBytes, false, 3);
   // No slice of R fits a CU: stream R from HBM every step instead.
   if (!tile.ok)
     return gru_forward_streamed(stream, training, T, N, C, H, W, R, bx, br, x, h, h_out, v, tmp_Wx,
@@ -782,7 +782,7 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
   // An 8-row tile is run as two sets of 4 rows when the partial tiles of both fit beside the
   // slice (exchange tiles: one per set, together as large as the tile's).
   const size_t paired_lds = paired_lds_bytes((H + 63) / 64 * 64, tile.ct);
-  const bool paired = tile.nb == 8 && paired_lds <= kWorkgroupLdsBytes && paired_sets_enabled() &&
+  const bool paired = tile.nb == 8 && paired_lds <= kWorkgroupLdsBytes &&
                       tile.reg_groups == 0;
 
   // Taken after the GEMM, which may replace the stream's scratch buffer with a larger one.
@@ -839,7 +839,7 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && v && dh_next);
   HASTE_HIP_REQUIRE(dx && dW && dR && dbx && dbr && dh && dp && dq);
   // per row: the partial tiles or the 6 bias-gradient columns of 16 floats
-  const BackwardTile tile = pick_backward_tile(gru_backward_k(H), N, H, 6 * 16, 0, resident_rows_enabled());
+  const BackwardTile tile = pick_backward_tile(gru_backward_k(H), N, H, 6 * 16, 0, true);
   if (!tile.ok)
     return gru_backward_streamed(stream, T, N, C, H, W_t, R_t, x_t, h, v, dh_next, dx, dW, dR, dbx,
                                  dbr, dh, dp, dq, zoneout_mask);
@@ -850,10 +850,10 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   // dh go to their owners instead of the gate gradients to everybody.
   // (Measured over H = 64 ... 512, T = 100: with two sets per workgroup it is 5-15 % faster
   // at every H, with one set from H = 384 on; below, one set is 5-20 % faster the other way.)
-  const bool scatter = scatter_backward_enabled() && tile.reg_groups == 0 && H <= 512 &&
+  const bool scatter = tile.reg_groups == 0 && H <= 512 &&
                        (tile.nb == 8 || (tile.nb == 4 && H > 320));
   const bool paired = scatter ? tile.nb == 8
-                              : tile.nb == 8 && paired_lds <= kMaxLdsBytes && paired_sets_enabled();
+                              : tile.nb == 8 && paired_lds <= kMaxLdsBytes;
   const int sets = paired ? 2 : 1;
 
   Workspace ws;

@@ -664,7 +664,7 @@ int haste_hip_layer_norm_gru_forward_f32(int training, int steps, int batch_size
   HASTE_HIP_REQUIRE(!training || v != nullptr);
   hipStream_t stream = as_stream(stream_);
   const ForwardTile tile = pick_forward_tile(3, N, H, 2 * sizeof(float), kMaxLdsBytes, true,
-                                             resident_rows_enabled() ? 3 : 0);
+                                             3);
   if (!tile.ok)
     return layer_norm_gru_forward_streamed(stream, training, T, N, C, H, W, R, bx, br, x, h, v, act_Wx,
                                            gamma1, cache1, tmp_Wx_norm, act_Rh, gamma2, cache2,
@@ -734,7 +734,7 @@ int haste_hip_layer_norm_gru_backward_f32(int steps, int batch_size, int input_s
   HASTE_HIP_REQUIRE(dp && dq && act_Wx && gamma1 && dgamma1 && act_Rh && gamma2 && dgamma2 && cache2);
   hipStream_t stream = as_stream(stream_);
   // per row: 9 column-sum accumulators of 16 floats (or the partial tiles, whichever is more) + 4 sums
-  const BackwardTile tile = pick_backward_tile(ln_gru_backward_k(H), N, H, 9 * 16, 4, resident_rows_enabled());
+  const BackwardTile tile = pick_backward_tile(ln_gru_backward_k(H), N, H, 9 * 16, 4, true);
   if (!tile.ok)
     return layer_norm_gru_backward_streamed(stream, T, N, C, H, W_t, R_t, x_t, h, v, dh_new, dx, dW, dR,
                                             dbx, dbr, dh, dp, dq, act_Wx, gamma1, dgamma1, act_Rh,

@@ -847,7 +847,7 @@ int haste_hip_layer_norm_lstm_forward_f32(int training, int steps, int batch_siz
   HASTE_HIP_REQUIRE(gamma2 && gamma_h && beta_h && act_c_norm);
   hipStream_t stream = as_stream(stream_);
   const ForwardTile tile = pick_forward_tile(4, N, H, 4 * sizeof(float), kMaxLdsBytes, true,
-                                             resident_rows_enabled() ? 2 : 0);
+                                             2);
   if (!tile.ok)
     return layer_norm_lstm_forward_streamed(stream, training, T, N, C, H, W, R, b, x, h, c, act_Wx,
                                             gamma1, cache1, act_Wx_norm, act_Rh, gamma2, cache2,
@@ -941,7 +941,7 @@ int haste_hip_layer_norm_lstm_backward_f32(int steps, int batch_size, int input_
   HASTE_HIP_REQUIRE(dgamma_h && dbeta_h && cache3 && act_c_norm);
   hipStream_t stream = as_stream(stream_);
   // per row: 10 column-sum accumulators of 16 floats (or the partial tiles, whichever is more) + 10 sums
-  const BackwardTile tile = pick_backward_tile(4 * H, N, H, 10 * 16, 10, resident_rows_enabled());
+  const BackwardTile tile = pick_backward_tile(4 * H, N, H, 10 * 16, 10, true);
   if (!tile.ok)
     return layer_norm_lstm_backward_streamed(stream, T, N, C, H, W_t, R_t, x_t, h, c, dh_new, dc_new,
                                              dx, dW, dR, db, dh, dc, act_Wx, gamma1, dgamma1,

@@ -822,10 +822,10 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
   if (T == 1 && single_step_applies(N, C, H))
     return lstm_forward_single_step(stream, training, N, C, H, W, R, b, x, h, c, h_out, c_out, v,
                                     zoneout_prob, zoneout_mask, dc_mask, dc_scale);
-  if (N == 1 && H <= 512 && xcd_local_fits((H + 15) / 16, 1) && single_row_enabled())
+  if (N == 1 && H <= 512 && xcd_local_fits((H + 15) / 16, 1))
     return lstm_forward_single_row(stream, training, T, C, H, W, R, b, x, h, c, h_out, c_out, v,
                                    zoneout_prob, zoneout_mask, dc_mask, dc_scale);
-  const ForwardTile tile = pick_forward_tile(4, N, H, 0, kWorkgroupLdsBytes, false, resident_rows_enabled() ? 2 : 0);
+  const ForwardTile tile = pick_forward_tile(4, N, H, 0, kWorkgroupLdsBytes, false, 2);
   // No slice of R fits a CU: stream R from HBM every step instead.
   if (!tile.ok)
     return lstm_forward_streamed(stream, training, T, N, C, H, W, R, b, x, h, c, h_out, c_out, v,
@@ -834,7 +834,7 @@ int lstm_forward_impl(hipStream_t stream, int training, int T, int N, int C, int
   // slice (exchange tiles: one per set, together as large as the tile's).  Measured at
   // H = 512: 6 % faster per step; two sets of 8 rows instead of a 16-row tile: 6 % slower.
   const size_t paired_lds = paired_lds_bytes((H + 63) / 64 * 64, tile.ct);
-  const bool paired = tile.nb == 8 && paired_lds <= kWorkgroupLdsBytes && paired_sets_enabled() &&
+  const bool paired = tile.nb == 8 && paired_lds <= kWorkgroupLdsBytes &&
                       tile.reg_groups == 0;
 
   // With 4-row tiles the recurrence computes x * W itself, beside its waits (every wavefront of
@@ -914,7 +914,7 @@ int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
   HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && c && c_next && dh_next && dc_next);
   HASTE_HIP_REQUIRE(dx && dW && dR && db && dh && dc && v);
-  const BackwardTile tile = pick_backward_tile(4 * H, N, H, 4 * 16, 0, resident_rows_enabled());
+  const BackwardTile tile = pick_backward_tile(4 * H, N, H, 4 * 16, 0, true);
   if (!tile.ok)
     return lstm_backward_streamed(stream, T, N, C, H, W_t, R_t, x_t, h, c, c_next, dh_next, dc_next,
                                   dx, dW, dR, db, dh, dc, v, zoneout_mask);
@@ -926,10 +926,10 @@ int lstm_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   // dh go to their owners instead of the gate gradients to everybody.
   // (Measured over H = 64 ... 512, T = 100: with two sets per workgroup it is 5-15 % faster
   // at every H, with one set from H = 384 on; below, one set is 5-20 % faster the other way.)
-  const bool scatter = scatter_backward_enabled() && tile.reg_groups == 0 && H <= 512 &&
+  const bool scatter = tile.reg_groups == 0 && H <= 512 &&
                        (tile.nb == 8 || (tile.nb == 4 && H > 320));
   const bool paired = scatter ? tile.nb == 8
-                              : tile.nb == 8 && paired_lds <= kMaxLdsBytes && paired_sets_enabled();
+                              : tile.nb == 8 && paired_lds <= kMaxLdsBytes;
   const int sets = paired ? 2 : 1;
   const int ctn = H <= 256 ? 1 : 2;  // column tiles of 64 per wavefront
 

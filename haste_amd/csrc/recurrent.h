@@ -1501,6 +1501,7 @@ inline int plan_launch(hipStream_t stream, const Workspace& ws, int gx, int gy, 
   plan->shape.per_xcd = 0;
   plan->shape.xcc_map = 0;
   HASTE_HIP_PROPAGATE(reserve_epochs(stream, epochs, &plan->shape.epoch));
+  HASTE_HIP_PROPAGATE(xcd_layout_ready(stream));
   const int cus = device_cu_count(), xcds = device_xcd_count();
   if (xcds > 0 && cus % xcds == 0 && gy <= xcds && gx <= cus / xcds) {
     plan->shape.xcd_local = 1;
@@ -1688,7 +1689,7 @@ inline BackwardTile pick_backward_tile(int K, int N, int H, size_t reduce_floats
       if (lds > kMaxLdsBytes && resident_rows && nb >= 16 && other < kMaxLdsBytes) {
         const int fit = (int)((kMaxLdsBytes - other) / group_bytes);
         reg_groups = (groups - fit + 7) / 8 * 8;
-        if (reg_groups > kMaxResidentGroups || reg_groups > groups) continue;
+        if (reg_groups > kMaxResidentGroups || reg_groups >= groups) continue;  // some of the slice stays in LDS
         lds = (size_t)(groups - reg_groups) * group_bytes + other;
       }
       if (lds > kMaxLdsBytes || gy > kMaxGroups || gx * gy > kMaxWorkgroups) continue;

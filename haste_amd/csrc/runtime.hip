@@ -185,12 +185,34 @@ XcdLayout& xcd_layout_locked(int dev) {
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0) {
       // A kernel of another process may hold CUs for a moment: up to three looks.
       for (int attempt = 0; attempt < 3 && x.count == 0; ++attempt) (void)probe_xcd_layout(cus, &x);
+      if (x.count == 0)
+        set_error_text("the look at the device's XCD placement failed (CUs held by other work, a partition "
+                       "mode or a CU mask): the persistent kernels use the placement-independent path");
     }
   }
   return x;
 }
 
 }  // namespace
+
+int xcd_layout_ready(hipStream_t stream) {
+  int dev = 0;
+  HASTE_HIP_TRY(hipGetDevice(&dev));
+  {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    auto it = g_xcd_layout.find(dev);
+    if (it != g_xcd_layout.end() && it->second.probed) return HASTE_HIP_OK;
+  }
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capture) != hipSuccess) (void)hipGetLastError();
+  if (capture != hipStreamCaptureStatusNone) {
+    set_error_text("the first persistent launch on a device looks at its XCD placement (allocation, device "
+                   "synchronization): call haste_hip_set_workspace or any entry point once before capturing");
+    return HASTE_HIP_ERROR_RUNTIME;
+  }
+  (void)device_xcd_count();
+  return HASTE_HIP_OK;
+}
 
 int device_xcd_count() {
   int dev = 0;
@@ -206,17 +228,31 @@ unsigned long long device_xcc_logical_map() {
   return xcd_layout_locked(dev).map;
 }
 
+namespace {
+bool test_hooks_requested() {
+  static const bool on = [] {
+    const char* v = std::getenv("HASTE_HIP_TEST_HOOKS");
+    return v != nullptr && v[0] == '1';
+  }();
+  return on;
+}
+}  // namespace
+
 unsigned int spin_limit() {
   static const unsigned int limit = [] {
     const char* v = std::getenv("HASTE_HIP_SPIN_LIMIT");
     const unsigned long n = v != nullptr ? std::strtoul(v, nullptr, 10) : 0ul;
-    return n > 0 && n < (1ul << 31) ? (unsigned int)n : 1u << 24;
+    if (n == 0 || n >= (1ul << 31)) return 1u << 24;
+    // an inherited variable must not make healthy launches give up: a floor of milliseconds
+    const unsigned long floor = test_hooks_requested() ? 1ul : 1ul << 16;
+    return (unsigned int)(n < floor ? floor : n);
   }();
   return limit;
 }
 
 int test_absent_workgroups() {
   static const int absent = [] {
+    if (!test_hooks_requested()) return 0;
     const char* v = std::getenv("HASTE_HIP_TEST_ABSENT_WORKGROUP");
     const long n = v != nullptr ? std::strtol(v, nullptr, 10) : 0l;
     return n > 0 && n <= 4 ? (int)n : 0;
@@ -224,41 +260,9 @@ int test_absent_workgroups() {
   return absent;
 }
 
-bool paired_sets_enabled() {
-  static const bool enabled = [] {
-    const char* v = std::getenv("HASTE_HIP_PAIRED_SETS");
-    return v == nullptr || v[0] != '0';
-  }();
-  return enabled;
-}
-
-bool single_row_enabled() {
-  static const bool enabled = [] {
-    const char* v = std::getenv("HASTE_HIP_SINGLE_ROW");
-    return v == nullptr || v[0] != '0';
-  }();
-  return enabled;
-}
-
 bool fused_input_enabled() {
   static const bool enabled = [] {
     const char* v = std::getenv("HASTE_HIP_FUSED_INPUT");
-    return v == nullptr || v[0] != '0';
-  }();
-  return enabled;
-}
-
-bool resident_rows_enabled() {
-  static const bool enabled = [] {
-    const char* v = std::getenv("HASTE_HIP_RESIDENT_ROWS");
-    return v == nullptr || v[0] != '0';
-  }();
-  return enabled;
-}
-
-bool scatter_backward_enabled() {
-  static const bool enabled = [] {
-    const char* v = std::getenv("HASTE_HIP_SCATTER_BACKWARD");
     return v == nullptr || v[0] != '0';
   }();
   return enabled;
@@ -352,6 +356,16 @@ int get_workspace(hipStream_t stream, size_t scratch_bytes, Workspace* out) {
   std::lock_guard<std::mutex> lock(g_mutex);
   Workspace& ws = g_workspaces[Key{dev, stream}];
   if (ws.control == nullptr) HASTE_HIP_PROPAGATE(create_control(stream, ws));
+  // A persistent kernel launched earlier on this stream gave up: whichever entry point comes
+  // next says so, once, instead of working on what that launch left behind.
+  if (ws.host_status != nullptr) {
+    volatile unsigned int* status = ws.host_status;
+    const unsigned int seen = *status;
+    if (seen != 0u) {
+      *status = 0u;
+      return recover_from_abort_locked(dev, stream, ws, seen);
+    }
+  }
   if (ws.scratch_bytes < scratch_bytes) {
     if (ws.caller_owned) {
       char buf[200];
@@ -476,10 +490,9 @@ int haste_hip_max_hidden_size(int gates, int batch_size) {
   auto fits = [&](int H) {
     const int k_back = gates == 3 ? 48 * ((H + 15) / 16) : gates * H;
     const size_t reduce_floats = gates == 3 ? 6 * 16 : (size_t)gates * 16;
-    const int max_ct = !haste_hip::resident_rows_enabled() ? 0 : (gates == 3 ? 3 : (gates == 4 ? 2 : 0));
+    const int max_ct = gates == 3 ? 3 : (gates == 4 ? 2 : 0);
     return haste_hip::pick_forward_tile(gates, batch_size, H, 0, haste_hip::kWorkgroupLdsBytes, false, max_ct).ok &&
-           haste_hip::pick_backward_tile(k_back, batch_size, H, reduce_floats, 0,
-                                         haste_hip::resident_rows_enabled()).ok;
+           haste_hip::pick_backward_tile(k_back, batch_size, H, reduce_floats, 0, true).ok;
   };
   int best = 0;
   for (int H = 16; H <= 8192; H += 16)
@@ -510,6 +523,9 @@ int haste_hip_set_workspace(void* stream_, void* memory, size_t bytes) {
     HASTE_HIP_REQUIRE((reinterpret_cast<uintptr_t>(memory) & 255u) == 0);
     HASTE_HIP_REQUIRE(bytes >= kControlBytes + 4096);
   }
+  // The look at the XCD placement (once per device) happens here rather than inside the first
+  // persistent launch, which may be recorded into a graph.
+  (void)device_xcd_count();
   std::lock_guard<std::mutex> lock(g_mutex);
   Workspace& ws = g_workspaces[Key{dev, stream}];
   // Work enqueued earlier may still use what is replaced.

@@ -174,7 +174,7 @@ def child_timeout():
 
 
 def test_a_wait_that_runs_out_is_reported_by_stream_status():
-    env = dict(os.environ, HASTE_HIP_SPIN_LIMIT="512", HASTE_HIP_TEST_ABSENT_WORKGROUP="1",
+    env = dict(os.environ, HASTE_HIP_TEST_HOOKS="1", HASTE_HIP_SPIN_LIMIT="512", HASTE_HIP_TEST_ABSENT_WORKGROUP="1",
                PYTHONPATH=os.pathsep.join([ROOT, os.path.join(ROOT, "tests")]))
     res = subprocess.run([sys.executable, os.path.abspath(__file__), "timeout"], env=env,
                          capture_output=True, text=True, timeout=110)

@@ -55,3 +55,42 @@ def test_no_alloc_layer_norm_backward_rejects_sizes_beyond_its_array():
         hlib.call("haste_hip_layer_norm_backward_noalloc_f32", 8, 5000, g, x, x, x.clone(), g.clone(),
                   None, None)
     assert e.value.code == 2 and "4096" in str(e.value)
+
+
+def test_no_alloc_layer_norm_backward_in_a_graph():
+    """What the entry point is for: two calls of different sizes recorded into a HIP graph on a
+    side stream (after one eager call, which looks up the array's address) and replayed twice,
+    with eager work between the replays; every replay gives the eager results' bits."""
+    import torch
+    from haste_amd import lib as hlib
+    name = "haste_hip_layer_norm_backward_noalloc_f32"
+    cases = [[dev(a) for a in _case(rows, D, 200 + i)] for i, (rows, D) in enumerate([(4000, 512), (333, 260)])]
+    eager = [_run(name, *args) for args in cases]
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    outs = []
+    with torch.cuda.stream(s):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s):
+            for x, gamma, dy, dg0, db0 in cases:
+                rows, D = x.shape
+                dx, dgamma, dbeta = torch.empty_like(x), torch.empty_like(dg0), torch.empty_like(db0)
+                dgamma.copy_(dg0)
+                dbeta.copy_(db0)
+                hlib.call(name, rows, D, gamma, x, dy, dx, dgamma, dbeta, None, stream=s.cuda_stream)
+                outs.append((dx, dgamma, dbeta))
+        for replay in range(2):
+            print("no_alloc replay", replay, flush=True)
+            for o in outs:
+                o[0].fill_(float("nan"))
+            s.synchronize()
+            between = _run(name, *cases[1])  # eager, on the current (side) stream
+            s.synchronize()
+            graph.replay()
+            s.synchronize()
+            for got, want in zip(outs, eager):
+                for g, w in zip(got, want):
+                    assert torch.equal(g, w), replay
+            for g, w in zip(between, eager[1]):
+                assert torch.equal(g, w)
+        del graph
