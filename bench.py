@@ -17,6 +17,8 @@ import sys
 import numpy as np
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_FP64_MFMA_TFLOPS = 78.6
+PEAK_FP16_MFMA_TFLOPS = 2500.0
 PEAK_HBM_GBS = 8000.0
 
 # HBM bytes per launch at the metric workload, from two rocprofv3 --pmc runs (FETCH_SIZE, then
@@ -24,6 +26,7 @@ PEAK_HBM_GBS = 8000.0
 # one FETCH_SIZE unit = 2.000 KiB, one WRITE_SIZE unit = 1.000 KiB.  A GEMM "launch" is the mean
 # of the step's three products (dx; dW and dR, which share a launch that counts as two), each with
 # its split reduce; the forward recurrence includes the input projection it computes itself.
+TRAFFIC_SOURCE = "profiles/lstm_fwd_bwd_N64_T100_H512_hbm_traffic_pmc.txt (a constant from that profile, not measured in this run)"
 MEASURED_TRAFFIC_BYTES = {"gemm_f32": 143.2e6, "lstm_forward_recurrence": 161.3e6,
                           "lstm_backward_recurrence": 183.1e6,
                           # at N=1 C=512 H=4096 (--workload stepwise): 131558.5 FETCH_SIZE units
@@ -177,6 +180,7 @@ def run_metric(args, torch, lib, ops, dev):
                 "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(dom["tflops"] / PEAK_FP32_MFMA_TFLOPS, 4),
                 "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
+                "traffic_source": TRAFFIC_SOURCE,
                 "us_per_launch": round(dom["avg_ms"] * 1e3, 2),
                 "whole_step_tflops": round(tflops_whole, 3),
                 "whole_step_frac": round(tflops_whole / PEAK_FP32_MFMA_TFLOPS, 4)}
@@ -423,12 +427,52 @@ def run_hbm_kernels(args, torch, lib, ops, dev):
 
     t = timed(("transpose_f32",), lambda: ops.transpose(xs))
     out["transpose_6400x512"] = entry(t["transpose_f32"], 4.0 * 2 * T * N * C)
+    del xs, x_t, dh_new
+
+    # The reference's IndRNN speed script (validation/pytorch_speed.py:7-20): T=2500, N=64,
+    # C=256, H=4096, where the recurrences move 5 / 8 GB and are bound by HBM.
+    T, N, C, H = 2500, 64, 256, 4096
+    xs = torch.randn(T, N, C, device=dev)
+    W = (torch.rand(C, H, device=dev) - 0.5) * H ** -0.5
+    u = torch.rand(H, device=dev) - 0.5
+    b = torch.zeros(H, device=dev)
+    h0 = torch.zeros(N, H, device=dev)
+    dh_new = torch.randn(T + 1, N, H, device=dev)
+    x_t, W_t = ops.transpose(xs), ops.transpose(W)
+    total = {}
+
+    def ind_speed():
+        e = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+        e[0].record()
+        h = ops.indrnn_forward(True, 0.0, xs, h0, W, u, b, no_mask)
+        e[1].record()
+        ops.indrnn_backward(x_t, W_t, u, b, no_mask, h, dh_new)
+        e[2].record()
+        torch.cuda.synchronize()
+        total["fwd"], total["bwd"] = e[0].elapsed_time(e[1]), e[1].elapsed_time(e[2])
+    t = timed(("indrnn_forward_recurrence", "indrnn_backward_recurrence"), ind_speed, reps=3)
+    out["indrnn_forward_N64_T2500_C256_H4096"] = entry(t["indrnn_forward_recurrence"], 4.0 * 2 * T * N * H)
+    out["indrnn_backward_N64_T2500_C256_H4096"] = entry(t["indrnn_backward_recurrence"], 4.0 * 3 * T * N * H)
+    out["indrnn_speed_script_shape"] = {"forward_pass_ms": round(total["fwd"], 3), "backward_pass_ms": round(total["bwd"], 3),
+                                        "note": "whole passes (x*W, recurrence; recurrence, dW, dx) at the shape of "
+                                                "the reference's validation/pytorch_speed.py"}
     return out
 
 
 def run_configs(args, torch, lib, ops, dev):
     """The other BASELINE.json configurations (parity-test cases; timed here for the record):
-    forward (+ backward with the caller-side transposes) in ms per call."""
+    forward (+ backward with the caller-side transposes) in ms per call, with the algorithmic
+    flops of the matrix products (2*T*N*G*H*(C + H) forward, three times that forward +
+    backward) and the fraction of the matrix cores' peak for the arithmetic type.  Also the
+    coverage-only instantiations of the reference at the metric shape: the double LSTM and the
+    half GRU (step-wise regime: one GEMM and one pointwise launch per step)."""
+    details = {}
+
+    def note(key, ms, flops, peak=PEAK_FP32_MFMA_TFLOPS, dtype="f32"):
+        tf = flops / (ms * 1e-3) / 1e12
+        details[key] = {"ms": ms, "flops": flops, "tflops": round(tf, 3), "dtype": dtype,
+                        "peak_tflops": peak, "frac_of_mfma_peak": round(tf / peak, 4)}
+
     def timed(fn, reps):
         for _ in range(3):
             fn()
@@ -457,6 +501,8 @@ def run_configs(args, torch, lib, ops, dev):
     z = torch.zeros(N, H, device=dev)
     out["lstm_inference_N16_T100_C128_H256_ms"] = timed(
         lambda: ops.lstm_forward(False, 0.0, x, z, z, W, R, b, no_mask), 50)
+    note("lstm_inference_N16_T100_C128_H256", out["lstm_inference_N16_T100_C128_H256_ms"],
+         2.0 * T * N * 4 * H * (C + H))
 
     T, N, C, H = 100, 64, 512, 512  # config 2: GRU training, zoneout 0.1, DropConnect 0.05
     k = H ** -0.5
@@ -471,6 +517,18 @@ def run_configs(args, torch, lib, ops, dev):
         Reff_t = ops.transpose(R * dm * (1.0 / 0.95))
         return ops.gru_backward(ops.transpose(x), ops.transpose(W), Reff_t, bx, br, zm, h, cache, dh_new)
     out["gru_fwd_bwd_N64_T100_H512_zoneout_dropconnect_ms"] = timed(gru_step, 30)
+    note("gru_fwd_bwd_N64_T100_H512_zoneout_dropconnect", out["gru_fwd_bwd_N64_T100_H512_zoneout_dropconnect_ms"],
+         3 * 2.0 * T * N * 3 * H * (C + H))
+
+    # the half GRU of the reference (lib/gru_forward_gpu.cu.cc:373) at the same shape
+    xh, Wh, Rh, bxh, brh, zh, zmh, dhh = (a.half() for a in (x, W, R, bx, br, z, zm, dh_new))
+
+    def gru_half_step():
+        h, cache = ops.gru_forward(True, 0.1, xh, zh, Wh, Rh, bxh, brh, zmh)
+        return ops.gru_backward(ops.transpose(xh), ops.transpose(Wh), ops.transpose(Rh), bxh, brh, zmh, h, cache, dhh)
+    ms = timed(gru_half_step, 5)
+    out["gru_f16_fwd_bwd_N64_T100_H512_zoneout_ms"] = ms
+    note("gru_f16_fwd_bwd_N64_T100_H512_zoneout", ms, 3 * 2.0 * T * N * 3 * H * (C + H), PEAK_FP16_MFMA_TFLOPS, "f16")
 
     T, N, C, H = 100, 128, 512, 512  # config 3: LSTM training, N=128
     x, W, R = rnd(T, N, C), uni(k, C, 4 * H), uni(k, H, 4 * H)
@@ -484,6 +542,20 @@ def run_configs(args, torch, lib, ops, dev):
         return ops.lstm_backward(*ops.transpose3(x, W, R), b, no_mask, h, c,
                                  cache, dh_new, dc_new)
     out["lstm_fwd_bwd_N128_T100_H512_ms"] = timed(lstm_step, 30)
+    note("lstm_fwd_bwd_N128_T100_H512", out["lstm_fwd_bwd_N128_T100_H512_ms"], 3 * 2.0 * T * N * 4 * H * (C + H))
+
+    # the double LSTM of the reference (lib/lstm_forward_gpu.cu.cc:368-369) at the metric shape
+    Nd = 64
+    xd_, Wd_, Rd_, bd_, zd_ = x[:, :Nd].double().contiguous(), W.double(), R.double(), b.double(), z[:Nd].double()
+    dhd_, dcd_ = dh_new[:, :Nd].double().contiguous(), dc_new[:, :Nd].double().contiguous()
+    no_mask64 = torch.empty(0, 0, 0, device=dev, dtype=torch.float64)
+
+    def lstm_double_step():
+        h, c, cache = ops.lstm_forward(True, 0.0, xd_, zd_, zd_, Wd_, Rd_, bd_, no_mask64)
+        return ops.lstm_backward(*ops.transpose3(xd_, Wd_, Rd_), bd_, no_mask64, h, c, cache, dhd_, dcd_)
+    ms = timed(lstm_double_step, 5)
+    out["lstm_f64_fwd_bwd_N64_T100_H512_ms"] = ms
+    note("lstm_f64_fwd_bwd_N64_T100_H512", ms, 3 * 2.0 * T * Nd * 4 * H * (C + H), PEAK_FP64_MFMA_TFLOPS, "f64")
 
     T, N, C, H = 500, 32, 256, 256  # config 4: LayerNormLSTM training, zoneout 0.1
     k = H ** -0.5
@@ -500,7 +572,9 @@ def run_configs(args, torch, lib, ops, dev):
         return ops.layer_norm_lstm_backward(*ops.transpose3(x, W, R), b, gamma,
                                             gamma_h, beta_h, zm, *fwd, dh_new, dc_new)
     out["layer_norm_lstm_fwd_bwd_N32_T500_H256_zoneout_ms"] = timed(ln_lstm_step, 10)
-    return out
+    note("layer_norm_lstm_fwd_bwd_N32_T500_H256_zoneout", out["layer_norm_lstm_fwd_bwd_N32_T500_H256_zoneout_ms"],
+         3 * 2.0 * T * N * 4 * H * (C + H))
+    return out, details
 
 
 def main():
@@ -535,7 +609,8 @@ def main():
                           "kernels": m["kernels"]}))
         return
     if args.workload == "configs":
-        print(json.dumps(run_configs(args, torch, lib, ops, dev)))
+        configs, details = run_configs(args, torch, lib, ops, dev)
+        print(json.dumps({"other_configs_ms": configs, "other_configs": details}))
         return
     if args.workload == "streaming":
         s, _ = run_streaming(args, torch, lib, ops, dev)
@@ -558,7 +633,7 @@ def main():
     streaming, host1 = run_streaming(args, torch, lib, ops, dev)
     stepwise = run_stepwise(args, torch, lib, ops, dev)
     hbm_kernels = run_hbm_kernels(args, torch, lib, ops, dev)
-    configs = run_configs(args, torch, lib, ops, dev)
+    configs, config_details = run_configs(args, torch, lib, ops, dev)
     measured_peak = run_measured_peak(args, torch, lib, ops, dev)
     iterate = run_iterate(args, torch, lib, ops, dev)
     m["roofline"]["measured_peak"] = measured_peak["tflops"]
@@ -605,6 +680,7 @@ def main():
         "stepwise_n1_h4096": stepwise,
         "hbm_kernels": hbm_kernels,
         "other_configs_ms": configs,
+        "other_configs": config_details,
         "measured_fp32_mfma_peak": measured_peak,
         "iterate_n1": iterate,
         "cpu_baseline": cpu,

@@ -9,7 +9,9 @@ pytestmark = pytest.mark.gpu
 
 # T on both sides of the kernels' batches of 16 steps: no whole batch, whole batches only, a tail
 SHAPES = [(1, 1, 1, 1), (3, 2, 3, 4), (9, 3, 7, 5), (15, 2, 3, 6), (16, 3, 5, 70), (17, 5, 20, 70),
-          (30, 16, 32, 256), (32, 2, 4, 33), (33, 2, 4, 33), (50, 64, 64, 512)]
+          (30, 16, 32, 256), (32, 2, 4, 33), (33, 2, 4, 33), (50, 64, 64, 512),
+          # the width of the reference's IndRNN speed script (validation/pytorch_speed.py:7-20)
+          (20, 64, 256, 4096)]
 
 
 @pytest.mark.parametrize("layer_norm", [False, True])
