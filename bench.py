@@ -28,7 +28,7 @@ PEAK_HBM_GBS = 8000.0
 # its split reduce; the forward recurrence includes the input projection it computes itself.
 TRAFFIC_SOURCE = "profiles/lstm_fwd_bwd_N64_T100_H512_hbm_traffic_pmc.txt (a constant from that profile, not measured in this run)"
 MEASURED_TRAFFIC_BYTES = {"gemm_f32": 143.2e6, "lstm_forward_recurrence": 161.3e6,
-                          "lstm_backward_recurrence": 183.1e6,
+                          "lstm_backward_recurrence": 196.1e6,
                           # at N=1 C=512 H=4096 (--workload stepwise): 131558.5 FETCH_SIZE units
                           # + 192 WRITE_SIZE units per launch of the streaming kernel
                           "gemm_f32_skinny": 269.6e6}
