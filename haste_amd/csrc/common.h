@@ -77,6 +77,24 @@ struct Workspace {
 // it is too small.
 int get_workspace(hipStream_t stream, size_t scratch_bytes, Workspace* out);
 
+// While one of these is alive on a host thread, get_workspace() on that thread hands out the
+// scratch area behind the first `bytes` bytes (a multiple of 256) of the stream's scratch
+// buffer: an entry point that stages tensors of its own there and then calls other entry
+// points' implementations keeps its staging area out of their way.  The buffer must already
+// be large enough for the prefix and everything asked for behind it (ask get_workspace for
+// the sum first): growing replaces the buffer, which would lose what is staged, so with a
+// prefix in force get_workspace refuses to grow (HASTE_HIP_ERROR_UNSUPPORTED_SIZE).
+class ScratchPrefix {
+ public:
+  explicit ScratchPrefix(size_t bytes);
+  ~ScratchPrefix();
+  ScratchPrefix(const ScratchPrefix&) = delete;
+  ScratchPrefix& operator=(const ScratchPrefix&) = delete;
+
+ private:
+  size_t saved_;
+};
+
 // Reserves `count` consecutive step-flag values on the workspace of (current device,
 // stream) and returns the value before the first of them.
 int reserve_epochs(hipStream_t stream, unsigned int count, unsigned int* base);

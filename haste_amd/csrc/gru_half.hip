@@ -1,0 +1,221 @@
+// The half-precision GRU over more than one step (what gru::ForwardPass<__half>::Run and
+// BackwardPass<__half>::Run bind to; reference lib/gru_forward_gpu.cu.cc:373,
+// lib/gru_backward_gpu.cu.cc:411).
+//
+// Half is the caller's storage format here, not the arithmetic: the recurrence is bound by
+// the latency of its per-step exchange and by instruction issue, not by the rate of the matrix
+// units or by HBM, so the persistent fp32 kernels are also the fastest way to run half
+// tensors.  The tensors are widened into a staging area at the front of the stream's scratch
+// buffer (one launch), the fp32 passes run on the staged copies, and what the caller gets back
+// is rounded to half (one launch).  Between the steps the state stays in fp32: the results are
+// those of exact half inputs, rounded once, where the reference rounds every step.
+#include "common.h"
+
+extern "C" size_t haste_hip_workspace_bytes(int time_steps, int batch_size, int input_size, int hidden_size);
+
+namespace haste_hip {
+
+int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int H,
+                     const float* W, const float* R, const float* bx, const float* br,
+                     const float* x, const float* h, float* h_out, float* v, float* tmp_Wx,
+                     float zoneout_prob, const float* zoneout_mask, const float* dc_mask,
+                     float dc_scale);
+int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
+                      const float* W_t, const float* R_t, const float* x_t, const float* h,
+                      const float* v, const float* dh_next, float* dx, float* dW, float* dR,
+                      float* dbx, float* dbr, float* dh, float* dp, float* dq,
+                      const float* zoneout_mask);
+
+namespace {
+
+typedef _Float16 half_t;
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kMaxSegments = 12;
+
+// Tensors to convert in one launch: segment s is `count[s]` elements from src[s] to dst[s].
+struct ConvertList {
+  const void* src[kMaxSegments];
+  void* dst[kMaxSegments];
+  unsigned long long count[kMaxSegments];
+  int n = 0;
+  unsigned long long longest = 0;
+  void add(const void* s, void* d, size_t c) {
+    if (s == nullptr || d == nullptr || c == 0) return;
+    src[n] = s;
+    dst[n] = d;
+    count[n] = c;
+    if (c > longest) longest = c;
+    ++n;
+  }
+};
+
+// blockIdx.y: the segment; a thread converts runs of 8 elements (16-byte accesses on the half
+// side when that side is 16-byte aligned; the float side is the staging area, aligned).
+template <bool WIDEN>
+__global__ __launch_bounds__(256)
+void convert_kernel(ConvertList l) {
+  const int s = blockIdx.y;
+  const unsigned long long n = l.count[s];
+  const unsigned long long stride = (unsigned long long)gridDim.x * 256 * 8;
+  const half_t* hsrc = static_cast<const half_t*>(l.src[s]);
+  half_t* hdst = static_cast<half_t*>(l.dst[s]);
+  const float* fsrc = static_cast<const float*>(l.src[s]);
+  float* fdst = static_cast<float*>(l.dst[s]);
+  const bool aligned = ((WIDEN ? reinterpret_cast<uintptr_t>(hsrc) : reinterpret_cast<uintptr_t>(hdst)) & 15u) == 0;
+  for (unsigned long long i = ((unsigned long long)blockIdx.x * 256 + threadIdx.x) * 8; i < n; i += stride) {
+    if (aligned && i + 8 <= n) {
+      if constexpr (WIDEN) {
+        const half8_t a = *reinterpret_cast<const half8_t*>(hsrc + i);
+        float4_t lo, hi;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          lo[e] = (float)a[e];
+          hi[e] = (float)a[4 + e];
+        }
+        *reinterpret_cast<float4_t*>(fdst + i) = lo;
+        *reinterpret_cast<float4_t*>(fdst + i + 4) = hi;
+      } else {
+        const float4_t lo = *reinterpret_cast<const float4_t*>(fsrc + i);
+        const float4_t hi = *reinterpret_cast<const float4_t*>(fsrc + i + 4);
+        half8_t a;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          a[e] = (half_t)lo[e];
+          a[4 + e] = (half_t)hi[e];
+        }
+        *reinterpret_cast<half8_t*>(hdst + i) = a;
+      }
+    } else {
+      const unsigned long long end = i + 8 < n ? i + 8 : n;
+      for (unsigned long long j = i; j < end; ++j) {
+        if constexpr (WIDEN) fdst[j] = (float)hsrc[j];
+        else hdst[j] = (half_t)fsrc[j];
+      }
+    }
+  }
+}
+
+template <bool WIDEN>
+int convert(hipStream_t stream, const ConvertList& l) {
+  if (l.n == 0) return HASTE_HIP_OK;
+  unsigned long long blocks = (l.longest + 2047) / 2048;
+  if (blocks > 4096) blocks = 4096;
+  convert_kernel<WIDEN><<<dim3((unsigned)blocks, (unsigned)l.n), dim3(256), 0, stream>>>(l);
+  HASTE_HIP_TRY(hipGetLastError());
+  return HASTE_HIP_OK;
+}
+
+// Lays float tensors out one after the other, each on a 256-byte boundary.
+struct Staging {
+  size_t floats = 0;
+  size_t take(size_t n) {
+    const size_t at = floats;
+    floats += (n + 63) / 64 * 64;
+    return at;
+  }
+};
+
+// The staging area of `bytes` bytes plus room behind it for everything the fp32 passes ask for.
+int staged_workspace(hipStream_t stream, int T, int N, int C, int H, size_t bytes, float** base) {
+  Workspace ws;
+  HASTE_HIP_PROPAGATE(get_workspace(stream, bytes + haste_hip_workspace_bytes(T, N, C, H), &ws));
+  *base = ws.scratch;
+  return HASTE_HIP_OK;
+}
+
+}  // namespace
+
+// h: [(T+1),N,H], the first [N,H] the state before the first step.
+int gru_forward_half(hipStream_t stream, int training, int T, int N, int C, int H, const void* W,
+                     const void* R, const void* bx, const void* br, const void* x, void* h, void* v,
+                     float zoneout_prob, const void* zoneout_mask, const void* dc_mask,
+                     float dc_scale) {
+  const size_t NH = (size_t)N * H, TN = (size_t)T * N;
+  Staging st;
+  const size_t oW = st.take((size_t)C * 3 * H), oR = st.take((size_t)H * 3 * H);
+  const size_t obx = st.take(3 * (size_t)H), obr = st.take(3 * (size_t)H);
+  const size_t ox = st.take(TN * C), oh = st.take((T + 1) * NH);
+  const size_t ov = training ? st.take(TN * 4 * H) : 0;
+  const size_t oWx = st.take(TN * 3 * H);
+  const size_t om = zoneout_mask ? st.take(TN * H) : 0;
+  const size_t od = dc_mask ? st.take((size_t)H * 3 * H) : 0;
+  const size_t bytes = st.floats * sizeof(float);
+  float* f = nullptr;
+  HASTE_HIP_PROPAGATE(staged_workspace(stream, T, N, C, H, bytes, &f));
+
+  ConvertList in;
+  in.add(W, f + oW, (size_t)C * 3 * H);
+  in.add(R, f + oR, (size_t)H * 3 * H);
+  in.add(bx, f + obx, 3 * (size_t)H);
+  in.add(br, f + obr, 3 * (size_t)H);
+  in.add(x, f + ox, TN * C);
+  in.add(h, f + oh, NH);
+  if (zoneout_mask) in.add(zoneout_mask, f + om, TN * H);
+  if (dc_mask) in.add(dc_mask, f + od, (size_t)H * 3 * H);
+  HASTE_HIP_PROPAGATE(convert<true>(stream, in));
+  {
+    ScratchPrefix keep(bytes);
+    HASTE_HIP_PROPAGATE(gru_forward_impl(stream, training, T, N, C, H, f + oW, f + oR, f + obx, f + obr,
+                                         f + ox, f + oh, f + oh + NH, training ? f + ov : nullptr, f + oWx,
+                                         zoneout_prob, zoneout_mask ? f + om : nullptr,
+                                         dc_mask ? f + od : nullptr, dc_scale));
+  }
+  ConvertList out;
+  out.add(f + oh + NH, static_cast<half_t*>(h) + NH, TN * H);
+  if (training) out.add(f + ov, v, TN * 4 * H);
+  return convert<false>(stream, out);
+}
+
+// h: [(T+1),N,H]; dh_next: [T,N,H], the gradients w.r.t. the states after each step.  dW, dR,
+// dbx, dbr and dh are added to, as in the fp32 pass (widened, added to in fp32, rounded).
+int gru_backward_half(hipStream_t stream, int T, int N, int C, int H, const void* W_t,
+                      const void* R_t, const void* x_t, const void* h, const void* v,
+                      const void* dh_next, void* dx, void* dW, void* dR, void* dbx, void* dbr,
+                      void* dh, void* dp, void* dq, const void* zoneout_mask) {
+  const size_t NH = (size_t)N * H, TN = (size_t)T * N, H3 = 3 * (size_t)H;
+  Staging st;
+  const size_t oWt = st.take(H3 * C), oRt = st.take(H3 * H), oxt = st.take(TN * C);
+  const size_t oh = st.take((T + 1) * NH), ov = st.take(TN * 4 * H), odn = st.take(TN * H);
+  const size_t om = zoneout_mask ? st.take(TN * H) : 0;
+  const size_t odx = st.take(TN * C), odW = st.take(C * H3), odR = st.take(H * H3);
+  const size_t odbx = st.take(H3), odbr = st.take(H3), odh = st.take(NH);
+  const size_t odp = st.take(TN * H3), odq = st.take(TN * H3);
+  const size_t bytes = st.floats * sizeof(float);
+  float* f = nullptr;
+  HASTE_HIP_PROPAGATE(staged_workspace(stream, T, N, C, H, bytes, &f));
+
+  ConvertList in;
+  in.add(W_t, f + oWt, H3 * C);
+  in.add(R_t, f + oRt, H3 * H);
+  in.add(x_t, f + oxt, TN * C);
+  in.add(h, f + oh, (T + 1) * NH);
+  in.add(v, f + ov, TN * 4 * H);
+  in.add(dh_next, f + odn, TN * H);
+  if (zoneout_mask) in.add(zoneout_mask, f + om, TN * H);
+  in.add(dW, f + odW, C * H3);
+  in.add(dR, f + odR, H * H3);
+  in.add(dbx, f + odbx, H3);
+  in.add(dbr, f + odbr, H3);
+  in.add(dh, f + odh, NH);
+  HASTE_HIP_PROPAGATE(convert<true>(stream, in));
+  {
+    ScratchPrefix keep(bytes);
+    HASTE_HIP_PROPAGATE(gru_backward_impl(stream, T, N, C, H, f + oWt, f + oRt, f + oxt, f + oh, f + ov,
+                                          f + odn, f + odx, f + odW, f + odR, f + odbx, f + odbr, f + odh,
+                                          f + odp, f + odq, zoneout_mask ? f + om : nullptr));
+  }
+  ConvertList out;
+  out.add(f + odx, dx, TN * C);
+  out.add(f + odW, dW, C * H3);
+  out.add(f + odR, dR, H * H3);
+  out.add(f + odbx, dbx, H3);
+  out.add(f + odbr, dbr, H3);
+  out.add(f + odh, dh, NH);
+  out.add(f + odp, dp, TN * H3);
+  out.add(f + odq, dq, TN * H3);
+  return convert<false>(stream, out);
+}
+
+}  // namespace haste_hip

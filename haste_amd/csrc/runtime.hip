@@ -350,9 +350,18 @@ int recover_from_abort_locked(int dev, hipStream_t stream, Workspace& ws, unsign
 
 }  // namespace
 
+namespace {
+thread_local size_t t_scratch_prefix = 0;
+}  // namespace
+
+ScratchPrefix::ScratchPrefix(size_t bytes) : saved_(t_scratch_prefix) { t_scratch_prefix = saved_ + bytes; }
+ScratchPrefix::~ScratchPrefix() { t_scratch_prefix = saved_; }
+
 int get_workspace(hipStream_t stream, size_t scratch_bytes, Workspace* out) {
   int dev = 0;
   HASTE_HIP_TRY(hipGetDevice(&dev));
+  const size_t prefix = t_scratch_prefix;
+  scratch_bytes += prefix;
   std::lock_guard<std::mutex> lock(g_mutex);
   Workspace& ws = g_workspaces[Key{dev, stream}];
   if (ws.control == nullptr) HASTE_HIP_PROPAGATE(create_control(stream, ws));
@@ -375,6 +384,11 @@ int get_workspace(hipStream_t stream, size_t scratch_bytes, Workspace* out) {
       set_error_text(buf);
       return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
     }
+    if (prefix != 0) {
+      set_error_text("internal: the scratch buffer would have to grow while an entry point keeps staged "
+                     "tensors in it");
+      return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
+    }
     // Growing replaces the buffer; work already enqueued on the stream may still be
     // using the old one, so the stream is drained first (rare: sizes stabilise
     // after the first call of each shape).
@@ -390,6 +404,8 @@ int get_workspace(hipStream_t stream, size_t scratch_bytes, Workspace* out) {
   }
   if (ws.scratch_high_water < scratch_bytes) ws.scratch_high_water = scratch_bytes;
   *out = ws;
+  out->scratch = reinterpret_cast<float*>(reinterpret_cast<char*>(ws.scratch) + prefix);
+  out->scratch_bytes = ws.scratch_bytes - prefix;
   return HASTE_HIP_OK;
 }
 

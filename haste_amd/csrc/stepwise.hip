@@ -28,6 +28,15 @@ int gemm_f64(hipStream_t stream, bool trans_a, int M, int N, int K, const double
              const double* B, int ldb, double* C, int ldc, bool accumulate);
 int gemm_f16(hipStream_t stream, bool trans_a, int M, int N, int K, const void* A, int lda,
              const void* B, int ldb, void* C, int ldc, bool accumulate);
+// gru_half.hip: the half GRU over more than one step, on the fp32 kernels.
+int gru_forward_half(hipStream_t stream, int training, int T, int N, int C, int H, const void* W,
+                     const void* R, const void* bx, const void* br, const void* x, void* h, void* v,
+                     float zoneout_prob, const void* zoneout_mask, const void* dc_mask,
+                     float dc_scale);
+int gru_backward_half(hipStream_t stream, int T, int N, int C, int H, const void* W_t,
+                      const void* R_t, const void* x_t, const void* h, const void* v,
+                      const void* dh_next, void* dx, void* dW, void* dR, void* dbx, void* dbr,
+                      void* dh, void* dp, void* dq, const void* zoneout_mask);
 
 namespace {
 
@@ -1476,7 +1485,9 @@ int haste_hip_layer_norm_indrnn_backward_f64(int steps, int batch_size, int inpu
 
 // ---- half (GRU only, as in the reference: lib/gru_forward_gpu.cu.cc:373,
 // lib/gru_backward_gpu.cu.cc:411).  Tensors are IEEE binary16 passed as void*; products are
-// accumulated and the pointwise math is done in float, results rounded to half.
+// accumulated and the pointwise math is done in float, results rounded to half.  Passes over
+// more than one step run on the persistent fp32 kernels (gru_half.hip); a single step
+// (Iterate) runs here, one product and one pointwise launch.
 static inline const half_t* hp(const void* p) { return static_cast<const half_t*>(p); }
 static inline half_t* hp(void* p) { return static_cast<half_t*>(p); }
 
@@ -1489,6 +1500,9 @@ int haste_hip_gru_forward_f16(int training, int steps, int batch_size, int input
   HASTE_HIP_REQUIRE(steps > 0 && batch_size > 0 && input_size > 0 && hidden_size > 0);
   HASTE_HIP_REQUIRE(W && R && bx && br && x && h && tmp_Wx && (v || !training));
   const size_t NH = (size_t)batch_size * hidden_size;
+  if (steps > 1)
+    return gru_forward_half(as_stream(stream), training, steps, batch_size, input_size, hidden_size, W, R,
+                            bx, br, x, h, v, zoneout_prob, zoneout_mask, nullptr, 1.f);
   return gru_forward_steps<half_t>(as_stream(stream), training, steps, batch_size, input_size,
                                    hidden_size, hp(W), hp(R), hp(bx), hp(br), hp(x), hp(h),
                                    hp(h) + NH, hp(v), hp(tmp_Wx), zoneout_prob, hp(zoneout_mask),
@@ -1504,6 +1518,10 @@ int haste_hip_gru_forward_dropconnect_f16(int training, int steps, int batch_siz
   HASTE_HIP_REQUIRE(steps > 0 && batch_size > 0 && input_size > 0 && hidden_size > 0);
   HASTE_HIP_REQUIRE(W && R && bx && br && x && h && tmp_Wx && (v || !training));
   const size_t NH = (size_t)batch_size * hidden_size;
+  if (steps > 1)
+    return gru_forward_half(as_stream(stream), training, steps, batch_size, input_size, hidden_size, W, R,
+                            bx, br, x, h, v, zoneout_prob, zoneout_mask, dropconnect_mask,
+                            dropconnect_scale);
   return gru_forward_steps<half_t>(as_stream(stream), training, steps, batch_size, input_size,
                                    hidden_size, hp(W), hp(R), hp(bx), hp(br), hp(x), hp(h),
                                    hp(h) + NH, hp(v), hp(tmp_Wx), zoneout_prob, hp(zoneout_mask),
@@ -1521,6 +1539,9 @@ int haste_hip_gru_backward_f16(int steps, int batch_size, int input_size, int hi
   HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && v && dh_new);
   HASTE_HIP_REQUIRE(dx && dW && dR && dbx && dbr && dh && dp && dq);
   const size_t NH = (size_t)batch_size * hidden_size;
+  if (steps > 1)
+    return gru_backward_half(as_stream(stream), steps, batch_size, input_size, hidden_size, W_t, R_t, x_t,
+                             h, v, hp(dh_new) + NH, dx, dW, dR, dbx, dbr, dh, dp, dq, zoneout_mask);
   return gru_backward_steps<half_t>(as_stream(stream), steps, batch_size, input_size, hidden_size,
                                     hp(W_t), hp(R_t), hp(x_t), hp(h), hp(v), hp(dh_new) + NH, hp(dx),
                                     hp(dW), hp(dR), hp(dbx), hp(dbr), hp(dh), hp(dp), hp(dq),
