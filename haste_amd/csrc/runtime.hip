@@ -605,6 +605,8 @@ size_t haste_hip_workspace_bytes(int time_steps, int batch_size, int input_size,
   // copy of R, column sums in at most 128 chunks, row statistics of all steps, two [N, H]
   // buffers; the stand-alone layer norm's column sums (two workgroups per CU, two rows each).
   b += (N * 4 * H + H * 4 * H + 128 * widest + T * N * 2 + 2 * N * H) * 8 + 16 * 256;
+  // ... and the K pieces of a double product of few tiles (at most one 64 x 64 piece per CU)
+  b += cus * 64 * 64 * 8;
   b += 2 * cus * 2 * widest * sizeof(float);
   // Single forward steps: partial sums of at most 64 runs of the contraction, both sides, for 8
   // rows and every gate column, and the staged state.

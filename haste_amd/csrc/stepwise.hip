@@ -25,7 +25,8 @@
 namespace haste_hip {
 
 int gemm_f64(hipStream_t stream, bool trans_a, int M, int N, int K, const double* A, int lda,
-             const double* B, int ldb, double* C, int ldc, bool accumulate);
+             const double* B, int ldb, double* C, int ldc, bool accumulate, size_t scratch_offset);
+size_t gemm_f64_scratch_bytes(int M, int N, int K);
 int gemm_f16(hipStream_t stream, bool trans_a, int M, int N, int K, const void* A, int lda,
              const void* B, int ldb, void* C, int ldc, bool accumulate);
 // gru_half.hip: the half GRU over more than one step, on the fp32 kernels.
@@ -72,8 +73,8 @@ inline int gemm(hipStream_t s, bool ta, int M, int N, int K, const float* A, int
   return gemm_f32(s, ta, M, N, K, A, lda, B, ldb, C, ldc, acc, scratch_offset);
 }
 inline int gemm(hipStream_t s, bool ta, int M, int N, int K, const double* A, int lda,
-                const double* B, int ldb, double* C, int ldc, bool acc, size_t) {
-  return gemm_f64(s, ta, M, N, K, A, lda, B, ldb, C, ldc, acc);
+                const double* B, int ldb, double* C, int ldc, bool acc, size_t scratch_offset) {
+  return gemm_f64(s, ta, M, N, K, A, lda, B, ldb, C, ldc, acc, scratch_offset);
 }
 inline int gemm(hipStream_t s, bool ta, int M, int N, int K, const half_t* A, int lda,
                 const half_t* B, int ldb, half_t* C, int ldc, bool acc, size_t) {
@@ -81,7 +82,7 @@ inline int gemm(hipStream_t s, bool ta, int M, int N, int K, const half_t* A, in
 }
 template <typename T> size_t gemm_room(int M, int N, int K);
 template <> size_t gemm_room<float>(int M, int N, int K) { return gemm_f32_scratch_bytes(M, N, K); }
-template <> size_t gemm_room<double>(int, int, int) { return 0; }
+template <> size_t gemm_room<double>(int M, int N, int K) { return gemm_f64_scratch_bytes(M, N, K); }
 template <> size_t gemm_room<half_t>(int, int, int) { return 0; }
 
 // A step's product as its consumer reads it: either one finished matrix (chunks == 1,
