@@ -214,7 +214,13 @@ int xcd_layout_ready(hipStream_t stream) {
   return HASTE_HIP_OK;
 }
 
+namespace {
+// A device shape assumed by this thread instead of the current device's (haste_hip_plan_tiles).
+thread_local int t_assumed_cus = 0, t_assumed_xcds = 0;
+}  // namespace
+
 int device_xcd_count() {
+  if (t_assumed_cus > 0) return t_assumed_xcds;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
   std::lock_guard<std::mutex> lock(g_mutex);
@@ -269,6 +275,7 @@ bool fused_input_enabled() {
 }
 
 int device_cu_count() {
+  if (t_assumed_cus > 0) return t_assumed_cus;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
   std::lock_guard<std::mutex> lock(g_mutex);
@@ -514,6 +521,24 @@ int haste_hip_max_hidden_size(int gates, int batch_size) {
   for (int H = 16; H <= 8192; H += 16)
     if (fits(H)) best = H;
   return best;
+}
+
+int haste_hip_plan_tiles(int cus, int xcds, int gates, int batch_size, int hidden_size, int* plan) {
+  HASTE_HIP_REQUIRE(plan != nullptr && (gates == 3 || gates == 4) && batch_size > 0 && hidden_size > 0);
+  HASTE_HIP_REQUIRE(cus >= 0 && xcds >= 0 && (cus > 0 || xcds == 0));
+  using namespace haste_hip;
+  const int H = hidden_size;
+  t_assumed_cus = cus;
+  t_assumed_xcds = xcds;
+  const int k_back = gates == 3 ? 48 * ((H + 15) / 16) : gates * H;
+  const ForwardTile f = pick_forward_tile(gates, batch_size, H, 0, kWorkgroupLdsBytes, false, gates == 3 ? 3 : 2);
+  const BackwardTile b = pick_backward_tile(k_back, batch_size, H, gates == 3 ? 6 * 16 : (size_t)gates * 16, 0, true);
+  t_assumed_cus = 0;
+  t_assumed_xcds = 0;
+  const int out[16] = {f.ok, f.nb, f.hs, f.ct, f.gx, f.gy, f.reg_groups, (H + 63) / 64,
+                       b.ok, b.nb, 16, 1, b.gx, b.gy, b.reg_groups, (k_back + 63) / 64};
+  for (int i = 0; i < 16; ++i) plan[i] = (i % 8 == 0 || out[i - i % 8]) ? out[i] : 0;
+  return HASTE_HIP_OK;
 }
 
 int haste_hip_stream_status(void* stream_) {

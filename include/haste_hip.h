@@ -44,6 +44,18 @@ const char* haste_hip_last_runtime_error(void);
  * kernels per step, as the reference does). */
 int haste_hip_max_hidden_size(int gates, int batch_size);
 
+/* How Run would lay the persistent recurrences of a cell with `gates` gate blocks (4 LSTM, 3 GRU)
+ * out for this batch and hidden size on a device of `cus` compute units in `xcds` XCDs that take
+ * workgroups evenly (cus == 0: the current device as the library found it; xcds == 0: no
+ * placement by XCD).  Touches no device when cus > 0.  plan[0..7] describes the forward
+ * recurrence, plan[8..15] the backward one: {found (0: the cell streams the recurrent matrix
+ * from HBM every step instead; the rest are then 0), batch rows per tile, hidden units per
+ * workgroup, 16-column tiles of the weight slice, column workgroups, batch tiles, groups of 16
+ * contraction rows per wavefront kept in registers, such groups in a wavefront's whole share}.
+ * No counterpart in the reference (its kernels have one geometry); for capacity planning and
+ * for tests of the geometry search. */
+int haste_hip_plan_tiles(int cus, int xcds, int gates, int batch_size, int hidden_size, int* plan);
+
 /* Drops this thread's cached per-stream workspaces on the current device (frees
  * device memory; the caller must have synchronized the streams that used them). */
 int haste_hip_release_workspaces(void);
