@@ -452,6 +452,22 @@ def run_hbm_kernels(args, torch, lib, ops, dev):
     t = timed(("indrnn_forward_recurrence", "indrnn_backward_recurrence"), ind_speed, reps=3)
     out["indrnn_forward_N64_T2500_C256_H4096"] = entry(t["indrnn_forward_recurrence"], 4.0 * 2 * T * N * H)
     out["indrnn_backward_N64_T2500_C256_H4096"] = entry(t["indrnn_backward_recurrence"], 4.0 * 3 * T * N * H)
+    del xs, x_t, dh_new
+
+    # Yardstick: what a plain device copy of 1 GiB (read once, written once: the same mix of
+    # traffic as the IndRNN recurrences) reaches on this box.
+    src = torch.empty(256 * 1024 * 1024, device=dev)
+    dst = torch.empty_like(src)
+    for _ in range(2):
+        dst.copy_(src)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(5):
+        dst.copy_(src)
+    e1.record()
+    torch.cuda.synchronize()
+    out["device_copy_1GiB"] = entry(e0.elapsed_time(e1) / 5.0, 2.0 * 4 * src.numel())
+    del src, dst
     out["indrnn_speed_script_shape"] = {"forward_pass_ms": round(total["fwd"], 3), "backward_pass_ms": round(total["bwd"], 3),
                                         "note": "whole passes (x*W, recurrence; recurrence, dW, dx) at the shape of "
                                                 "the reference's validation/pytorch_speed.py"}
