@@ -95,6 +95,10 @@ class ScratchPrefix {
   size_t saved_;
 };
 
+// The scratch part of haste_hip_workspace_bytes(T, N, C, H): what a workspace of that size
+// offers behind its control block.
+size_t workspace_scratch_bound(int T, int N, int C, int H);
+
 // Reserves `count` consecutive step-flag values on the workspace of (current device,
 // stream) and returns the value before the first of them.
 int reserve_epochs(hipStream_t stream, unsigned int count, unsigned int* base);

@@ -120,9 +120,47 @@ struct Staging {
 // The staging area of `bytes` bytes plus room behind it for everything the fp32 passes ask for.
 int staged_workspace(hipStream_t stream, int T, int N, int C, int H, size_t bytes, float** base) {
   Workspace ws;
-  HASTE_HIP_PROPAGATE(get_workspace(stream, bytes + haste_hip_workspace_bytes(T, N, C, H), &ws));
+  HASTE_HIP_PROPAGATE(get_workspace(stream, bytes + workspace_scratch_bound(T, N, C, H), &ws));
   *base = ws.scratch;
   return HASTE_HIP_OK;
+}
+
+// Where the staged tensors of a forward / backward pass lie (offsets in floats).
+struct ForwardStaging {
+  size_t W, R, bx, br, x, h, v, Wx, mask, dc, bytes;
+  ForwardStaging(int T, int N, int C, int H, bool training, bool has_mask, bool has_dc) {
+    const size_t NH = (size_t)N * H, TN = (size_t)T * N;
+    Staging st;
+    W = st.take((size_t)C * 3 * H); R = st.take((size_t)H * 3 * H);
+    bx = st.take(3 * (size_t)H); br = st.take(3 * (size_t)H);
+    x = st.take(TN * C); h = st.take((T + 1) * NH);
+    v = training ? st.take(TN * 4 * H) : 0;
+    Wx = st.take(TN * 3 * H);
+    mask = has_mask ? st.take(TN * H) : 0;
+    dc = has_dc ? st.take((size_t)H * 3 * H) : 0;
+    bytes = st.floats * sizeof(float);
+  }
+};
+
+struct BackwardStaging {
+  size_t Wt, Rt, xt, h, v, dhn, mask, dx, dW, dR, dbx, dbr, dh, dp, dq, bytes;
+  BackwardStaging(int T, int N, int C, int H, bool has_mask) {
+    const size_t NH = (size_t)N * H, TN = (size_t)T * N, H3 = 3 * (size_t)H;
+    Staging st;
+    Wt = st.take(H3 * C); Rt = st.take(H3 * H); xt = st.take(TN * C);
+    h = st.take((T + 1) * NH); v = st.take(TN * 4 * H); dhn = st.take(TN * H);
+    mask = has_mask ? st.take(TN * H) : 0;
+    dx = st.take(TN * C); dW = st.take(C * H3); dR = st.take(H * H3);
+    dbx = st.take(H3); dbr = st.take(H3); dh = st.take(NH);
+    dp = st.take(TN * H3); dq = st.take(TN * H3);
+    bytes = st.floats * sizeof(float);
+  }
+};
+
+size_t gru_half_staging_bytes(int T, int N, int C, int H) {
+  const size_t f = ForwardStaging(T, N, C, H, true, true, true).bytes;
+  const size_t b = BackwardStaging(T, N, C, H, true).bytes;
+  return f > b ? f : b;
 }
 
 }  // namespace
@@ -133,15 +171,9 @@ int gru_forward_half(hipStream_t stream, int training, int T, int N, int C, int 
                      float zoneout_prob, const void* zoneout_mask, const void* dc_mask,
                      float dc_scale) {
   const size_t NH = (size_t)N * H, TN = (size_t)T * N;
-  Staging st;
-  const size_t oW = st.take((size_t)C * 3 * H), oR = st.take((size_t)H * 3 * H);
-  const size_t obx = st.take(3 * (size_t)H), obr = st.take(3 * (size_t)H);
-  const size_t ox = st.take(TN * C), oh = st.take((T + 1) * NH);
-  const size_t ov = training ? st.take(TN * 4 * H) : 0;
-  const size_t oWx = st.take(TN * 3 * H);
-  const size_t om = zoneout_mask ? st.take(TN * H) : 0;
-  const size_t od = dc_mask ? st.take((size_t)H * 3 * H) : 0;
-  const size_t bytes = st.floats * sizeof(float);
+  const ForwardStaging at(T, N, C, H, training != 0, zoneout_mask != nullptr, dc_mask != nullptr);
+  const size_t oW = at.W, oR = at.R, obx = at.bx, obr = at.br, ox = at.x, oh = at.h, ov = at.v, oWx = at.Wx;
+  const size_t om = at.mask, od = at.dc, bytes = at.bytes;
   float* f = nullptr;
   HASTE_HIP_PROPAGATE(staged_workspace(stream, T, N, C, H, bytes, &f));
 
@@ -175,14 +207,10 @@ int gru_backward_half(hipStream_t stream, int T, int N, int C, int H, const void
                       const void* dh_next, void* dx, void* dW, void* dR, void* dbx, void* dbr,
                       void* dh, void* dp, void* dq, const void* zoneout_mask) {
   const size_t NH = (size_t)N * H, TN = (size_t)T * N, H3 = 3 * (size_t)H;
-  Staging st;
-  const size_t oWt = st.take(H3 * C), oRt = st.take(H3 * H), oxt = st.take(TN * C);
-  const size_t oh = st.take((T + 1) * NH), ov = st.take(TN * 4 * H), odn = st.take(TN * H);
-  const size_t om = zoneout_mask ? st.take(TN * H) : 0;
-  const size_t odx = st.take(TN * C), odW = st.take(C * H3), odR = st.take(H * H3);
-  const size_t odbx = st.take(H3), odbr = st.take(H3), odh = st.take(NH);
-  const size_t odp = st.take(TN * H3), odq = st.take(TN * H3);
-  const size_t bytes = st.floats * sizeof(float);
+  const BackwardStaging at(T, N, C, H, zoneout_mask != nullptr);
+  const size_t oWt = at.Wt, oRt = at.Rt, oxt = at.xt, oh = at.h, ov = at.v, odn = at.dhn, om = at.mask;
+  const size_t odx = at.dx, odW = at.dW, odR = at.dR, odbx = at.dbx, odbr = at.dbr, odh = at.dh;
+  const size_t odp = at.dp, odq = at.dq, bytes = at.bytes;
   float* f = nullptr;
   HASTE_HIP_PROPAGATE(staged_workspace(stream, T, N, C, H, bytes, &f));
 
@@ -219,3 +247,10 @@ int gru_backward_half(hipStream_t stream, int T, int N, int C, int H, const void
 }
 
 }  // namespace haste_hip
+
+extern "C" size_t haste_hip_gru_half_workspace_bytes(int time_steps, int batch_size, int input_size,
+                                                     int hidden_size) {
+  if (time_steps < 1 || batch_size < 1 || input_size < 1 || hidden_size < 1) return 0;
+  return haste_hip_workspace_bytes(time_steps, batch_size, input_size, hidden_size) +
+         haste_hip::gru_half_staging_bytes(time_steps, batch_size, input_size, hidden_size);
+}

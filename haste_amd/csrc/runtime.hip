@@ -639,6 +639,17 @@ size_t haste_hip_workspace_bytes(int time_steps, int batch_size, int input_size,
   return kControlBytes + 4096 + (b + 255) / 256 * 256;
 }
 
+}  // extern "C"
+
+namespace haste_hip {
+size_t workspace_scratch_bound(int T, int N, int C, int H) {
+  const size_t all = haste_hip_workspace_bytes(T, N, C, H);
+  return all > kControlBytes ? all - kControlBytes : 0;
+}
+}  // namespace haste_hip
+
+extern "C" {
+
 int haste_hip_profile_enable(int on) {
   std::lock_guard<std::mutex> lock(haste_hip::g_mutex);
   haste_hip::g_profile_on = on != 0;

@@ -54,13 +54,15 @@ def stream_status(stream=None):
         raise lib.HasteHipError(rc, "haste_hip_stream_status")
 
 
-def workspace_bytes(time_steps, batch_size, input_size, hidden_size):
-    """Upper bound of the scratch memory any cell needs for these sizes on the current device."""
+def workspace_bytes(time_steps, batch_size, input_size, hidden_size, half_gru=False):
+    """Upper bound of the scratch memory any cell needs for these sizes on the current device
+    (half_gru: the GRU on half tensors, which also stages fp32 copies of its tensors there)."""
     import ctypes
     handle = lib.load()
-    handle.haste_hip_workspace_bytes.restype = ctypes.c_size_t
-    handle.haste_hip_workspace_bytes.argtypes = [ctypes.c_int] * 4
-    return int(handle.haste_hip_workspace_bytes(time_steps, batch_size, input_size, hidden_size))
+    fn = handle.haste_hip_gru_half_workspace_bytes if half_gru else handle.haste_hip_workspace_bytes
+    fn.restype = ctypes.c_size_t
+    fn.argtypes = [ctypes.c_int] * 4
+    return int(fn(time_steps, batch_size, input_size, hidden_size))
 
 
 def set_workspace(buffer, stream=None):

@@ -87,11 +87,18 @@ int haste_hip_stream_status(void* stream);
  * (lib/haste/lstm.h:98-117).
  *
  * haste_hip_workspace_bytes: an upper bound of what any cell, direction and scalar type
- * needs for (T, N, C, H) on the current device (for the stand-alone layer norm: T = 1,
+ * (but for the half GRU, below) needs for (T, N, C, H) on the current device (for the stand-alone layer norm: T = 1,
  * N = rows, C = H = dim): 64 MiB for the partial tiles of split GEMMs plus terms in N*H,
  * H*H and T*N.  haste_hip_workspace_high_water: what the calls made on `stream` so far
  * have actually needed (after a rehearsal of the same calls, the exact size to lend). */
 size_t haste_hip_workspace_bytes(int time_steps, int batch_size, int input_size, int hidden_size);
+
+/* The same bound for haste_hip_gru_{forward,forward_dropconnect,backward}_f16, which over more
+ * than one step stage fp32 copies of their tensors in the workspace (4 bytes per element of
+ * every tensor of the call) in front of what the fp32 passes they run ask for.  No counterpart
+ * in the reference. */
+size_t haste_hip_gru_half_workspace_bytes(int time_steps, int batch_size, int input_size,
+                                          int hidden_size);
 int haste_hip_set_workspace(void* stream, void* memory, size_t bytes);
 int haste_hip_workspace_high_water(void* stream, size_t* bytes);
 

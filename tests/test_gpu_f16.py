@@ -118,6 +118,43 @@ def test_f16_gru_dropconnect_and_accumulated_gradients():
         assert relerr(host(out[name]), theirs + start[name]) < TOL16, name
 
 
+def test_f16_gru_with_a_lent_workspace():
+    """The staging area of the half GRU lives in the stream's workspace: a lent buffer that is too
+    small is refused with the size in the error text; one of haste_hip_gru_half_workspace_bytes
+    gives the bits of the library-owned run."""
+    from haste_amd import ops, lib as hlib
+    import torch
+    T, N, C, H = 7, 10, 24, 64
+    p = half_problem(77, T, N, C, H, 0.2)
+    args = [dev16(p[k]) for k in ("x", "h0", "W", "R", "b", "b2", "mask")]
+
+    def run():
+        h, cache = ops.gru_forward(True, 0.2, *args)
+        grads = ops.gru_backward(ops.transpose(args[0]), ops.transpose(args[2]), ops.transpose(args[3]), args[4],
+                                 args[5], args[6], h, cache, dev16(p["dh_new"]))
+        torch.cuda.synchronize()
+        return (h, cache) + tuple(grads)
+
+    want = run()
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        small = torch.empty(ops.workspace_bytes(T, N, C, H) // 4 // 64, dtype=torch.float32, device="cuda")
+        ops.set_workspace(small)
+        try:
+            with pytest.raises(hlib.HasteHipError) as e:
+                ops.gru_forward(True, 0.2, *args)
+            assert e.value.code == 2 and "too small" in str(e.value)
+            lent = torch.empty(ops.workspace_bytes(T, N, C, H, half_gru=True) // 4 + 64, dtype=torch.float32,
+                               device="cuda")
+            ops.set_workspace(lent)
+            got = run()
+        finally:
+            torch.cuda.synchronize()
+            ops.set_workspace(None)
+    for g, w in zip(got, want):
+        assert torch.equal(g, w)
+
+
 def test_f16_lstm_is_refused():
     """As in the reference, half exists for the GRU only."""
     from haste_amd import ops
