@@ -543,10 +543,10 @@ def run_configs(args, torch, lib, ops, dev):
         return ops.gru_backward(ops.transpose(xh), ops.transpose(Wh), ops.transpose(Rh), bxh, brh, zmh, h, cache, dhh)
     ms = timed(gru_half_step, 5)
     out["gru_f16_fwd_bwd_N64_T100_H512_zoneout_ms"] = ms
-    # half is the storage format: passes over more than one step widen the tensors and run the
-    # fp32 kernels, so the fraction is of the fp32 peak
+    # half tensors; the recurrences (half of the flops) run in fp32 on widened copies, the
+    # products around them on the half matrix cores: quoted against the fp32 peak, like the rest
     note("gru_f16_fwd_bwd_N64_T100_H512_zoneout", ms, 3 * 2.0 * T * N * 3 * H * (C + H), PEAK_FP32_MFMA_TFLOPS,
-         "f16 tensors, f32 arithmetic")
+         "f16 tensors, f32 recurrences, f16 products with f32 accumulation")
 
     T, N, C, H = 100, 128, 512, 512  # config 3: LSTM training, N=128
     x, W, R = rnd(T, N, C), uni(k, C, 4 * H), uni(k, H, 4 * H)

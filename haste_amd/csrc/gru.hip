@@ -731,8 +731,9 @@ struct GruScatterCell {
 int gru_forward_single_row(hipStream_t stream, int training, int T, int C, int H, const float* W,
                            const float* R, const float* bx, const float* br, const float* x,
                            const float* h, float* h_out, float* v, float* tmp_Wx, float zoneout_prob,
-                           const float* zoneout_mask, const float* dc_mask, float dc_scale) {
-  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T, 3 * H, C, x, C, W, 3 * H, tmp_Wx, 3 * H, false));
+                           const float* zoneout_mask, const float* dc_mask, float dc_scale, bool wx_ready) {
+  if (!wx_ready)
+    HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T, 3 * H, C, x, C, W, 3 * H, tmp_Wx, 3 * H, false));
   const int Kpad = (H + 63) / 64 * 64;
   Workspace ws;
   HASTE_HIP_PROPAGATE(get_workspace(stream, (size_t)kPolledTiles * Kpad * sizeof(float), &ws));
@@ -755,15 +756,28 @@ int gru_forward_single_row(hipStream_t stream, int training, int T, int C, int H
   return launch_persistent(name, gru_forward_single_row_kernel<128>, plan, p, stream);
 }
 
+// True when a pass over more than one step keeps the recurrent weights on chip (the persistent
+// kernels) instead of streaming them every step: then the recurrence can be run by itself, on
+// products computed elsewhere (wx_ready / products below).
+bool gru_forward_resident(int N, int H) {
+  if (N == 1 && H <= 512 && xcd_local_fits((H + 15) / 16, 1)) return true;
+  return pick_forward_tile(3, N, H, 0, kWorkgroupLdsBytes, false, 3).ok;
+}
+bool gru_backward_resident(int N, int H) {
+  return pick_backward_tile(gru_backward_k(H), N, H, 6 * 16, 0, true).ok;
+}
+
 // h: [N,H] state before the first step; h_out: [T,N,H] states after each step.
+// wx_ready (T > 1, gru_forward_resident): tmp_Wx already holds x*W, and W and x are not looked at.
 int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int H,
                      const float* W, const float* R, const float* bx, const float* br,
                      const float* x, const float* h, float* h_out, float* v, float* tmp_Wx,
                      float zoneout_prob, const float* zoneout_mask, const float* dc_mask,
-                     float dc_scale) {
+                     float dc_scale, bool wx_ready) {
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
-  HASTE_HIP_REQUIRE(W && R && bx && br && x && h && h_out && tmp_Wx);
+  HASTE_HIP_REQUIRE(R && bx && br && h && h_out && tmp_Wx && (wx_ready || (W && x)));
   HASTE_HIP_REQUIRE(!training || v != nullptr);
+  HASTE_HIP_REQUIRE(!wx_ready || (T > 1 && gru_forward_resident(N, H)));
   // A single step of a small batch (Iterate): one kernel, nothing kept on chip (tmp_Wx is
   // scratch of the other paths and is left alone).
   if (T == 1 && single_step_applies(N, C, H))
@@ -771,13 +785,14 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
                                    zoneout_prob, zoneout_mask, dc_mask, dc_scale);
   if (N == 1 && H <= 512 && xcd_local_fits((H + 15) / 16, 1))
     return gru_forward_single_row(stream, training, T, C, H, W, R, bx, br, x, h, h_out, v, tmp_Wx,
-                                  zoneout_prob, zoneout_mask, dc_mask, dc_scale);
+                                  zoneout_prob, zoneout_mask, dc_mask, dc_scale, wx_ready);
   const ForwardTile tile = pick_forward_tile(3, N, H, 0, kWorkgroupLdsBytes, false, 3);
   // No slice of R fits a CU: stream R from HBM every step instead.
   if (!tile.ok)
     return gru_forward_streamed(stream, training, T, N, C, H, W, R, bx, br, x, h, h_out, v, tmp_Wx,
                                 zoneout_prob, zoneout_mask, dc_mask, dc_scale);
-  HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 3 * H, C, x, C, W, 3 * H, tmp_Wx, 3 * H, false));
+  if (!wx_ready)
+    HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 3 * H, C, x, C, W, 3 * H, tmp_Wx, 3 * H, false));
 
   // An 8-row tile is run as two sets of 4 rows when the partial tiles of both fit beside the
   // slice (exchange tiles: one per set, together as large as the tile's).
@@ -830,14 +845,17 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
   return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 }
 
+// products == false (gru_backward_resident): the recurrence only -- dp, dq, dbx, dbr, dh; the
+// caller computes dx, dW and dR from dp and dq itself, and W_t, x_t, dx, dW, dR are not looked at.
 int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
                       const float* W_t, const float* R_t, const float* x_t, const float* h,
                       const float* v, const float* dh_next, float* dx, float* dW, float* dR,
                       float* dbx, float* dbr, float* dh, float* dp, float* dq,
-                      const float* zoneout_mask) {
+                      const float* zoneout_mask, bool products) {
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
-  HASTE_HIP_REQUIRE(W_t && R_t && x_t && h && v && dh_next);
-  HASTE_HIP_REQUIRE(dx && dW && dR && dbx && dbr && dh && dp && dq);
+  HASTE_HIP_REQUIRE(R_t && h && v && dh_next && (!products || (W_t && x_t)));
+  HASTE_HIP_REQUIRE(dbx && dbr && dh && dp && dq && (!products || (dx && dW && dR)));
+  HASTE_HIP_REQUIRE(products || gru_backward_resident(N, H));
   // per row: the partial tiles or the 6 bias-gradient columns of 16 floats
   const BackwardTile tile = pick_backward_tile(gru_backward_k(H), N, H, 6 * 16, 0, true);
   if (!tile.ok)
@@ -899,6 +917,7 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   else if (tile.nb == 32) rc = launch_persistent(name, gru_backward_kernel<32, 1>, plan, p, stream);
   else if (tile.nb == 64) rc = launch_persistent(name, gru_backward_kernel<64, 1>, plan, p, stream);
   HASTE_HIP_PROPAGATE(rc);
+  if (!products) return HASTE_HIP_OK;
 
   const int TN = T * N;
   HASTE_HIP_PROPAGATE(gemm_f32(stream, false, TN, C, 3 * H, dp, 3 * H, W_t, C, dx, C, false));
@@ -922,7 +941,7 @@ int haste_hip_gru_forward_f32(int training, int steps, int batch_size, int input
   return haste_hip::gru_forward_impl(haste_hip::as_stream(stream), training, steps, batch_size,
                                      input_size, hidden_size, W, R, bx, br, x, h,
                                      h + (size_t)batch_size * hidden_size, v, tmp_Wx,
-                                     zoneout_prob, zoneout_mask, nullptr, 1.0f);
+                                     zoneout_prob, zoneout_mask, nullptr, 1.0f, false);
 }
 
 int haste_hip_gru_forward_dropconnect_f32(int training, int steps, int batch_size,
@@ -938,7 +957,7 @@ int haste_hip_gru_forward_dropconnect_f32(int training, int steps, int batch_siz
                                      input_size, hidden_size, W, R, bx, br, x, h,
                                      h + (size_t)batch_size * hidden_size, v, tmp_Wx,
                                      zoneout_prob, zoneout_mask, dropconnect_mask,
-                                     dropconnect_scale);
+                                     dropconnect_scale, false);
 }
 
 int haste_hip_gru_backward_f32(int steps, int batch_size, int input_size, int hidden_size,
@@ -953,7 +972,7 @@ int haste_hip_gru_backward_f32(int steps, int batch_size, int input_size, int hi
   return haste_hip::gru_backward_impl(haste_hip::as_stream(stream), steps, batch_size, input_size,
                                       hidden_size, W_t, R_t, x_t, h, v,
                                       dh_new + (size_t)batch_size * hidden_size, dx, dW, dR, dbx,
-                                      dbr, dh, dp, dq, zoneout_mask);
+                                      dbr, dh, dp, dq, zoneout_mask, true);
 }
 
 int haste_hip_gru_forward_iterate_f32(int training, int batch_size, int input_size,
@@ -966,7 +985,7 @@ int haste_hip_gru_forward_iterate_f32(int training, int batch_size, int input_si
   (void)tmp_Rh;
   return haste_hip::gru_forward_impl(haste_hip::as_stream(stream), training, 1, batch_size,
                                      input_size, hidden_size, W, R, bx, br, x, h, h_out, v, tmp_Wx,
-                                     zoneout_prob, zoneout_mask, nullptr, 1.0f);
+                                     zoneout_prob, zoneout_mask, nullptr, 1.0f, false);
 }
 
 int haste_hip_gru_backward_iterate_f32(int batch_size, int input_size, int hidden_size,
@@ -979,7 +998,7 @@ int haste_hip_gru_backward_iterate_f32(int batch_size, int input_size, int hidde
   (void)br;
   return haste_hip::gru_backward_impl(haste_hip::as_stream(stream), 1, batch_size, input_size,
                                       hidden_size, W_t, R_t, x_t, h, v, dh_new, dx, dW, dR, dbx,
-                                      dbr, dh, dp, dq, zoneout_mask);
+                                      dbr, dh, dp, dq, zoneout_mask, true);
 }
 
 }  // extern "C"

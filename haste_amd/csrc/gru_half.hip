@@ -2,13 +2,17 @@
 // BackwardPass<__half>::Run bind to; reference lib/gru_forward_gpu.cu.cc:373,
 // lib/gru_backward_gpu.cu.cc:411).
 //
-// Half is the caller's storage format here, not the arithmetic: the recurrence is bound by
-// the latency of its per-step exchange and by instruction issue, not by the rate of the matrix
-// units or by HBM, so the persistent fp32 kernels are also the fastest way to run half
-// tensors.  The tensors are widened into a staging area at the front of the stream's scratch
-// buffer (one launch), the fp32 passes run on the staged copies, and what the caller gets back
-// is rounded to half (one launch).  Between the steps the state stays in fp32: the results are
-// those of exact half inputs, rounded once, where the reference rounds every step.
+// The recurrence is bound by the latency of its per-step exchange and by instruction issue,
+// not by the rate of the matrix units or by HBM, so the persistent fp32 kernels are also the
+// fastest way to run it on half tensors: what it reads is widened into a staging area at the
+// front of the stream's scratch buffer (one launch), it runs on the staged copies, and what the
+// caller gets back is rounded to half (one launch).  Between the steps the state stays in fp32:
+// the results are those of exact half inputs, rounded once, where the reference rounds every
+// step.  The products around the recurrence (x*W; dx, dW, dR) are bound by the matrix units,
+// and those run on the half matrix cores (gemm_half_nt.hip: half operands, the gate gradients
+// rounded to half as the reference stores them, fp32 accumulation) whenever the operands are
+// laid out for it (sizes multiples of 8, 16-byte aligned) and the recurrence is a persistent
+// one; otherwise the whole pass runs in fp32 on widened tensors.
 #include "common.h"
 
 extern "C" size_t haste_hip_workspace_bytes(int time_steps, int batch_size, int input_size, int hidden_size);
@@ -19,12 +23,19 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
                      const float* W, const float* R, const float* bx, const float* br,
                      const float* x, const float* h, float* h_out, float* v, float* tmp_Wx,
                      float zoneout_prob, const float* zoneout_mask, const float* dc_mask,
-                     float dc_scale);
+                     float dc_scale, bool wx_ready);
 int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
                       const float* W_t, const float* R_t, const float* x_t, const float* h,
                       const float* v, const float* dh_next, float* dx, float* dW, float* dR,
                       float* dbx, float* dbr, float* dh, float* dp, float* dq,
-                      const float* zoneout_mask);
+                      const float* zoneout_mask, bool products);
+bool gru_forward_resident(int N, int H);
+bool gru_backward_resident(int N, int H);
+// gemm_half_nt.hip
+bool gemm_half_nt_applies(bool a_float, int M, int N, int K, const void* A, int lda, const void* Bt, int ldb);
+int gemm_half_nt(hipStream_t stream, bool a_float, int M, int N, int K, const void* A, int lda,
+                 const void* Bt, int ldb, float* C, int ldc, bool accumulate, size_t scratch_offset);
+int transpose_to_half(hipStream_t stream, bool in_float, int rows, int cols, const void* in, void* out);
 
 namespace {
 
@@ -127,7 +138,7 @@ int staged_workspace(hipStream_t stream, int T, int N, int C, int H, size_t byte
 
 // Where the staged tensors of a forward / backward pass lie (offsets in floats).
 struct ForwardStaging {
-  size_t W, R, bx, br, x, h, v, Wx, mask, dc, bytes;
+  size_t W, R, bx, br, x, h, v, Wx, mask, dc, Wt_half, bytes;
   ForwardStaging(int T, int N, int C, int H, bool training, bool has_mask, bool has_dc) {
     const size_t NH = (size_t)N * H, TN = (size_t)T * N;
     Staging st;
@@ -138,12 +149,13 @@ struct ForwardStaging {
     Wx = st.take(TN * 3 * H);
     mask = has_mask ? st.take(TN * H) : 0;
     dc = has_dc ? st.take((size_t)H * 3 * H) : 0;
+    Wt_half = st.take(((size_t)C * 3 * H + 1) / 2);  // W transposed, in half
     bytes = st.floats * sizeof(float);
   }
 };
 
 struct BackwardStaging {
-  size_t Wt, Rt, xt, h, v, dhn, mask, dx, dW, dR, dbx, dbr, dh, dp, dq, bytes;
+  size_t Wt, Rt, xt, h, v, dhn, mask, dx, dW, dR, dbx, dbr, dh, dp, dq, W_half, dpT_half, dqT_half, hT_half, bytes;
   BackwardStaging(int T, int N, int C, int H, bool has_mask) {
     const size_t NH = (size_t)N * H, TN = (size_t)T * N, H3 = 3 * (size_t)H;
     Staging st;
@@ -153,6 +165,10 @@ struct BackwardStaging {
     dx = st.take(TN * C); dW = st.take(C * H3); dR = st.take(H * H3);
     dbx = st.take(H3); dbr = st.take(H3); dh = st.take(NH);
     dp = st.take(TN * H3); dq = st.take(TN * H3);
+    // in half: W (W_t transposed), the gate gradients and h transposed (time contiguous)
+    W_half = st.take((C * H3 + 1) / 2);
+    dpT_half = st.take((TN * H3 + 1) / 2); dqT_half = st.take((TN * H3 + 1) / 2);
+    hT_half = st.take((TN * H + 1) / 2);
     bytes = st.floats * sizeof(float);
   }
 };
@@ -177,6 +193,33 @@ int gru_forward_half(hipStream_t stream, int training, int T, int N, int C, int 
   float* f = nullptr;
   HASTE_HIP_PROPAGATE(staged_workspace(stream, T, N, C, H, bytes, &f));
 
+  // x*W on the half matrix cores, the recurrence alone in fp32
+  if (gru_forward_resident(N, H) && (long long)T * N < (1ll << 31) &&
+      gemm_half_nt_applies(false, (int)TN, 3 * H, C, x, C, f + at.Wt_half, C)) {
+    ConvertList in;
+    in.add(R, f + oR, (size_t)H * 3 * H);
+    in.add(bx, f + obx, 3 * (size_t)H);
+    in.add(br, f + obr, 3 * (size_t)H);
+    in.add(h, f + oh, NH);
+    if (zoneout_mask) in.add(zoneout_mask, f + om, TN * H);
+    if (dc_mask) in.add(dc_mask, f + od, (size_t)H * 3 * H);
+    HASTE_HIP_PROPAGATE(convert<true>(stream, in));
+    HASTE_HIP_PROPAGATE(transpose_to_half(stream, false, C, 3 * H, W, f + at.Wt_half));
+    {
+      ScratchPrefix keep(bytes);
+      HASTE_HIP_PROPAGATE(gemm_half_nt(stream, false, (int)TN, 3 * H, C, x, C, f + at.Wt_half, C, f + oWx, 3 * H,
+                                       false, 0));
+      HASTE_HIP_PROPAGATE(gru_forward_impl(stream, training, T, N, C, H, nullptr, f + oR, f + obx, f + obr, nullptr,
+                                           f + oh, f + oh + NH, training ? f + ov : nullptr, f + oWx, zoneout_prob,
+                                           zoneout_mask ? f + om : nullptr, dc_mask ? f + od : nullptr, dc_scale,
+                                           true));
+    }
+    ConvertList out;
+    out.add(f + oh + NH, static_cast<half_t*>(h) + NH, TN * H);
+    if (training) out.add(f + ov, v, TN * 4 * H);
+    return convert<false>(stream, out);
+  }
+
   ConvertList in;
   in.add(W, f + oW, (size_t)C * 3 * H);
   in.add(R, f + oR, (size_t)H * 3 * H);
@@ -192,7 +235,7 @@ int gru_forward_half(hipStream_t stream, int training, int T, int N, int C, int 
     HASTE_HIP_PROPAGATE(gru_forward_impl(stream, training, T, N, C, H, f + oW, f + oR, f + obx, f + obr,
                                          f + ox, f + oh, f + oh + NH, training ? f + ov : nullptr, f + oWx,
                                          zoneout_prob, zoneout_mask ? f + om : nullptr,
-                                         dc_mask ? f + od : nullptr, dc_scale));
+                                         dc_mask ? f + od : nullptr, dc_scale, false));
   }
   ConvertList out;
   out.add(f + oh + NH, static_cast<half_t*>(h) + NH, TN * H);
@@ -201,11 +244,15 @@ int gru_forward_half(hipStream_t stream, int training, int T, int N, int C, int 
 }
 
 // h: [(T+1),N,H]; dh_next: [T,N,H], the gradients w.r.t. the states after each step.  dW, dR,
-// dbx, dbr and dh are added to, as in the fp32 pass (widened, added to in fp32, rounded).
+// dbx, dbr and dh are added to, as in the fp32 pass (widened, added to in fp32, rounded).  dp and
+// dq are work space whose contents the caller is not to use (reference lib/haste/gru.h:164-169):
+// the gate gradients live in the staging area and the caller's two buffers are left alone.
 int gru_backward_half(hipStream_t stream, int T, int N, int C, int H, const void* W_t,
                       const void* R_t, const void* x_t, const void* h, const void* v,
                       const void* dh_next, void* dx, void* dW, void* dR, void* dbx, void* dbr,
                       void* dh, void* dp, void* dq, const void* zoneout_mask) {
+  (void)dp;
+  (void)dq;
   const size_t NH = (size_t)N * H, TN = (size_t)T * N, H3 = 3 * (size_t)H;
   const BackwardStaging at(T, N, C, H, zoneout_mask != nullptr);
   const size_t oWt = at.Wt, oRt = at.Rt, oxt = at.xt, oh = at.h, ov = at.v, odn = at.dhn, om = at.mask;
@@ -213,6 +260,49 @@ int gru_backward_half(hipStream_t stream, int T, int N, int C, int H, const void
   const size_t odp = at.dp, odq = at.dq, bytes = at.bytes;
   float* f = nullptr;
   HASTE_HIP_PROPAGATE(staged_workspace(stream, T, N, C, H, bytes, &f));
+
+  // the recurrence alone in fp32; dx = dp * W_t, dW += x_t * dp, dR += h^T * dq on the half
+  // matrix cores, every operand with the contraction index contiguous
+  const int iTN = (int)TN, iH3 = 3 * H;
+  if (gru_backward_resident(N, H) && (long long)T * N < (1ll << 31) &&
+      gemm_half_nt_applies(true, iTN, C, iH3, f + odp, iH3, f + at.W_half, iH3) &&
+      gemm_half_nt_applies(false, C, iH3, iTN, x_t, iTN, f + at.dpT_half, iTN) &&
+      gemm_half_nt_applies(false, H, iH3, iTN, f + at.hT_half, iTN, f + at.dqT_half, iTN)) {
+    ConvertList in;
+    in.add(R_t, f + oRt, H3 * H);
+    in.add(h, f + oh, (T + 1) * NH);
+    in.add(v, f + ov, TN * 4 * H);
+    in.add(dh_next, f + odn, TN * H);
+    if (zoneout_mask) in.add(zoneout_mask, f + om, TN * H);
+    in.add(dW, f + odW, C * H3);
+    in.add(dR, f + odR, H * H3);
+    in.add(dbx, f + odbx, H3);
+    in.add(dbr, f + odbr, H3);
+    in.add(dh, f + odh, NH);
+    HASTE_HIP_PROPAGATE(convert<true>(stream, in));
+    HASTE_HIP_PROPAGATE(transpose_to_half(stream, false, iH3, C, W_t, f + at.W_half));
+    HASTE_HIP_PROPAGATE(transpose_to_half(stream, false, iTN, H, h, f + at.hT_half));
+    {
+      ScratchPrefix keep(bytes);
+      HASTE_HIP_PROPAGATE(gru_backward_impl(stream, T, N, C, H, nullptr, f + oRt, nullptr, f + oh, f + ov, f + odn,
+                                            nullptr, nullptr, nullptr, f + odbx, f + odbr, f + odh, f + odp, f + odq,
+                                            zoneout_mask ? f + om : nullptr, false));
+      HASTE_HIP_PROPAGATE(transpose_to_half(stream, true, iTN, iH3, f + odp, f + at.dpT_half));
+      HASTE_HIP_PROPAGATE(transpose_to_half(stream, true, iTN, iH3, f + odq, f + at.dqT_half));
+      HASTE_HIP_PROPAGATE(gemm_half_nt(stream, true, iTN, C, iH3, f + odp, iH3, f + at.W_half, iH3, f + odx, C, false, 0));
+      HASTE_HIP_PROPAGATE(gemm_half_nt(stream, false, C, iH3, iTN, x_t, iTN, f + at.dpT_half, iTN, f + odW, iH3, true, 0));
+      HASTE_HIP_PROPAGATE(gemm_half_nt(stream, false, H, iH3, iTN, f + at.hT_half, iTN, f + at.dqT_half, iTN, f + odR,
+                                       iH3, true, 0));
+    }
+    ConvertList out;
+    out.add(f + odx, dx, TN * C);
+    out.add(f + odW, dW, C * H3);
+    out.add(f + odR, dR, H * H3);
+    out.add(f + odbx, dbx, H3);
+    out.add(f + odbr, dbr, H3);
+    out.add(f + odh, dh, NH);
+    return convert<false>(stream, out);
+  }
 
   ConvertList in;
   in.add(W_t, f + oWt, H3 * C);
@@ -232,7 +322,7 @@ int gru_backward_half(hipStream_t stream, int T, int N, int C, int H, const void
     ScratchPrefix keep(bytes);
     HASTE_HIP_PROPAGATE(gru_backward_impl(stream, T, N, C, H, f + oWt, f + oRt, f + oxt, f + oh, f + ov,
                                           f + odn, f + odx, f + odW, f + odR, f + odbx, f + odbr, f + odh,
-                                          f + odp, f + odq, zoneout_mask ? f + om : nullptr));
+                                          f + odp, f + odq, zoneout_mask ? f + om : nullptr, true));
   }
   ConvertList out;
   out.add(f + odx, dx, TN * C);
@@ -241,8 +331,6 @@ int gru_backward_half(hipStream_t stream, int T, int N, int C, int H, const void
   out.add(f + odbx, dbx, H3);
   out.add(f + odbr, dbr, H3);
   out.add(f + odh, dh, NH);
-  out.add(f + odp, dp, TN * H3);
-  out.add(f + odq, dq, TN * H3);
   return convert<false>(stream, out);
 }
 

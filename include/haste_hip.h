@@ -555,6 +555,15 @@ int haste_hip_layer_norm_indrnn_backward_f64(int steps, int batch_size, int inpu
 int haste_hip_gemm_f16(int trans_a, int M, int N, int K, const void* A, int lda, const void* B,
                        int ldb, void* C, int ldc, int accumulate, void* stream);
 int haste_hip_transpose_f16(int rows, int cols, const void* in, void* out, void* stream);
+/* C[M,N] (+)= A[M,K] * Bt[N,K]^T with fp32 accumulation and an fp32 result: the product kernel
+ * of the half GRU's passes over more than one step.  Bt holds IEEE binary16 values, A binary16
+ * or (a_is_float != 0) fp32 values that are rounded to half as they are read; both have the
+ * contraction index contiguous.  K, lda and ldb must be multiples of 8 (4 for an fp32 A) and
+ * the operands 16-byte aligned (HASTE_HIP_ERROR_UNSUPPORTED_SIZE otherwise).  No counterpart in
+ * the reference (cublasHgemm with a transposition flag); exported for tests and for callers
+ * that want the kernel by itself. */
+int haste_hip_gemm_half_nt(int a_is_float, int M, int N, int K, const void* A, int lda,
+                           const void* Bt, int ldb, float* C, int ldc, int accumulate, void* stream);
 int haste_hip_gru_forward_f16(int training, int steps, int batch_size, int input_size,
                               int hidden_size, const void* W, const void* R, const void* bx,
                               const void* br, const void* x, void* h, void* v, void* tmp_Wx,

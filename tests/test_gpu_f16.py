@@ -16,7 +16,9 @@ TOL16 = 2e-2
 # the last two: the persistent kernels' two-set and 16-row tiles; BASELINE configuration 2's shape
 # (shortened) with an unaligned batch
 SHAPES = [(3, 2, 3, 4), (4, 5, 7, 20), (6, 16, 32, 64), (8, 33, 48, 128), (3, 70, 24, 300),
-          (1, 5, 12, 40), (20, 63, 512, 512)]
+          (1, 5, 12, 40), (20, 63, 512, 512),
+          # sizes that are multiples of 8: the products run on the half matrix cores
+          (20, 64, 512, 512), (50, 8, 64, 264)]
 
 
 def dev16(a):
@@ -153,6 +155,41 @@ def test_f16_gru_with_a_lent_workspace():
             ops.set_workspace(None)
     for g, w in zip(got, want):
         assert torch.equal(g, w)
+
+
+@pytest.mark.parametrize("a_float", [False, True])
+@pytest.mark.parametrize("accumulate", [False, True])
+@pytest.mark.parametrize("M,N,K", [(1, 1, 8), (37, 53, 24), (128, 128, 64), (130, 257, 200), (300, 100, 1000),
+                                   (64, 1536, 512), (512, 200, 6400), (1000, 512, 1536)])
+def test_f16_gemm_nt(M, N, K, accumulate, a_float):
+    """The half GRU's product kernel, C (+)= A * Bt^T in fp32 from half operands (A also from
+    fp32, rounded as it is read), against numpy on the same half values: whole and ragged tiles,
+    tails of K, products cut along K."""
+    from haste_amd import lib as hlib
+    import torch
+    r = np.random.default_rng(M + 3 * N + 7 * K)
+    a = r.standard_normal((M, K))
+    bt = r.standard_normal((N, K))
+    c0 = r.standard_normal((M, N)).astype(np.float32)
+    # an fp32 A reaches half through float, as in the kernel
+    a16, bt16 = a.astype(np.float32).astype(np.float16), bt.astype(np.float16)
+    A = torch.from_numpy(a.astype(np.float32)).cuda() if a_float else torch.from_numpy(a16).cuda()
+    Bt = torch.from_numpy(bt16).cuda()
+    C = torch.from_numpy(c0).cuda()
+    hlib.call("haste_hip_gemm_half_nt", int(a_float), M, N, K, A, K, Bt, K, C, N, int(accumulate))
+    torch.cuda.synchronize()
+    ref = a16.astype(np.float64) @ bt16.astype(np.float64).T + (c0 if accumulate else 0.0)
+    assert relerr(host(C), ref) < 1e-5  # fp32 accumulation over up to 6400 terms
+
+
+def test_f16_gemm_nt_refuses_what_it_cannot_address():
+    from haste_amd import lib as hlib
+    import torch
+    A = torch.zeros(4, 12, dtype=torch.float16, device="cuda")
+    C = torch.zeros(4, 4, device="cuda")
+    with pytest.raises(hlib.HasteHipError) as e:
+        hlib.call("haste_hip_gemm_half_nt", 0, 4, 4, 12, A, 12, A, 12, C, 4, 0)  # K not a multiple of 8
+    assert e.value.code == 2
 
 
 def test_f16_lstm_is_refused():
