@@ -34,9 +34,11 @@ struct GruFwdParams {
 // which a single tile of 2*NB rows cannot do.
 // REG > 0 (tiles of 16 rows and more): the slice exceeds LDS; every wavefront keeps the first REG
 // k-groups of its share of the contraction in registers (tall_tile_product).
-template <int NB, int CT, int HS, int SETS, int REG = 0>
+// HALF (4-row tiles): the step's product on the half matrix cores, for widened half tensors.
+template <int NB, int CT, int HS, int SETS, int REG = 0, bool HALF = false>
 __global__ __launch_bounds__(256 * SETS, 1)
 void gru_forward_kernel(GruFwdParams p) {
+  static_assert(!HALF || (NB == 4 && REG == 0), "half product: 4-row tiles");
   static_assert(3 * HS <= 16 * CT, "slice too narrow");
   static_assert(SETS == 1 || (SETS == 2 && NB < 16), "two sets: short tiles only");
   static_assert(REG == 0 || (NB >= 16 && SETS == 1), "register-resident slice rows: tall tiles only");
@@ -172,7 +174,8 @@ void gru_forward_kernel(GruFwdParams p) {
       tile_product<NB, CT, false, true, false, NoSideWork, REG, float4_t[REG][CT]>(
           xhb, (t & 3) * tile_floats, Kpad, w_lds, red_t, &gs, nullptr, &breg);
     else
-      tile_product<NB, CT, false, true, kPolledPartials>(xhb, (t & 3) * tile_floats, Kpad, w_lds, red_t, &gs);
+      tile_product<NB, CT, false, true, kPolledPartials, NoSideWork, 0, NoResidentRows, HALF>(
+          xhb, (t & 3) * tile_floats, Kpad, w_lds, red_t, &gs);
     if constexpr (!kPolledPartials) __syncthreads();
 
     float saved[PP][4];  // z, r, g, q of the step for the caller's cache
@@ -769,11 +772,13 @@ bool gru_backward_resident(int N, int H) {
 
 // h: [N,H] state before the first step; h_out: [T,N,H] states after each step.
 // wx_ready (T > 1, gru_forward_resident): tmp_Wx already holds x*W, and W and x are not looked at.
+// half_product: the tensors are widened half tensors (gru_half.hip); with 4-row tiles the step's
+// product h * R goes to the half matrix cores (h rounded to half there, as such a cell stores it).
 int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int H,
                      const float* W, const float* R, const float* bx, const float* br,
                      const float* x, const float* h, float* h_out, float* v, float* tmp_Wx,
                      float zoneout_prob, const float* zoneout_mask, const float* dc_mask,
-                     float dc_scale, bool wx_ready) {
+                     float dc_scale, bool wx_ready, bool half_product) {
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
   HASTE_HIP_REQUIRE(R && bx && br && h && h_out && tmp_Wx && (wx_ready || (W && x)));
   HASTE_HIP_REQUIRE(!training || v != nullptr);
@@ -827,6 +832,9 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
 #undef HASTE_LAUNCH_FWD_RESIDENT
   if (tile.reg_groups > 0) return HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
 #define HASTE_LAUNCH_FWD_PAIRED(CT_, HS_)                                                     \
+  if (paired && tile.hs == HS_ && half_product)                                               \
+    return launch_persistent("gru_forward_recurrence", gru_forward_kernel<4, CT_, HS_, 2, 0, true>, \
+                             plan, p, stream);                                                \
   if (paired && tile.hs == HS_)                                                               \
     return launch_persistent("gru_forward_recurrence", gru_forward_kernel<4, CT_, HS_, 2>,    \
                              plan, p, stream);
@@ -836,6 +844,12 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
   if (tile.nb == NB_ && tile.hs == HS_)                                                       \
     return launch_persistent("gru_forward_recurrence", gru_forward_kernel<NB_, CT_, HS_, 1>,  \
                              plan, p, stream);
+#define HASTE_LAUNCH_FWD_HALF(CT_, HS_)                                                             \
+  if (half_product && tile.nb == 4 && tile.hs == HS_)                                               \
+    return launch_persistent("gru_forward_recurrence", gru_forward_kernel<4, CT_, HS_, 1, 0, true>, \
+                             plan, p, stream);
+  HASTE_LAUNCH_FWD_HALF(1, 4) HASTE_LAUNCH_FWD_HALF(2, 8) HASTE_LAUNCH_FWD_HALF(3, 16)
+#undef HASTE_LAUNCH_FWD_HALF
   HASTE_LAUNCH_FWD(4, 1, 4) HASTE_LAUNCH_FWD(4, 2, 8) HASTE_LAUNCH_FWD(4, 3, 16)
   HASTE_LAUNCH_FWD(8, 1, 4) HASTE_LAUNCH_FWD(8, 2, 8) HASTE_LAUNCH_FWD(8, 3, 16)
   HASTE_LAUNCH_FWD(16, 1, 4) HASTE_LAUNCH_FWD(16, 2, 8) HASTE_LAUNCH_FWD(16, 3, 16)
@@ -847,11 +861,13 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
 
 // products == false (gru_backward_resident): the recurrence only -- dp, dq, dbx, dbr, dh; the
 // caller computes dx, dW and dR from dp and dq itself, and W_t, x_t, dx, dW, dR are not looked at.
+// half_product: the tensors are widened half tensors (gru_half.hip); where the scattered form
+// runs, its product dh = (gate gradients) * R_t goes to the half matrix cores.
 int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
                       const float* W_t, const float* R_t, const float* x_t, const float* h,
                       const float* v, const float* dh_next, float* dx, float* dW, float* dR,
                       float* dbx, float* dbr, float* dh, float* dp, float* dq,
-                      const float* zoneout_mask, bool products) {
+                      const float* zoneout_mask, bool products, bool half_product) {
   HASTE_HIP_REQUIRE(T > 0 && N > 0 && C > 0 && H > 0);
   HASTE_HIP_REQUIRE(R_t && h && v && dh_next && (!products || (W_t && x_t)));
   HASTE_HIP_REQUIRE(dbx && dbr && dh && dp && dq && (!products || (dx && dW && dR)));
@@ -897,7 +913,8 @@ int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
   if (paired) plan.threads = 512;
   int rc = HASTE_HIP_ERROR_UNSUPPORTED_SIZE;
   const char* name = "gru_backward_recurrence";
-  if (scatter) rc = launch_scatter_backward<GruScatterCell>(name, H, sets, plan, p, stream);
+  if (scatter && half_product) rc = launch_scatter_backward<GruScatterCell, true>(name, H, sets, plan, p, stream);
+  else if (scatter) rc = launch_scatter_backward<GruScatterCell>(name, H, sets, plan, p, stream);
   else
 #define HASTE_LAUNCH_BWD_RESIDENT(NB_)                                                           \
   (tile.reg_groups == 8    ? launch_persistent(name, gru_backward_kernel<NB_, 1, 8>, plan, p, stream)  \
@@ -941,7 +958,7 @@ int haste_hip_gru_forward_f32(int training, int steps, int batch_size, int input
   return haste_hip::gru_forward_impl(haste_hip::as_stream(stream), training, steps, batch_size,
                                      input_size, hidden_size, W, R, bx, br, x, h,
                                      h + (size_t)batch_size * hidden_size, v, tmp_Wx,
-                                     zoneout_prob, zoneout_mask, nullptr, 1.0f, false);
+                                     zoneout_prob, zoneout_mask, nullptr, 1.0f, false, false);
 }
 
 int haste_hip_gru_forward_dropconnect_f32(int training, int steps, int batch_size,
@@ -957,7 +974,7 @@ int haste_hip_gru_forward_dropconnect_f32(int training, int steps, int batch_siz
                                      input_size, hidden_size, W, R, bx, br, x, h,
                                      h + (size_t)batch_size * hidden_size, v, tmp_Wx,
                                      zoneout_prob, zoneout_mask, dropconnect_mask,
-                                     dropconnect_scale, false);
+                                     dropconnect_scale, false, false);
 }
 
 int haste_hip_gru_backward_f32(int steps, int batch_size, int input_size, int hidden_size,
@@ -972,7 +989,7 @@ int haste_hip_gru_backward_f32(int steps, int batch_size, int input_size, int hi
   return haste_hip::gru_backward_impl(haste_hip::as_stream(stream), steps, batch_size, input_size,
                                       hidden_size, W_t, R_t, x_t, h, v,
                                       dh_new + (size_t)batch_size * hidden_size, dx, dW, dR, dbx,
-                                      dbr, dh, dp, dq, zoneout_mask, true);
+                                      dbr, dh, dp, dq, zoneout_mask, true, false);
 }
 
 int haste_hip_gru_forward_iterate_f32(int training, int batch_size, int input_size,
@@ -985,7 +1002,7 @@ int haste_hip_gru_forward_iterate_f32(int training, int batch_size, int input_si
   (void)tmp_Rh;
   return haste_hip::gru_forward_impl(haste_hip::as_stream(stream), training, 1, batch_size,
                                      input_size, hidden_size, W, R, bx, br, x, h, h_out, v, tmp_Wx,
-                                     zoneout_prob, zoneout_mask, nullptr, 1.0f, false);
+                                     zoneout_prob, zoneout_mask, nullptr, 1.0f, false, false);
 }
 
 int haste_hip_gru_backward_iterate_f32(int batch_size, int input_size, int hidden_size,
@@ -998,7 +1015,7 @@ int haste_hip_gru_backward_iterate_f32(int batch_size, int input_size, int hidde
   (void)br;
   return haste_hip::gru_backward_impl(haste_hip::as_stream(stream), 1, batch_size, input_size,
                                       hidden_size, W_t, R_t, x_t, h, v, dh_new, dx, dW, dR, dbx,
-                                      dbr, dh, dp, dq, zoneout_mask, true);
+                                      dbr, dh, dp, dq, zoneout_mask, true, false);
 }
 
 }  // extern "C"

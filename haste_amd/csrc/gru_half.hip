@@ -23,12 +23,12 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
                      const float* W, const float* R, const float* bx, const float* br,
                      const float* x, const float* h, float* h_out, float* v, float* tmp_Wx,
                      float zoneout_prob, const float* zoneout_mask, const float* dc_mask,
-                     float dc_scale, bool wx_ready);
+                     float dc_scale, bool wx_ready, bool half_product);
 int gru_backward_impl(hipStream_t stream, int T, int N, int C, int H,
                       const float* W_t, const float* R_t, const float* x_t, const float* h,
                       const float* v, const float* dh_next, float* dx, float* dW, float* dR,
                       float* dbx, float* dbr, float* dh, float* dp, float* dq,
-                      const float* zoneout_mask, bool products);
+                      const float* zoneout_mask, bool products, bool half_product);
 bool gru_forward_resident(int N, int H);
 bool gru_backward_resident(int N, int H);
 // gemm_half_nt.hip
@@ -212,7 +212,7 @@ int gru_forward_half(hipStream_t stream, int training, int T, int N, int C, int 
       HASTE_HIP_PROPAGATE(gru_forward_impl(stream, training, T, N, C, H, nullptr, f + oR, f + obx, f + obr, nullptr,
                                            f + oh, f + oh + NH, training ? f + ov : nullptr, f + oWx, zoneout_prob,
                                            zoneout_mask ? f + om : nullptr, dc_mask ? f + od : nullptr, dc_scale,
-                                           true));
+                                           true, true));
     }
     ConvertList out;
     out.add(f + oh + NH, static_cast<half_t*>(h) + NH, TN * H);
@@ -235,7 +235,7 @@ int gru_forward_half(hipStream_t stream, int training, int T, int N, int C, int 
     HASTE_HIP_PROPAGATE(gru_forward_impl(stream, training, T, N, C, H, f + oW, f + oR, f + obx, f + obr,
                                          f + ox, f + oh, f + oh + NH, training ? f + ov : nullptr, f + oWx,
                                          zoneout_prob, zoneout_mask ? f + om : nullptr,
-                                         dc_mask ? f + od : nullptr, dc_scale, false));
+                                         dc_mask ? f + od : nullptr, dc_scale, false, true));
   }
   ConvertList out;
   out.add(f + oh + NH, static_cast<half_t*>(h) + NH, TN * H);
@@ -286,7 +286,7 @@ int gru_backward_half(hipStream_t stream, int T, int N, int C, int H, const void
       ScratchPrefix keep(bytes);
       HASTE_HIP_PROPAGATE(gru_backward_impl(stream, T, N, C, H, nullptr, f + oRt, nullptr, f + oh, f + ov, f + odn,
                                             nullptr, nullptr, nullptr, f + odbx, f + odbr, f + odh, f + odp, f + odq,
-                                            zoneout_mask ? f + om : nullptr, false));
+                                            zoneout_mask ? f + om : nullptr, false, true));
       HASTE_HIP_PROPAGATE(transpose_to_half(stream, true, iTN, iH3, f + odp, f + at.dpT_half));
       HASTE_HIP_PROPAGATE(transpose_to_half(stream, true, iTN, iH3, f + odq, f + at.dqT_half));
       HASTE_HIP_PROPAGATE(gemm_half_nt(stream, true, iTN, C, iH3, f + odp, iH3, f + at.W_half, iH3, f + odx, C, false, 0));
@@ -322,7 +322,7 @@ int gru_backward_half(hipStream_t stream, int T, int N, int C, int H, const void
     ScratchPrefix keep(bytes);
     HASTE_HIP_PROPAGATE(gru_backward_impl(stream, T, N, C, H, f + oWt, f + oRt, f + oxt, f + oh, f + ov,
                                           f + odn, f + odx, f + odW, f + odR, f + odbx, f + odbr, f + odh,
-                                          f + odp, f + odq, zoneout_mask ? f + om : nullptr, true));
+                                          f + odp, f + odq, zoneout_mask ? f + om : nullptr, true, true));
   }
   ConvertList out;
   out.add(f + odx, dx, TN * C);

@@ -22,6 +22,7 @@
 namespace haste_hip {
 
 typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 
 
 // Gate nonlinearities on the hardware exp2 and reciprocal (about 1 ulp each): absolute
@@ -790,7 +791,10 @@ __device__ __forceinline__ void load_tile_rows4(const TileBuffer& xb, int tile_o
 // Consecutive MFMAs on one output tile alternate between two accumulators.
 constexpr int kLdsAhead = 3;
 
-template <int RB, int CT, int CH>
+// HALF: on the half matrix cores -- the four k of an operand register are the four k of one
+// v_mfma_f32_4x4x4_16B_f16 (both operands rounded to half: a cell whose tensors are half),
+// one MFMA where the fp32 form issues four.
+template <int RB, int CT, int CH, bool HALF = false>
 __device__ __forceinline__ void mfma_tile_rows4(const float* w_lds, int s,
                                                 const float4_t (&av)[CH][RB],
                                                 float4_t (&acc0)[RB][ShortTileShape<CT>::CTN],
@@ -810,6 +814,15 @@ __device__ __forceinline__ void mfma_tile_rows4(const float* w_lds, int s,
     for (int ct = 0; ct < S::CTN; ++ct)
       b[I][ct] = *reinterpret_cast<const float4_t*>(wp + step_offset(I) + ct * S::MC * 4);
   });
+  half4_t ah[HALF ? CH : 1][RB];
+  if constexpr (HALF) {
+#pragma unroll
+    for (int ci = 0; ci < CH; ++ci)
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ah[ci][rb][e] = (_Float16)av[ci][rb][e];
+  }
   static_for<STEPS>([&](auto ic) {
     constexpr int I = decltype(ic)::value;
     constexpr int A = I % S::NBC;
@@ -821,6 +834,22 @@ __device__ __forceinline__ void mfma_tile_rows4(const float* w_lds, int s,
             wp + step_offset(I + kLdsAhead) + ct * S::MC * 4);
       // keep the read here: the scheduler would otherwise sink it to just before its use
       __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (HALF) {
+#pragma unroll
+      for (int ct = 0; ct < S::CTN; ++ct) {
+        half4_t bh;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) bh[e] = (_Float16)b[I][ct][e];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+          if constexpr (I % 2 == 0)
+            acc0[rb][ct] = __builtin_amdgcn_mfma_f32_4x4x4f16(ah[CI][rb], bh, acc0[rb][ct], S::CBSZ, A, 0);
+          else
+            acc1[rb][ct] = __builtin_amdgcn_mfma_f32_4x4x4f16(ah[CI][rb], bh, acc1[rb][ct], S::CBSZ, A, 0);
+        }
+      }
+      return;
     }
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
@@ -968,7 +997,7 @@ struct InputProjection {
 // register buffers alternate so that nothing is copied.  The four wavefronts are those of one
 // 256-thread set of the workgroup.  TAGGED: the partial tiles are themselves polled by their
 // readers (take_product), so no element may carry the "unwritten" pattern.
-template <int RB, int CT, int CH, bool POLLED, bool TAGGED = false, class Side = NoSideWork>
+template <int RB, int CT, int CH, bool POLLED, bool TAGGED = false, class Side = NoSideWork, bool HALF = false>
 __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int tile_off, int Kpad,
                                                        const float* w_lds, float* red,
                                                        const GroupSync* gs, Side* side = nullptr) {
@@ -1021,14 +1050,14 @@ __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int
       if constexpr (POLLED)
         poll_until_written(*gs, [&] { load_tile_rows4<RB, CT, CH>(xb, tile_off, s, buf0); },
                            [&] { return all_written(buf0); });
-      mfma_tile_rows4<RB, CT, CH>(w_lds, s, buf0, acc0, acc1);
+      mfma_tile_rows4<RB, CT, CH, HALF>(w_lds, s, buf0, acc0, acc1);
       s += 4 * CH;
       if (++c == chunks) break;
       if (c + 1 < chunks) load_tile_rows4<RB, CT, CH>(xb, tile_off, s + 4 * CH, buf0);
       if constexpr (POLLED)
         poll_until_written(*gs, [&] { load_tile_rows4<RB, CT, CH>(xb, tile_off, s, buf1); },
                            [&] { return all_written(buf1); });
-      mfma_tile_rows4<RB, CT, CH>(w_lds, s, buf1, acc0, acc1);
+      mfma_tile_rows4<RB, CT, CH, HALF>(w_lds, s, buf1, acc0, acc1);
       s += 4 * CH;
       if (++c == chunks) break;
     }
@@ -1039,7 +1068,7 @@ __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int
     if constexpr (POLLED)
       poll_until_written(*gs, [&] { load_tile_rows4<RB, CT, 1>(xb, tile_off, s, one); },
                          [&] { return all_written(one); });
-    mfma_tile_rows4<RB, CT, 1>(w_lds, s, one, acc0, acc1);
+    mfma_tile_rows4<RB, CT, 1, HALF>(w_lds, s, one, acc0, acc1);
   }
 
   // The KS lane groups hold partial sums of the same elements: they are added here, so that a
@@ -1082,16 +1111,17 @@ __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int
 // wait; otherwise the caller has waited at the group's step barrier and `gs` is unused.
 // REG > 0 (tall tiles): the slice is split between registers and LDS, see tall_tile_product.
 template <int NB, int CT, bool LONG_K, bool POLLED = false, bool TAGGED = false, class Side = NoSideWork,
-          int REG = 0, class Resident = NoResidentRows>
+          int REG = 0, class Resident = NoResidentRows, bool HALF = false>
 __device__ __forceinline__ void tile_product(const TileBuffer& xb, int tile_off, int Kpad,
                                              const float* w_lds, float* red,
                                              const GroupSync* gs = nullptr, Side* side = nullptr,
                                              const Resident* breg = nullptr) {
   if constexpr (ProductTile<NB, CT>::kShort) {
     static_assert(REG == 0, "register-resident slice rows exist for tall tiles only");
-    short_exchange_product<NB / 4, CT, LONG_K ? 4 : 2, POLLED, TAGGED, Side>(xb, tile_off, Kpad, w_lds,
-                                                                              red, gs, side);
+    short_exchange_product<NB / 4, CT, LONG_K ? 4 : 2, POLLED, TAGGED, Side, HALF>(xb, tile_off, Kpad, w_lds,
+                                                                                    red, gs, side);
   } else {
+    static_assert(!HALF, "the product on the half matrix cores exists for short tiles only");
     static_assert(!TAGGED, "polled partial tiles exist for short tiles only");
     static_assert(Side::kBatches == 0, "side work exists for short tiles only");
     constexpr int RT = NB / 16;
@@ -1378,6 +1408,26 @@ __device__ __forceinline__ void scatter_product(const float4_t& a, const float (
 #pragma unroll
       for (int ct = 0; ct < CTN; ++ct)
         acc[c & 1][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(a[c], w[A][c][ct], acc[c & 1][ct], 4, A, 0);
+  });
+}
+
+// The same product on the half matrix cores (a cell whose tensors are half: the gate gradients
+// are rounded to half, as such a cell stores them, and the weights are exact in half): the G
+// gate gradients of an element are the four k of one v_mfma_f32_4x4x4_16B_f16, so a unit takes
+// one MFMA per column tile instead of G -- 16 * CTN in all.  w[block][ct]: the lane's weights of
+// the block's unit for gates 0 .. 3 (zero beyond G).
+
+template <int G, int CTN>
+__device__ __forceinline__ void scatter_product_half(const float4_t& a, const half4_t (&w)[16][CTN],
+                                                     float4_t (&acc)[2][CTN]) {
+  half4_t ah;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) ah[c] = c < G ? (_Float16)a[c] : (_Float16)0.f;
+  static_for<16>([&](auto bc) {
+    constexpr int A = decltype(bc)::value;
+#pragma unroll
+    for (int ct = 0; ct < CTN; ++ct)
+      acc[A & 1][ct] = __builtin_amdgcn_mfma_f32_4x4x4f16(ah, w[A][ct], acc[A & 1][ct], 4, A, 0);
   });
 }
 

@@ -36,7 +36,9 @@ namespace haste_hip {
 //   add_gathered(sum)      dh of the next step = what step() kept + the gathered sums
 //   store_copy(p, t, row, unit, a)   the caller's copy of the gate gradients
 //   add_sums(p, col, s)    column sum `col` (of kSums*H) of the whole batch
-template <class Cell, int CTN, int SETS>
+// HALF: the product runs on the half matrix cores (scatter_product_half), for cells whose
+// tensors are half; everything else of the step stays in fp32.
+template <class Cell, int CTN, int SETS, bool HALF = false>
 __global__ __launch_bounds__(256 * SETS, 1)
 void scatter_backward_kernel(typename Cell::Params p) {
   using S = ScatterShape<CTN>;
@@ -86,17 +88,21 @@ void scatter_backward_kernel(typename Cell::Params p) {
   const TileBuffer xpb = make_tile_buffer(xp, kScatterTiles * tile_floats);
 
   // The wavefront's weights: rows (gate c, unit j0 + a) of R_t, columns (wave*CTN + ct)*64 + lane.
-  float wreg[16][G][CTN];
+  float wreg[HALF ? 1 : 16][G][CTN];
+  half4_t whalf[HALF ? 16 : 1][CTN];
 #pragma unroll
   for (int a = 0; a < 16; ++a)
 #pragma unroll
-    for (int c = 0; c < G; ++c)
+    for (int c = 0; c < 4; ++c)
 #pragma unroll
       for (int ct = 0; ct < CTN; ++ct) {
         const int unit = j0 + a, col = (wave * CTN + ct) * 64 + lane;
-        const bool ok = unit < H && col < H;
-        const float x = p.R_t[ok ? ((size_t)c * H + unit) * H + col : 0];
-        wreg[a][c][ct] = ok ? x : 0.f;
+        const bool ok = c < G && unit < H && col < H;
+        if (c < G || HALF) {
+          const float x = p.R_t[ok ? ((size_t)c * H + unit) * H + col : 0];
+          if constexpr (HALF) whalf[a][ct][c] = (_Float16)(ok ? x : 0.f);
+          else wreg[a][c < G ? c : 0][ct] = ok ? x : 0.f;
+        }
       }
 
   // The pieces this lane publishes: columns (wave*CTN + ct)*64 + lane belong to owner col/16,
@@ -239,7 +245,8 @@ void scatter_backward_kernel(typename Cell::Params p) {
       for (int c = 0; c < 2; ++c)
 #pragma unroll
         for (int ct = 0; ct < CTN; ++ct) acc[c][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
-      scatter_product<G, CTN>(a, wreg, acc);
+      if constexpr (HALF) scatter_product_half<G, CTN>(a, whalf, acc);
+      else scatter_product<G, CTN>(a, wreg, acc);
       float* tile_pub = xp + (size_t)(d & 1) * tile_floats;
       const unsigned int tag = scatter_tag(d);
 #pragma unroll
@@ -286,14 +293,14 @@ void scatter_backward_kernel(typename Cell::Params p) {
 
 
 // Launches the kernel for `sets` sets per workgroup and hidden size H <= 512.
-template <class Cell>
+template <class Cell, bool HALF = false>
 int launch_scatter_backward(const char* name, int H, int sets, const LaunchPlan& plan, typename Cell::Params& p,
                             hipStream_t stream) {
   if (H <= 256)
-    return sets == 2 ? launch_persistent(name, scatter_backward_kernel<Cell, 1, 2>, plan, p, stream)
-                     : launch_persistent(name, scatter_backward_kernel<Cell, 1, 1>, plan, p, stream);
-  return sets == 2 ? launch_persistent(name, scatter_backward_kernel<Cell, 2, 2>, plan, p, stream)
-                   : launch_persistent(name, scatter_backward_kernel<Cell, 2, 1>, plan, p, stream);
+    return sets == 2 ? launch_persistent(name, scatter_backward_kernel<Cell, 1, 2, HALF>, plan, p, stream)
+                     : launch_persistent(name, scatter_backward_kernel<Cell, 1, 1, HALF>, plan, p, stream);
+  return sets == 2 ? launch_persistent(name, scatter_backward_kernel<Cell, 2, 2, HALF>, plan, p, stream)
+                   : launch_persistent(name, scatter_backward_kernel<Cell, 2, 1, HALF>, plan, p, stream);
 }
 
 }  // namespace haste_hip
