@@ -16,7 +16,7 @@
 // [k = 8*(lane/32) .. +7], b = Bt[j = lane%32][the same k], d[e] = D[i = 8*(e/4) + 4*(lane/32) +
 // e%4][j = lane%32].
 //
-// A product with fewer tiles than two per CU is cut along K into pieces (each at least 256 k)
+// A product with fewer tiles than three quarters of the CUs is cut along K into pieces (each at least 256 k)
 // that park [M][N] partial results in the stream's scratch buffer; a second kernel adds them in
 // index order.  The cut depends on the shape only: results are reproducible.
 #include "common.h"
@@ -71,32 +71,53 @@ void gemm_half_nt_kernel(int M, int N, int K, const void* __restrict__ A, int ld
       panel(static_cast<const char*>(A) + (size_t)m0 * lda * ASZ, ((long long)(rows_a - 1) * lda + K) * ASZ);
   const __amdgpu_buffer_rsrc_t pb = panel(Bt + (size_t)n0 * ldb, ((long long)(rows_b - 1) * ldb + K) * 2);
 
-  // A thread's four chunks of each tile: chunk c = tid % 8 of rows tid / 8 + 32 * i.
+  // A thread's four chunks of each tile: chunk c = tid % 8 of rows tid / 8 + 32 * i.  Two
+  // steps of operands are kept in flight in two register sets (a step's 512 cycles of MFMAs
+  // are a fraction of a load's latency).  An fp32 A stays as loaded until it is parked:
+  // converted at the request it would make the request wait for its own loads.
   const int c = tid & 7, r = tid >> 3;
-  uint4_t ra[4], rb[4];
-  auto request = [&](int k0) {
-    const bool in_k = k0 + 8 * c < k_end;
+  constexpr int AR = A_FLOAT ? 8 : 4;
+  uint4_t ra[2][AR], rb[2][4];
+  // A thread's offsets into the panels are fixed; the step enters as the loads' scalar offset
+  // (which the range check ignores: chunks beyond the end of K, in the last step of a ragged K
+  // only, get an offset beyond the panel instead).  The offsets pass through an empty asm
+  // statement: left to see the select, the compiler puts every load behind a branch of its own
+  // and a wait for all loads before it (8192^3: 565 -> 814 TFLOP/s without them).  Loads issued
+  // straight from the fixed offsets, with nothing between them, are slower again (783): more
+  // loads in flight are not what the step lacks.
+  unsigned int va[4], vb[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    va[i] = (unsigned int)(((size_t)(r + 32 * i) * lda + 8 * c) * ASZ);
+    vb[i] = (unsigned int)(((size_t)(r + 32 * i) * ldb + 8 * c) * 2);
+  }
+  auto request = [&](auto set_c, int k0) {
+    constexpr int SET = decltype(set_c)::value;
+    const int sa = k0 * ASZ, sb = k0 * 2;
+    const bool gone = k0 + 8 * c >= k_end;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int row = r + 32 * i;
+      unsigned int oa = gone ? kNowhere : va[i], ob = gone ? kNowhere : vb[i];
+      asm volatile("" : "+v"(oa), "+v"(ob));
       if constexpr (A_FLOAT) {
-        const unsigned int off = in_k ? (unsigned int)(((size_t)row * lda + k0 + 8 * c) * 4) : kNowhere;
-        const uint4_t lo = __builtin_amdgcn_raw_buffer_load_b128(pa, off, 0, 0);
-        const uint4_t hi = __builtin_amdgcn_raw_buffer_load_b128(pa, in_k ? off + 16 : kNowhere, 0, 0);
-        ra[i] = pack8(__builtin_bit_cast(float4_t, lo), __builtin_bit_cast(float4_t, hi));
+        ra[SET][2 * i] = __builtin_amdgcn_raw_buffer_load_b128(pa, oa, sa, 0);
+        ra[SET][2 * i + 1] = __builtin_amdgcn_raw_buffer_load_b128(pa, oa + 16, sa, 0);
       } else {
-        const unsigned int off = in_k ? (unsigned int)(((size_t)row * lda + k0 + 8 * c) * 2) : kNowhere;
-        ra[i] = __builtin_amdgcn_raw_buffer_load_b128(pa, off, 0, 0);
+        ra[SET][i] = __builtin_amdgcn_raw_buffer_load_b128(pa, oa, sa, 0);
       }
-      const unsigned int offb = in_k ? (unsigned int)(((size_t)row * ldb + k0 + 8 * c) * 2) : kNowhere;
-      rb[i] = __builtin_amdgcn_raw_buffer_load_b128(pb, offb, 0, 0);
+      rb[SET][i] = __builtin_amdgcn_raw_buffer_load_b128(pb, ob, sb, 0);
     }
   };
-  auto park = [&](int buf) {
+  auto park = [&](auto set_c) {
+    constexpr int SET = decltype(set_c)::value;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      lds[buf][0][lds_chunk(r + 32 * i, c)] = ra[i];
-      lds[buf][1][lds_chunk(r + 32 * i, c)] = rb[i];
+      if constexpr (A_FLOAT)
+        lds[SET][0][lds_chunk(r + 32 * i, c)] = pack8(__builtin_bit_cast(float4_t, ra[SET][2 * i]),
+                                                      __builtin_bit_cast(float4_t, ra[SET][2 * i + 1]));
+      else
+        lds[SET][0][lds_chunk(r + 32 * i, c)] = ra[SET][i];
+      lds[SET][1][lds_chunk(r + 32 * i, c)] = rb[SET][i];
     }
   };
 
@@ -108,32 +129,42 @@ void gemm_half_nt_kernel(int M, int N, int K, const void* __restrict__ A, int ld
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  if (k_begin < k_end) {
-    request(k_begin);
-    park(0);
-    __syncthreads();
-    int buf = 0;
-    for (int k0 = k_begin; k0 < k_end; k0 += QK) {
-      const bool more = k0 + QK < k_end;
-      if (more) request(k0 + QK);
+  auto compute = [&](int buf) {
 #pragma unroll
-      for (int ks = 0; ks < QK / 16; ++ks) {
-        const int cc = 2 * ks + (lane >> 5), o = lane & 31;
-        half8_t a[2], b[2];
+    for (int ks = 0; ks < QK / 16; ++ks) {
+      const int cc = 2 * ks + (lane >> 5), o = lane & 31;
+      half8_t a[2], b[2];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          a[i] = __builtin_bit_cast(half8_t, lds[buf][0][lds_chunk(wm + 32 * i + o, cc)]);
-          b[i] = __builtin_bit_cast(half8_t, lds[buf][1][lds_chunk(wn + 32 * i + o, cc)]);
-        }
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int j = 0; j < 2; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+      for (int i = 0; i < 2; ++i) {
+        a[i] = __builtin_bit_cast(half8_t, lds[buf][0][lds_chunk(wm + 32 * i + o, cc)]);
+        b[i] = __builtin_bit_cast(half8_t, lds[buf][1][lds_chunk(wn + 32 * i + o, cc)]);
       }
-      if (more) park(buf ^ 1);
-      __syncthreads();
-      buf ^= 1;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+  };
+  // step at k0 from LDS buffer / register set CUR: request the step after the next one into the
+  // set this step was parked from, multiply, park the next step (its loads were issued a step ago)
+  auto step = [&](auto cur_c, int k0) {
+    constexpr int CUR = decltype(cur_c)::value;
+    if (k0 + 2 * QK < k_end) request(cur_c, k0 + 2 * QK);
+    compute(CUR);
+    if (k0 + QK < k_end) park(std::integral_constant<int, 1 - CUR>{});
+    __syncthreads();
+  };
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
+  if (k_begin < k_end) {
+    request(Set0{}, k_begin);
+    if (k_begin + QK < k_end) request(Set1{}, k_begin + QK);
+    park(Set0{});
+    __syncthreads();
+    for (int k0 = k_begin; k0 < k_end; k0 += 2 * QK) {
+      step(Set0{}, k0);
+      if (k0 + QK < k_end) step(Set1{}, k0 + QK);
     }
   }
 
@@ -176,8 +207,12 @@ void plan_half_nt(int M, int N, int K, int* pieces, int* k_per_piece) {
   const long long tiles = (long long)((M + QM - 1) / QM) * ((N + QN - 1) / QN);
   const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
   int s = 1;
-  if (tiles < 2LL * cus) {
-    s = (int)((2LL * cus + tiles - 1) / tiles);
+  // three quarters of a workgroup per CU: at the shapes of a GRU step with N = 64, T = 100,
+  // C = H = 512, two per CU costs dx (200 tiles) 47 us in three pieces against 32 us whole, and
+  // dW, dR (48 tiles) as much in ten pieces as in four
+  const long long want = (long long)cus * 3 / 4;
+  if (tiles < want) {
+    s = (int)((want + tiles - 1) / tiles);
     const int most = K / 256;
     s = s < most ? s : most;
     s = s > 1 ? s : 1;
