@@ -18,7 +18,9 @@ TOL16 = 2e-2
 SHAPES = [(3, 2, 3, 4), (4, 5, 7, 20), (6, 16, 32, 64), (8, 33, 48, 128), (3, 70, 24, 300),
           (1, 5, 12, 40), (20, 63, 512, 512),
           # sizes that are multiples of 8: the products run on the half matrix cores
-          (20, 64, 512, 512), (50, 8, 64, 264), (40, 1, 16, 64)]
+          (20, 64, 512, 512), (50, 8, 64, 264), (40, 1, 16, 64),
+          # long sequences: on the half matrix cores, and ragged (fp32 on widened tensors)
+          (100, 16, 32, 128), (101, 7, 24, 100)]
 
 
 def dev16(a):
