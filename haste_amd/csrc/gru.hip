@@ -18,7 +18,10 @@ struct GruFwdParams {
   const float* h;        // [N,H] state before the first step
   float* h_out;          // [T,N,H] states after each step (may start at h + N*H)
   float* v;              // [T,N,4H] (training) or null
-  const float* Wx;       // [T,N,3H] = x*W
+  const float* Wx;       // [T,N,3H] = x*W (kernels that compute the input projection themselves: unused)
+  const float* W;        // [C,3H] and
+  const float* x;        // [T,N,C], for those kernels
+  int C;
   float zoneout_prob;
   const float* zoneout_mask;
   const float* dc_mask;  // DropConnect mask [H,3H] or null
@@ -35,16 +38,24 @@ struct GruFwdParams {
 // REG > 0 (tiles of 16 rows and more): the slice exceeds LDS; every wavefront keeps the first REG
 // k-groups of its share of the contraction in registers (tall_tile_product).
 // HALF (4-row tiles): the step's product on the half matrix cores, for widened half tensors.
-template <int NB, int CT, int HS, int SETS, int REG = 0, bool HALF = false>
+// XSG > 0 (4-row tiles, 16 units per workgroup): the kernel also computes the input projection
+// x[t] * W beside its waits (see InputProjection): the z and r columns into the accumulators of
+// the recurrent product, the candidate gate's -- which needs x*W and h*R apart -- into a tile of
+// its own, which rides behind the slice's three in the partial tiles (rows of 64 columns).
+template <int NB, int CT, int HS, int SETS, int REG = 0, bool HALF = false, int XSG = 0>
 __global__ __launch_bounds__(256 * SETS, 1)
 void gru_forward_kernel(GruFwdParams p) {
   static_assert(!HALF || (NB == 4 && REG == 0), "half product: 4-row tiles");
+  constexpr bool kFusedInput = XSG > 0;
+  static_assert(!kFusedInput || (NB == 4 && CT == 3 && HS == 16 && REG == 0 && !HALF), "fused input projection");
+  constexpr int RCT = kFusedInput ? 4 : CT;  // column tiles of a partial tile's rows
+  constexpr int NG = kFusedInput ? 4 : 3;    // sums per element: z, r, h*R of g (, x*W of g)
   static_assert(3 * HS <= 16 * CT, "slice too narrow");
   static_assert(SETS == 1 || (SETS == 2 && NB < 16), "two sets: short tiles only");
   static_assert(REG == 0 || (NB >= 16 && SETS == 1), "register-resident slice rows: tall tiles only");
   constexpr int NCOLS = 16 * CT;
   constexpr int PP = (NB * HS + 255) / 256;
-  constexpr int RED = ProductTile<NB, CT>::kRedFloats;
+  constexpr int RED = ProductTile<NB, RCT>::kRedFloats;
   constexpr bool kPolledPartials = SETS == 2;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int H = p.H, N = p.N, T = p.T;
@@ -77,6 +88,19 @@ void gru_forward_kernel(GruFwdParams p) {
   // k beyond the problem stay zero for the whole launch.
   zero_tile_share<SETS>(gs, xh, tile_floats, NB, j0 / 4,
                         (role.cw == p.ls.gx - 1 ? Kpad - j0 : HS) / 4, kPolledTiles);
+
+  // The wavefront's share of W, in registers (requested before the slice, whose loads then
+  // overlap with these).
+  using Projection = std::conditional_t<kFusedInput, InputProjection<CT, kFusedInput ? XSG : 1, true>, NoSideWork>;
+  Projection proj;
+  if constexpr (kFusedInput) {
+    proj.setup(p.W, p.x, p.C, N, 3 * H, set_wave<SETS>(), n0 < N ? n0 : N - 1, [=](int col) {
+      const int gate = col / HS, j = j0 + col % HS;
+      return j < H ? (long long)gate * H + j : -1ll;
+    });
+    proj.request();
+    proj.settle();
+  }
 
   float4_t breg[REG > 0 ? REG : 1][CT];
   {
@@ -130,7 +154,7 @@ void gru_forward_kernel(GruFwdParams p) {
       store_exchanged(gs, e, publishable(h_prev[pp]));
       for (int b = 1; b < kPolledTiles; ++b) store_exchanged(gs, e + (size_t)b * tile_floats, unwritten_value());
     }
-  if constexpr (SETS == 2) reset_partials<NB, CT>(red, live_partials<CT>(Kpad));
+  if constexpr (SETS == 2) reset_partials<NB, RCT>(red, live_partials<CT>(Kpad));
   group_arrive(gs);  // also: the slice is complete in LDS
   group_wait(gs);
   if (SETS == 2 && rows_here <= 0) return;  // no workgroup barrier from here on
@@ -152,9 +176,11 @@ void gru_forward_kernel(GruFwdParams p) {
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
       const size_t row = act[pp] ? (size_t)pn[pp] : 0, unit = act[pp] ? (size_t)pj[pp] : 0;
-      const float* wt = p.Wx + ((size_t)tt * N + row) * 3 * H + unit;
+      if constexpr (!kFusedInput) {
+        const float* wt = p.Wx + ((size_t)tt * N + row) * 3 * H + unit;
 #pragma unroll
-      for (int g = 0; g < 3; ++g) wx_next[pp][g] = wt[g * H];
+        for (int g = 0; g < 3; ++g) wx_next[pp][g] = wt[g * H];
+      }
       if (zoneout && p.training) mk_next[pp] = p.zoneout_mask[(size_t)tt * NH + row * H + unit];
     }
   };
@@ -170,33 +196,43 @@ void gru_forward_kernel(GruFwdParams p) {
     }
     // The operand loads wait for h[t] themselves (polled tile t % 4).
     float* red_t = !kPolledPartials ? red : red + (t & 1) * RED;
-    if constexpr (REG > 0)
+    if constexpr (kFusedInput) {
+      tile_product<NB, CT, false, true, kPolledPartials, Projection, 0, NoResidentRows, false, RCT>(
+          xhb, (t & 3) * tile_floats, Kpad, w_lds, red_t, &gs, &proj);
+      if (t + 1 < T) proj.request();  // x[t+1]: a whole step to arrive
+    } else if constexpr (REG > 0) {
       tile_product<NB, CT, false, true, false, NoSideWork, REG, float4_t[REG][CT]>(
           xhb, (t & 3) * tile_floats, Kpad, w_lds, red_t, &gs, nullptr, &breg);
-    else
+    } else {
       tile_product<NB, CT, false, true, kPolledPartials, NoSideWork, 0, NoResidentRows, HALF>(
           xhb, (t & 3) * tile_floats, Kpad, w_lds, red_t, &gs);
+    }
     if constexpr (!kPolledPartials) __syncthreads();
 
     float saved[PP][4];  // z, r, g, q of the step for the caller's cache
     float h_pub[PP];
 #pragma unroll
     for (int pp = 0; pp < PP; ++pp) {
-      float rh[3] = {0.f, 0.f, 0.f};
+      // z and r: h*R (with x*W when the projection runs here); h*R of g; x*W of g
+      float rh[NG];
+#pragma unroll
+      for (int g = 0; g < NG; ++g) rh[g] = 0.f;
       if constexpr (kPolledPartials) {
         // whole wavefronts: the wait is a wavefront-wide vote
         if (((tid + 256 * pp) & ~63) < NB * HS)
-          take_product<NB, CT, 3>(gs, red_t, pl[pp], pc[pp], HS, tid + 256 * pp < NB * HS,
-                                  live_partials<CT>(Kpad), rh);
+          take_product<NB, RCT, NG>(gs, red_t, pl[pp], pc[pp], HS, tid + 256 * pp < NB * HS,
+                                    live_partials<CT>(Kpad), rh);
       } else if (act[pp]) {
 #pragma unroll
-        for (int g = 0; g < 3; ++g) rh[g] = sum_product<NB, CT>(red, pl[pp], g * HS + pc[pp]);
+        for (int g = 0; g < NG; ++g) rh[g] = sum_product<NB, RCT>(red, pl[pp], g * HS + pc[pp]);
       }
       if (act[pp]) {
-        const float z = sigmoid_f(wx[pp][0] + rh[0] + bxv[pp][0] + brv[pp][0]);
-        const float r = sigmoid_f(wx[pp][1] + rh[1] + bxv[pp][1] + brv[pp][1]);
+        const float wz = kFusedInput ? 0.f : wx[pp][0], wr = kFusedInput ? 0.f : wx[pp][1];
+        const float wg = kFusedInput ? rh[NG - 1] : wx[pp][2];
+        const float z = sigmoid_f(wz + rh[0] + bxv[pp][0] + brv[pp][0]);
+        const float r = sigmoid_f(wr + rh[1] + bxv[pp][1] + brv[pp][1]);
         const float qg = rh[2] + brv[pp][2];
-        const float g = tanh_f(wx[pp][2] + r * qg + bxv[pp][2]);
+        const float g = tanh_f(wg + r * qg + bxv[pp][2]);
         saved[pp][0] = z;
         saved[pp][1] = r;
         saved[pp][2] = g;
@@ -211,8 +247,9 @@ void gru_forward_kernel(GruFwdParams p) {
       h_pub[pp] = publishable(h_prev[pp]);
     }
     // Everything this wavefront stored during the previous step (its resets among it) has
-    // landed before h[t+1] becomes visible.
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // landed before h[t+1] becomes visible.  (x[t+1] arrives with the same wait.)
+    if constexpr (kFusedInput) proj.settle();
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     if (t + 1 < T) {
       float* xh_next = xh + ((t + 1) & 3) * tile_floats;
       float* xh_done = xh + ((t + 3) & 3) * tile_floats;  // read at step t-1: nobody needs it any more
@@ -796,14 +833,25 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
   if (!tile.ok)
     return gru_forward_streamed(stream, training, T, N, C, H, W, R, bx, br, x, h, h_out, v, tmp_Wx,
                                 zoneout_prob, zoneout_mask, dc_mask, dc_scale);
-  if (!wx_ready)
-    HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 3 * H, C, x, C, W, 3 * H, tmp_Wx, 3 * H, false));
-
   // An 8-row tile is run as two sets of 4 rows when the partial tiles of both fit beside the
   // slice (exchange tiles: one per set, together as large as the tile's).
-  const size_t paired_lds = paired_lds_bytes((H + 63) / 64 * 64, tile.ct);
+  const int Kpad = (H + 63) / 64 * 64;
+  size_t paired_lds = paired_lds_bytes(Kpad, tile.ct);
   const bool paired = tile.nb == 8 && paired_lds <= kWorkgroupLdsBytes &&
                       tile.reg_groups == 0;
+  // 4-row tiles of 16-unit workgroups compute x*W themselves, beside their waits, when a
+  // wavefront's share of W (C/4 x 48 columns) fits its registers (the step's x*W GEMM, its split
+  // reduce and the round trip of tmp_Wx through memory go away).  The partial tiles then have
+  // rows of 64 columns: the slice's 48 and the candidate gate's x*W.
+  const bool fused = !wx_ready && !half_product && (paired || tile.nb == 4) && tile.hs == 16 &&
+                     tile.reg_groups == 0 && C <= 512 && C % 4 == 0 &&
+                     (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && fused_input_enabled();
+  const int xsg = C <= 256 ? 1 : 2;
+  size_t lds_bytes = paired ? paired_lds : tile.lds_bytes;
+  if (fused)
+    lds_bytes = ((size_t)Kpad * 48 + (paired ? 4 : 1) * (size_t)ProductTile<4, 4>::kRedFloats) * sizeof(float);
+  if (!wx_ready && !fused)
+    HASTE_HIP_PROPAGATE(gemm_f32(stream, false, T * N, 3 * H, C, x, C, W, 3 * H, tmp_Wx, 3 * H, false));
 
   // Taken after the GEMM, which may replace the stream's scratch buffer with a larger one.
   Workspace ws;
@@ -814,14 +862,24 @@ int gru_forward_impl(hipStream_t stream, int training, int T, int N, int C, int 
   GruFwdParams p;
   p.training = training; p.T = T; p.N = N; p.H = H;
   p.R = R; p.bx = bx; p.br = br; p.h = h; p.h_out = h_out; p.v = v; p.Wx = tmp_Wx;
+  p.W = W; p.x = x; p.C = C;
   p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
   p.dc_mask = dc_mask; p.dc_scale = dc_scale;
   p.xh = ws.scratch;
   LaunchPlan plan;
-  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.nb,
-                                  paired ? paired_lds : tile.lds_bytes, (unsigned)T + 1, &plan));
+  HASTE_HIP_PROPAGATE(plan_launch(stream, ws, tile.gx, tile.gy, tile.nb, lds_bytes, (unsigned)T + 1, &plan));
   p.ls = plan.shape;
   if (paired) plan.threads = 512;
+#define HASTE_LAUNCH_FWD_FUSED(XSG_)                                                                       \
+  if (fused && xsg == XSG_) {                                                                              \
+    if (paired)                                                                                            \
+      return launch_persistent("gru_forward_recurrence", gru_forward_kernel<4, 3, 16, 2, 0, false, XSG_>,  \
+                               plan, p, stream);                                                           \
+    return launch_persistent("gru_forward_recurrence", gru_forward_kernel<4, 3, 16, 1, 0, false, XSG_>,    \
+                             plan, p, stream);                                                             \
+  }
+  HASTE_LAUNCH_FWD_FUSED(1) HASTE_LAUNCH_FWD_FUSED(2)
+#undef HASTE_LAUNCH_FWD_FUSED
 #define HASTE_LAUNCH_FWD_RESIDENT(NB_, CT_, HS_, REG_)                                              \
   if (tile.reg_groups == REG_ && tile.nb == NB_ && tile.hs == HS_)                                 \
     return launch_persistent("gru_forward_recurrence", gru_forward_kernel<NB_, CT_, HS_, 1, REG_>, \

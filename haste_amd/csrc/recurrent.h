@@ -885,6 +885,7 @@ __device__ __forceinline__ void mfma_tile_rows4(const float* w_lds, int s,
 // the operand loads it is polling.
 struct NoSideWork {
   static constexpr int kBatches = 0;
+  static constexpr bool kExtraTile = false;
 };
 
 // x[t][4 rows of a batch tile][C] * W[C][16*CT slice columns] on the 4x4x1 path, the
@@ -892,9 +893,14 @@ struct NoSideWork {
 // wavefront takes the XSG super-groups (64 k each) wave, wave + 4, ...  A lane keeps the weights
 // its MFMAs need in registers for the whole launch: 4 * CT * XSG floats, i.e. 128 for a
 // 64-column slice and C = 512 (two wavefronts per SIMD leave 256 registers per lane).
-template <int CT, int XSG>
+// SPLIT (a GRU: the candidate gate needs x*W and h*R apart): the projection's last column tile
+// accumulates into a tile of its own instead of the recurrent product's, which the product
+// leaves behind the slice's tiles in the partial tile (column tile CTN).
+template <int CT, int XSG, bool SPLIT = false>
 struct InputProjection {
   using S = ShortTileShape<CT>;
+  static constexpr bool kExtraTile = SPLIT;
+  float4_t extra0, extra1;   // SPLIT: the sums of the last column tile
   static constexpr int kSteps = XSG * S::NBC;   // one step: 4 * CTN MFMAs on one A block
   static constexpr int kStepsPerBatch = 4;
   static constexpr int kBatches = (kSteps + kStepsPerBatch - 1) / kStepsPerBatch;
@@ -966,29 +972,58 @@ struct InputProjection {
     }
   }
 
+  __device__ __forceinline__ void begin() { extra0 = extra1 = float4_t{0.f, 0.f, 0.f, 0.f}; }
+
   template <int B>
-  __device__ __forceinline__ void batch(float4_t (&acc0)[1][S::CTN], float4_t (&acc1)[1][S::CTN]) const {
+  __device__ __forceinline__ void batch(float4_t (&acc0)[1][S::CTN], float4_t (&acc1)[1][S::CTN]) {
     static_for<kStepsPerBatch>([&](auto ic) {
       constexpr int I = B * kStepsPerBatch + decltype(ic)::value;
       if constexpr (I < kSteps) {
         constexpr int XS = I / S::NBC;
         constexpr int A = I % S::NBC;
+        // component c of the operand goes to accumulator c % 2; the last tile to the extra one
+        static_for<4>([&](auto cc) {
+          constexpr int C4 = decltype(cc)::value;
+          const float xc = xa[XS][C4];
 #pragma unroll
-        for (int ct = 0; ct < S::CTN; ++ct)
-          acc0[0][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(xa[XS].x, w[XS][A][ct][0], acc0[0][ct], S::CBSZ, A, 0);
-#pragma unroll
-        for (int ct = 0; ct < S::CTN; ++ct)
-          acc1[0][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(xa[XS].y, w[XS][A][ct][1], acc1[0][ct], S::CBSZ, A, 0);
-#pragma unroll
-        for (int ct = 0; ct < S::CTN; ++ct)
-          acc0[0][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(xa[XS].z, w[XS][A][ct][2], acc0[0][ct], S::CBSZ, A, 0);
-#pragma unroll
-        for (int ct = 0; ct < S::CTN; ++ct)
-          acc1[0][ct] = __builtin_amdgcn_mfma_f32_4x4x1f32(xa[XS].w, w[XS][A][ct][3], acc1[0][ct], S::CBSZ, A, 0);
+          for (int ct = 0; ct < S::CTN; ++ct) {
+            float4_t& acc = (SPLIT && ct == S::CTN - 1) ? (C4 % 2 == 0 ? extra0 : extra1)
+                                                        : (C4 % 2 == 0 ? acc0[0][ct] : acc1[0][ct]);
+            acc = __builtin_amdgcn_mfma_f32_4x4x1f32(xc, w[XS][A][ct][C4], acc, S::CBSZ, A, 0);
+          }
+        });
       }
     });
   }
 };
+
+// One 4-row accumulator tile to its place in a partial tile: the KS lane groups hold sums over
+// different k of the same elements; they are added here, and every lane stores 4/KS of the 4
+// rows.  q: the tile's first row at this lane's column; `pitch`: floats per row.
+template <int KS, bool TAGGED>
+__device__ __forceinline__ void store_tile_sum(float* q, int pitch, float4_t v, int lane) {
+  if constexpr (KS == 4) {
+    // lane group 0, 1, 2, 3 ends up with row 0, 2, 1, 3
+    const float xz = swap_add16(v.x, v.z), yw = swap_add16(v.y, v.w);
+    float r = swap_add32(xz, yw);
+    if constexpr (TAGGED) r = publishable(r);
+    const int g = lane >> 4;
+    q[(((g & 1) << 1) | (g >> 1)) * pitch] = r;
+  } else if constexpr (KS == 2) {
+    // lane group 0: rows 0 and 2; lane group 1: rows 1 and 3
+    float r0 = swap_add32(v.x, v.y), r1 = swap_add32(v.z, v.w);
+    if constexpr (TAGGED) { r0 = publishable(r0); r1 = publishable(r1); }
+    const int g = lane >> 5;
+    q[g * pitch] = r0;
+    q[(g + 2) * pitch] = r1;
+  } else {
+    if constexpr (TAGGED) v = float4_t{publishable(v.x), publishable(v.y), publishable(v.z), publishable(v.w)};
+    q[0] = v.x;
+    q[pitch] = v.y;
+    q[2 * pitch] = v.z;
+    q[3 * pitch] = v.w;
+  }
+}
 
 // Product of a short exchange tile: red[wave][4*RB][16*CT] <- this wavefront's partial tile
 // (accumulator element r of acc[rb][ct] in lane l is row 4*rb + r, column ct*MC + l%MC, of
@@ -997,7 +1032,10 @@ struct InputProjection {
 // register buffers alternate so that nothing is copied.  The four wavefronts are those of one
 // 256-thread set of the workgroup.  TAGGED: the partial tiles are themselves polled by their
 // readers (take_product), so no element may carry the "unwritten" pattern.
-template <int RB, int CT, int CH, bool POLLED, bool TAGGED = false, class Side = NoSideWork, bool HALF = false>
+// RED_CT: column tiles of a partial tile's rows (more than CT when the side work leaves a tile of
+// its own behind the slice's).
+template <int RB, int CT, int CH, bool POLLED, bool TAGGED = false, class Side = NoSideWork, bool HALF = false,
+          int RED_CT = CT>
 __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int tile_off, int Kpad,
                                                        const float* w_lds, float* red,
                                                        const GroupSync* gs, Side* side = nullptr) {
@@ -1018,6 +1056,7 @@ __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int
     for (int ct = 0; ct < S::CTN; ++ct) acc0[rb][ct] = acc1[rb][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
 
   int s = wave;
+  if constexpr (Side::kExtraTile) side->begin();
   if constexpr (Side::kBatches > 0) {
     static_assert(RB == 1 && POLLED, "side work: polled 4-row tiles");
     // no operand chunk to look at between the batches: the side work runs on its own
@@ -1073,35 +1112,17 @@ __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int
 
   // The KS lane groups hold partial sums of the same elements: they are added here, so that a
   // wavefront leaves one partial tile, and every lane stores 4/KS of the 4 rows.
-  float* base = red + (wave * NB) * S::NCOLS + lane % S::MC;
+  constexpr int PITCH = 16 * RED_CT;
+  float* base = red + (wave * NB) * PITCH + lane % S::MC;
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-    for (int ct = 0; ct < S::CTN; ++ct) {
-      float4_t v = acc0[rb][ct] + acc1[rb][ct];
-      float* q = base + (4 * rb) * S::NCOLS + ct * S::MC;
-      if constexpr (S::KS == 4) {
-        // lane group 0, 1, 2, 3 ends up with row 0, 2, 1, 3
-        const float xz = swap_add16(v.x, v.z), yw = swap_add16(v.y, v.w);
-        float r = swap_add32(xz, yw);
-        if constexpr (TAGGED) r = publishable(r);
-        const int g = lane >> 4;
-        q[(((g & 1) << 1) | (g >> 1)) * S::NCOLS] = r;
-      } else if constexpr (S::KS == 2) {
-        // lane group 0: rows 0 and 2; lane group 1: rows 1 and 3
-        float r0 = swap_add32(v.x, v.y), r1 = swap_add32(v.z, v.w);
-        if constexpr (TAGGED) { r0 = publishable(r0); r1 = publishable(r1); }
-        const int g = lane >> 5;
-        q[g * S::NCOLS] = r0;
-        q[(g + 2) * S::NCOLS] = r1;
-      } else {
-        if constexpr (TAGGED) v = float4_t{publishable(v.x), publishable(v.y), publishable(v.z), publishable(v.w)};
-        q[0] = v.x;
-        q[S::NCOLS] = v.y;
-        q[2 * S::NCOLS] = v.z;
-        q[3 * S::NCOLS] = v.w;
-      }
-    }
+    for (int ct = 0; ct < S::CTN; ++ct)
+      store_tile_sum<S::KS, TAGGED>(base + (4 * rb) * PITCH + ct * S::MC, PITCH, acc0[rb][ct] + acc1[rb][ct], lane);
+  if constexpr (Side::kExtraTile) {
+    static_assert(RED_CT * 16 >= (S::CTN + 1) * S::MC, "no room for the side work's tile");
+    store_tile_sum<S::KS, TAGGED>(base + S::CTN * S::MC, PITCH, side->extra0 + side->extra1, lane);
+  }
 }
 
 // red <- partial tiles of tile[NB rows, Kpad] * slice[Kpad, 16*CT]; the exchange tile
@@ -1111,15 +1132,15 @@ __device__ __forceinline__ void short_exchange_product(const TileBuffer& xb, int
 // wait; otherwise the caller has waited at the group's step barrier and `gs` is unused.
 // REG > 0 (tall tiles): the slice is split between registers and LDS, see tall_tile_product.
 template <int NB, int CT, bool LONG_K, bool POLLED = false, bool TAGGED = false, class Side = NoSideWork,
-          int REG = 0, class Resident = NoResidentRows, bool HALF = false>
+          int REG = 0, class Resident = NoResidentRows, bool HALF = false, int RED_CT = CT>
 __device__ __forceinline__ void tile_product(const TileBuffer& xb, int tile_off, int Kpad,
                                              const float* w_lds, float* red,
                                              const GroupSync* gs = nullptr, Side* side = nullptr,
                                              const Resident* breg = nullptr) {
   if constexpr (ProductTile<NB, CT>::kShort) {
     static_assert(REG == 0, "register-resident slice rows exist for tall tiles only");
-    short_exchange_product<NB / 4, CT, LONG_K ? 4 : 2, POLLED, TAGGED, Side, HALF>(xb, tile_off, Kpad, w_lds,
-                                                                                    red, gs, side);
+    short_exchange_product<NB / 4, CT, LONG_K ? 4 : 2, POLLED, TAGGED, Side, HALF, RED_CT>(xb, tile_off, Kpad,
+                                                                                            w_lds, red, gs, side);
   } else {
     static_assert(!HALF, "the product on the half matrix cores exists for short tiles only");
     static_assert(!TAGGED, "polled partial tiles exist for short tiles only");

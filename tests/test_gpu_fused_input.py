@@ -1,4 +1,4 @@
-"""LSTM forward recurrence: x*W computed inside the recurrence (4-row tiles) gives, to rounding,
+"""LSTM and GRU forward recurrences: x*W computed inside the recurrence (4-row tiles) gives, to rounding,
 what the recurrence gives on x*W from a GEMM launched before it.
 
 The variant with the separate GEMM is selected by an environment variable that the library reads
@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 # (T, N, C, H)
-SHAPES = [(6, 41, 24, 512), (5, 64, 32, 256), (4, 36, 8, 72)]
+SHAPES = [(6, 41, 24, 512), (5, 64, 32, 256), (4, 36, 8, 72), (5, 40, 300, 320), (4, 13, 512, 400)]
 
 
 def run_cells(T, N, C, H):
