@@ -267,6 +267,11 @@ int gru_forward_single_step(hipStream_t stream, int training, int N, int C, int 
                             const float* R, const float* bx, const float* br, const float* x,
                             const float* h, float* h_out, float* v, float zoneout_prob,
                             const float* zoneout_mask, const float* dc_mask, float dc_scale);
+// Half tensors (IEEE binary16), sums and pointwise step in float.
+int gru_forward_single_step_half(hipStream_t stream, int training, int N, int C, int H, const void* W,
+                                 const void* R, const void* bx, const void* br, const void* x,
+                                 const void* h, void* h_out, void* v, float zoneout_prob,
+                                 const void* zoneout_mask, const void* dc_mask, float dc_scale);
 
 // The same for rows too wide for layer_norm.hip's row-in-registers kernels (stepwise.hip).
 int layer_norm_forward_wide(hipStream_t stream, int rows, int dim, const float* gamma,

@@ -7,7 +7,8 @@
 // [W; R] straight from memory: a workgroup takes 16 hidden units (all their gate columns) and
 // a run of the contraction, parks its partial sums, and the last workgroup of a column block
 // to finish adds the runs in index order and does the pointwise step (gates, cell update,
-// zoneout) -- one launch, no float atomics, results independent of timing.
+// zoneout) -- one launch, no float atomics, results independent of timing.  The GRU's half
+// entry points use the same kernel on half tensors (sums and pointwise step in float).
 //
 // Arithmetic: reference lib/lstm_forward_gpu.cu.cc:55-86, lib/gru_forward_gpu.cu.cc:46-84.
 #include "recurrent.h"
@@ -18,21 +19,25 @@ namespace {
 constexpr int kStepUnits = 16;      // hidden units per workgroup
 constexpr int kStepMaxRun = 512;    // contraction indices per workgroup and side
 
+typedef _Float16 half_t;
+
+// T: the caller's tensors (float, or half with the sums and the pointwise step in float).
+template <typename T>
 struct StepParams {
   int training, N, C, H;
-  const float* W;        // [C, G*H]
-  const float* R;        // [H, G*H]
-  const float* b;        // LSTM: [4H]; GRU: bx [3H]
-  const float* br;       // GRU: [3H]
-  const float* x;        // [N, C]
-  const float* h;        // [N, H]
-  const float* c;        // LSTM: [N, H]
-  float* h_out;          // [N, H]
-  float* c_out;          // LSTM: [N, H]
-  float* v;              // [N, 4H] (training; GRU: always when non-null)
+  const T* W;            // [C, G*H]
+  const T* R;            // [H, G*H]
+  const T* b;            // LSTM: [4H]; GRU: bx [3H]
+  const T* br;           // GRU: [3H]
+  const T* x;            // [N, C]
+  const T* h;            // [N, H]
+  const T* c;            // LSTM: [N, H]
+  T* h_out;              // [N, H]
+  T* c_out;              // LSTM: [N, H]
+  T* v;                  // [N, 4H] (training; GRU: always when non-null)
   float zoneout_prob;
-  const float* zoneout_mask;  // [N, H] or null
-  const float* dc_mask;       // DropConnect mask of R or null
+  const T* zoneout_mask;      // [N, H] or null
+  const T* dc_mask;           // DropConnect mask of R or null
   float dc_scale;
   float* h_stage;        // [N, H] when h_out overlaps h (state updated in place), else null
   float* partial;        // [runs][2 sides][NB][column blocks * 64]; unused with one run
@@ -41,49 +46,50 @@ struct StepParams {
 
 // Unit j = 16 cw + u of row n: its pre-activations from x * W (wx) and h * R (rh), then the
 // pointwise step.
-template <int GATES>
-__device__ __forceinline__ void finish_unit(const StepParams& p, int n, int j, const float (&wx)[GATES],
+template <int GATES, typename T>
+__device__ __forceinline__ void finish_unit(const StepParams<T>& p, int n, int j, const float (&wx)[GATES],
                                             const float (&rh)[GATES]) {
   const int H = p.H;
   const size_t e = (size_t)n * H + j;
-  const float h_old = p.h[e];
+  const float h_old = (float)p.h[e];
   const bool zoneout = p.zoneout_prob != 0.f && p.zoneout_mask != nullptr;
   float h_new;
   if constexpr (GATES == 4) {
     float a[4];
 #pragma unroll
-    for (int g = 0; g < 4; ++g) a[g] = wx[g] + rh[g] + p.b[g * H + j];
+    for (int g = 0; g < 4; ++g) a[g] = wx[g] + rh[g] + (float)p.b[g * H + j];
     const float gi = sigmoid_f(a[0]), gg = tanh_f(a[1]), gf = sigmoid_f(a[2]), go = sigmoid_f(a[3]);
-    const float c_new = gf * p.c[e] + gi * gg;
+    const float c_new = gf * (float)p.c[e] + gi * gg;
     h_new = go * tanh_f(c_new);
-    p.c_out[e] = c_new;
+    p.c_out[e] = (T)c_new;
     if (p.training) {
-      float* vt = p.v + (size_t)n * 4 * H + j;
-      vt[0] = gi; vt[H] = gg; vt[2 * H] = gf; vt[3 * H] = go;
+      T* vt = p.v + (size_t)n * 4 * H + j;
+      vt[0] = (T)gi; vt[H] = (T)gg; vt[2 * H] = (T)gf; vt[3 * H] = (T)go;
     }
   } else {
-    const float z = sigmoid_f(wx[0] + rh[0] + p.b[j] + p.br[j]);
-    const float r = sigmoid_f(wx[1] + rh[1] + p.b[H + j] + p.br[H + j]);
-    const float qg = rh[2] + p.br[2 * H + j];
-    const float g = tanh_f(wx[2] + r * qg + p.b[2 * H + j]);
+    const float z = sigmoid_f(wx[0] + rh[0] + (float)p.b[j] + (float)p.br[j]);
+    const float r = sigmoid_f(wx[1] + rh[1] + (float)p.b[H + j] + (float)p.br[H + j]);
+    const float qg = rh[2] + (float)p.br[2 * H + j];
+    const float g = tanh_f(wx[2] + r * qg + (float)p.b[2 * H + j]);
     h_new = z * h_old + (1.0f - z) * g;
     if (p.training && p.v != nullptr) {
-      float* vt = p.v + (size_t)n * 4 * H + j;
-      vt[0] = z; vt[H] = r; vt[2 * H] = g; vt[3 * H] = qg;
+      T* vt = p.v + (size_t)n * 4 * H + j;
+      vt[0] = (T)z; vt[H] = (T)r; vt[2 * H] = (T)g; vt[3 * H] = (T)qg;
     }
   }
   if (zoneout) {
-    if (p.training) h_new = (h_new - h_old) * p.zoneout_mask[e] + h_old;
+    if (p.training) h_new = (h_new - h_old) * (float)p.zoneout_mask[e] + h_old;
     else h_new = p.zoneout_prob * h_old + (1.0f - p.zoneout_prob) * h_new;
   }
-  if (p.h_stage == nullptr) p.h_out[e] = h_new;
+  if (p.h_stage == nullptr) p.h_out[e] = (T)h_new;
   else store_agent(&p.h_stage[e], h_new);
 }
 
 // h_out overlaps h: other workgroups may still be reading h when a column block is finished,
 // so the new state is parked and copied out by the last column block to finish, when every
 // run of every block has been read.  Called by the finishing workgroups, all threads.
-__device__ __forceinline__ void copy_staged_state(const StepParams& p, unsigned int* flag) {
+template <typename T>
+__device__ __forceinline__ void copy_staged_state(const StepParams<T>& p, unsigned int* flag) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -97,16 +103,16 @@ __device__ __forceinline__ void copy_staged_state(const StepParams& p, unsigned 
   __syncthreads();
   if (*flag == 0u) return;
   const int count = p.N * p.H;
-  for (int i = threadIdx.x; i < count; i += 256) p.h_out[i] = load_exchanged(&p.h_stage[i]);
+  for (int i = threadIdx.x; i < count; i += 256) p.h_out[i] = (T)load_exchanged(&p.h_stage[i]);
 }
 
 // GATES = 4: LSTM (i, g, f, o); GATES = 3: GRU (z, r, g).  NB: batch rows (N <= NB).
 // Workgroup (cw, run): columns of units 16 cw .. 16 cw + 15, run `run` of gridDim.y of the rows
 // of W and of the rows of R.  With a single run the workgroup finishes its units itself,
 // straight from LDS.
-template <int GATES, int NB>
+template <int GATES, int NB, typename T>
 __global__ __launch_bounds__(256)
-void forward_step_kernel(StepParams p) {
+void forward_step_kernel(StepParams<T> p) {
   constexpr int COLS = 64;  // 16 units x up to 4 gates (a GRU leaves the last 16 idle)
   extern __shared__ float s_dyn[];
   __shared__ float s_red[2][4][NB][COLS];
@@ -131,11 +137,11 @@ void forward_step_kernel(StepParams p) {
   // Row k of side `side` (0: W, 1: R under DropConnect), this thread's column; rows beyond the
   // run read row kb and are not used.
   auto weight = [&](int side, int k) {
-    const float* M = side == 0 ? p.W : p.R;
+    const T* M = side == 0 ? p.W : p.R;
     const bool any = kb[side] < ke[side] && col_ok;
     const size_t at = (size_t)(k < ke[side] ? k : kb[side]) * GH + col_off;
-    float w = any ? M[at] : 0.f;
-    if (side == 1 && p.dc_mask != nullptr && any) w = w * p.dc_mask[at] * p.dc_scale;
+    float w = any ? (float)M[at] : 0.f;
+    if (side == 1 && p.dc_mask != nullptr && any) w = w * (float)p.dc_mask[at] * p.dc_scale;
     return w;
   };
   // The first eight rows of each side are requested before anything waits for the inputs.
@@ -147,10 +153,10 @@ void forward_step_kernel(StepParams p) {
 
 #pragma unroll
   for (int side = 0; side < 2; ++side) {
-    const float* in = side == 0 ? p.x : p.h;
+    const T* in = side == 0 ? p.x : p.h;
     for (int i = tid; i < NB * per_run[side]; i += 256) {
       const int n = i / per_run[side], k = kb[side] + i % per_run[side];
-      s_in[side][i] = (n < N && k < ke[side]) ? in[(size_t)n * len[side] + k] : 0.f;
+      s_in[side][i] = (n < N && k < ke[side]) ? (float)in[(size_t)n * len[side] + k] : 0.f;
     }
   }
   __syncthreads();
@@ -203,7 +209,7 @@ void forward_step_kernel(StepParams p) {
         wx[g] = quarter_sum(0, n, g * kStepUnits + u);
         rh[g] = quarter_sum(1, n, g * kStepUnits + u);
       }
-      finish_unit<GATES>(p, n, j, wx, rh);
+      finish_unit<GATES, T>(p, n, j, wx, rh);
     }
     if (p.h_stage != nullptr) copy_staged_state(p, &s_flag);
     return;
@@ -241,13 +247,13 @@ void forward_step_kernel(StepParams p) {
           rh[g] += part[1][g][i];
         }
     }
-    finish_unit<GATES>(p, n, j, wx, rh);
+    finish_unit<GATES, T>(p, n, j, wx, rh);
   }
   if (p.h_stage != nullptr) copy_staged_state(p, &s_flag);
 }
 
-template <int GATES>
-int launch_step(hipStream_t stream, StepParams& p, const char* name) {
+template <int GATES, typename T>
+int launch_step(hipStream_t stream, StepParams<T>& p, const char* name) {
   const int gx = (p.H + kStepUnits - 1) / kStepUnits;
   // Runs of the contraction: enough workgroups for about two per CU, at most 64 runs, a run
   // keeping at least 32 rows of the longer side.  The step is bound by memory latency, not
@@ -276,10 +282,10 @@ int launch_step(hipStream_t stream, StepParams& p, const char* name) {
   auto padded_run = [&](int len) { return ((len + runs - 1) / runs + 3) / 4 * 4; };
   const size_t lds = (size_t)nb * (padded_run(p.C) + padded_run(p.H)) * sizeof(float);
   ScopedKernelTimer timer(name, stream);
-  if (nb == 1) forward_step_kernel<GATES, 1><<<grid, dim3(256), lds, stream>>>(p);
-  else if (nb == 2) forward_step_kernel<GATES, 2><<<grid, dim3(256), lds, stream>>>(p);
-  else if (nb == 4) forward_step_kernel<GATES, 4><<<grid, dim3(256), lds, stream>>>(p);
-  else forward_step_kernel<GATES, 8><<<grid, dim3(256), lds, stream>>>(p);
+  if (nb == 1) forward_step_kernel<GATES, 1, T><<<grid, dim3(256), lds, stream>>>(p);
+  else if (nb == 2) forward_step_kernel<GATES, 2, T><<<grid, dim3(256), lds, stream>>>(p);
+  else if (nb == 4) forward_step_kernel<GATES, 4, T><<<grid, dim3(256), lds, stream>>>(p);
+  else forward_step_kernel<GATES, 8, T><<<grid, dim3(256), lds, stream>>>(p);
   HASTE_HIP_TRY(hipGetLastError());
   return HASTE_HIP_OK;
 }
@@ -297,7 +303,7 @@ int lstm_forward_single_step(hipStream_t stream, int training, int N, int C, int
                              const float* c, float* h_out, float* c_out, float* v,
                              float zoneout_prob, const float* zoneout_mask, const float* dc_mask,
                              float dc_scale) {
-  StepParams p = {};
+  StepParams<float> p = {};
   p.training = training; p.N = N; p.C = C; p.H = H;
   p.W = W; p.R = R; p.b = b; p.x = x; p.h = h; p.c = c;
   p.h_out = h_out; p.c_out = c_out; p.v = v;
@@ -310,13 +316,27 @@ int gru_forward_single_step(hipStream_t stream, int training, int N, int C, int 
                             const float* R, const float* bx, const float* br, const float* x,
                             const float* h, float* h_out, float* v, float zoneout_prob,
                             const float* zoneout_mask, const float* dc_mask, float dc_scale) {
-  StepParams p = {};
+  StepParams<float> p = {};
   p.training = training; p.N = N; p.C = C; p.H = H;
   p.W = W; p.R = R; p.b = bx; p.br = br; p.x = x; p.h = h;
   p.h_out = h_out; p.v = v;
   p.zoneout_prob = zoneout_prob; p.zoneout_mask = zoneout_mask;
   p.dc_mask = dc_mask; p.dc_scale = dc_scale;
   return launch_step<3>(stream, p, "gru_forward_step");
+}
+
+int gru_forward_single_step_half(hipStream_t stream, int training, int N, int C, int H, const void* W,
+                                 const void* R, const void* bx, const void* br, const void* x,
+                                 const void* h, void* h_out, void* v, float zoneout_prob,
+                                 const void* zoneout_mask, const void* dc_mask, float dc_scale) {
+  auto in = [](const void* q) { return static_cast<const half_t*>(q); };
+  StepParams<half_t> p = {};
+  p.training = training; p.N = N; p.C = C; p.H = H;
+  p.W = in(W); p.R = in(R); p.b = in(bx); p.br = in(br); p.x = in(x); p.h = in(h);
+  p.h_out = static_cast<half_t*>(h_out); p.v = static_cast<half_t*>(v);
+  p.zoneout_prob = zoneout_prob; p.zoneout_mask = in(zoneout_mask);
+  p.dc_mask = in(dc_mask); p.dc_scale = dc_scale;
+  return launch_step<3>(stream, p, "gru_forward_step_half");
 }
 
 }  // namespace haste_hip

@@ -1488,7 +1488,8 @@ int haste_hip_layer_norm_indrnn_backward_f64(int steps, int batch_size, int inpu
 // lib/gru_backward_gpu.cu.cc:411).  Tensors are IEEE binary16 passed as void*; products are
 // accumulated and the pointwise math is done in float, results rounded to half.  Passes over
 // more than one step run on the persistent fp32 kernels (gru_half.hip); a single step
-// (Iterate) runs here, one product and one pointwise launch.
+// (Iterate) of at most 8 rows is one kernel (single_step.hip), of more rows it runs here, one
+// product and one pointwise launch per side.
 static inline const half_t* hp(const void* p) { return static_cast<const half_t*>(p); }
 static inline half_t* hp(void* p) { return static_cast<half_t*>(p); }
 
@@ -1504,6 +1505,10 @@ int haste_hip_gru_forward_f16(int training, int steps, int batch_size, int input
   if (steps > 1)
     return gru_forward_half(as_stream(stream), training, steps, batch_size, input_size, hidden_size, W, R,
                             bx, br, x, h, v, zoneout_prob, zoneout_mask, nullptr, 1.f);
+  if (single_step_applies(batch_size, input_size, hidden_size))
+    return gru_forward_single_step_half(as_stream(stream), training, batch_size, input_size, hidden_size,
+                                        W, R, bx, br, x, h, hp(h) + NH, v, zoneout_prob, zoneout_mask,
+                                        nullptr, 1.f);
   return gru_forward_steps<half_t>(as_stream(stream), training, steps, batch_size, input_size,
                                    hidden_size, hp(W), hp(R), hp(bx), hp(br), hp(x), hp(h),
                                    hp(h) + NH, hp(v), hp(tmp_Wx), zoneout_prob, hp(zoneout_mask),
@@ -1523,6 +1528,10 @@ int haste_hip_gru_forward_dropconnect_f16(int training, int steps, int batch_siz
     return gru_forward_half(as_stream(stream), training, steps, batch_size, input_size, hidden_size, W, R,
                             bx, br, x, h, v, zoneout_prob, zoneout_mask, dropconnect_mask,
                             dropconnect_scale);
+  if (single_step_applies(batch_size, input_size, hidden_size))
+    return gru_forward_single_step_half(as_stream(stream), training, batch_size, input_size, hidden_size,
+                                        W, R, bx, br, x, h, hp(h) + NH, v, zoneout_prob, zoneout_mask,
+                                        dropconnect_mask, dropconnect_scale);
   return gru_forward_steps<half_t>(as_stream(stream), training, steps, batch_size, input_size,
                                    hidden_size, hp(W), hp(R), hp(bx), hp(br), hp(x), hp(h),
                                    hp(h) + NH, hp(v), hp(tmp_Wx), zoneout_prob, hp(zoneout_mask),
@@ -1557,6 +1566,10 @@ int haste_hip_gru_forward_iterate_f16(int training, int batch_size, int input_si
   (void)tmp_Rh;
   HASTE_HIP_REQUIRE(batch_size > 0 && input_size > 0 && hidden_size > 0);
   HASTE_HIP_REQUIRE(W && R && bx && br && x && h && h_out && tmp_Wx && (v || !training));
+  if (single_step_applies(batch_size, input_size, hidden_size))
+    return gru_forward_single_step_half(as_stream(stream), training, batch_size, input_size, hidden_size,
+                                        W, R, bx, br, x, h, h_out, v, zoneout_prob, zoneout_mask, nullptr,
+                                        1.f);
   return gru_forward_steps<half_t>(as_stream(stream), training, 1, batch_size, input_size,
                                    hidden_size, hp(W), hp(R), hp(bx), hp(br), hp(x), hp(h), hp(h_out),
                                    hp(v), hp(tmp_Wx), zoneout_prob, hp(zoneout_mask), nullptr, 1.f);

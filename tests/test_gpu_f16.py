@@ -84,6 +84,38 @@ def test_f16_gru_inference_and_iterate():
     assert relerr(host(torch.stack(hs)), host(h)) < 4e-3
 
 
+@pytest.mark.parametrize("N,C,H", [(1, 512, 512), (3, 40, 100), (8, 24, 36), (5, 700, 16)])
+def test_f16_gru_single_step_of_a_small_batch(N, C, H):
+    """A step of at most 8 rows is one kernel on the half tensors: Iterate for training (gates
+    stored, zoneout by mask) and inference (zoneout by expectation), the state updated in place,
+    and a one-step Run under DropConnect, each against the oracle's step."""
+    from haste_amd import ops
+    import torch
+    print("gru f16 single step", N, C, H, flush=True)
+    T = 3
+    p = half_problem(50 + N + C + H, T, N, C, H, 0.3)
+    W, R, bx, br, x, mask = (dev16(p[k]) for k in ("W", "R", "b", "b2", "x", "mask"))
+    for training in (True, False):
+        ho, vo = O.gru_forward(p["W"], p["R"], p["b"], p["b2"], p["x"], p["h0"], training, 0.3, p["mask"])
+        state = dev16(p["h0"])
+        for t in range(T):
+            h1, v1 = ops.gru_forward_iterate(training, 0.3, x[t].contiguous(), state, W, R, bx, br,
+                                             mask[t].contiguous(), h_out=state)
+            assert h1.data_ptr() == state.data_ptr()
+            torch.cuda.synchronize()
+            assert relerr(host(state), ho[t + 1]) < TOL16, (training, t)
+            if training:
+                assert relerr(host(v1), vo[t]) < TOL16, t
+    r = np.random.default_rng(N)
+    m = (r.uniform(size=(H, 3 * H)) > 0.25).astype(np.float64)
+    h, cache = ops.gru_forward(True, 0.3, x[:1].contiguous(), dev16(p["h0"]), W, R, bx, br,
+                               mask[:1].contiguous(), dropconnect_mask=dev16(m), dropconnect_scale=2.0)
+    ho, vo = O.gru_forward(p["W"], p["R"] * m * 2.0, p["b"], p["b2"], p["x"][:1], p["h0"], True, 0.3,
+                           p["mask"][:1])
+    assert relerr(host(h), ho) < TOL16
+    assert relerr(host(cache), vo) < TOL16
+
+
 def test_f16_gru_dropconnect_and_accumulated_gradients():
     """DropConnect on the half GRU against the oracle on pre-masked recurrent weights (the mask's
     scale chosen so that the masked weights are exact in half), and the backward pass adding
