@@ -43,7 +43,7 @@ typedef _Float16 half_t;
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
-constexpr int kMaxSegments = 12;
+constexpr int kMaxSegments = 16;  // the backward pass stages twelve tensors
 
 // Tensors to convert in one launch: segment s is `count[s]` elements from src[s] to dst[s].
 struct ConvertList {
@@ -51,9 +51,14 @@ struct ConvertList {
   void* dst[kMaxSegments];
   unsigned long long count[kMaxSegments];
   int n = 0;
+  bool overflow = false;
   unsigned long long longest = 0;
   void add(const void* s, void* d, size_t c) {
     if (s == nullptr || d == nullptr || c == 0) return;
+    if (n == kMaxSegments) {
+      overflow = true;
+      return;
+    }
     src[n] = s;
     dst[n] = d;
     count[n] = c;
@@ -110,6 +115,7 @@ void convert_kernel(ConvertList l) {
 
 template <bool WIDEN>
 int convert(hipStream_t stream, const ConvertList& l) {
+  HASTE_HIP_REQUIRE(!l.overflow);
   if (l.n == 0) return HASTE_HIP_OK;
   unsigned long long blocks = (l.longest + 2047) / 2048;
   if (blocks > 4096) blocks = 4096;
