@@ -27,6 +27,8 @@ namespace haste_hip {
 int gemm_f64(hipStream_t stream, bool trans_a, int M, int N, int K, const double* A, int lda,
              const double* B, int ldb, double* C, int ldc, bool accumulate, size_t scratch_offset);
 size_t gemm_f64_scratch_bytes(int M, int N, int K);
+int gemm_f64_chunks(hipStream_t stream, int M, int N, int K, const double* A, int lda, const double* B,
+                    int ldb, size_t scratch_offset, const double** partial, int* chunks);
 int gemm_f16(hipStream_t stream, bool trans_a, int M, int N, int K, const void* A, int lda,
              const void* B, int ldb, void* C, int ldc, bool accumulate);
 // gru_half.hip: the half GRU over more than one step, on the fp32 kernels.
@@ -157,6 +159,20 @@ int step_product(hipStream_t s, int M, int N, int K, const T* A, const T* B, T* 
   return HASTE_HIP_OK;
 }
 template <>
+int step_product<double>(hipStream_t s, int M, int N, int K, const double* A, const double* B,
+                         double* out, size_t scratch_offset, StepProduct<double>* p) {
+  HASTE_HIP_PROPAGATE(gemm_f64_chunks(s, M, N, K, A, K, B, N, scratch_offset, &p->base, &p->chunks));
+  if (p->chunks > 0) {
+    p->stride = (size_t)M * N;
+    return HASTE_HIP_OK;
+  }
+  HASTE_HIP_PROPAGATE(gemm_f64(s, false, M, N, K, A, K, B, N, out, N, false, scratch_offset));
+  p->base = out;
+  p->chunks = 1;
+  p->stride = 0;
+  return HASTE_HIP_OK;
+}
+template <>
 int step_product<float>(hipStream_t s, int M, int N, int K, const float* A, const float* B,
                         float* out, size_t scratch_offset, StepProduct<float>* p) {
   if (gemm_f32_skinny_applies(false, M, N, K, A, K, B, N, out, N)) {
@@ -195,6 +211,17 @@ int reverse_product(hipStream_t s, int M, int N, int K, const T* A, const T* B, 
                     size_t scratch_offset, StepProduct<T>* pend) {
   pend->chunks = 0;
   return gemm(s, false, M, N, K, A, K, B, N, dh, N, true, scratch_offset);
+}
+template <>
+int reverse_product<double>(hipStream_t s, int M, int N, int K, const double* A, const double* B,
+                            double* dh, size_t scratch_offset, StepProduct<double>* pend) {
+  *pend = StepProduct<double>();
+  HASTE_HIP_PROPAGATE(gemm_f64_chunks(s, M, N, K, A, K, B, N, scratch_offset, &pend->base, &pend->chunks));
+  if (pend->chunks > 0) {
+    pend->stride = (size_t)M * N;
+    return HASTE_HIP_OK;
+  }
+  return gemm_f64(s, false, M, N, K, A, K, B, N, dh, N, true, scratch_offset);
 }
 template <>
 int reverse_product<float>(hipStream_t s, int M, int N, int K, const float* A, const float* B,
