@@ -87,7 +87,10 @@ def test_f64_iterate(double_precision, T, N, C, H, zoneout):
 @pytest.mark.parametrize("trans_a,M,N,K", [(False, 1, 1, 1), (False, 37, 53, 29), (False, 128, 192, 64),
                                            (True, 70, 130, 45), (True, 5, 20, 33), (False, 300, 100, 1000),
                                            # few tiles, long contractions: cut along K into pieces
-                                           (False, 64, 512, 2048), (True, 33, 70, 3001)])
+                                           (False, 64, 512, 2048), (True, 33, 70, 3001),
+                                           # whole panels and columns inside the problem: the loads without
+                                           # bounds checks (rows beyond M beyond the buffer's range)
+                                           (True, 128, 256, 640), (False, 100, 128, 96), (True, 192, 128, 2080)])
 @pytest.mark.parametrize("accumulate", [False, True])
 def test_f64_gemm_and_transpose(trans_a, M, N, K, accumulate):
     from haste_amd import ops
